@@ -1,0 +1,202 @@
+// Dense matrix multiplication C[M,N] += A[M,K] @ B[K,N].
+//
+//   mfma     f32, M % 128 == 0, N % 128 == 0, K % 32 == 0: 128x128 block tiles, four wavefronts in a
+//            2x2 arrangement, each owning a 64x64 sub-tile as 2x2 v_mfma_f32_32x32x2_f32
+//            accumulators; A and B k-slices of depth 32 are staged through double-buffered LDS with
+//            register prefetch of the next slice.  Block ids are regrouped so that the blocks that
+//            are co-resident on one XCD (block id mod 8) form a compact patch of the tile grid
+//            and share A row panels and B column panels in that XCD's L2.
+//   simple   everything else (any size, f64): one thread per element of C, the k loop in the
+//            reference's order with the product rounded before the add, which makes it bit-identical
+//            to GEMM.partial_F32_MxN_RM + AXPY (J/backend/main/operations/linear/internal/blas/GEMM.java:282-304,
+//            AXPY.java:47-59).
+//
+// Column-major operands are handled as the transposed row-major problem C^T = B^T A^T.
+#include "nk_internal.h"
+
+namespace nk {
+
+template <typename T>
+__global__ __launch_bounds__(256) void matmul_simple_kernel(int M, int K, int N, const T* __restrict__ A,
+                                                            const T* __restrict__ B, T* __restrict__ C) {
+    const int n = blockIdx.x * 64 + (threadIdx.x & 63);
+    const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (m >= M || n >= N) return;
+    T acc = C[(int64_t)m * N + n];
+    const T* a = A + (int64_t)m * K;
+    for (int k = 0; k < K; k++) {
+        T prod = a[k] * B[(int64_t)k * N + n];   // rounded product, then add: no contraction
+        acc = acc + prod;
+    }
+    C[(int64_t)m * N + n] = acc;
+}
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int A_PITCH = BK + 4;     // floats; keeps 16-byte alignment of every row
+constexpr int B_PITCH = BN + 4;
+
+struct MfmaArgs {
+    int M, K, N;
+    int tiles_m, tiles_n;
+    int group_rows;      // tile rows per group of the block-id regrouping
+};
+
+__device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int& tm, int& tn) {
+    // hardware deals consecutive block ids round-robin to the 8 XCDs: give XCD x the x-th contiguous
+    // eighth of a grouped ordering (groups of `group_rows` tile rows, walked column by column)
+    const int nblk = g.tiles_m * g.tiles_n;
+    int bid = blockIdx.x;
+    int logical = bid;
+    if (nblk % 8 == 0) logical = (bid % 8) * (nblk / 8) + bid / 8;
+    const int per_group = g.group_rows * g.tiles_n;
+    const int grp = logical / per_group;
+    const int first_row = grp * g.group_rows;
+    int rows = g.tiles_m - first_row;
+    if (rows > g.group_rows) rows = g.group_rows;
+    const int in_grp = logical - grp * per_group;
+    tm = first_row + in_grp % rows;
+    tn = in_grp / rows;
+}
+
+__global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const float* __restrict__ A,
+                                                          const float* __restrict__ B, float* __restrict__ C) {
+    __shared__ __attribute__((aligned(16))) float As[2][BM * A_PITCH];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * B_PITCH];
+
+    int tm, tn;
+    tile_of_block(g, tm, tn);
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;     // wave's sub-tile origin inside the block tile
+    const int l32 = lane & 31, h = lane >> 5;
+
+    const float* Ag = A + (int64_t)tm * BM * g.K;
+    const float* Bg = B + (int64_t)tn * BN;
+
+    // global -> register staging: A slice 128x32, B slice 32x128, 4 float4 each per thread
+    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32*i
+    const int b_row = tid >> 5, b_col = (tid & 31) * 4;     // rows b_row + 8*i
+    f32x4 ra[4], rb[4];
+
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 8 * i) * g.N + b_col);
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            *(f32x4*)(&As[buf][(a_row + 32 * i) * A_PITCH + a_col]) = ra[i];
+            *(f32x4*)(&Bs[buf][(b_row + 8 * i) * B_PITCH + b_col]) = rb[i];
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    const int nk = g.K / BK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) load_global((kt + 1) * BK);
+        const float* as = As[cur];
+        const float* bs = Bs[cur];
+#pragma unroll
+        for (int c = 0; c < BK / 8; c++) {
+            // lane half h owns k = 8c + 4h .. 8c + 4h + 3 of this chunk; the four MFMA steps pair
+            // (k, k + 4): any pairing works as long as A and B use the same one
+            f32x4 a0 = *(const f32x4*)(&as[(wm + l32) * A_PITCH + 8 * c + 4 * h]);
+            f32x4 a1 = *(const f32x4*)(&as[(wm + 32 + l32) * A_PITCH + 8 * c + 4 * h]);
+            float b0[4], b1[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                b0[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + l32];
+                b1[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + 32 + l32];
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[t], b0[t], acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[t], b1[t], acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[t], b0[t], acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[t], b1[t], acc[1][1], 0, 0, 0);
+            }
+        }
+        if (kt + 1 < nk) {
+            store_lds(cur ^ 1);
+            __syncthreads();
+        }
+    }
+
+    // epilogue: accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4, column l32
+    float* Cg = C + (int64_t)(tm * BM + wm) * g.N + tn * BN + wn;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
+                float* p = Cg + (int64_t)row * g.N + 32 * j + l32;
+                *p = *p + acc[i][j][v];
+            }
+}
+
+template <typename T>
+static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* A, const T* B, T* C) {
+    dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4));
+    NK_REQUIRE(grid.y <= 65535u * 1024u, "nk_matmul: M too large");
+    set_path("simple");
+    hipLaunchKernelGGL(matmul_simple_kernel<T>, grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, A, B, C);
+    NK_HIP(hipGetLastError());
+    return NK_OK;
+}
+
+static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+    if (dtype == NK_F64) return launch_simple<double>(dev, M, K, N, (const double*)A, (const double*)B, (double*)C);
+    const bool aligned = (A % 16 == 0) && (B % 16 == 0) && (C % 16 == 0);
+    if (aligned && M % BM == 0 && N % BN == 0 && K % BK == 0) {
+        MfmaArgs g{};
+        g.M = (int)M; g.K = (int)K; g.N = (int)N;
+        g.tiles_m = (int)(M / BM); g.tiles_n = (int)(N / BN);
+        g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
+        set_path("mfma");
+        hipLaunchKernelGGL(matmul_mfma_kernel, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
+                           (const float*)A, (const float*)B, (float*)C);
+        NK_HIP(hipGetLastError());
+        return NK_OK;
+    }
+    return launch_simple<float>(dev, M, K, N, (const float*)A, (const float*)B, (float*)C);
+}
+
+}  // namespace nk
+
+using namespace nk;
+
+extern "C" int nk_matmul(nk_dev h, int dtype, int layout, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+    NK_DEVICE(dev, h);
+    NK_REQUIRE(dtype == NK_F32 || dtype == NK_F64, "nk_matmul: unknown dtype %d", dtype);
+    NK_REQUIRE(layout == NK_LAYOUT_ROW_MAJOR || layout == NK_LAYOUT_COLUMN_MAJOR, "nk_matmul: unknown layout %d", layout);
+    NK_REQUIRE(M >= 1 && K >= 1 && N >= 1, "nk_matmul: M, K, N must be positive (got %lld, %lld, %lld)", (long long)M, (long long)K, (long long)N);
+    NK_REQUIRE(M * K < ((int64_t)1 << 31) && K * N < ((int64_t)1 << 31) && M * N < ((int64_t)1 << 31),
+               "nk_matmul: operands are limited to 2^31-1 elements");
+    const int eb = dtype_bytes(dtype);
+    if (int e = check_range(dev, "nk_matmul(A)", A, 0, (uint64_t)(M * K) * eb)) return e;
+    if (int e = check_range(dev, "nk_matmul(B)", B, 0, (uint64_t)(K * N) * eb)) return e;
+    if (int e = check_range(dev, "nk_matmul(C)", C, 0, (uint64_t)(M * N) * eb)) return e;
+    if (layout == NK_LAYOUT_ROW_MAJOR) return matmul_rm(dev, dtype, M, K, N, A, B, C);
+    // column-major data of X[r,c] is the row-major data of X^T[c,r]:  C^T[N,M] += B^T[N,K] @ A^T[K,M]
+    return matmul_rm(dev, dtype, N, K, M, B, A, C);
+}

@@ -1,0 +1,276 @@
+// Scalar functions of the elementwise kernel family, device side.
+//
+// Semantics follow the CPU lambdas of the reference, J/backend/main/implementations/fun/Scalar*.java
+// (J/ = src/main/java/neureka/).  The reference evaluates most f32 activations as
+// `(float) f((double) x)` (fun/api/CPUFun.java:7-9); here f32 is evaluated in f32 with formulations
+// that avoid the cancellation a literal f32 transcription would suffer, so results stay within 1e-5
+// relative of the reference.  Functions the reference overrides with pure float arithmetic
+// (fast_gaus, softsign, gasu, fast_tanh, relu, quad, ...) are transcribed operation for operation and are
+// bit-identical (the library is compiled with -ffp-contract=off and correctly rounded division).
+// f64 uses the reference's own formulas.
+#pragma once
+#include <hip/hip_runtime.h>
+#include "../../include/neureka_hip.h"
+
+namespace nk {
+
+template <typename T> struct Num;
+template <> struct Num<float> {
+    static __device__ __forceinline__ float exp(float x) { return ::expf(x); }
+    static __device__ __forceinline__ float expm1(float x) { return ::expm1f(x); }
+    static __device__ __forceinline__ float log(float x) { return ::logf(x); }
+    static __device__ __forceinline__ float log1p(float x) { return ::log1pf(x); }
+    static __device__ __forceinline__ float log10(float x) { return ::log10f(x); }
+    static __device__ __forceinline__ float sin(float x) { return ::sinf(x); }
+    static __device__ __forceinline__ float cos(float x) { return ::cosf(x); }
+    static __device__ __forceinline__ float sqrt(float x) { return ::sqrtf(x); }
+    static __device__ __forceinline__ float cbrt(float x) { return ::cbrtf(x); }
+    static __device__ __forceinline__ float pow(float a, float b) { return ::powf(a, b); }
+    static __device__ __forceinline__ float fmod(float a, float b) { return ::fmodf(a, b); }
+    static __device__ __forceinline__ float abs(float x) { return ::fabsf(x); }
+    static __device__ __forceinline__ float tanh(float x) { return ::tanhf(x); }
+    static __device__ __forceinline__ float fma(float a, float b, float c) { return ::fmaf(a, b, c); }
+};
+template <> struct Num<double> {
+    static __device__ __forceinline__ double exp(double x) { return ::exp(x); }
+    static __device__ __forceinline__ double expm1(double x) { return ::expm1(x); }
+    static __device__ __forceinline__ double log(double x) { return ::log(x); }
+    static __device__ __forceinline__ double log1p(double x) { return ::log1p(x); }
+    static __device__ __forceinline__ double log10(double x) { return ::log10(x); }
+    static __device__ __forceinline__ double sin(double x) { return ::sin(x); }
+    static __device__ __forceinline__ double cos(double x) { return ::cos(x); }
+    static __device__ __forceinline__ double sqrt(double x) { return ::sqrt(x); }
+    static __device__ __forceinline__ double cbrt(double x) { return ::cbrt(x); }
+    static __device__ __forceinline__ double pow(double a, double b) { return ::pow(a, b); }
+    static __device__ __forceinline__ double fmod(double a, double b) { return ::fmod(a, b); }
+    static __device__ __forceinline__ double abs(double x) { return ::fabs(x); }
+    static __device__ __forceinline__ double tanh(double x) { return ::tanh(x); }
+    static __device__ __forceinline__ double fma(double a, double b, double c) { return ::fma(a, b, c); }
+};
+
+// FunUtil.invSqrt (fun/FunUtil.java:5-27): the bit-trick inverse square root with 4 (double) or 2
+// (float) Newton steps, transcribed operation for operation.
+__device__ __forceinline__ double inv_sqrt_ref(double x) {
+    double xhalf = 0.5 * x;
+    long long i = __double_as_longlong(x);
+    i = 0x5fe6ec85e7de30daLL - (i >> 1);
+    x = __longlong_as_double(i);
+    x *= (1.5 - xhalf * x * x);
+    x *= (1.5 - xhalf * x * x);
+    x *= (1.5 - xhalf * x * x);
+    x *= (1.5 - xhalf * x * x);
+    return x;
+}
+__device__ __forceinline__ float inv_sqrt_ref(float x) {
+    float xhalf = 0.5f * x;
+    int i = __float_as_int(x);
+    i = 0x5f3759df - (i >> 1);
+    x = __int_as_float(i);
+    x *= (1.5f - xhalf * x * x);
+    x *= (1.5f - xhalf * x * x);
+    return x;
+}
+
+// ScalarSigmoid.sig (fun/ScalarSigmoid.java:38): 1/(1+exp(-x)).
+__device__ __forceinline__ double sigmoid(double x) { return 1.0 / (1.0 + ::exp(-x)); }
+// f32: the same quantity; the branch keeps exp() in range where the reference's double
+// intermediate would not overflow either.
+__device__ __forceinline__ float sigmoid(float x) {
+    if (x >= 0.0f) return 1.0f / (1.0f + ::expf(-x));
+    float e = ::expf(x);
+    return e / (1.0f + e);
+}
+
+// ScalarTanh.tanh (fun/ScalarTanh.java:37-38): 2/(1+exp(-2x))-1.
+__device__ __forceinline__ double tanh_ref(double x) { return 2.0 / (1.0 + ::exp(-x * 2.0)) - 1.0; }
+__device__ __forceinline__ float tanh_ref(float x) { return ::tanhf(x); }
+
+// 1 - tanh(x)^2 (ScalarTanh derivative, fun/ScalarTanh.java:31-34)
+__device__ __forceinline__ double dtanh_ref(double x) { double t = tanh_ref(x); return 1.0 - t * t; }
+__device__ __forceinline__ float dtanh_ref(float x) {
+    float e = ::expf(-2.0f * ::fabsf(x));       // sech^2 = 4e/(1+e)^2, no cancellation for large |x|
+    float s = 1.0f + e;
+    return 4.0f * e / (s * s);
+}
+
+template <typename T>
+__device__ __forceinline__ T softsign(T x) { return x / (T(1) + Num<T>::abs(x)); }
+
+// exp(-(x*x)) (fun/ScalarGaussian.java).  f32 carries the rounding error of x*x into the result so
+// that it matches the reference's double evaluation to f32 accuracy.
+__device__ __forceinline__ double gauss(double x) { return ::exp(-(x * x)); }
+__device__ __forceinline__ float gauss(float x) {
+    float hi = x * x;
+    float lo = ::fmaf(x, x, -hi);
+    float e = ::expf(-hi);
+    return e - e * lo;
+}
+
+// The evaluators below work on V values at once with the switch outside the lane loop: the op-code
+// is uniform over the whole grid, so the dispatch is done once per instruction, not once per value.
+#define NK_EACH(expr)                                   \
+    {                                                   \
+        _Pragma("unroll") for (int v = 0; v < V; v++) { \
+            const T x = a[v]; (void)x;                  \
+            a[v] = (expr);                              \
+        }                                               \
+    }                                                   \
+    break
+
+template <typename T> __device__ __forceinline__ T selu_ref(T x) {
+    const double ALPHA = 1.6732632423543772848170429916717, SCALE = 1.0507009873554804934193349852946;
+    if (x > T(0)) return T(SCALE) * x;
+    if (x <= T(0)) {
+        if (sizeof(T) == 8) return T(SCALE * ALPHA * ((double)Num<T>::exp(x) - 1.0));
+        return T(SCALE * ALPHA) * Num<T>::expm1(x);
+    }
+    return T(NAN);
+}
+template <typename T> __device__ __forceinline__ T dselu_ref(T x) {
+    const double ALPHA = 1.6732632423543772848170429916717, SCALE = 1.0507009873554804934193349852946;
+    if (x > T(0)) return T(SCALE);
+    if (x <= T(0)) return T(SCALE * ALPHA) * Num<T>::exp(x);
+    return T(NAN);
+}
+template <typename T> __device__ __forceinline__ T softplus_ref(T x) {
+    using N = Num<T>;
+    if (sizeof(T) == 8) return N::log(T(1) + N::exp(x));
+    return x > T(0) ? x + N::log1p(N::exp(-x)) : N::log1p(N::exp(x));
+}
+template <typename T> __device__ __forceinline__ T dgasu_ref(T x) {
+    T x2 = x * x, x6 = x2 * x2 * x2;
+    return T(3) * x2 / (T(2) * x2 * Num<T>::abs(x) + x6 + T(1));
+}
+template <typename T> __device__ __forceinline__ T dgatu_ref(T x) {
+    T x2 = x * x, x3 = x2 * x, temp = T(3) * x2;
+    if (sizeof(T) == 8) { T t = tanh_ref(x3); return -temp * (t * t) + temp; }
+    return temp * dtanh_ref(x3);     // = -temp*tanh^2 + temp without the cancellation
+}
+template <typename T> __device__ __forceinline__ T dfast_gaus_ref(T x) {
+    T x2 = x * x;
+    return T(-2) * x / (x2 * x2 + T(2) * x2 + T(1));
+}
+template <typename T> __device__ __forceinline__ T dgelu_ref(T x) {
+    T sig = sigmoid(x * T(1.702)), ds = sig * (T(1) - sig);
+    return sig + ds * x * T(1.702);
+}
+template <typename T> __device__ __forceinline__ T dsig_ref(T x) { T s = sigmoid(x); return s * (T(1) - s); }
+template <typename T> __device__ __forceinline__ T dsilu_ref(T x) { T s = sigmoid(x); return s + (x * s * (T(1) - s)); }
+template <typename T> __device__ __forceinline__ T dfast_tanh_ref(T x) {
+    T t1 = x * x, t2 = Num<T>::sqrt(T(1) + t1);
+    return T(1) / (t1 * t2 + t2);
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
+    using N = Num<T>;
+    switch (id) {
+        case NK_FUN_ABS: NK_EACH(N::abs(x));
+        case NK_FUN_COS: NK_EACH(N::cos(x));
+        case NK_FUN_GASU: NK_EACH(softsign(x * x * x));
+        case NK_FUN_GATU: NK_EACH(tanh_ref(x * x * x));
+        case NK_FUN_GAUS: NK_EACH(gauss(x));
+        case NK_FUN_FAST_GAUS: NK_EACH(T(1) / (T(1) + x * x));
+        case NK_FUN_GELU: NK_EACH(x * sigmoid(x * T(1.702)));
+        case NK_FUN_IDY: break;
+        case NK_FUN_LN: NK_EACH(N::log(x));
+        case NK_FUN_QUAD: NK_EACH(x * x);
+        case NK_FUN_RELU: NK_EACH(x >= T(0) ? x : x * T(.01));
+        case NK_FUN_SELU: NK_EACH(selu_ref(x));
+        case NK_FUN_SIG: NK_EACH(sigmoid(x));
+        case NK_FUN_SILU: NK_EACH(x * sigmoid(x));
+        case NK_FUN_SIN: NK_EACH(N::sin(x));
+        case NK_FUN_SOFTPLUS: NK_EACH(softplus_ref(x));
+        case NK_FUN_SOFTSIGN: NK_EACH(softsign(x));
+        case NK_FUN_TANH: NK_EACH(tanh_ref(x));
+        case NK_FUN_FAST_TANH: NK_EACH(x * inv_sqrt_ref(T(1) + x * x));
+        case NK_FUN_EXP: NK_EACH(N::exp(x));
+        case NK_FUN_LOG10: NK_EACH(N::log10(x));
+        case NK_FUN_SQRT: NK_EACH(N::sqrt(x));
+        case NK_FUN_CBRT: NK_EACH(N::cbrt(x));
+        default: NK_EACH(T(NAN) + x);
+    }
+}
+
+template <typename T, int V>
+__device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
+    using N = Num<T>;
+    switch (id) {
+        case NK_FUN_ABS: NK_EACH(x < T(0) ? T(-1) : T(1));
+        case NK_FUN_COS: NK_EACH(-N::sin(x));
+        case NK_FUN_GASU: NK_EACH(dgasu_ref(x));
+        case NK_FUN_GATU: NK_EACH(dgatu_ref(x));
+        case NK_FUN_GAUS: NK_EACH(T(-2) * x * gauss(x));
+        case NK_FUN_FAST_GAUS: NK_EACH(dfast_gaus_ref(x));
+        case NK_FUN_GELU: NK_EACH(dgelu_ref(x));
+        case NK_FUN_IDY: NK_EACH(T(1));
+        case NK_FUN_LN: NK_EACH(T(1) / x);
+        case NK_FUN_QUAD: NK_EACH(T(2) * x);
+        case NK_FUN_RELU: NK_EACH(x >= T(0) ? T(1) : T(.01));
+        case NK_FUN_SELU: NK_EACH(dselu_ref(x));
+        case NK_FUN_SIG: NK_EACH(dsig_ref(x));
+        case NK_FUN_SILU: NK_EACH(dsilu_ref(x));
+        case NK_FUN_SIN: NK_EACH(N::cos(x));
+        case NK_FUN_SOFTPLUS: NK_EACH(sigmoid(x));
+        case NK_FUN_SOFTSIGN: NK_EACH(T(1) / (T(2) * N::abs(x) + x * x + T(1)));
+        case NK_FUN_TANH: NK_EACH(dtanh_ref(x));
+        case NK_FUN_FAST_TANH: NK_EACH(dfast_tanh_ref(x));
+        case NK_FUN_EXP: NK_EACH(N::exp(x));
+        case NK_FUN_LOG10: NK_EACH(T(1) / (x * T(2.302585092994046)));   // x * ln(10)
+        case NK_FUN_SQRT: NK_EACH(T(0.5) * inv_sqrt_ref(x));
+        case NK_FUN_CBRT: NK_EACH(T(1) / (T(3) * N::pow(x, T(2.0) / T(3.0))));
+        default: NK_EACH(T(NAN) + x);
+    }
+}
+#undef NK_EACH
+
+// binary operators: CPUBiElementWise*.java / CPUBroadcast*.java (_getFun).  a = a op b.
+#define NK_EACH2(expr)                                  \
+    {                                                   \
+        _Pragma("unroll") for (int v = 0; v < V; v++) { \
+            const T x = a[v], y = b[v]; (void)x; (void)y; \
+            a[v] = (expr);                              \
+        }                                               \
+    }                                                   \
+    break
+
+template <typename T, int V>
+__device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
+    using N = Num<T>;
+    switch (op) {
+        case NK_OP_ADD: NK_EACH2(x + y);
+        case NK_OP_SUB: NK_EACH2(x - y);
+        case NK_OP_MUL: NK_EACH2(x * y);
+        case NK_OP_DIV: NK_EACH2(x / y);
+        case NK_OP_MOD: NK_EACH2(N::fmod(x, y));     // Java's % on floating point is C's fmod
+        case NK_OP_POW: NK_EACH2(N::pow(x, y));
+        case NK_OP_IDY: NK_EACH2(y);
+        default: NK_EACH2(T(NAN) + x + y);
+    }
+}
+
+// partial derivatives: CPUBiElementWise*.java (_getDeriveAt0 / _getDeriveAt1).  a = d(a op b)/d(operand d).
+template <typename T, int V>
+__device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b)[V]) {
+    using N = Num<T>;
+    switch (op * 2 + d) {
+        case NK_OP_ADD * 2 + 0:
+        case NK_OP_ADD * 2 + 1:
+        case NK_OP_SUB * 2 + 0: NK_EACH2(T(1));
+        case NK_OP_SUB * 2 + 1: NK_EACH2(T(-1));
+        case NK_OP_MUL * 2 + 0: NK_EACH2(y);
+        case NK_OP_MUL * 2 + 1: NK_EACH2(x);
+        case NK_OP_DIV * 2 + 0:
+        case NK_OP_MOD * 2 + 0: NK_EACH2(T(1) / y);
+        case NK_OP_DIV * 2 + 1:
+        case NK_OP_MOD * 2 + 1: NK_EACH2(-(x / (y * y)));
+        case NK_OP_POW * 2 + 0: NK_EACH2(y * N::pow(x, y - T(1)));
+        case NK_OP_POW * 2 + 1: NK_EACH2(N::pow(x, y) * N::log(x));
+        case NK_OP_IDY * 2 + 0: NK_EACH2(T(0));
+        case NK_OP_IDY * 2 + 1: NK_EACH2(T(1));
+        default: NK_EACH2(T(NAN) + x + y);
+    }
+}
+#undef NK_EACH2
+
+}  // namespace nk
