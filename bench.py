@@ -1,0 +1,222 @@
+#!/usr/bin/env python3
+"""Benchmark of the HipDevice hot path on one MI355X.
+
+Workload (the configuration the metric is quoted on): broadcast elementwise add and multiply,
+f32 [1024,1,512] o [1,2048,512] -> [1024,2048,512], uniform[-1,1] from a seed.  One step = one add launch
+plus one multiply launch through the C ABI of libneureka_hip.so, inputs and output resident in HBM.
+
+Prints ONE JSON line: whole-job throughput in GB/s of algorithmic bytes (`value`), the roofline of the
+dominant kernel measured with HIP events on the device's own stream (`roofline`), the CPU oracle timed
+on this box's host cores on a bounded sample (`cpu_baseline`), and kernel-level figures for the other
+configurations (`others`: GB/s or GFLOP/s with their fraction of the HBM / fp32-matrix peak).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
+
+
+def event_time_ms(dev, launch, reps):
+    """Average duration of `launch` over `reps` back-to-back launches, HIP events on the device stream."""
+    e0, e1 = dev.event(), dev.event()
+    dev.record(e0)
+    for _ in range(reps):
+        launch()
+    dev.record(e1)
+    return dev.elapsed_ms(e0, e1) / reps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the figures of the other configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one MI355X: this build has no multi-GPU path (every kernel shards without "
+              "exchange; see DESIGN.md), run it with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    from neureka_amd import Function, HipDevice, Tensor, _lib
+
+    dev = HipDevice.get(0)
+    rng = np.random.default_rng(2)
+    f32 = np.float32
+
+    # ---- the headline workload -------------------------------------------------------------------------
+    s1, s2, so = (1024, 1, 512), (1, 2048, 512), (1024, 2048, 512)
+    a = rng.uniform(-1, 1, s1).astype(f32)
+    b = rng.uniform(-1, 1, s2).astype(f32)
+    ta = Tensor.of(f32, s1, a).to(dev)
+    tb = Tensor.of(f32, s2, b).to(dev)
+    out = Tensor._on_device(dev, f32, so)
+    n_out = int(np.prod(so))
+    bytes_per_launch = 4 * (n_out + a.size + b.size)          # 4 301 258 752: write the output once, read each input once
+
+    def step():
+        dev.launch_broadcast("add", -1, out, ta, tb)
+        dev.launch_broadcast("multiply", -1, out, ta, tb)
+
+    for _ in range(args.warmup):
+        step()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    dev.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = 2 * bytes_per_launch / (ms_per_step * 1e-3) / 1e9
+    path = _lib.last_path()
+
+    k_add = event_time_ms(dev, lambda: dev.launch_broadcast("add", -1, out, ta, tb), args.steps)
+    k_mul = event_time_ms(dev, lambda: dev.launch_broadcast("multiply", -1, out, ta, tb), args.steps)
+    k_ms = 0.5 * (k_add + k_mul)
+    achieved = bytes_per_launch / (k_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"rows_kernel<float,4> ({path})",
+                "launch_ms": round(k_ms, 4), "algorithmic_bytes": bytes_per_launch}
+
+    # spot check of the timed output against numpy (the full parity tests live in tests/)
+    got = dev._read(out._data, 5 * 2048 * 512 + 7 * 512, 512)
+    assert got.tobytes() == (a[5, 0] * b[0, 7]).tobytes(), "benchmark output is wrong"
+
+    # ---- CPU baseline: the oracle's restatement of CPUBroadcast, scheduled like JVMExecutor ----------------
+    cpu = None
+    if not args.no_cpu:
+        from oracle import cpu_oracle as orc
+        cores = min(16, len(os.sched_getaffinity(0)))
+        rows = 64                                              # sample: the first 64 of 1024 slabs of the output
+        sample_shape = (rows, 2048, 512)
+        drn = np.zeros(int(np.prod(sample_shape)), dtype=f32)
+        a_s = a[:rows].reshape(-1).copy()
+        t0 = time.perf_counter()
+        orc.broadcast("add", -1, drn, orc.dense_cfg(sample_shape), a_s, orc.dense_cfg((rows, 1, 512)), b.reshape(-1), orc.dense_cfg(s2), workers=cores)
+        dt = time.perf_counter() - t0
+        sample_bytes = 4 * (drn.size + a_s.size + b.size)
+        assert drn[7 * 512:8 * 512].tobytes() == (a[0, 0] + b[0, 7]).tobytes()
+        cpu = {"value": round(sample_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": f"broadcast add on the first {rows}/1024 slabs of the output ({drn.size} elements, {dt:.2f} s), "
+                         "oracle restatement of CPUBroadcast._broadcastF32 split like JVMExecutor (no JVM on this box)"}
+        del drn
+    dev.free(out)
+
+    # ---- the other configurations: kernel figures only ------------------------------------------------------
+    others = {}
+    if not args.no_others:
+        reps = max(3, min(args.steps, 10))
+
+        def hbm(name, nbytes, launch):
+            launch(); dev.sync()
+            ms = event_time_ms(dev, launch, reps)
+            gbs = nbytes / (ms * 1e-3) / 1e9
+            others[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "path": _lib.last_path()}
+
+        def flops(name, nflop, nbytes, launch):
+            launch(); dev.sync()
+            ms = event_time_ms(dev, launch, reps)
+            tf = nflop / (ms * 1e-3) / 1e12
+            others[name] = {"ms": round(ms, 4), "GFLOP/s": round(tf * 1e3, 1), "frac_fp32": round(tf / FP32_PEAK_TFLOPS, 4),
+                            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "path": _lib.last_path()}
+
+        # C2 f64
+        a64 = Tensor.of(np.float64, (256, 1, 512), rng.uniform(-1, 1, 256 * 512)).to(dev)
+        b64 = Tensor.of(np.float64, (1, 1024, 512), rng.uniform(-1, 1, 1024 * 512)).to(dev)
+        o64 = Tensor._on_device(dev, np.float64, (256, 1024, 512))
+        hbm("broadcast_add_f64", 8 * (o64.size + a64.size + b64.size), lambda: dev.launch_broadcast("add", -1, o64, a64, b64))
+        for t in (a64, b64, o64): dev.free(t)
+
+        # C3: tanh(sig(a)*b+c) on 2^26 elements: fused, and the reference's 4-kernel sequence
+        n = 1 << 26
+        srcs = [Tensor.of(f32, (n,), rng.standard_normal(n).astype(f32)).to(dev) for _ in range(3)]
+        o = Tensor._on_device(dev, f32, (n,))
+        tmp = Tensor._on_device(dev, f32, (n,))
+        fn = Function.of("tanh(sig(I[0])*I[1]+I[2])")
+        fused = dev.optimizedFunctionOf(fn, "chain")
+        hbm("chain_fused_contiguous", 16 * n, lambda: dev.launch_fused(fused.program, fused.consts, o, srcs))
+
+        def unfused():
+            dev.launch_activation("sig", -1, tmp, srcs[0])
+            dev.launch_elementwise("multiply", -1, o, tmp, srcs[1])
+            dev.launch_elementwise("add", -1, tmp, o, srcs[2])
+            dev.launch_activation("tanh", -1, o, tmp)
+        hbm("chain_unfused_4_kernels", 40 * n, unfused)
+        hbm("activation_tanh", 8 * n, lambda: dev.launch_activation("tanh", -1, o, srcs[0]))
+        hbm("elementwise_add", 12 * n, lambda: dev.launch_elementwise("add", -1, o, srcs[0], srcs[1]))
+        # permuted [4096,16384] views of row-major [16384,4096]
+        from neureka_amd import NDConfiguration
+        pv = []
+        for t in srcs:
+            v = Tensor(f32, NDConfiguration.ofShape((16384, 4096)).newReshaped((1, 0)), None)
+            v._set_data(t._data, dev)
+            pv.append(v)
+        o2 = Tensor(f32, NDConfiguration.ofShape((4096, 16384)), None); o2._set_data(o._data, dev)
+        hbm("chain_fused_permuted", 16 * n, lambda: dev.launch_fused(fused.program, fused.consts, o2, pv))
+        # slice [::2, 1:8193] of [8192,16384] (the three 2^26 buffers are too small: use 2^27-element parents)
+        for t in srcs + [tmp]: dev.free(t)
+        parents = [Tensor.of(f32, (8192, 16384), rng.standard_normal(8192 * 16384).astype(f32)).to(dev) for _ in range(3)]
+        sv = [p[::2, 1:8193] for p in parents]
+        o3 = Tensor(f32, NDConfiguration.ofShape((4096, 8192)), None); o3._set_data(o._data, dev)
+        hbm("chain_fused_sliced", 16 * (1 << 25), lambda: dev.launch_fused(fused.program, fused.consts, o3, sv))
+        for p in parents: dev.free(p)
+        dev.free(o)
+
+        # C4 matmul
+        for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256))):
+            A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
+            B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
+            Cm = Tensor._on_device(dev, f32, (M, N))
+            flops(name, 2.0 * M * K * N, 4 * (M * K + K * N + M * N), lambda: dev.launch_matmul(True, M, K, N, A, B, Cm))
+            for t in (A, B, Cm): dev.free(t)
+
+        # C1 and C5 convolutions
+        x1 = Tensor.of(f32, (64, 64), rng.uniform(-1, 1, 4096).astype(f32)).to(dev)
+        k1 = Tensor.of(f32, (3, 3), rng.uniform(-1, 1, 9).astype(f32)).to(dev)
+        y1 = Tensor._on_device(dev, f32, (62, 62))
+        flops("conv2d_64x64_3x3", 69192, 31796, lambda: dev.launch_convolution(-1, y1, x1, k1))
+        x5 = Tensor.of(f32, (64, 256, 256), (rng.standard_normal(64 * 256 * 256) * 0.1).astype(f32)).to(dev)
+        k5 = Tensor.of(f32, (64, 5, 5), (rng.standard_normal(1600) * 0.1).astype(f32)).to(dev)
+        y5 = Tensor._on_device(dev, f32, (1, 252, 252))
+        e5 = Tensor.of(f32, (1, 252, 252), rng.standard_normal(252 * 252).astype(f32)).to(dev)
+        dx5 = Tensor._on_device(dev, f32, (64, 256, 256))
+        dk5 = Tensor._on_device(dev, f32, (64, 5, 5))
+        flops("conv_c5_forward", 203212800, 17037632, lambda: dev.launch_convolution(-1, y5, x5, k5))
+        flops("conv_c5_grad_input", 203212800, 17037632, lambda: dev.launch_convolution(0, dx5, k5, e5))
+        flops("conv_c5_grad_kernel", 203212800, 17037632, lambda: dev.launch_convolution(0, dk5, x5, e5))
+
+    result = {
+        "metric": "GB/s & % HBM peak (broadcast/elementwise)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "broadcast add + multiply, f32 [1024,1,512] o [1,2048,512] -> [1024,2048,512], "
+                               "one step = one add launch + one multiply launch, 4 301 258 752 algorithmic bytes each",
+                   "device": dev.name(), "compute_units": dev.maxComputeUnits()},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "others": others,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,448 @@
+"""The plugin seam: ``ExecutionCall``, the device-agnostic ``Algorithm`` objects and ``HipBackend``, the
+registration table that hangs ``ImplementationFor<HipDevice>`` objects on them.
+
+Mirrors, for the hot path only:
+  - ``backend/api/ExecutionCall.java`` / ``Call.java`` (slot 0 = drain, ``Arg.DerivIdx``)
+  - ``backend/main/algorithms/{BiElementwise,Broadcast,BiScalarBroadcast,ElementwiseAlgorithm,NDConvolution,MatMulAlgorithm}.java``
+    (suitability scores and call preparation = output allocation)
+  - ``backend/api/template/algorithms/AbstractDeviceAlgorithm.java:127-156`` (executeDeviceAlgorithm) and
+    ``:427-449`` (executeOnCommonDevice)
+  - ``backend/ocl/CLBackend.java:200-325`` (the op x algorithm -> implementation table)
+(paths relative to src/main/java/neureka/ of the reference).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field, replace
+from typing import Callable, Dict, List, Optional, Sequence
+
+import numpy as np
+
+from .device import HipDevice
+from .ndim import IllegalArgumentException, IllegalStateException, Layout
+
+# suitability scores: backend/api/fun/SuitabilityPredicate.java:21-29
+VERY_GOOD, GOOD, BAD, UNSUITABLE = 0.75, 0.625, 0.25, 0.0
+
+ACTIVATIONS = ["abs", "cos", "gasu", "gatu", "gaus", "fast_gaus", "gelu", "idy", "ln", "quad", "relu", "selu", "sig",
+               "silu", "sin", "softplus", "softsign", "tanh", "fast_tanh", "exp", "log10", "sqrt", "cbrt"]
+OPERATORS = {"+": "add", "-": "subtract", "*": "multiply", "/": "divide", "%": "modulo", "**": "power", "^": "power",
+             "x": "mul_conv", "@": "matMul"}
+
+
+@dataclass
+class ExecutionCall:
+    device: Optional[HipDevice]
+    operation: "Operation"
+    inputs: List[Optional[object]]
+    derivIdx: int = -1
+    algorithm: Optional["Algorithm"] = None
+
+    def input(self, i: int):
+        return self.inputs[i]
+
+    @property
+    def arity(self) -> int:
+        return len(self.inputs)
+
+    def getDerivativeIndex(self) -> int:
+        return self.derivIdx
+
+    def withInputAt(self, i: int, t) -> "ExecutionCall":
+        inputs = list(self.inputs)
+        inputs[i] = t
+        return replace(self, inputs=inputs)
+
+    def withAddedInputAt(self, i: int, t) -> "ExecutionCall":
+        inputs = list(self.inputs)
+        inputs.insert(i, t)
+        return replace(self, inputs=inputs)
+
+    def withInputs(self, inputs: Sequence) -> "ExecutionCall":
+        return replace(self, inputs=list(inputs))
+
+
+class Algorithm:
+    """A device-agnostic algorithm with per-device implementations (backend/api/DeviceAlgorithm.java:40-66)."""
+
+    name = "algorithm"
+
+    def __init__(self):
+        self._impls: Dict[type, Callable[[ExecutionCall], object]] = {}
+
+    def setImplementationFor(self, device_class: type, impl) -> "Algorithm":
+        self._impls[device_class] = impl
+        return self
+
+    def getImplementationFor(self, device) -> Optional[Callable]:
+        for cls in type(device).__mro__:
+            if cls in self._impls:
+                return self._impls[cls]
+        return None
+
+    def isSuitableFor(self, call: ExecutionCall) -> float:
+        return UNSUITABLE
+
+    def prepare(self, call: ExecutionCall) -> ExecutionCall:
+        return call
+
+
+def _new_output(device: HipDevice, dtype, shape, layout: Layout = Layout.ROW_MAJOR):
+    """``Tensor.of(type).withShape(shape).all(0)`` + ``setIsVirtual(false)`` + ``device.store`` as the call
+    preparations do it (e.g. Broadcast.java:90-94); the zeros are produced by a device fill."""
+    from .tensor import Tensor
+    t = Tensor._on_device(device, dtype, shape, layout)
+    t._intermediate = True
+    return t
+
+
+class BiElementwise(Algorithm):
+    name = "elementwise"
+
+    def isSuitableFor(self, call):       # BiElementwise.java:17-24
+        ts = [t for t in call.inputs if t is not None]
+        if all(t.shape == ts[0].shape for t in ts):
+            return GOOD
+        return UNSUITABLE
+
+    def prepare(self, call):             # BiElementwise.java:42-61
+        if call.arity < 3:
+            call = call.withAddedInputAt(0, None)
+        if call.input(0) is None:
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape))
+        return call
+
+
+class Broadcast(Algorithm):
+    name = "broadcast"
+
+    def isSuitableFor(self, call):       # Broadcast.java:18-46
+        ts = [t for t in call.inputs if t is not None]
+        max_rank = max(t.rank for t in ts)
+        for i in range(max_rank):
+            current = -1
+            for t in ts:
+                if i < t.rank:
+                    if current == -1:
+                        current = t.shape[i]
+                    elif current != t.shape[i] and current != 1 and t.shape[i] != 1:
+                        return UNSUITABLE
+        return GOOD
+
+    def prepare(self, call):             # Broadcast.java:60-97
+        from .tensor import make_fit
+        if call.arity < 3:
+            call = call.withAddedInputAt(0, None)
+        offset = 1 if call.input(0) is None else 0
+        if call.input(offset).rank != call.input(1 + offset).rank:
+            a, b = make_fit([call.input(offset), call.input(1 + offset)])
+            call = call.withInputs([None, a, b])
+        if call.input(0) is None:
+            s1, s2 = call.input(1).shape, call.input(2).shape
+            out_shape = tuple(s2[i] if s1[i] == 1 else s1[i] for i in range(len(s1)))
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, out_shape))
+        return call
+
+
+class BiScalarBroadcast(Algorithm):
+    name = "scalarization"
+
+    def isSuitableFor(self, call):       # BiScalarBroadcast.java:16-29
+        ts = call.inputs
+        if len(ts) not in (2, 3):
+            return UNSUITABLE
+        offset = len(ts) - 2
+        if ts[1 + offset] is None or ts[offset] is None:
+            return UNSUITABLE
+        if ts[1 + offset].size > 1 and not ts[1 + offset].isVirtual():
+            return UNSUITABLE
+        return VERY_GOOD
+
+    def prepare(self, call):             # BiScalarBroadcast.java:30-45
+        offset = 1 if call.input(0) is None else 0
+        if call.arity == 2:
+            offset = 0
+        src = call.input(offset)
+        out = _new_output(call.device, src.dtype, src.shape)
+        if call.arity == 3:
+            return call.withInputAt(0, out)
+        return call.withAddedInputAt(0, out)
+
+
+class ElementwiseAlgorithm(Algorithm):
+    name = "activation"
+
+    def isSuitableFor(self, call):
+        return GOOD
+
+    def prepare(self, call):             # ElementwiseAlgorithm.java:39-53: a fresh row-major output
+        if call.arity < 2:
+            call = call.withAddedInputAt(0, None)
+        if call.input(0) is None:
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape))
+        return call
+
+
+class NDConvolution(Algorithm):
+    name = "convolution"
+
+    def isSuitableFor(self, call):
+        return GOOD
+
+    def prepare(self, call):             # linear/Convolution.java:91-103, ConvUtil.shapeOfCon (ConvUtil.java:61-66)
+        if call.arity <= 2:
+            call = call.withAddedInputAt(0, None)
+        if call.input(0) is None:
+            s1, s2 = call.input(1).shape, call.input(2).shape
+            shp = tuple(abs(s1[i] - s2[i]) + 1 for i in range(min(len(s1), len(s2))))
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, shp))
+        return call
+
+
+class MatMulAlgorithm(Algorithm):
+    name = "simple_matmul"
+
+    def isSuitableFor(self, call):
+        return GOOD
+
+    @staticmethod
+    def _is_rm_or_cm(layout: Layout) -> bool:
+        return layout in (Layout.ROW_MAJOR, Layout.COLUMN_MAJOR)
+
+    def prepare(self, call):             # MatMulAlgorithm.java:64-155
+        if call.arity == 2:
+            call = call.withAddedInputAt(0, None)
+        if call.input(0) is None:
+            a, b = call.input(1), call.input(2)
+            la, lb = a.ndc.getLayout(), b.ndc.getLayout()
+            if self._is_rm_or_cm(la):
+                if lb is not Layout.SYMMETRIC and lb is not la:
+                    b = b.toLayoutCopy(la)
+                lc = la
+            elif self._is_rm_or_cm(lb):
+                if la is not Layout.SYMMETRIC and la is not lb:
+                    a = a.toLayoutCopy(lb)
+                lc = lb
+            else:
+                lc = Layout.ROW_MAJOR
+                a, b = a.toLayoutCopy(lc), b.toLayoutCopy(lc)
+            out = _new_output(call.device, a.dtype, (a.shape[0], b.shape[1]), lc)
+            call = call.withInputs([out, a, b])
+        # _autoClone: anything that is not a dense RM or CM matrix is copied before the kernel sees it
+        inputs = []
+        for t in call.inputs:
+            lay = t.ndc.getLayout()
+            if t.rank != 2 or lay not in (Layout.ROW_MAJOR, Layout.COLUMN_MAJOR, Layout.SYMMETRIC) or t.isPartialSlice():
+                t = t.deepCopy()
+            inputs.append(t)
+        return call.withInputs(inputs)
+
+
+class Operation:
+    """An operation with its algorithms (backend/api/Operation.java; template/operations/AbstractOperation.java:178-211)."""
+
+    def __init__(self, identifier: str, operator: str, algorithms: Sequence[Algorithm]):
+        self.identifier = identifier
+        self.operator = operator
+        self.algorithms = list(algorithms)
+
+    def getAlgorithm(self, cls: type) -> Optional[Algorithm]:
+        for a in self.algorithms:
+            if isinstance(a, cls):
+                return a
+        return None
+
+    def getAlgorithmFor(self, call: ExecutionCall) -> Algorithm:
+        best, score = None, 0.0
+        for a in self.algorithms:
+            s = a.isSuitableFor(call)
+            if s > score:
+                best, score = a, s
+        if best is None:
+            raise IllegalStateException(f"No suitable algorithm found for operation '{self.identifier}'")
+        return best
+
+
+def execute_device_algorithm(call: ExecutionCall):
+    """AbstractDeviceAlgorithm.executeDeviceAlgorithm (AbstractDeviceAlgorithm.java:127-156)."""
+    for t in call.inputs:
+        if t is None:
+            raise IllegalArgumentException("Device arguments may not be null!")
+    impl = call.algorithm.getImplementationFor(call.device)
+    if impl is None:
+        raise IllegalStateException(
+            f"No '{type(call.device).__name__}' implementation found for algorithm '{call.algorithm.name}' "
+            f"of operation '{call.operation.identifier}'")
+    call.device.approve(call)
+    impl(call)
+    return call.input(0)
+
+
+def execute_on_common_device(call: ExecutionCall, run: Callable[[ExecutionCall], object]):
+    """AbstractDeviceAlgorithm.executeOnCommonDevice (:427-449): operands that are not on the device are
+    stored for the duration of the call and restored afterwards."""
+    device = call.device
+    guests = [t for t in call.inputs if t is not None and not t.isOutsourced()]
+    for t in guests:
+        device.store(t)
+    try:
+        return run(call)
+    finally:
+        for t in guests:
+            if device.has(t):
+                device.restore(t)
+
+
+class BackendContext:
+    """Operations by identifier + the extensions registered on them (backend/api/BackendContext.java:170-346)."""
+
+    def __init__(self):
+        self.operations: Dict[str, Operation] = {}
+        for op_id, sym in [("add", "+"), ("subtract", "-"), ("multiply", "*"), ("divide", "/"), ("modulo", "%"), ("power", "**")]:
+            self.operations[op_id] = Operation(op_id, sym, [BiElementwise(), Broadcast(), BiScalarBroadcast()])
+        for op_id, sym in [("mul_conv", "x"), ("inv_convolve_mul_left", "«x"), ("inv_convolve_mul_right", "x»")]:
+            self.operations[op_id] = Operation(op_id, sym, [NDConvolution()])
+        self.operations["matMul"] = Operation("matMul", "@", [MatMulAlgorithm()])
+        for f in ACTIVATIONS:
+            self.operations[f] = Operation(f, f, [ElementwiseAlgorithm()])
+        self.extensions: List[object] = []
+
+    def getOperation(self, identifier: str) -> Operation:
+        op = self.operations.get(identifier)
+        if op is None:
+            raise IllegalArgumentException(f"unknown operation '{identifier}'")
+        return op
+
+    def set(self, extension) -> "BackendContext":
+        """BackendContext.set(BackendExtension) (:289-322): every registration must find its target."""
+        extension.load(_Registry(self, extension.device_class()))
+        self.extensions.append(extension)
+        return self
+
+    def find(self, key: str):
+        best, conf = None, 0.0
+        for ext in self.extensions:
+            dev, c = ext.find(key)
+            if c > conf:
+                best, conf = dev, c
+        return best if conf > 0.42 else None     # devices/Query.java:66-75
+
+
+class _Registry:
+    """The registration DSL (backend/api/ini/BackendRegistry.java:24-51)."""
+
+    def __init__(self, ctx: BackendContext, device_class: type):
+        self.ctx, self.device_class = ctx, device_class
+
+    def forOperation(self, identifier: str) -> "_Registry":
+        self._op = self.ctx.operations.get(identifier)
+        if self._op is None:
+            raise IllegalStateException(f"No operation '{identifier}' found for registration")
+        return self
+
+    def set(self, algorithm_class: type, impl) -> "_Registry":
+        alg = self._op.getAlgorithm(algorithm_class)
+        if alg is None:
+            raise IllegalStateException(f"Operation '{self._op.identifier}' has no algorithm {algorithm_class.__name__}")
+        alg.setImplementationFor(self.device_class, impl)
+        return self
+
+
+# ---- ImplementationFor<HipDevice> ------------------------------------------------------------------
+def hip_bi_elementwise(op: str):
+    """CLBiElementwise (implementations/elementwise/CLBiElementwise.java:11-24)."""
+    def run(call: ExecutionCall):
+        call.device.launch_elementwise(op, call.derivIdx, call.input(0), call.input(1), call.input(2))
+        return call.input(0)
+    return run
+
+
+def hip_broadcast(op: str):
+    """CLBroadcast (implementations/broadcast/CLBroadcast.java:12-24)."""
+    def run(call: ExecutionCall):
+        call.device.launch_broadcast(op, call.derivIdx, call.input(0), call.input(1), call.input(2))
+        return call.input(0)
+    return run
+
+
+def hip_scalar_broadcast(op: str):
+    """CLScalarBroadcast<Op>.run (e.g. implementations/broadcast/CLScalarBroadcastAddition.java:15-34)."""
+    def run(call: ExecutionCall):
+        value = float(call.input(2).item(0))
+        call.device.launch_scalarization(op, call.derivIdx, call.input(0), call.input(1), value)
+        return call.input(0)
+    return run
+
+
+def hip_elementwise_function(fun: str):
+    """CLElementwiseFunction (implementations/elementwise/CLElementwiseFunction.java:27-41)."""
+    def run(call: ExecutionCall):
+        call.device.launch_activation(fun, call.derivIdx, call.input(0), call.input(1))
+        return call.input(0)
+    return run
+
+
+def hip_convolution(call: ExecutionCall):
+    """CLConvolution (implementations/convolution/CLConvolution.java:11-23)."""
+    call.device.launch_convolution(call.derivIdx, call.input(0), call.input(1), call.input(2))
+    return call.input(0)
+
+
+def hip_matmul(call: ExecutionCall):
+    """CLMatMul / CPUMatMul (implementations/matmul/CPUMatMul.java:17-96): layout check, then the GEMM."""
+    c, a, b = call.input(0), call.input(1), call.input(2)
+    la, lb = a.ndc.getLayout(), b.ndc.getLayout()
+    if not (la.isCompatible(lb) and la.isCompatible(c.ndc.getLayout()) and lb.isCompatible(c.ndc.getLayout())):
+        raise IllegalArgumentException("Data layout inconsistency between provided tensors encountered. All tensors must be of the same layout.")
+    if not (a.dtype == b.dtype == c.dtype):
+        raise IllegalArgumentException("Type inconsistency between provided tensors encountered. All tensors must be of the same type.")
+    row_major = all(l in (Layout.ROW_MAJOR, Layout.SYMMETRIC) for l in (la, lb))
+    if a.shape[1] != b.shape[0]:
+        raise IllegalArgumentException(f"'A' matrix rows {a.shape[1]} did not match 'B' matrix columns {b.shape[0]}.")
+    call.device.launch_matmul(row_major, a.shape[0], a.shape[1], b.shape[1], a, b, c)
+    return c
+
+
+class HipBackend:
+    """``BackendExtension`` for HipDevice (model: backend/ocl/CLBackend.java:56-325)."""
+
+    KEYWORDS = ("hip", "rocm", "amd", "radeon", "gpu", "first gpu", "mi355x", "instinct")
+
+    def device_class(self) -> type:
+        return HipDevice
+
+    def find(self, key: str):
+        """DeviceOption(device, confidence): keyword match on the search key (CLBackend.java:56-94; devices/Query.java:22-24)."""
+        k = key.lower().strip()
+        if HipDevice.count() == 0:
+            return None, 0.0
+        dev = HipDevice.get(0)
+        if any(w == k or w in k.split() for w in self.KEYWORDS) or k in dev.name().lower():
+            return dev, 1.0
+        return dev, 0.0
+
+    def load(self, registry: _Registry) -> None:
+        for op in ("add", "subtract", "multiply", "divide", "modulo", "power"):
+            (registry.forOperation(op)
+                .set(BiScalarBroadcast, hip_scalar_broadcast(op))
+                .set(Broadcast, hip_broadcast(op))
+                .set(BiElementwise, hip_bi_elementwise(op)))
+        for op in ("mul_conv", "inv_convolve_mul_left", "inv_convolve_mul_right"):
+            registry.forOperation(op).set(NDConvolution, hip_convolution)
+        registry.forOperation("matMul").set(MatMulAlgorithm, hip_matmul)
+        for f in ACTIVATIONS:
+            registry.forOperation(f).set(ElementwiseAlgorithm, hip_elementwise_function(f))
+
+    def dispose(self) -> None:
+        for dev in list(HipDevice._open.values()):
+            dev.dispose()
+
+
+_context: Optional[BackendContext] = None
+
+
+def backend() -> BackendContext:
+    """The process-wide context with HipBackend registered (Neureka.get().backend(), Neureka.java:113-147)."""
+    global _context
+    if _context is None:
+        _context = BackendContext().set(HipBackend())
+    return _context

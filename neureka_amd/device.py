@@ -1,0 +1,330 @@
+"""``HipDevice``: the device object that satisfies Neureka's ``Device`` contract on an MI355X.
+
+Mirrors ``src/main/java/neureka/devices/opencl/OpenCLDevice.java`` (store/restore/free/has, buffer
+ownership through reference-counted data objects, virtual tensors, blocking reads and writes) on top of
+the C ABI of ``libneureka_hip.so``.  Method names follow ``neureka.devices.Device``
+(``src/main/java/neureka/devices/Device.java:73-410``) and ``AbstractDevice`` (``AbstractDevice.java:86-206``).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+
+from . import _lib
+from .ndim import IllegalArgumentException, IllegalStateException, NDConfiguration
+
+
+def _dtype_code(dtype) -> int:
+    dt = np.dtype(dtype)
+    if dt == np.float32:
+        return _lib.F32
+    if dt == np.float64:
+        return _lib.F64
+    raise IllegalArgumentException(f"HipDevice computes in float32 and float64, not {dt}")
+
+
+class HipData:
+    """A device buffer with a usage count: ``AbstractDeviceData`` (devices/AbstractDeviceData.java:7-59) /
+    ``OpenCLDevice.CLData`` (OpenCLDevice.java:950-966).  Tensors that share storage (slices, permuted
+    views) share one HipData; the buffer is released when the count drops to zero."""
+
+    def __init__(self, device: "HipDevice", ptr: int, dtype, size: int):
+        self.device = device
+        self.ptr = ptr
+        self.dtype = np.dtype(dtype)
+        self.size = size            # elements
+        self._usage = 0
+        self._freed = False
+        device._data_objects += 1
+
+    def owner(self) -> "HipDevice":
+        return self.device
+
+    def usages(self) -> int:
+        return self._usage
+
+    def incrementUsageCount(self) -> None:
+        self._usage += 1
+
+    def decrementUsageCount(self) -> None:
+        self._usage -= 1
+        if self._usage <= 0:
+            self.release()
+
+    def release(self) -> None:
+        if not self._freed:
+            self._freed = True
+            self.device._data_objects -= 1
+            if not self.device._disposed:
+                _lib.check(self.device._lib.nk_free(self.device.handle, self.ptr))
+
+    def __del__(self):  # the role of CustomDeviceCleaner (devices/CustomDeviceCleaner.java:21-121)
+        try:
+            self.release()
+        except Exception:
+            pass
+
+
+class HipDevice:
+    """One MI355X: one in-order HIP stream, blocking host transfers, asynchronous kernel launches."""
+
+    _open: Dict[int, "HipDevice"] = {}
+
+    # ---- discovery ---------------------------------------------------------------------------
+    @staticmethod
+    def count() -> int:
+        n = C.c_int(0)
+        _lib.check(_lib.load().nk_device_count(C.byref(n)))
+        return n.value
+
+    @staticmethod
+    def get(index: int = 0) -> "HipDevice":
+        dev = HipDevice._open.get(index)
+        if dev is None or dev._disposed:
+            dev = HipDevice(index)
+            HipDevice._open[index] = dev
+        return dev
+
+    def __init__(self, index: int = 0):
+        self._lib = _lib.load()
+        h = C.c_uint64(0)
+        _lib.check(self._lib.nk_device_open(index, C.byref(h)))
+        self.handle = h.value
+        self.index = index
+        self._disposed = False
+        self._data_objects = 0
+        self._stored: List[object] = []          # tensors currently outsourced to this device
+        name = C.create_string_buffer(256)
+        cu, mhz, lds, wave = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
+        mem = C.c_uint64(0)
+        _lib.check(self._lib.nk_device_props(self.handle, name, 256, C.byref(cu), C.byref(mhz), C.byref(mem), C.byref(lds), C.byref(wave)))
+        self._name = name.value.decode()
+        self._cu, self._mhz, self._mem, self._lds, self._wave = cu.value, mhz.value, mem.value, lds.value, wave.value
+
+    # properties: OpenCLDevice.java:738-809
+    def name(self) -> str: return self._name
+    def maxComputeUnits(self) -> int: return self._cu
+    def maxClockFrequenzy(self) -> int: return self._mhz       # spelling of the reference (OpenCLDevice.java:768)
+    def globalMemSize(self) -> int: return self._mem
+    def localMemSize(self) -> int: return self._lds
+    def wavefrontSize(self) -> int: return self._wave
+    def __repr__(self) -> str: return f"HipDevice[{self.index}: {self._name}, {self._cu} CUs]"
+
+    # ---- Device contract ---------------------------------------------------------------------
+    def numberOfStored(self) -> int:
+        return len(self._stored)
+
+    def numberOfDataObjects(self) -> int:
+        return self._data_objects
+
+    def isEmpty(self) -> bool:
+        return not self._stored
+
+    def has(self, tensor) -> bool:
+        return any(t is tensor for t in self._stored)
+
+    def contains(self, tensor) -> bool:
+        return self.has(tensor)
+
+    def store(self, tensor) -> "HipDevice":
+        """``Tensor.to(device)`` lands here: AbstractDevice.update (AbstractDevice.java:86-107) +
+        OpenCLDevice._updateInternal/_add (OpenCLDevice.java:346-405,661-674)."""
+        self._check_open()
+        if self.has(tensor):
+            return self
+        parent = tensor._parent
+        if parent is not None:
+            root = tensor._root()
+            if not self.has(root):
+                raise IllegalStateException("Data parent is not outsourced!")
+            tensor._set_data(root._data, self)      # share the root's buffer
+        else:
+            host = tensor._data
+            if isinstance(host, HipData):
+                if host.device is self:
+                    tensor._set_data(host, self)
+                    self._stored.append(tensor)
+                    return self
+                raise IllegalStateException("tensor already lives on another device")
+            data = self._upload(host, tensor.dtype, tensor.isVirtual())
+            tensor._set_data(data, self)
+        self._stored.append(tensor)
+        return self
+
+    def restore(self, tensor) -> "HipDevice":
+        """Brings a tensor back to host memory (OpenCLDevice.java:315-334)."""
+        if not self.has(tensor):
+            raise IllegalArgumentException("The passed tensor cannot be restored from this device as it is not stored on the device.")
+        host = self._read_all(tensor._data)
+        self.free(tensor)
+        tensor._set_data(host, None)
+        return self
+
+    def free(self, tensor) -> "HipDevice":
+        """Drops the device's claim on the tensor (OpenCLDevice.java:609-620)."""
+        for i, t in enumerate(self._stored):
+            if t is tensor:
+                del self._stored[i]
+                break
+        else:
+            raise IllegalArgumentException("tensor is not stored on this device")
+        data = tensor._data
+        tensor._data = None
+        tensor._device = None
+        if isinstance(data, HipData):
+            data.decrementUsageCount()
+        return self
+
+    def approve(self, call) -> "HipDevice":
+        """Device.approve (Device.java:205-214): every operand must be on this device."""
+        for t in call.inputs:
+            if t is not None and t._device is not self:
+                raise IllegalStateException("ExecutionCall holds a tensor that is not stored on the executing HipDevice")
+        return self
+
+    def sync(self) -> None:
+        _lib.check(self._lib.nk_device_sync(self.handle))
+
+    def dispose(self) -> None:
+        """OpenCLDevice.dispose (OpenCLDevice.java:299-304): finishes the queue and drops every buffer."""
+        if self._disposed:
+            return
+        for t in list(self._stored):
+            t._data = None
+            t._device = None
+        self._stored.clear()
+        _lib.check(self._lib.nk_device_close(self.handle))
+        self._disposed = True
+
+    def liveBuffers(self) -> int:
+        n, b = C.c_uint64(0), C.c_uint64(0)
+        _lib.check(self._lib.nk_device_stats(self.handle, C.byref(n), C.byref(b)))
+        return n.value
+
+    # ---- data access: AbstractDevice._readAll/_readItem/_readArray/_writeItem/_writeArray ------------
+    def allocate(self, dtype, size: int) -> HipData:
+        """Device.allocate (OpenCLDevice.java:520-530)."""
+        self._check_open()
+        ptr = C.c_uint64(0)
+        _lib.check(self._lib.nk_alloc(self.handle, int(size) * np.dtype(dtype).itemsize, C.byref(ptr)))
+        return HipData(self, ptr.value, dtype, int(size))
+
+    def allocateFromOne(self, dtype, size: int, value) -> HipData:
+        """Device.allocateFromOne: a buffer filled with one value by the device (OpenCLDevice.java:478-486)."""
+        data = self.allocate(dtype, size)
+        self._fill(data, 0, size, value)
+        return data
+
+    def allocateFromAll(self, array: np.ndarray) -> HipData:
+        array = np.ascontiguousarray(array)
+        data = self.allocate(array.dtype, array.size)
+        self._write(data, 0, array)
+        return data
+
+    def _upload(self, host: np.ndarray, dtype, virtual: bool) -> HipData:
+        host = np.ascontiguousarray(host, dtype=dtype)
+        if virtual:     # a virtual tensor keeps a single element on the device
+            return self.allocateFromOne(dtype, 1, host.reshape(-1)[0])
+        return self.allocateFromAll(host.reshape(-1))
+
+    def _fill(self, data: HipData, start: int, count: int, value) -> None:
+        pat = np.array([value], dtype=data.dtype)
+        _lib.check(self._lib.nk_fill(self.handle, data.ptr, start * data.dtype.itemsize, pat.ctypes.data_as(C.c_void_p),
+                                     data.dtype.itemsize, count))
+
+    def _write(self, data: HipData, start: int, array: np.ndarray) -> None:
+        array = np.ascontiguousarray(array, dtype=data.dtype)
+        _lib.check(self._lib.nk_h2d(self.handle, data.ptr, start * data.dtype.itemsize, array.ctypes.data_as(C.c_void_p), array.nbytes))
+
+    def _read(self, data: HipData, start: int, count: int) -> np.ndarray:
+        out = np.empty(count, dtype=data.dtype)
+        _lib.check(self._lib.nk_d2h(self.handle, out.ctypes.data_as(C.c_void_p), data.ptr, start * data.dtype.itemsize, out.nbytes))
+        return out
+
+    def _read_all(self, data: HipData) -> np.ndarray:
+        return self._read(data, 0, data.size)
+
+    def _actualize(self, tensor) -> None:
+        """virtual -> full buffer, filled by the device (OpenCLDevice.java:573-593)."""
+        old: HipData = tensor._data
+        value = self._read(old, 0, 1)[0]
+        new = self.allocateFromOne(tensor.dtype, tensor.ndc.size, value)
+        tensor._replace_data(new)
+
+    def _virtualize(self, tensor) -> None:
+        old: HipData = tensor._data
+        value = self._read(old, tensor.ndc.indexOfIndex(0) if not tensor.ndc.isVirtual() else 0, 1)[0]
+        new = self.allocateFromOne(tensor.dtype, 1, value)
+        tensor._replace_data(new)
+
+    def _check_open(self) -> None:
+        if self._disposed:
+            raise IllegalStateException("HipDevice has been disposed")
+
+    # ---- fused functions: Device.optimizedFunctionOf (Device.java:216-243) -------------------------
+    def optimizedFunctionOf(self, function, name: str):
+        from .function import OptimizedFunction
+        return OptimizedFunction(self, function, name)
+
+    # ---- kernel launches (thin wrappers over the C ABI; operands are device tensors) ----------------
+    @staticmethod
+    def _ops(*tensors):
+        out = []
+        for t in tensors:
+            # a virtual tensor keeps one element on the device and is addressed through all-zero tables
+            inline = (NDConfiguration.virtualOf(t.shape) if t.isVirtual() else t.ndc).asInlineArray()
+            out.append((C.c_uint64(t._data.ptr), inline, _lib.cfg_ptr(inline)))
+        return out
+
+    def launch_activation(self, fun: str, d: int, drn, src) -> None:
+        (p0, k0, c0), (p1, k1, c1) = self._ops(drn, src)
+        _lib.check(self._lib.nk_activation(self.handle, _lib.FUN[fun], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, drn.ndc.size))
+
+    def launch_elementwise(self, op: str, d: int, drn, a, b) -> None:
+        (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = self._ops(drn, a, b)
+        _lib.check(self._lib.nk_elementwise(self.handle, _lib.OP[op], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, drn.ndc.size))
+
+    def launch_scalarization(self, op: str, d: int, drn, src, value: float) -> None:
+        (p0, k0, c0), (p1, k1, c1) = self._ops(drn, src)
+        _lib.check(self._lib.nk_scalarization(self.handle, _lib.OP[op], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, float(value), drn.ndc.size))
+
+    def launch_scalar_fill(self, drn, value: float) -> None:
+        ((p0, k0, c0),) = self._ops(drn)
+        _lib.check(self._lib.nk_scalar_fill(self.handle, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, float(value), drn.ndc.size))
+
+    def launch_broadcast(self, op: str, d: int, drn, a, b) -> None:
+        (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = self._ops(drn, a, b)
+        _lib.check(self._lib.nk_broadcast(self.handle, _lib.OP[op], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, drn.ndc.size))
+
+    def launch_convolution(self, d: int, drn, a, b) -> None:
+        (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = self._ops(drn, a, b)
+        _lib.check(self._lib.nk_convolution(self.handle, d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, drn.ndc.size))
+
+    def launch_matmul(self, row_major: bool, M: int, K: int, N: int, a, b, c) -> None:
+        _lib.check(self._lib.nk_matmul(self.handle, _dtype_code(c.dtype), _lib.ROW_MAJOR if row_major else _lib.COLUMN_MAJOR,
+                                       M, K, N, a._data.ptr, b._data.ptr, c._data.ptr))
+
+    def launch_fused(self, program: Sequence[int], consts: Sequence[float], drn, srcs) -> None:
+        ops = self._ops(drn, *srcs)
+        prog = (C.c_int32 * len(program))(*program)
+        cs = (C.c_double * max(1, len(consts)))(*consts)
+        ptrs = (C.c_uint64 * max(1, len(srcs)))(*[o[0].value for o in ops[1:]])
+        cfgs = (C.POINTER(C.c_int32) * max(1, len(srcs)))(*[o[2] for o in ops[1:]])
+        _lib.check(self._lib.nk_fused(self.handle, prog, len(program) // 2, cs, len(consts), _dtype_code(drn.dtype), drn.ndc.rank,
+                                      ops[0][0], ops[0][2], len(srcs), ptrs, cfgs, drn.ndc.size))
+
+    # timing on the device stream
+    def event(self) -> int:
+        e = C.c_uint64(0)
+        _lib.check(self._lib.nk_event_create(self.handle, C.byref(e)))
+        return e.value
+
+    def record(self, event: int) -> None:
+        _lib.check(self._lib.nk_event_record(self.handle, event))
+
+    def elapsed_ms(self, start: int, stop: int) -> float:
+        ms = C.c_float(0)
+        _lib.check(self._lib.nk_event_elapsed_ms(self.handle, start, stop, C.byref(ms)))
+        return ms.value

@@ -1,0 +1,290 @@
+"""Expression strings, operation dispatch and reverse-mode wiring for the hot path.
+
+  - ``Function.of("tanh(sig(I[0])*I[1]+I[2])")``: a small parser in the spirit of
+    ``math/parsing/FunctionParser.java``; nested expressions execute operation by operation through
+    temporaries, exactly as ``AbstractDeviceAlgorithm.flatten`` makes the reference do
+    (``backend/api/template/algorithms/AbstractDeviceAlgorithm.java:177-204``).
+  - ``execute(op, inputs)``: ``Operation.execute`` (``backend/api/Operation.java:200-237``): pick the algorithm,
+    prepare the call (allocate the drain), run the HipDevice implementation, record the ADActions.
+  - ``OptimizedFunction``: what ``Device.optimizedFunctionOf`` returns (``devices/Device.java:216-243``): the
+    whole expression as one fused kernel launch (``nk_fused``).
+(paths relative to src/main/java/neureka/ of the reference)
+"""
+from __future__ import annotations
+
+import re
+from typing import List, Optional, Sequence, Union
+
+from . import _lib
+from .backend import (ACTIVATIONS, BiElementwise, BiScalarBroadcast, Broadcast, ExecutionCall, backend,
+                      execute_device_algorithm, execute_on_common_device)
+from .ndim import IllegalArgumentException, IllegalStateException
+from .tensor import GraphNode, Tensor, make_fit
+
+
+def _device_for(inputs: Sequence[Tensor]):
+    """FunctionNode._deviceFor (math/implementations/FunctionNode.java:109-137)."""
+    for t in inputs:
+        if t is not None and t.isOutsourced():
+            return t.getDevice()
+    raise IllegalStateException("none of the operands is stored on a HipDevice; this package has no host arithmetic path")
+
+
+def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = True) -> Tensor:
+    ctx = backend()
+    operation = ctx.getOperation(op_id)
+    device = _device_for(inputs)
+    if len(inputs) > 1 and len({t.rank for t in inputs}) > 1:
+        inputs = make_fit(list(inputs))      # FunctionNode.execute pads ranks first (FunctionNode.java:92-93)
+    call = ExecutionCall(device, operation, list(inputs), d)
+    call.algorithm = operation.getAlgorithmFor(call)
+
+    def run(c: ExecutionCall):
+        c = c.algorithm.prepare(c)
+        for t in c.inputs[1:]:
+            if t.isVirtual() and not isinstance(c.algorithm, BiScalarBroadcast):
+                t.setIsVirtual(False)       # sources are de-virtualised before the kernels (CPUBiElementWise.java:103-104)
+        return execute_device_algorithm(c), c
+
+    result, prepared = execute_on_common_device(call, run)
+    if record and d < 0 and any(t.rqsGradient() or t._node is not None for t in inputs):
+        result._node = _graph_node(op_id, prepared, list(inputs), result)
+    return result
+
+
+# ---- ADActions -------------------------------------------------------------------------------------
+def _graph_node(op_id: str, call: ExecutionCall, inputs: List[Tensor], result: Tensor) -> GraphNode:
+    alg = call.algorithm
+    actions = []
+    for d, parent in enumerate(inputs):
+        if not (parent.rqsGradient() or parent._node is not None):
+            actions.append(None)
+            continue
+        actions.append(_ad_action(op_id, alg, call, inputs, d))
+    return GraphNode(inputs, actions)
+
+
+def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: int):
+    device = call.device
+    prepared_in = call.inputs[1:]            # operands as the kernel saw them (rank-fitted)
+    if op_id == "mul_conv":
+        # linear/Convolution.java:56-89: "I[0] x>> I[1] x>> I[2]" on (error, derivative, zeros like the target);
+        # ConvUtil.executeRecursively rearranges to (zeros, derivative, error) and runs the kernel with d >= 0
+        other = prepared_in[1 - d]
+        target_shape = prepared_in[d].shape
+        def act(error: Tensor) -> Tensor:
+            zeros = Tensor._on_device(device, other.dtype, target_shape)
+            c = ExecutionCall(device, backend().getOperation("inv_convolve_mul_right"), [zeros, other, error], 0)
+            c.algorithm = c.operation.algorithms[0]
+            return execute_on_common_device(c, lambda cc: execute_device_algorithm(cc))
+        return act
+    if op_id == "matMul":
+        # MatMulAlgorithm.java:37-59: d' = (1 + d) % 2 picks the operand to transpose
+        a, b = prepared_in
+        if d == 0:
+            return lambda error: execute("matMul", [error, b.T().deepCopy()], record=False)
+        return lambda error: execute("matMul", [a.T().deepCopy(), error], record=False)
+    if op_id in ACTIVATIONS:
+        src = prepared_in[0]
+        def act(error: Tensor) -> Tensor:
+            local = execute(op_id, [src], d=0, record=False)
+            return execute("multiply", [error, local], record=False)
+        return act
+    broadcasting = isinstance(alg, Broadcast) or (isinstance(alg, BiScalarBroadcast) and prepared_in[0].shape != prepared_in[1].shape)
+    if broadcasting and op_id in ("add", "subtract"):
+        alg = call.operation.getAlgorithm(Broadcast)
+        # operator/Addition.java:90-109 (_autogradBroadcast): the reducing backward kernel on
+        # (zeros like operand d, zeros like the other operand, error)
+        tgt, other = prepared_in[d], prepared_in[1 - d]
+        def act(error: Tensor) -> Tensor:
+            to_be_derived = Tensor._on_device(device, tgt.dtype, tgt.shape)
+            derivative = Tensor._on_device(device, other.dtype, other.shape)
+            c = ExecutionCall(device, call.operation, [to_be_derived, derivative, error], d, alg)
+            return execute_on_common_device(c, lambda cc: execute_device_algorithm(cc))
+        return act
+    if op_id in ("add", "subtract", "multiply", "divide", "modulo", "power"):
+        # default ADAction: error * d f / d operand (FallbackAlgorithm.ADAction); for a broadcast multiply
+        # this keeps the output's shape, as operator/Multiplication.java:55-69 does
+        def act(error: Tensor) -> Tensor:
+            a, b = prepared_in
+            if op_id == "multiply":
+                local = b if d == 0 else a
+            else:
+                c = ExecutionCall(device, call.operation, [None, a, b], d, call.operation.getAlgorithm(BiElementwise))
+                c = c.algorithm.prepare(c)
+                local = execute_on_common_device(c, lambda cc: execute_device_algorithm(cc))
+            return execute("multiply", [error, local], record=False)
+        return act
+    raise IllegalStateException(f"no ADAction for operation '{op_id}'")
+
+
+# ---- expression parsing ---------------------------------------------------------------------------
+class Node:
+    def __init__(self, kind: str, value=None, children: Optional[List["Node"]] = None):
+        self.kind, self.value, self.children = kind, value, children or []    # kind: input | const | fun | op
+
+    def __repr__(self):
+        if self.kind in ("input", "const"):
+            return f"I[{self.value}]" if self.kind == "input" else repr(self.value)
+        if self.kind == "fun":
+            return f"{self.value}({self.children[0]!r})"
+        return f"({self.children[0]!r} {self.value} {self.children[1]!r})"
+
+
+_TOKEN = re.compile(r"\s*(?:(\d+\.\d*(?:[eE][-+]?\d+)?|\d+(?:[eE][-+]?\d+)?)|([iI]\[?\s*\d+\s*\]?)|([A-Za-z_][A-Za-z_0-9]*)|(\*\*|[-+*/%^()@,]))")
+_BIN_OPS = {"+": ("add", 1), "-": ("subtract", 1), "*": ("multiply", 2), "/": ("divide", 2), "%": ("modulo", 2),
+            "x": ("mul_conv", 2), "@": ("matMul", 2), "^": ("power", 3), "**": ("power", 3)}
+
+
+def _tokenize(expr: str) -> List[tuple]:
+    out, pos = [], 0
+    expr = expr.strip()
+    while pos < len(expr):
+        m = _TOKEN.match(expr, pos)
+        if not m:
+            raise IllegalArgumentException(f"cannot parse '{expr}' at position {pos}")
+        num, inp, name, sym = m.groups()
+        if num is not None: out.append(("num", float(num)))
+        elif inp is not None: out.append(("input", int(re.sub(r"\D", "", inp))))
+        elif name is not None: out.append(("name", name))
+        else: out.append(("sym", sym))
+        pos = m.end()
+    return out
+
+
+class _Parser:
+    def __init__(self, tokens): self.t, self.i = tokens, 0
+    def peek(self): return self.t[self.i] if self.i < len(self.t) else (None, None)
+    def next(self): tok = self.peek(); self.i += 1; return tok
+
+    def expr(self, min_prec: int = 1) -> Node:
+        left = self.atom()
+        while True:
+            kind, val = self.peek()
+            sym = val if kind == "sym" else ("x" if (kind, val) == ("name", "x") else None)
+            if sym not in _BIN_OPS or _BIN_OPS[sym][1] < min_prec:
+                return left
+            self.next()
+            op, prec = _BIN_OPS[sym]
+            right = self.expr(prec + 1)
+            left = Node("op", op, [left, right])
+
+    def atom(self) -> Node:
+        kind, val = self.next()
+        if kind == "num": return Node("const", val)
+        if kind == "input": return Node("input", val)
+        if kind == "sym" and val == "(":
+            n = self.expr()
+            if self.next() != ("sym", ")"): raise IllegalArgumentException("missing ')'")
+            return n
+        if kind == "sym" and val == "-":
+            return Node("op", "multiply", [Node("const", -1.0), self.atom()])
+        if kind == "name":
+            if val not in ACTIVATIONS: raise IllegalArgumentException(f"unknown function '{val}'")
+            if self.next() != ("sym", "("): raise IllegalArgumentException(f"'(' expected after {val}")
+            arg = self.expr()
+            if self.next() != ("sym", ")"): raise IllegalArgumentException("missing ')'")
+            return Node("fun", val, [arg])
+        raise IllegalArgumentException(f"unexpected token {val!r}")
+
+
+class Function:
+    """``Function.of(expression)``; calling it executes operation by operation on the operands' device."""
+
+    def __init__(self, expression: str, doAD: bool = True):
+        self.expression = expression
+        self.doAD = doAD
+        p = _Parser(_tokenize(expression))
+        self.root = p.expr()
+        if p.i != len(p.t):
+            raise IllegalArgumentException(f"trailing input in '{expression}'")
+
+    @staticmethod
+    def of(expression: str, doAD: bool = True) -> "Function":
+        return Function(expression, doAD)
+
+    def numberOfArgs(self) -> int:
+        def walk(n): return max([n.value + 1] if n.kind == "input" else [0] + [walk(c) for c in n.children])
+        return walk(self.root)
+
+    def isFlat(self) -> bool:
+        return all(c.kind in ("input", "const") for c in self.root.children)
+
+    def call(self, *inputs: Tensor) -> Tensor:
+        if len(inputs) == 1 and isinstance(inputs[0], (list, tuple)):
+            inputs = tuple(inputs[0])
+        return self._eval(self.root, inputs)
+
+    __call__ = call
+    execute = call
+
+    def _eval(self, n: Node, inputs) -> Union[Tensor, float]:
+        if n.kind == "input":
+            if n.value >= len(inputs):
+                raise IllegalArgumentException(f"function '{self.expression}' needs input {n.value}, {len(inputs)} given")
+            return inputs[n.value]
+        if n.kind == "const":
+            ref = next(t for t in inputs if isinstance(t, Tensor))
+            return Tensor.of(ref.dtype, (1,), n.value)
+        args = [self._eval(c, inputs) for c in n.children]
+        return execute(n.value, args, record=self.doAD)
+
+    def derive(self, inputs: Sequence[Tensor], index: int) -> Tensor:
+        """d f / d I[index] for a flat unary function (``func.derive([t], 0)`` of Calculus_Stress_Test.groovy:255-256)."""
+        if self.root.kind == "fun" and self.root.children[0].kind == "input" and self.root.children[0].value == index:
+            return execute(self.root.value, [inputs[index]], d=0, record=False)
+        raise IllegalArgumentException("derive() is provided for flat activation functions only")
+
+
+class OptimizedFunction:
+    """One fused kernel for a whole elementwise expression (the counterpart of CLFunctionCompiler,
+    devices/opencl/utility/CLFunctionCompiler.java:27-238): the expression tree is lowered to the postfix
+    op-codes of ``nk_fused``; operands must share one shape (views are fine)."""
+
+    def __init__(self, device, function: Function, name: str):
+        self.device, self.function, self.name = device, function, name
+        self.program: List[int] = []
+        self.consts: List[float] = []
+        self._lower(function.root)
+        self.n_src = function.numberOfArgs()
+
+    def _lower(self, n: Node) -> None:
+        if n.kind == "input":
+            self.program += [_lib.FUSE_LOAD, n.value]
+        elif n.kind == "const":
+            if n.value not in self.consts:
+                self.consts.append(n.value)
+            self.program += [_lib.FUSE_CONST, self.consts.index(n.value)]
+        elif n.kind == "fun":
+            self._lower(n.children[0])
+            self.program += [_lib.FUSE_FUN, _lib.FUN[n.value]]
+        else:
+            if n.value not in _lib.OP:
+                raise IllegalArgumentException(f"operator '{n.value}' cannot be fused into an elementwise kernel")
+            self._lower(n.children[0])
+            self._lower(n.children[1])
+            self.program += [_lib.FUSE_BIN, _lib.OP[n.value]]
+
+    def call(self, *inputs: Tensor) -> Tensor:
+        if len(inputs) == 1 and isinstance(inputs[0], (list, tuple)):
+            inputs = tuple(inputs[0])
+        if len(inputs) < self.n_src:
+            raise IllegalArgumentException(f"'{self.name}' needs {self.n_src} inputs, {len(inputs)} given")
+        srcs = list(inputs[: self.n_src])
+        for t in srcs:
+            if t.shape != srcs[0].shape:
+                raise IllegalArgumentException("operands of a fused function must share one shape")
+        guests = [t for t in srcs if not t.isOutsourced()]
+        for t in guests:
+            self.device.store(t)
+        try:
+            for t in srcs:
+                t.setIsVirtual(False)
+            out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
+            self.device.launch_fused(self.program, self.consts, out, srcs)
+            return out
+        finally:
+            for t in guests:
+                self.device.restore(t)
+
+    __call__ = call

@@ -1,0 +1,550 @@
+"""Parity of the HIP path (through the C ABI of libneureka_hip.so) with the CPU oracle, on the same
+seeded inputs.  Bit-exact for + - * and copies (and every kernel that keeps the reference's summation
+order); rtol 1e-5 (f32) / 1e-12 (f64) for transcendental activations; norm-wise 1e-5 / 1e-12 for
+re-ordered reductions.  Every test prints what it is about to run before touching the GPU."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import ATOL, RTOL, assert_bits, assert_close, fill_it, java_array_hash
+from neureka_amd import Function, HipError, IllegalArgumentException, IllegalStateException, Layout, NDConfiguration, Tensor, _lib
+from neureka_amd.tensor import physical_indices
+
+pytestmark = pytest.mark.gpu
+
+F = {"f32": np.float32, "f64": np.float64}
+ACTS = ["abs", "cos", "gasu", "gatu", "gaus", "fast_gaus", "gelu", "idy", "ln", "quad", "relu", "selu", "sig", "silu",
+        "sin", "softplus", "softsign", "tanh", "fast_tanh", "exp", "log10", "sqrt", "cbrt"]
+POSITIVE_ONLY = {"ln", "log10", "sqrt", "cbrt"}
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def on(device, array, shape=None):
+    array = np.asarray(array)
+    return Tensor.of(array.dtype, shape if shape is not None else array.shape, array.reshape(-1)).to(device)
+
+
+def cfg(t):
+    return t.ndc.asInlineArray()
+
+
+# ---- device contract -----------------------------------------------------------------------------------
+def test_memory_roundtrip_fill_and_accounting(device):
+    say("memory roundtrip")
+    before = device.liveBuffers()
+    data = device.allocate(np.float32, 1000)
+    host = np.arange(1000, dtype=np.float32)
+    device._write(data, 0, host)
+    assert (device._read_all(data) == host).all()
+    device._write(data, 10, np.full(5, -1, dtype=np.float32))           # partial write (setItems at an offset)
+    assert (device._read(data, 8, 9) == [8, 9, -1, -1, -1, -1, -1, 15, 16]).all()
+    device._fill(data, 100, 50, 7.5)
+    got = device._read_all(data)
+    assert (got[100:150] == 7.5).all() and got[99] == 99 and got[150] == 150
+    d64 = device.allocateFromOne(np.float64, 33, -0.0)
+    assert np.signbit(device._read_all(d64)).all()
+    assert device.liveBuffers() == before + 2
+    ptr = data.ptr
+    data.release(); d64.release()
+    assert device.liveBuffers() == before
+    with pytest.raises(HipError):                                      # double free is reported, not ignored
+        _lib.check(device._lib.nk_free(device.handle, ptr))
+    with pytest.raises(HipError):                                      # out-of-range transfer is refused on the host
+        small = device.allocate(np.float32, 4)
+        try:
+            device._read(small, 2, 10)
+        finally:
+            small.release()
+
+
+def test_store_restore_free_virtual_and_slices(device):
+    say("device contract")
+    stored, objs = device.numberOfStored(), device.numberOfDataObjects()
+    t = Tensor.of(np.float64, [3, 4], np.arange(12.0))
+    assert not t.isOutsourced() and not device.has(t)
+    t.to(device)
+    assert t.isOutsourced() and device.has(t) and device.numberOfStored() == stored + 1
+    assert (t.items == np.arange(12.0)).all()
+    s = t[1:3, 1:4]                                                      # a slice shares the parent's buffer
+    assert device.has(s) and s._data is t._data and device.numberOfDataObjects() == objs + 1
+    assert (s.items == np.arange(12.0).reshape(3, 4)[1:3, 1:4].reshape(-1)).all()
+    v = Tensor.of(np.float32, [1000, 1000], 4.0).to(device)              # virtual: one element on the device
+    assert v.isVirtual() and v._data.size == 1 and (v.items[:3] == 4.0).all()
+    v.setIsVirtual(False)
+    assert v._data.size == 1000000 and (v.getData() == 4.0).all()
+    device.restore(t)
+    assert not t.isOutsourced() and (t.items == np.arange(12.0)).all()
+    with pytest.raises(IllegalArgumentException):
+        device.restore(t)                                                # OpenCLDevice.java:317-322
+    orphan = Tensor.of(np.float32, [4], [1, 2, 3, 4])
+    child = orphan[1:3]
+    with pytest.raises(IllegalStateException, match="Data parent is not outsourced!"):
+        device.store(child)                                              # AbstractDevice.java:96-97
+    device.free(s); device.free(v)
+    assert device.numberOfStored() == stored and device.numberOfDataObjects() == objs
+
+
+def test_bad_arguments_are_reported(device):
+    say("argument errors")
+    a = on(device, np.ones(8, dtype=np.float32))
+    out = on(device, np.zeros(8, dtype=np.float32))
+    lib, h = device._lib, device.handle
+    c8 = cfg(a)
+    big = NDConfiguration.ofShape([16]).asInlineArray()
+    with pytest.raises(HipError, match="exceeds the buffer"):           # a view larger than its buffer never reaches the GPU
+        _lib.check(lib.nk_activation(h, 0, -1, 0, 1, out._data.ptr, _lib.cfg_ptr(big), a._data.ptr, _lib.cfg_ptr(big), 16))
+    with pytest.raises(HipError, match="n = 5"):
+        _lib.check(lib.nk_activation(h, 0, -1, 0, 1, out._data.ptr, _lib.cfg_ptr(c8), a._data.ptr, _lib.cfg_ptr(c8), 5))
+    with pytest.raises(HipError, match="unknown function id"):
+        _lib.check(lib.nk_activation(h, 99, -1, 0, 1, out._data.ptr, _lib.cfg_ptr(c8), a._data.ptr, _lib.cfg_ptr(c8), 8))
+    with pytest.raises(HipError, match="rank"):
+        _lib.check(lib.nk_activation(h, 0, -1, 0, 9, out._data.ptr, _lib.cfg_ptr(c8), a._data.ptr, _lib.cfg_ptr(c8), 8))
+    with pytest.raises(HipError, match="unknown device handle"):
+        _lib.check(lib.nk_device_sync(987654))
+
+
+# ---- elementwise family --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("n", [1, 5, 7907, 1 << 16])
+def test_binary_elementwise_bit_exact(device, orc, dt, n):
+    say("elementwise", dt, n)
+    rng = np.random.default_rng(n)
+    a = rng.uniform(-1, 1, n).astype(F[dt]); b = rng.uniform(-1, 1, n).astype(F[dt])
+    ta, tb = on(device, a), on(device, b)
+    c = orc.dense_cfg([n])
+    for op in ("add", "subtract", "multiply", "divide", "modulo"):
+        for d in (-1, 0, 1):
+            out = on(device, np.zeros(n, dtype=F[dt]))
+            device.launch_elementwise(op, d, out, ta, tb)
+            want = orc.elementwise(op, d, np.zeros(n, dtype=F[dt]), c, a, c, b, c)
+            if op in ("add", "subtract", "multiply") or d < 0 or (d == 0):
+                assert_bits(out.getData(), want, f"{op} d={d}")
+            else:
+                assert_close(out.getData(), want, f"{op} d={d}")
+    out = on(device, np.zeros(n, dtype=F[dt]))
+    ap = np.abs(a) + 0.5
+    device.launch_elementwise("power", -1, out, on(device, ap), tb)
+    assert_close(out.getData(), orc.elementwise("power", -1, np.zeros(n, dtype=F[dt]), c, ap, c, b, c), "power")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_all_activations_and_derivatives(device, orc, dt):
+    n = 7907
+    x = orc.seeded(F[dt], n, "Tempeh")
+    x = np.where(np.abs(x) < 1e-3, F[dt](0.25), x)          # the reference's 2/(1+e^-2x)-1 loses relative accuracy at 0
+    c = orc.dense_cfg([n])
+    for name in ACTS:
+        xi = (np.abs(x) + F[dt](0.01)).astype(F[dt]) if name in POSITIVE_ONLY else x
+        tx = on(device, xi)
+        for d in (-1, 0):
+            say("activation", name, d, dt)
+            out = on(device, np.zeros(n, dtype=F[dt]))
+            device.launch_activation(name, d, out, tx)
+            want = orc.activation(name, d, np.zeros(n, dtype=F[dt]), c, xi, c)
+            got = out.getData()
+            if dt == "f32" and name in ("abs", "idy", "quad", "relu", "fast_gaus", "softsign", "gasu", "fast_tanh") and (d < 0 or name != "fast_tanh"):
+                assert_bits(got, want, f"{name} d={d}")     # pure float arithmetic in the reference: identical
+            else:
+                assert_close(got, want, f"{name} d={d}")
+
+
+def test_activation_golden_vectors_on_device(device, orc, golden):
+    g = golden["activation_vectors"]
+    for row in g["rows"]:
+        say("golden activation", row["fun"], row["derive"], row["type"])
+        dt = F[row["type"]]
+        x = orc.seeded(dt, g["size"], g["seed"])
+        fn = Function.of(f"{row['fun']}(I[0])")
+        t = on(device, x)
+        res = fn.derive([t], 0) if row["derive"] else fn(t)
+        assert_close(res.items, np.array(row["expected"], dtype=dt), str(row))
+        # the same through a slice of a larger tensor, as the reference test does (t2 = zeros(5)[1..3])
+        big = on(device, np.zeros(5, dtype=dt))
+        sl = big[1:4]
+        sl.setItems(x)
+        res2 = fn.derive([sl], 0) if row["derive"] else fn(sl)
+        assert_close(res2.items, np.array(row["expected"], dtype=dt), str(row) + " (slice)")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_scalarization_and_fill(device, orc, dt):
+    say("scalarization", dt)
+    n = 4099
+    rng = np.random.default_rng(4)
+    a = rng.uniform(-2, 2, n).astype(F[dt])
+    ta = on(device, a)
+    c = orc.dense_cfg([n])
+    for op, val in (("add", 0.1), ("subtract", 3.0), ("multiply", 100.0), ("divide", 3.0), ("modulo", 0.7), ("idy", -2.5)):
+        out = on(device, np.zeros(n, dtype=F[dt]))
+        device.launch_scalarization(op, -1, out, ta, val)
+        assert_bits(out.getData(), orc.scalarization(op, -1, np.zeros(n, dtype=F[dt]), c, a, c, val), op)
+    out = on(device, np.zeros(n, dtype=F[dt]))
+    device.launch_scalarization("power", -1, out, on(device, np.abs(a) + 0.5), 2.5)
+    assert_close(out.getData(), orc.scalarization("power", -1, np.zeros(n, dtype=F[dt]), c, np.abs(a) + F[dt](0.5), c, 2.5), "power")
+    # fill through a strided view: only the viewed elements change
+    base = on(device, np.zeros((6, 8), dtype=F[dt]))
+    view = base[1:6:2, 2:7]
+    device.launch_scalar_fill(view, 0.1)
+    want = np.zeros(48, dtype=F[dt])
+    orc.scalar_fill(want, cfg(view), 0.1)
+    assert_bits(base.getData(), want, "fill view")
+    assert np.count_nonzero(want) == 15
+
+
+VIEWS = {
+    "permuted": lambda t: t.T(),
+    "sliced": lambda t: t[::2, 1:t.shape[1] // 2 + 1],
+    "sliced_rows": lambda t: t[1:t.shape[0] - 1, :],
+    "perm3": None,
+}
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_views_take_the_fast_paths_and_match(device, orc, dt):
+    """Non-contiguous NDConfigurations: transposed, strided-slice and row-band views as sources, a dense
+    drain; bit-exact against the oracle walking the same descriptors; the kernel path is asserted."""
+    rng = np.random.default_rng(8)
+    R, Cc = 70, 130
+    base_a = rng.uniform(-1, 1, (R, Cc)).astype(F[dt]); base_b = rng.uniform(-1, 1, (R, Cc)).astype(F[dt])
+    ta, tb = on(device, base_a), on(device, base_b)
+    for name, expect_path in (("permuted", "tile_transpose"), ("sliced", "rows"), ("sliced_rows", "rows")):
+        say("view", name, dt)
+        va, vb = VIEWS[name](ta), VIEWS[name](tb)
+        out = Tensor._on_device(device, F[dt], va.shape)
+        device.launch_elementwise("multiply", -1, out, va, vb)
+        assert _lib.last_path().startswith(expect_path), (name, _lib.last_path())
+        want = orc.elementwise("multiply", -1, np.zeros(out.size, dtype=F[dt]), cfg(out), base_a.reshape(-1), cfg(va), base_b.reshape(-1), cfg(vb))
+        assert_bits(out.getData(), want, name)
+        # one view, one dense operand; and a view as the DRAIN
+        dense = on(device, rng.uniform(-1, 1, va.shape).astype(F[dt]))
+        device.launch_elementwise("add", -1, out, va, dense)
+        want = orc.elementwise("add", -1, np.zeros(out.size, dtype=F[dt]), cfg(out), base_a.reshape(-1), cfg(va), dense.getData(), cfg(dense))
+        assert_bits(out.getData(), want, name + " mixed")
+        target = on(device, np.zeros((R, Cc), dtype=F[dt]))
+        vt = VIEWS[name](target)
+        device.launch_activation("idy", -1, vt, dense)
+        want = orc.activation("idy", -1, np.zeros(R * Cc, dtype=F[dt]), cfg(vt), dense.getData(), cfg(dense))
+        assert_bits(target.getData(), want, name + " as drain")
+    # rank 3 permutation with the contiguous axis moved to the front
+    say("view perm3", dt)
+    b3 = rng.uniform(-1, 1, (9, 20, 33)).astype(F[dt])
+    t3 = on(device, b3)
+    v3 = t3.permute(2, 0, 1)
+    out = Tensor._on_device(device, F[dt], v3.shape)
+    device.launch_activation("quad", -1, out, v3)
+    assert_bits(out.getData(), orc.activation("quad", -1, np.zeros(out.size, dtype=F[dt]), cfg(out), b3.reshape(-1), cfg(v3)), "perm3")
+
+
+def test_exotic_descriptor_falls_back_to_the_literal_formula(device, orc):
+    """A descriptor whose indicesMap is not the row-major one (row 10 of NDConfiguration_Spec: strides
+    [81,42], indicesMap [3,99]) cannot be canonicalised: the literal kernel must agree with the oracle."""
+    say("literal fallback")
+    ndc = NDConfiguration.of([2, 3], [3, 1], [3, 2], [1, 1], [0, 0])        # flat 2 -> (0, 1)! (2 % 3 = 2, 2 // 2 = 1)
+    src = np.arange(1, 13, dtype=np.float32)
+    tsrc = on(device, src)
+    weird = Tensor(np.float32, ndc, None); weird._set_data(tsrc._data, device)
+    out = on(device, np.zeros(6, dtype=np.float32))
+    dense6 = on(device, np.arange(6, dtype=np.float32))
+    device.launch_elementwise("add", -1, out, weird, dense6)
+    assert _lib.last_path() == "literal"
+    c6 = orc.dense_cfg([2, 3])
+    want = orc.elementwise("add", -1, np.zeros(6, dtype=np.float32), c6, src, ndc.asInlineArray(), dense6.getData(), c6)
+    assert_bits(out.getData(), want, "literal")
+    # virtual source: all-zero tables address element 0
+    virt = Tensor.of(np.float32, [2, 3], 2.5).to(device)
+    device.launch_elementwise("multiply", -1, out, virt, dense6)
+    assert_bits(out.getData(), dense6.getData() * np.float32(2.5), "virtual")
+
+
+# ---- broadcast ----------------------------------------------------------------------------------------------
+def test_broadcast_forward_golden_on_device(device, golden):
+    g = golden["broadcast_stress"]
+    for row in g["rows"]:
+        say("golden broadcast", row["op"], row["shape1"], row["shape2"])
+        a = Tensor.of(np.float64, row["shape1"], g["t1_range"]).to(device)
+        b = Tensor.of(np.float64, row["shape2"], g["t2_range"]).to(device)
+        fn = {"modulo": lambda x, y: x % y, "multiply": lambda x, y: x * y, "add": lambda x, y: x + y,
+              "subtract": lambda x, y: x - y, "divide": lambda x, y: x / y}[row["op"]]
+        out = fn(a, b)
+        assert list(out.shape) == row["shape"]
+        def fmt(v):
+            if np.isnan(v): return "NaN"
+            if np.isinf(v): return "-inf" if v < 0 else "inf"
+            r = round(float(v), 5)
+            return repr(r) if r != 0 else ("-0.0" if np.signbit(v) else "0.0")
+        assert [fmt(v) for v in out.items] == row["expected"], row
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_broadcast_forward_bit_exact(device, orc, dt):
+    rng = np.random.default_rng(21)
+    cases = [([64, 1, 96], [1, 40, 96]), ([1, 40, 1], [64, 40, 96]), ([33, 1], [1, 77]), ([5, 6, 7], [5, 6, 7]),
+             ([3, 1, 5, 1], [1, 4, 1, 6]), ([1], [1]), ([128, 1, 4], [1, 9, 4])]
+    for s1, s2 in cases:
+        say("broadcast fwd", s1, s2, dt)
+        so = [q if p == 1 else p for p, q in zip(s1, s2)]
+        a = rng.uniform(-1, 1, s1).astype(F[dt]); b = rng.uniform(-1, 1, s2).astype(F[dt])
+        ta, tb = on(device, a), on(device, b)
+        for op, f in (("add", np.add), ("subtract", np.subtract), ("multiply", np.multiply)):
+            out = Tensor._on_device(device, F[dt], so)
+            device.launch_broadcast(op, -1, out, ta, tb)
+            want = orc.broadcast(op, -1, np.zeros(out.size, dtype=F[dt]), orc.dense_cfg(so), a.reshape(-1), orc.dense_cfg(s1), b.reshape(-1), orc.dense_cfg(s2))
+            assert_bits(out.getData(), want, f"{op} {s1} {s2}")
+            assert_bits(out.getData().reshape(so), f(a, b), f"{op} numpy")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_broadcast_backward_bit_exact(device, orc, dt):
+    rng = np.random.default_rng(22)
+    full = [6, 5, 7]
+    e = rng.uniform(-1, 1, full).astype(F[dt])
+    te = on(device, e)
+    for tgt in ([6, 1, 7], [1, 5, 1], [1, 1, 1], [6, 5, 7], [6, 5, 1]):
+        for op in ("add", "subtract", "multiply"):
+            for d in (0, 1):
+                say("broadcast bwd", tgt, op, d, dt)
+                other = rng.uniform(-1, 1, full).astype(F[dt]) if op == "multiply" else np.zeros(full, dtype=F[dt])
+                tother = on(device, other)
+                drn = Tensor._on_device(device, F[dt], tgt)
+                device.launch_broadcast(op, d, drn, tother, te)
+                want = orc.broadcast(op, d, np.zeros(drn.size, dtype=F[dt]), orc.dense_cfg(tgt), other.reshape(-1), orc.dense_cfg(full), e.reshape(-1), orc.dense_cfg(full))
+                assert_bits(drn.getData(), want, f"{tgt} {op} {d}")
+
+
+def test_broadcast_autograd_golden(device, golden):
+    g = golden["broadcast_autograd"]
+    for row in g["rows"]:
+        for dt in (np.float64, np.float32):
+            say("golden broadcast autograd", row, dt.__name__)
+            a = Tensor.of(dt, g["a"]["shape"], g["a"]["data"]).setRqsGradient(row["which_grad"] == "a").to(device)
+            b = Tensor.of(dt, row["b_shape"], g["b_range"]).setRqsGradient(row["which_grad"] == "b").to(device)
+            c = {"a+b": lambda: a + b, "a*b": lambda: a * b, "a-b": lambda: a - b, "b-a": lambda: b - a}[row["op"]]()
+            assert c.items.tolist() == [float(v) for v in row["c"]]
+            c.backward(Tensor.of(dt, [2, 2], g["error"]))
+            w = a if row["which_grad"] == "a" else b
+            assert w.gradient.items.tolist() == [float(v) for v in row["gradient"]], row
+
+
+# ---- fused expressions -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_fused_chain_equals_unfused_and_oracle(device, orc, dt):
+    """tanh(sig(a)*b+c): the fused kernel, the four-kernel sequence the reference runs, and the oracle.
+    Contiguous operands, a permuted view and a strided slice."""
+    rng = np.random.default_rng(31)
+    R, Cc = 96, 200
+    fn = Function.of("tanh(sig(I[0])*I[1]+I[2])")
+    fused = device.optimizedFunctionOf(fn, "chain")
+    bases = [rng.standard_normal((R, Cc)).astype(F[dt]) for _ in range(3)]
+    tens = [on(device, b) for b in bases]
+    for name, view in (("contiguous", lambda t: t), ("permuted", lambda t: t.T()), ("sliced", lambda t: t[::2, 1:101])):
+        say("fused chain", name, dt)
+        vs = [view(t) for t in tens]
+        got_fused = fused(*vs)
+        path = _lib.last_path()
+        got_unfused = fn(*vs)
+        n = vs[0].size
+        oc = orc.dense_cfg(list(vs[0].shape))
+        s = orc.activation("sig", -1, np.zeros(n, dtype=F[dt]), oc, bases[0].reshape(-1), cfg(vs[0]))
+        m = orc.elementwise("multiply", -1, np.zeros(n, dtype=F[dt]), oc, s, oc, bases[1].reshape(-1), cfg(vs[1]))
+        p = orc.elementwise("add", -1, np.zeros(n, dtype=F[dt]), oc, m, oc, bases[2].reshape(-1), cfg(vs[2]))
+        want = orc.activation("tanh", -1, np.zeros(n, dtype=F[dt]), oc, p, oc)
+        assert_close(got_fused.items, want, f"fused {name}")
+        assert_close(got_unfused.items, want, f"unfused {name}")
+        assert_bits(got_fused.items, got_unfused.items, f"fused vs unfused {name}")   # same roundings, same kernels' maths
+        assert path.startswith({"contiguous": "rows", "permuted": "tile_transpose", "sliced": "rows"}[name]), path
+    # nested right operands exercise the saved-intermediate stack of the fused program
+    say("fused nested", dt)
+    f2 = Function.of("(I[0]*I[1]) + (I[1]-I[2]) * (I[2] / (I[0]*I[0] + 2))")
+    assert_bits(device.optimizedFunctionOf(f2, "nested")(*tens).items, f2(*tens).items, "nested")
+    if dt == "f64":
+        x, y, z = bases
+        assert_close(f2(*tens).items, ((x * y) + (y - z) * (z / (x * x + 2))).reshape(-1), "nested vs numpy")
+
+
+# ---- convolution ----------------------------------------------------------------------------------------------
+def test_convolution_golden_on_device(device, golden):
+    for row in golden["convolution_forward"]["rows"]:
+        for dt in (np.float32, np.float64):
+            say("golden conv", row["x_shape"], row["k_shape"], dt.__name__)
+            x = Tensor.of(dt, row["x_shape"], row["x"]).to(device)
+            k = Tensor.of(dt, row["k_shape"], row["k"]).to(device)
+            y = x.conv(k)
+            assert list(y.shape) == row["y_shape"] and y.items.tolist() == [float(v) for v in row["y"]], row
+            y2 = Function.of("I[0] x I[1]")(x, k)
+            assert y2.items.tolist() == [float(v) for v in row["y"]]
+
+
+def test_convolution_autograd_golden_graph(device, golden):
+    g = golden["convolution_autograd"]
+    say("golden conv autograd")
+    f8 = np.float64
+    i_a = Tensor.of(f8, g["i_a"]["shape"], g["i_a"]["data"]).to(device)
+    w_a = Tensor.of(f8, g["w_a"]["shape"], g["w_a"]["data"]).setRqsGradient(True).to(device)
+    w_b = Tensor.of(f8, g["w_b"]["shape"], g["w_b"]["data"]).setRqsGradient(True).to(device)
+    w_c = Tensor.of(f8, g["w_c"]["shape"], g["w_c"]["data"]).setRqsGradient(True).to(device)
+    o_a = i_a.conv(w_a); o_b = o_a.conv(w_b); o_c = o_a.conv(w_c)
+    out = o_b * o_c
+    assert o_a.items.tolist() == g["o_a"] and o_b.items.tolist() == g["o_b"] and o_c.items.tolist() == g["o_c"]
+    assert out.items.tolist() == g["out"]
+    out.backward(Tensor.of(f8, g["backward_error"]["shape"], g["backward_error"]["value"]))
+    assert w_b.gradient.items.tolist() == g["w_b_gradient"]
+    w_a.applyGradient()
+    assert w_a.items.tolist() == g["w_a_after_apply"]
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_convolution_literal_kernels_bit_exact(device, orc, dt):
+    """Any rank, either operand order, dense and viewed operands: the literal kernels keep the reference's
+    summation order and are bit-identical to the oracle's state machines."""
+    rng = np.random.default_rng(41)
+    cases = [([9], [4]), ([12, 11], [3, 4]), ([3, 4], [12, 11]), ([3, 9, 8], [3, 2, 3]), ([2, 6, 6], [1, 3, 3]),
+             ([2, 3, 1], [1, 3, 2]), ([2, 3, 5, 4], [2, 3, 2, 2])]
+    for xs, ks in cases:
+        say("conv literal", xs, ks, dt)
+        ys = [abs(p - q) + 1 for p, q in zip(xs, ks)]
+        x = rng.uniform(-1, 1, xs).astype(F[dt]); k = rng.uniform(-1, 1, ks).astype(F[dt]); e = rng.uniform(-1, 1, ys).astype(F[dt])
+        tx, tk, te = on(device, x), on(device, k), on(device, e)
+        out = Tensor._on_device(device, F[dt], ys)
+        device.launch_convolution(-1, out, tx, tk)
+        want = orc.convolve(np.zeros(out.size, dtype=F[dt]), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
+        assert_bits(out.getData(), want, f"fwd {xs} {ks}")
+        for tgt, tgt_shape, other, other_arr, other_shape in ((tx, xs, tk, k, ks), (tk, ks, tx, x, xs)):
+            drn = Tensor._on_device(device, F[dt], tgt_shape)
+            device.launch_convolution(0, drn, other, te)
+            want = orc.deconvolve(np.zeros(drn.size, dtype=F[dt]), orc.dense_cfg(tgt_shape), other_arr.reshape(-1), orc.dense_cfg(other_shape), e.reshape(-1), orc.dense_cfg(ys))
+            assert_bits(drn.getData(), want, f"bwd {tgt_shape} {other_shape}")
+    say("conv literal on a transposed operand", dt)
+    x = rng.uniform(-1, 1, (8, 10)).astype(F[dt]); k = rng.uniform(-1, 1, (3, 3)).astype(F[dt])
+    tx, tk = on(device, x), on(device, k)
+    vx = tx.T()
+    out = Tensor._on_device(device, F[dt], [8, 6])
+    device.launch_convolution(-1, out, vx, tk)
+    want = orc.convolve(np.zeros(48, dtype=F[dt]), orc.dense_cfg([8, 6]), x.reshape(-1), cfg(vx), k.reshape(-1), orc.dense_cfg([3, 3]))
+    assert_bits(out.getData(), want, "transposed operand")
+
+
+def _abs_bound(orc, xs, ks, x, k, dt):
+    ys = [abs(p - q) + 1 for p, q in zip(xs, ks)]
+    return orc.convolve(np.zeros(int(np.prod(ys))), orc.dense_cfg(ys), np.abs(x).astype(np.float64).reshape(-1), orc.dense_cfg(xs),
+                        np.abs(k).astype(np.float64).reshape(-1), orc.dense_cfg(ks))
+
+
+@pytest.mark.parametrize("shape", [([8, 40, 70], [8, 5, 5]), ([6, 33, 65], [6, 3, 3]), ([5, 20, 21], [5, 4, 2]), ([64, 64, 64], [64, 5, 5])])
+def test_channel_convolution_fast_paths(device, orc, shape):
+    """[C,H,W] x [C,kh,kw] forward and both gradients on the LDS-tiled kernels: re-ordered f32 sums, compared
+    norm-wise: |delta| <= 1e-5 * sum|a||b| per output."""
+    xs, ks = shape
+    ys = [1, xs[1] - ks[1] + 1, xs[2] - ks[2] + 1]
+    rng = np.random.default_rng(43)
+    x = (rng.standard_normal(xs) * 0.1).astype(np.float32); k = (rng.standard_normal(ks) * 0.1).astype(np.float32)
+    e = rng.standard_normal(ys).astype(np.float32)
+    tx, tk, te = on(device, x), on(device, k), on(device, e)
+    say("chan_fwd", xs, ks)
+    out = Tensor._on_device(device, np.float32, ys)
+    device.launch_convolution(-1, out, tx, tk)
+    assert _lib.last_path() == "chan_fwd"
+    want = orc.convolve(np.zeros(out.size, dtype=np.float32), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
+    bound = RTOL[np.dtype(np.float32)] * _abs_bound(orc, xs, ks, x, k, np.float32) + 1e-30
+    assert (np.abs(out.getData().astype(np.float64) - want) <= bound).all(), "chan_fwd"
+    out2 = Tensor._on_device(device, np.float32, ys)
+    device.launch_convolution(-1, out2, tk, tx)                       # kernel first
+    assert _lib.last_path() == "chan_fwd"
+    assert_bits(out2.getData(), out.getData(), "operand order")
+    say("chan_dx", xs, ks)
+    dx = Tensor._on_device(device, np.float32, xs)
+    device.launch_convolution(0, dx, tk, te)
+    assert _lib.last_path() == "chan_dx"
+    want = orc.deconvolve(np.zeros(dx.size, dtype=np.float32), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks), e.reshape(-1), orc.dense_cfg(ys), fast=True)
+    babs = orc.deconvolve(np.zeros(dx.size), orc.dense_cfg(xs), np.abs(k).astype(np.float64).reshape(-1), orc.dense_cfg(ks), np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
+    assert (np.abs(dx.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dx"
+    say("chan_dk", xs, ks)
+    dk = Tensor._on_device(device, np.float32, ks)
+    device.launch_convolution(0, dk, tx, te)
+    assert _lib.last_path() == "chan_dk"
+    want = orc.deconvolve(np.zeros(dk.size, dtype=np.float32), orc.dense_cfg(ks), x.reshape(-1), orc.dense_cfg(xs), e.reshape(-1), orc.dense_cfg(ys), fast=True)
+    babs = orc.deconvolve(np.zeros(dk.size), orc.dense_cfg(ks), np.abs(x).astype(np.float64).reshape(-1), orc.dense_cfg(xs), np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
+    assert (np.abs(dk.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dk"
+
+
+def test_conv2d_config1_shape(device, orc):
+    """[64,64] x [3,3] -> [62,62] (the reference runs this on SimpleCPUConvolution: ky outer, kx inner)."""
+    say("conv2d 64x64 x 3x3")
+    rng = np.random.default_rng(1)
+    x = rng.uniform(-1, 1, (64, 64)).astype(np.float32); k = rng.uniform(-1, 1, (3, 3)).astype(np.float32)
+    y = on(device, x).conv(on(device, k))
+    assert y.shape == (62, 62)
+    want = orc.simple_conv2d(x.reshape(-1), k.reshape(-1), 64, 64, 3, 3)
+    bound = 1e-5 * orc.simple_conv2d(np.abs(x).reshape(-1), np.abs(k).reshape(-1), 64, 64, 3, 3)
+    assert (np.abs(y.items - want) <= bound).all()
+
+
+# ---- matmul ---------------------------------------------------------------------------------------------------
+def test_matmul_hash_known_answers_on_device(device, golden):
+    g = golden["matmul_hashes"]
+    for rows, rm in ((g["row_major"], True), (g["column_major"], False), (g["column_major_large"], False)):
+        for M, K, N, want in rows:
+            for dt in (np.float32, np.float64):
+                say("golden matmul", M, K, N, "RM" if rm else "CM", dt.__name__)
+                A, B = on(device, fill_it(M * K, 43, dt)), on(device, fill_it(K * N, 87, dt))
+                Cm = on(device, np.zeros(M * N, dtype=dt))
+                device.launch_matmul(rm, M, K, N, A, B, Cm)
+                assert java_array_hash(Cm.getData()) == want, (M, K, N, rm, dt)
+
+
+def test_matmul_simple_kernel_bit_exact(device, orc):
+    rng = np.random.default_rng(51)
+    for M, K, N in ((17, 23, 13), (1, 64, 1), (70, 5, 129)):
+        for dt in (np.float32, np.float64):
+            for rm in (True, False):
+                say("matmul simple", M, K, N, dt.__name__, rm)
+                A = rng.uniform(-1, 1, M * K).astype(dt); B = rng.uniform(-1, 1, K * N).astype(dt); C0 = rng.uniform(-1, 1, M * N).astype(dt)
+                tc = on(device, C0)
+                device.launch_matmul(rm, M, K, N, on(device, A), on(device, B), tc)
+                assert _lib.last_path() == "simple"
+                assert_bits(tc.getData(), orc.gemm(rm, A, B, M, K, N, C_init=C0.copy()), "simple")
+
+
+@pytest.mark.parametrize("mkn", [(128, 32, 128), (256, 96, 128), (384, 256, 512), (1024, 256, 256)])
+def test_matmul_mfma_path(device, orc, mkn):
+    """The MFMA kernel: exact on integer-valued data (any correct GEMM is), norm-wise 1e-5 on uniform
+    data, accumulation into C, both layouts."""
+    M, K, N = mkn
+    rng = np.random.default_rng(52)
+    say("matmul mfma integer", mkn)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float32); B = rng.integers(-5, 6, (K, N)).astype(np.float32)
+    C0 = rng.integers(-9, 10, (M, N)).astype(np.float32)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == "mfma"
+    assert (tc.getData().reshape(M, N) == (A.astype(np.float64) @ B.astype(np.float64) + C0)).all()
+    say("matmul mfma column major", mkn)
+    tc = on(device, np.zeros((M, N), dtype=np.float32))
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)      # CM storage of A, B
+    assert (tc.getData().reshape(N, M).T == A.astype(np.float64) @ B.astype(np.float64)).all()
+    say("matmul mfma uniform", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    tc = on(device, np.zeros((M, N), dtype=np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
+def test_matmul_through_the_tensor_api(device):
+    """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
+    say("matmul tensor api")
+    rng = np.random.default_rng(53)
+    a = rng.integers(-4, 5, (6, 9)).astype(np.float64); b = rng.integers(-4, 5, (9, 5)).astype(np.float64)
+    ta, tb = on(device, a).setRqsGradient(True), on(device, b).setRqsGradient(True)
+    c = ta.matMul(tb)
+    assert (c.items.reshape(6, 5) == a @ b).all()
+    assert (on(device, a.T.copy()).T().matMul(tb).items.reshape(6, 5) == a @ b).all()        # a CM view of A
+    big = on(device, np.pad(a, ((1, 1), (2, 2))))
+    assert (big[1:7, 2:11].matMul(tb).items.reshape(6, 5) == a @ b).all()                    # partial slice -> cloned
+    e = rng.integers(-3, 4, (6, 5)).astype(np.float64)
+    c.backward(on(device, e))
+    assert (ta.gradient.items.reshape(6, 9) == e @ b.T).all() and (tb.gradient.items.reshape(9, 5) == a.T @ e).all()

@@ -1,0 +1,119 @@
+"""CPU-only tests of the host-side mirror: view descriptors, the expression parser, the C ABI surface
+(library loads, every declared symbol is exported).  No compute calls, no GPU."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from neureka_amd import IllegalArgumentException, IllegalStateException, Layout, NDConfiguration, _lib
+from neureka_amd.function import Function, OptimizedFunction
+from neureka_amd.tensor import Tensor, physical_indices
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "neureka_hip.h")).read()
+    declared = set(re.findall(r"\b(nk_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    missing = [name for name in sorted(declared) if not hasattr(lib, name)]
+    assert not missing, f"declared in include/neureka_hip.h but not exported: {missing}"
+    assert declared == set(_lib.SYMBOLS), "the ctypes table and the header disagree"
+    _lib.load()
+
+
+def test_specialised_class_choice_matches_ndconfiguration_spec(golden):
+    for shape, strides, imap, spread, offset, expected in golden["ndconfiguration_spec"]["rows"]:
+        ndc = NDConfiguration.of(shape, strides, imap, spread, offset)
+        assert ndc.kind() == expected, (shape, strides, imap, spread, offset)
+        inline = ndc.asInlineArray().tolist()
+        assert inline == shape + strides + imap + offset + spread      # device order: offset before spread
+
+
+def test_index_maths_matches_oracle(golden, orc):
+    for shape, strides, imap, spread, offset, _ in golden["ndconfiguration_spec"]["rows"]:
+        ndc = NDConfiguration.of(shape, strides, imap, spread, offset)
+        phys = physical_indices(ndc)
+        for i in range(ndc.size):
+            assert ndc.indexOfIndex(i) == orc.index_of_index(ndc.asInlineArray(), i) == phys[i]
+
+
+def test_construct_rejects_what_the_reference_rejects():
+    with pytest.raises(IllegalStateException):
+        NDConfiguration.of([2, 0], [1, 1], [1, 1], [1, 1], [0, 0])
+    with pytest.raises(IllegalStateException):
+        NDConfiguration.of([1, 3], [3, 1], [3, 1], [2, 1], [0, 0])     # step > 1 on an axis of extent 1
+
+
+def test_layouts():
+    assert Layout.ROW_MAJOR.newStridesFor([2, 3, 4]) == (12, 4, 1)
+    assert Layout.COLUMN_MAJOR.newStridesFor([3, 4]) == (1, 3)
+    # rank 3: only the two innermost axes trade places in the fill order (NDConfiguration.java:114-119)
+    assert Layout.COLUMN_MAJOR.newStridesFor([2, 3, 4]) == (12, 1, 3)
+    assert NDConfiguration.ofShape([3, 4]).getLayout() is Layout.ROW_MAJOR
+    assert NDConfiguration.ofShape([3, 4], Layout.COLUMN_MAJOR).getLayout() is Layout.COLUMN_MAJOR
+    assert NDConfiguration.ofShape([1, 1]).getLayout() is Layout.SYMMETRIC
+    assert NDConfiguration.ofShape([3, 4]).isSimple()
+    assert not NDConfiguration.ofShape([3, 4]).newReshaped([1, 0]).isSimple()
+    assert Layout.SYMMETRIC.isCompatible(Layout.COLUMN_MAJOR) and not Layout.ROW_MAJOR.isCompatible(Layout.COLUMN_MAJOR)
+    assert not Layout.UNSPECIFIC.isCompatible(Layout.UNSPECIFIC)
+
+
+def test_views_of_the_benchmark_configs():
+    """The descriptors the north-star configs name."""
+    t = NDConfiguration.ofShape([16384, 4096]).newReshaped([1, 0])
+    assert (t.shape, t.strides, t.indicesMap, t.spread, t.offset) == ((4096, 16384), (1, 4096), (16384, 1), (1, 1), (0, 0))
+    assert t.kind() == "Permuted2DConfiguration" and t.getLayout() is Layout.COLUMN_MAJOR   # a transposed RM matrix IS a CM matrix (NDConfiguration.java:157-173)
+    s = NDConfiguration.ofShape([8192, 16384]).sliced([4096, 8192], [0, 1], [2, 1])
+    assert (s.shape, s.strides, s.indicesMap, s.spread, s.offset) == ((4096, 8192), (16384, 1), (8192, 1), (2, 1), (0, 1))
+    assert s.kind() == "Sliced2DConfiguration"
+    v = NDConfiguration.virtualOf([3, 4])
+    assert v.asInlineArray().tolist() == [3, 4] + [0] * 8 and v.indexOfIndex(7) == 0
+
+
+def test_views_against_numpy():
+    base = np.arange(6 * 5 * 4, dtype=np.float32)
+    t = Tensor.of(np.float32, [6, 5, 4], base)
+    assert (t.T().items == base.reshape(6, 5, 4).transpose(2, 1, 0).reshape(-1)).all()
+    assert (t.permute(1, 0, 2).items == base.reshape(6, 5, 4).transpose(1, 0, 2).reshape(-1)).all()
+    sl = t[1:6:2, 2:5, 3]
+    assert sl.shape == (3, 3, 1)
+    assert (sl.items == base.reshape(6, 5, 4)[1:6:2, 2:5, 3:4].reshape(-1)).all()
+    # slice of a transposed view: the offsets and steps travel with their axes (SimpleReshapeView)
+    st = t[1:3, 0:5, 0:4].T()
+    assert (st.items == base.reshape(6, 5, 4)[1:3].transpose(2, 1, 0).reshape(-1)).all()
+    with pytest.raises(IllegalArgumentException):
+        t[0:0, 0:5, 0:4]
+
+
+def test_slice_then_transpose_matches_reference_string():
+    """Tensor_Slice_Permute_Spec: A = [6,8] range, A[1..3, 4..5].T() starts at physical offsets 12, 20, 28, 13."""
+    a = Tensor.of(np.float64, [6, 8], np.arange(48))
+    v = a[1:4, 4:6].T()
+    assert physical_indices(v.ndc).tolist()[:4] == [12, 20, 28, 13]
+
+
+def test_parser_and_fused_lowering():
+    f = Function.of("tanh(sig(I[0])*I[1]+I[2])")
+    assert repr(f.root) == "tanh(((sig(I[0]) multiply I[1]) add I[2]))"
+    assert f.numberOfArgs() == 3 and not f.isFlat()
+    assert Function.of("I[0] x I[1]").root.value == "mul_conv"
+    assert Function.of("i0 @ i1").root.value == "matMul"
+    assert repr(Function.of("gaus(i0)*100 % i0").root) == "((gaus(I[0]) multiply 100.0) modulo I[0])"
+    assert repr(Function.of("i0+i1*i2").root) == "(I[0] add (I[1] multiply I[2]))"
+    opt = OptimizedFunction(None, f, "chain")
+    L, Cn, Fn, B = _lib.FUSE_LOAD, _lib.FUSE_CONST, _lib.FUSE_FUN, _lib.FUSE_BIN
+    assert opt.program == [L, 0, Fn, _lib.FUN["sig"], L, 1, B, _lib.OP["multiply"], L, 2, B, _lib.OP["add"], Fn, _lib.FUN["tanh"]]
+    with pytest.raises(IllegalArgumentException):
+        Function.of("nope(i0)")
+    with pytest.raises(IllegalArgumentException):
+        OptimizedFunction(None, Function.of("i0 x i1"), "conv")
+
+
+def test_no_host_arithmetic_path():
+    a = Tensor.of(np.float32, [2, 2], [1, 2, 3, 4])
+    with pytest.raises(IllegalStateException):
+        a + a
