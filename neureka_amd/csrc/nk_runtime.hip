@@ -214,7 +214,8 @@ int nk_device_props(nk_dev h, char* name, size_t name_cap, int* compute_units, i
                     uint64_t* global_mem_bytes, int* lds_bytes_per_block, int* wavefront_size) {
     NK_DEVICE(dev, h);
     if (name && name_cap) {
-        strncpy(name, dev->props.name, name_cap - 1);
+        const char* n = dev->props.name[0] ? dev->props.name : dev->props.gcnArchName;
+        strncpy(name, n, name_cap - 1);
         name[name_cap - 1] = 0;
     }
     if (compute_units) *compute_units = dev->props.multiProcessorCount;

@@ -126,12 +126,17 @@ template <typename T> __device__ __forceinline__ T selu_ref(T x) {
     }
     return T(NAN);
 }
+// Derivatives are not on any bandwidth-critical path, and several of the reference's float formulas
+// cancel (1 - tanh^2, s*(1-s), -t*tanh^2 + t).  To stay within tolerance of the reference's *results*,
+// the f32 derivatives below repeat its float lambdas literally, including their double intermediates.
 template <typename T> __device__ __forceinline__ T dselu_ref(T x) {
     const double ALPHA = 1.6732632423543772848170429916717, SCALE = 1.0507009873554804934193349852946;
     if (x > T(0)) return T(SCALE);
-    if (x <= T(0)) return T(SCALE * ALPHA) * Num<T>::exp(x);
+    if (x <= T(0)) return T(SCALE * ALPHA * ::exp((double)x));
     return T(NAN);
 }
+__device__ __forceinline__ float tanh_f32_via_f64(float x) { return (float)(2.0 / (1.0 + ::exp((double)(-x * 2.0f))) - 1.0); }
+__device__ __forceinline__ float sig_f32_via_f64(float x) { return (float)(1.0 / (1.0 + ::exp(-(double)x))); }
 template <typename T> __device__ __forceinline__ T softplus_ref(T x) {
     using N = Num<T>;
     if (sizeof(T) == 8) return N::log(T(1) + N::exp(x));
@@ -141,21 +146,30 @@ template <typename T> __device__ __forceinline__ T dgasu_ref(T x) {
     T x2 = x * x, x6 = x2 * x2 * x2;
     return T(3) * x2 / (T(2) * x2 * Num<T>::abs(x) + x6 + T(1));
 }
-template <typename T> __device__ __forceinline__ T dgatu_ref(T x) {
+template <typename T> __device__ __forceinline__ T dgatu_ref(T x) {      // fun/ScalarGaTU.java
     T x2 = x * x, x3 = x2 * x, temp = T(3) * x2;
-    if (sizeof(T) == 8) { T t = tanh_ref(x3); return -temp * (t * t) + temp; }
-    return temp * dtanh_ref(x3);     // = -temp*tanh^2 + temp without the cancellation
+    if constexpr (sizeof(T) == 8) { T t = tanh_ref(x3); return -temp * (t * t) + temp; }
+    else { double t = (double)tanh_f32_via_f64(x3); float tanh2 = (float)(t * t); return -temp * tanh2 + temp; }
 }
 template <typename T> __device__ __forceinline__ T dfast_gaus_ref(T x) {
     T x2 = x * x;
     return T(-2) * x / (x2 * x2 + T(2) * x2 + T(1));
 }
-template <typename T> __device__ __forceinline__ T dgelu_ref(T x) {
-    T sig = sigmoid(x * T(1.702)), ds = sig * (T(1) - sig);
+template <typename T> __device__ __forceinline__ T dgelu_ref(T x) {      // fun/ScalarGeLU.java
+    T sig;
+    if constexpr (sizeof(T) == 8) sig = sigmoid(x * 1.702); else sig = (float)(1.0 / (1.0 + ::exp(-((double)x * 1.702))));
+    T ds = sig * (T(1) - sig);
     return sig + ds * x * T(1.702);
 }
-template <typename T> __device__ __forceinline__ T dsig_ref(T x) { T s = sigmoid(x); return s * (T(1) - s); }
-template <typename T> __device__ __forceinline__ T dsilu_ref(T x) { T s = sigmoid(x); return s + (x * s * (T(1) - s)); }
+template <typename T> __device__ __forceinline__ T sig_as_ref(T x) {
+    if constexpr (sizeof(T) == 8) return sigmoid(x); else return sig_f32_via_f64(x);
+}
+template <typename T> __device__ __forceinline__ T dsig_ref(T x) { T s = sig_as_ref(x); return s * (T(1) - s); }
+template <typename T> __device__ __forceinline__ T dsilu_ref(T x) { T s = sig_as_ref(x); return s + (x * s * (T(1) - s)); }
+template <typename T> __device__ __forceinline__ T dtanh_as_ref(T x) {   // fun/ScalarTanh.java:31-34
+    if constexpr (sizeof(T) == 8) return dtanh_ref(x);
+    else { double t = (double)tanh_f32_via_f64(x); return (float)(1.0 - t * t); }
+}
 template <typename T> __device__ __forceinline__ T dfast_tanh_ref(T x) {
     T t1 = x * x, t2 = Num<T>::sqrt(T(1) + t1);
     return T(1) / (t1 * t2 + t2);
@@ -197,10 +211,10 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
     using N = Num<T>;
     switch (id) {
         case NK_FUN_ABS: NK_EACH(x < T(0) ? T(-1) : T(1));
-        case NK_FUN_COS: NK_EACH(-N::sin(x));
+        case NK_FUN_COS: NK_EACH(T(-::sin((double)x)));
         case NK_FUN_GASU: NK_EACH(dgasu_ref(x));
         case NK_FUN_GATU: NK_EACH(dgatu_ref(x));
-        case NK_FUN_GAUS: NK_EACH(T(-2) * x * gauss(x));
+        case NK_FUN_GAUS: NK_EACH(T(-2.0 * (double)x * ::exp(-((double)x * (double)x))));
         case NK_FUN_FAST_GAUS: NK_EACH(dfast_gaus_ref(x));
         case NK_FUN_GELU: NK_EACH(dgelu_ref(x));
         case NK_FUN_IDY: NK_EACH(T(1));
@@ -210,15 +224,15 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
         case NK_FUN_SELU: NK_EACH(dselu_ref(x));
         case NK_FUN_SIG: NK_EACH(dsig_ref(x));
         case NK_FUN_SILU: NK_EACH(dsilu_ref(x));
-        case NK_FUN_SIN: NK_EACH(N::cos(x));
-        case NK_FUN_SOFTPLUS: NK_EACH(sigmoid(x));
+        case NK_FUN_SIN: NK_EACH(T(::cos((double)x)));
+        case NK_FUN_SOFTPLUS: NK_EACH(T(1.0 / (1.0 + ::exp(-(double)x))));
         case NK_FUN_SOFTSIGN: NK_EACH(T(1) / (T(2) * N::abs(x) + x * x + T(1)));
-        case NK_FUN_TANH: NK_EACH(dtanh_ref(x));
+        case NK_FUN_TANH: NK_EACH(dtanh_as_ref(x));
         case NK_FUN_FAST_TANH: NK_EACH(dfast_tanh_ref(x));
-        case NK_FUN_EXP: NK_EACH(N::exp(x));
+        case NK_FUN_EXP: NK_EACH(T(::exp((double)x)));
         case NK_FUN_LOG10: NK_EACH(T(1) / (x * T(2.302585092994046)));   // x * ln(10)
         case NK_FUN_SQRT: NK_EACH(T(0.5) * inv_sqrt_ref(x));
-        case NK_FUN_CBRT: NK_EACH(T(1) / (T(3) * N::pow(x, T(2.0) / T(3.0))));
+        case NK_FUN_CBRT: NK_EACH(T(1) / (T(3) * T(::pow((double)x, (double)(T(2.0) / T(3.0))))));
         default: NK_EACH(T(NAN) + x);
     }
 }

@@ -272,6 +272,8 @@ class HipDevice:
     @staticmethod
     def _ops(*tensors):
         out = []
+        if len({t.rank for t in tensors}) > 1:
+            raise IllegalArgumentException(f"operands of one kernel must have one rank, got {[t.rank for t in tensors]}")
         for t in tensors:
             # a virtual tensor keeps one element on the device and is addressed through all-zero tables
             inline = (NDConfiguration.virtualOf(t.shape) if t.isVirtual() else t.ndc).asInlineArray()

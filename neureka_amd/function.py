@@ -34,6 +34,7 @@ def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = Tr
     ctx = backend()
     operation = ctx.getOperation(op_id)
     device = _device_for(inputs)
+    parents = list(inputs)                   # the tensors the caller holds: gradients attach to these
     if len(inputs) > 1 and len({t.rank for t in inputs}) > 1:
         inputs = make_fit(list(inputs))      # FunctionNode.execute pads ranks first (FunctionNode.java:92-93)
     call = ExecutionCall(device, operation, list(inputs), d)
@@ -47,8 +48,8 @@ def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = Tr
         return execute_device_algorithm(c), c
 
     result, prepared = execute_on_common_device(call, run)
-    if record and d < 0 and any(t.rqsGradient() or t._node is not None for t in inputs):
-        result._node = _graph_node(op_id, prepared, list(inputs), result)
+    if record and d < 0 and any(t.rqsGradient() or t._node is not None for t in parents):
+        result._node = _graph_node(op_id, prepared, parents, result)
     return result
 
 

@@ -305,7 +305,12 @@ def make_fit(tensors: Sequence[Tensor]) -> List[Tensor]:
                 form = [-1] * padding + list(range(rank - padding))
             else:
                 form = list(range(rank - padding)) + [-1] * padding
-            t = t.permute(*form)
+            if t.isOutsourced():
+                t = t.permute(*form)
+            else:       # a host operand: the padded tensor shares the host array, no parent relation needed
+                padded = Tensor(t.dtype, t.ndc.newReshaped(form), t._data, t._virtual)
+                padded._rqs_gradient = t._rqs_gradient
+                t = padded
         out.append(t)
     return out
 
