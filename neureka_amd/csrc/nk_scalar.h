@@ -175,12 +175,13 @@ template <typename T> __device__ __forceinline__ T dfast_tanh_ref(T x) {
     return T(1) / (t1 * t2 + t2);
 }
 
-template <typename T, int V>
+// FUNSET selects how much of the function table a kernel instantiation carries (register pressure):
+//   1  the f32-cheap forward activations; 2  everything (sin/cos/log10/cbrt, all derivatives, fmod, pow).
+template <typename T, int V, int FUNSET>
 __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
     using N = Num<T>;
     switch (id) {
         case NK_FUN_ABS: NK_EACH(N::abs(x));
-        case NK_FUN_COS: NK_EACH(N::cos(x));
         case NK_FUN_GASU: NK_EACH(softsign(x * x * x));
         case NK_FUN_GATU: NK_EACH(tanh_ref(x * x * x));
         case NK_FUN_GAUS: NK_EACH(gauss(x));
@@ -193,18 +194,27 @@ __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
         case NK_FUN_SELU: NK_EACH(selu_ref(x));
         case NK_FUN_SIG: NK_EACH(sigmoid(x));
         case NK_FUN_SILU: NK_EACH(x * sigmoid(x));
-        case NK_FUN_SIN: NK_EACH(N::sin(x));
         case NK_FUN_SOFTPLUS: NK_EACH(softplus_ref(x));
         case NK_FUN_SOFTSIGN: NK_EACH(softsign(x));
         case NK_FUN_TANH: NK_EACH(tanh_ref(x));
         case NK_FUN_FAST_TANH: NK_EACH(x * inv_sqrt_ref(T(1) + x * x));
         case NK_FUN_EXP: NK_EACH(N::exp(x));
-        case NK_FUN_LOG10: NK_EACH(N::log10(x));
         case NK_FUN_SQRT: NK_EACH(N::sqrt(x));
-        case NK_FUN_CBRT: NK_EACH(N::cbrt(x));
-        default: NK_EACH(T(NAN) + x);
+        default:
+            if constexpr (FUNSET >= 2) {
+                switch (id) {
+                    case NK_FUN_COS: NK_EACH(N::cos(x));
+                    case NK_FUN_SIN: NK_EACH(N::sin(x));
+                    case NK_FUN_LOG10: NK_EACH(N::log10(x));
+                    case NK_FUN_CBRT: NK_EACH(N::cbrt(x));
+                    default: NK_EACH(T(NAN) + x);
+                }
+            } else NK_EACH(T(NAN) + x);
     }
 }
+
+// does function `id` need the full table?
+inline bool fun_is_heavy(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN || id == NK_FUN_LOG10 || id == NK_FUN_CBRT; }
 
 template <typename T, int V>
 __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
@@ -248,7 +258,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
     }                                                   \
     break
 
-template <typename T, int V>
+template <typename T, int V, int FUNSET>
 __device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
     using N = Num<T>;
     switch (op) {
@@ -256,15 +266,21 @@ __device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
         case NK_OP_SUB: NK_EACH2(x - y);
         case NK_OP_MUL: NK_EACH2(x * y);
         case NK_OP_DIV: NK_EACH2(x / y);
-        case NK_OP_MOD: NK_EACH2(N::fmod(x, y));     // Java's % on floating point is C's fmod
-        case NK_OP_POW: NK_EACH2(N::pow(x, y));
         case NK_OP_IDY: NK_EACH2(y);
-        default: NK_EACH2(T(NAN) + x + y);
+        default:
+            if constexpr (FUNSET >= 2) {
+                switch (op) {
+                    case NK_OP_MOD: NK_EACH2(N::fmod(x, y));     // Java's % on floating point is C's fmod
+                    case NK_OP_POW: NK_EACH2(N::pow(x, y));
+                    default: NK_EACH2(T(NAN) + x + y);
+                }
+            } else NK_EACH2(T(NAN) + x + y);
     }
 }
+inline bool bin_is_heavy(int op) { return op == NK_OP_MOD || op == NK_OP_POW; }
 
 // partial derivatives: CPUBiElementWise*.java (_getDeriveAt0 / _getDeriveAt1).  a = d(a op b)/d(operand d).
-template <typename T, int V>
+template <typename T, int V, int FUNSET>
 __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b)[V]) {
     using N = Num<T>;
     switch (op * 2 + d) {
@@ -274,17 +290,23 @@ __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b
         case NK_OP_SUB * 2 + 1: NK_EACH2(T(-1));
         case NK_OP_MUL * 2 + 0: NK_EACH2(y);
         case NK_OP_MUL * 2 + 1: NK_EACH2(x);
-        case NK_OP_DIV * 2 + 0:
-        case NK_OP_MOD * 2 + 0: NK_EACH2(T(1) / y);
-        case NK_OP_DIV * 2 + 1:
-        case NK_OP_MOD * 2 + 1: NK_EACH2(-(x / (y * y)));
-        case NK_OP_POW * 2 + 0: NK_EACH2(y * N::pow(x, y - T(1)));
-        case NK_OP_POW * 2 + 1: NK_EACH2(N::pow(x, y) * N::log(x));
         case NK_OP_IDY * 2 + 0: NK_EACH2(T(0));
         case NK_OP_IDY * 2 + 1: NK_EACH2(T(1));
-        default: NK_EACH2(T(NAN) + x + y);
+        default:
+            if constexpr (FUNSET >= 2) {
+                switch (op * 2 + d) {
+                    case NK_OP_DIV * 2 + 0:
+                    case NK_OP_MOD * 2 + 0: NK_EACH2(T(1) / y);
+                    case NK_OP_DIV * 2 + 1:
+                    case NK_OP_MOD * 2 + 1: NK_EACH2(-(x / (y * y)));
+                    case NK_OP_POW * 2 + 0: NK_EACH2(y * N::pow(x, y - T(1)));
+                    case NK_OP_POW * 2 + 1: NK_EACH2(N::pow(x, y) * N::log(x));
+                    default: NK_EACH2(T(NAN) + x + y);
+                }
+            } else NK_EACH2(T(NAN) + x + y);
     }
 }
+inline bool dbin_is_heavy(int op) { return op == NK_OP_DIV || op == NK_OP_MOD || op == NK_OP_POW; }
 #undef NK_EACH2
 
 }  // namespace nk
