@@ -99,6 +99,79 @@ __device__ __forceinline__ void run_prog(const Prog& P, const T (&src)[NSRC][V],
     }
 }
 
+// Short programs (at most LIGHT_INSTR instructions, LIGHT_CONST constants, no saved intermediates) are
+// handed to the specialised families in packed form: all instruction words sit in one aligned block of
+// the kernel arguments and are fetched with a single wide scalar load, then consumed from a shift
+// register, so the interpreter never waits for memory between instructions.
+constexpr int LIGHT_INSTR = 8, LIGHT_CONST = 4;
+struct alignas(16) LightProg {
+    unsigned code[LIGHT_INSTR];    // op | arg << 8 | src << 16
+    double consts[LIGHT_CONST];
+    int n;
+};
+
+template <typename T, int V, int NSRC, int FUNSET>
+__device__ __forceinline__ void run_light(const LightProg& P, const T (&src)[NSRC][V], T (&acc)[V]) {
+    unsigned c0 = P.code[0], c1 = P.code[1], c2 = P.code[2], c3 = P.code[3], c4 = P.code[4], c5 = P.code[5], c6 = P.code[6], c7 = P.code[7];
+    T k[LIGHT_CONST];
+#pragma unroll
+    for (int i = 0; i < LIGHT_CONST; i++) k[i] = (T)P.consts[i];
+#pragma unroll
+    for (int v = 0; v < V; v++) acc[v] = T(0);
+    for (int pc = 0; pc < P.n; pc++) {
+        const unsigned code = c0;
+        c0 = c1; c1 = c2; c2 = c3; c3 = c4; c4 = c5; c5 = c6; c6 = c7;
+        const int op = code & 0xff, arg = (code >> 8) & 0xff, s = (code >> 16) & 0xff;
+        T x[V];
+        if (op != I_FUN) {
+            if (s >= SRC_CONST0) {
+                T c = k[0];
+#pragma unroll
+                for (int i = 1; i < LIGHT_CONST; i++) if (s == SRC_CONST0 + i) c = k[i];
+#pragma unroll
+                for (int v = 0; v < V; v++) x[v] = c;
+            } else {
+#pragma unroll
+                for (int v = 0; v < V; v++) x[v] = src[0][v];
+#pragma unroll
+                for (int j = 1; j < NSRC; j++)
+                    if (s == j) {
+#pragma unroll
+                        for (int v = 0; v < V; v++) x[v] = src[j][v];
+                    }
+            }
+        }
+        switch (op) {
+            case I_SET:
+#pragma unroll
+                for (int v = 0; v < V; v++) acc[v] = x[v];
+                break;
+            case I_FUN:
+                if constexpr (FUNSET >= 1) apply_fun<T, V, FUNSET>(arg, acc);
+                break;
+            case I_BIN: apply_bin<T, V, FUNSET>(arg, acc, x); break;
+            case I_RBIN:
+                apply_bin<T, V, FUNSET>(arg, x, acc);
+#pragma unroll
+                for (int v = 0; v < V; v++) acc[v] = x[v];
+                break;
+            case I_DBIN: apply_dbin<T, V, FUNSET>(arg >> 1, arg & 1, acc, x); break;
+            case I_RDBIN:
+                apply_dbin<T, V, FUNSET>(arg >> 1, arg & 1, x, acc);
+#pragma unroll
+                for (int v = 0; v < V; v++) acc[v] = x[v];
+                break;
+        }
+    }
+}
+
+// family-independent entry: the full family interprets the long form, the others the packed form
+template <typename T, int V, int NSRC, int FUNSET>
+__device__ __forceinline__ void run_any(const Prog& P, const LightProg& LP, const T (&src)[NSRC][V], T (&acc)[V]) {
+    if constexpr (FUNSET >= 2) run_prog<T, V, NSRC, FUNSET>(P, src, acc);
+    else run_light<T, V, NSRC, FUNSET>(LP, src, acc);
+}
+
 // ---- helpers ---------------------------------------------------------------------------------------
 // unsigned division by an invariant divisor, valid for numerators below 2^31
 struct FastDiv {
@@ -150,84 +223,160 @@ __device__ __forceinline__ void store_vec(T* p, const T (&src)[V], bool streamin
 
 // ---- rows kernel -----------------------------------------------------------------------------------
 // Every operand is contiguous (stride 1) or constant (stride 0) along the innermost collapsed axis.
-// A block of 256 threads covers `256 >> tpr_log2` rows per pass and PASSES passes per tile; a thread
-// issues the loads of all its passes before it computes and stores, so that several 16-byte requests
-// per source are in flight per lane.
+// The work is cut into units of (256 >> tpr_log2 rows) x (tpr threads x V elements); a block owns PASSES
+// consecutive units; a thread issues the loads of all its passes, runs the program once over all of
+// them, then stores.  When a row spans at least a wavefront (tpr >= 64) the row index is wave-uniform:
+// the nd-index arithmetic then runs on the scalar unit.  Element offsets are 32-bit (the host checks),
+// at most ROWS_MAX_OUTER outer axes (more fall to the canon kernel); the argument block is small and
+// fixed-size so that it is fetched with a few wide scalar loads at kernel start.
+constexpr int ROWS_MAX_OUTER = 3;
 struct RowsArgs {
-    int rank;                  // collapsed rank >= 1
+    int nouter;                // collapsed outer axes, 0..ROWS_MAX_OUTER
     int nsrc;
     unsigned L;                // innermost extent
     unsigned n_rows;           // product of the outer extents
     int tpr_log2;              // threads per row, log2
     unsigned chunks;           // column chunks per row
-    unsigned n_tiles;
+    unsigned n_units;          // row groups x chunks
     unsigned scalar_load;      // bit j: source j is not 16-byte aligned: element-wise loads
+    unsigned const_last;       // bit j: source j has stride 0 along the innermost axis
+    int simple_loads;          // every source register is filled by a plain aligned vector load
+    int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
     int streaming;             // non-temporal stores for the drain
     FastDiv chunk_div;
-    FastDiv outer[NK_MAX_RANK];             // outer[k] divides by shape[k], k < rank-1
-    int64_t base[MAX_OPERANDS];
-    int64_t stride[MAX_OPERANDS][NK_MAX_RANK];
+    FastDiv outer[ROWS_MAX_OUTER];           // outer[0] is the innermost outer axis
+    int base[MAX_OPERANDS];
+    int stride[MAX_OPERANDS][ROWS_MAX_OUTER];
 };
 
-template <typename T, int V, int NSRC, int FUNSET, int PASSES>
-__global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, T* __restrict__ drn, Ptrs srcs) {
+// addressing shared by the rows kernels: unit -> (row, col), row -> element offset of every operand
+template <int NOPS>
+struct RowsAddr {
+    int off[NOPS];
+    unsigned col;
+    bool live;
+};
+template <int NOPS>
+__device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsigned u) {
     const unsigned tpr = 1u << A.tpr_log2;
     const unsigned rows_per_pass = 256u >> A.tpr_log2;
     const unsigned sub = threadIdx.x >> A.tpr_log2, lane = threadIdx.x & (tpr - 1);
-    const int last = A.rank - 1;
-    for (unsigned tile = blockIdx.x; tile < A.n_tiles; tile += gridDim.x) {
-        const unsigned row_tile = A.chunk_div.div(tile);
-        const unsigned chunk = tile - row_tile * A.chunks;
-        const unsigned col = (chunk * tpr + lane) * V;
-        if (col >= A.L) continue;
-        T x[PASSES][NSRC][V];
-        int64_t doff[PASSES];
-        bool live[PASSES];
+    const unsigned rg = A.chunk_div.div(u);                         // u is block-uniform
+    const unsigned chunk = u - rg * A.chunks;
+    unsigned row = rg * rows_per_pass + sub;
+    RowsAddr<NOPS> R;
+    R.col = (chunk * tpr + lane) * (unsigned)A.vec;
+    const bool row_ok = u < A.n_units && row < A.n_rows;            // wave-uniform when a row spans a wavefront
+    R.live = row_ok && R.col < A.L;
+    if (!row_ok) row = 0;                                           // dead lanes get a valid address:
+    if (!R.live) R.col = 0;                                         // loads need no predicate
+    auto resolve = [&](unsigned r) {
 #pragma unroll
-        for (int p = 0; p < PASSES; p++) {
-            const unsigned row = (row_tile * PASSES + p) * rows_per_pass + sub;
-            live[p] = row < A.n_rows;
-            int64_t off[NSRC + 1];
+        for (int o = 0; o < NOPS; o++) R.off[o] = A.base[o];
 #pragma unroll
-            for (int o = 0; o <= NSRC; o++) off[o] = A.base[o];
-            unsigned r = live[p] ? row : 0;
-            for (int k = last - 1; k >= 0; k--) {
+        for (int k = 0; k < ROWS_MAX_OUTER; k++) {
+            if (k < A.nouter) {
                 const unsigned q = A.outer[k].div(r);
-                const unsigned idx = r - q * A.outer[k].d;
+                const int idx = (int)(r - q * A.outer[k].d);
                 r = q;
 #pragma unroll
-                for (int o = 0; o <= NSRC; o++) off[o] += (int64_t)idx * A.stride[o][k];
+                for (int o = 0; o < NOPS; o++) R.off[o] += idx * A.stride[o][k];
             }
-            doff[p] = off[0] + col;
+        }
+    };
+    // a row that spans a whole wavefront is wave-uniform: resolve it on the scalar unit
+    if (A.tpr_log2 >= 6) resolve(__builtin_amdgcn_readfirstlane(row));
+    else resolve(row);
+    return R;
+}
+
+template <typename T, int V, int NSRC, int FUNSET, int PASSES>
+__global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
+    T x[NSRC][PASSES * V];
+    int doff[PASSES];
+    bool live[PASSES];
+    if (A.simple_loads) {
+        // every source is a plain aligned vector load: no branches between the loads of all passes
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, blockIdx.x * PASSES + p);
+            live[p] = R.live;
+            doff[p] = R.off[0] + (int)R.col;
 #pragma unroll
             for (int j = 0; j < NSRC; j++) {
-                if (j < A.nsrc && live[p]) {
-                    const T* sp = (const T*)srcs.p[j] + off[j + 1];
-                    if (A.stride[j + 1][last] == 0) {
+                T (&xj)[V] = *reinterpret_cast<T (*)[V]>(&x[j][p * V]);
+                load_vec<T, V>(xj, (const T*)srcs.p[j] + R.off[j + 1] + R.col);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int p = 0; p < PASSES; p++) {
+            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, blockIdx.x * PASSES + p);
+            live[p] = R.live;
+            doff[p] = R.off[0] + (int)R.col;
+#pragma unroll
+            for (int j = 0; j < NSRC; j++) {
+                T (&xj)[V] = *reinterpret_cast<T (*)[V]>(&x[j][p * V]);
+                if (j < A.nsrc) {
+                    const T* sp = (const T*)srcs.p[j] + R.off[j + 1];
+                    if ((A.const_last >> j) & 1u) {
                         const T c = *sp;
 #pragma unroll
-                        for (int v = 0; v < V; v++) x[p][j][v] = c;
+                        for (int v = 0; v < V; v++) xj[v] = c;
                     } else if ((A.scalar_load >> j) & 1u) {
 #pragma unroll
-                        for (int v = 0; v < V; v++) x[p][j][v] = sp[col + v];
+                        for (int v = 0; v < V; v++) xj[v] = sp[R.col + v];
                     } else {
-                        load_vec<T, V>(x[p][j], sp + col);
+                        load_vec<T, V>(xj, sp + R.col);
                     }
                 } else {
 #pragma unroll
-                    for (int v = 0; v < V; v++) x[p][j][v] = T(0);
+                    for (int v = 0; v < V; v++) xj[v] = T(0);
                 }
             }
         }
+    }
+    T out[PASSES * V];
+    run_any<T, PASSES * V, NSRC, FUNSET>(P, LP, x, out);
 #pragma unroll
-        for (int p = 0; p < PASSES; p++) {
-            if (live[p]) {
-                T out[V];
-                run_prog<T, V, NSRC, FUNSET>(P, x[p], out);
-                store_vec<T, V>(drn + doff[p], out, A.streaming != 0);
-            }
+    for (int p = 0; p < PASSES; p++) {
+        if (live[p]) {
+            T (&op)[V] = *reinterpret_cast<T (*)[V]>(&out[p * V]);
+            store_vec<T, V>(drn + doff[p], op, A.streaming != 0);
         }
     }
+}
+
+// drain = src0 op src1 with op in {+, -, *, /} and plain aligned loads: the bandwidth-critical case
+// (same-shape elementwise and forward broadcast).  The operator is resolved once, outside the passes,
+// and each pass is stored as soon as its operands have arrived.
+template <typename T, int V, int PASSES>
+__global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T* __restrict__ drn, const T* __restrict__ s0,
+                                                          const T* __restrict__ s1) {
+    T x0[PASSES][V], x1[PASSES][V];
+    int doff[PASSES];
+    bool live[PASSES];
+#pragma unroll
+    for (int p = 0; p < PASSES; p++) {
+        const RowsAddr<3> R = rows_address<3>(A, blockIdx.x * PASSES + p);
+        live[p] = R.live;
+        doff[p] = R.off[0] + (int)R.col;
+        load_vec<T, V>(x0[p], s0 + R.off[1] + R.col);
+        load_vec<T, V>(x1[p], s1 + R.off[2] + R.col);
+    }
+#define NK_BINARY_PASSES(EXPR)                                                        \
+    _Pragma("unroll") for (int p = 0; p < PASSES; p++) {                              \
+        T out[V];                                                                     \
+        _Pragma("unroll") for (int v = 0; v < V; v++) { const T a = x0[p][v], b = x1[p][v]; out[v] = (EXPR); } \
+        if (live[p]) store_vec<T, V>(drn + doff[p], out, A.streaming != 0);           \
+    }
+    switch (op) {
+        case NK_OP_ADD: NK_BINARY_PASSES(a + b) break;
+        case NK_OP_SUB: NK_BINARY_PASSES(a - b) break;
+        case NK_OP_MUL: NK_BINARY_PASSES(a * b) break;
+        default: NK_BINARY_PASSES(a / b) break;
+    }
+#undef NK_BINARY_PASSES
 }
 
 // ---- canon kernel: arbitrary strides, one element per thread -------------------------------------------
@@ -241,7 +390,7 @@ struct CanonArgs {
 };
 
 template <typename T, int NSRC, int FUNSET>
-__global__ __launch_bounds__(256) void canon_kernel(CanonArgs A, Prog P, T* __restrict__ drn, Ptrs srcs) {
+__global__ __launch_bounds__(256) void canon_kernel(CanonArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
     const unsigned step = gridDim.x * blockDim.x;
     for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < A.n; i += step) {
         int64_t off[NSRC + 1];
@@ -259,7 +408,7 @@ __global__ __launch_bounds__(256) void canon_kernel(CanonArgs A, Prog P, T* __re
 #pragma unroll
         for (int j = 0; j < NSRC; j++) x[j][0] = j < A.nsrc ? ((const T*)srcs.p[j])[off[j + 1]] : T(0);
         T out[1];
-        run_prog<T, 1, NSRC, FUNSET>(P, x, out);
+        run_any<T, 1, NSRC, FUNSET>(P, LP, x, out);
         drn[off[0]] = out[0];
     }
 }
@@ -285,7 +434,7 @@ struct TileArgs {
 };
 
 template <typename T, int NSRC, int FUNSET>
-__global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, T* __restrict__ drn, Ptrs srcs) {
+__global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
     __shared__ T tile[64][65];
     const int last = A.rank - 1;
     const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;   // 64 x 4
@@ -337,7 +486,7 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, T* __rest
         }
         const int64_t dP = A.stride[0][A.pax], dL = A.stride[0][last];
         T out[16];
-        run_prog<T, 16, NSRC, FUNSET>(P, x, out);
+        run_any<T, 16, NSRC, FUNSET>(P, LP, x, out);
 #pragma unroll
         for (int it = 0; it < 16; it++) {
             const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
@@ -390,10 +539,11 @@ __global__ __launch_bounds__(256) void literal_kernel(LiteralArgs A, Prog P, T* 
 }
 
 // ---- launch plan (filled by the host analysis, executed by launch_family<T, FUNSET>) --------------------
-enum PlanKind { PLAN_ROWS, PLAN_TILE, PLAN_CANON, PLAN_LITERAL };
+enum PlanKind { PLAN_ROWS, PLAN_ROWS_BINARY, PLAN_TILE, PLAN_CANON, PLAN_LITERAL };
 struct Plan {
     PlanKind kind;
     bool vec;                  // rows: 16-byte vectors
+    int binary_op;             // PLAN_ROWS_BINARY
     int nsrc;
     unsigned grid;
     RowsArgs rows;
@@ -401,6 +551,7 @@ struct Plan {
     CanonArgs canon;
     LiteralArgs literal;
     Prog prog;
+    LightProg light;
     void* drn;
     Ptrs srcs;
 };

@@ -120,9 +120,13 @@ struct EltCall {
 };
 
 static unsigned grid_for(Device* dev, uint64_t work_blocks) {
-    uint64_t cap = (uint64_t)dev->props.multiProcessorCount * 16;
-    if (cap < 256) cap = 256;
-    return (unsigned)(work_blocks < cap ? (work_blocks ? work_blocks : 1) : cap);
+    // One block per tile: on this part a streaming kernel is fastest when the grid is far larger than the
+    // machine (262144 blocks of 256 threads write at 6.3 TB/s, 4096 grid-striding blocks at 4.6 TB/s).
+    // NK_GRID_CAP (blocks per compute unit, 0 = no cap) exists for experiments.
+    static const long cap_per_cu = [] { const char* v = getenv("NK_GRID_CAP"); return v && *v ? atol(v) : 0L; }();
+    uint64_t cap = cap_per_cu > 0 ? (uint64_t)dev->props.multiProcessorCount * cap_per_cu : ((uint64_t)1 << 31) - 1;
+    if (work_blocks == 0) work_blocks = 1;
+    return (unsigned)(work_blocks < cap ? work_blocks : cap);
 }
 
 static bool env_flag(const char* name, bool dflt) {
@@ -154,6 +158,17 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     for (int j = 0; j < c.nsrc; j++) plan.srcs.p[j] = (const void*)c.src[j];
     int funset = funset_of(prog);
     if (c.nsrc > 3) funset = 2;            // the specialised families carry at most 3 source registers
+    // ... and run the packed short form of the program
+    int n_consts = 0;
+    for (int i = 0; i < prog.n; i++)
+        if (prog.op[i] != I_FUN && prog.op[i] != I_DFUN && prog.op[i] != I_PUSH && prog.src[i] >= SRC_CONST0 && prog.src[i] < SRC_POP)
+            n_consts = n_consts > prog.src[i] - SRC_CONST0 + 1 ? n_consts : prog.src[i] - SRC_CONST0 + 1;
+    if (prog.n > LIGHT_INSTR || n_consts > LIGHT_CONST) funset = 2;
+    if (funset < 2) {
+        plan.light.n = prog.n;
+        for (int i = 0; i < prog.n; i++) plan.light.code[i] = prog.op[i] | (prog.arg[i] << 8) | (prog.src[i] << 16);
+        for (int i = 0; i < LIGHT_CONST; i++) plan.light.consts[i] = prog.consts[i];
+    }
     // outputs far larger than the last-level cache are written with non-temporal stores
     const bool streaming = env_flag("NK_STREAMING_STORES", true) && (uint64_t)c.n * sizeof(T) >= ((uint64_t)64 << 20);
 
@@ -171,10 +186,22 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     }
     if (cn.rank == 0) { cn.rank = 1; cn.shape[0] = 1; for (int o = 0; o <= c.nsrc; o++) cn.stride[o][0] = 1; }
     const int last = cn.rank - 1;
-    bool rows_ok = cn.stride[0][last] == 1;
+    bool rows_ok = cn.stride[0][last] == 1 && cn.rank - 1 <= ROWS_MAX_OUTER;
     for (int j = 0; j < c.nsrc; j++) rows_ok = rows_ok && (cn.stride[j + 1][last] == 0 || cn.stride[j + 1][last] == 1);
     bool done = false;
 
+    // the rows kernel keeps element offsets in 32 bits: every reachable offset must fit
+    if (rows_ok) {
+        for (int o = 0; o <= c.nsrc && rows_ok; o++) {
+            int64_t lo = cn.base[o], hi = cn.base[o];
+            for (int k = 0; k < cn.rank; k++) {
+                const int64_t span = (cn.shape[k] - 1) * cn.stride[o][k];
+                if (span < 0) lo += span; else hi += span;
+                if (cn.stride[o][k] > INT32_MAX || cn.stride[o][k] < INT32_MIN) rows_ok = false;
+            }
+            if (lo < INT32_MIN || hi > INT32_MAX) rows_ok = false;
+        }
+    }
     if (rows_ok) {
         constexpr int VMAX = 16 / sizeof(T);
         // the drain decides the vector width; a misaligned source is read element by element
@@ -190,11 +217,14 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         }
         const int V = vec ? VMAX : 1;
         const int passes = funset >= 2 ? 1 : 4;
-        A.rank = cn.rank; A.nsrc = c.nsrc;
+        A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
         A.streaming = streaming ? 1 : 0;
+        A.const_last = 0;
+        for (int j = 0; j < c.nsrc; j++) if (cn.stride[j + 1][last] == 0) A.const_last |= 1u << j;
         uint64_t n_rows = 1;
-        for (int k = 0; k < last; k++) { n_rows *= cn.shape[k]; A.outer[k] = FastDiv((unsigned)cn.shape[k]); }
+        // kernel axis k counts outward from the innermost outer axis
+        for (int k = 0; k < last; k++) { n_rows *= cn.shape[k]; A.outer[k] = FastDiv((unsigned)cn.shape[last - 1 - k]); }
         A.n_rows = (unsigned)n_rows;
         const uint64_t vec_per_row = (A.L + V - 1) / V;
         int l2 = 0;
@@ -202,19 +232,28 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         A.tpr_log2 = l2;
         const unsigned tpr = 1u << l2, rpp = 256u >> l2;
         A.chunks = (unsigned)((vec_per_row + tpr - 1) / tpr);
-        const uint64_t row_tiles = (n_rows + (uint64_t)rpp * passes - 1) / ((uint64_t)rpp * passes);
-        const uint64_t n_tiles = row_tiles * A.chunks;
-        if (n_tiles >= ((uint64_t)1 << 31)) return set_error(NK_ERR_UNSUPPORTED, "%s: too many tiles", c.name);
-        A.n_tiles = (unsigned)n_tiles;
+        const uint64_t row_groups = (n_rows + rpp - 1) / rpp;
+        const uint64_t n_units = row_groups * A.chunks;
+        if (n_units >= ((uint64_t)1 << 31)) return set_error(NK_ERR_UNSUPPORTED, "%s: too many work units", c.name);
+        A.n_units = (unsigned)n_units;
         A.chunk_div = FastDiv(A.chunks);
         for (int o = 0; o <= c.nsrc; o++) {
-            A.base[o] = cn.base[o];
-            for (int k = 0; k < cn.rank; k++) A.stride[o][k] = cn.stride[o][k];
+            A.base[o] = (int)cn.base[o];
+            for (int k = 0; k < last; k++) A.stride[o][k] = (int)cn.stride[o][last - 1 - k];
         }
+        A.vec = V;
+        A.simple_loads = (funset < 2 && A.scalar_load == 0 && A.const_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
+        // drain = src0 op src1 with + - * /: the dedicated kernel
+        if (A.simple_loads && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
+            prog.op[1] == I_BIN && prog.src[1] == 1 && prog.arg[1] <= NK_OP_DIV) {
+            plan.kind = PLAN_ROWS_BINARY;
+            plan.binary_op = prog.arg[1];
+        }
         plan.vec = vec;
-        plan.grid = grid_for(dev, n_tiles);
-        set_path(vec ? (A.scalar_load ? "rows_vec_unaligned_src" : "rows_vec") : "rows");
+        plan.grid = (unsigned)((n_units + passes - 1) / passes);     // one block per PASSES units, no grid-stride loop
+        set_path(plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary")
+                                               : vec ? (A.scalar_load ? "rows_vec_unaligned_src" : "rows_vec") : "rows");
         done = true;
     }
 
