@@ -64,9 +64,14 @@ def main():
     n_out = int(np.prod(so))
     bytes_per_launch = 4 * (n_out + a.size + b.size)          # 4 301 258 752: write the output once, read each input once
 
+    # the two launches of a step, with their C-ABI arguments marshalled once (the Python wrapper would
+    # otherwise spend tens of microseconds per call building descriptors)
+    launch_add = dev.prepared_launch("broadcast", "add", -1, out, ta, tb)
+    launch_mul = dev.prepared_launch("broadcast", "multiply", -1, out, ta, tb)
+
     def step():
-        dev.launch_broadcast("add", -1, out, ta, tb)
-        dev.launch_broadcast("multiply", -1, out, ta, tb)
+        launch_add()
+        launch_mul()
 
     for _ in range(args.warmup):
         step()
@@ -80,8 +85,8 @@ def main():
     value = 2 * bytes_per_launch / (ms_per_step * 1e-3) / 1e9
     path = _lib.last_path()
 
-    k_add = event_time_ms(dev, lambda: dev.launch_broadcast("add", -1, out, ta, tb), args.steps)
-    k_mul = event_time_ms(dev, lambda: dev.launch_broadcast("multiply", -1, out, ta, tb), args.steps)
+    k_add = event_time_ms(dev, launch_add, args.steps)
+    k_mul = event_time_ms(dev, launch_mul, args.steps)
     k_ms = 0.5 * (k_add + k_mul)
     achieved = bytes_per_launch / (k_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -121,7 +126,7 @@ def main():
     # ---- the other configurations: kernel figures only ------------------------------------------------------
     others = {}
     if not args.no_others:
-        reps = max(3, min(args.steps, 10))
+        reps = max(5, args.steps)
 
         def hbm(name, nbytes, launch):
             launch(); dev.sync()
@@ -140,7 +145,7 @@ def main():
         a64 = Tensor.of(np.float64, (256, 1, 512), rng.uniform(-1, 1, 256 * 512)).to(dev)
         b64 = Tensor.of(np.float64, (1, 1024, 512), rng.uniform(-1, 1, 1024 * 512)).to(dev)
         o64 = Tensor._on_device(dev, np.float64, (256, 1024, 512))
-        hbm("broadcast_add_f64", 8 * (o64.size + a64.size + b64.size), lambda: dev.launch_broadcast("add", -1, o64, a64, b64))
+        hbm("broadcast_add_f64", 8 * (o64.size + a64.size + b64.size), dev.prepared_launch("broadcast", "add", -1, o64, a64, b64))
         for t in (a64, b64, o64): dev.free(t)
 
         # C3: tanh(sig(a)*b+c) on 2^26 elements: fused, and the reference's 4-kernel sequence
@@ -150,16 +155,18 @@ def main():
         tmp = Tensor._on_device(dev, f32, (n,))
         fn = Function.of("tanh(sig(I[0])*I[1]+I[2])")
         fused = dev.optimizedFunctionOf(fn, "chain")
-        hbm("chain_fused_contiguous", 16 * n, lambda: dev.launch_fused(fused.program, fused.consts, o, srcs))
+        hbm("chain_fused_contiguous", 16 * n, dev.prepared_launch("fused", fused.program, fused.consts, o, srcs))
+        four = [dev.prepared_launch("activation", "sig", -1, tmp, srcs[0]), dev.prepared_launch("elementwise", "multiply", -1, o, tmp, srcs[1]),
+                dev.prepared_launch("elementwise", "add", -1, tmp, o, srcs[2]), dev.prepared_launch("activation", "tanh", -1, o, tmp)]
 
         def unfused():
-            dev.launch_activation("sig", -1, tmp, srcs[0])
-            dev.launch_elementwise("multiply", -1, o, tmp, srcs[1])
-            dev.launch_elementwise("add", -1, tmp, o, srcs[2])
-            dev.launch_activation("tanh", -1, o, tmp)
+            for k in four:
+                k()
         hbm("chain_unfused_4_kernels", 40 * n, unfused)
-        hbm("activation_tanh", 8 * n, lambda: dev.launch_activation("tanh", -1, o, srcs[0]))
-        hbm("elementwise_add", 12 * n, lambda: dev.launch_elementwise("add", -1, o, srcs[0], srcs[1]))
+        hbm("activation_tanh", 8 * n, dev.prepared_launch("activation", "tanh", -1, o, srcs[0]))
+        hbm("activation_sig", 8 * n, dev.prepared_launch("activation", "sig", -1, o, srcs[0]))
+        hbm("elementwise_add", 12 * n, dev.prepared_launch("elementwise", "add", -1, o, srcs[0], srcs[1]))
+        hbm("elementwise_mul", 12 * n, dev.prepared_launch("elementwise", "multiply", -1, o, srcs[0], srcs[1]))
         # permuted [4096,16384] views of row-major [16384,4096]
         from neureka_amd import NDConfiguration
         pv = []
@@ -168,13 +175,13 @@ def main():
             v._set_data(t._data, dev)
             pv.append(v)
         o2 = Tensor(f32, NDConfiguration.ofShape((4096, 16384)), None); o2._set_data(o._data, dev)
-        hbm("chain_fused_permuted", 16 * n, lambda: dev.launch_fused(fused.program, fused.consts, o2, pv))
+        hbm("chain_fused_permuted", 16 * n, dev.prepared_launch("fused", fused.program, fused.consts, o2, pv))
         # slice [::2, 1:8193] of [8192,16384] (the three 2^26 buffers are too small: use 2^27-element parents)
         for t in srcs + [tmp]: dev.free(t)
         parents = [Tensor.of(f32, (8192, 16384), rng.standard_normal(8192 * 16384).astype(f32)).to(dev) for _ in range(3)]
         sv = [p[::2, 1:8193] for p in parents]
         o3 = Tensor(f32, NDConfiguration.ofShape((4096, 8192)), None); o3._set_data(o._data, dev)
-        hbm("chain_fused_sliced", 16 * (1 << 25), lambda: dev.launch_fused(fused.program, fused.consts, o3, sv))
+        hbm("chain_fused_sliced", 16 * (1 << 25), dev.prepared_launch("fused", fused.program, fused.consts, o3, sv))
         for p in parents: dev.free(p)
         dev.free(o)
 
@@ -183,23 +190,23 @@ def main():
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
             Cm = Tensor._on_device(dev, f32, (M, N))
-            flops(name, 2.0 * M * K * N, 4 * (M * K + K * N + M * N), lambda: dev.launch_matmul(True, M, K, N, A, B, Cm))
+            flops(name, 2.0 * M * K * N, 4 * (M * K + K * N + M * N), dev.prepared_launch("matmul", True, M, K, N, A, B, Cm))
             for t in (A, B, Cm): dev.free(t)
 
         # C1 and C5 convolutions
         x1 = Tensor.of(f32, (64, 64), rng.uniform(-1, 1, 4096).astype(f32)).to(dev)
         k1 = Tensor.of(f32, (3, 3), rng.uniform(-1, 1, 9).astype(f32)).to(dev)
         y1 = Tensor._on_device(dev, f32, (62, 62))
-        flops("conv2d_64x64_3x3", 69192, 31796, lambda: dev.launch_convolution(-1, y1, x1, k1))
+        flops("conv2d_64x64_3x3", 69192, 31796, dev.prepared_launch("convolution", -1, y1, x1, k1))
         x5 = Tensor.of(f32, (64, 256, 256), (rng.standard_normal(64 * 256 * 256) * 0.1).astype(f32)).to(dev)
         k5 = Tensor.of(f32, (64, 5, 5), (rng.standard_normal(1600) * 0.1).astype(f32)).to(dev)
         y5 = Tensor._on_device(dev, f32, (1, 252, 252))
         e5 = Tensor.of(f32, (1, 252, 252), rng.standard_normal(252 * 252).astype(f32)).to(dev)
         dx5 = Tensor._on_device(dev, f32, (64, 256, 256))
         dk5 = Tensor._on_device(dev, f32, (64, 5, 5))
-        flops("conv_c5_forward", 203212800, 17037632, lambda: dev.launch_convolution(-1, y5, x5, k5))
-        flops("conv_c5_grad_input", 203212800, 17037632, lambda: dev.launch_convolution(0, dx5, k5, e5))
-        flops("conv_c5_grad_kernel", 203212800, 17037632, lambda: dev.launch_convolution(0, dk5, x5, e5))
+        flops("conv_c5_forward", 203212800, 17037632, dev.prepared_launch("convolution", -1, y5, x5, k5))
+        flops("conv_c5_grad_input", 203212800, 17037632, dev.prepared_launch("convolution", 0, dx5, k5, e5))
+        flops("conv_c5_grad_kernel", 203212800, 17037632, dev.prepared_launch("convolution", 0, dk5, x5, e5))
 
     result = {
         "metric": "GB/s & % HBM peak (broadcast/elementwise)",

@@ -196,7 +196,9 @@ struct FastDiv {
 
 struct Ptrs { const void* p[NK_FUSE_MAX_SRC]; };
 
-template <typename T, int V> struct VecOf { typedef T type __attribute__((ext_vector_type(V))); };
+// Vector access types are only element-aligned: gfx950 global loads and stores of 2 or 4 dwords need
+// dword alignment only, so views that start at an odd element (slices) still move 16 bytes per lane.
+template <typename T, int V> struct VecOf { typedef T type __attribute__((ext_vector_type(V), aligned(sizeof(T)))); };
 template <typename T> struct VecOf<T, 1> { typedef T type; };
 
 template <typename T, int V>
@@ -238,9 +240,8 @@ struct RowsArgs {
     int tpr_log2;              // threads per row, log2
     unsigned chunks;           // column chunks per row
     unsigned n_units;          // row groups x chunks
-    unsigned scalar_load;      // bit j: source j is not 16-byte aligned: element-wise loads
     unsigned const_last;       // bit j: source j has stride 0 along the innermost axis
-    int simple_loads;          // every source register is filled by a plain aligned vector load
+    int simple_loads;          // every source register is filled by a plain vector load
     int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
     int streaming;             // non-temporal stores for the drain
     FastDiv chunk_div;
@@ -323,9 +324,6 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
                         const T c = *sp;
 #pragma unroll
                         for (int v = 0; v < V; v++) xj[v] = c;
-                    } else if ((A.scalar_load >> j) & 1u) {
-#pragma unroll
-                        for (int v = 0; v < V; v++) xj[v] = sp[R.col + v];
                     } else {
                         load_vec<T, V>(xj, sp + R.col);
                     }
@@ -544,6 +542,7 @@ struct Plan {
     PlanKind kind;
     bool vec;                  // rows: 16-byte vectors
     int binary_op;             // PLAN_ROWS_BINARY
+    int passes;                // PLAN_ROWS_BINARY: units per block (2, 4 or 8)
     int nsrc;
     unsigned grid;
     RowsArgs rows;

@@ -204,19 +204,11 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     }
     if (rows_ok) {
         constexpr int VMAX = 16 / sizeof(T);
-        // the drain decides the vector width; a misaligned source is read element by element
-        bool vec = cn.shape[last] % VMAX == 0 && c.drn % 16 == 0 && cn.base[0] % VMAX == 0;
-        for (int k = 0; k < last; k++) if (cn.stride[0][k] % VMAX != 0) vec = false;
+        // 16 bytes per lane whenever a row is a whole number of vectors (no alignment requirement)
+        const bool vec = cn.shape[last] % VMAX == 0;
         RowsArgs& A = plan.rows;
-        A.scalar_load = 0;
-        for (int j = 0; j < c.nsrc && vec; j++) {
-            if (cn.stride[j + 1][last] == 0) continue;      // one element per row: no alignment needed
-            bool aligned = c.src[j] % 16 == 0 && cn.base[j + 1] % VMAX == 0;
-            for (int k = 0; k < last; k++) if (cn.stride[j + 1][k] % VMAX != 0) aligned = false;
-            if (!aligned) A.scalar_load |= 1u << j;
-        }
         const int V = vec ? VMAX : 1;
-        const int passes = funset >= 2 ? 1 : 4;
+        int passes = funset >= 2 ? 1 : 4;
         A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
         A.streaming = streaming ? 1 : 0;
@@ -242,18 +234,23 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             for (int k = 0; k < last; k++) A.stride[o][k] = (int)cn.stride[o][last - 1 - k];
         }
         A.vec = V;
-        A.simple_loads = (funset < 2 && A.scalar_load == 0 && A.const_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
+        A.simple_loads = (funset < 2 && A.const_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel
         if (A.simple_loads && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
             prog.op[1] == I_BIN && prog.src[1] == 1 && prog.arg[1] <= NK_OP_DIV) {
             plan.kind = PLAN_ROWS_BINARY;
             plan.binary_op = prog.arg[1];
+            if (vec) {
+                static const int env_passes = [] { const char* v = getenv("NK_BINARY_PASSES"); return v && *v ? atoi(v) : 8; }();
+                passes = env_passes == 2 || env_passes == 4 ? env_passes : 8;
+            }
+            plan.passes = passes;
         }
         plan.vec = vec;
-        plan.grid = (unsigned)((n_units + passes - 1) / passes);     // one block per PASSES units, no grid-stride loop
+        plan.grid = (unsigned)((n_units + passes - 1) / passes);     // one block per `passes` units, no grid-stride loop
         set_path(plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary")
-                                               : vec ? (A.scalar_load ? "rows_vec_unaligned_src" : "rows_vec") : "rows");
+                                               : vec ? "rows_vec" : "rows");
         done = true;
     }
 

@@ -317,6 +317,52 @@ class HipDevice:
         _lib.check(self._lib.nk_fused(self.handle, prog, len(program) // 2, cs, len(consts), _dtype_code(drn.dtype), drn.ndc.rank,
                                       ops[0][0], ops[0][2], len(srcs), ptrs, cfgs, drn.ndc.size))
 
+    def prepared(self, entry: str, *args):
+        """Binds one C-ABI call with its arguments converted once; the returned callable repeats exactly
+        that launch (used where the per-call cost of building descriptors would distort a measurement).
+        Tensors are passed as (pointer, descriptor) pairs by the caller-facing helpers below."""
+        fn = getattr(self._lib, entry)
+        keep = args                      # keeps descriptor arrays alive
+        def call():
+            _lib.check(fn(*keep))
+        return call
+
+    def prepared_launch(self, kind: str, *a):
+        """kind: 'broadcast' | 'elementwise' (op, d, drn, x, y) | 'activation' (fun, d, drn, x) |
+        'fused' (program, consts, drn, srcs) | 'convolution' (d, drn, x, y) | 'matmul' (row_major, M, K, N, x, y, z)"""
+        h = C.c_uint64(self.handle)
+        if kind in ("broadcast", "elementwise"):
+            op, d, drn, x, y = a
+            (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = ops = self._ops(drn, x, y)
+            call = self.prepared("nk_" + kind, h, _lib.OP[op], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, C.c_int64(drn.ndc.size))
+        elif kind == "activation":
+            fun, d, drn, x = a
+            (p0, k0, c0), (p1, k1, c1) = ops = self._ops(drn, x)
+            call = self.prepared("nk_activation", h, _lib.FUN[fun], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, C.c_int64(drn.ndc.size))
+        elif kind == "convolution":
+            d, drn, x, y = a
+            (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = ops = self._ops(drn, x, y)
+            call = self.prepared("nk_convolution", h, d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, C.c_int64(drn.ndc.size))
+        elif kind == "matmul":
+            rm, M, K, N, x, y, z = a
+            ops = None
+            call = self.prepared("nk_matmul", h, _dtype_code(z.dtype), _lib.ROW_MAJOR if rm else _lib.COLUMN_MAJOR, C.c_int64(M), C.c_int64(K), C.c_int64(N),
+                                 C.c_uint64(x._data.ptr), C.c_uint64(y._data.ptr), C.c_uint64(z._data.ptr))
+        elif kind == "fused":
+            program, consts, drn, srcs = a
+            ops = self._ops(drn, *srcs)
+            prog = (C.c_int32 * len(program))(*program)
+            cs = (C.c_double * max(1, len(consts)))(*consts)
+            ptrs = (C.c_uint64 * max(1, len(srcs)))(*[o[0].value for o in ops[1:]])
+            cfgs = (C.POINTER(C.c_int32) * max(1, len(srcs)))(*[o[2] for o in ops[1:]])
+            call = self.prepared("nk_fused", h, prog, len(program) // 2, cs, len(consts), _dtype_code(drn.dtype), drn.ndc.rank,
+                                 ops[0][0], ops[0][2], len(srcs), ptrs, cfgs, C.c_int64(drn.ndc.size))
+            ops = (ops, prog, cs, ptrs, cfgs)
+        else:
+            raise IllegalArgumentException(f"unknown launch kind '{kind}'")
+        call._keepalive = ops
+        return call
+
     # timing on the device stream
     def event(self) -> int:
         e = C.c_uint64(0)
