@@ -414,8 +414,11 @@ __global__ __launch_bounds__(256) void canon_kernel(CanonArgs A, Prog P, LightPr
 // ---- tile_transpose kernel ----------------------------------------------------------------------------
 // Collapsed axis `pax` (not the innermost) is the contiguous one of the sources flagged in `turned`; all
 // other operands are contiguous or constant along the innermost axis.  A block owns a 64 (pax) x 64
-// (innermost) tile for one combination of the remaining axes; turned sources are read with lanes along
-// pax and handed to the lanes along the innermost axis through a padded LDS tile.
+// (innermost) tile for one combination of the remaining axes.  Turned sources are read with 16-byte
+// accesses along pax into one padded LDS tile each (all loads in flight before the single barrier) and
+// handed to the lanes that own 16-byte pieces along the innermost axis; the drain is written with
+// 16-byte stores.  LDS rows have a pitch of 65 elements, which makes both the row-wise writes and the
+// column-wise reads conflict-free.
 struct TileArgs {
     int rank;
     int nsrc;
@@ -425,6 +428,7 @@ struct TileArgs {
     unsigned tiles_p, tiles_l;
     unsigned n_blocks;
     int streaming;
+    int careful;                            // some direct operand is constant along the innermost axis: no vector path
     FastDiv div_tiles_l, div_tiles_p;
     FastDiv outer[NK_MAX_RANK];             // extents of the remaining axes
     int64_t base[MAX_OPERANDS];
@@ -433,65 +437,128 @@ struct TileArgs {
 
 template <typename T, int NSRC, int FUNSET>
 __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
-    __shared__ T tile[64][65];
+    constexpr int VEC = 16 / sizeof(T);            // elements per 16-byte access
+    constexpr int LPR = 64 / VEC;                  // lanes that cover one 64-element tile row
+    constexpr int RPI = 256 / LPR;                 // tile rows covered by one access of the whole block
+    constexpr int NIT = 64 / RPI;                  // accesses per thread and operand
+    constexpr int EPT = NIT * VEC;                 // elements per thread (16)
+    __shared__ T tiles[NSRC][64][65];
     const int last = A.rank - 1;
-    const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;   // 64 x 4
-    for (unsigned blk = blockIdx.x; blk < A.n_blocks; blk += gridDim.x) {
-        unsigned r = blk;
-        unsigned q = A.div_tiles_l.div(r);
-        const unsigned tl = r - q * A.tiles_l; r = q;
-        q = A.div_tiles_p.div(r);
-        const unsigned tp = r - q * A.tiles_p; r = q;
-        int64_t off[NSRC + 1];
+    const unsigned q = threadIdx.x % LPR, r = threadIdx.x / LPR;
+
+    unsigned rest = blockIdx.x;
+    unsigned d = A.div_tiles_l.div(rest);
+    const unsigned tl = rest - d * A.tiles_l; rest = d;
+    d = A.div_tiles_p.div(rest);
+    const unsigned tp = rest - d * A.tiles_p; rest = d;
+    int64_t off[NSRC + 1];
 #pragma unroll
-        for (int o = 0; o <= NSRC; o++) off[o] = A.base[o];
-        for (int k = last - 1; k >= 0; k--) {
-            if (k == A.pax) continue;
-            const unsigned qq = A.outer[k].div(r);
-            const unsigned idx = r - qq * A.outer[k].d;
-            r = qq;
+    for (int o = 0; o <= NSRC; o++) off[o] = A.base[o];
+    for (int k = last - 1; k >= 0; k--) {
+        if (k == A.pax) continue;
+        const unsigned qq = A.outer[k].div(rest);
+        const unsigned idx = rest - qq * A.outer[k].d;
+        rest = qq;
 #pragma unroll
-            for (int o = 0; o <= NSRC; o++) off[o] += (int64_t)idx * A.stride[o][k];
+        for (int o = 0; o <= NSRC; o++) off[o] += (int64_t)idx * A.stride[o][k];
+    }
+    const unsigned p0 = tp * 64, l0 = tl * 64;
+    const int64_t dP = A.stride[0][A.pax];
+    T x[NSRC][EPT];
+    T out[EPT];
+
+    // whole tile inside the tensor, every operand either along pax or along the innermost axis:
+    // 16-byte accesses on both sides, one barrier
+    if (p0 + 64 <= A.P && l0 + 64 <= A.L && !A.careful) {
+#pragma unroll
+        for (int j = 0; j < NSRC; j++) {
+            if (j < A.nsrc && ((A.turned >> j) & 1u)) {
+                const T* sp = (const T*)srcs.p[j] + off[j + 1] + p0 + q * VEC;           // stride 1 along pax
+                const int64_t sL = A.stride[j + 1][last];
+#pragma unroll
+                for (int it = 0; it < NIT; it++) {
+                    const unsigned ll = r + RPI * it;
+                    T v[VEC];
+                    load_vec<T, VEC>(v, sp + (int64_t)(l0 + ll) * sL);
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) tiles[j][ll][q * VEC + e] = v[e];
+                }
+            }
         }
-        const unsigned p0 = tp * 64, l0 = tl * 64;
-        T x[NSRC][16];
+        __syncthreads();
 #pragma unroll
         for (int j = 0; j < NSRC; j++) {
             if (j < A.nsrc) {
-                const T* sp = (const T*)srcs.p[j] + off[j + 1];
-                const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
                 if ((A.turned >> j) & 1u) {
-                    __syncthreads();
 #pragma unroll
-                    for (int it = 0; it < 16; it++) {
-                        const unsigned l = l0 + ty + 4 * it, p = p0 + tx;
-                        if (l < A.L && p < A.P) tile[ty + 4 * it][tx] = sp[(int64_t)p * sP + (int64_t)l * sL];
-                    }
-                    __syncthreads();
+                    for (int it = 0; it < NIT; it++)
 #pragma unroll
-                    for (int it = 0; it < 16; it++) x[j][it] = tile[tx][ty + 4 * it];
+                        for (int e = 0; e < VEC; e++) x[j][it * VEC + e] = tiles[j][q * VEC + e][r + RPI * it];
                 } else {
+                    const T* sp = (const T*)srcs.p[j] + off[j + 1] + l0 + q * VEC;       // stride 1 along the innermost axis
+                    const int64_t sP = A.stride[j + 1][A.pax];
 #pragma unroll
-                    for (int it = 0; it < 16; it++) {
-                        const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
-                        x[j][it] = (p < A.P && l < A.L) ? sp[(int64_t)p * sP + (int64_t)l * sL] : T(0);
+                    for (int it = 0; it < NIT; it++) {
+                        T (&xv)[VEC] = *reinterpret_cast<T (*)[VEC]>(&x[j][it * VEC]);
+                        load_vec<T, VEC>(xv, sp + (int64_t)(p0 + r + RPI * it) * sP);
                     }
                 }
             } else {
 #pragma unroll
-                for (int it = 0; it < 16; it++) x[j][it] = T(0);
+                for (int e = 0; e < EPT; e++) x[j][e] = T(0);
             }
         }
-        const int64_t dP = A.stride[0][A.pax], dL = A.stride[0][last];
-        T out[16];
-        run_any<T, 16, NSRC, FUNSET>(P, LP, x, out);
+        run_any<T, EPT, NSRC, FUNSET>(P, LP, x, out);
+        T* dp = drn + off[0] + l0 + q * VEC;
 #pragma unroll
-        for (int it = 0; it < 16; it++) {
-            const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
-            if (p < A.P && l < A.L) {
-                T* dst = drn + off[0] + (int64_t)p * dP + (int64_t)l * dL;
-                if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
+        for (int it = 0; it < NIT; it++) {
+            T (&ov)[VEC] = *reinterpret_cast<T (*)[VEC]>(&out[it * VEC]);
+            store_vec<T, VEC>(dp + (int64_t)(p0 + r + RPI * it) * dP, ov, A.streaming != 0);
+        }
+        return;
+    }
+
+    // edge tiles and operands that are constant along the innermost axis: element by element, bounds checked
+    const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+    for (int j = 0; j < NSRC; j++) {
+        if (j < A.nsrc && ((A.turned >> j) & 1u)) {
+            const T* sp = (const T*)srcs.p[j] + off[j + 1];
+            const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
+            for (int it = 0; it < 16; it++) {
+                const unsigned l = l0 + ty + 4 * it, p = p0 + tx;
+                if (l < A.L && p < A.P) tiles[j][ty + 4 * it][tx] = sp[(int64_t)p * sP + (int64_t)l * sL];
             }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NSRC; j++) {
+        if (j < A.nsrc) {
+            if ((A.turned >> j) & 1u) {
+#pragma unroll
+                for (int it = 0; it < 16; it++) x[j][it] = tiles[j][tx][ty + 4 * it];
+            } else {
+                const T* sp = (const T*)srcs.p[j] + off[j + 1];
+                const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
+#pragma unroll
+                for (int it = 0; it < 16; it++) {
+                    const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
+                    x[j][it] = (p < A.P && l < A.L) ? sp[(int64_t)p * sP + (int64_t)l * sL] : T(0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < 16; it++) x[j][it] = T(0);
+        }
+    }
+    run_any<T, EPT, NSRC, FUNSET>(P, LP, x, out);
+#pragma unroll
+    for (int it = 0; it < 16; it++) {
+        const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
+        if (p < A.P && l < A.L) {
+            T* dst = drn + off[0] + (int64_t)p * dP + l;
+            if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
         }
     }
 }

@@ -256,7 +256,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
 
     // tile_transpose: the drain and some operands run along the innermost axis, the others along one
     // common outer axis
-    if (!done && cn.stride[0][last] == 1 && cn.rank >= 2) {
+    if (!done && funset < 2 && cn.stride[0][last] == 1 && cn.rank >= 2) {
         int pax = -1;
         unsigned turned = 0;
         bool ok = true;
@@ -272,6 +272,9 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             TileArgs& A = plan.tile;
             A.rank = cn.rank; A.nsrc = c.nsrc; A.pax = pax; A.turned = turned;
             A.streaming = streaming ? 1 : 0;
+            A.careful = 0;
+            for (int j = 0; j < c.nsrc; j++)
+                if (!((turned >> j) & 1u) && cn.stride[j + 1][last] == 0) A.careful = 1;
             A.P = (unsigned)cn.shape[pax]; A.L = (unsigned)cn.shape[last];
             A.tiles_p = (A.P + 63) / 64; A.tiles_l = (A.L + 63) / 64;
             uint64_t nb = (uint64_t)A.tiles_p * A.tiles_l;
@@ -288,7 +291,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
                     for (int k = 0; k < cn.rank; k++) A.stride[o][k] = cn.stride[o][k];
                 }
                 plan.kind = PLAN_TILE;
-                plan.grid = grid_for(dev, nb);
+                plan.grid = (unsigned)nb;                    // one block per tile
                 set_path("tile_transpose");
                 done = true;
             }
