@@ -23,6 +23,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
+# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
+# against a plain 1 GiB copy): profiles/rows_binary_kernel_broadcast_c2.md
+C2_TRAFFIC_BYTES = 4317140700
 
 
 def event_time_ms(dev, launch, reps):
@@ -42,6 +45,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the figures of the other configurations")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run one plain 1 GiB device-to-device copy (a copy kernel of known size), so that a "
+                         "rocprofv3 --pmc run of this command holds a reference for FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: this build has no multi-GPU path (every kernel shards without "
@@ -73,6 +79,8 @@ def main():
         launch_add()
         launch_mul()
 
+    if args.calibrate:
+        _lib.check(dev._lib.nk_d2d(dev.handle, out._data.ptr, 0, out._data.ptr, 2 << 30, 1 << 30))
     for _ in range(args.warmup):
         step()
     dev.sync()
@@ -90,7 +98,8 @@ def main():
     k_ms = 0.5 * (k_add + k_mul)
     achieved = bytes_per_launch / (k_ms * 1e-3) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": f"rows_kernel<float,4> ({path})",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_TRAFFIC_BYTES if path == "rows_vec_binary" else None,
+                "kernel": f"nk::rows_binary_kernel<float, 4, 8> ({path})",
                 "launch_ms": round(k_ms, 4), "algorithmic_bytes": bytes_per_launch}
 
     # spot check of the timed output against numpy (the full parity tests live in tests/)
