@@ -1,0 +1,180 @@
+"""The five benchmark configurations at their full sizes, through the C ABI.  Where the oracle finishes in
+seconds the whole result is compared; the 4 GiB broadcast and the 4096^3 matmul are checked through
+sampled slabs plus size-independent properties (linearity, exactness on integer data, a checksum)."""
+import numpy as np
+import pytest
+
+from helpers import RTOL, assert_bits
+from neureka_amd import Function, NDConfiguration, Tensor, _lib
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+def say(*a):
+    print("[case]", *a, flush=True)
+
+
+def on(device, array, shape=None):
+    array = np.asarray(array)
+    return Tensor.of(array.dtype, shape if shape is not None else array.shape, array.reshape(-1)).to(device)
+
+
+def free(device, *tensors):
+    for t in tensors:
+        if device.has(t):
+            device.free(t)
+
+
+def test_config1_conv2d_64x64_3x3(device, orc):
+    say("C1 conv2d")
+    rng = np.random.default_rng(1)
+    x = rng.uniform(-1, 1, (64, 64)).astype(f32); k = rng.uniform(-1, 1, (3, 3)).astype(f32)
+    y = on(device, x).conv(on(device, k))
+    assert y.shape == (62, 62)
+    want = orc.simple_conv2d(x.reshape(-1), k.reshape(-1), 64, 64, 3, 3)          # the path the reference takes for this config
+    bound = 1e-5 * orc.simple_conv2d(np.abs(x).reshape(-1), np.abs(k).reshape(-1), 64, 64, 3, 3)
+    assert (np.abs(y.items - want) <= bound).all()
+    general = orc.convolve(np.zeros(62 * 62, dtype=f32), orc.dense_cfg([62, 62]), x.reshape(-1), orc.dense_cfg([64, 64]), k.reshape(-1), orc.dense_cfg([3, 3]))
+    assert_bits(y.items, general, "general path order")
+
+
+@pytest.mark.parametrize("dt,s1,s2", [("f32", (1024, 1, 512), (1, 2048, 512)), ("f64", (256, 1, 512), (1, 1024, 512))])
+def test_config2_broadcast_full_size(device, orc, dt, s1, s2):
+    say("C2 broadcast", dt)
+    T = np.dtype(dt.replace("f", "float"))
+    rng = np.random.default_rng(2)
+    a = rng.uniform(-1, 1, s1).astype(T); b = rng.uniform(-1, 1, s2).astype(T)
+    ta, tb = on(device, a), on(device, b)
+    so = (s1[0], s2[1], 512)
+    out = Tensor._on_device(device, T, so)
+    for op, f in (("add", np.add), ("multiply", np.multiply)):
+        device.launch_broadcast(op, -1, out, ta, tb)
+        assert _lib.last_path() == "rows_vec_binary"
+        got = out.getData().reshape(so)
+        # slabs against the oracle (bit for bit) ...
+        for o0 in (0, 1, so[0] // 2, so[0] - 1):
+            want = orc.broadcast(op, -1, np.zeros(so[1] * 512, dtype=T), orc.dense_cfg((1, so[1], 512)), a[o0].reshape(-1).copy(),
+                                 orc.dense_cfg((1, 1, 512)), b.reshape(-1), orc.dense_cfg(s2))
+            assert_bits(got[o0].reshape(-1), want, f"{op} slab {o0}")
+        # ... and the whole 4 GiB / 1 GiB against numpy broadcasting, slab by slab to bound host memory
+        for lo in range(0, so[0], 64):
+            assert_bits(got[lo:lo + 64], f(a[lo:lo + 64], b), f"{op} rows {lo}")
+        del got
+    free(device, out, ta, tb)
+
+
+def _chain_oracle(orc, bases, cfgs, shape, workers=16):
+    n = int(np.prod(shape))
+    oc = orc.dense_cfg(list(shape))
+    s = orc.activation("sig", -1, np.zeros(n, dtype=f32), oc, bases[0], cfgs[0], workers=workers)
+    m = orc.elementwise("multiply", -1, np.zeros(n, dtype=f32), oc, s, oc, bases[1], cfgs[1], workers=workers)
+    p = orc.elementwise("add", -1, np.zeros(n, dtype=f32), oc, m, oc, bases[2], cfgs[2], workers=workers)
+    want = orc.activation("tanh", -1, np.zeros(n, dtype=f32), oc, p, oc, workers=workers)
+    return want, m
+
+
+def _check_chain(got, want, m, c_view):
+    bound = RTOL[np.dtype(f32)] * (np.abs(m) + np.abs(c_view) + np.abs(want)) + 1e-10
+    bad = np.abs(got - want) > bound
+    assert not bad.any(), f"{bad.sum()} of {bad.size} outside the bound; first {np.flatnonzero(bad)[:3]}"
+
+
+def test_config3_chain_contiguous_permuted_sliced(device, orc):
+    """tanh(sig(a)*b+c): 2^26 contiguous elements, the permuted [4096,16384] view of row-major [16384,4096],
+    and the slice [::2, 1:8193] of [8192,16384]; fused kernel against the oracle's four-kernel sequence."""
+    rng = np.random.default_rng(3)
+    fn = Function.of("tanh(sig(I[0])*I[1]+I[2])")
+    fused = device.optimizedFunctionOf(fn, "chain")
+    n = 1 << 26
+    bases = [rng.standard_normal(n).astype(f32) for _ in range(3)]
+    tens = [on(device, b, (16384, 4096)) for b in bases]
+    say("C3 contiguous")
+    flat = [Tensor(f32, NDConfiguration.ofShape((n,)), None) for _ in tens]
+    for v, t in zip(flat, tens): v._set_data(t._data, device)
+    got = fused(*flat)
+    assert _lib.last_path() == "rows_vec"
+    cfg1 = orc.dense_cfg([n])
+    want, m = _chain_oracle(orc, bases, [cfg1] * 3, (n,))
+    _check_chain(got.items, want, m, bases[2])
+    free(device, got)
+    say("C3 permuted")
+    views = [t.T() for t in tens]
+    got = fused(*views)
+    assert _lib.last_path() == "tile_transpose" and got.shape == (4096, 16384)
+    cfgs = [v.ndc.asInlineArray() for v in views]
+    want, m = _chain_oracle(orc, bases, cfgs, (4096, 16384))
+    _check_chain(got.items, want, m, bases[2].reshape(16384, 4096).T.reshape(-1))
+    unf = fn(*views)                                                     # the reference's four launches
+    assert_bits(unf.items, got.items, "fused vs unfused, permuted")
+    free(device, got, unf, *views, *tens)
+    say("C3 sliced")
+    parents = [rng.standard_normal(8192 * 16384).astype(f32) for _ in range(3)]
+    ptens = [on(device, p, (8192, 16384)) for p in parents]
+    views = [t[::2, 1:8193] for t in ptens]
+    assert views[0].ndc.asInlineArray().tolist() == [4096, 8192, 16384, 1, 8192, 1, 0, 1, 2, 1]
+    got = fused(*views)
+    assert _lib.last_path() == "rows_vec" and got.shape == (4096, 8192)
+    cfgs = [v.ndc.asInlineArray() for v in views]
+    want, m = _chain_oracle(orc, parents, cfgs, (4096, 8192))
+    _check_chain(got.items, want, m, parents[2].reshape(8192, 16384)[::2, 1:8193].reshape(-1))
+    free(device, got, *views, *ptens)
+
+
+@pytest.mark.parametrize("mkn", [(4096, 4096, 4096), (65536, 256, 256)])
+def test_config4_matmul_full_size(device, mkn):
+    M, K, N = mkn
+    rng = np.random.default_rng(4)
+    say("C4 matmul integer data (exact)", mkn)
+    A = rng.integers(-3, 4, (M, K)).astype(f32); B = rng.integers(-3, 4, (K, N)).astype(f32)
+    ta, tb = on(device, A), on(device, B)
+    c = ta.matMul(tb)
+    assert _lib.last_path() == "mfma"
+    got = c.items.reshape(M, N)
+    rows = rng.choice(M, 48, replace=False)
+    assert (got[rows] == A[rows].astype(np.float64) @ B.astype(np.float64)).all()
+    # checksum of checksums over the whole product: 1^T (A B) 1 = (1^T A)(B 1), exact in float64 for this data
+    assert got.sum(dtype=np.float64) == float(A.sum(axis=0, dtype=np.float64) @ B.sum(axis=1, dtype=np.float64))
+    free(device, c, ta, tb)
+    say("C4 matmul uniform data (norm-wise 1e-5)", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(f32); B = rng.uniform(-1, 1, (K, N)).astype(f32)
+    ta, tb = on(device, A), on(device, B)
+    c = ta.matMul(tb)
+    got = c.items.reshape(M, N)
+    ref = A[rows].astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-5 * (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(got[rows] - ref) <= bound).all()
+    # linearity: (2A) B == 2 (A B) bit for bit (scaling by a power of two is exact)
+    c2 = on(device, 2 * A).matMul(tb)
+    assert_bits(c2.items, 2 * c.items, "linearity")
+    free(device, c, c2, ta, tb)
+
+
+def test_config5_conv_forward_and_backward_full_size(device, orc):
+    """[64,256,256] x [64,5,5] -> [1,252,252] with autograd: input and kernel gradients."""
+    rng = np.random.default_rng(5)
+    xs, ks, ys = [64, 256, 256], [64, 5, 5], [1, 252, 252]
+    x = (rng.standard_normal(xs) * 0.1).astype(f32); k = (rng.standard_normal(ks) * 0.1).astype(f32)
+    e = rng.standard_normal(ys).astype(f32)
+    tx = on(device, x).setRqsGradient(True); tk = on(device, k).setRqsGradient(True)
+    say("C5 forward")
+    y = tx.conv(tk)
+    assert _lib.last_path() == "chan_fwd" and list(y.shape) == ys
+    dc = orc.dense_cfg
+    want = orc.convolve(np.zeros(252 * 252, dtype=f32), dc(ys), x.reshape(-1), dc(xs), k.reshape(-1), dc(ks), workers=16)
+    babs = orc.convolve(np.zeros(252 * 252), dc(ys), np.abs(x).astype(np.float64).reshape(-1), dc(xs), np.abs(k).astype(np.float64).reshape(-1), dc(ks), workers=16)
+    assert (np.abs(y.items.astype(np.float64) - want) <= 1e-5 * babs).all()
+    say("C5 backward")
+    y.backward(on(device, e))
+    gx, gk = tx.gradient, tk.gradient
+    assert list(gx.shape) == xs and list(gk.shape) == ks
+    want = orc.deconvolve(np.zeros(x.size, dtype=f32), dc(xs), k.reshape(-1), dc(ks), e.reshape(-1), dc(ys), fast=True, workers=16)
+    babs = orc.deconvolve(np.zeros(x.size), dc(xs), np.abs(k).astype(np.float64).reshape(-1), dc(ks), np.abs(e).astype(np.float64).reshape(-1), dc(ys), fast=True, workers=16)
+    assert (np.abs(gx.items.astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all()
+    want = orc.deconvolve(np.zeros(k.size, dtype=f32), dc(ks), x.reshape(-1), dc(xs), e.reshape(-1), dc(ys), fast=True, workers=16)
+    babs = orc.deconvolve(np.zeros(k.size), dc(ks), np.abs(x).astype(np.float64).reshape(-1), dc(xs), np.abs(e).astype(np.float64).reshape(-1), dc(ys), fast=True, workers=16)
+    assert (np.abs(gk.items.astype(np.float64) - want) <= 1e-5 * babs).all()
+    # adjoint identity in float64: <e, x (*) k> = <dL/dx, x> = <dL/dk, k>
+    lhs = float(np.dot(e.reshape(-1).astype(np.float64), y.items.astype(np.float64)))
+    assert abs(float(np.dot(gx.items.astype(np.float64), x.reshape(-1).astype(np.float64))) - lhs) <= 1e-4 * abs(lhs) + 1e-6
+    assert abs(float(np.dot(gk.items.astype(np.float64), k.reshape(-1).astype(np.float64))) - lhs) <= 1e-4 * abs(lhs) + 1e-6
