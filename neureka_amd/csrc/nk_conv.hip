@@ -10,16 +10,13 @@
 //   literal        any rank / layout / view: one thread per drain element, the sum in the reference's
 //                  order with rounded products, bit-identical to the CPU device.  The gradient only
 //                  visits the e-range that can pass the bounds test (skipped terms add +0).
-//   chan_fwd       rank 3, dense row-major, full reduction over axis 0 (channels):
-//                  [C,H,W] x [C,kh,kw] -> [1,H-kh+1,W-kw+1].  Channels are split over the four
-//                  wavefronts of a block and over `splits` blocks; each wavefront stages its channel's
-//                  input halo tile in LDS, the kernel taps sit in LDS too; partial sums are reduced
-//                  across wavefronts in LDS and across blocks by a second pass over a scratch buffer.
-//   chan_dx        gradient w.r.t. the [C,H,W] operand: per channel a "full" correlation of the error
-//                  with that channel's kh x kw taps, error tile + halo staged in LDS.
-//   chan_dk        gradient w.r.t. the [C,kh,kw] operand: per (channel, tap) a dot product of the
-//                  shifted input plane with the error, block-wide reduction (wavefront shuffles + LDS).
+//   chan_fwd/dx/dk rank 3, dense row-major f32, full reduction over axis 0 (channels), square taps of extent
+//                  2, 3, 4, 5 or 7: [C,H,W] x [C,k,k] -> [1,H-k+1,W-k+1] and its two gradients, register
+//                  sliding-window kernels (see below); sums are re-ordered, results agree with the reference
+//                  norm-wise (1e-5 * sum |a||b| per output).
 #include "nk_internal.h"
+#include <type_traits>
+#include <cstdlib>
 
 namespace nk {
 
@@ -100,198 +97,305 @@ __global__ __launch_bounds__(256) void conv_bwd_literal(ConvArgs A, T* __restric
 }
 
 // ------------------------------------------------------------------------------------------------
-// chan_fwd: out[y][x] = sum_c sum_ky sum_kx in[c][y+ky][x+kx] * w[c][ky][kx]
+// Channel convolution, dense row-major f32: big [C,H,W], taps [C,KH,KW], out/err [1,OH,OW], OH = H-KH+1.
+//
+// All three kernels give a lane CX = 4 adjacent columns and a strip of rows and keep the window they work
+// on in registers: the 4 + KW - 1 values a row contributes are reused across the KW horizontal and the KH
+// vertical shifts without touching memory again.  Row bases are wave-uniform (scalar unit); a lane adds a
+// 32-bit byte offset computed once, so the vector unit spends its issue slots on multiply-adds instead of
+// 64-bit address arithmetic.  Dead lanes and rows past the end read clamped, valid addresses and their
+// results are dropped, which keeps every load unconditional.  The per-channel taps are wave-uniform and come
+// in through scalar loads.  Extents of the taps are template parameters so every loop is unrolled and every
+// accumulator lives in a register.  Work is split over channel groups (or strips) until there are enough
+// wavefronts to fill the machine; partial results go to a device-owned scratch buffer and a second pass
+// adds them in a fixed order (deterministic, no atomics).
 struct ChanArgs {
-    int C, H, W, KH, KW, OH, OW;
-    int splits;          // channel groups (blocks along z)
-    int cps;             // channels per split
+    int C, H, W, OH, OW;
+    int cg;              // channels per group (grid z)
+    int col_blocks;      // 256-column blocks across the lane axis
 };
 
-constexpr int FT_Y = 16, FT_X = 64;      // output tile of chan_fwd
-constexpr int MAX_KH = 8, MAX_KW = 8;
-
-__device__ __forceinline__ void wave_lds_sync() {
-    // LDS traffic of one wavefront is processed in order; the fences keep the compiler from moving the
-    // accesses across this point, no block-wide barrier is needed for data private to a wavefront
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// TKH/TKW > 0: tap extents known at compile time (the column of the halo a lane needs is kept in
-// registers and reused by all ky); 0: run-time extents up to MAX_KH x MAX_KW.
-template <typename T, int TKH, int TKW>
-__global__ __launch_bounds__(256) void conv_chan_fwd(ChanArgs g, const T* __restrict__ in, const T* __restrict__ w,
-                                                     T* __restrict__ partial) {
-    constexpr int HP = FT_X + MAX_KW;               // halo pitch in elements
-    constexpr int HR = FT_Y + MAX_KH - 1;
-    __shared__ T halo[4][HR * HP];
-    __shared__ T taps[4][MAX_KH * MAX_KW];
-    __shared__ T red[4][FT_Y * FT_X];
-
-    const int KH = TKH ? TKH : g.KH, KW = TKW ? TKW : g.KW;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int x0 = blockIdx.x * FT_X, y0 = blockIdx.y * FT_Y;
-    const int c_begin = blockIdx.z * g.cps;
-    int c_end = c_begin + g.cps; if (c_end > g.C) c_end = g.C;
-    const int hw = FT_X + KW - 1, hh = FT_Y + KH - 1;
-
-    T acc[FT_Y];
-#pragma unroll
-    for (int r = 0; r < FT_Y; r++) acc[r] = T(0);
-
-    // a lane owns output column x0 + lane for all FT_Y rows of the tile; a wavefront owns every 4th
-    // channel of the block's channel group
-    for (int c = c_begin + wave; c < c_end; c += 4) {
-        const T* plane = in + (int64_t)c * g.H * g.W;
-        for (int r = 0; r < hh; r++) {
-            const int y = y0 + r;
-            for (int xx = lane; xx < hw; xx += 64) {
-                const int x = x0 + xx;
-                T v = T(0);
-                if (y < g.H && x < g.W) v = plane[(int64_t)y * g.W + x];
-                halo[wave][r * HP + xx] = v;
-            }
-        }
-        if (lane < KH * KW) taps[wave][lane] = w[(int64_t)c * KH * KW + lane];
-        wave_lds_sync();
-        if constexpr (TKH > 0) {
-#pragma unroll
-            for (int kx = 0; kx < TKW; kx++) {
-                T col[FT_Y + TKH - 1];
-#pragma unroll
-                for (int r = 0; r < FT_Y + TKH - 1; r++) col[r] = halo[wave][r * HP + lane + kx];
-#pragma unroll
-                for (int ky = 0; ky < TKH; ky++) {
-                    const T t = taps[wave][ky * TKW + kx];
-#pragma unroll
-                    for (int r = 0; r < FT_Y; r++) acc[r] = __builtin_fma(col[r + ky], t, acc[r]);
-                }
-            }
-        } else {
-            for (int ky = 0; ky < KH; ky++)
-                for (int kx = 0; kx < KW; kx++) {
-                    const T t = taps[wave][ky * KW + kx];
-#pragma unroll
-                    for (int r = 0; r < FT_Y; r++) acc[r] = __builtin_fma(halo[wave][(r + ky) * HP + lane + kx], t, acc[r]);
-                }
-        }
-        wave_lds_sync();
-    }
-    // reduce the four wavefronts
-#pragma unroll
-    for (int r = 0; r < FT_Y; r++) red[wave][r * FT_X + lane] = acc[r];
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < FT_Y * FT_X; idx += 256) {
-        const int r = idx / FT_X, xx = idx % FT_X;
-        const int y = y0 + r, x = x0 + xx;
-        if (y < g.OH && x < g.OW) {
-            T s = (red[0][idx] + red[1][idx]) + (red[2][idx] + red[3][idx]);
-            partial[((int64_t)blockIdx.z * g.OH + y) * g.OW + x] = s;
-        }
-    }
-}
-
 template <typename T>
-__global__ __launch_bounds__(256) void conv_chan_fwd_reduce(int splits, int n, const T* __restrict__ partial, T* __restrict__ out) {
+__global__ __launch_bounds__(256) void conv_partial_reduce(int parts, int n, const T* __restrict__ partial, T* __restrict__ out) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     T s = T(0);
-    for (int k = 0; k < splits; k++) s = s + partial[(int64_t)k * n + i];
+    int k = 0;
+    for (; k + 8 <= parts; k += 8) {              // eight independent loads in flight, added in a fixed order
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = partial[(int64_t)(k + u) * n + i];
+#pragma unroll
+        for (int u = 0; u < 8; u++) s = s + v[u];
+    }
+    for (; k < parts; k++) s = s + partial[(int64_t)k * n + i];
     out[i] = s;
 }
 
-// chan_dx: dx[c][y][x] = sum_ky sum_kx w[c][ky][kx] * err[y-ky][x-kx]   (terms with err out of range vanish)
-constexpr int DT_Y = 16, DT_X = 64;
+// few outputs, many partials (the tap gradient): one wavefront per output, lanes stride over the partials
 template <typename T>
-__global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restrict__ err, const T* __restrict__ w,
-                                                    T* __restrict__ dx) {
-    constexpr int EP = DT_X + MAX_KW;
-    constexpr int ER = DT_Y + MAX_KH - 1;
-    __shared__ T etile[ER * EP];
-    __shared__ T taps[64 * MAX_KH * MAX_KW / 4];   // taps of the channels this block handles (up to 16)
-    const int x0 = blockIdx.x * DT_X, y0 = blockIdx.y * DT_Y;
-    const int c_begin = blockIdx.z * g.cps;
-    int c_end = c_begin + g.cps; if (c_end > g.C) c_end = g.C;
-    const int ew = DT_X + g.KW - 1, eh = DT_Y + g.KH - 1;
-    // error halo: rows y0-(KH-1) .. y0+DT_Y-1, cols x0-(KW-1) .. x0+DT_X-1
-    for (int idx = threadIdx.x; idx < eh * ew; idx += 256) {
-        const int r = idx / ew, cc = idx % ew;
-        const int y = y0 - (g.KH - 1) + r, x = x0 - (g.KW - 1) + cc;
-        T v = T(0);
-        if (y >= 0 && y < g.OH && x >= 0 && x < g.OW) v = err[(int64_t)y * g.OW + x];
-        etile[r * EP + cc] = v;
-    }
-    const int ntaps = g.KH * g.KW;
-    for (int idx = threadIdx.x; idx < (c_end - c_begin) * ntaps; idx += 256) taps[idx] = w[(int64_t)c_begin * ntaps + idx];
-    __syncthreads();
-    const int lane_x = threadIdx.x & 63, wy = threadIdx.x >> 6;    // 4 row groups of DT_Y/4 rows
-    for (int c = c_begin; c < c_end; c++) {
-        const T* t = &taps[(c - c_begin) * ntaps];
-        T acc[DT_Y / 4];
+__global__ __launch_bounds__(256) void conv_partial_reduce_wide(int parts, int n, const T* __restrict__ partial, T* __restrict__ out) {
+    const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (i >= n) return;
+    T s = T(0);
+    for (int k = lane; k < parts; k += 64) s = s + partial[(int64_t)k * n + i];
 #pragma unroll
-        for (int r = 0; r < DT_Y / 4; r++) acc[r] = T(0);
-        for (int ky = 0; ky < g.KH; ky++)
-            for (int kx = 0; kx < g.KW; kx++) {
-                const T tv = t[ky * g.KW + kx];
+    for (int off = 32; off >= 1; off >>= 1) s += __shfl_down(s, off, 64);
+    if (lane == 0) out[i] = s;
+}
+
+constexpr int CX = 4;                       // columns per lane
+typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
+
+// one fused multiply-add in the operand's own precision (the bare builtin is the double one)
+__device__ __forceinline__ float fused_mad(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fused_mad(double a, double b, double c) { return __builtin_fma(a, b, c); }
+
+// Buffer addressing: a wave-uniform descriptor (base, extent in bytes) in scalar registers, a scalar byte
+// offset for the row and one 32-bit per-lane byte offset -- no 64-bit vector arithmetic per access.  The
+// extent must stay below 2^32 bytes (checked on the host).
+typedef __amdgpu_buffer_rsrc_t BufRsrc;
+__device__ __forceinline__ BufRsrc buffer_of(const float* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);      // raw buffer, 32-bit data format
+}
+__device__ __forceinline__ float buffer_load(BufRsrc r, unsigned lane_off, unsigned row_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_off, row_off, 0));
+}
+__device__ __forceinline__ f32x4u buffer_load4(BufRsrc r, unsigned lane_off, unsigned row_off) {
+    return __builtin_bit_cast(f32x4u, __builtin_amdgcn_raw_buffer_load_b128(r, lane_off, row_off, 0));
+}
+
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// forward: partial[z][y][x] = sum_{c in group z} sum_ky sum_kx in[c][y+ky][x+kx] * w[c][ky][kx]
+// block -> (256-column block, strip of R output rows, channel group); its four wavefronts take every fourth
+// channel of the group and are summed through LDS before the block writes its partial plane.
+template <typename T, int KH, int KW, int R>
+__global__ __launch_bounds__(256) void conv_chan_fwd(ChanArgs g, const T* __restrict__ in, const T* __restrict__ w, T* __restrict__ partial) {
+    __shared__ T red[4][R][64 * CX];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int x = blockIdx.x * (64 * CX) + lane * CX;            // first of the lane's CX output columns
+    const int xl = x < g.OW ? x : 0;                             // lanes without a valid column read column 0
+    const bool whole = xl + CX <= g.W;                           // false only for the ragged last lane of a row
+    unsigned off[CX + KW - 1];                                   // byte offsets inside a row, clamped to the row
 #pragma unroll
-                for (int r = 0; r < DT_Y / 4; r++) {
-                    const int ry = wy * (DT_Y / 4) + r;
-                    // err[y-ky][x-kx] -> tile row ry + (KH-1) - ky, col lane_x + (KW-1) - kx
-                    acc[r] = __builtin_fma(etile[(ry + g.KH - 1 - ky) * EP + lane_x + g.KW - 1 - kx], tv, acc[r]);
+    for (int e = 0; e < CX + KW - 1; e++) off[e] = (unsigned)clampi(xl + e, 0, g.W - 1) * (unsigned)sizeof(T);
+    const int y0 = blockIdx.y * R;
+    const int c0 = blockIdx.z * g.cg;
+    int c1 = c0 + g.cg; if (c1 > g.C) c1 = g.C;
+    T acc[R][CX];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int j = 0; j < CX; j++) acc[r][j] = T(0);
+    for (int c = c0 + wave; c < c1; c += 4) {
+        T wt[KH][KW];
+        const T* wc = w + (int64_t)c * (KH * KW);
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) wt[ky][kx] = wc[ky * KW + kx];
+        const BufRsrc plane = buffer_of(in + (int64_t)c * g.H * g.W, (unsigned)(g.H * g.W) * 4u);
+        T v[R + KH - 1][CX + KW - 1];
+#pragma unroll
+        for (int yy = 0; yy < R + KH - 1; yy++) {                // all loads of the window first: one wait for the lot
+            const int y = y0 + yy < g.H ? y0 + yy : g.H - 1;      // rows past the end only feed outputs that are not stored
+            const unsigned row = (unsigned)(y * g.W) * 4u;
+            if (whole) {
+                const f32x4u head = buffer_load4(plane, off[0], row);
+#pragma unroll
+                for (int e = 0; e < CX; e++) v[yy][e] = head[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < CX; e++) v[yy][e] = buffer_load(plane, off[e], row);
+            }
+#pragma unroll
+            for (int e = CX; e < CX + KW - 1; e++) v[yy][e] = buffer_load(plane, off[e], row);
+        }
+#pragma unroll
+        for (int yy = 0; yy < R + KH - 1; yy++)
+#pragma unroll
+            for (int ky = 0; ky < KH; ky++) {
+                const int r = yy - ky;
+                if (r >= 0 && r < R) {
+#pragma unroll
+                    for (int j = 0; j < CX; j++)
+#pragma unroll
+                        for (int kx = 0; kx < KW; kx++) acc[r][j] = fused_mad(v[yy][j + kx], wt[ky][kx], acc[r][j]);
                 }
             }
-        const int x = x0 + lane_x;
+    }
 #pragma unroll
-        for (int r = 0; r < DT_Y / 4; r++) {
-            const int y = y0 + wy * (DT_Y / 4) + r;
-            if (y < g.H && x < g.W) dx[((int64_t)c * g.H + y) * g.W + x] = acc[r];
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int j = 0; j < CX; j++) red[wave][r][lane * CX + j] = acc[r][j];
+    __syncthreads();
+    T* dst = partial + (int64_t)blockIdx.z * g.OH * g.OW;
+    for (int e = threadIdx.x; e < R * 64 * CX; e += 256) {
+        const int r = e / (64 * CX), col = e % (64 * CX);
+        const int yo = y0 + r, xo = blockIdx.x * (64 * CX) + col;
+        if (yo < g.OH && xo < g.OW)
+            dst[(int64_t)yo * g.OW + xo] = (red[0][r][col] + red[1][r][col]) + (red[2][r][col] + red[3][r][col]);
+    }
+}
+
+// gradient w.r.t. the big operand: dx[c][y][x] = sum_ky sum_kx w[c][ky][kx] * err[y-ky][x-kx] (zero outside err)
+// wave -> (256-column block over W, strip of R rows of dx, channel group); the err window of the strip is
+// loaded once and reused by every channel of the group
+template <typename T, int KH, int KW, int R>
+__global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restrict__ err, const T* __restrict__ w, T* __restrict__ dx) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int x = blockIdx.x * (64 * CX) + lane * CX;
+    const int y0 = (blockIdx.y * 4 + wave) * R;
+    if (y0 >= g.H) return;                                        // whole wavefronts leave together
+    const int c0 = blockIdx.z * g.cg;
+    int c1 = c0 + g.cg; if (c1 > g.C) c1 = g.C;
+    // E[rr][i] = err[y0 - (KH-1) + rr][x - (KW-1) + i], zero outside err
+    unsigned eoff[CX + KW - 1];
+    bool col_ok[CX + KW - 1];
+#pragma unroll
+    for (int i = 0; i < CX + KW - 1; i++) {
+        const int ex = x - (KW - 1) + i;
+        col_ok[i] = ex >= 0 && ex < g.OW;
+        eoff[i] = (unsigned)clampi(ex, 0, g.OW - 1) * (unsigned)sizeof(T);
+    }
+    const BufRsrc ebuf = buffer_of(err, (unsigned)(g.OH * g.OW) * 4u);
+    T E[R + KH - 1][CX + KW - 1];
+#pragma unroll
+    for (int rr = 0; rr < R + KH - 1; rr++) {
+        const int ey = y0 - (KH - 1) + rr;
+        const bool row_ok = ey >= 0 && ey < g.OH;
+        const unsigned row = (unsigned)(clampi(ey, 0, g.OH - 1) * g.OW) * 4u;
+#pragma unroll
+        for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = buffer_load(ebuf, eoff[i], row);
+#pragma unroll
+        for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = row_ok && col_ok[i] ? E[rr][i] : T(0);
+    }
+    const bool vec_ok = x + CX <= g.W;
+    const unsigned xoff = (unsigned)(x < g.W ? x : 0) * (unsigned)sizeof(T);
+    for (int c = c0; c < c1; c++) {
+        const T* wc = w + (int64_t)c * (KH * KW);
+        T wt[KH][KW];
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) wt[ky][kx] = wc[ky * KW + kx];
+        T* plane = dx + (int64_t)c * g.H * g.W;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            T acc[CX];
+#pragma unroll
+            for (int j = 0; j < CX; j++) acc[j] = T(0);
+#pragma unroll
+            for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++)
+#pragma unroll
+                    for (int j = 0; j < CX; j++) acc[j] = fused_mad(E[r + KH - 1 - ky][j - kx + KW - 1], wt[ky][kx], acc[j]);
+            if (y0 + r < g.H) {
+                T* dst = (T*)((char*)(plane + (int64_t)(y0 + r) * g.W) + xoff);
+                if (vec_ok) {
+                    f32x4u o; o[0] = acc[0]; o[1] = acc[1]; o[2] = acc[2]; o[3] = acc[3];
+                    __builtin_nontemporal_store(o, (f32x4u*)dst);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < CX; j++) if (x + j < g.W) dst[j] = acc[j];
+                }
+            }
         }
     }
 }
 
-// chan_dk: dk[c][ky][kx] = sum_y sum_x in[c][y+ky][x+kx] * err[y][x]; one block per (c, row band),
-// every thread accumulates all taps over its share of the band, then a block-wide reduction.
-template <typename T>
-__global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int bands, int rows_per_band, const T* __restrict__ in,
-                                                    const T* __restrict__ err, T* __restrict__ partial) {
-    __shared__ T red[4][MAX_KH * MAX_KW];
-    const int c = blockIdx.x, band = blockIdx.y;
-    const int ya = band * rows_per_band;
-    int yb = ya + rows_per_band; if (yb > g.OH) yb = g.OH;
-    const T* plane = in + (int64_t)c * g.H * g.W;
-    T acc[MAX_KH * MAX_KW];
+// gradient w.r.t. the taps: dk[c][ky][kx] = sum_y sum_x in[c][y+ky][x+kx] * err[y][x]
+//   = sum over input elements (yy, xx) of in[c][yy][xx] * err[yy-ky][xx-kx]
+// wave -> (256-column block over W, strip of S input rows, channel).  The KH-row err window around the
+// lane's CX input elements slides down the strip; every input element is loaded once (16-byte loads) and
+// multiplied into KH*KW accumulators; the loads of the next row are issued before the current row's
+// arithmetic.  Lanes are reduced with wavefront shuffles, strips by a second pass.
+template <typename T, int KH, int KW>
+__global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstrips, const T* __restrict__ in, const T* __restrict__ err, T* __restrict__ partial) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int strip = blockIdx.y * 4 + wave;
+    if (strip >= nstrips) return;                                 // whole wavefronts leave together
+    const int xx = blockIdx.x * (64 * CX) + lane * CX;
+    const bool vec_ok = xx + CX <= g.W;
+    const int yy0 = strip * S;
+    int yy1 = yy0 + S; if (yy1 > g.H) yy1 = g.H;
+    const int c = blockIdx.z;
+    unsigned eoff[CX + KW - 1], voff[CX];
+    bool col_ok[CX + KW - 1], v_ok[CX];
 #pragma unroll
-    for (int t = 0; t < MAX_KH * MAX_KW; t++) acc[t] = T(0);
-    for (int y = ya; y < yb; y++)
-        for (int x = threadIdx.x; x < g.OW; x += 256) {
-            const T e = err[(int64_t)y * g.OW + x];
-#pragma unroll
-            for (int ky = 0; ky < MAX_KH; ky++)
-#pragma unroll
-                for (int kx = 0; kx < MAX_KW; kx++)
-                    if (ky < g.KH && kx < g.KW)
-                        acc[ky * MAX_KW + kx] = __builtin_fma(plane[(int64_t)(y + ky) * g.W + x + kx], e, acc[ky * MAX_KW + kx]);
-        }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-#pragma unroll
-    for (int ky = 0; ky < MAX_KH; ky++)
-#pragma unroll
-        for (int kx = 0; kx < MAX_KW; kx++)
-            if (ky < g.KH && kx < g.KW) {
-                T v = acc[ky * MAX_KW + kx];
-#pragma unroll
-                for (int off = 32; off >= 1; off >>= 1) v += __shfl_down(v, off, 64);
-                if (lane == 0) red[wave][ky * MAX_KW + kx] = v;
-            }
-    __syncthreads();
-    if (threadIdx.x < MAX_KH * MAX_KW) {
-        const int ky = threadIdx.x / MAX_KW, kx = threadIdx.x % MAX_KW;
-        if (ky < g.KH && kx < g.KW) {
-            T s = (red[0][threadIdx.x] + red[1][threadIdx.x]) + (red[2][threadIdx.x] + red[3][threadIdx.x]);
-            partial[((int64_t)band * g.C + c) * (g.KH * g.KW) + ky * g.KW + kx] = s;
-        }
+    for (int i = 0; i < CX + KW - 1; i++) {
+        const int ex = xx - (KW - 1) + i;
+        col_ok[i] = ex >= 0 && ex < g.OW;
+        eoff[i] = (unsigned)clampi(ex, 0, g.OW - 1) * (unsigned)sizeof(T);
     }
+#pragma unroll
+    for (int j = 0; j < CX; j++) {
+        v_ok[j] = xx + j < g.W;
+        voff[j] = (unsigned)clampi(xx + j, 0, g.W - 1) * (unsigned)sizeof(T);
+    }
+    T acc[KH][KW];
+#pragma unroll
+    for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+        for (int kx = 0; kx < KW; kx++) acc[ky][kx] = T(0);
+    const BufRsrc ebuf = buffer_of(err, (unsigned)(g.OH * g.OW) * 4u);
+    auto err_row = [&](int ey, T (&dst)[CX + KW - 1]) {           // dst[i] = err[ey][xx - (KW-1) + i], zero outside
+        const bool row_ok = ey >= 0 && ey < g.OH;
+        const unsigned row = (unsigned)(clampi(ey, 0, g.OH - 1) * g.OW) * 4u;
+#pragma unroll
+        for (int i = 0; i < CX + KW - 1; i++) dst[i] = buffer_load(ebuf, eoff[i], row);
+#pragma unroll
+        for (int i = 0; i < CX + KW - 1; i++) dst[i] = row_ok && col_ok[i] ? dst[i] : T(0);
+    };
+    const BufRsrc plane = buffer_of(in + (int64_t)c * g.H * g.W, (unsigned)(g.H * g.W) * 4u);
+    auto in_row = [&](int yy, T (&dst)[CX]) {                     // dst[j] = in[c][yy][xx + j], zero past the row
+        const unsigned row = (unsigned)((yy < g.H ? yy : g.H - 1) * g.W) * 4u;
+        if (vec_ok) {
+            const f32x4u q = buffer_load4(plane, voff[0], row);
+#pragma unroll
+            for (int j = 0; j < CX; j++) dst[j] = q[j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < CX; j++) { const T t = buffer_load(plane, voff[j], row); dst[j] = v_ok[j] ? t : T(0); }
+        }
+    };
+    T Ew[KH][CX + KW - 1];                                        // Ew[ky] = err row yy - ky
+#pragma unroll
+    for (int ky = 1; ky < KH; ky++) err_row(yy0 - ky, Ew[ky]);
+    T nextE[CX + KW - 1], nextV[CX];
+    err_row(yy0, nextE);
+    in_row(yy0, nextV);
+    for (int yy = yy0; yy < yy1; yy++) {
+        T v[CX];
+#pragma unroll
+        for (int i = 0; i < CX + KW - 1; i++) Ew[0][i] = nextE[i];
+#pragma unroll
+        for (int j = 0; j < CX; j++) v[j] = nextV[j];
+        err_row(yy + 1, nextE);                                   // one row ahead; past the strip it is loaded (clamped) and dropped
+        in_row(yy + 1, nextV);
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++)
+#pragma unroll
+                for (int j = 0; j < CX; j++) acc[ky][kx] = fused_mad(v[j], Ew[ky][j - kx + KW - 1], acc[ky][kx]);
+#pragma unroll
+        for (int ky = KH - 1; ky >= 1; ky--)
+#pragma unroll
+            for (int i = 0; i < CX + KW - 1; i++) Ew[ky][i] = Ew[ky - 1][i];
+    }
+    const int part = strip * gridDim.x + blockIdx.x;
+#pragma unroll
+    for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+        for (int kx = 0; kx < KW; kx++) {
+            T v = acc[ky][kx];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_down(v, off, 64);
+            if (lane == 0) partial[((int64_t)part * g.C + c) * (KH * KW) + ky * KW + kx] = v;
+        }
 }
 
 static bool dense_rm(const Cfg& c, int rank) {
@@ -304,93 +408,142 @@ static bool dense_rm(const Cfg& c, int rank) {
     return true;
 }
 
+// channel groups: as few channels per group as it takes to put about `want` wavefronts on the machine
+static int channels_per_group(int C, int64_t waves_per_group_set, int64_t want) {
+    int64_t groups = (want + waves_per_group_set - 1) / waves_per_group_set;
+    if (groups < 1) groups = 1;
+    if (groups > C) groups = C;
+    return (int)((C + groups - 1) / groups);
+}
+
+// run-time tap extents -> the template instantiations that exist; false when there is none
+template <typename F>
+static bool for_taps(int KH, int KW, F&& f) {
+    if (KH != KW) return false;
+    switch (KH) {
+        case 2: f(std::integral_constant<int, 2>{}); return true;
+        case 3: f(std::integral_constant<int, 3>{}); return true;
+        case 4: f(std::integral_constant<int, 4>{}); return true;
+        case 5: f(std::integral_constant<int, 5>{}); return true;
+        case 7: f(std::integral_constant<int, 7>{}); return true;
+        default: return false;
+    }
+}
+
+// the three channel kernels for dense f32 operands; returns NK_OK with *taken = true when one was launched
+static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, const float* s1, const Cfg& c1,
+                              const float* s2, const Cfg& c2, bool* taken) {
+    using T = float;
+    *taken = false;
+    static const long waves_per_cu = [] { const char* v = getenv("NK_CONV_WAVES_PER_CU"); return v && *v ? atol(v) : 8L; }();
+    const int64_t want_waves = (int64_t)dev->props.multiProcessorCount * waves_per_cu;
+    for (const Cfg* c : {&c0, &c1, &c2})          // a plane is addressed with 32-bit byte offsets; grid y and z are 16-bit
+        if ((int64_t)c->shape[1] * c->shape[2] * (int64_t)sizeof(T) >= (int64_t(1) << 31) || c->shape[0] > 65535 || c->shape[1] > 65535) return NK_OK;
+    if (d < 0 && c0.shape[0] == 1 && c1.shape[0] == c2.shape[0] && c1.shape[0] > 1) {
+        const bool a_big = c1.shape[1] >= c2.shape[1] && c1.shape[2] >= c2.shape[2];
+        const bool b_big = c2.shape[1] >= c1.shape[1] && c2.shape[2] >= c1.shape[2];
+        if (!a_big && !b_big) return NK_OK;
+        const Cfg& big = a_big ? c1 : c2;
+        const Cfg& small = a_big ? c2 : c1;
+        const T* bigp = a_big ? s1 : s2;
+        const T* smallp = a_big ? s2 : s1;
+        constexpr int R = 8;
+        ChanArgs g{};
+        g.C = big.shape[0]; g.H = big.shape[1]; g.W = big.shape[2];
+        g.OH = g.H - small.shape[1] + 1; g.OW = g.W - small.shape[2] + 1;
+        g.col_blocks = (g.OW + 64 * CX - 1) / (64 * CX);
+        const int strips = (g.OH + R - 1) / R;
+        // a block's four wavefronts take one channel each: groups are multiples of 4 channels
+        g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips * 4, want_waves);
+        g.cg = (g.cg + 3) / 4 * 4;
+        const int groups = (g.C + g.cg - 1) / g.cg;
+        int rc = NK_OK;
+        const bool ok = for_taps(small.shape[1], small.shape[2], [&](auto K) {
+            constexpr int KK = decltype(K)::value;
+            void* ws = nullptr;
+            const int on = g.OH * g.OW;
+            if ((rc = workspace(dev, (uint64_t)groups * on * sizeof(T), &ws))) return;
+            dim3 grid(g.col_blocks, strips, groups);
+            hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, bigp, smallp, groups == 1 ? out : (T*)ws);
+            if (groups > 1)
+                hipLaunchKernelGGL(conv_partial_reduce<T>, dim3((on + 255) / 256), dim3(256), 0, dev->stream, groups, on, (const T*)ws, out);
+        });
+        if (!ok) return NK_OK;
+        if (rc) return rc;
+        NK_HIP(hipGetLastError());
+        set_path("chan_fwd");
+        *taken = true;
+        return NK_OK;
+    }
+    if (d >= 0 && c2.shape[0] == 1 && c0.shape[0] == c1.shape[0] && c0.shape[0] > 1) {
+        const int OH = c2.shape[1], OW = c2.shape[2];      // src2 = error [1,OH,OW]
+        // dx: the drain is the big operand, src1 the taps
+        if (c0.shape[1] == OH + c1.shape[1] - 1 && c0.shape[2] == OW + c1.shape[2] - 1 &&
+            (c0.shape[1] > c1.shape[1] || c1.shape[1] == 1) && (c0.shape[2] > c1.shape[2] || c1.shape[2] == 1)) {
+            constexpr int R = 4;
+            ChanArgs g{};
+            g.C = c0.shape[0]; g.H = c0.shape[1]; g.W = c0.shape[2]; g.OH = OH; g.OW = OW;
+            g.col_blocks = (g.W + 64 * CX - 1) / (64 * CX);
+            const int strips = (g.H + R - 1) / R;
+            g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips, want_waves);
+            if (g.cg < 2 && g.C >= 2) g.cg = 2;              // amortise the err window over at least two channels
+            const int groups = (g.C + g.cg - 1) / g.cg;
+            const bool ok = for_taps(c1.shape[1], c1.shape[2], [&](auto K) {
+                constexpr int KK = decltype(K)::value;
+                dim3 grid(g.col_blocks, (strips + 3) / 4, groups);
+                hipLaunchKernelGGL((conv_chan_dx<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, s2, s1, out);
+            });
+            if (!ok) return NK_OK;
+            NK_HIP(hipGetLastError());
+            set_path("chan_dx");
+            *taken = true;
+            return NK_OK;
+        }
+        // dk: the drain is the taps, src1 the big operand
+        if (c1.shape[1] == OH + c0.shape[1] - 1 && c1.shape[2] == OW + c0.shape[2] - 1 && c0.shape[1] < c1.shape[1] && c0.shape[2] < c1.shape[2]) {
+            ChanArgs g{};
+            g.C = c0.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2]; g.OH = OH; g.OW = OW;
+            g.col_blocks = (g.W + 64 * CX - 1) / (64 * CX);
+            g.cg = 1;
+            // rows per strip: enough strips for the machine, at least 8 rows to amortise the window set-up
+            int64_t strips = (want_waves + (int64_t)g.col_blocks * g.C - 1) / ((int64_t)g.col_blocks * g.C);
+            if (strips < 1) strips = 1;
+            int S = (int)((g.H + strips - 1) / strips);
+            if (S < 8) S = 8;
+            const int nstrips = (g.H + S - 1) / S;
+            const int parts = nstrips * g.col_blocks;
+            int rc = NK_OK;
+            const bool ok = for_taps(c0.shape[1], c0.shape[2], [&](auto K) {
+                constexpr int KK = decltype(K)::value;
+                const int on = g.C * KK * KK;
+                void* ws = nullptr;
+                if ((rc = workspace(dev, (uint64_t)parts * on * sizeof(T), &ws))) return;
+                dim3 grid(g.col_blocks, (nstrips + 3) / 4, g.C);
+                hipLaunchKernelGGL((conv_chan_dk<T, KK, KK>), grid, dim3(256), 0, dev->stream, g, S, nstrips, s1, s2, (T*)ws);
+                hipLaunchKernelGGL(conv_partial_reduce_wide<T>, dim3((on + 3) / 4), dim3(256), 0, dev->stream, parts, on, (const T*)ws, out);
+            });
+            if (!ok) return NK_OK;
+            if (rc) return rc;
+            NK_HIP(hipGetLastError());
+            set_path("chan_dk");
+            *taken = true;
+            return NK_OK;
+        }
+    }
+    return NK_OK;
+}
+
 template <typename T>
 static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, nk_buf a, const Cfg& c1, nk_buf b,
                       const Cfg& c2, int64_t n) {
     T* out = (T*)drn;
     const T* s1 = (const T*)a;
     const T* s2 = (const T*)b;
-    const bool dense = dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank);
-    if (dense && rank == 3 && sizeof(T) == 4) {
-        if (d < 0 && c0.shape[0] == 1 && c1.shape[0] == c2.shape[0] && c1.shape[0] > 1) {
-            // which operand is the big one?
-            const bool a_big = c1.shape[1] >= c2.shape[1] && c1.shape[2] >= c2.shape[2];
-            const bool b_big = c2.shape[1] >= c1.shape[1] && c2.shape[2] >= c1.shape[2];
-            if (a_big || b_big) {
-                const Cfg& big = a_big ? c1 : c2;
-                const Cfg& small = a_big ? c2 : c1;
-                if (small.shape[1] <= MAX_KH && small.shape[2] <= MAX_KW) {
-                    ChanArgs g{};
-                    g.C = big.shape[0]; g.H = big.shape[1]; g.W = big.shape[2];
-                    g.KH = small.shape[1]; g.KW = small.shape[2];
-                    g.OH = g.H - g.KH + 1; g.OW = g.W - g.KW + 1;
-                    const int tiles = ((g.OW + FT_X - 1) / FT_X) * ((g.OH + FT_Y - 1) / FT_Y);
-                    int splits = (dev->props.multiProcessorCount * 2 + tiles - 1) / tiles;
-                    if (splits > (g.C + 3) / 4) splits = (g.C + 3) / 4;
-                    if (splits < 1) splits = 1;
-                    g.cps = (g.C + splits - 1) / splits;
-                    splits = (g.C + g.cps - 1) / g.cps;
-                    g.splits = splits;
-                    void* ws = nullptr;
-                    if (int e = workspace(dev, (uint64_t)splits * g.OH * g.OW * sizeof(T), &ws)) return e;
-                    dim3 grid((g.OW + FT_X - 1) / FT_X, (g.OH + FT_Y - 1) / FT_Y, splits);
-                    set_path("chan_fwd");
-                    const T* bigp = a_big ? s1 : s2;
-                    const T* smallp = a_big ? s2 : s1;
-                    if (g.KH == 5 && g.KW == 5)
-                        hipLaunchKernelGGL((conv_chan_fwd<T, 5, 5>), grid, dim3(256), 0, dev->stream, g, bigp, smallp, (T*)ws);
-                    else if (g.KH == 3 && g.KW == 3)
-                        hipLaunchKernelGGL((conv_chan_fwd<T, 3, 3>), grid, dim3(256), 0, dev->stream, g, bigp, smallp, (T*)ws);
-                    else
-                        hipLaunchKernelGGL((conv_chan_fwd<T, 0, 0>), grid, dim3(256), 0, dev->stream, g, bigp, smallp, (T*)ws);
-                    NK_HIP(hipGetLastError());
-                    const int on = g.OH * g.OW;
-                    hipLaunchKernelGGL(conv_chan_fwd_reduce<T>, dim3((on + 255) / 256), dim3(256), 0, dev->stream, splits, on, (const T*)ws, out);
-                    NK_HIP(hipGetLastError());
-                    return NK_OK;
-                }
-            }
-        }
-        if (d >= 0 && c2.shape[0] == 1 && c0.shape[0] == c1.shape[0] && c0.shape[0] > 1) {
-            // src2 = error [1,OH,OW]
-            const int OH = c2.shape[1], OW = c2.shape[2];
-            // dx: drain [C,H,W] bigger than src1 = taps [C,KH,KW] with H = OH + KH - 1
-            if (c0.shape[1] >= c1.shape[1] && c0.shape[2] >= c1.shape[2] && c1.shape[1] <= MAX_KH && c1.shape[2] <= MAX_KW &&
-                c0.shape[1] == OH + c1.shape[1] - 1 && c0.shape[2] == OW + c1.shape[2] - 1 &&
-                (c0.shape[1] > c1.shape[1] || c1.shape[1] == 1) && (c0.shape[2] > c1.shape[2] || c1.shape[2] == 1)) {
-                ChanArgs g{};
-                g.C = c0.shape[0]; g.H = c0.shape[1]; g.W = c0.shape[2];
-                g.KH = c1.shape[1]; g.KW = c1.shape[2]; g.OH = OH; g.OW = OW;
-                g.cps = 4;
-                g.splits = (g.C + g.cps - 1) / g.cps;
-                dim3 grid((g.W + DT_X - 1) / DT_X, (g.H + DT_Y - 1) / DT_Y, g.splits);
-                set_path("chan_dx");
-                hipLaunchKernelGGL(conv_chan_dx<T>, grid, dim3(256), 0, dev->stream, g, s2, s1, out);
-                NK_HIP(hipGetLastError());
-                return NK_OK;
-            }
-            // dk: drain [C,KH,KW] smaller than src1 = input [C,H,W]
-            if (c0.shape[1] <= MAX_KH && c0.shape[2] <= MAX_KW && c1.shape[1] == OH + c0.shape[1] - 1 &&
-                c1.shape[2] == OW + c0.shape[2] - 1 && c0.shape[1] < c1.shape[1] && c0.shape[2] < c1.shape[2]) {
-                ChanArgs g{};
-                g.C = c0.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2];
-                g.KH = c0.shape[1]; g.KW = c0.shape[2]; g.OH = OH; g.OW = OW;
-                int bands = (dev->props.multiProcessorCount * 4 + g.C - 1) / g.C;
-                if (bands > OH) bands = OH;
-                if (bands < 1) bands = 1;
-                const int rpb = (OH + bands - 1) / bands;
-                bands = (OH + rpb - 1) / rpb;
-                const int ntaps = g.KH * g.KW;
-                void* ws = nullptr;
-                if (int e = workspace(dev, (uint64_t)bands * g.C * ntaps * sizeof(T), &ws)) return e;
-                set_path("chan_dk");
-                hipLaunchKernelGGL(conv_chan_dk<T>, dim3(g.C, bands), dim3(256), 0, dev->stream, g, bands, rpb, s1, s2, (T*)ws);
-                NK_HIP(hipGetLastError());
-                const int on = g.C * ntaps;
-                hipLaunchKernelGGL(conv_chan_fwd_reduce<T>, dim3((on + 255) / 256), dim3(256), 0, dev->stream, bands, on, (const T*)ws, out);
-                NK_HIP(hipGetLastError());
-                return NK_OK;
-            }
+    if constexpr (sizeof(T) == 4) {
+        if (rank == 3 && dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank)) {
+            bool taken = false;
+            if (int e = conv_channel_paths(dev, d, out, c0, s1, c1, s2, c2, &taken)) return e;
+            if (taken) return NK_OK;
         }
     }
     ConvArgs A{};

@@ -457,7 +457,9 @@ def _abs_bound(orc, xs, ks, x, k, dt):
                         np.abs(k).astype(np.float64).reshape(-1), orc.dense_cfg(ks))
 
 
-@pytest.mark.parametrize("shape", [([8, 40, 70], [8, 5, 5]), ([6, 33, 65], [6, 3, 3]), ([5, 20, 21], [5, 4, 2]), ([64, 64, 64], [64, 5, 5])])
+@pytest.mark.parametrize("shape", [([8, 40, 70], [8, 5, 5]), ([6, 33, 65], [6, 3, 3]), ([5, 20, 21], [5, 4, 2]), ([64, 64, 64], [64, 5, 5]),
+                                   ([3, 130, 200], [3, 7, 7]), ([9, 17, 300], [9, 2, 2]), ([2, 12, 12], [2, 4, 4]),
+                                   ([3, 10, 71], [3, 3, 3]), ([5, 9, 302], [5, 2, 2]), ([70, 30, 261], [70, 5, 5])])
 def test_channel_convolution_fast_paths(device, orc, shape):
     """[C,H,W] x [C,kh,kw] forward and both gradients on the LDS-tiled kernels: re-ordered f32 sums, compared
     norm-wise: |delta| <= 1e-5 * sum|a||b| per output."""
@@ -467,28 +469,30 @@ def test_channel_convolution_fast_paths(device, orc, shape):
     x = (rng.standard_normal(xs) * 0.1).astype(np.float32); k = (rng.standard_normal(ks) * 0.1).astype(np.float32)
     e = rng.standard_normal(ys).astype(np.float32)
     tx, tk, te = on(device, x), on(device, k), on(device, e)
+    square = ks[1] == ks[2]          # the register-window kernels exist for square taps of extent 2, 3, 4, 5, 7
+    fwd, dxp, dkp = ("chan_fwd", "chan_dx", "chan_dk") if square else ("literal_fwd", "literal_bwd", "literal_bwd")
     say("chan_fwd", xs, ks)
     out = Tensor._on_device(device, np.float32, ys)
     device.launch_convolution(-1, out, tx, tk)
-    assert _lib.last_path() == "chan_fwd"
+    assert _lib.last_path() == fwd
     want = orc.convolve(np.zeros(out.size, dtype=np.float32), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
     bound = RTOL[np.dtype(np.float32)] * _abs_bound(orc, xs, ks, x, k, np.float32) + 1e-30
     assert (np.abs(out.getData().astype(np.float64) - want) <= bound).all(), "chan_fwd"
     out2 = Tensor._on_device(device, np.float32, ys)
     device.launch_convolution(-1, out2, tk, tx)                       # kernel first
-    assert _lib.last_path() == "chan_fwd"
+    assert _lib.last_path() == fwd
     assert_bits(out2.getData(), out.getData(), "operand order")
     say("chan_dx", xs, ks)
     dx = Tensor._on_device(device, np.float32, xs)
     device.launch_convolution(0, dx, tk, te)
-    assert _lib.last_path() == "chan_dx"
+    assert _lib.last_path() == dxp
     want = orc.deconvolve(np.zeros(dx.size, dtype=np.float32), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks), e.reshape(-1), orc.dense_cfg(ys), fast=True)
     babs = orc.deconvolve(np.zeros(dx.size), orc.dense_cfg(xs), np.abs(k).astype(np.float64).reshape(-1), orc.dense_cfg(ks), np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
     assert (np.abs(dx.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dx"
     say("chan_dk", xs, ks)
     dk = Tensor._on_device(device, np.float32, ks)
     device.launch_convolution(0, dk, tx, te)
-    assert _lib.last_path() == "chan_dk"
+    assert _lib.last_path() == dkp
     want = orc.deconvolve(np.zeros(dk.size, dtype=np.float32), orc.dense_cfg(ks), x.reshape(-1), orc.dense_cfg(xs), e.reshape(-1), orc.dense_cfg(ys), fast=True)
     babs = orc.deconvolve(np.zeros(dk.size), orc.dense_cfg(ks), np.abs(x).astype(np.float64).reshape(-1), orc.dense_cfg(xs), np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
     assert (np.abs(dk.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dk"
