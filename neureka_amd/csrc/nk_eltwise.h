@@ -201,11 +201,15 @@ struct Ptrs { const void* p[NK_FUSE_MAX_SRC]; };
 template <typename T, int V> struct VecOf { typedef T type __attribute__((ext_vector_type(V), aligned(sizeof(T)))); };
 template <typename T> struct VecOf<T, 1> { typedef T type; };
 
-template <typename T, int V>
+// NT: the value is read once by the whole launch -- a non-temporal load keeps it from displacing
+// lines that will be used again and is measurably faster for streams far larger than the caches.
+template <typename T, int V, bool NT = false>
 __device__ __forceinline__ void load_vec(T (&dst)[V], const T* p) {
-    if constexpr (V == 1) dst[0] = *p;
+    if constexpr (V == 1) dst[0] = NT ? __builtin_nontemporal_load(p) : *p;
     else {
-        typename VecOf<T, V>::type v = *(const typename VecOf<T, V>::type*)p;
+        typedef typename VecOf<T, V>::type Vec;
+        Vec v;
+        if constexpr (NT) v = __builtin_nontemporal_load((const Vec*)p); else v = *(const Vec*)p;
 #pragma unroll
         for (int i = 0; i < V; i++) dst[i] = v[i];
     }
@@ -244,6 +248,7 @@ struct RowsArgs {
     int simple_loads;          // every source register is filled by a plain vector load
     int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
     int streaming;             // non-temporal stores for the drain
+    int nt_loads;              // every source element is read exactly once: the host picks the non-temporal-load variant
     FastDiv chunk_div;
     FastDiv outer[ROWS_MAX_OUTER];           // outer[0] is the innermost outer axis
     int base[MAX_OPERANDS];
@@ -291,13 +296,13 @@ __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsign
     return R;
 }
 
-template <typename T, int V, int NSRC, int FUNSET, int PASSES>
+template <typename T, int V, int NSRC, int FUNSET, int PASSES, bool NT = false>
 __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
     T x[NSRC][PASSES * V];
     int doff[PASSES];
     bool live[PASSES];
     if (A.simple_loads) {
-        // every source is a plain aligned vector load: no branches between the loads of all passes
+        // every source is a plain vector load: no branches between the loads of all passes
 #pragma unroll
         for (int p = 0; p < PASSES; p++) {
             const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, blockIdx.x * PASSES + p);
@@ -306,7 +311,7 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
 #pragma unroll
             for (int j = 0; j < NSRC; j++) {
                 T (&xj)[V] = *reinterpret_cast<T (*)[V]>(&x[j][p * V]);
-                load_vec<T, V>(xj, (const T*)srcs.p[j] + R.off[j + 1] + R.col);
+                load_vec<T, V, NT>(xj, (const T*)srcs.p[j] + R.off[j + 1] + R.col);
             }
         }
     } else {
@@ -348,7 +353,7 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
 // drain = src0 op src1 with op in {+, -, *, /} and plain aligned loads: the bandwidth-critical case
 // (same-shape elementwise and forward broadcast).  The operator is resolved once, outside the passes,
 // and each pass is stored as soon as its operands have arrived.
-template <typename T, int V, int PASSES>
+template <typename T, int V, int PASSES, bool NT = false>
 __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T* __restrict__ drn, const T* __restrict__ s0,
                                                           const T* __restrict__ s1) {
     T x0[PASSES][V], x1[PASSES][V];
@@ -359,8 +364,8 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
         const RowsAddr<3> R = rows_address<3>(A, blockIdx.x * PASSES + p);
         live[p] = R.live;
         doff[p] = R.off[0] + (int)R.col;
-        load_vec<T, V>(x0[p], s0 + R.off[1] + R.col);
-        load_vec<T, V>(x1[p], s1 + R.off[2] + R.col);
+        load_vec<T, V, NT>(x0[p], s0 + R.off[1] + R.col);
+        load_vec<T, V, NT>(x1[p], s1 + R.off[2] + R.col);
     }
 #define NK_BINARY_PASSES(EXPR)                                                        \
     _Pragma("unroll") for (int p = 0; p < PASSES; p++) {                              \

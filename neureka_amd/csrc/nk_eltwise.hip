@@ -212,6 +212,11 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
         A.streaming = streaming ? 1 : 0;
+        // sources at least as large as the drain's threshold whose every element is read once stream past the caches
+        bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
+        for (int j = 0; j < c.nsrc && once; j++)
+            for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) once = false;
+        A.nt_loads = once ? 1 : 0;
         A.const_last = 0;
         for (int j = 0; j < c.nsrc; j++) if (cn.stride[j + 1][last] == 0) A.const_last |= 1u << j;
         uint64_t n_rows = 1;
