@@ -236,6 +236,9 @@ __device__ __forceinline__ void store_vec(T* p, const T (&src)[V], bool streamin
 // at most ROWS_MAX_OUTER outer axes (more fall to the canon kernel); the argument block is small and
 // fixed-size so that it is fetched with a few wide scalar loads at kernel start.
 constexpr int ROWS_MAX_OUTER = 3;
+// units per block of rows_kernel: enough loads in flight to cover latency, few enough registers to keep
+// several wavefronts per SIMD (three sources x 16 values already costs half the occupancy)
+constexpr int rows_passes(int funset, int nsrc) { return funset >= 2 ? 1 : (nsrc >= 3 ? 2 : 4); }
 struct RowsArgs {
     int nouter;                // collapsed outer axes, 0..ROWS_MAX_OUTER
     int nsrc;
@@ -432,6 +435,7 @@ struct TileArgs {
     unsigned P, L;                          // extents of pax and of the innermost axis
     unsigned tiles_p, tiles_l;
     unsigned n_blocks;
+    int group_log2;                         // blocks are numbered through G x G groups of tiles, G = 1 << group_log2
     int streaming;
     int careful;                            // some direct operand is constant along the innermost axis: no vector path
     FastDiv div_tiles_l, div_tiles_p;
@@ -446,16 +450,21 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
     constexpr int LPR = 64 / VEC;                  // lanes that cover one 64-element tile row
     constexpr int RPI = 256 / LPR;                 // tile rows covered by one access of the whole block
     constexpr int NIT = 64 / RPI;                  // accesses per thread and operand
-    constexpr int EPT = NIT * VEC;                 // elements per thread (16)
     __shared__ T tiles[NSRC][64][65];
     const int last = A.rank - 1;
     const unsigned q = threadIdx.x % LPR, r = threadIdx.x / LPR;
 
+    // Consecutive blocks run at the same time.  Numbering them through G x G groups of tiles makes the 256-byte
+    // pieces that neighbouring blocks read (along pax) and write (along the innermost axis) add up to G x 256
+    // contiguous bytes on both sides, instead of one side seeing isolated 256-byte pieces.
     unsigned rest = blockIdx.x;
-    unsigned d = A.div_tiles_l.div(rest);
-    const unsigned tl = rest - d * A.tiles_l; rest = d;
+    const unsigned G = 1u << A.group_log2;
+    const unsigned local = rest & (G * G - 1);
+    rest >>= 2 * A.group_log2;
+    unsigned d = A.div_tiles_l.div(rest);                  // divisors are the group counts tiles_l / G and tiles_p / G
+    const unsigned tl = (rest - d * A.div_tiles_l.d) * G + (local & (G - 1)); rest = d;
     d = A.div_tiles_p.div(rest);
-    const unsigned tp = rest - d * A.tiles_p; rest = d;
+    const unsigned tp = (rest - d * A.div_tiles_p.d) * G + (local >> A.group_log2); rest = d;
     int64_t off[NSRC + 1];
 #pragma unroll
     for (int o = 0; o <= NSRC; o++) off[o] = A.base[o];
@@ -469,8 +478,10 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
     }
     const unsigned p0 = tp * 64, l0 = tl * 64;
     const int64_t dP = A.stride[0][A.pax];
-    T x[NSRC][EPT];
-    T out[EPT];
+    // the program runs over CHUNK elements at a time: the tiles wait in LDS, so a thread never holds more than
+    // CHUNK values per source in registers (occupancy is bounded by registers here)
+    constexpr int CIT = NIT >= 2 ? 2 : 1;          // 16-byte accesses per chunk
+    constexpr int CHUNK = CIT * VEC;
 
     // whole tile inside the tensor, every operand either along pax or along the innermost axis:
     // 16-byte accesses on both sides, one barrier
@@ -491,34 +502,39 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
             }
         }
         __syncthreads();
-#pragma unroll
-        for (int j = 0; j < NSRC; j++) {
-            if (j < A.nsrc) {
-                if ((A.turned >> j) & 1u) {
-#pragma unroll
-                    for (int it = 0; it < NIT; it++)
-#pragma unroll
-                        for (int e = 0; e < VEC; e++) x[j][it * VEC + e] = tiles[j][q * VEC + e][r + RPI * it];
-                } else {
-                    const T* sp = (const T*)srcs.p[j] + off[j + 1] + l0 + q * VEC;       // stride 1 along the innermost axis
-                    const int64_t sP = A.stride[j + 1][A.pax];
-#pragma unroll
-                    for (int it = 0; it < NIT; it++) {
-                        T (&xv)[VEC] = *reinterpret_cast<T (*)[VEC]>(&x[j][it * VEC]);
-                        load_vec<T, VEC>(xv, sp + (int64_t)(p0 + r + RPI * it) * sP);
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < EPT; e++) x[j][e] = T(0);
-            }
-        }
-        run_any<T, EPT, NSRC, FUNSET>(P, LP, x, out);
         T* dp = drn + off[0] + l0 + q * VEC;
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            T (&ov)[VEC] = *reinterpret_cast<T (*)[VEC]>(&out[it * VEC]);
-            store_vec<T, VEC>(dp + (int64_t)(p0 + r + RPI * it) * dP, ov, A.streaming != 0);
+        for (int c = 0; c < NIT; c += CIT) {
+            T x[NSRC][CHUNK];
+            T out[CHUNK];
+#pragma unroll
+            for (int j = 0; j < NSRC; j++) {
+                if (j < A.nsrc) {
+                    if ((A.turned >> j) & 1u) {
+#pragma unroll
+                        for (int it = 0; it < CIT; it++)
+#pragma unroll
+                            for (int e = 0; e < VEC; e++) x[j][it * VEC + e] = tiles[j][q * VEC + e][r + RPI * (c + it)];
+                    } else {
+                        const T* sp = (const T*)srcs.p[j] + off[j + 1] + l0 + q * VEC;   // stride 1 along the innermost axis
+                        const int64_t sP = A.stride[j + 1][A.pax];
+#pragma unroll
+                        for (int it = 0; it < CIT; it++) {
+                            T (&xv)[VEC] = *reinterpret_cast<T (*)[VEC]>(&x[j][it * VEC]);
+                            load_vec<T, VEC>(xv, sp + (int64_t)(p0 + r + RPI * (c + it)) * sP);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < CHUNK; e++) x[j][e] = T(0);
+                }
+            }
+            run_any<T, CHUNK, NSRC, FUNSET>(P, LP, x, out);
+#pragma unroll
+            for (int it = 0; it < CIT; it++) {
+                T (&ov)[VEC] = *reinterpret_cast<T (*)[VEC]>(&out[it * VEC]);
+                store_vec<T, VEC>(dp + (int64_t)(p0 + r + RPI * (c + it)) * dP, ov, A.streaming != 0);
+            }
         }
         return;
     }
@@ -537,33 +553,37 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
         }
     }
     __syncthreads();
+    for (int c = 0; c < 16; c += 8) {
+        T x[NSRC][8];
+        T out[8];
 #pragma unroll
-    for (int j = 0; j < NSRC; j++) {
-        if (j < A.nsrc) {
-            if ((A.turned >> j) & 1u) {
+        for (int j = 0; j < NSRC; j++) {
+            if (j < A.nsrc) {
+                if ((A.turned >> j) & 1u) {
 #pragma unroll
-                for (int it = 0; it < 16; it++) x[j][it] = tiles[j][tx][ty + 4 * it];
-            } else {
-                const T* sp = (const T*)srcs.p[j] + off[j + 1];
-                const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
+                    for (int it = 0; it < 8; it++) x[j][it] = tiles[j][tx][ty + 4 * (c + it)];
+                } else {
+                    const T* sp = (const T*)srcs.p[j] + off[j + 1];
+                    const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
 #pragma unroll
-                for (int it = 0; it < 16; it++) {
-                    const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
-                    x[j][it] = (p < A.P && l < A.L) ? sp[(int64_t)p * sP + (int64_t)l * sL] : T(0);
+                    for (int it = 0; it < 8; it++) {
+                        const unsigned p = p0 + ty + 4 * (c + it), l = l0 + tx;
+                        x[j][it] = (p < A.P && l < A.L) ? sp[(int64_t)p * sP + (int64_t)l * sL] : T(0);
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int it = 0; it < 8; it++) x[j][it] = T(0);
             }
-        } else {
-#pragma unroll
-            for (int it = 0; it < 16; it++) x[j][it] = T(0);
         }
-    }
-    run_any<T, EPT, NSRC, FUNSET>(P, LP, x, out);
+        run_any<T, 8, NSRC, FUNSET>(P, LP, x, out);
 #pragma unroll
-    for (int it = 0; it < 16; it++) {
-        const unsigned p = p0 + ty + 4 * it, l = l0 + tx;
-        if (p < A.P && l < A.L) {
-            T* dst = drn + off[0] + (int64_t)p * dP + l;
-            if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
+        for (int it = 0; it < 8; it++) {
+            const unsigned p = p0 + ty + 4 * (c + it), l = l0 + tx;
+            if (p < A.P && l < A.L) {
+                T* dst = drn + off[0] + (int64_t)p * dP + l;
+                if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
+            }
         }
     }
 }

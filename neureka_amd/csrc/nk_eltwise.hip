@@ -208,7 +208,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         const bool vec = cn.shape[last] % VMAX == 0;
         RowsArgs& A = plan.rows;
         const int V = vec ? VMAX : 1;
-        int passes = funset >= 2 ? 1 : 4;
+        int passes = rows_passes(funset, funset >= 2 ? NK_FUSE_MAX_SRC : (c.nsrc <= 1 ? 1 : c.nsrc));
         A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
         A.streaming = streaming ? 1 : 0;
@@ -290,7 +290,11 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             }
             if (nb < ((uint64_t)1 << 31)) {
                 A.n_blocks = (unsigned)nb;
-                A.div_tiles_l = FastDiv(A.tiles_l); A.div_tiles_p = FastDiv(A.tiles_p);
+                static const int env_group = [] { const char* v = getenv("NK_TILE_GROUP_LOG2"); return v && *v ? atoi(v) : 2; }();
+                int gl = env_group < 0 ? 0 : (env_group > 4 ? 4 : env_group);
+                while (gl > 0 && (A.tiles_l % (1u << gl) || A.tiles_p % (1u << gl))) gl--;
+                A.group_log2 = gl;
+                A.div_tiles_l = FastDiv(A.tiles_l >> gl); A.div_tiles_p = FastDiv(A.tiles_p >> gl);
                 for (int o = 0; o <= c.nsrc; o++) {
                     A.base[o] = cn.base[o];
                     for (int k = 0; k < cn.rank; k++) A.stride[o][k] = cn.stride[o][k];
