@@ -421,12 +421,14 @@ __global__ __launch_bounds__(256) void canon_kernel(CanonArgs A, Prog P, LightPr
 
 // ---- tile_transpose kernel ----------------------------------------------------------------------------
 // Collapsed axis `pax` (not the innermost) is the contiguous one of the sources flagged in `turned`; all
-// other operands are contiguous or constant along the innermost axis.  A block owns a 64 (pax) x 64
-// (innermost) tile for one combination of the remaining axes.  Turned sources are read with 16-byte
+// other operands are contiguous or constant along the innermost axis.  A block owns a TILE_P (pax) x
+// TILE_L (innermost) tile for one combination of the remaining axes.  Turned sources are read with 16-byte
 // accesses along pax into one padded LDS tile each (all loads in flight before the single barrier) and
 // handed to the lanes that own 16-byte pieces along the innermost axis; the drain is written with
-// 16-byte stores.  LDS rows have a pitch of 65 elements, which makes both the row-wise writes and the
-// column-wise reads conflict-free.
+// 16-byte stores.  64 x 32 keeps a thread at 8 elements per source and a block at 25 KB of LDS (f32), so
+// that several blocks share a compute unit; measured on this part, longer runs on the read side matter
+// more than on the write side.
+constexpr int TILE_P = 64, TILE_L = 32;
 struct TileArgs {
     int rank;
     int nsrc;
@@ -437,6 +439,7 @@ struct TileArgs {
     unsigned n_blocks;
     int group_log2;                         // blocks are numbered through G x G groups of tiles, G = 1 << group_log2
     int streaming;
+    int nt_loads;                           // every source element is read exactly once: the host picks the non-temporal-load variant
     int careful;                            // some direct operand is constant along the innermost axis: no vector path
     FastDiv div_tiles_l, div_tiles_p;
     FastDiv outer[NK_MAX_RANK];             // extents of the remaining axes
@@ -444,19 +447,25 @@ struct TileArgs {
     int64_t stride[MAX_OPERANDS][NK_MAX_RANK];
 };
 
-template <typename T, int NSRC, int FUNSET>
+template <typename T, int NSRC, int FUNSET, bool NT = false>
 __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
     constexpr int VEC = 16 / sizeof(T);            // elements per 16-byte access
-    constexpr int LPR = 64 / VEC;                  // lanes that cover one 64-element tile row
-    constexpr int RPI = 256 / LPR;                 // tile rows covered by one access of the whole block
-    constexpr int NIT = 64 / RPI;                  // accesses per thread and operand
-    __shared__ T tiles[NSRC][64][65];
+    constexpr int EPT = TILE_P * TILE_L / 256;     // elements per thread and operand (8)
+    // read side: 16-byte pieces along pax
+    constexpr int R_LPR = TILE_P / VEC;            // lanes that cover one tile row of a turned source
+    constexpr int R_RPI = 256 / R_LPR;             // tile rows covered by one access of the whole block
+    constexpr int R_NIT = TILE_L / R_RPI;          // accesses per thread and turned source
+    // write side (and direct sources): 16-byte pieces along the innermost axis
+    constexpr int W_LPR = TILE_L / VEC;
+    constexpr int W_RPI = 256 / W_LPR;
+    constexpr int W_NIT = TILE_P / W_RPI;
+    static_assert(R_NIT * VEC == EPT && W_NIT * VEC == EPT, "tile shape and block size disagree");
+    __shared__ T tiles[NSRC][TILE_L][TILE_P + 1];
     const int last = A.rank - 1;
-    const unsigned q = threadIdx.x % LPR, r = threadIdx.x / LPR;
 
-    // Consecutive blocks run at the same time.  Numbering them through G x G groups of tiles makes the 256-byte
-    // pieces that neighbouring blocks read (along pax) and write (along the innermost axis) add up to G x 256
-    // contiguous bytes on both sides, instead of one side seeing isolated 256-byte pieces.
+    // Consecutive blocks run at the same time.  Numbering them through G x G groups of tiles makes the pieces
+    // that neighbouring blocks read (along pax) and write (along the innermost axis) add up to longer
+    // contiguous runs on both sides.
     unsigned rest = blockIdx.x;
     const unsigned G = 1u << A.group_log2;
     const unsigned local = rest & (G * G - 1);
@@ -476,114 +485,109 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
 #pragma unroll
         for (int o = 0; o <= NSRC; o++) off[o] += (int64_t)idx * A.stride[o][k];
     }
-    const unsigned p0 = tp * 64, l0 = tl * 64;
+    const unsigned p0 = tp * TILE_P, l0 = tl * TILE_L;
     const int64_t dP = A.stride[0][A.pax];
-    // the program runs over CHUNK elements at a time: the tiles wait in LDS, so a thread never holds more than
-    // CHUNK values per source in registers (occupancy is bounded by registers here)
-    constexpr int CIT = NIT >= 2 ? 2 : 1;          // 16-byte accesses per chunk
-    constexpr int CHUNK = CIT * VEC;
+    T x[NSRC][EPT];
+    T out[EPT];
 
     // whole tile inside the tensor, every operand either along pax or along the innermost axis:
     // 16-byte accesses on both sides, one barrier
-    if (p0 + 64 <= A.P && l0 + 64 <= A.L && !A.careful) {
+    if (p0 + TILE_P <= A.P && l0 + TILE_L <= A.L && !A.careful) {
+        const unsigned rq = threadIdx.x % R_LPR, rr = threadIdx.x / R_LPR;
+        const unsigned wq = threadIdx.x % W_LPR, wr = threadIdx.x / W_LPR;
 #pragma unroll
         for (int j = 0; j < NSRC; j++) {
-            if (j < A.nsrc && ((A.turned >> j) & 1u)) {
-                const T* sp = (const T*)srcs.p[j] + off[j + 1] + p0 + q * VEC;           // stride 1 along pax
-                const int64_t sL = A.stride[j + 1][last];
+            if (j < A.nsrc) {
+                if ((A.turned >> j) & 1u) {
+                    const T* sp = (const T*)srcs.p[j] + off[j + 1] + p0 + rq * VEC;      // stride 1 along pax
+                    const int64_t sL = A.stride[j + 1][last];
 #pragma unroll
-                for (int it = 0; it < NIT; it++) {
-                    const unsigned ll = r + RPI * it;
-                    T v[VEC];
-                    load_vec<T, VEC>(v, sp + (int64_t)(l0 + ll) * sL);
+                    for (int it = 0; it < R_NIT; it++) {
+                        const unsigned ll = rr + R_RPI * it;
+                        T v[VEC];
+                        load_vec<T, VEC, NT>(v, sp + (int64_t)(l0 + ll) * sL);
 #pragma unroll
-                    for (int e = 0; e < VEC; e++) tiles[j][ll][q * VEC + e] = v[e];
+                        for (int e = 0; e < VEC; e++) tiles[j][ll][rq * VEC + e] = v[e];
+                    }
+                } else {
+                    const T* sp = (const T*)srcs.p[j] + off[j + 1] + l0 + wq * VEC;      // stride 1 along the innermost axis
+                    const int64_t sP = A.stride[j + 1][A.pax];
+#pragma unroll
+                    for (int it = 0; it < W_NIT; it++) {
+                        T (&xv)[VEC] = *reinterpret_cast<T (*)[VEC]>(&x[j][it * VEC]);
+                        load_vec<T, VEC, NT>(xv, sp + (int64_t)(p0 + wr + W_RPI * it) * sP);
+                    }
                 }
+            } else {
+#pragma unroll
+                for (int e = 0; e < EPT; e++) x[j][e] = T(0);
             }
         }
         __syncthreads();
-        T* dp = drn + off[0] + l0 + q * VEC;
 #pragma unroll
-        for (int c = 0; c < NIT; c += CIT) {
-            T x[NSRC][CHUNK];
-            T out[CHUNK];
+        for (int j = 0; j < NSRC; j++) {
+            if (j < A.nsrc && ((A.turned >> j) & 1u)) {
 #pragma unroll
-            for (int j = 0; j < NSRC; j++) {
-                if (j < A.nsrc) {
-                    if ((A.turned >> j) & 1u) {
+                for (int it = 0; it < W_NIT; it++)
 #pragma unroll
-                        for (int it = 0; it < CIT; it++)
-#pragma unroll
-                            for (int e = 0; e < VEC; e++) x[j][it * VEC + e] = tiles[j][q * VEC + e][r + RPI * (c + it)];
-                    } else {
-                        const T* sp = (const T*)srcs.p[j] + off[j + 1] + l0 + q * VEC;   // stride 1 along the innermost axis
-                        const int64_t sP = A.stride[j + 1][A.pax];
-#pragma unroll
-                        for (int it = 0; it < CIT; it++) {
-                            T (&xv)[VEC] = *reinterpret_cast<T (*)[VEC]>(&x[j][it * VEC]);
-                            load_vec<T, VEC>(xv, sp + (int64_t)(p0 + r + RPI * (c + it)) * sP);
-                        }
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < CHUNK; e++) x[j][e] = T(0);
-                }
+                    for (int e = 0; e < VEC; e++) x[j][it * VEC + e] = tiles[j][wq * VEC + e][wr + W_RPI * it];
             }
-            run_any<T, CHUNK, NSRC, FUNSET>(P, LP, x, out);
+        }
+        run_any<T, EPT, NSRC, FUNSET>(P, LP, x, out);
+        T* dp = drn + off[0] + l0 + wq * VEC;
 #pragma unroll
-            for (int it = 0; it < CIT; it++) {
-                T (&ov)[VEC] = *reinterpret_cast<T (*)[VEC]>(&out[it * VEC]);
-                store_vec<T, VEC>(dp + (int64_t)(p0 + r + RPI * (c + it)) * dP, ov, A.streaming != 0);
-            }
+        for (int it = 0; it < W_NIT; it++) {
+            T (&ov)[VEC] = *reinterpret_cast<T (*)[VEC]>(&out[it * VEC]);
+            store_vec<T, VEC>(dp + (int64_t)(p0 + wr + W_RPI * it) * dP, ov, A.streaming != 0);
         }
         return;
     }
 
     // edge tiles and operands that are constant along the innermost axis: element by element, bounds checked
-    const unsigned tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    constexpr int S_RPI = 256 / TILE_P;            // rows of TILE_P lanes in the block
+    const unsigned tx = threadIdx.x % TILE_P, ty = threadIdx.x / TILE_P;
 #pragma unroll
     for (int j = 0; j < NSRC; j++) {
         if (j < A.nsrc && ((A.turned >> j) & 1u)) {
             const T* sp = (const T*)srcs.p[j] + off[j + 1];
             const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
-            for (int it = 0; it < 16; it++) {
-                const unsigned l = l0 + ty + 4 * it, p = p0 + tx;
-                if (l < A.L && p < A.P) tiles[j][ty + 4 * it][tx] = sp[(int64_t)p * sP + (int64_t)l * sL];
+            for (int it = 0; it < EPT; it++) {
+                const unsigned l = l0 + ty + S_RPI * it, p = p0 + tx;
+                if (l < A.L && p < A.P) tiles[j][ty + S_RPI * it][tx] = sp[(int64_t)p * sP + (int64_t)l * sL];
             }
         }
     }
     __syncthreads();
-    for (int c = 0; c < 16; c += 8) {
-        T x[NSRC][8];
-        T out[8];
+    // drain side of the slow path: lane -> innermost index, TILE_L lanes per row of the tile
+    constexpr int D_RPI = 256 / TILE_L;
+    const unsigned dx = threadIdx.x % TILE_L, dy = threadIdx.x / TILE_L;
 #pragma unroll
-        for (int j = 0; j < NSRC; j++) {
-            if (j < A.nsrc) {
-                if ((A.turned >> j) & 1u) {
+    for (int j = 0; j < NSRC; j++) {
+        if (j < A.nsrc) {
+            if ((A.turned >> j) & 1u) {
 #pragma unroll
-                    for (int it = 0; it < 8; it++) x[j][it] = tiles[j][tx][ty + 4 * (c + it)];
-                } else {
-                    const T* sp = (const T*)srcs.p[j] + off[j + 1];
-                    const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
-#pragma unroll
-                    for (int it = 0; it < 8; it++) {
-                        const unsigned p = p0 + ty + 4 * (c + it), l = l0 + tx;
-                        x[j][it] = (p < A.P && l < A.L) ? sp[(int64_t)p * sP + (int64_t)l * sL] : T(0);
-                    }
-                }
+                for (int it = 0; it < EPT; it++) x[j][it] = tiles[j][dx][dy + D_RPI * it];
             } else {
+                const T* sp = (const T*)srcs.p[j] + off[j + 1];
+                const int64_t sP = A.stride[j + 1][A.pax], sL = A.stride[j + 1][last];
 #pragma unroll
-                for (int it = 0; it < 8; it++) x[j][it] = T(0);
+                for (int it = 0; it < EPT; it++) {
+                    const unsigned p = p0 + dy + D_RPI * it, l = l0 + dx;
+                    x[j][it] = (p < A.P && l < A.L) ? sp[(int64_t)p * sP + (int64_t)l * sL] : T(0);
+                }
             }
+        } else {
+#pragma unroll
+            for (int it = 0; it < EPT; it++) x[j][it] = T(0);
         }
-        run_any<T, 8, NSRC, FUNSET>(P, LP, x, out);
+    }
+    run_any<T, EPT, NSRC, FUNSET>(P, LP, x, out);
 #pragma unroll
-        for (int it = 0; it < 8; it++) {
-            const unsigned p = p0 + ty + 4 * (c + it), l = l0 + tx;
-            if (p < A.P && l < A.L) {
-                T* dst = drn + off[0] + (int64_t)p * dP + l;
-                if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
-            }
+    for (int it = 0; it < EPT; it++) {
+        const unsigned p = p0 + dy + D_RPI * it, l = l0 + dx;
+        if (p < A.P && l < A.L) {
+            T* dst = drn + off[0] + (int64_t)p * dP + l;
+            if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
         }
     }
 }

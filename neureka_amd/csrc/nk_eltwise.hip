@@ -277,11 +277,15 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             TileArgs& A = plan.tile;
             A.rank = cn.rank; A.nsrc = c.nsrc; A.pax = pax; A.turned = turned;
             A.streaming = streaming ? 1 : 0;
+            bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
+            for (int j = 0; j < c.nsrc && once; j++)
+                for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) once = false;
+            A.nt_loads = once ? 1 : 0;
             A.careful = 0;
             for (int j = 0; j < c.nsrc; j++)
                 if (!((turned >> j) & 1u) && cn.stride[j + 1][last] == 0) A.careful = 1;
             A.P = (unsigned)cn.shape[pax]; A.L = (unsigned)cn.shape[last];
-            A.tiles_p = (A.P + 63) / 64; A.tiles_l = (A.L + 63) / 64;
+            A.tiles_p = (A.P + TILE_P - 1) / TILE_P; A.tiles_l = (A.L + TILE_L - 1) / TILE_L;
             uint64_t nb = (uint64_t)A.tiles_p * A.tiles_l;
             for (int k = 0; k < last; k++) {
                 if (k == pax) continue;
@@ -290,7 +294,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             }
             if (nb < ((uint64_t)1 << 31)) {
                 A.n_blocks = (unsigned)nb;
-                static const int env_group = [] { const char* v = getenv("NK_TILE_GROUP_LOG2"); return v && *v ? atoi(v) : 2; }();
+                static const int env_group = [] { const char* v = getenv("NK_TILE_GROUP_LOG2"); return v && *v ? atoi(v) : 3; }();
                 int gl = env_group < 0 ? 0 : (env_group > 4 ? 4 : env_group);
                 while (gl > 0 && (A.tiles_l % (1u << gl) || A.tiles_p % (1u << gl))) gl--;
                 A.group_log2 = gl;
