@@ -61,10 +61,22 @@ __device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int& tm, int& t
     tn = in_grp / rows;
 }
 
+// operands of one depth-8 chunk of a k-slice for the wave's 64x64 sub-tile
+struct Frag {
+    f32x4 a0, a1;          // rows wm + l32 and wm + 32 + l32, k = 8c + 4h .. + 3
+    float b0[4], b1[4];    // columns wn + l32 and wn + 32 + l32, same k
+};
+
+constexpr int C_PITCH = BN + 4;
+constexpr int LDS_FLOATS_AB = 2 * BM * A_PITCH + 2 * BK * B_PITCH;
+constexpr int LDS_FLOATS_C = BM * C_PITCH;
+constexpr int LDS_FLOATS = LDS_FLOATS_AB > LDS_FLOATS_C ? LDS_FLOATS_AB : LDS_FLOATS_C;
+
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const float* __restrict__ A,
                                                           const float* __restrict__ B, float* __restrict__ C) {
-    __shared__ __attribute__((aligned(16))) float As[2][BM * A_PITCH];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK * B_PITCH];
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    float* const As0 = lds;                                   // [2][BM * A_PITCH]
+    float* const Bs0 = lds + 2 * BM * A_PITCH;                // [2][BK * B_PITCH]
 
     int tm, tn;
     tile_of_block(g, tm, tn);
@@ -89,10 +101,25 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
         }
     };
     auto store_lds = [&](int buf) {
+        float* as = As0 + buf * (BM * A_PITCH);
+        float* bs = Bs0 + buf * (BK * B_PITCH);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            *(f32x4*)(&As[buf][(a_row + 32 * i) * A_PITCH + a_col]) = ra[i];
-            *(f32x4*)(&Bs[buf][(b_row + 8 * i) * B_PITCH + b_col]) = rb[i];
+            *(f32x4*)(&as[(a_row + 32 * i) * A_PITCH + a_col]) = ra[i];
+            *(f32x4*)(&bs[(b_row + 8 * i) * B_PITCH + b_col]) = rb[i];
+        }
+    };
+    // lane half h owns k = 8c + 4h .. 8c + 4h + 3 of chunk c; the four MFMA steps pair (k, k + 4):
+    // any pairing works as long as A and B use the same one
+    auto read_frag = [&](Frag& f, int buf, int c) {
+        const float* as = As0 + buf * (BM * A_PITCH);
+        const float* bs = Bs0 + buf * (BK * B_PITCH);
+        f.a0 = *(const f32x4*)(&as[(wm + l32) * A_PITCH + 8 * c + 4 * h]);
+        f.a1 = *(const f32x4*)(&as[(wm + 32 + l32) * A_PITCH + 8 * c + 4 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            f.b0[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + l32];
+            f.b1[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + 32 + l32];
         }
     };
 
@@ -103,55 +130,78 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    auto mma = [&](const Frag& f) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b0[t], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b1[t], acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b0[t], acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b1[t], acc[1][1], 0, 0, 0);
+        }
+    };
 
+    // Software pipeline over the k-slices.  While the matrix cores work on chunk c of the current slice the
+    // operands of chunk c + 1 are read from LDS; the next slice (fetched from global memory at the top of
+    // the slice) is written to the other LDS buffer in the middle of the slice; the single barrier sits
+    // before the last chunk's multiply-adds, which then cover the read of the next slice's first chunk.
+    // A buffer is rewritten only after a barrier that every wavefront reaches with all its reads of that
+    // buffer complete.
+    static_assert(BK == 32, "the pipeline below is written for four depth-8 chunks per slice");
     const int nk = g.K / BK;
+    Frag f0, f1;
     load_global(0);
     store_lds(0);
     __syncthreads();
-
-    for (int kt = 0; kt < nk; kt++) {
+    read_frag(f0, 0, 0);
+    for (int kt = 0; kt + 1 < nk; kt++) {                  // branch-free body; the last slice is peeled off below
         const int cur = kt & 1;
-        if (kt + 1 < nk) load_global((kt + 1) * BK);
-        const float* as = As[cur];
-        const float* bs = Bs[cur];
-#pragma unroll
-        for (int c = 0; c < BK / 8; c++) {
-            // lane half h owns k = 8c + 4h .. 8c + 4h + 3 of this chunk; the four MFMA steps pair
-            // (k, k + 4): any pairing works as long as A and B use the same one
-            f32x4 a0 = *(const f32x4*)(&as[(wm + l32) * A_PITCH + 8 * c + 4 * h]);
-            f32x4 a1 = *(const f32x4*)(&as[(wm + 32 + l32) * A_PITCH + 8 * c + 4 * h]);
-            float b0[4], b1[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                b0[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + l32];
-                b1[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + 32 + l32];
-            }
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[t], b0[t], acc[0][0], 0, 0, 0);
-                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[t], b1[t], acc[0][1], 0, 0, 0);
-                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[t], b0[t], acc[1][0], 0, 0, 0);
-                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[t], b1[t], acc[1][1], 0, 0, 0);
-            }
-        }
-        if (kt + 1 < nk) {
-            store_lds(cur ^ 1);
-            __syncthreads();
-        }
+        load_global((kt + 1) * BK);
+        read_frag(f1, cur, 1);
+        mma(f0);
+        read_frag(f0, cur, 2);
+        mma(f1);
+        store_lds(cur ^ 1);
+        read_frag(f1, cur, 3);
+        mma(f0);
+        __syncthreads();
+        read_frag(f0, cur ^ 1, 0);
+        mma(f1);
+    }
+    {
+        const int cur = (nk - 1) & 1;
+        read_frag(f1, cur, 1);
+        mma(f0);
+        read_frag(f0, cur, 2);
+        mma(f1);
+        read_frag(f1, cur, 3);
+        mma(f0);
+        mma(f1);
     }
 
-    // epilogue: accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4, column l32
-    float* Cg = C + (int64_t)(tm * BM + wm) * g.N + tn * BN + wn;
+    // epilogue: the block's 128x128 result goes through LDS so that C is read and written in 16-byte pieces
+    // along its rows; accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4, column l32
+    __syncthreads();
+    float* cs = lds;
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int row = 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
-                float* p = Cg + (int64_t)row * g.N + 32 * j + l32;
-                *p = *p + acc[i][j][v];
+                const int row = wm + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
+                cs[row * C_PITCH + wn + 32 * j + l32] = acc[i][j][v];
             }
+    __syncthreads();
+    float* Cg = C + (int64_t)tm * BM * g.N + tn * BN;
+    const int c_col = (tid & 31) * 4, c_row = tid >> 5;
+    f32x4 old[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) old[i] = *(const f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col);
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const f32x4 add = *(const f32x4*)(&cs[(c_row + 8 * i) * C_PITCH + c_col]);
+        *(f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col) = old[i] + add;
+    }
 }
 
 template <typename T>
