@@ -308,11 +308,11 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
 
 // gradient w.r.t. the taps: dk[c][ky][kx] = sum_y sum_x in[c][y+ky][x+kx] * err[y][x]
 //   = sum over input elements (yy, xx) of in[c][yy][xx] * err[yy-ky][xx-kx]
-// wave -> (256-column block over W, strip of S input rows, channel).  The KH-row err window around the
-// lane's CX input elements slides down the strip; every input element is loaded once (16-byte loads) and
-// multiplied into KH*KW accumulators; the loads of the next row are issued before the current row's
-// arithmetic.  Lanes are reduced with wavefront shuffles, strips by a second pass.
-template <typename T, int KH, int KW>
+// wave -> (256-column block over W, strip of S input rows, channel).  The strip is worked off in chunks of R
+// rows: the chunk's R input rows (16-byte loads) and the R + KH - 1 err rows around them are all requested
+// before the first multiply-add, then every input element is multiplied into the KH*KW accumulators with
+// statically indexed registers.  Lanes are reduced with wavefront shuffles, strips by a second pass.
+template <typename T, int KH, int KW, int R>
 __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstrips, const T* __restrict__ in, const T* __restrict__ err, T* __restrict__ partial) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int strip = blockIdx.y * 4 + wave;
@@ -341,61 +341,72 @@ __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstri
 #pragma unroll
         for (int kx = 0; kx < KW; kx++) acc[ky][kx] = T(0);
     const BufRsrc ebuf = buffer_of(err, (unsigned)(g.OH * g.OW) * 4u);
-    auto err_row = [&](int ey, T (&dst)[CX + KW - 1]) {           // dst[i] = err[ey][xx - (KW-1) + i], zero outside
-        const bool row_ok = ey >= 0 && ey < g.OH;
-        const unsigned row = (unsigned)(clampi(ey, 0, g.OH - 1) * g.OW) * 4u;
-#pragma unroll
-        for (int i = 0; i < CX + KW - 1; i++) dst[i] = buffer_load(ebuf, eoff[i], row);
-#pragma unroll
-        for (int i = 0; i < CX + KW - 1; i++) dst[i] = row_ok && col_ok[i] ? dst[i] : T(0);
-    };
     const BufRsrc plane = buffer_of(in + (int64_t)c * g.H * g.W, (unsigned)(g.H * g.W) * 4u);
-    auto in_row = [&](int yy, T (&dst)[CX]) {                     // dst[j] = in[c][yy][xx + j], zero past the row
-        const unsigned row = (unsigned)((yy < g.H ? yy : g.H - 1) * g.W) * 4u;
-        if (vec_ok) {
-            const f32x4u q = buffer_load4(plane, voff[0], row);
+    for (int y = yy0; y < yy1; y += R) {
+        T E[R + KH - 1][CX + KW - 1];                             // E[rr] = err row y - (KH-1) + rr, zero outside err
+        T V[R][CX];                                               // V[r] = input row y + r, zero past the strip
 #pragma unroll
-            for (int j = 0; j < CX; j++) dst[j] = q[j];
-        } else {
+        for (int r = 0; r < R; r++) {
+            const unsigned row = (unsigned)((y + r < g.H ? y + r : g.H - 1) * g.W) * 4u;
+            if (vec_ok) {
+                const f32x4u q = buffer_load4(plane, voff[0], row);
 #pragma unroll
-            for (int j = 0; j < CX; j++) { const T t = buffer_load(plane, voff[j], row); dst[j] = v_ok[j] ? t : T(0); }
+                for (int j = 0; j < CX; j++) V[r][j] = q[j];
+            } else {
+#pragma unroll
+                for (int j = 0; j < CX; j++) V[r][j] = buffer_load(plane, voff[j], row);
+            }
         }
-    };
-    T Ew[KH][CX + KW - 1];                                        // Ew[ky] = err row yy - ky
 #pragma unroll
-    for (int ky = 1; ky < KH; ky++) err_row(yy0 - ky, Ew[ky]);
-    T nextE[CX + KW - 1], nextV[CX];
-    err_row(yy0, nextE);
-    in_row(yy0, nextV);
-    for (int yy = yy0; yy < yy1; yy++) {
-        T v[CX];
+        for (int rr = 0; rr < R + KH - 1; rr++) {
+            const unsigned row = (unsigned)(clampi(y - (KH - 1) + rr, 0, g.OH - 1) * g.OW) * 4u;
 #pragma unroll
-        for (int i = 0; i < CX + KW - 1; i++) Ew[0][i] = nextE[i];
+            for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = buffer_load(ebuf, eoff[i], row);
+        }
 #pragma unroll
-        for (int j = 0; j < CX; j++) v[j] = nextV[j];
-        err_row(yy + 1, nextE);                                   // one row ahead; past the strip it is loaded (clamped) and dropped
-        in_row(yy + 1, nextV);
+        for (int r = 0; r < R; r++) {
+            const bool row_live = y + r < yy1;
+#pragma unroll
+            for (int j = 0; j < CX; j++) V[r][j] = row_live && v_ok[j] ? V[r][j] : T(0);
+        }
+#pragma unroll
+        for (int rr = 0; rr < R + KH - 1; rr++) {
+            const int ey = y - (KH - 1) + rr;
+            const bool row_ok = ey >= 0 && ey < g.OH;
+#pragma unroll
+            for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = row_ok && col_ok[i] ? E[rr][i] : T(0);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++)
+#pragma unroll
+                    for (int j = 0; j < CX; j++) acc[ky][kx] = fused_mad(V[r][j], E[r - ky + KH - 1][j - kx + KW - 1], acc[ky][kx]);
+    }
+    // lanes -> lane 0: every step moves all KH*KW sums before any of them is added, so the cross-lane
+    // exchanges of one step are in flight together instead of one dependent chain per sum
+    const int part = strip * gridDim.x + blockIdx.x;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        T moved[KH][KW];
 #pragma unroll
         for (int ky = 0; ky < KH; ky++)
 #pragma unroll
-            for (int kx = 0; kx < KW; kx++)
+            for (int kx = 0; kx < KW; kx++) moved[ky][kx] = __shfl_down(acc[ky][kx], off, 64);
 #pragma unroll
-                for (int j = 0; j < CX; j++) acc[ky][kx] = fused_mad(v[j], Ew[ky][j - kx + KW - 1], acc[ky][kx]);
+        for (int ky = 0; ky < KH; ky++)
 #pragma unroll
-        for (int ky = KH - 1; ky >= 1; ky--)
-#pragma unroll
-            for (int i = 0; i < CX + KW - 1; i++) Ew[ky][i] = Ew[ky - 1][i];
+            for (int kx = 0; kx < KW; kx++) acc[ky][kx] += moved[ky][kx];
     }
-    const int part = strip * gridDim.x + blockIdx.x;
+    if (lane == 0) {
+        T* dst = partial + ((int64_t)part * g.C + c) * (KH * KW);
 #pragma unroll
-    for (int ky = 0; ky < KH; ky++)
+        for (int ky = 0; ky < KH; ky++)
 #pragma unroll
-        for (int kx = 0; kx < KW; kx++) {
-            T v = acc[ky][kx];
-#pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) v += __shfl_down(v, off, 64);
-            if (lane == 0) partial[((int64_t)part * g.C + c) * (KH * KW) + ky * KW + kx] = v;
-        }
+            for (int kx = 0; kx < KW; kx++) dst[ky * KW + kx] = acc[ky][kx];
+    }
 }
 
 static bool dense_rm(const Cfg& c, int rank) {
@@ -505,11 +516,12 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
             g.C = c0.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2]; g.OH = OH; g.OW = OW;
             g.col_blocks = (g.W + 64 * CX - 1) / (64 * CX);
             g.cg = 1;
-            // rows per strip: enough strips for the machine, at least 8 rows to amortise the window set-up
+            // rows per strip: enough strips for the machine, a whole number of R-row chunks each
+            constexpr int R = 8;
             int64_t strips = (want_waves + (int64_t)g.col_blocks * g.C - 1) / ((int64_t)g.col_blocks * g.C);
             if (strips < 1) strips = 1;
             int S = (int)((g.H + strips - 1) / strips);
-            if (S < 8) S = 8;
+            S = (S + R - 1) / R * R;
             const int nstrips = (g.H + S - 1) / S;
             const int parts = nstrips * g.col_blocks;
             int rc = NK_OK;
@@ -519,7 +531,7 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
                 void* ws = nullptr;
                 if ((rc = workspace(dev, (uint64_t)parts * on * sizeof(T), &ws))) return;
                 dim3 grid(g.col_blocks, (nstrips + 3) / 4, g.C);
-                hipLaunchKernelGGL((conv_chan_dk<T, KK, KK>), grid, dim3(256), 0, dev->stream, g, S, nstrips, s1, s2, (T*)ws);
+                hipLaunchKernelGGL((conv_chan_dk<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, S, nstrips, s1, s2, (T*)ws);
                 hipLaunchKernelGGL(conv_partial_reduce_wide<T>, dim3((on + 3) / 4), dim3(256), 0, dev->stream, parts, on, (const T*)ws, out);
             });
             if (!ok) return NK_OK;
