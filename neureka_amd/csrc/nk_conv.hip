@@ -545,12 +545,60 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
     return NK_OK;
 }
 
+// Forward 2-D convolution of dense row-major operands with one set of taps, [H,W] x [kh,kw] or
+// [B,H,W] x [1,kh,kw]: the case the reference's CPU device hands to SimpleCPUConvolution
+// (J/backend/main/implementations/convolution/AbstractCPUConvolution.java:18-23, SimpleCPUConvolution.java:143-159).
+// One thread per output element, taps through scalar loads, the sum in that class's order (ky outer, kx inner,
+// product rounded before the add): bit-identical to it in f32 and f64.
+template <typename T>
+__global__ __launch_bounds__(256) void conv2d_direct(int B, int H, int W, int KH, int KW, const T* __restrict__ img,
+                                                     const T* __restrict__ taps, T* __restrict__ out) {
+    const int OH = H - KH + 1, OW = W - KW + 1;
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= B * OH * OW) return;
+    const int b = idx / (OH * OW);
+    const int rem = idx - b * (OH * OW);
+    const int y = rem / OW, x = rem - y * OW;
+    const T* p = img + ((int64_t)b * H + y) * W + x;
+    T sum = T(0);
+    for (int ky = 0; ky < KH; ky++)
+        for (int kx = 0; kx < KW; kx++) {
+            const T prod = p[ky * W + kx] * taps[ky * KW + kx];
+            sum = sum + prod;
+        }
+    out[idx] = sum;
+}
+
+template <typename T>
+static bool conv2d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& c0, const T* s1, const Cfg& c1, const T* s2, const Cfg& c2) {
+    if (d >= 0 || (rank != 2 && rank != 3)) return false;
+    if (!dense_rm(c0, rank) || !dense_rm(c1, rank) || !dense_rm(c2, rank)) return false;
+    const int o = rank - 2;
+    const bool a_img = c1.shape[o] >= c2.shape[o] && c1.shape[o + 1] >= c2.shape[o + 1];
+    const bool b_img = c2.shape[o] >= c1.shape[o] && c2.shape[o + 1] >= c1.shape[o + 1];
+    if (!a_img && !b_img) return false;
+    const Cfg& img = a_img ? c1 : c2;
+    const Cfg& tap = a_img ? c2 : c1;
+    if (rank == 3 && tap.shape[0] != 1) return false;
+    const int B = rank == 3 ? (int)img.shape[0] : 1;
+    const int64_t n = (int64_t)B * (img.shape[o] - tap.shape[o] + 1) * (img.shape[o + 1] - tap.shape[o + 1] + 1);
+    if (n >= ((int64_t)1 << 31)) return false;
+    set_path("simple2d");
+    hipLaunchKernelGGL(conv2d_direct<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, dev->stream, B, (int)img.shape[o], (int)img.shape[o + 1],
+                       (int)tap.shape[o], (int)tap.shape[o + 1], a_img ? s1 : s2, a_img ? s2 : s1, out);
+    return true;
+}
+
 template <typename T>
 static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, nk_buf a, const Cfg& c1, nk_buf b,
                       const Cfg& c2, int64_t n) {
     T* out = (T*)drn;
     const T* s1 = (const T*)a;
     const T* s2 = (const T*)b;
+    if (conv2d_direct_path<T>(dev, d, rank, out, c0, s1, c1, s2, c2)) {
+        NK_HIP(hipGetLastError());
+        return NK_OK;
+    }
     if constexpr (sizeof(T) == 4) {
         if (rank == 3 && dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank)) {
             bool taken = false;

@@ -429,7 +429,13 @@ def test_convolution_literal_kernels_bit_exact(device, orc, dt):
         want = orc.convolve(np.zeros(out.size, dtype=F[dt]), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
         if _lib.last_path().startswith("literal"):
             assert_bits(out.getData(), want, f"fwd {xs} {ks}")
-        else:       # dense f32 [C,H,W] x [C,kh,kw] takes the LDS kernel: same sums in another order
+        elif _lib.last_path() == "simple2d":        # what the reference hands to SimpleCPUConvolution: its order, bit for bit
+            img, tap, ishape, tshape = (x, k, xs, ks) if xs[-1] >= ks[-1] else (k, x, ks, xs)
+            assert len(xs) == 2 or tshape[0] == 1
+            simple = orc.simple_conv2d(img.reshape(-1), tap.reshape(-1), ishape[-1], ishape[-2], tshape[-1], tshape[-2], batch=ishape[0] if len(xs) == 3 else 1)
+            assert_bits(out.getData(), simple, f"fwd simple {xs} {ks}")
+            np.testing.assert_allclose(out.getData(), want, rtol=1e-5 if dt == "f32" else 1e-12, atol=1e-5 if dt == "f32" else 1e-12)
+        else:       # dense f32 [C,H,W] x [C,kh,kw] takes the channel kernel: same sums in another order
             assert dt == "f32" and len(xs) == 3
             np.testing.assert_allclose(out.getData(), want, rtol=1e-5, atol=1e-5)
         for tgt, tgt_shape, other, other_arr, other_shape in ((tx, xs, tk, k, ks), (tk, ks, tx, x, xs)):
@@ -505,9 +511,9 @@ def test_conv2d_config1_shape(device, orc):
     x = rng.uniform(-1, 1, (64, 64)).astype(np.float32); k = rng.uniform(-1, 1, (3, 3)).astype(np.float32)
     y = on(device, x).conv(on(device, k))
     assert y.shape == (62, 62)
+    assert _lib.last_path() == "simple2d"
     want = orc.simple_conv2d(x.reshape(-1), k.reshape(-1), 64, 64, 3, 3)
-    bound = 1e-5 * orc.simple_conv2d(np.abs(x).reshape(-1), np.abs(k).reshape(-1), 64, 64, 3, 3)
-    assert (np.abs(y.items - want) <= bound).all()
+    assert_bits(y.items, want, "SimpleCPUConvolution order")
 
 
 # ---- matmul ---------------------------------------------------------------------------------------------------
