@@ -230,8 +230,9 @@ __device__ __forceinline__ void store_vec(T* p, const T (&src)[V], bool streamin
 // ---- rows kernel -----------------------------------------------------------------------------------
 // Every operand is contiguous (stride 1) or constant (stride 0) along the innermost collapsed axis.
 // The work is cut into units of (256 >> tpr_log2 rows) x (tpr threads x V elements); a block owns PASSES
-// consecutive units; a thread issues the loads of all its passes, runs the program once over all of
-// them, then stores.  When a row spans at least a wavefront (tpr >= 64) the row index is wave-uniform:
+// units: consecutive ones, or (forward broadcast) the same column chunk of PASSES consecutive row groups, so
+// that an operand which does not change along the rows is the same piece of memory in every pass.  A thread
+// issues the loads of all its passes, runs the program once over all of them, then stores.  When a row spans at least a wavefront (tpr >= 64) the row index is wave-uniform:
 // the nd-index arithmetic then runs on the scalar unit.  Element offsets are 32-bit (the host checks),
 // at most ROWS_MAX_OUTER outer axes (more fall to the canon kernel); the argument block is small and
 // fixed-size so that it is fetched with a few wide scalar loads at kernel start.
@@ -246,7 +247,8 @@ struct RowsArgs {
     unsigned n_rows;           // product of the outer extents
     int tpr_log2;              // threads per row, log2
     unsigned chunks;           // column chunks per row
-    unsigned n_units;          // row groups x chunks
+    unsigned row_groups;       // groups of (256 >> tpr_log2) rows
+    int pass_rows;             // a block's passes walk down the rows (same chunk) instead of along the chunks
     unsigned const_last;       // bit j: source j has stride 0 along the innermost axis
     int simple_loads;          // every source register is filled by a plain vector load
     int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
@@ -266,16 +268,14 @@ struct RowsAddr {
     bool live;
 };
 template <int NOPS>
-__device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsigned u) {
+__device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsigned rg, unsigned chunk) {
     const unsigned tpr = 1u << A.tpr_log2;
     const unsigned rows_per_pass = 256u >> A.tpr_log2;
     const unsigned sub = threadIdx.x >> A.tpr_log2, lane = threadIdx.x & (tpr - 1);
-    const unsigned rg = A.chunk_div.div(u);                         // u is block-uniform
-    const unsigned chunk = u - rg * A.chunks;
-    unsigned row = rg * rows_per_pass + sub;
+    unsigned row = rg * rows_per_pass + sub;                        // rg and chunk are block-uniform
     RowsAddr<NOPS> R;
     R.col = (chunk * tpr + lane) * (unsigned)A.vec;
-    const bool row_ok = u < A.n_units && row < A.n_rows;            // wave-uniform when a row spans a wavefront
+    const bool row_ok = rg < A.row_groups && row < A.n_rows;        // wave-uniform when a row spans a wavefront
     R.live = row_ok && R.col < A.L;
     if (!row_ok) row = 0;                                           // dead lanes get a valid address:
     if (!R.live) R.col = 0;                                         // loads need no predicate
@@ -299,6 +299,20 @@ __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsign
     return R;
 }
 
+// (block id, pass) -> (row group, column chunk).  Units are numbered with the chunk varying fastest; a block
+// either owns `passes` consecutive units, or -- pass_rows -- the same chunk of `passes` consecutive row groups.
+__device__ __forceinline__ void rows_unit(const RowsArgs& A, int passes, int p, unsigned& rg, unsigned& chunk) {
+    if (A.pass_rows) {
+        const unsigned rgb = A.chunk_div.div(blockIdx.x);
+        chunk = blockIdx.x - rgb * A.chunks;
+        rg = rgb * (unsigned)passes + (unsigned)p;
+    } else {
+        const unsigned u = blockIdx.x * (unsigned)passes + (unsigned)p;
+        rg = A.chunk_div.div(u);
+        chunk = u - rg * A.chunks;
+    }
+}
+
 template <typename T, int V, int NSRC, int FUNSET, int PASSES, bool NT = false>
 __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
     T x[NSRC][PASSES * V];
@@ -308,7 +322,9 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
         // every source is a plain vector load: no branches between the loads of all passes
 #pragma unroll
         for (int p = 0; p < PASSES; p++) {
-            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, blockIdx.x * PASSES + p);
+            unsigned rg, chunk;
+            rows_unit(A, PASSES, p, rg, chunk);
+            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, rg, chunk);
             live[p] = R.live;
             doff[p] = R.off[0] + (int)R.col;
 #pragma unroll
@@ -320,7 +336,9 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
     } else {
 #pragma unroll
         for (int p = 0; p < PASSES; p++) {
-            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, blockIdx.x * PASSES + p);
+            unsigned rg, chunk;
+            rows_unit(A, PASSES, p, rg, chunk);
+            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, rg, chunk);
             live[p] = R.live;
             doff[p] = R.off[0] + (int)R.col;
 #pragma unroll
@@ -356,7 +374,8 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
 // drain = src0 op src1 with op in {+, -, *, /} and plain aligned loads: the bandwidth-critical case
 // (same-shape elementwise and forward broadcast).  The operator is resolved once, outside the passes,
 // and each pass is stored as soon as its operands have arrived.
-template <typename T, int V, int PASSES, bool NT = false>
+// HOIST bit j: source j does not change along the rows a block covers (forward broadcast): it is loaded once.
+template <typename T, int V, int PASSES, bool NT = false, int HOIST = 0>
 __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T* __restrict__ drn, const T* __restrict__ s0,
                                                           const T* __restrict__ s1) {
     T x0[PASSES][V], x1[PASSES][V];
@@ -364,11 +383,22 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
     bool live[PASSES];
 #pragma unroll
     for (int p = 0; p < PASSES; p++) {
-        const RowsAddr<3> R = rows_address<3>(A, blockIdx.x * PASSES + p);
+        unsigned rg, chunk;
+        rows_unit(A, PASSES, p, rg, chunk);
+        const RowsAddr<3> R = rows_address<3>(A, rg, chunk);
         live[p] = R.live;
         doff[p] = R.off[0] + (int)R.col;
-        load_vec<T, V, NT>(x0[p], s0 + R.off[1] + R.col);
-        load_vec<T, V, NT>(x1[p], s1 + R.off[2] + R.col);
+        if (p == 0 || !(HOIST & 1)) load_vec<T, V, NT>(x0[p], s0 + R.off[1] + R.col);
+        if (p == 0 || !(HOIST & 2)) load_vec<T, V, NT>(x1[p], s1 + R.off[2] + R.col);
+    }
+    if (HOIST) {
+#pragma unroll
+        for (int p = 1; p < PASSES; p++)
+#pragma unroll
+            for (int v = 0; v < V; v++) {
+                if (HOIST & 1) x0[p][v] = x0[0][v];
+                if (HOIST & 2) x1[p][v] = x1[0][v];
+            }
     }
 #define NK_BINARY_PASSES(EXPR)                                                        \
     _Pragma("unroll") for (int p = 0; p < PASSES; p++) {                              \
@@ -637,6 +667,7 @@ enum PlanKind { PLAN_ROWS, PLAN_ROWS_BINARY, PLAN_TILE, PLAN_CANON, PLAN_LITERAL
 struct Plan {
     PlanKind kind;
     bool vec;                  // rows: 16-byte vectors
+    int hoist = 0;             // rows_binary_kernel: bit j = source j is loaded once per block
     int binary_op;             // PLAN_ROWS_BINARY
     int passes;                // PLAN_ROWS_BINARY: units per block (2, 4 or 8)
     int nsrc;

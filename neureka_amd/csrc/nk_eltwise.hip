@@ -230,9 +230,8 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         const unsigned tpr = 1u << l2, rpp = 256u >> l2;
         A.chunks = (unsigned)((vec_per_row + tpr - 1) / tpr);
         const uint64_t row_groups = (n_rows + rpp - 1) / rpp;
-        const uint64_t n_units = row_groups * A.chunks;
-        if (n_units >= ((uint64_t)1 << 31)) return set_error(NK_ERR_UNSUPPORTED, "%s: too many work units", c.name);
-        A.n_units = (unsigned)n_units;
+        if (row_groups * A.chunks >= ((uint64_t)1 << 31)) return set_error(NK_ERR_UNSUPPORTED, "%s: too many work units", c.name);
+        A.row_groups = (unsigned)row_groups;
         A.chunk_div = FastDiv(A.chunks);
         for (int o = 0; o <= c.nsrc; o++) {
             A.base[o] = (int)cn.base[o];
@@ -253,7 +252,23 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             plan.passes = passes;
         }
         plan.vec = vec;
-        plan.grid = (unsigned)((n_units + passes - 1) / passes);     // one block per `passes` units, no grid-stride loop
+        // a source that is constant along the innermost outer axis is the same memory in every pass of a block
+        // when the block's rows never straddle that axis: the binary kernel then loads it once
+        plan.hoist = 0;
+        A.pass_rows = 0;
+        if (plan.kind == PLAN_ROWS_BINARY && last >= 1 && row_groups >= (uint64_t)passes) {
+            int constant = 0;
+            for (int j = 0; j < 2; j++) if (cn.stride[j + 1][last - 1] == 0) constant |= 1 << j;
+            if (constant) A.pass_rows = 1;
+            // measured at steady state: loading the constant source once gains 2..14 % when a row fills the block
+            // (256 threads) and loses 4..14 % when a block covers several rows per pass
+            if (constant && env_flag("NK_HOIST", true) && vec && passes == 8 && !A.nt_loads && rpp == 1 &&
+                cn.shape[last - 1] % ((int64_t)passes * rpp) == 0)
+                plan.hoist = constant;
+        }
+        // one block per `passes` units, no grid-stride loop
+        plan.grid = A.pass_rows ? (unsigned)(((row_groups + passes - 1) / passes) * A.chunks)
+                                : (unsigned)((row_groups * A.chunks + passes - 1) / passes);
         set_path(plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary")
                                                : vec ? "rows_vec" : "rows");
         done = true;
