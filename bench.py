@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
 # against a plain 1 GiB copy): profiles/rows_binary_kernel_broadcast_c2.md
-C2_TRAFFIC_BYTES = 4317140700
+C2_TRAFFIC_BYTES = 4316807974
 
 
 def event_time_ms(dev, launch, reps):
@@ -51,7 +51,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one MI355X: this build has no multi-GPU path (every kernel shards without "
-              "exchange; see DESIGN.md), run it with --gpus 1", file=sys.stderr)
+              "exchange), run it with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     from neureka_amd import Function, HipDevice, Tensor, _lib
