@@ -167,19 +167,79 @@ __device__ __forceinline__ f32x4u buffer_load4(BufRsrc r, unsigned lane_off, uns
 
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
-// forward: partial[z][y][x] = sum_{c in group z} sum_ky sum_kx in[c][y+ky][x+kx] * w[c][ky][kx]
-// block -> (256-column block, strip of R output rows, channel group); its four wavefronts take every fourth
-// channel of the group and are summed through LDS before the block writes its partial plane.
-template <typename T, int KH, int KW, int R>
-__global__ __launch_bounds__(256) void conv_chan_fwd(ChanArgs g, const T* __restrict__ in, const T* __restrict__ w, T* __restrict__ partial) {
-    __shared__ T red[4][R][64 * CX];
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int x = blockIdx.x * (64 * CX) + lane * CX;            // first of the lane's CX output columns
-    const int xl = x < g.OW ? x : 0;                             // lanes without a valid column read column 0
-    const bool whole = xl + CX <= g.W;                           // false only for the ragged last lane of a row
-    unsigned off[CX + KW - 1];                                   // byte offsets inside a row, clamped to the row
+// Rows are addressed through one buffer descriptor per row (base = first element of the row, extent = the row):
+// the hardware range check then returns 0 for every dword left or right of the row (negative lane offsets wrap to
+// huge unsigned ones) and, with an extent of 0, for a whole row that does not exist.  No clamp, no mask.
+__device__ __forceinline__ BufRsrc row_of(const float* base, int64_t row, int width, bool exists) {
+    return buffer_of(base + (exists ? row * width : 0), exists ? (unsigned)width * 4u : 0u);
+}
+
+// A lane holds CX adjacent columns; the KW - 1 further columns its window needs are the first (forward) or last
+// (gradients) registers of its neighbours.  They arrive through wavefront shifts of the registers instead of
+// through more loads: one 16-byte load per lane and row is all the memory traffic a window costs.  Only the
+// lane at the end (start) of the wavefront, which has no neighbour, loads its extra columns itself; the shift
+// leaves that lane's registers as they are.
+__device__ __forceinline__ float from_next_lane(float keep, float v) {     // lane i <- lane i + 1, lane 63 keeps `keep`
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, v), 0x130, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float from_prev_lane(float keep, float v) {     // lane i <- lane i - 1, lane 0 keeps `keep`
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, v), 0x138, 0xf, 0xf, false));
+}
+constexpr int WAVE_COLS = 64 * CX;          // columns per wavefront
+
+// window[0 .. CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[CX .. CX+EXTRA-1] with the
+// columns to the right of them
+template <int EXTRA>
+__device__ __forceinline__ void extend_right(float (&window)[CX + EXTRA], BufRsrc row, unsigned xoff, int lane) {
+    static_assert(EXTRA <= 2 * CX, "at most two further 16-byte pieces");
 #pragma unroll
-    for (int e = 0; e < CX + KW - 1; e++) off[e] = (unsigned)clampi(xl + e, 0, g.W - 1) * (unsigned)sizeof(T);
+    for (int e = CX; e < CX + EXTRA; e++) window[e] = 0.0f;
+    if (lane == 63) {
+        const f32x4u a = buffer_load4(row, xoff + 16u, 0);
+#pragma unroll
+        for (int e = 0; e < CX && e < EXTRA; e++) window[CX + e] = a[e];
+        if (EXTRA > CX) {
+            const f32x4u b = buffer_load4(row, xoff + 32u, 0);
+#pragma unroll
+            for (int e = CX; e < EXTRA; e++) window[CX + e] = b[e - CX];
+        }
+    }
+#pragma unroll
+    for (int e = CX; e < CX + EXTRA; e++) window[e] = from_next_lane(window[e], window[e - CX]);
+}
+
+// window[EXTRA .. EXTRA+CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[0 .. EXTRA-1] with
+// the columns x-EXTRA .. x-1 to the left of them (lane offsets below the row start read as zero)
+template <int EXTRA>
+__device__ __forceinline__ void extend_left(float (&window)[CX + EXTRA], BufRsrc row, unsigned xoff, int lane) {
+    static_assert(EXTRA <= 2 * CX, "at most two further 16-byte pieces");
+#pragma unroll
+    for (int i = 0; i < EXTRA; i++) window[i] = 0.0f;
+    if (lane == 0) {
+        const f32x4u a = buffer_load4(row, xoff - 16u, 0);                 // columns x-4 .. x-1
+#pragma unroll
+        for (int e = 0; e < CX; e++) if (EXTRA - CX + e >= 0) window[EXTRA - CX + e] = a[e];
+        if (EXTRA > CX) {
+            const f32x4u b = buffer_load4(row, xoff - 32u, 0);             // columns x-8 .. x-5
+#pragma unroll
+            for (int e = 0; e < CX; e++) if (EXTRA - 2 * CX + e >= 0) window[EXTRA - 2 * CX + e] = b[e];
+        }
+    }
+#pragma unroll
+    for (int i = EXTRA - 1; i >= 0; i--) window[i] = from_prev_lane(window[i], window[i + CX]);
+}
+
+// forward: partial[z][y][x] = sum_{c in group z} sum_ky sum_kx in[c][y+ky][x+kx] * w[c][ky][kx]
+// block -> (column block, strip of R output rows, channel group); its NW wavefronts take every NW-th channel of
+// the group and are summed through LDS in a fixed order before the block writes its (partial) plane.  With
+// NW = 16 and one group the block reduces all channels itself and no second pass is needed.
+template <typename T, int KH, int KW, int R, int NW>
+__global__ __launch_bounds__(NW * 64) void conv_chan_fwd(ChanArgs g, const T* __restrict__ in, const T* __restrict__ w, T* __restrict__ partial) {
+    constexpr int COLS = WAVE_COLS;
+    __shared__ T red[NW][R][64 * CX];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int x = blockIdx.x * COLS + lane * CX;                 // first of the lane's CX columns
+    const unsigned xoff = (unsigned)x * 4u;
     const int y0 = blockIdx.y * R;
     const int c0 = blockIdx.z * g.cg;
     int c1 = c0 + g.cg; if (c1 > g.C) c1 = g.C;
@@ -188,30 +248,24 @@ __global__ __launch_bounds__(256) void conv_chan_fwd(ChanArgs g, const T* __rest
     for (int r = 0; r < R; r++)
 #pragma unroll
         for (int j = 0; j < CX; j++) acc[r][j] = T(0);
-    for (int c = c0 + wave; c < c1; c += 4) {
+    for (int c = c0 + wave; c < c1; c += NW) {
         T wt[KH][KW];
         const T* wc = w + (int64_t)c * (KH * KW);
 #pragma unroll
         for (int ky = 0; ky < KH; ky++)
 #pragma unroll
             for (int kx = 0; kx < KW; kx++) wt[ky][kx] = wc[ky * KW + kx];
-        const BufRsrc plane = buffer_of(in + (int64_t)c * g.H * g.W, (unsigned)(g.H * g.W) * 4u);
+        const T* plane = in + (int64_t)c * g.H * g.W;
         T v[R + KH - 1][CX + KW - 1];
 #pragma unroll
         for (int yy = 0; yy < R + KH - 1; yy++) {                // all loads of the window first: one wait for the lot
-            const int y = y0 + yy < g.H ? y0 + yy : g.H - 1;      // rows past the end only feed outputs that are not stored
-            const unsigned row = (unsigned)(y * g.W) * 4u;
-            if (whole) {
-                const f32x4u head = buffer_load4(plane, off[0], row);
+            const f32x4u head = buffer_load4(row_of(plane, y0 + yy, g.W, y0 + yy < g.H), xoff, 0);
 #pragma unroll
-                for (int e = 0; e < CX; e++) v[yy][e] = head[e];
-            } else {
-#pragma unroll
-                for (int e = 0; e < CX; e++) v[yy][e] = buffer_load(plane, off[e], row);
-            }
-#pragma unroll
-            for (int e = CX; e < CX + KW - 1; e++) v[yy][e] = buffer_load(plane, off[e], row);
+            for (int e = 0; e < CX; e++) v[yy][e] = head[e];
         }
+#pragma unroll
+        for (int yy = 0; yy < R + KH - 1; yy++)
+            extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, g.W, y0 + yy < g.H), xoff, lane);
 #pragma unroll
         for (int yy = 0; yy < R + KH - 1; yy++)
 #pragma unroll
@@ -231,48 +285,45 @@ __global__ __launch_bounds__(256) void conv_chan_fwd(ChanArgs g, const T* __rest
         for (int j = 0; j < CX; j++) red[wave][r][lane * CX + j] = acc[r][j];
     __syncthreads();
     T* dst = partial + (int64_t)blockIdx.z * g.OH * g.OW;
-    for (int e = threadIdx.x; e < R * 64 * CX; e += 256) {
-        const int r = e / (64 * CX), col = e % (64 * CX);
-        const int yo = y0 + r, xo = blockIdx.x * (64 * CX) + col;
-        if (yo < g.OH && xo < g.OW)
-            dst[(int64_t)yo * g.OW + xo] = (red[0][r][col] + red[1][r][col]) + (red[2][r][col] + red[3][r][col]);
+    for (int e = threadIdx.x; e < R * COLS; e += NW * 64) {
+        const int r = e / COLS, col = e - r * COLS;
+        const int yo = y0 + r, xo = blockIdx.x * COLS + col;
+        if (yo < g.OH && xo < g.OW) {
+            T s = red[0][r][col];
+#pragma unroll
+            for (int k = 1; k < NW; k++) s = s + red[k][r][col];
+            dst[(int64_t)yo * g.OW + xo] = s;
+        }
     }
 }
 
 // gradient w.r.t. the big operand: dx[c][y][x] = sum_ky sum_kx w[c][ky][kx] * err[y-ky][x-kx] (zero outside err)
-// wave -> (256-column block over W, strip of R rows of dx, channel group); the err window of the strip is
-// loaded once and reused by every channel of the group
+// wave -> (column block over W, strip of R rows of dx, channel group); the err window of the strip is loaded once
+// (one 16-byte load per row) and reused by every channel of the group.  
 template <typename T, int KH, int KW, int R>
 __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restrict__ err, const T* __restrict__ w, T* __restrict__ dx) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int x = blockIdx.x * (64 * CX) + lane * CX;
+    const int x = blockIdx.x * WAVE_COLS + lane * CX;
     const int y0 = (blockIdx.y * 4 + wave) * R;
     if (y0 >= g.H) return;                                        // whole wavefronts leave together
     const int c0 = blockIdx.z * g.cg;
     int c1 = c0 + g.cg; if (c1 > g.C) c1 = g.C;
     // E[rr][i] = err[y0 - (KH-1) + rr][x - (KW-1) + i], zero outside err
-    unsigned eoff[CX + KW - 1];
-    bool col_ok[CX + KW - 1];
-#pragma unroll
-    for (int i = 0; i < CX + KW - 1; i++) {
-        const int ex = x - (KW - 1) + i;
-        col_ok[i] = ex >= 0 && ex < g.OW;
-        eoff[i] = (unsigned)clampi(ex, 0, g.OW - 1) * (unsigned)sizeof(T);
-    }
-    const BufRsrc ebuf = buffer_of(err, (unsigned)(g.OH * g.OW) * 4u);
     T E[R + KH - 1][CX + KW - 1];
 #pragma unroll
     for (int rr = 0; rr < R + KH - 1; rr++) {
         const int ey = y0 - (KH - 1) + rr;
-        const bool row_ok = ey >= 0 && ey < g.OH;
-        const unsigned row = (unsigned)(clampi(ey, 0, g.OH - 1) * g.OW) * 4u;
+        const f32x4u own = buffer_load4(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), (unsigned)x * 4u, 0);
 #pragma unroll
-        for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = buffer_load(ebuf, eoff[i], row);
-#pragma unroll
-        for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = row_ok && col_ok[i] ? E[rr][i] : T(0);
+        for (int j = 0; j < CX; j++) E[rr][KW - 1 + j] = own[j];
     }
+#pragma unroll
+    for (int rr = 0; rr < R + KH - 1; rr++) {
+        const int ey = y0 - (KH - 1) + rr;
+        extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), (unsigned)x * 4u, lane);
+    }
+    const bool stores = x < g.W;
     const bool vec_ok = x + CX <= g.W;
-    const unsigned xoff = (unsigned)(x < g.W ? x : 0) * (unsigned)sizeof(T);
     for (int c = c0; c < c1; c++) {
         const T* wc = w + (int64_t)c * (KH * KW);
         T wt[KH][KW];
@@ -292,8 +343,8 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
                 for (int kx = 0; kx < KW; kx++)
 #pragma unroll
                     for (int j = 0; j < CX; j++) acc[j] = fused_mad(E[r + KH - 1 - ky][j - kx + KW - 1], wt[ky][kx], acc[j]);
-            if (y0 + r < g.H) {
-                T* dst = (T*)((char*)(plane + (int64_t)(y0 + r) * g.W) + xoff);
+            if (stores && y0 + r < g.H) {
+                T* dst = plane + (int64_t)(y0 + r) * g.W + x;
                 if (vec_ok) {
                     f32x4u o; o[0] = acc[0]; o[1] = acc[1]; o[2] = acc[2]; o[3] = acc[3];
                     __builtin_nontemporal_store(o, (f32x4u*)dst);
@@ -308,73 +359,46 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
 
 // gradient w.r.t. the taps: dk[c][ky][kx] = sum_y sum_x in[c][y+ky][x+kx] * err[y][x]
 //   = sum over input elements (yy, xx) of in[c][yy][xx] * err[yy-ky][xx-kx]
-// wave -> (256-column block over W, strip of S input rows, channel).  The strip is worked off in chunks of R
-// rows: the chunk's R input rows (16-byte loads) and the R + KH - 1 err rows around them are all requested
-// before the first multiply-add, then every input element is multiplied into the KH*KW accumulators with
-// statically indexed registers.  Lanes are reduced with wavefront shuffles, strips by a second pass.
+// wave -> (column block over W, strip of S input rows, channel).  The strip is worked off in chunks of R
+// rows: the chunk's R input rows and the R + KH - 1 err rows around them are requested (one 16-byte load per
+// lane and row) before the first multiply-add, then every input element is multiplied into the KH*KW
+// accumulators with statically indexed registers.  Lanes are reduced with wavefront shuffles, strips by a second pass.
 template <typename T, int KH, int KW, int R>
 __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstrips, const T* __restrict__ in, const T* __restrict__ err, T* __restrict__ partial) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int strip = blockIdx.y * 4 + wave;
     if (strip >= nstrips) return;                                 // whole wavefronts leave together
-    const int xx = blockIdx.x * (64 * CX) + lane * CX;
-    const bool vec_ok = xx + CX <= g.W;
+    const int xx = blockIdx.x * WAVE_COLS + lane * CX;
+    const unsigned eoff = (unsigned)xx * 4u, voff = eoff;
     const int yy0 = strip * S;
     int yy1 = yy0 + S; if (yy1 > g.H) yy1 = g.H;
     const int c = blockIdx.z;
-    unsigned eoff[CX + KW - 1], voff[CX];
-    bool col_ok[CX + KW - 1], v_ok[CX];
-#pragma unroll
-    for (int i = 0; i < CX + KW - 1; i++) {
-        const int ex = xx - (KW - 1) + i;
-        col_ok[i] = ex >= 0 && ex < g.OW;
-        eoff[i] = (unsigned)clampi(ex, 0, g.OW - 1) * (unsigned)sizeof(T);
-    }
-#pragma unroll
-    for (int j = 0; j < CX; j++) {
-        v_ok[j] = xx + j < g.W;
-        voff[j] = (unsigned)clampi(xx + j, 0, g.W - 1) * (unsigned)sizeof(T);
-    }
     T acc[KH][KW];
 #pragma unroll
     for (int ky = 0; ky < KH; ky++)
 #pragma unroll
         for (int kx = 0; kx < KW; kx++) acc[ky][kx] = T(0);
-    const BufRsrc ebuf = buffer_of(err, (unsigned)(g.OH * g.OW) * 4u);
-    const BufRsrc plane = buffer_of(in + (int64_t)c * g.H * g.W, (unsigned)(g.H * g.W) * 4u);
+    const T* plane = in + (int64_t)c * g.H * g.W;
     for (int y = yy0; y < yy1; y += R) {
-        T E[R + KH - 1][CX + KW - 1];                             // E[rr] = err row y - (KH-1) + rr, zero outside err
+        T E[R + KH - 1][CX + KW - 1];                             // E[rr][i] = err[y - (KH-1) + rr][xx - (KW-1) + i], zero outside err
         T V[R][CX];                                               // V[r] = input row y + r, zero past the strip
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            const unsigned row = (unsigned)((y + r < g.H ? y + r : g.H - 1) * g.W) * 4u;
-            if (vec_ok) {
-                const f32x4u q = buffer_load4(plane, voff[0], row);
+            const f32x4u q = buffer_load4(row_of(plane, y + r, g.W, y + r < yy1), voff, 0);
 #pragma unroll
-                for (int j = 0; j < CX; j++) V[r][j] = q[j];
-            } else {
-#pragma unroll
-                for (int j = 0; j < CX; j++) V[r][j] = buffer_load(plane, voff[j], row);
-            }
-        }
-#pragma unroll
-        for (int rr = 0; rr < R + KH - 1; rr++) {
-            const unsigned row = (unsigned)(clampi(y - (KH - 1) + rr, 0, g.OH - 1) * g.OW) * 4u;
-#pragma unroll
-            for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = buffer_load(ebuf, eoff[i], row);
-        }
-#pragma unroll
-        for (int r = 0; r < R; r++) {
-            const bool row_live = y + r < yy1;
-#pragma unroll
-            for (int j = 0; j < CX; j++) V[r][j] = row_live && v_ok[j] ? V[r][j] : T(0);
+            for (int j = 0; j < CX; j++) V[r][j] = q[j];
         }
 #pragma unroll
         for (int rr = 0; rr < R + KH - 1; rr++) {
             const int ey = y - (KH - 1) + rr;
-            const bool row_ok = ey >= 0 && ey < g.OH;
+            const f32x4u own = buffer_load4(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), eoff, 0);
 #pragma unroll
-            for (int i = 0; i < CX + KW - 1; i++) E[rr][i] = row_ok && col_ok[i] ? E[rr][i] : T(0);
+            for (int j = 0; j < CX; j++) E[rr][KW - 1 + j] = own[j];
+        }
+#pragma unroll
+        for (int rr = 0; rr < R + KH - 1; rr++) {
+            const int ey = y - (KH - 1) + rr;
+            extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), eoff, lane);
         }
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -458,24 +482,40 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
         const Cfg& small = a_big ? c2 : c1;
         const T* bigp = a_big ? s1 : s2;
         const T* smallp = a_big ? s2 : s1;
-        constexpr int R = 8;
         ChanArgs g{};
         g.C = big.shape[0]; g.H = big.shape[1]; g.W = big.shape[2];
         g.OH = g.H - small.shape[1] + 1; g.OW = g.W - small.shape[2] + 1;
-        g.col_blocks = (g.OW + 64 * CX - 1) / (64 * CX);
-        const int strips = (g.OH + R - 1) / R;
-        // a block's four wavefronts take one channel each: groups are multiples of 4 channels
-        g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips * 4, want_waves);
-        g.cg = (g.cg + 3) / 4 * 4;
-        const int groups = (g.C + g.cg - 1) / g.cg;
+        const int cus = dev->props.multiProcessorCount;
         int rc = NK_OK;
         const bool ok = for_taps(small.shape[1], small.shape[2], [&](auto K) {
             constexpr int KK = decltype(K)::value;
+            g.col_blocks = (g.OW + WAVE_COLS - 1) / WAVE_COLS;
+            // Preferred: one block of 16 wavefronts reduces all channels of its (column block, R rows) itself -- no
+            // second pass -- when the plane is large enough to give every compute unit such a block (with short strips the
+            // window rows a block loads twice outweigh the saved pass: measured on [64,256,256]).
+            int tall_r = 0;
+            if (g.C >= 16)
+                for (int r : {8, 4})
+                    if ((int64_t)g.col_blocks * ((g.OH + r - 1) / r) >= cus) { tall_r = r; break; }
+            if (tall_r) {
+                g.cg = g.C;
+                dim3 grid(g.col_blocks, (g.OH + tall_r - 1) / tall_r, 1);
+                if (tall_r == 8) hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 8, 16>), grid, dim3(1024), 0, dev->stream, g, bigp, smallp, out);
+                else             hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 4, 16>), grid, dim3(1024), 0, dev->stream, g, bigp, smallp, out);
+                return;
+            }
+            // Small planes: parallelism has to come from the channels.  Blocks of four wavefronts take groups of
+            // channels (multiples of 4), a second pass adds the partial planes in a fixed order.
+            constexpr int R = 8;
+            const int strips = (g.OH + R - 1) / R;
+            g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips * 4, want_waves);
+            g.cg = (g.cg + 3) / 4 * 4;
+            const int groups = (g.C + g.cg - 1) / g.cg;
             void* ws = nullptr;
             const int on = g.OH * g.OW;
             if ((rc = workspace(dev, (uint64_t)groups * on * sizeof(T), &ws))) return;
             dim3 grid(g.col_blocks, strips, groups);
-            hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, bigp, smallp, groups == 1 ? out : (T*)ws);
+            hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, R, 4>), grid, dim3(256), 0, dev->stream, g, bigp, smallp, groups == 1 ? out : (T*)ws);
             if (groups > 1)
                 hipLaunchKernelGGL(conv_partial_reduce<T>, dim3((on + 255) / 256), dim3(256), 0, dev->stream, groups, on, (const T*)ws, out);
         });
@@ -494,13 +534,13 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
             constexpr int R = 4;
             ChanArgs g{};
             g.C = c0.shape[0]; g.H = c0.shape[1]; g.W = c0.shape[2]; g.OH = OH; g.OW = OW;
-            g.col_blocks = (g.W + 64 * CX - 1) / (64 * CX);
             const int strips = (g.H + R - 1) / R;
-            g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips, want_waves);
-            if (g.cg < 2 && g.C >= 2) g.cg = 2;              // amortise the err window over at least two channels
-            const int groups = (g.C + g.cg - 1) / g.cg;
             const bool ok = for_taps(c1.shape[1], c1.shape[2], [&](auto K) {
                 constexpr int KK = decltype(K)::value;
+                g.col_blocks = (g.W + WAVE_COLS - 1) / WAVE_COLS;
+                g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips, want_waves);
+                if (g.cg < 2 && g.C >= 2) g.cg = 2;          // amortise the err window over at least two channels
+                const int groups = (g.C + g.cg - 1) / g.cg;
                 dim3 grid(g.col_blocks, (strips + 3) / 4, groups);
                 hipLaunchKernelGGL((conv_chan_dx<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, s2, s1, out);
             });
@@ -514,19 +554,19 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
         if (c1.shape[1] == OH + c0.shape[1] - 1 && c1.shape[2] == OW + c0.shape[2] - 1 && c0.shape[1] < c1.shape[1] && c0.shape[2] < c1.shape[2]) {
             ChanArgs g{};
             g.C = c0.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2]; g.OH = OH; g.OW = OW;
-            g.col_blocks = (g.W + 64 * CX - 1) / (64 * CX);
             g.cg = 1;
-            // rows per strip: enough strips for the machine, a whole number of R-row chunks each
             constexpr int R = 8;
-            int64_t strips = (want_waves + (int64_t)g.col_blocks * g.C - 1) / ((int64_t)g.col_blocks * g.C);
-            if (strips < 1) strips = 1;
-            int S = (int)((g.H + strips - 1) / strips);
-            S = (S + R - 1) / R * R;
-            const int nstrips = (g.H + S - 1) / S;
-            const int parts = nstrips * g.col_blocks;
             int rc = NK_OK;
             const bool ok = for_taps(c0.shape[1], c0.shape[2], [&](auto K) {
                 constexpr int KK = decltype(K)::value;
+                g.col_blocks = (g.W + WAVE_COLS - 1) / WAVE_COLS;
+                // rows per strip: enough strips for the machine, a whole number of R-row chunks each
+                int64_t strips = (want_waves + (int64_t)g.col_blocks * g.C - 1) / ((int64_t)g.col_blocks * g.C);
+                if (strips < 1) strips = 1;
+                int S = (int)((g.H + strips - 1) / strips);
+                S = (S + R - 1) / R * R;
+                const int nstrips = (g.H + S - 1) / S;
+                const int parts = nstrips * g.col_blocks;
                 const int on = g.C * KK * KK;
                 void* ws = nullptr;
                 if ((rc = workspace(dev, (uint64_t)parts * on * sizeof(T), &ws))) return;
