@@ -465,10 +465,12 @@ def _abs_bound(orc, xs, ks, x, k, dt):
 
 @pytest.mark.parametrize("shape", [([8, 40, 70], [8, 5, 5]), ([6, 33, 65], [6, 3, 3]), ([5, 20, 21], [5, 4, 2]), ([64, 64, 64], [64, 5, 5]),
                                    ([3, 130, 200], [3, 7, 7]), ([9, 17, 300], [9, 2, 2]), ([2, 12, 12], [2, 4, 4]),
-                                   ([3, 10, 71], [3, 3, 3]), ([5, 9, 302], [5, 2, 2]), ([70, 30, 261], [70, 5, 5])])
+                                   ([3, 10, 71], [3, 3, 3]), ([5, 9, 302], [5, 2, 2]), ([70, 30, 261], [70, 5, 5]),
+                                   ([16, 520, 1030], [16, 3, 3]), ([16, 300, 1100], [16, 7, 7])])
 def test_channel_convolution_fast_paths(device, orc, shape):
-    """[C,H,W] x [C,kh,kw] forward and both gradients on the LDS-tiled kernels: re-ordered f32 sums, compared
-    norm-wise: |delta| <= 1e-5 * sum|a||b| per output."""
+    """[C,H,W] x [C,kh,kw] forward and both gradients on the register-window kernels: re-ordered f32 sums, compared
+    norm-wise: |delta| <= 1e-5 * sum|a||b| per output.  Covers ragged widths, several column blocks per row, taps
+    that reach two lanes to the side, and planes large enough for the 16-wavefront forward blocks."""
     xs, ks = shape
     ys = [1, xs[1] - ks[1] + 1, xs[2] - ks[2] + 1]
     rng = np.random.default_rng(43)
