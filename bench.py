@@ -38,6 +38,16 @@ def event_time_ms(dev, launch, reps):
     return dev.elapsed_ms(e0, e1) / reps
 
 
+def event_times_ms(dev, launch, reps):
+    """Durations of `reps` single launches, each bracketed by its own pair of HIP events on the device stream."""
+    events = [dev.event() for _ in range(reps + 1)]
+    dev.record(events[0])
+    for i in range(reps):
+        launch()
+        dev.record(events[i + 1])
+    return [dev.elapsed_ms(events[i], events[i + 1]) for i in range(reps)]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -97,10 +107,13 @@ def main():
     k_mul = event_time_ms(dev, launch_mul, args.steps)
     k_ms = 0.5 * (k_add + k_mul)
     achieved = bytes_per_launch / (k_ms * 1e-3) / 1e9
+    singles = sorted(event_times_ms(dev, launch_add, 50) + event_times_ms(dev, launch_mul, 50))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_TRAFFIC_BYTES if path == "rows_vec_binary" else None,
                 "kernel": f"nk::rows_binary_kernel<float, 4, 8> ({path})",
-                "launch_ms": round(k_ms, 4), "algorithmic_bytes": bytes_per_launch}
+                "launch_ms": round(k_ms, 4), "algorithmic_bytes": bytes_per_launch,
+                "single_launch_ms": {"p10": round(singles[len(singles) // 10], 4), "median": round(singles[len(singles) // 2], 4),
+                                     "p90": round(singles[(len(singles) * 9) // 10], 4), "launches": len(singles)}}
 
     # spot check of the timed output against numpy (the full parity tests live in tests/)
     got = dev._read(out._data, 5 * 2048 * 512 + 7 * 512, 512)
@@ -135,16 +148,21 @@ def main():
     # ---- the other configurations: kernel figures only ------------------------------------------------------
     others = {}
     if not args.no_others:
-        reps = max(5, args.steps)
+        reps = max(50, args.steps)                             # after 10 warm-up launches each
+
+        def warm(launch):
+            for _ in range(10):
+                launch()
+            dev.sync()
 
         def hbm(name, nbytes, launch):
-            launch(); dev.sync()
+            warm(launch)
             ms = event_time_ms(dev, launch, reps)
             gbs = nbytes / (ms * 1e-3) / 1e9
             others[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "path": _lib.last_path()}
 
         def flops(name, nflop, nbytes, launch):
-            launch(); dev.sync()
+            warm(launch)
             ms = event_time_ms(dev, launch, reps)
             tf = nflop / (ms * 1e-3) / 1e12
             others[name] = {"ms": round(ms, 4), "GFLOP/s": round(tf * 1e3, 1), "frac_fp32": round(tf / FP32_PEAK_TFLOPS, 4),
