@@ -194,6 +194,13 @@ def main():
         hbm("activation_sig", 8 * n, dev.prepared_launch("activation", "sig", -1, o, srcs[0]))
         hbm("elementwise_add", 12 * n, dev.prepared_launch("elementwise", "add", -1, o, srcs[0], srcs[1]))
         hbm("elementwise_mul", 12 * n, dev.prepared_launch("elementwise", "multiply", -1, o, srcs[0], srcs[1]))
+        # whole-tensor reductions of the same 2^26 elements (the operations that follow the hot path in training loops)
+        one = Tensor._on_device(dev, f32, (1,))
+        slot = dev.allocate(np.int32, 1)
+        hbm("sum_2^26", 4 * n, dev.prepared("nk_sum", dev.handle, 0, srcs[0]._data.ptr, n, one._data.ptr))
+        hbm("max_index_2^26", 4 * n, dev.prepared("nk_reduce_index", dev.handle, 1, 0, srcs[0]._data.ptr, n, slot.ptr))
+        hbm("dot_2^26", 8 * n, dev.prepared("nk_dot", dev.handle, 0, srcs[0]._data.ptr, srcs[1]._data.ptr, n, one._data.ptr))
+        dev.free(one); slot.release()
         # permuted [4096,16384] views of row-major [16384,4096]
         from neureka_amd import NDConfiguration
         pv = []

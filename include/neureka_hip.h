@@ -147,6 +147,24 @@ int nk_convolution(nk_dev dev, int d, int dtype, int rank,
                    nk_buf drn, const int32_t* drn_cfg, nk_buf a, const int32_t* a_cfg,
                    nk_buf b, const int32_t* b_cfg, int64_t n);
 
+/* fast_local_mem_based_sum / fast_private_sum_reduction: J/backend/main/operations/linear/internal/opencl/CLSum.java:24-62.
+ * out[0] = sum of the n elements of the dense buffer `in` (16-byte aligned), reduced in the CPU device's tree --
+ * tiles of 128 front to back, recursively (J/backend/main/operations/other/internal/CPUSum.java:26-74) -- so the
+ * result is bit-identical to the CPU device's. */
+int nk_sum(nk_dev dev, int dtype, nk_buf in, int64_t n, nk_buf out);
+
+/* CLReduce (min / max): J/backend/main/operations/linear/internal/opencl/CLReduce.java, registered in
+ * J/backend/main/operations/other/Min.java:72-73 and Max.java:72-73.  Writes to out_index[0] (int32) the index of
+ * the minimum or maximum of the n elements of `in`, found as the CPU device finds it: tiles of 64, strict
+ * comparison, first winner stays (J/backend/main/operations/other/internal/CPUReduce.java:90-157). */
+enum { NK_REDUCE_MIN = 0, NK_REDUCE_MAX = 1 };
+int nk_reduce_index(nk_dev dev, int kind, int dtype, nk_buf in, int64_t n, nk_buf out_index);
+
+/* multiply_arrays_for_dot_product + CLSum: J/backend/main/implementations/linear/CLDot.java:20-56.
+ * out[0] = sum of a[i] * b[i]: rounded products, summed in the tree of nk_sum (the CPU device's
+ * DOT.unrolled04 keeps four serial running sums; results agree within the reduction tolerance). */
+int nk_dot(nk_dev dev, int dtype, nk_buf a, nk_buf b, int64_t n, nk_buf out);
+
 /* simple_matMul / fast_CM_MM_*: J/backend/main/implementations/matmul/CLMatMul.java:11-53,
  * J/backend/main/operations/linear/internal/opencl/CLGEMM.java:11-100.
  * C[M,N] += A[M,K] @ B[K,N] on dense matrices of one layout; C is accumulated into, as the reference

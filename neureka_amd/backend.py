@@ -237,6 +237,58 @@ class MatMulAlgorithm(Algorithm):
         return call.withInputs(inputs)
 
 
+def _dense(t):
+    """The reductions read a tensor's buffer front to back: views and virtual tensors are materialised first."""
+    if t.isVirtual():
+        t.setIsVirtual(False)
+    if not t.ndc.isSimple() or t.isPartialSlice() or t.ndc.getLayout() is Layout.COLUMN_MAJOR:
+        t = t.deepCopy()
+    return t
+
+
+class SumAlgorithm(Algorithm):
+    """algorithms/SumAlgorithm.java:10-52."""
+    name = "sum_algorithm"
+
+    def isSuitableFor(self, call):
+        return GOOD
+
+    def prepare(self, call):
+        return call.withInputs([_dense(call.input(0))])
+
+
+class ReduceAlgorithm(Algorithm):
+    """The min_algorithm / max_algorithm of operations/other/Min.java:33-74 and Max.java."""
+    name = "reduce_algorithm"
+
+    def isSuitableFor(self, call):
+        return GOOD
+
+    def prepare(self, call):
+        return call.withInputs([_dense(call.input(0))])
+
+
+class DotProductAlgorithm(Algorithm):
+    """algorithms/DotProductAlgorithm.java:23-117: vectors only (after trimming extent-1 axes), dense copies."""
+    name = "dot_algorithm"
+
+    def isSuitableFor(self, call):
+        return GOOD if all(sum(1 for d in t.shape if d > 1) <= 1 for t in call.inputs if t is not None) else UNSUITABLE
+
+    def prepare(self, call):
+        from .ndim import NDConfiguration
+        from .tensor import Tensor
+        ins = []
+        for t in call.inputs:
+            t = _dense(t)
+            if t.rank > 1:               # dimTrim: the same buffer seen as a vector
+                v = Tensor(t.dtype, NDConfiguration.ofShape((t.ndc.size,)), None)
+                v._set_data(t._data, call.device)
+                t = v
+            ins.append(t)
+        return call.withInputs(ins)
+
+
 class Operation:
     """An operation with its algorithms (backend/api/Operation.java; template/operations/AbstractOperation.java:178-211)."""
 
@@ -273,8 +325,8 @@ def execute_device_algorithm(call: ExecutionCall):
             f"No '{type(call.device).__name__}' implementation found for algorithm '{call.algorithm.name}' "
             f"of operation '{call.operation.identifier}'")
     call.device.approve(call)
-    impl(call)
-    return call.input(0)
+    result = impl(call)
+    return call.input(0) if result is None else result
 
 
 def execute_on_common_device(call: ExecutionCall, run: Callable[[ExecutionCall], object]):
@@ -302,6 +354,10 @@ class BackendContext:
         for op_id, sym in [("mul_conv", "x"), ("inv_convolve_mul_left", "«x"), ("inv_convolve_mul_right", "x»")]:
             self.operations[op_id] = Operation(op_id, sym, [NDConvolution()])
         self.operations["matMul"] = Operation("matMul", "@", [MatMulAlgorithm()])
+        self.operations["sumItems"] = Operation("sumItems", "sumItems", [SumAlgorithm()])
+        self.operations["min"] = Operation("min", "min", [ReduceAlgorithm()])
+        self.operations["max"] = Operation("max", "max", [ReduceAlgorithm()])
+        self.operations["dot"] = Operation("dot", "dot", [DotProductAlgorithm()])
         for f in ACTIVATIONS:
             self.operations[f] = Operation(f, f, [ElementwiseAlgorithm()])
         self.extensions: List[object] = []
@@ -402,6 +458,41 @@ def hip_matmul(call: ExecutionCall):
     return c
 
 
+def hip_sum(call: ExecutionCall):
+    """CLSum (operations/linear/internal/opencl/CLSum.java:12-62)."""
+    from .tensor import Tensor
+    src = call.input(0)
+    out = Tensor._on_device(call.device, src.dtype, (1,))
+    call.device.launch_sum(src, out)
+    return out
+
+
+def hip_reduce(kind: str):
+    """CLReduce + the execution of operations/other/Min.java:43-52: the kernel finds the index, the item is read
+    back and wrapped into a tensor of one element that remembers the index for the backward pass."""
+    def run(call: ExecutionCall):
+        from .tensor import Tensor
+        src = call.input(0)
+        i = call.device.reduce_index(kind, src)
+        out = Tensor.of(src.dtype, (1,), src.item(i)).to(call.device)
+        out._found_index = i
+        return out
+    return run
+
+
+def hip_dot(call: ExecutionCall):
+    """CLDot (implementations/linear/CLDot.java:17-56)."""
+    from .tensor import Tensor
+    a, b = call.input(0), call.input(1)
+    if a.rank != 1 or b.rank != 1:
+        raise IllegalArgumentException("Input tensors must be vectors.")
+    if a.shape[0] != b.shape[0]:
+        raise IllegalArgumentException("Input vectors must have the same length.")
+    out = Tensor._on_device(call.device, a.dtype, (1,))
+    call.device.launch_dot(a, b, out)
+    return out
+
+
 class HipBackend:
     """``BackendExtension`` for HipDevice (model: backend/ocl/CLBackend.java:56-325)."""
 
@@ -429,6 +520,10 @@ class HipBackend:
         for op in ("mul_conv", "inv_convolve_mul_left", "inv_convolve_mul_right"):
             registry.forOperation(op).set(NDConvolution, hip_convolution)
         registry.forOperation("matMul").set(MatMulAlgorithm, hip_matmul)
+        registry.forOperation("sumItems").set(SumAlgorithm, hip_sum)
+        registry.forOperation("min").set(ReduceAlgorithm, hip_reduce("min"))
+        registry.forOperation("max").set(ReduceAlgorithm, hip_reduce("max"))
+        registry.forOperation("dot").set(DotProductAlgorithm, hip_dot)
         for f in ACTIVATIONS:
             registry.forOperation(f).set(ElementwiseAlgorithm, hip_elementwise_function(f))
 

@@ -1,0 +1,192 @@
+// nk_sum, nk_reduce_index, nk_dot: whole-tensor reductions of a dense buffer.
+//
+// The reference's CPU device reduces in a fixed tree: tiles of RTS consecutive elements are reduced front to
+// back, the tile results are reduced the same way, until one value is left (CPUSum: RTS = 128, the value starts
+// at 0; CPUReduce: RTS = 64, strict comparison, the first winner keeps its place and its index into the
+// original data is the result).  J/backend/main/operations/other/internal/CPUSum.java:26-74, CPUReduce.java:90-157.
+// The kernels here keep exactly that tree, so sums are bit-identical to the CPU device and min/max return the
+// same index, ties and NaNs included.
+//
+// One level of the tree: a wavefront owns 64 consecutive tiles, i.e. one contiguous piece of memory.  It moves
+// the piece through LDS 32 columns at a time -- 16-byte buffer loads that run along memory, rows of 33
+// elements in LDS -- and lane t then walks front to back through the 32 values of tile t (conflict-free).  The
+// loads of the next 32 columns are in flight while the current ones are reduced.  Elements past the end of the
+// data read as zero through the buffer range check and are skipped by the tile's own limit.
+#include "nk_internal.h"
+
+namespace nk {
+
+typedef __amdgpu_buffer_rsrc_t BufRsrc;
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+enum { STAT_SUM = 0, STAT_MIN = 1, STAT_MAX = 2, STAT_DOT = 3 };
+
+template <typename T, int RTS, int MODE>
+__global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ in, const T* __restrict__ in2,
+                                                          const int* __restrict__ idx_in, int64_t n,
+                                                          T* __restrict__ out, int* __restrict__ idx_out) {
+    constexpr int VEC = 16 / sizeof(T);             // elements per 16-byte load
+    constexpr int COLS = 32;                        // columns staged at a time
+    constexpr int NCH = RTS / COLS;
+    constexpr int LOADS = 64 * COLS / VEC / 64;     // 16-byte loads per lane and chunk
+    constexpr int PPR = COLS / VEC;                 // 16-byte pieces per tile row of a chunk
+    __shared__ T stage[4][64][COLS + 1];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int64_t tile0 = ((int64_t)blockIdx.x * 4 + wave) * 64;          // first tile of the wavefront
+    const int64_t elem0 = tile0 * RTS;
+    if (elem0 >= n) return;                                              // whole wavefronts leave together
+    const int64_t left = n - elem0;
+    const unsigned bytes = left * (int64_t)sizeof(T) > 0xffffffffll ? 0xffffffffu : (unsigned)(left * sizeof(T));
+    const BufRsrc r1 = __builtin_amdgcn_make_buffer_rsrc((void*)(in + elem0), 0, bytes, 0x00020000);
+    const BufRsrc r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == STAT_DOT ? in2 : in) + elem0), 0, bytes, 0x00020000);
+    T (*mine)[COLS + 1] = stage[wave];
+
+    // piece k of the lane inside a chunk: tile row and column of its 16 bytes
+    unsigned voff[LOADS];
+    int prow[LOADS], pcol[LOADS];
+#pragma unroll
+    for (int k = 0; k < LOADS; k++) {
+        const int p = lane + 64 * k;
+        prow[k] = p / PPR;
+        pcol[k] = (p % PPR) * VEC;
+        voff[k] = (unsigned)((prow[k] * RTS + pcol[k]) * sizeof(T));
+    }
+    u32x4 cur[LOADS], cur2[LOADS];
+    constexpr int NON_TEMPORAL = 2;                 // cache policy of the loads: every element is read exactly once
+    auto request = [&](int c) {
+#pragma unroll
+        for (int k = 0; k < LOADS; k++) {
+            cur[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r1, voff[k], (unsigned)(c * COLS * sizeof(T)), NON_TEMPORAL));
+            if (MODE == STAT_DOT)
+                cur2[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r2, voff[k], (unsigned)(c * COLS * sizeof(T)), NON_TEMPORAL));
+        }
+    };
+
+    // the lane's own tile
+    const int64_t my_first = elem0 + (int64_t)lane * RTS;
+    int limit = 0;
+    if (my_first < n) limit = n - my_first < RTS ? (int)(n - my_first) : RTS;
+    T value = T(0);
+    int found = 0;
+
+    request(0);
+#pragma unroll
+    for (int c = 0; c < NCH; c++) {
+#pragma unroll
+        for (int k = 0; k < LOADS; k++) {
+            typedef T Vec __attribute__((ext_vector_type(VEC)));
+            const Vec v = __builtin_bit_cast(Vec, cur[k]);
+            if (MODE == STAT_DOT) {
+                const Vec w = __builtin_bit_cast(Vec, cur2[k]);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) mine[prow[k]][pcol[k] + e] = v[e] * w[e];       // rounded product
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) mine[prow[k]][pcol[k] + e] = v[e];
+            }
+        }
+        if (c + 1 < NCH) request(c + 1);
+        __builtin_amdgcn_wave_barrier();            // LDS operations of a wavefront complete in order
+#pragma unroll
+        for (int i = 0; i < COLS; i++) {
+            const T x = mine[lane][i];
+            const int pos = c * COLS + i;
+            if (MODE == STAT_SUM || MODE == STAT_DOT) {
+                if (pos < limit) value = value + x;
+            } else {
+                const bool better = MODE == STAT_MIN ? x < value : x > value;
+                if (pos < limit && (pos == 0 || better)) { value = x; found = pos; }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (limit > 0) {
+        const int64_t tile = tile0 + lane;
+        out[tile] = value;
+        if (MODE == STAT_MIN || MODE == STAT_MAX) {
+            const int64_t at = my_first + found;                      // position in this level's input
+            idx_out[tile] = idx_in ? idx_in[at] : (int)at;            // ... mapped back to the original data
+        }
+    }
+}
+
+template <typename T, int RTS, int MODE>
+static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* out_value, int* out_index) {
+    constexpr bool indexed = MODE == STAT_MIN || MODE == STAT_MAX;
+    if (MODE == STAT_SUM && n == 1) {               // CPUSum returns a single element as it is (keeps a -0)
+        NK_HIP(hipMemcpyAsync(out_value, in, sizeof(T), hipMemcpyDeviceToDevice, dev->stream));
+        return NK_OK;
+    }
+    // partial results of all levels but the last live in the device workspace: values first, then indices
+    int64_t total = 0;
+    { int64_t m = n; do { m = (m + RTS - 1) / RTS; total += m; } while (m > 1); }
+    void* ws = nullptr;
+    if (int e = workspace(dev, (uint64_t)total * (sizeof(T) + sizeof(int)) + 64, &ws)) return e;
+    T* vals = (T*)ws;
+    int* idxs = (int*)((char*)ws + (((uint64_t)total * sizeof(T) + 15) & ~(uint64_t)15));
+    const T* cur = in;
+    const T* cur2 = in2;
+    const int* cur_idx = nullptr;
+    int64_t m = n, used = 0;
+    int level = 0;
+    do {
+        const int64_t tiles = (m + RTS - 1) / RTS;
+        const bool last = tiles == 1;
+        T* dst = last && out_value ? out_value : vals + used;
+        int* dst_idx = !indexed ? nullptr : (last && out_index ? out_index : idxs + used);
+        const unsigned blocks = (unsigned)((tiles + 255) / 256);
+        if (MODE == STAT_DOT && level > 0)
+            hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, STAT_SUM>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur, cur_idx, m, dst, dst_idx);
+        else
+            hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, MODE>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur2, cur_idx, m, dst, dst_idx);
+        cur = dst; cur2 = dst; cur_idx = dst_idx;
+        used += tiles;
+        m = tiles;
+        level++;
+    } while (m > 1);
+    NK_HIP(hipGetLastError());
+    return NK_OK;
+}
+
+static int check_vector(Device* dev, const char* what, int dtype, nk_buf buf, int64_t n) {
+    NK_REQUIRE(dtype == NK_F32 || dtype == NK_F64, "%s: unknown dtype %d", what, dtype);
+    NK_REQUIRE(n >= 1 && n < ((int64_t)1 << 31), "%s: n = %lld outside [1, 2^31)", what, (long long)n);
+    NK_REQUIRE(buf % 16 == 0, "%s: the data must start on a 16-byte boundary", what);
+    return check_range(dev, what, buf, 0, (uint64_t)n * dtype_bytes(dtype));
+}
+
+}  // namespace nk
+
+using namespace nk;
+
+extern "C" int nk_sum(nk_dev h, int dtype, nk_buf in, int64_t n, nk_buf out) {
+    NK_DEVICE(dev, h);
+    if (int e = check_vector(dev, "nk_sum(in)", dtype, in, n)) return e;
+    if (int e = check_range(dev, "nk_sum(out)", out, 0, dtype_bytes(dtype))) return e;
+    set_path("tile_tree_128");
+    return dtype == NK_F32 ? reduce_levels<float, 128, STAT_SUM>(dev, (const float*)in, nullptr, n, (float*)out, nullptr)
+                           : reduce_levels<double, 128, STAT_SUM>(dev, (const double*)in, nullptr, n, (double*)out, nullptr);
+}
+
+extern "C" int nk_reduce_index(nk_dev h, int kind, int dtype, nk_buf in, int64_t n, nk_buf out_index) {
+    NK_DEVICE(dev, h);
+    NK_REQUIRE(kind == NK_REDUCE_MIN || kind == NK_REDUCE_MAX, "nk_reduce_index: unknown kind %d", kind);
+    if (int e = check_vector(dev, "nk_reduce_index(in)", dtype, in, n)) return e;
+    if (int e = check_range(dev, "nk_reduce_index(out)", out_index, 0, sizeof(int))) return e;
+    set_path("tile_tree_64");
+    if (dtype == NK_F32)
+        return kind == NK_REDUCE_MIN ? reduce_levels<float, 64, STAT_MIN>(dev, (const float*)in, nullptr, n, nullptr, (int*)out_index)
+                                     : reduce_levels<float, 64, STAT_MAX>(dev, (const float*)in, nullptr, n, nullptr, (int*)out_index);
+    return kind == NK_REDUCE_MIN ? reduce_levels<double, 64, STAT_MIN>(dev, (const double*)in, nullptr, n, nullptr, (int*)out_index)
+                                 : reduce_levels<double, 64, STAT_MAX>(dev, (const double*)in, nullptr, n, nullptr, (int*)out_index);
+}
+
+extern "C" int nk_dot(nk_dev h, int dtype, nk_buf a, nk_buf b, int64_t n, nk_buf out) {
+    NK_DEVICE(dev, h);
+    if (int e = check_vector(dev, "nk_dot(a)", dtype, a, n)) return e;
+    if (int e = check_vector(dev, "nk_dot(b)", dtype, b, n)) return e;
+    if (int e = check_range(dev, "nk_dot(out)", out, 0, dtype_bytes(dtype))) return e;
+    set_path("tile_tree_128");
+    return dtype == NK_F32 ? reduce_levels<float, 128, STAT_DOT>(dev, (const float*)a, (const float*)b, n, (float*)out, nullptr)
+                           : reduce_levels<double, 128, STAT_DOT>(dev, (const double*)a, (const double*)b, n, (double*)out, nullptr);
+}

@@ -308,6 +308,25 @@ class HipDevice:
         _lib.check(self._lib.nk_matmul(self.handle, _dtype_code(c.dtype), _lib.ROW_MAJOR if row_major else _lib.COLUMN_MAJOR,
                                        M, K, N, a._data.ptr, b._data.ptr, c._data.ptr))
 
+    def launch_sum(self, src, out) -> None:
+        """CLSum.run (operations/linear/internal/opencl/CLSum.java:24-62): out[0] = sum of the dense tensor `src`."""
+        _lib.check(self._lib.nk_sum(self.handle, _dtype_code(src.dtype), src._data.ptr, src.ndc.size, out._data.ptr))
+
+    def launch_dot(self, a, b, out) -> None:
+        """CLDot (implementations/linear/CLDot.java:20-56)."""
+        _lib.check(self._lib.nk_dot(self.handle, _dtype_code(a.dtype), a._data.ptr, b._data.ptr, a.ndc.size, out._data.ptr))
+
+    def reduce_index(self, kind: str, src) -> int:
+        """CLReduce: index of the minimum / maximum of the dense tensor `src` (operations/other/Min.java:47-49 reads it
+        back with ``index.item(0)``)."""
+        slot = self.allocate(np.int32, 1)
+        try:
+            _lib.check(self._lib.nk_reduce_index(self.handle, {"min": 0, "max": 1}[kind], _dtype_code(src.dtype), src._data.ptr,
+                                                 src.ndc.size, slot.ptr))
+            return int(self._read(slot, 0, 1)[0])
+        finally:
+            slot.release()
+
     def launch_fused(self, program: Sequence[int], consts: Sequence[float], drn, srcs) -> None:
         ops = self._ops(drn, *srcs)
         prog = (C.c_int32 * len(program))(*program)

@@ -13,6 +13,8 @@
 from __future__ import annotations
 
 import re
+
+import numpy as np
 from typing import List, Optional, Sequence, Union
 
 from . import _lib
@@ -35,7 +37,7 @@ def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = Tr
     operation = ctx.getOperation(op_id)
     device = _device_for(inputs)
     parents = list(inputs)                   # the tensors the caller holds: gradients attach to these
-    if len(inputs) > 1 and len({t.rank for t in inputs}) > 1:
+    if len(inputs) > 1 and len({t.rank for t in inputs}) > 1 and op_id != "dot":
         inputs = make_fit(list(inputs))      # FunctionNode.execute pads ranks first (FunctionNode.java:92-93)
     call = ExecutionCall(device, operation, list(inputs), d)
     call.algorithm = operation.getAlgorithmFor(call)
@@ -61,11 +63,11 @@ def _graph_node(op_id: str, call: ExecutionCall, inputs: List[Tensor], result: T
         if not (parent.rqsGradient() or parent._node is not None):
             actions.append(None)
             continue
-        actions.append(_ad_action(op_id, alg, call, inputs, d))
+        actions.append(_ad_action(op_id, alg, call, inputs, d, result))
     return GraphNode(inputs, actions)
 
 
-def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: int):
+def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: int, result: Optional[Tensor] = None):
     device = call.device
     prepared_in = call.inputs[1:]            # operands as the kernel saw them (rank-fitted)
     if op_id == "mul_conv":
@@ -79,6 +81,22 @@ def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: in
             c.algorithm = c.operation.algorithms[0]
             return execute_on_common_device(c, lambda cc: execute_device_algorithm(cc))
         return act
+    if op_id == "sumItems":
+        # SumAlgorithm.java:27-31: the error of one element becomes a tensor of the summed shape filled with it
+        shape, dtype = inputs[0].shape, inputs[0].dtype
+        return lambda error: Tensor.of(dtype, shape, error.item(0)).to(device).setIsVirtual(False)
+    if op_id in ("min", "max"):
+        # Min.java:53-60: zeros like the input with the error at the index that was found
+        shape, dtype, found = inputs[0].shape, inputs[0].dtype, result._found_index
+        def act(error: Tensor) -> Tensor:
+            g = np.zeros(int(np.prod(shape)), dtype=dtype)
+            g[found] = error.item(0)
+            return Tensor.of(dtype, shape, g).to(device)
+        return act
+    if op_id == "dot":
+        # DotProductAlgorithm.java:40-47: error (one element) times a copy of the other operand
+        other = inputs[(1 + d) % 2]
+        return lambda error: execute("multiply", [error, other.deepCopy()], record=False)
     if op_id == "matMul":
         # MatMulAlgorithm.java:37-59: d' = (1 + d) % 2 picks the operand to transpose
         a, b = prepared_in
@@ -117,6 +135,9 @@ def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: in
             return execute("multiply", [error, local], record=False)
         return act
     raise IllegalStateException(f"no ADAction for operation '{op_id}'")
+
+
+REDUCTIONS = ("min", "max", "sumItems")       # functions of one argument that are not elementwise
 
 
 # ---- expression parsing ---------------------------------------------------------------------------
@@ -181,7 +202,7 @@ class _Parser:
         if kind == "sym" and val == "-":
             return Node("op", "multiply", [Node("const", -1.0), self.atom()])
         if kind == "name":
-            if val not in ACTIVATIONS: raise IllegalArgumentException(f"unknown function '{val}'")
+            if val not in ACTIVATIONS and val not in REDUCTIONS: raise IllegalArgumentException(f"unknown function '{val}'")
             if self.next() != ("sym", "("): raise IllegalArgumentException(f"'(' expected after {val}")
             arg = self.expr()
             if self.next() != ("sym", ")"): raise IllegalArgumentException("missing ')'")
@@ -257,6 +278,8 @@ class OptimizedFunction:
                 self.consts.append(n.value)
             self.program += [_lib.FUSE_CONST, self.consts.index(n.value)]
         elif n.kind == "fun":
+            if n.value not in _lib.FUN:
+                raise IllegalArgumentException(f"function '{n.value}' cannot be fused into an elementwise kernel")
             self._lower(n.children[0])
             self.program += [_lib.FUSE_FUN, _lib.FUN[n.value]]
         else:

@@ -240,6 +240,23 @@ class Tensor:
 
     __matmul__ = matMul
 
+    def sum(self) -> "Tensor":
+        """Tensor.sum(): the operation "sumItems" (operations/other/Sum.java)."""
+        from .function import execute
+        return execute("sumItems", [self])
+
+    def min(self) -> "Tensor":
+        from .function import execute
+        return execute("min", [self])
+
+    def max(self) -> "Tensor":
+        from .function import execute
+        return execute("max", [self])
+
+    def dot(self, b: "Tensor") -> "Tensor":
+        from .function import execute
+        return execute("dot", [self, b])
+
     def __getattr__(self, name):
         # activation shorthands: t.tanh(), t.sig(), t.relu() ...
         from .backend import ACTIVATIONS

@@ -56,6 +56,12 @@ def lib() -> C.CDLL:
                                        C.c_void_p, C.c_void_p, C.c_double, C.c_int, C.c_int, C.c_int]
         l.orc_gemm_threaded.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int]
         l.orc_gemm_partial.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int]
+        l.orc_sum_tree.restype = C.c_double
+        l.orc_sum_tree.argtypes = [C.c_int, C.c_void_p, C.c_int]
+        l.orc_reduce_index.restype = C.c_int
+        l.orc_reduce_index.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int]
+        l.orc_dot.restype = C.c_double
+        l.orc_dot.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int]
         l.orc_simple_conv2d.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = l
     return _lib
@@ -155,6 +161,21 @@ def simple_conv2d(image: np.ndarray, kernel: np.ndarray, width: int, height: int
     for bi in range(batch):
         lib().orc_simple_conv2d(_is64(image), _p(image), _p(kernel), _p(out), width, height, kw, kh, bi)
     return out
+
+
+def sum_tree(data: np.ndarray):
+    """CPUSum: tiles of 128 summed front to back, recursively; returns a scalar of the array's dtype."""
+    return data.dtype.type(lib().orc_sum_tree(_is64(data), _p(data), data.size))
+
+
+def reduce_index(kind: str, data: np.ndarray) -> int:
+    """CPUReduce: index of the minimum ('min') or maximum ('max') as the reference's tile recursion finds it."""
+    return lib().orc_reduce_index({"min": 0, "max": 1}[kind], _is64(data), _p(data), data.size)
+
+
+def dot(a: np.ndarray, b: np.ndarray):
+    """DOT.unrolled04 of two vectors."""
+    return a.dtype.type(lib().orc_dot(_is64(a), _p(a), _p(b), a.size))
 
 
 def gemm(row_major: bool, A: np.ndarray, B: np.ndarray, M: int, K: int, N: int, C_init=None, workers: int = 1) -> np.ndarray:

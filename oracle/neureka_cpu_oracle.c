@@ -601,6 +601,98 @@ void orc_simple_conv2d(int is_f64, const void* image, const void* kernel, void* 
         }
 }
 
+/* CPUSum._runRecursively, J/backend/main/operations/other/internal/CPUSum.java:26-74: tiles of RTS = 128 elements are
+ * summed front to back into a value that starts at 0; the partial sums are reduced the same way until one is left. */
+double orc_sum_tree(int is_f64, const void* data, int size) {
+    const int RTS = 128;
+    if (size == 1) return is_f64 ? ((const double*)data)[0] : (double)((const float*)data)[0];
+    int N = (size + RTS - 1) / RTS;
+    double result;
+    if (is_f64) {
+        double* out = (double*)malloc(sizeof(double) * (size_t)N);
+        for (int ni = 0; ni < N; ni++) {
+            int offset = ni * RTS, limit = offset + RTS < size ? offset + RTS : size;
+            double value = 0;
+            for (int i = offset; i < limit; ++i) value += ((const double*)data)[i];
+            out[ni] = value;
+        }
+        result = N > 1 ? orc_sum_tree(1, out, N) : out[0];
+        free(out);
+    } else {
+        float* out = (float*)malloc(sizeof(float) * (size_t)N);
+        for (int ni = 0; ni < N; ni++) {
+            int offset = ni * RTS, limit = offset + RTS < size ? offset + RTS : size;
+            float value = 0;
+            for (int i = offset; i < limit; ++i) value += ((const float*)data)[i];
+            out[ni] = value;
+        }
+        result = N > 1 ? orc_sum_tree(0, out, N) : (double)out[0];
+        free(out);
+    }
+    return result;
+}
+
+/* CPUReduce._runRecursively, J/backend/main/operations/other/internal/CPUReduce.java:90-157: per tile of RTS = 64
+ * the index of the first element that beats (strictly) everything before it; the winners are gathered and reduced
+ * the same way; the result is an index into the original data.  type 0 = MIN, 1 = MAX. */
+int orc_reduce_index(int type, int is_f64, const void* data, int size) {
+    const int RTS = 64;
+    int N = (size + RTS - 1) / RTS;
+    if (size == 1) return 0;
+    int* out = (int*)malloc(sizeof(int) * (size_t)N);
+    for (int ni = 0; ni < N; ni++) {
+        int offset = ni * RTS, limit = offset + RTS < size ? offset + RTS : size;
+        int found_index = offset;
+        if (is_f64) {
+            double value = ((const double*)data)[offset];
+            for (int i = offset + 1; i < limit; ++i) {
+                double current = ((const double*)data)[i];
+                if (type == 0 ? current < value : current > value) { value = current; found_index = i; }
+            }
+        } else {
+            float value = ((const float*)data)[offset];
+            for (int i = offset + 1; i < limit; ++i) {
+                float current = ((const float*)data)[i];
+                if (type == 0 ? current < value : current > value) { value = current; found_index = i; }
+            }
+        }
+        out[ni] = found_index;
+    }
+    int result = out[0];
+    if (N > 1) {
+        size_t es = is_f64 ? sizeof(double) : sizeof(float);
+        char* reduced = (char*)malloc(es * (size_t)N);
+        for (int i = 0; i < N; i++) memcpy(reduced + es * (size_t)i, (const char*)data + es * (size_t)out[i], es);
+        result = out[orc_reduce_index(type, is_f64, reduced, N)];
+        free(reduced);
+    }
+    free(out);
+    return result;
+}
+
+/* DOT.unrolled04, J/backend/main/operations/linear/internal/blas/DOT.java (float and double overloads): four running
+ * sums over every fourth element, the remainder into the first, added left to right; products are rounded. */
+double orc_dot(int is_f64, const void* a, const void* b, int size) {
+    int remainder = size % 4, i = 0;
+    if (is_f64) {
+        const double *x = (const double*)a, *y = (const double*)b;
+        double sum0 = 0, sum1 = 0, sum2 = 0, sum3 = 0;
+        for (int lim = size - remainder; i < lim; i += 4) {
+            sum0 += x[i] * y[i]; sum1 += x[i + 1] * y[i + 1]; sum2 += x[i + 2] * y[i + 2]; sum3 += x[i + 3] * y[i + 3];
+        }
+        for (; i < size; i++) sum0 += x[i] * y[i];
+        return sum0 + sum1 + sum2 + sum3;
+    } else {
+        const float *x = (const float*)a, *y = (const float*)b;
+        float sum0 = 0, sum1 = 0, sum2 = 0, sum3 = 0;
+        for (int lim = size - remainder; i < lim; i += 4) {
+            sum0 += x[i] * y[i]; sum1 += x[i + 1] * y[i + 1]; sum2 += x[i + 2] * y[i + 2]; sum3 += x[i + 3] * y[i + 3];
+        }
+        for (; i < size; i++) sum0 += x[i] * y[i];
+        return (double)(sum0 + sum1 + sum2 + sum3);
+    }
+}
+
 /* GEMM.partial_F32_MxN_RM / partial_F64_MxN_RM and the CM twins with AXPY inlined:
  * J/backend/main/operations/linear/internal/blas/GEMM.java:258-304, AXPY.java:32-59.
  * [first, limit) is a range of rows of A (row major) or of columns of B (column major). */

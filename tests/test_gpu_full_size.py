@@ -180,3 +180,22 @@ def test_config5_conv_forward_and_backward_full_size(device, orc):
     lhs = float(np.dot(e.reshape(-1).astype(np.float64), y.items.astype(np.float64)))
     assert abs(float(np.dot(gx.items.astype(np.float64), x.reshape(-1).astype(np.float64))) - lhs) <= 1e-4 * abs(lhs) + 1e-6
     assert abs(float(np.dot(gk.items.astype(np.float64), k.reshape(-1).astype(np.float64))) - lhs) <= 1e-4 * abs(lhs) + 1e-6
+
+
+def test_reductions_over_2_pow_26_elements(device, orc):
+    """sum, min/max index and dot product of the chain's operand size: the CPU device's trees, bit for bit."""
+    rng = np.random.default_rng(6)
+    n = 1 << 26
+    a = rng.standard_normal(n).astype(f32); b = rng.standard_normal(n).astype(f32)
+    ta, tb = on(device, a), on(device, b)
+    say("sum 2^26")
+    assert_bits(ta.sum().items, np.array([orc.sum_tree(a)], dtype=f32), "sum")
+    assert abs(float(ta.sum().items[0]) - float(a.sum(dtype=np.float64))) <= 1e-5 * float(np.abs(a).sum(dtype=np.float64))
+    say("min / max 2^26")
+    assert device.reduce_index("min", ta) == orc.reduce_index("min", a) == int(np.argmin(a))
+    assert device.reduce_index("max", ta) == orc.reduce_index("max", a) == int(np.argmax(a))
+    say("dot 2^26")
+    got = ta.dot(tb).items
+    assert_bits(got, np.array([orc.sum_tree(a * b)], dtype=f32), "dot as multiply + sum")
+    assert abs(float(got[0]) - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) <= 1e-5 * float(np.abs(a * b).sum(dtype=np.float64))
+    free(device, ta, tb)

@@ -584,3 +584,94 @@ def test_matmul_through_the_tensor_api(device):
     e = rng.integers(-3, 4, (6, 5)).astype(np.float64)
     c.backward(on(device, e))
     assert (ta.gradient.items.reshape(6, 9) == e @ b.T).all() and (tb.gradient.items.reshape(9, 5) == a.T @ e).all()
+
+
+# ---- whole-tensor reductions ------------------------------------------------------------------------------
+def test_stats_golden_on_device(device, golden):
+    """Tensor_Stats_Spec / Tensor_Dot_Product_Spec with the tensors on the device."""
+    from test_oracle_pinned import stats_function_input
+    g = golden["stats"]
+    for reduce_type, type_name, expected in g["min_max_function"]["rows"]:
+        dt = np.float32 if type_name == "Float" else np.float64
+        a = on(device, stats_function_input(reduce_type, type_name, dt), (19, 7))
+        r = Function.of(reduce_type.lower() + "(I[0])")(a)
+        assert r.shape == (1,) and r.items[0] == expected, (reduce_type, type_name)
+    a = on(device, np.array([((31 ** (i + 42)) % 301) - 151 for i in range(133)], dtype=np.float32), (19, 7))
+    assert a.min().item(0) == g["min_max_methods"]["min"] and a.max().item(0) == g["min_max_methods"]["max"]
+    s = on(device, np.array([((7 ** i) % 11) - 5 for i in range(13 * 73 * 11)], dtype=np.float32), (13, 73, 11)).sum()
+    assert s.shape == (1,) and s.item(0) == g["sum"]["expected"] and _lib.last_path() == "tile_tree_128"
+    for row in g["dot"]:
+        r = on(device, np.array(row["a"], dtype=np.float32)).dot(on(device, np.array(row["b"], dtype=np.float32)))
+        assert r.shape == (1,) and r.item(0) == row["expected"]
+
+
+def test_stats_autograd_golden(device, golden):
+    g = golden["stats"]
+    a = on(device, np.array(g["min_max_autograd"]["a"], dtype=np.float32)).setRqsGradient(True)
+    b = a * Tensor.of(np.float32, (1,), 3.0)
+    x = b.min() / Tensor.of(np.float32, (1,), 2.0)
+    y = b.max() / Tensor.of(np.float32, (1,), 4.0)
+    (x + y).backward()
+    assert a.gradient.items.tolist() == g["min_max_autograd"]["gradient"]
+    a = on(device, np.array(g["sum_autograd"]["a"], dtype=np.float32)).setRqsGradient(True)
+    (a * Tensor.of(np.float32, (1,), 3.0)).sum().backward()
+    assert a.gradient.items.tolist() == g["sum_autograd"]["gradient"]
+    d = g["dot_autograd"]
+    a = on(device, np.array(d["a"], dtype=np.float32))
+    w = on(device, np.array(d["w"], dtype=np.float32)).setRqsGradient(True)
+    r = a.dot(w)
+    assert r.items.tolist() == [d["result"]]
+    r.backward(Tensor.of(np.float32, (1,), d["backward_error"]))
+    assert w.gradient.shape == (3,) and w.gradient.items.tolist() == d["w_gradient"]
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_sum_is_bit_identical_to_the_cpu_tree(device, orc, dt):
+    rng = np.random.default_rng(61)
+    for n in (1, 2, 31, 127, 128, 129, 8191, 8192, 16385, 100003, (1 << 21) + 77):
+        say("sum", dt, n)
+        x = rng.standard_normal(n).astype(F[dt])
+        got = on(device, x).sum()
+        assert_bits(got.items, np.array([orc.sum_tree(x)], dtype=F[dt]), f"sum n={n}")
+    x = np.array([-0.0], dtype=F[dt])                              # a single element is returned as it is
+    assert np.signbit(on(device, x).sum().items[0])
+    # views are summed through a dense copy: a transposed slice
+    m = rng.standard_normal((40, 50)).astype(F[dt])
+    v = on(device, m)[3:33, 5:45].T()
+    assert_bits(v.sum().items, np.array([orc.sum_tree(np.ascontiguousarray(m[3:33, 5:45].T).reshape(-1))], dtype=F[dt]), "sum of a view")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_min_max_return_the_reference_index(device, orc, dt):
+    rng = np.random.default_rng(62)
+    for n in (1, 2, 63, 64, 65, 4095, 4096, 4097, 70001, (1 << 20) + 3):
+        say("min/max", dt, n)
+        x = rng.integers(-40, 40, n).astype(F[dt])                 # many ties: the first one must win
+        t = on(device, x)
+        for kind in ("min", "max"):
+            assert device.reduce_index(kind, t) == orc.reduce_index(kind, x), (kind, n)
+    x = rng.standard_normal(5000).astype(F[dt])
+    for at in (0, 64, 70, 4096, 4999):                              # NaNs: sticky only where they open a tile
+        y = x.copy(); y[at] = np.nan
+        t = on(device, y)
+        for kind in ("min", "max"):
+            assert device.reduce_index(kind, t) == orc.reduce_index(kind, y), (kind, at)
+    assert _lib.last_path() == "tile_tree_64"
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_dot_product(device, orc, dt):
+    rng = np.random.default_rng(63)
+    for n in (1, 5, 128, 129, 100003):
+        say("dot", dt, n)
+        a, b = rng.standard_normal(n).astype(F[dt]), rng.standard_normal(n).astype(F[dt])
+        got = on(device, a).dot(on(device, b)).items
+        # rounded products summed in the tree of CPUSum: bit for bit
+        assert_bits(got, np.array([orc.sum_tree(a * b)], dtype=F[dt]), f"dot as multiply + sum, n={n}")
+        # against the CPU device's DOT.unrolled04 (another summation order): norm-wise
+        want = orc.dot(a, b)
+        assert abs(float(got[0]) - float(want)) <= RTOL[np.dtype(F[dt])] * float(np.abs(a * b).sum()) + 1e-30
+        ai, bi = rng.integers(-9, 10, n).astype(F[dt]), rng.integers(-9, 10, n).astype(F[dt])
+        assert on(device, ai).dot(on(device, bi)).items[0] == orc.dot(ai, bi)       # exact on small integers
+    with pytest.raises(IllegalArgumentException):
+        on(device, np.ones(3, dtype=F[dt])).dot(on(device, np.ones(4, dtype=F[dt])))

@@ -338,3 +338,84 @@ def test_threaded_equals_sequential(orc):
     a = orc.activation("tanh", -1, np.zeros_like(x), cfg, x, cfg, workers=1)
     b = orc.activation("tanh", -1, np.zeros_like(x), cfg, x, cfg, workers=8)
     assert_bits(a, b)
+
+
+# ---- whole-tensor reductions: CPUSum, CPUReduce, DOT ------------------------------------------------------
+def _java_string_hash(s: str) -> int:
+    h = 0
+    for ch in s:
+        h = (31 * h + ord(ch)) & 0xFFFFFFFF
+    return h - (1 << 32) if h >= (1 << 31) else h
+
+
+def stats_function_input(reduce_type: str, type_name: str, dtype) -> np.ndarray:
+    """The tensor of Tensor_Stats_Spec.groovy:33-37: Groovy evaluates 31**(i+13) exactly (BigInteger)."""
+    seed = _java_string_hash(type_name) + _java_string_hash(reduce_type)
+    return np.array([((seed + 31 ** (i + 13)) % 301) - 151 for i in range(19 * 7)], dtype=dtype)
+
+
+def test_reduce_index_reproduces_the_stats_spec(golden, orc):
+    g = golden["stats"]
+    for reduce_type, type_name, expected in g["min_max_function"]["rows"]:
+        a = stats_function_input(reduce_type, type_name, np.float32 if type_name == "Float" else np.float64)
+        i = orc.reduce_index(reduce_type.lower(), a)
+        assert a[i] == expected
+        assert i == (np.argmin(a) if reduce_type == "MIN" else np.argmax(a))          # first occurrence
+    a = np.array([((31 ** (i + 42)) % 301) - 151 for i in range(133)], dtype=np.float32)
+    assert a[orc.reduce_index("min", a)] == g["min_max_methods"]["min"] and a[orc.reduce_index("max", a)] == g["min_max_methods"]["max"]
+
+
+def test_reduce_index_ties_and_tile_structure(orc):
+    """Strict comparison keeps the first of equal values, within a tile of 64 and across the recursion; a NaN
+    is only ever selected when it opens a tile (CPUReduce.java:117-127)."""
+    rng = np.random.default_rng(5)
+    for n in (1, 2, 63, 64, 65, 4095, 4096, 4097, 70001):
+        a = rng.integers(-50, 50, n).astype(np.float32)        # many ties
+        assert orc.reduce_index("min", a) == int(np.argmin(a)) and orc.reduce_index("max", a) == int(np.argmax(a))
+    a = np.arange(200, dtype=np.float64)
+    a[70] = np.nan                                             # inside a tile: never beats, never beaten -> ignored
+    assert orc.reduce_index("max", a) == 199 and orc.reduce_index("min", a) == 0
+    a = np.arange(200, dtype=np.float64)
+    a[64] = np.nan                                             # opens the second tile: that tile's value is NaN ...
+    assert orc.reduce_index("max", a) == 199                   # ... and loses to nothing, wins nothing, in the next level (it is not first there)
+    a[0] = np.nan                                              # opens the first tile of every level: sticks
+    assert orc.reduce_index("max", a) == 0 and orc.reduce_index("min", a) == 0
+
+
+def test_sum_tree_reproduces_the_stats_spec_and_its_own_definition(golden, orc):
+    g = golden["stats"]["sum"]
+    a = np.array([((7 ** i) % 11) - 5 for i in range(13 * 73 * 11)], dtype=np.float32)
+    assert orc.sum_tree(a) == g["expected"]
+    # the definition, restated with numpy: tiles of 128 front to back, recursively
+    def tree(x):
+        while x.size > 1:
+            pad = (-x.size) % 128
+            tiles = np.concatenate([x, np.zeros(pad, dtype=x.dtype)]).reshape(-1, 128)
+            acc = np.zeros(tiles.shape[0], dtype=x.dtype)
+            for j in range(128):
+                acc = acc + tiles[:, j]
+            x = acc
+        return x[0]
+    rng = np.random.default_rng(6)
+    for dt in (np.float32, np.float64):
+        for n in (2, 127, 128, 129, 16384, 16385, 100003):
+            x = rng.standard_normal(n).astype(dt)
+            got = orc.sum_tree(x)
+            assert got == tree(x), (dt, n)
+            assert abs(float(got) - math.fsum(x.tolist())) <= (1e-5 if dt == np.float32 else 1e-12) * float(np.abs(x).sum())
+
+
+def test_dot_reproduces_the_dot_product_spec(golden, orc):
+    for row in golden["stats"]["dot"]:
+        a, b = np.array(row["a"], dtype=np.float32), np.array(row["b"], dtype=np.float32)
+        assert orc.dot(a, b) == row["expected"]
+    rng = np.random.default_rng(7)
+    for n in (1, 3, 4, 5, 1001):
+        a, b = rng.integers(-9, 10, n).astype(np.float64), rng.integers(-9, 10, n).astype(np.float64)
+        assert orc.dot(a, b) == float(np.dot(a, b))           # exact on small integers, any order
+    a, b = rng.standard_normal(1001).astype(np.float32), rng.standard_normal(1001).astype(np.float32)
+    s = [np.float32(0)] * 4                                    # four running sums, remainder into the first
+    for i in range(1000):
+        s[i % 4] = s[i % 4] + a[i] * b[i]
+    s[0] = s[0] + a[1000] * b[1000]
+    assert orc.dot(a, b) == ((s[0] + s[1]) + s[2]) + s[3]
