@@ -175,6 +175,14 @@ def main():
         hbm("broadcast_add_f64", 8 * (o64.size + a64.size + b64.size), dev.prepared_launch("broadcast", "add", -1, o64, a64, b64))
         for t in (a64, b64, o64): dev.free(t)
 
+        # C2 backward: the reducing kernel, error [1024,2048,512] -> gradient [1024,1,512] (axis 1 summed) and [1,2048,512]
+        err = Tensor._on_device(dev, f32, (1024, 2048, 512))
+        for d, tgt, oth in ((0, (1024, 1, 512), (1, 2048, 512)), (1, (1, 2048, 512), (1024, 1, 512))):
+            g_t = Tensor._on_device(dev, f32, tgt); z_t = Tensor._on_device(dev, f32, oth)
+            hbm(f"broadcast_backward_grad{d}", 4 * (err.size + g_t.size + z_t.size), dev.prepared_launch("broadcast", "add", d, g_t, z_t, err))
+            dev.free(g_t); dev.free(z_t)
+        dev.free(err)
+
         # C3: tanh(sig(a)*b+c) on 2^26 elements: fused, and the reference's 4-kernel sequence
         n = 1 << 26
         srcs = [Tensor.of(f32, (n,), rng.standard_normal(n).astype(f32)).to(dev) for _ in range(3)]

@@ -2,10 +2,11 @@
 //
 // Backward (d >= 0), CPUBroadcast.java:207-259 (J/backend/main/implementations/broadcast/): the drain is
 // the smaller tensor; per drain element the kernel sums g(src1, src2) over the axes on which the drain
-// is smaller than src1, axis 0 fastest.  One thread per drain element with the sum in the reference's
+// is smaller than src1, axis 0 fastest.  Every drain element is summed by one thread in the reference's
 // order, so + and - results are bit-identical to the CPU device.
 #include "nk_internal.h"
 #include "nk_scalar.h"
+#include <type_traits>
 
 namespace nk {
 
@@ -28,47 +29,95 @@ __device__ __forceinline__ T bcast_derive(int op, int d, T a, T b) {
     return T(NAN);
 }
 
+// Physical offsets are linear in the nd-index (phys = sum (idx*spread + offset) * stride), so per launch the host
+// reduces the three descriptors to: a base offset and one effective stride per axis for each operand as it
+// follows the drain's index, plus the list of reduced axes (axis 0 first = fastest, the reference's order) with
+// their extents and strides in src1 and src2.  A thread owns V drain elements that are neighbours along the
+// last axis and walks the reduced axes with running offsets; the loads of UNROLL terms are requested together and
+// then added in order, so the sum keeps the reference's order while the memory system sees deep queues.
 struct BcastBwdArgs {
     int rank, op, d;
-    unsigned n;
-    Cfg c0, c1, c2;
+    unsigned n_threads;                  // drain elements / V
+    int nred;
+    Cfg c0;                              // the drain (flat index -> nd-index -> offset)
+    int64_t base1, base2;
+    int64_t keep1[NK_MAX_RANK], keep2[NK_MAX_RANK];       // stride of src1 / src2 along axis k as the drain's index moves (0: pinned)
+    int red_extent[NK_MAX_RANK];
+    int64_t red1[NK_MAX_RANK], red2[NK_MAX_RANK];
 };
 
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* __restrict__ drn,
                                                             const T* __restrict__ s1, const T* __restrict__ s2) {
-    const unsigned step = gridDim.x * blockDim.x;
-    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < A.n; i += step) {
-        int o[NK_MAX_RANK], i1[NK_MAX_RANK], i2[NK_MAX_RANK];
-        nd_of_flat(A.c0, A.rank, (int)i, o);
-        for (int k = 0; k < A.rank; k++) {
-            const int e0 = A.c0.shape[k], e1 = A.c1.shape[k], e2 = A.c2.shape[k];
-            if (e0 == e1) { i1[k] = o[k]; i2[k] = (e2 == 1) ? 0 : o[k]; }
-            else if (e0 > e1) { i1[k] = 0; i2[k] = o[k]; }
-            else { i1[k] = 0; i2[k] = 0; }     // reduced axis: walks 0 .. e1-1
+    constexpr int UNROLL = 8;
+    typedef typename std::conditional<V == 1, T, T __attribute__((ext_vector_type(V == 1 ? 2 : V), aligned(sizeof(T))))>::type Vec;
+    const unsigned t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= A.n_threads) return;
+    int o[NK_MAX_RANK];
+    nd_of_flat(A.c0, A.rank, (int)(t * V), o);
+    int64_t o1 = A.base1, o2 = A.base2;
+    for (int k = 0; k < A.rank; k++) { o1 += o[k] * A.keep1[k]; o2 += o[k] * A.keep2[k]; }
+    const int64_t last1 = A.keep1[A.rank - 1];       // V > 1: 1 (contiguous) or 0 (pinned); src2 is contiguous there
+    auto load1 = [&](int64_t at, T (&dst)[V]) {
+        if (V == 1) dst[0] = s1[at];
+        else if (last1 == 0) { const T x = s1[at]; for (int v = 0; v < V; v++) dst[v] = x; }
+        else { const Vec x = *(const Vec*)(s1 + at); for (int v = 0; v < V; v++) dst[v] = ((const T*)&x)[v]; }
+    };
+    auto load2 = [&](int64_t at, T (&dst)[V]) {
+        if (V == 1) dst[0] = s2[at];
+        else { const Vec x = __builtin_nontemporal_load((const Vec*)(s2 + at)); for (int v = 0; v < V; v++) dst[v] = ((const T*)&x)[v]; }
+    };
+    T value[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) value[v] = T(0);
+    int r[NK_MAX_RANK];
+    for (int k = 0; k < NK_MAX_RANK; k++) r[k] = 0;
+    const int n0 = A.nred > 0 ? A.red_extent[0] : 1;
+    const int64_t st1 = A.nred > 0 ? A.red1[0] : 0, st2 = A.nred > 0 ? A.red2[0] : 0;
+    for (;;) {
+        int j = 0;
+        for (; j + UNROLL <= n0; j += UNROLL) {
+            T a[UNROLL][V], b[UNROLL][V];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) { load1(o1 + (j + u) * st1, a[u]); load2(o2 + (j + u) * st2, b[u]); }
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                for (int v = 0; v < V; v++) value[v] = value[v] + bcast_derive<T>(A.op, A.d, a[u][v], b[u][v]);
         }
-        T value = T(0);
-        bool running = true;
-        while (running) {
-            value = value + bcast_derive<T>(A.op, A.d, s1[phys_of_nd(A.c1, A.rank, i1)], s2[phys_of_nd(A.c2, A.rank, i2)]);
-            // odometer over the reduced axes, axis 0 fastest
-            int k = 0;
-            for (; k < A.rank; k++) {
-                if (A.c0.shape[k] < A.c1.shape[k]) {
-                    i1[k]++; i2[k]++;
-                    if (i1[k] == A.c1.shape[k]) { i1[k] = 0; i2[k] = 0; }
-                    else break;
-                }
-            }
-            running = k < A.rank;
+        for (; j < n0; j++) {
+            T a[V], b[V];
+            load1(o1 + j * st1, a); load2(o2 + j * st2, b);
+#pragma unroll
+            for (int v = 0; v < V; v++) value[v] = value[v] + bcast_derive<T>(A.op, A.d, a[v], b[v]);
         }
-        drn[phys_of_nd(A.c0, A.rank, o)] = value;
+        // carry into the slower reduced axes
+        int k = 1;
+        for (; k < A.nred; k++) {
+            r[k]++; o1 += A.red1[k]; o2 += A.red2[k];
+            if (r[k] < A.red_extent[k]) break;
+            o1 -= (int64_t)A.red_extent[k] * A.red1[k]; o2 -= (int64_t)A.red_extent[k] * A.red2[k];
+            r[k] = 0;
+        }
+        if (k >= A.nred) break;
+    }
+    const int at = phys_of_nd(A.c0, A.rank, o);
+    if (V == 1) drn[at] = value[0];
+    else {
+        Vec out;
+        for (int v = 0; v < V; v++) ((T*)&out)[v] = value[v];
+        *(Vec*)(drn + at) = out;
     }
 }
 
 }  // namespace nk
 
 using namespace nk;
+
+static bool env_vec_ok() {
+    static const bool on = [] { const char* v = getenv("NK_BWD_VECTOR"); return !(v && v[0] == '0'); }();
+    return on;
+}
 
 extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_buf drn, const int32_t* drn_cfg,
                             nk_buf a, const int32_t* a_cfg, nk_buf b, const int32_t* b_cfg, int64_t n) {
@@ -97,15 +146,37 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
     if (int e = check_extent(dev, "nk_broadcast(src1)", a, a_cfg, rank, eb)) return e;
     if (int e = check_extent(dev, "nk_broadcast(src2)", b, b_cfg, rank, eb)) return e;
     BcastBwdArgs A{};
-    A.rank = rank; A.op = op_id; A.d = d; A.n = (unsigned)n;
-    load_cfg(A.c0, drn_cfg, rank); load_cfg(A.c1, a_cfg, rank); load_cfg(A.c2, b_cfg, rank);
-    unsigned blocks = (unsigned)((n + 255) / 256);
-    if (blocks > 65536) blocks = 65536;
-    set_path("broadcast_backward");
-    if (dtype == NK_F32)
-        hipLaunchKernelGGL(broadcast_bwd_kernel<float>, dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
-    else
-        hipLaunchKernelGGL(broadcast_bwd_kernel<double>, dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+    A.rank = rank; A.op = op_id; A.d = d;
+    Cfg c1, c2;
+    load_cfg(A.c0, drn_cfg, rank); load_cfg(c1, a_cfg, rank); load_cfg(c2, b_cfg, rank);
+    A.base1 = 0; A.base2 = 0; A.nred = 0;
+    for (int k = 0; k < rank; k++) {
+        const int e0 = A.c0.shape[k], e1 = c1.shape[k], e2 = c2.shape[k];
+        const int64_t f1 = (int64_t)c1.spread[k] * c1.strides[k], f2 = (int64_t)c2.spread[k] * c2.strides[k];
+        A.base1 += (int64_t)c1.offset[k] * c1.strides[k];
+        A.base2 += (int64_t)c2.offset[k] * c2.strides[k];
+        A.keep1[k] = 0; A.keep2[k] = 0;
+        if (e0 == e1) { A.keep1[k] = f1; A.keep2[k] = e2 == 1 ? 0 : f2; }    // both follow the drain (src2 pinned if it has extent 1)
+        else if (e0 > e1) { A.keep2[k] = f2; }                                // src1 pinned to 0
+        else { A.red_extent[A.nred] = e1; A.red1[A.nred] = f1; A.red2[A.nred] = f2; A.nred++; }   // reduced: both walk 0 .. e1-1
+    }
+    // four (two) drain neighbours per thread when they are neighbours in memory for the drain and src2 and
+    // neighbours or one value for src1, and the drain's flat index unravels row-major on the last axis
+    constexpr int VB = 16;
+    const int V = VB / eb, last = rank - 1;
+    const bool vec = A.c0.shape[last] % V == 0 && A.c0.imap[last] == 1 && (int64_t)A.c0.spread[last] * A.c0.strides[last] == 1 &&
+                     A.c0.shape[last] >= c1.shape[last] && A.keep2[last] == 1 && (A.keep1[last] == 1 || A.keep1[last] == 0) &&
+                     env_vec_ok();
+    A.n_threads = (unsigned)(vec ? n / V : n);
+    const unsigned blocks = (A.n_threads + 255) / 256;
+    set_path(vec ? "broadcast_backward_vec" : "broadcast_backward");
+    if (dtype == NK_F32) {
+        if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<float, 4>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
+        else     hipLaunchKernelGGL((broadcast_bwd_kernel<float, 1>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
+    } else {
+        if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<double, 2>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+        else     hipLaunchKernelGGL((broadcast_bwd_kernel<double, 1>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+    }
     NK_HIP(hipGetLastError());
     return NK_OK;
 }

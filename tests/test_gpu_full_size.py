@@ -66,6 +66,39 @@ def test_config2_broadcast_full_size(device, orc, dt, s1, s2):
     free(device, out, ta, tb)
 
 
+def test_config2_broadcast_backward_full_size(device, orc):
+    """The reducing backward of config 2: error [1024,2048,512] -> gradients of shape [1024,1,512] and [1,2048,512].
+    Integer-valued errors make every order of summation exact (numpy is the check); a slab with random
+    errors is compared bit for bit with the oracle's state machine."""
+    rng = np.random.default_rng(22)
+    shape = (1024, 2048, 512)
+    say("C2 backward, integer-valued error")
+    e = rng.integers(-4, 5, shape).astype(f32)
+    te = on(device, e)
+    for d, tgt, oth in ((0, (1024, 1, 512), (1, 2048, 512)), (1, (1, 2048, 512), (1024, 1, 512))):
+        drn = Tensor._on_device(device, f32, tgt)
+        zeros = Tensor._on_device(device, f32, oth)
+        device.launch_broadcast("add", d, drn, zeros, te)
+        assert _lib.last_path() == "broadcast_backward_vec"
+        assert_bits(drn.getData().reshape(tgt), e.sum(axis=1 - d, keepdims=True, dtype=np.float64).astype(f32), f"gradient {d}")
+        free(device, drn, zeros)
+    free(device, te)
+    del e
+    say("C2 backward, random error, slab against the oracle")
+    sub = (8, 2048, 512)
+    e = rng.standard_normal(sub).astype(f32)
+    te = on(device, e)
+    for d, tgt, oth in ((0, (8, 1, 512), (1, 2048, 512)), (1, (1, 2048, 512), (8, 1, 512))):
+        drn = Tensor._on_device(device, f32, tgt)
+        zeros = Tensor._on_device(device, f32, oth)
+        device.launch_broadcast("add", d, drn, zeros, te)
+        want = orc.broadcast("add", d, np.zeros(drn.size, dtype=f32), orc.dense_cfg(tgt), np.zeros(int(np.prod(oth)), dtype=f32), orc.dense_cfg(oth),
+                             e.reshape(-1), orc.dense_cfg(sub))
+        assert_bits(drn.getData(), want, f"slab gradient {d}")
+        free(device, drn, zeros)
+    free(device, te)
+
+
 def _chain_oracle(orc, bases, cfgs, shape, workers=16):
     n = int(np.prod(shape))
     oc = orc.dense_cfg(list(shape))

@@ -327,6 +327,39 @@ def test_broadcast_backward_bit_exact(device, orc, dt):
                 assert_bits(drn.getData(), want, f"{tgt} {op} {d}")
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_broadcast_backward_vector_path_and_views(device, orc, dt):
+    """Drains whose last axis is kept and a multiple of the vector width (16-byte accesses, several drain
+    elements per thread), one and two reduced axes, sources of the operands' own shapes as autograd passes
+    them, and a strided view as the error: all bit-identical to the CPU state machine."""
+    rng = np.random.default_rng(23)
+    full = [9, 21, 16]
+    e = rng.uniform(-1, 1, full).astype(F[dt])
+    te = on(device, e)
+    for tgt, oth in (([9, 1, 16], full), ([1, 21, 16], full), ([1, 1, 16], full), ([9, 21, 1], full), ([9, 21, 16], full),
+                     ([9, 1, 16], [1, 21, 16]), ([1, 21, 16], [9, 1, 16]), ([1, 1, 16], [9, 21, 16]), ([9, 1, 1], [1, 21, 16])):
+        for op in ("add", "subtract", "multiply"):
+            for d in (0, 1):
+                say("broadcast bwd vec", tgt, oth, op, d, dt)
+                other = rng.uniform(-1, 1, oth).astype(F[dt])
+                tother = on(device, other)
+                drn = Tensor._on_device(device, F[dt], tgt)
+                device.launch_broadcast(op, d, drn, tother, te)
+                assert _lib.last_path() == ("broadcast_backward_vec" if tgt[2] == 16 else "broadcast_backward")
+                want = orc.broadcast(op, d, np.zeros(drn.size, dtype=F[dt]), orc.dense_cfg(tgt), other.reshape(-1), orc.dense_cfg(oth), e.reshape(-1), orc.dense_cfg(full))
+                assert_bits(drn.getData(), want, f"{tgt} {oth} {op} {d}")
+    say("broadcast bwd with a sliced error", dt)
+    big = rng.uniform(-1, 1, (18, 21, 33)).astype(F[dt])
+    view = on(device, big)[::2, :, 1:33:2]                       # shape [9, 21, 16], strides (2*21*33, 33, 2)
+    for tgt in ([9, 1, 16], [1, 1, 16], [1, 21, 1]):
+        other = np.zeros(full, dtype=F[dt])
+        drn = Tensor._on_device(device, F[dt], tgt)
+        device.launch_broadcast("add", 0, drn, on(device, other), view)
+        assert _lib.last_path() == "broadcast_backward"
+        want = orc.broadcast("add", 0, np.zeros(drn.size, dtype=F[dt]), orc.dense_cfg(tgt), other.reshape(-1), orc.dense_cfg(full), big.reshape(-1), cfg(view))
+        assert_bits(drn.getData(), want, f"sliced error {tgt}")
+
+
 def test_broadcast_autograd_golden(device, golden):
     g = golden["broadcast_autograd"]
     for row in g["rows"]:
