@@ -6,7 +6,9 @@
 //            register prefetch of the next slice.  Block ids are regrouped so that the blocks that
 //            are co-resident on one XCD (block id mod 8) form a compact patch of the tile grid
 //            and share A row panels and B column panels in that XCD's L2.
-//   simple   everything else (any size, f64): one thread per element of C, the k loop in the
+//   mfma_edge  the same kernel for f32 shapes that are not whole tiles, from 2^24 multiply-adds on: clamped
+//            edges, zeroed k tail, element-wise stores along the edges.
+//   simple   everything else (small products, f64): one thread per element of C, the k loop in the
 //            reference's order with the product rounded before the add, which makes it bit-identical
 //            to GEMM.partial_F32_MxN_RM + AXPY (J/backend/main/operations/linear/internal/blas/GEMM.java:282-304,
 //            AXPY.java:47-59).
@@ -72,6 +74,11 @@ constexpr int LDS_FLOATS_AB = 2 * BM * A_PITCH + 2 * BK * B_PITCH;
 constexpr int LDS_FLOATS_C = BM * C_PITCH;
 constexpr int LDS_FLOATS = LDS_FLOATS_AB > LDS_FLOATS_C ? LDS_FLOATS_AB : LDS_FLOATS_C;
 
+// EDGE: M, N, K need not be multiples of the tile.  Loads go through buffer descriptors over the whole
+// matrices (nothing past their end is touched, the range check returns 0 there), rows and columns past the
+// edge are clamped or left as they come (they only feed results that are not stored), and the k tail is zeroed
+// in both operands so that it adds exactly nothing; the epilogue stores element-wise along the edges.
+template <bool EDGE>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const float* __restrict__ A,
                                                           const float* __restrict__ B, float* __restrict__ C) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
@@ -93,11 +100,26 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     const int b_row = tid >> 5, b_col = (tid & 31) * 4;     // rows b_row + 8*i
     f32x4 ra[4], rb[4];
 
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 4), 0x00020000);
     auto load_global = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 8 * i) * g.N + b_col);
+            if (!EDGE) {
+                ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+                rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 8 * i) * g.N + b_col);
+            } else {
+                int row = tm * BM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
+                const int ka = k0 + a_col;
+                ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * g.K + ka) * 4u, 0, 0)));
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (ka + e >= g.K) ra[i][e] = 0.0f;
+                const int kb = k0 + b_row + 8 * i;
+                const int krow = kb < g.K ? kb : g.K - 1;
+                rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * g.N + tn * BN + b_col) * 4u, 0, 0)));
+                if (kb >= g.K) rb[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
         }
     };
     auto store_lds = [&](int buf) {
@@ -147,7 +169,7 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     // A buffer is rewritten only after a barrier that every wavefront reaches with all its reads of that
     // buffer complete.
     static_assert(BK == 32, "the pipeline below is written for four depth-8 chunks per slice");
-    const int nk = g.K / BK;
+    const int nk = (g.K + BK - 1) / BK;
     Frag f0, f1;
     load_global(0);
     store_lds(0);
@@ -194,6 +216,20 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     __syncthreads();
     float* Cg = C + (int64_t)tm * BM * g.N + tn * BN;
     const int c_col = (tid & 31) * 4, c_row = tid >> 5;
+    if (EDGE) {
+        const int rows = g.M - tm * BM, cols = g.N - tn * BN;          // what is left of C from this tile's origin
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int r = c_row + 8 * i;
+            if (r < rows) {
+                const float* add = &cs[r * C_PITCH + c_col];
+                float* dst = Cg + (int64_t)r * g.N + c_col;
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = dst[e] + add[e];
+            }
+        }
+        return;
+    }
     f32x4 old[16];
 #pragma unroll
     for (int i = 0; i < 16; i++) old[i] = *(const f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col);
@@ -217,14 +253,23 @@ static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* 
 static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
     if (dtype == NK_F64) return launch_simple<double>(dev, M, K, N, (const double*)A, (const double*)B, (double*)C);
     const bool aligned = (A % 16 == 0) && (B % 16 == 0) && (C % 16 == 0);
-    if (aligned && M % BM == 0 && N % BN == 0 && K % BK == 0) {
+    const bool whole_tiles = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
+    // Small products stay on the simple kernel, which keeps the reference's summation order bit for bit; from
+    // 2^24 multiply-adds on, shapes that are not whole tiles take the matrix cores through the edge variant.
+    static const int64_t edge_from = [] { const char* v = getenv("NK_MFMA_EDGE_FROM"); return v && *v ? atoll(v) : (int64_t)1 << 24; }();
+    const bool edge = !whole_tiles && M * K * N >= edge_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
+    if (whole_tiles || edge) {
         MfmaArgs g{};
         g.M = (int)M; g.K = (int)K; g.N = (int)N;
-        g.tiles_m = (int)(M / BM); g.tiles_n = (int)(N / BN);
+        g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
         g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
-        set_path("mfma");
-        hipLaunchKernelGGL(matmul_mfma_kernel, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
-                           (const float*)A, (const float*)B, (float*)C);
+        set_path(whole_tiles ? "mfma" : "mfma_edge");
+        if (whole_tiles)
+            hipLaunchKernelGGL(matmul_mfma_kernel<false>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
+                               (const float*)A, (const float*)B, (float*)C);
+        else
+            hipLaunchKernelGGL(matmul_mfma_kernel<true>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
+                               (const float*)A, (const float*)B, (float*)C);
         NK_HIP(hipGetLastError());
         return NK_OK;
     }

@@ -603,6 +603,46 @@ def test_matmul_mfma_path(device, orc, mkn):
     assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("mkn", [(300, 257, 270), (129, 1001, 131), (1000, 33, 1000), (127, 4097, 40), (641, 130, 385)])
+def test_matmul_mfma_edge_path(device, orc, mkn):
+    """Shapes that are not whole tiles, from 2^24 multiply-adds on: the matrix-core kernel with clamped edges and a
+    zeroed k tail.  Exact on integer-valued data, norm-wise 1e-5 on uniform data, accumulation into C, both
+    layouts; NaNs parked right behind the operands' rows must not leak into the result."""
+    M, K, N = mkn
+    rng = np.random.default_rng(54)
+    say("matmul mfma edge integer", mkn)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float32); B = rng.integers(-5, 6, (K, N)).astype(np.float32)
+    C0 = rng.integers(-9, 10, (M, N)).astype(np.float32)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == "mfma_edge"
+    assert (tc.getData().reshape(M, N) == (A.astype(np.float64) @ B.astype(np.float64) + C0)).all()
+    say("matmul mfma edge column major", mkn)
+    tc = on(device, np.zeros((M, N), dtype=np.float32))
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+    assert _lib.last_path() == "mfma_edge"
+    assert (tc.getData().reshape(N, M).T == A.astype(np.float64) @ B.astype(np.float64)).all()
+    say("matmul mfma edge uniform", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    tc = on(device, np.zeros((M, N), dtype=np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+    say("matmul mfma edge, operands inside larger buffers full of NaN", mkn)
+    # the C ABI takes addresses: place A, B and C in the middle of NaN-filled allocations
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(np.zeros((M, N), dtype=np.float32))
+    _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
