@@ -258,6 +258,61 @@ class Function:
         raise IllegalArgumentException("derive() is provided for flat activation functions only")
 
 
+def _const(v: float) -> Node:
+    return Node("const", float(v))
+
+
+def _is_const(n: Node, v: float) -> bool:
+    return n.kind == "const" and n.value == v
+
+
+def _mul(a: Node, b: Node) -> Node:
+    if _is_const(a, 0.0) or _is_const(b, 0.0): return _const(0.0)
+    if _is_const(a, 1.0): return b
+    if _is_const(b, 1.0): return a
+    return Node("op", "multiply", [a, b])
+
+
+def _add(a: Node, b: Node) -> Node:
+    if _is_const(a, 0.0): return b
+    if _is_const(b, 0.0): return a
+    return Node("op", "add", [a, b])
+
+
+def _sub(a: Node, b: Node) -> Node:
+    if _is_const(b, 0.0): return a
+    if _is_const(a, 0.0): return _mul(_const(-1.0), b)
+    return Node("op", "subtract", [a, b])
+
+
+def derivative_of(n: Node, index: int) -> Node:
+    """The expression tree of d n / d I[index] (the role of Function.getDerivative in
+    devices/opencl/utility/CLFunctionCompiler.java:155-157), with 0 and 1 folded away.  ``dfun`` nodes stand for
+    the derivative of a unary function at their argument."""
+    if n.kind == "input":
+        return _const(1.0 if n.value == index else 0.0)
+    if n.kind == "const":
+        return _const(0.0)
+    if n.kind == "fun":
+        u = n.children[0]
+        return _mul(Node("dfun", n.value, [u]), derivative_of(u, index))
+    if n.kind == "dfun":
+        raise IllegalArgumentException("second derivatives of fused functions are not supported")
+    u, v = n.children
+    du, dv = derivative_of(u, index), derivative_of(v, index)
+    if n.value == "add": return _add(du, dv)
+    if n.value == "subtract": return _sub(du, dv)
+    if n.value == "multiply": return _add(_mul(du, v), _mul(u, dv))
+    if n.value == "divide":          # du / v - u * dv / v^2
+        return _sub(Node("op", "divide", [du, v]) if not _is_const(du, 0.0) else _const(0.0),
+                    _mul(dv, Node("op", "divide", [u, Node("op", "multiply", [v, v])])))
+    if n.value == "power":           # d(u^v) = v * u^(v-1) * du + u^v * ln(u) * dv
+        first = _mul(_mul(v, Node("op", "power", [u, Node("op", "subtract", [v, _const(1.0)])])), du)
+        second = _mul(_mul(Node("op", "power", [u, v]), Node("fun", "ln", [u])), dv)
+        return _add(first, second)
+    raise IllegalArgumentException(f"operator '{n.value}' has no fused derivative")
+
+
 class OptimizedFunction:
     """One fused kernel for a whole elementwise expression (the counterpart of CLFunctionCompiler,
     devices/opencl/utility/CLFunctionCompiler.java:27-238): the expression tree is lowered to the postfix
@@ -267,27 +322,45 @@ class OptimizedFunction:
         self.device, self.function, self.name = device, function, name
         self.program: List[int] = []
         self.consts: List[float] = []
-        self._lower(function.root)
+        self._lower(function.root, self.program, self.consts)
         self.n_src = function.numberOfArgs()
+        self._derivatives = {}               # input index -> (program, consts) of the derivative kernel
 
-    def _lower(self, n: Node) -> None:
+    @staticmethod
+    def _lower(n: Node, program: List[int], consts: List[float]) -> None:
         if n.kind == "input":
-            self.program += [_lib.FUSE_LOAD, n.value]
+            program += [_lib.FUSE_LOAD, n.value]
         elif n.kind == "const":
-            if n.value not in self.consts:
-                self.consts.append(n.value)
-            self.program += [_lib.FUSE_CONST, self.consts.index(n.value)]
-        elif n.kind == "fun":
+            if n.value not in consts:
+                consts.append(n.value)
+            program += [_lib.FUSE_CONST, consts.index(n.value)]
+        elif n.kind in ("fun", "dfun"):
             if n.value not in _lib.FUN:
                 raise IllegalArgumentException(f"function '{n.value}' cannot be fused into an elementwise kernel")
-            self._lower(n.children[0])
-            self.program += [_lib.FUSE_FUN, _lib.FUN[n.value]]
+            OptimizedFunction._lower(n.children[0], program, consts)
+            program += [_lib.FUSE_FUN if n.kind == "fun" else _lib.FUSE_DFUN, _lib.FUN[n.value]]
         else:
             if n.value not in _lib.OP:
                 raise IllegalArgumentException(f"operator '{n.value}' cannot be fused into an elementwise kernel")
-            self._lower(n.children[0])
-            self._lower(n.children[1])
-            self.program += [_lib.FUSE_BIN, _lib.OP[n.value]]
+            OptimizedFunction._lower(n.children[0], program, consts)
+            OptimizedFunction._lower(n.children[1], program, consts)
+            program += [_lib.FUSE_BIN, _lib.OP[n.value]]
+
+    def derivative_program(self, index: int):
+        """Op-codes of the kernel for d f / d I[index] (CLFunctionCompiler compiles it next to the activation)."""
+        if index not in self._derivatives:
+            program, consts = [], []
+            self._lower(derivative_of(self.function.root, index), program, consts)
+            self._derivatives[index] = (program, consts)
+        return self._derivatives[index]
+
+    def derive(self, inputs: Sequence[Tensor], index: int) -> Tensor:
+        """d f / d I[index] at the inputs, in one launch."""
+        srcs = list(inputs[: self.n_src])
+        program, consts = self.derivative_program(index)
+        out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
+        self.device.launch_fused(program, consts, out, srcs)
+        return out
 
     def call(self, *inputs: Tensor) -> Tensor:
         if len(inputs) == 1 and isinstance(inputs[0], (list, tuple)):
@@ -306,6 +379,11 @@ class OptimizedFunction:
                 t.setIsVirtual(False)
             out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
             self.device.launch_fused(self.program, self.consts, out, srcs)
+            if self.function.doAD and not guests and any(t.rqsGradient() or t._node is not None for t in srcs):
+                # reverse mode: error * (d f / d I[d]), the derivative in one fused launch
+                def action(d):
+                    return lambda error: execute("multiply", [error, self.derive(srcs, d)], record=False)
+                out._node = GraphNode(srcs, [action(d) if (t.rqsGradient() or t._node is not None) else None for d, t in enumerate(srcs)])
             return out
         finally:
             for t in guests:

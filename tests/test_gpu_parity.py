@@ -414,6 +414,38 @@ def test_fused_chain_equals_unfused_and_oracle(device, orc, dt):
         assert_close(f2(*tens).items, ((x * y) + (y - z) * (z / (x * x + 2))).reshape(-1), "nested vs numpy")
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_fused_derivative_kernels_and_autograd(device, orc, dt):
+    """A fused function also carries one kernel per input for its derivative (CLFunctionCompiler.java:155-157).
+    They must agree with the chain rule applied by the unfused graph, and with central differences in f64."""
+    rng = np.random.default_rng(33)
+    shape = (37, 24)
+    arrays = [rng.uniform(0.5, 1.5, shape).astype(F[dt]) for _ in range(3)]
+    for expr in ("tanh(sig(I[0])*I[1]+I[2])", "sin(I[0])/cos(I[1])+I[2]*I[2]", "(I[0]+2)**I[1]-exp(I[2])"):
+        say("fused derivative", expr, dt)
+        fn = Function.of(expr)
+        fused = device.optimizedFunctionOf(fn, "f")
+        # autograd through the fused kernel against autograd through the unfused graph
+        e = rng.uniform(-1, 1, shape).astype(F[dt])
+        grads = []
+        for runner in (fused, fn):
+            ts = [on(device, a).setRqsGradient(True) for a in arrays]
+            runner(*ts).backward(on(device, e))
+            grads.append([t.gradient.items for t in ts])
+        for i in range(3):
+            scale = np.abs(grads[1][i]) + np.abs(e.reshape(-1))
+            assert (np.abs(grads[0][i] - grads[1][i]) <= 20 * RTOL[np.dtype(F[dt])] * scale + ATOL[np.dtype(F[dt])]).all(), (expr, i)
+        if dt == "f64":                                   # and the derivative kernels themselves against central differences
+            ts = [on(device, a) for a in arrays]
+            for i in range(3):
+                h = 1e-6
+                up, dn = [a.copy() for a in arrays], [a.copy() for a in arrays]
+                up[i] += h; dn[i] -= h
+                numeric = (fused(*[on(device, a) for a in up]).items - fused(*[on(device, a) for a in dn]).items) / (2 * h)
+                got = fused.derive(ts, i).items
+                assert (np.abs(got - numeric) <= 1e-6 * np.maximum(1.0, np.abs(numeric))).all(), (expr, i)
+
+
 # ---- convolution ----------------------------------------------------------------------------------------------
 def test_convolution_golden_on_device(device, golden):
     for row in golden["convolution_forward"]["rows"]:

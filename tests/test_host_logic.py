@@ -117,3 +117,40 @@ def test_no_host_arithmetic_path():
     a = Tensor.of(np.float32, [2, 2], [1, 2, 3, 4])
     with pytest.raises(IllegalStateException):
         a + a
+
+
+def test_symbolic_derivative_of_fused_expressions():
+    """derivative_of builds d f / d I[i] with 0 and 1 folded away; checked against central differences in
+    float64 with a small evaluator of the same trees."""
+    import math
+    from neureka_amd.function import Function, derivative_of
+
+    funs = {"tanh": math.tanh, "sig": lambda x: 1 / (1 + math.exp(-x)), "sin": math.sin, "cos": math.cos, "exp": math.exp,
+            "ln": math.log, "quad": lambda x: x * x, "sqrt": math.sqrt}
+    dfuns = {"tanh": lambda x: 1 - math.tanh(x) ** 2, "sig": lambda x: (1 / (1 + math.exp(-x))) * (1 - 1 / (1 + math.exp(-x))),
+             "sin": math.cos, "cos": lambda x: -math.sin(x), "exp": math.exp, "ln": lambda x: 1 / x, "quad": lambda x: 2 * x,
+             "sqrt": lambda x: 0.5 / math.sqrt(x)}
+    ops = {"add": lambda a, b: a + b, "subtract": lambda a, b: a - b, "multiply": lambda a, b: a * b, "divide": lambda a, b: a / b,
+           "power": lambda a, b: a ** b}
+
+    def ev(n, x):
+        if n.kind == "input": return x[n.value]
+        if n.kind == "const": return n.value
+        if n.kind == "fun": return funs[n.value](ev(n.children[0], x))
+        if n.kind == "dfun": return dfuns[n.value](ev(n.children[0], x))
+        return ops[n.value](ev(n.children[0], x), ev(n.children[1], x))
+
+    x = [0.7, 1.3, 0.4]
+    for expr in ("tanh(sig(I[0])*I[1]+I[2])", "I[0]*I[0]*I[1]", "sin(I[0])/cos(I[1])", "(I[0]+2)**I[1]", "exp(I[0]-I[2])*3", "quad(I[1])-ln(I[0])",
+                 "sqrt(I[0]*I[1])/I[2]"):
+        root = Function.of(expr).root
+        for i in range(3):
+            d = derivative_of(root, i)
+            h = 1e-6
+            xp, xm = list(x), list(x)
+            xp[i] += h; xm[i] -= h
+            numeric = (ev(root, xp) - ev(root, xm)) / (2 * h)
+            assert abs(ev(d, x) - numeric) <= 1e-6 * max(1.0, abs(numeric)), (expr, i)
+    # folding: the derivative with respect to an absent input is the constant 0, of I[0]+I[1] the constant 1
+    assert repr(derivative_of(Function.of("sig(I[0])*I[1]").root, 2)) == "0.0"
+    assert repr(derivative_of(Function.of("I[0]+I[1]").root, 1)) == "1.0"
