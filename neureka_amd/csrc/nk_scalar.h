@@ -122,7 +122,7 @@ __device__ __forceinline__ float gauss(float x) {
     float hi = x * x;
     float lo = ::fmaf(x, x, -hi);
     float e = ::expf(-hi);
-    return e - e * lo;
+    return e > 0.0f ? e - e * lo : e;       // e == 0 (x*x overflowed or is huge): lo may be infinite; NaN stays NaN
 }
 
 // The evaluators below work on V values at once with the switch outside the lane loop: the op-code

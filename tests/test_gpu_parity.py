@@ -152,6 +152,25 @@ def test_all_activations_and_derivatives(device, orc, dt):
                 assert_close(got, want, f"{name} d={d}")
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_activations_on_special_values(device, orc, dt):
+    """Zeros of both signs, infinities, NaN, huge, tiny and subnormal arguments: NaN where the CPU device gives NaN,
+    the same infinity where it gives one, within tolerance elsewhere."""
+    T = F[dt]
+    x = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 100.0, -100.0, 1e30, -1e30, 1e-30, -1e-30, 1e-40, 20.0, -20.0, 0.1249, 0.1251, -0.125, 88.0, -88.0,
+                  709.0, -709.0], dtype=T)
+    c = orc.dense_cfg([x.size])
+    tx = on(device, x)
+    for name in ACTS:
+        for d in (-1, 0):
+            say("activation specials", name, d, dt)
+            out = on(device, np.zeros(x.size, dtype=T))
+            device.launch_activation(name, d, out, tx)
+            with np.errstate(all="ignore"):
+                want = orc.activation(name, d, np.zeros(x.size, dtype=T), c, x, c)
+                assert_close(out.getData(), want, f"{name} d={d} on {x.tolist()}")
+
+
 def test_activation_golden_vectors_on_device(device, orc, golden):
     g = golden["activation_vectors"]
     for row in g["rows"]:
