@@ -23,8 +23,8 @@ __device__ __forceinline__ T bcast_derive(int op, int d, T a, T b) {
         case NK_OP_SUB: return d == 0 ? a + b : a - b;
         case NK_OP_MUL: return d == 0 ? b : a;
         case NK_OP_DIV:
-        case NK_OP_MOD: return d == 0 ? T(1) / b : -(a / (b * b));
-        case NK_OP_POW: return d == 0 ? a * N::pow(a, b - T(1)) : N::pow(a, b) * N::log(a);
+        case NK_OP_MOD: return d == 0 ? T(1) / b : ddiv_db_ref(a, b);
+        case NK_OP_POW: return d == 0 ? bcast_dpow_da_ref(a, b) : dpow_db_ref(a, b);
     }
     return T(NAN);
 }

@@ -48,6 +48,22 @@ template <> struct Num<double> {
     static __device__ __forceinline__ double fma(double a, double b, double c) { return ::fma(a, b, c); }
 };
 
+// Binary operators whose f32 form the reference evaluates through double (Math.pow / Math.log take and return
+// double; implementations/elementwise/CPUBiElementWisePower.java:11,21,31, CPUBiElementWiseDivision.java:31,
+// CPUBiElementWiseModulo.java:31 and the broadcast twins): the intermediates neither overflow nor underflow
+// where float ones would.
+__device__ __forceinline__ double pow_ref(double a, double b) { return ::pow(a, b); }
+__device__ __forceinline__ float pow_ref(float a, float b) { return (float)::pow((double)a, (double)b); }
+__device__ __forceinline__ double dpow_da_ref(double a, double b) { return b * ::pow(a, b - 1); }
+__device__ __forceinline__ float dpow_da_ref(float a, float b) { return (float)((double)b * ::pow((double)a, (double)(b - 1.0f))); }
+// the broadcast twin multiplies by a, not by b (implementations/broadcast/CPUBroadcastPower.java:20-21)
+__device__ __forceinline__ double bcast_dpow_da_ref(double a, double b) { return a * ::pow(a, b - 1); }
+__device__ __forceinline__ float bcast_dpow_da_ref(float a, float b) { return (float)((double)a * ::pow((double)a, (double)(b - 1.0f))); }
+__device__ __forceinline__ double dpow_db_ref(double a, double b) { return ::pow(a, b) * ::log(a); }
+__device__ __forceinline__ float dpow_db_ref(float a, float b) { return (float)(::pow((double)a, (double)b) * ::log((double)a)); }
+__device__ __forceinline__ double ddiv_db_ref(double a, double b) { return -(a / (b * b)); }
+__device__ __forceinline__ float ddiv_db_ref(float a, float b) { return (float)-((double)a / ((double)b * (double)b)); }   // b*b is exact in double
+
 // FunUtil.invSqrt (fun/FunUtil.java:5-27): the bit-trick inverse square root with 4 (double) or 2
 // (float) Newton steps, transcribed operation for operation.
 __device__ __forceinline__ double inv_sqrt_ref(double x) {
@@ -290,7 +306,7 @@ __device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
             if constexpr (FUNSET >= 2) {
                 switch (op) {
                     case NK_OP_MOD: NK_EACH2(N::fmod(x, y));     // Java's % on floating point is C's fmod
-                    case NK_OP_POW: NK_EACH2(N::pow(x, y));
+                    case NK_OP_POW: NK_EACH2(pow_ref(x, y));
                     default: NK_EACH2(T(NAN) + x + y);
                 }
             } else NK_EACH2(T(NAN) + x + y);
@@ -317,9 +333,9 @@ __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b
                     case NK_OP_DIV * 2 + 0:
                     case NK_OP_MOD * 2 + 0: NK_EACH2(T(1) / y);
                     case NK_OP_DIV * 2 + 1:
-                    case NK_OP_MOD * 2 + 1: NK_EACH2(-(x / (y * y)));
-                    case NK_OP_POW * 2 + 0: NK_EACH2(y * N::pow(x, y - T(1)));
-                    case NK_OP_POW * 2 + 1: NK_EACH2(N::pow(x, y) * N::log(x));
+                    case NK_OP_MOD * 2 + 1: NK_EACH2(ddiv_db_ref(x, y));
+                    case NK_OP_POW * 2 + 0: NK_EACH2(dpow_da_ref(x, y));
+                    case NK_OP_POW * 2 + 1: NK_EACH2(dpow_db_ref(x, y));
                     default: NK_EACH2(T(NAN) + x + y);
                 }
             } else NK_EACH2(T(NAN) + x + y);

@@ -153,6 +153,27 @@ def test_all_activations_and_derivatives(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_binary_operators_on_special_values(device, orc, dt):
+    """Every pair from a set of special values through + - * / % ** and their partial derivatives."""
+    T = F[dt]
+    vals = np.array([0.0, -0.0, 1.0, -1.0, 0.5, -2.5, 3.0, np.inf, -np.inf, np.nan, 1e30, -1e-30], dtype=T)
+    a = np.repeat(vals, vals.size); b = np.tile(vals, vals.size)
+    c = orc.dense_cfg([a.size])
+    ta, tb = on(device, a), on(device, b)
+    for op in ("add", "subtract", "multiply", "divide", "modulo", "power"):
+        for d in (-1, 0, 1):
+            say("operator specials", op, d, dt)
+            out = on(device, np.zeros(a.size, dtype=T))
+            device.launch_elementwise(op, d, out, ta, tb)
+            with np.errstate(all="ignore"):
+                want = orc.elementwise(op, d, np.zeros(a.size, dtype=T), c, a, c, b, c)
+            if op in ("add", "subtract", "multiply", "divide", "modulo") and d < 0:
+                assert_bits(out.getData(), want, f"{op}")
+            else:
+                assert_close(out.getData(), want, f"{op} d={d}")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_activations_on_special_values(device, orc, dt):
     """Zeros of both signs, infinities, NaN, huge, tiny and subnormal arguments: NaN where the CPU device gives NaN,
     the same infinity where it gives one, within tolerance elsewhere."""
