@@ -16,7 +16,8 @@ def assert_close(got, want, what=""):
     dt = np.dtype(want.dtype)
     both_nan = np.isnan(got) & np.isnan(want)
     both_inf = np.isinf(want) & (got == want)
-    ok = both_nan | both_inf | (np.abs(got - want) <= RTOL[dt] * np.abs(want) + ATOL[dt])
+    with np.errstate(invalid="ignore"):          # inf - inf in the difference of matching infinities
+        ok = both_nan | both_inf | (np.abs(got - want) <= RTOL[dt] * np.abs(want) + ATOL[dt])
     if not ok.all():
         bad = np.flatnonzero(~ok.reshape(-1))
         i = bad[0]
