@@ -820,3 +820,74 @@ def test_dot_product(device, orc, dt):
         assert on(device, ai).dot(on(device, bi)).items[0] == orc.dot(ai, bi)       # exact on small integers
     with pytest.raises(IllegalArgumentException):
         on(device, np.ones(3, dtype=F[dt])).dot(on(device, np.ones(4, dtype=F[dt])))
+
+
+# ---- randomised views: every plan of the elementwise engine against the oracle walking the same descriptors ------
+def _random_view(device, rng, shape, dt):
+    """A tensor of the given shape that is a random permutation of a random strided slice of a larger parent.
+    Returns (view, parent data)."""
+    rank = len(shape)
+    perm = list(rng.permutation(rank))
+    pre = [0] * rank                      # shape of the slice: permute(*perm) must turn it into `shape`
+    for k in range(rank):
+        pre[perm[k]] = shape[k]
+    starts = [int(rng.integers(0, 3)) for _ in range(rank)]
+    steps = [int(rng.integers(1, 4)) for _ in range(rank)]
+    parent_shape = [starts[k] + (pre[k] - 1) * steps[k] + 1 + int(rng.integers(0, 2)) for k in range(rank)]
+    data = rng.uniform(-2, 2, parent_shape).astype(dt)
+    t = on(device, data)
+    sl = t[tuple(slice(starts[k], starts[k] + (pre[k] - 1) * steps[k] + 1, steps[k]) for k in range(rank))]
+    assert list(sl.shape) == pre
+    v = sl.permute(*perm) if rank > 1 else sl
+    assert list(v.shape) == list(shape)
+    return v, data
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_random_views_through_every_kernel_plan(device, orc, dt):
+    T = F[dt]
+    rng = np.random.default_rng(77)
+    paths = set()
+    for case in range(160):
+        rank = int(rng.integers(1, 6))
+        shape = [int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 33])) for _ in range(rank)]
+        while int(np.prod(shape)) > 6000:
+            shape[int(np.argmax(shape))] = 2
+        kind = ("elementwise", "activation", "scalarization", "broadcast")[case % 4]
+        say("random view", case, kind, shape, dt)
+        n = int(np.prod(shape))
+        if kind == "broadcast":
+            sa = [s if rng.random() < 0.6 else 1 for s in shape]
+            sb = [s if (a == 1 or rng.random() < 0.6) else 1 for s, a in zip(shape, sa)]
+            so = [max(a, b) for a, b in zip(sa, sb)]
+            (va, da), (vb, db) = _random_view(device, rng, sa, T), _random_view(device, rng, sb, T)
+            out = Tensor._on_device(device, T, so)
+            op = str(rng.choice(["add", "subtract", "multiply"]))
+            device.launch_broadcast(op, -1, out, va, vb)
+            want = orc.broadcast(op, -1, np.zeros(out.size, dtype=T), cfg(out), da.reshape(-1), cfg(va), db.reshape(-1), cfg(vb))
+            assert_bits(out.getData(), want, f"case {case} broadcast {op} {sa} {sb}")
+        else:
+            (va, da), (vb, db) = _random_view(device, rng, shape, T), _random_view(device, rng, shape, T)
+            drain_is_view = rng.random() < 0.3
+            if drain_is_view:
+                vo, do = _random_view(device, rng, shape, T)
+                host_out = do.reshape(-1).copy()
+            else:
+                vo = Tensor._on_device(device, T, shape); host_out = np.zeros(n, dtype=T)
+            if kind == "elementwise":
+                op = str(rng.choice(["add", "subtract", "multiply", "divide"]))
+                device.launch_elementwise(op, -1, vo, va, vb)
+                want = orc.elementwise(op, -1, host_out, cfg(vo), da.reshape(-1), cfg(va), db.reshape(-1), cfg(vb))
+            elif kind == "activation":
+                fun = str(rng.choice(["relu", "quad", "abs", "idy", "softsign"]))
+                device.launch_activation(fun, -1, vo, va)
+                want = orc.activation(fun, -1, host_out, cfg(vo), da.reshape(-1), cfg(va))
+            else:
+                op = str(rng.choice(["add", "multiply", "divide", "idy"]))
+                device.launch_scalarization(op, -1, vo, va, 1.75)
+                want = orc.scalarization(op, -1, host_out, cfg(vo), da.reshape(-1), cfg(va), 1.75)
+            got = device._read_all(vo._data) if drain_is_view else vo.getData()
+            assert_bits(got, want, f"case {case} {kind} {shape}")
+        paths.add(_lib.last_path())
+    say("plans seen", sorted(paths))
+    assert {"rows", "canon"} <= {p.split("_")[0] for p in paths}
