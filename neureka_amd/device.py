@@ -259,6 +259,45 @@ class HipDevice:
         new = self.allocateFromOne(tensor.dtype, 1, value)
         tensor._replace_data(new)
 
+    # ---- the protected contract of AbstractDevice (devices/AbstractDevice.java:188-206), as OpenCLDevice fills it in
+    #      (devices/opencl/OpenCLDevice.java:527-660); indices are positions in the tensor's buffer ------------------
+    def _readAll(self, tensor, clone: bool = True) -> np.ndarray:
+        return self._read_all(tensor._data)
+
+    def _readItem(self, tensor, index: int):
+        return self._read(tensor._data, index, 1)[0]
+
+    def _readArray(self, tensor, start: int, size: int) -> np.ndarray:
+        return self._read(tensor._data, start, size)
+
+    def _writeItem(self, tensor, item, start: int, size: int) -> None:
+        """One value repeated over [start, start + size): a device fill (OpenCLDevice.java:537-541)."""
+        self._fill(tensor._data, start, size, item)
+
+    def _writeArray(self, tensor, array, offset: int, start: int, size: int) -> None:
+        """array[offset : offset + size] -> buffer[start : start + size] (OpenCLDevice.java:542-552)."""
+        self._write(tensor._data, start, np.asarray(array).reshape(-1)[offset:offset + size])
+
+    def _swap(self, former, replacement) -> None:
+        """The replacement takes over the former tensor's device data (OpenCLDevice.java:635-640)."""
+        replacement._set_data(former._data, self)
+
+    def _sizeOccupiedBy(self, tensor) -> int:
+        return tensor._data.size
+
+    def _dataTypeOf(self, raw) -> np.dtype:
+        return np.dtype(raw.dtype)
+
+    def update(self, tensor, added: bool) -> bool:
+        """Component.update(OwnerChangeRequest) (OpenCLDevice.java:340-371): a tensor that gains this device as a
+        component is stored on it, one that loses it is restored to the host."""
+        if added:
+            if not self.has(tensor):
+                self.store(tensor)
+        elif self.has(tensor):
+            self.restore(tensor)
+        return True
+
     def _check_open(self) -> None:
         if self._disposed:
             raise IllegalStateException("HipDevice has been disposed")

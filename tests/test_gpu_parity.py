@@ -88,6 +88,25 @@ def test_store_restore_free_virtual_and_slices(device):
     assert device.numberOfStored() == stored and device.numberOfDataObjects() == objs
 
 
+def test_protected_device_contract(device):
+    """_readItem/_readArray/_writeItem/_writeArray/_swap/_sizeOccupiedBy/update as AbstractDevice declares them
+    (devices/AbstractDevice.java:188-206), partial reads and writes included (Cross_Device_IO_Spec)."""
+    say("protected device contract")
+    t = Tensor.of(np.float64, [3, 4], np.arange(12.0)).to(device)
+    assert device._sizeOccupiedBy(t) == 12 and device._dataTypeOf(t._data) == np.float64
+    assert device._readItem(t, 7) == 7.0 and device._readArray(t, 4, 3).tolist() == [4.0, 5.0, 6.0]
+    device._writeItem(t, -1.5, 2, 3)                       # one value over three positions
+    device._writeArray(t, [100.0, 200.0, 300.0, 400.0], 1, 9, 2)      # array[1:3] -> positions 9, 10
+    assert device._readAll(t).tolist() == [0, 1, -1.5, -1.5, -1.5, 5, 6, 7, 8, 200, 300, 11]
+    other = Tensor(np.float64, NDConfiguration.ofShape((12,)), None)
+    device._swap(t, other)
+    assert other.isOutsourced() and other.items.tolist() == device._readAll(t).tolist()
+    host = Tensor.of(np.float32, [4], [1, 2, 3, 4])
+    assert device.update(host, True) and host.isOutsourced()
+    assert device.update(host, False) and not host.isOutsourced() and host.items.tolist() == [1, 2, 3, 4]
+    device.free(t)
+
+
 def test_bad_arguments_are_reported(device):
     say("argument errors")
     a = on(device, np.ones(8, dtype=np.float32))
