@@ -23,6 +23,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
+FP64_PEAK_TFLOPS = 78.6        # MI355X dense fp64 matrix, published
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
 # against a plain 1 GiB copy): profiles/rows_binary_kernel_broadcast_c2.md
 C2_TRAFFIC_BYTES = 4316807974
@@ -161,11 +162,12 @@ def main():
             gbs = nbytes / (ms * 1e-3) / 1e9
             others[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "path": _lib.last_path()}
 
-        def flops(name, nflop, nbytes, launch):
+        def flops(name, nflop, nbytes, launch, f64=False):
             warm(launch)
             ms = event_time_ms(dev, launch, reps)
             tf = nflop / (ms * 1e-3) / 1e12
-            others[name] = {"ms": round(ms, 4), "GFLOP/s": round(tf * 1e3, 1), "frac_fp32": round(tf / FP32_PEAK_TFLOPS, 4),
+            frac = {"frac_fp64": round(tf / FP64_PEAK_TFLOPS, 4)} if f64 else {"frac_fp32": round(tf / FP32_PEAK_TFLOPS, 4)}
+            others[name] = {"ms": round(ms, 4), "GFLOP/s": round(tf * 1e3, 1), **frac,
                             "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "path": _lib.last_path()}
 
         # C2 f64
@@ -234,6 +236,12 @@ def main():
             Cm = Tensor._on_device(dev, f32, (M, N))
             flops(name, 2.0 * M * K * N, 4 * (M * K + K * N + M * N), dev.prepared_launch("matmul", True, M, K, N, A, B, Cm))
             for t in (A, B, Cm): dev.free(t)
+        M = K = N = 4096
+        A = Tensor.of(np.float64, (M, K), rng.uniform(-1, 1, M * K)).to(dev)
+        B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)
+        Cm = Tensor._on_device(dev, np.float64, (M, N))
+        flops("matmul_4096_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul", True, M, K, N, A, B, Cm), f64=True)
+        for t in (A, B, Cm): dev.free(t)
 
         # C1 and C5 convolutions
         x1 = Tensor.of(f32, (64, 64), rng.uniform(-1, 1, 4096).astype(f32)).to(dev)

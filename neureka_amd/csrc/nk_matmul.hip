@@ -8,7 +8,8 @@
 //            and share A row panels and B column panels in that XCD's L2.
 //   mfma_edge  the same kernel for f32 shapes that are not whole tiles, from 2^24 multiply-adds on: clamped
 //            edges, zeroed k tail, element-wise stores along the edges.
-//   simple   everything else (small products, f64): one thread per element of C, the k loop in the
+//   mfma_f64 / mfma_f64_edge  f64 from 2^24 multiply-adds on: v_mfma_f64_16x16x4_f64, same tiling.
+//   simple   everything else (small products): one thread per element of C, the k loop in the
 //            reference's order with the product rounded before the add, which makes it bit-identical
 //            to GEMM.partial_F32_MxN_RM + AXPY (J/backend/main/operations/linear/internal/blas/GEMM.java:282-304,
 //            AXPY.java:47-59).
@@ -240,6 +241,122 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     }
 }
 
+// ---- f64 on the matrix cores ----------------------------------------------------------------------------------
+// 128x128 block tile, four wavefronts in a 2x2 arrangement, each owning 64x64 as 4x4 accumulators of
+// v_mfma_f64_16x16x4_f64 (register v of lane l holds row 4*v + l/16 of column l%16 of a 16x16 tile; it feeds A[row l%16]
+// [k l/16] and B[k l/16][column l%16]).  k-slices of 16 in double-buffered LDS: A rows have a pitch of 17
+// doubles, which spreads the 16 rows a quarter-wavefront reads over all banks.
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+namespace d64 {
+constexpr int DK = 16;
+constexpr int DA_PITCH = DK + 1;
+constexpr int DB_PITCH = BN + 2;
+constexpr int LDS_DOUBLES = 2 * BM * DA_PITCH + 2 * DK * DB_PITCH;
+}
+
+template <bool EDGE>
+__global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, const double* __restrict__ A,
+                                                              const double* __restrict__ B, double* __restrict__ C) {
+    using namespace d64;
+    __shared__ __attribute__((aligned(16))) double lds[LDS_DOUBLES];
+    double* const As0 = lds;                                   // [2][BM * DA_PITCH]
+    double* const Bs0 = lds + 2 * BM * DA_PITCH;                // [2][DK * DB_PITCH]
+    int tm, tn;
+    tile_of_block(g, tm, tn);
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int l16 = lane & 15, q = lane >> 4;
+
+    // global -> registers: A slice 128x16 and B slice 16x128, four 16-byte pieces each per thread
+    const int a_row = tid >> 3, a_col = (tid & 7) * 2;       // rows a_row + 32*i
+    const int b_row = tid >> 6, b_col = (tid & 63) * 2;      // rows b_row + 4*i
+    f64x2 ra[4], rb[4];
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 8), 0x00020000);
+    const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 8), 0x00020000);
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if (!EDGE) {
+                ra[i] = *(const f64x2*)(A + ((int64_t)tm * BM + a_row + 32 * i) * g.K + k0 + a_col);
+                rb[i] = *(const f64x2*)(B + (int64_t)(k0 + b_row + 4 * i) * g.N + tn * BN + b_col);
+            } else {
+                int row = tm * BM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
+                const int ka = k0 + a_col;
+                ra[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * g.K + ka) * 8u, 0, 0)));
+#pragma unroll
+                for (int e = 0; e < 2; e++) if (ka + e >= g.K) ra[i][e] = 0.0;
+                const int kb = k0 + b_row + 4 * i;
+                const int krow = kb < g.K ? kb : g.K - 1;
+                rb[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * g.N + tn * BN + b_col) * 8u, 0, 0)));
+                if (kb >= g.K) rb[i] = f64x2{0.0, 0.0};
+            }
+        }
+    };
+    auto store_lds = [&](int buf) {
+        double* as = As0 + buf * (BM * DA_PITCH);
+        double* bs = Bs0 + buf * (DK * DB_PITCH);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            as[(a_row + 32 * i) * DA_PITCH + a_col] = ra[i][0];
+            as[(a_row + 32 * i) * DA_PITCH + a_col + 1] = ra[i][1];
+            *(f64x2*)(&bs[(b_row + 4 * i) * DB_PITCH + b_col]) = rb[i];
+        }
+    };
+
+    f64x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0};
+
+    const int nk = (g.K + DK - 1) / DK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < nk;
+        if (more) load_global((kt + 1) * DK);
+        const double* as = As0 + cur * (BM * DA_PITCH);
+        const double* bs = Bs0 + cur * (DK * DB_PITCH);
+#pragma unroll
+        for (int c = 0; c < DK / 4; c++) {
+            double a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) a[i] = as[(wm + 16 * i + l16) * DA_PITCH + 4 * c + q];
+#pragma unroll
+            for (int j = 0; j < 4; j++) b[j] = bs[(4 * c + q) * DB_PITCH + wn + 16 * j + l16];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            store_lds(cur ^ 1);
+            __syncthreads();
+        }
+    }
+
+    // epilogue: C is accumulated into; a quarter-wavefront covers 16 consecutive doubles of a row
+    const int rows = g.M - tm * BM, cols = g.N - tn * BN;
+    double* Cg = C + (int64_t)tm * BM * g.N + tn * BN;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = wm + 16 * i + 4 * v + q, col = wn + 16 * j + l16;
+                if (!EDGE || (row < rows && col < cols)) {
+                    double* p = Cg + (int64_t)row * g.N + col;
+                    *p = *p + acc[i][j][v];
+                }
+            }
+}
+
 template <typename T>
 static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* A, const T* B, T* C) {
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4));
@@ -251,12 +368,32 @@ static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* 
 }
 
 static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
-    if (dtype == NK_F64) return launch_simple<double>(dev, M, K, N, (const double*)A, (const double*)B, (double*)C);
+    static const int64_t mfma_from = [] { const char* v = getenv("NK_MFMA_EDGE_FROM"); return v && *v ? atoll(v) : (int64_t)1 << 24; }();
+    if (dtype == NK_F64) {
+        // from 2^24 multiply-adds on the matrix cores take over (sums re-ordered, within 1e-12 of the reference);
+        // smaller products keep the reference's summation order bit for bit
+        const bool fits = M * K * 8 < ((int64_t)1 << 32) && K * N * 8 < ((int64_t)1 << 32);
+        if (M * K * N >= mfma_from && fits) {
+            const bool whole = (A % 16 == 0) && (B % 16 == 0) && M % BM == 0 && N % BN == 0 && K % d64::DK == 0;
+            MfmaArgs g{};
+            g.M = (int)M; g.K = (int)K; g.N = (int)N;
+            g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
+            g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
+            set_path(whole ? "mfma_f64" : "mfma_f64_edge");
+            if (whole) hipLaunchKernelGGL(matmul_mfma_f64_kernel<false>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
+                                          (const double*)A, (const double*)B, (double*)C);
+            else       hipLaunchKernelGGL(matmul_mfma_f64_kernel<true>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
+                                          (const double*)A, (const double*)B, (double*)C);
+            NK_HIP(hipGetLastError());
+            return NK_OK;
+        }
+        return launch_simple<double>(dev, M, K, N, (const double*)A, (const double*)B, (double*)C);
+    }
     const bool aligned = (A % 16 == 0) && (B % 16 == 0) && (C % 16 == 0);
     const bool whole_tiles = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
     // Small products stay on the simple kernel, which keeps the reference's summation order bit for bit; from
     // 2^24 multiply-adds on, shapes that are not whole tiles take the matrix cores through the edge variant.
-    static const int64_t edge_from = [] { const char* v = getenv("NK_MFMA_EDGE_FROM"); return v && *v ? atoll(v) : (int64_t)1 << 24; }();
+    const int64_t edge_from = mfma_from;
     const bool edge = !whole_tiles && M * K * N >= edge_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
     if (whole_tiles || edge) {
         MfmaArgs g{};

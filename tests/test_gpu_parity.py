@@ -734,6 +734,48 @@ def test_matmul_mfma_edge_path(device, orc, mkn):
     assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("mkn,path", [((256, 256, 256), "mfma_f64"), ((384, 112, 512), "mfma_f64"), ((128, 1024, 128), "mfma_f64"),
+                                      ((300, 257, 270), "mfma_f64_edge"), ((129, 1001, 131), "mfma_f64_edge"),
+                                      ((1000, 33, 1000), "mfma_f64_edge"), ((127, 4097, 40), "mfma_f64_edge"),
+                                      ((255, 255, 250), "simple")])
+def test_matmul_f64_matrix_core_path(device, orc, mkn, path):
+    """f64 products from 2^24 multiply-adds on run on the f64 matrix cores: exact on integer-valued data, within
+    1e-12 norm-wise of the reference's order on uniform data, accumulation into C, both layouts, nothing written
+    or read outside the operands; below the threshold the reference's order is kept bit for bit."""
+    M, K, N = mkn
+    rng = np.random.default_rng(55)
+    say("matmul f64 integer", mkn)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float64); B = rng.integers(-5, 6, (K, N)).astype(np.float64)
+    C0 = rng.integers(-9, 10, (M, N)).astype(np.float64)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path
+    assert (tc.getData().reshape(M, N) == A @ B + C0).all()
+    say("matmul f64 column major", mkn)
+    tc = on(device, np.zeros((M, N), dtype=np.float64))
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+    assert _lib.last_path() == path
+    assert (tc.getData().reshape(N, M).T == A @ B).all()
+    say("matmul f64 uniform, operands inside larger buffers full of NaN", mkn)
+    A = rng.uniform(-1, 1, (M, K)); B = rng.uniform(-1, 1, (K, N))
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = 1e-12 * (np.abs(A) @ np.abs(B))
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float64)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(np.zeros((M, N)))
+    _lib.check(device._lib.nk_matmul(device.handle, 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 8 * pad, pb._data.ptr + 8 * pad, pc._data.ptr + 8 * pad))
+    assert _lib.last_path() == path
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()
+    if path == "simple":
+        assert_bits(got[pad:pad + M * N], ref.reshape(-1), "simple f64")
+    else:
+        assert (np.abs(got[pad:pad + M * N].reshape(M, N) - ref) <= bound).all()
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
