@@ -257,6 +257,18 @@ def main():
         flops("conv_c5_forward", 203212800, 17037632, dev.prepared_launch("convolution", -1, y5, x5, k5))
         flops("conv_c5_grad_input", 203212800, 17037632, dev.prepared_launch("convolution", 0, dx5, k5, e5))
         flops("conv_c5_grad_kernel", 203212800, 17037632, dev.prepared_launch("convolution", 0, dk5, x5, e5))
+        for t in (x5, k5, y5, e5, dx5, dk5): dev.free(t)
+        # the same shapes in f64 take the general kernels (any rank, layout and view)
+        f64 = np.float64
+        x5 = Tensor.of(f64, (64, 256, 256), rng.standard_normal(64 * 256 * 256) * 0.1).to(dev)
+        k5 = Tensor.of(f64, (64, 5, 5), rng.standard_normal(1600) * 0.1).to(dev)
+        y5 = Tensor._on_device(dev, f64, (1, 252, 252))
+        e5 = Tensor.of(f64, (1, 252, 252), rng.standard_normal(252 * 252)).to(dev)
+        dx5 = Tensor._on_device(dev, f64, (64, 256, 256))
+        dk5 = Tensor._on_device(dev, f64, (64, 5, 5))
+        flops("conv_c5_forward_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", -1, y5, x5, k5), f64=True)
+        flops("conv_c5_grad_input_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", 0, dx5, k5, e5), f64=True)
+        flops("conv_c5_grad_kernel_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", 0, dk5, x5, e5), f64=True)
 
     result = {
         "metric": "GB/s & % HBM peak (broadcast/elementwise)",

@@ -10,6 +10,8 @@
 //   literal        any rank / layout / view: one thread per drain element, the sum in the reference's
 //                  order with rounded products, bit-identical to the CPU device.  The gradient only
 //                  visits the e-range that can pass the bounds test (skipped terms add +0).
+//   split          the same terms for few drain elements with long sums (at least 1024 terms, at most 2^18
+//                  elements): a block per element, re-ordered sum.
 //   chan_fwd/dx/dk rank 3, dense row-major f32, full reduction over axis 0 (channels), square taps of extent
 //                  2, 3, 4, 5 or 7: [C,H,W] x [C,k,k] -> [1,H-k+1,W-k+1] and its two gradients, register
 //                  sliding-window kernels (see below); sums are re-ordered, results agree with the reference
@@ -26,14 +28,16 @@ struct ConvArgs {
     Cfg c0, c1, c2;
 };
 
-template <typename T>
+template <typename T, int RANK>
 __global__ __launch_bounds__(256) void conv_fwd_literal(ConvArgs A, T* __restrict__ drn, const T* __restrict__ s1,
                                                         const T* __restrict__ s2) {
     const unsigned step = gridDim.x * blockDim.x;
+    const int rank = RANK ? RANK : A.rank;          // RANK = 0: any rank up to NK_MAX_RANK
+    constexpr int NR = RANK ? RANK : NK_MAX_RANK;
     for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < A.n; i += step) {
-        int o[NK_MAX_RANK], b1[NK_MAX_RANK], b2[NK_MAX_RANK], j[NK_MAX_RANK], m[NK_MAX_RANK];
-        nd_of_flat(A.c0, A.rank, (int)i, o);
-        for (int k = 0; k < A.rank; k++) {
+        int o[NR], b1[NR], b2[NR], j[NR], m[NR];
+        nd_of_flat(A.c0, rank, (int)i, o);
+        for (int k = 0; k < rank; k++) {
             const int e1 = A.c1.shape[k], e2 = A.c2.shape[k];
             b1[k] = e1 >= e2 ? o[k] : 0;
             b2[k] = e1 <= e2 ? o[k] : 0;
@@ -43,30 +47,32 @@ __global__ __launch_bounds__(256) void conv_fwd_literal(ConvArgs A, T* __restric
         T value = T(0);
         bool running = true;
         while (running) {
-            int i1[NK_MAX_RANK], i2[NK_MAX_RANK];
-            for (int k = 0; k < A.rank; k++) { i1[k] = b1[k] + j[k]; i2[k] = b2[k] + j[k]; }
-            T prod = s1[phys_of_nd(A.c1, A.rank, i1)] * s2[phys_of_nd(A.c2, A.rank, i2)];
+            int i1[NR], i2[NR];
+            for (int k = 0; k < rank; k++) { i1[k] = b1[k] + j[k]; i2[k] = b2[k] + j[k]; }
+            T prod = s1[phys_of_nd(A.c1, rank, i1)] * s2[phys_of_nd(A.c2, rank, i2)];
             value = value + prod;
             int k = 0;
-            for (; k < A.rank; k++) {
+            for (; k < rank; k++) {
                 if (++j[k] < m[k]) break;
                 j[k] = 0;
             }
-            running = k < A.rank;
+            running = k < rank;
         }
-        drn[phys_of_nd(A.c0, A.rank, o)] = value;
+        drn[phys_of_nd(A.c0, rank, o)] = value;
     }
 }
 
-template <typename T>
+template <typename T, int RANK>
 __global__ __launch_bounds__(256) void conv_bwd_literal(ConvArgs A, T* __restrict__ drn, const T* __restrict__ s1,
                                                         const T* __restrict__ s2) {
     const unsigned step = gridDim.x * blockDim.x;
+    const int rank = RANK ? RANK : A.rank;          // RANK = 0: any rank up to NK_MAX_RANK
+    constexpr int NR = RANK ? RANK : NK_MAX_RANK;
     for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < A.n; i += step) {
-        int o[NK_MAX_RANK], lo[NK_MAX_RANK], hi[NK_MAX_RANK], e[NK_MAX_RANK];
-        nd_of_flat(A.c0, A.rank, (int)i, o);
+        int o[NR], lo[NR], hi[NR], e[NR];
+        nd_of_flat(A.c0, rank, (int)i, o);
         bool empty = false;
-        for (int k = 0; k < A.rank; k++) {
+        for (int k = 0; k < rank; k++) {
             const int e0 = A.c0.shape[k], e1 = A.c1.shape[k], e2 = A.c2.shape[k];
             if (e0 > e1) {            // i1 = o - e in [0, e1)
                 lo[k] = o[k] - e1 + 1; if (lo[k] < 0) lo[k] = 0;
@@ -81,18 +87,87 @@ __global__ __launch_bounds__(256) void conv_bwd_literal(ConvArgs A, T* __restric
         T value = T(0);
         bool running = !empty;
         while (running) {
-            int i1[NK_MAX_RANK];
-            for (int k = 0; k < A.rank; k++) i1[k] = A.c0.shape[k] > A.c1.shape[k] ? o[k] - e[k] : o[k] + e[k];
-            T prod = s1[phys_of_nd(A.c1, A.rank, i1)] * s2[phys_of_nd(A.c2, A.rank, e)];
+            int i1[NR];
+            for (int k = 0; k < rank; k++) i1[k] = A.c0.shape[k] > A.c1.shape[k] ? o[k] - e[k] : o[k] + e[k];
+            T prod = s1[phys_of_nd(A.c1, rank, i1)] * s2[phys_of_nd(A.c2, rank, e)];
             value = value + prod;
             int k = 0;
-            for (; k < A.rank; k++) {
+            for (; k < rank; k++) {
                 if (++e[k] < hi[k]) break;
                 e[k] = lo[k];
             }
-            running = k < A.rank;
+            running = k < rank;
         }
-        drn[phys_of_nd(A.c0, A.rank, o)] = value;
+        drn[phys_of_nd(A.c0, rank, o)] = value;
+    }
+}
+
+// Long sums into few drain elements (a tap gradient, a full reduction over channels in f64, ...): with one
+// thread per drain element the machine would idle behind a handful of very long serial sums.  Here a block
+// owns a drain element: its 256 threads take every 256th term -- enumerated with the last axis fastest, the
+// order memory runs in for row-major operands -- and their partial sums meet in a fixed LDS tree.  Each thread
+// steps its nd term index by 256 with a mixed-radix add (no division inside the loop).  Same terms as the
+// literal kernels, another order: results agree with the reference norm-wise, not bit for bit.
+template <typename T, bool BWD, int RANK>
+__global__ __launch_bounds__(256) void conv_split(ConvArgs A, T* __restrict__ drn, const T* __restrict__ s1,
+                                                  const T* __restrict__ s2) {
+    __shared__ T part[256];
+    const int tid = threadIdx.x;
+    const int rank = RANK ? RANK : A.rank;          // RANK = 0: any rank up to NK_MAX_RANK
+    constexpr int NR = RANK ? RANK : NK_MAX_RANK;
+    for (unsigned i = blockIdx.x; i < A.n; i += gridDim.x) {
+        int o[NR], lo[NR], ext[NR], b1[NR], j[NR], d[NR];
+        nd_of_flat(A.c0, rank, (int)i, o);
+        unsigned terms = 1;
+        for (int k = 0; k < rank; k++) {
+            const int e0 = A.c0.shape[k], e1 = A.c1.shape[k], e2 = A.c2.shape[k];
+            if (!BWD) {
+                b1[k] = e1 >= e2 ? o[k] : 0;
+                lo[k] = e1 <= e2 ? o[k] : 0;                 // start in src2
+                ext[k] = e1 < e2 ? e1 : e2;
+            } else {
+                int l, h;
+                if (e0 > e1) { l = o[k] - e1 + 1; if (l < 0) l = 0; h = o[k] + 1; if (h > e2) h = e2; }
+                else         { l = 0; h = e1 - o[k]; if (h > e2) h = e2; }
+                lo[k] = l;
+                ext[k] = h > l ? h - l : 0;
+                b1[k] = 0;
+            }
+            terms *= (unsigned)ext[k];
+        }
+        T value = T(0);
+        if (terms) {
+            unsigned r = (unsigned)tid, q = 256u;
+            for (int k = rank - 1; k >= 0; k--) {
+                j[k] = (int)(r % (unsigned)ext[k]); r /= (unsigned)ext[k];
+                d[k] = (int)(q % (unsigned)ext[k]); q /= (unsigned)ext[k];
+            }
+#pragma unroll 4
+            for (unsigned t = (unsigned)tid; t < terms; t += 256u) {
+                int i1[NR], i2[NR];
+                for (int k = 0; k < rank; k++) {
+                    i2[k] = lo[k] + j[k];
+                    if (!BWD) i1[k] = b1[k] + j[k];
+                    else      i1[k] = A.c0.shape[k] > A.c1.shape[k] ? o[k] - i2[k] : o[k] + i2[k];
+                }
+                const T prod = s1[phys_of_nd(A.c1, rank, i1)] * s2[phys_of_nd(A.c2, rank, i2)];
+                value = value + prod;
+                int carry = 0;
+                for (int k = rank - 1; k >= 0; k--) {
+                    j[k] += d[k] + carry;
+                    carry = j[k] >= ext[k];
+                    if (carry) j[k] -= ext[k];
+                }
+            }
+        }
+        part[tid] = value;
+        __syncthreads();
+        for (int w = 128; w > 0; w >>= 1) {
+            if (tid < w) part[tid] = part[tid] + part[tid + w];
+            __syncthreads();
+        }
+        if (tid == 0) drn[phys_of_nd(A.c0, rank, o)] = part[0];
+        __syncthreads();
     }
 }
 
@@ -648,11 +723,39 @@ static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, n
     }
     ConvArgs A{};
     A.rank = rank; A.n = (unsigned)n; A.c0 = c0; A.c1 = c1; A.c2 = c2;
+    // terms of one sum (the gradient's upper bound: all of src2); few long sums go to the kernel that splits them
+    int64_t terms = 1;
+    for (int k = 0; k < rank; k++) terms *= d < 0 ? (c1.shape[k] < c2.shape[k] ? c1.shape[k] : c2.shape[k]) : c2.shape[k];
+    if (d >= 0) {                                  // ... of which only the window that passes the bounds test counts
+        int64_t window = 1;
+        for (int k = 0; k < rank; k++) window *= c1.shape[k] < c2.shape[k] ? c1.shape[k] : c2.shape[k];
+        if (window < terms) terms = window;
+    }
+    if (terms >= 1024 && n <= ((int64_t)1 << 18)) {
+        set_path(d < 0 ? "split_fwd" : "split_bwd");
+        const unsigned grid = (unsigned)n;
+        auto go = [&](auto R) {
+            constexpr int RANK = decltype(R)::value;
+            if (d < 0) hipLaunchKernelGGL((conv_split<T, false, RANK>), dim3(grid), dim3(256), 0, dev->stream, A, out, s1, s2);
+            else       hipLaunchKernelGGL((conv_split<T, true, RANK>), dim3(grid), dim3(256), 0, dev->stream, A, out, s1, s2);
+        };
+        if (rank == 2) go(std::integral_constant<int, 2>{});
+        else if (rank == 3) go(std::integral_constant<int, 3>{});
+        else go(std::integral_constant<int, 0>{});
+        NK_HIP(hipGetLastError());
+        return NK_OK;
+    }
     unsigned blocks = (unsigned)((n + 255) / 256);
     if (blocks > 65536) blocks = 65536;
     set_path(d < 0 ? "literal_fwd" : "literal_bwd");
-    if (d < 0) hipLaunchKernelGGL(conv_fwd_literal<T>, dim3(blocks), dim3(256), 0, dev->stream, A, out, s1, s2);
-    else       hipLaunchKernelGGL(conv_bwd_literal<T>, dim3(blocks), dim3(256), 0, dev->stream, A, out, s1, s2);
+    auto go = [&](auto R) {
+        constexpr int RANK = decltype(R)::value;
+        if (d < 0) hipLaunchKernelGGL((conv_fwd_literal<T, RANK>), dim3(blocks), dim3(256), 0, dev->stream, A, out, s1, s2);
+        else       hipLaunchKernelGGL((conv_bwd_literal<T, RANK>), dim3(blocks), dim3(256), 0, dev->stream, A, out, s1, s2);
+    };
+    if (rank == 2) go(std::integral_constant<int, 2>{});
+    else if (rank == 3) go(std::integral_constant<int, 3>{});
+    else go(std::integral_constant<int, 0>{});
     NK_HIP(hipGetLastError());
     return NK_OK;
 }

@@ -630,6 +630,60 @@ def test_channel_convolution_fast_paths(device, orc, shape):
     assert (np.abs(dk.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dk"
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("shape", [([48, 40, 44], [48, 5, 5]), ([200, 20, 21], [200, 4, 2]), ([4, 60, 70], [4, 4, 2]),
+                                   ([80, 90], [40, 45]), ([30, 1100, 1], [1, 1100, 20]), ([2, 3, 44, 34], [2, 3, 6, 5])])
+def test_convolution_split_sums(device, orc, shape, dt):
+    """Few drain elements with sums of 1024 terms or more: a block per element adds the reference's terms in another
+    order.  Norm-wise |delta| <= tol * sum|a||b| per output (tol 1e-5 / 1e-12), exact on integer-valued data; every
+    rank, both gradient branches, and a transposed operand."""
+    xs, ks = shape
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    ys = [abs(p - q) + 1 for p, q in zip(xs, ks)]
+    rng = np.random.default_rng(44)
+    seen = set()
+    for integer in (True, False):
+        draw = (lambda sh: rng.integers(-3, 4, sh).astype(T)) if integer else (lambda sh: rng.uniform(-1, 1, sh).astype(T))
+        x, k, e = draw(xs), draw(ks), draw(ys)
+        tx, tk, te = on(device, x), on(device, k), on(device, e)
+        say("conv split fwd", xs, ks, dt, "integer" if integer else "uniform")
+        out = Tensor._on_device(device, T, ys)
+        device.launch_convolution(-1, out, tx, tk)
+        seen.add(_lib.last_path())
+        want = orc.convolve(np.zeros(out.size, dtype=T), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
+        if integer:
+            assert_bits(out.getData(), want, "fwd on integers")
+        else:
+            assert (np.abs(out.getData().astype(np.float64) - want) <= tol * _abs_bound(orc, xs, ks, x, k, T) + 1e-30).all()
+        for name, tgt_shape, other, other_arr, other_shape in (("dx", xs, tk, k, ks), ("dk", ks, tx, x, xs)):
+            say("conv split", name, xs, ks, dt)
+            drn = Tensor._on_device(device, T, tgt_shape)
+            device.launch_convolution(0, drn, other, te)
+            seen.add(_lib.last_path())
+            want = orc.deconvolve(np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt_shape), other_arr.reshape(-1), orc.dense_cfg(other_shape), e.reshape(-1), orc.dense_cfg(ys), fast=True)
+            if integer:
+                assert_bits(drn.getData(), want, name + " on integers")
+            else:
+                babs = orc.deconvolve(np.zeros(drn.size), orc.dense_cfg(tgt_shape), np.abs(other_arr).astype(np.float64).reshape(-1), orc.dense_cfg(other_shape),
+                                      np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
+                assert (np.abs(drn.getData().astype(np.float64) - want) <= tol * babs + 1e-30).all(), name
+    if dt == "f32" and ks == [48, 5, 5]:
+        assert seen == {"chan_fwd", "chan_dx", "chan_dk"}, seen          # the register-window kernels take dense f32 square taps
+    else:
+        assert seen & {"split_fwd", "split_bwd"}, seen
+    if len(xs) == 2:
+        say("conv split on a transposed operand", dt)
+        x = rng.integers(-3, 4, (xs[1], xs[0])).astype(T)
+        vx = on(device, x).T()                                         # shape xs, strides (1, xs[0])
+        e = rng.integers(-3, 4, ys).astype(T)
+        dk = Tensor._on_device(device, T, ks)
+        device.launch_convolution(0, dk, vx, on(device, e))
+        assert _lib.last_path() == "split_bwd"
+        want = orc.deconvolve(np.zeros(dk.size, dtype=T), orc.dense_cfg(ks), x.reshape(-1), cfg(vx), e.reshape(-1), orc.dense_cfg(ys))
+        assert_bits(dk.getData(), want, "transposed operand")
+
+
 def test_conv2d_config1_shape(device, orc):
     """[64,64] x [3,3] -> [62,62] (the reference runs this on SimpleCPUConvolution: ky outer, kx inner)."""
     say("conv2d 64x64 x 3x3")
