@@ -211,6 +211,12 @@ def main():
         hbm("max_index_2^26", 4 * n, dev.prepared("nk_reduce_index", dev.handle, 1, 0, srcs[0]._data.ptr, n, slot.ptr))
         hbm("dot_2^26", 8 * n, dev.prepared("nk_dot", dev.handle, 0, srcs[0]._data.ptr, srcs[1]._data.ptr, n, one._data.ptr))
         dev.free(one); slot.release()
+        # integer scalarization of 2^26 int32 elements
+        i_src = Tensor.of(np.int32, (n,), rng.integers(-2**31, 2**31 - 1, n, dtype=np.int32)).to(dev)
+        i_out = Tensor._on_device(dev, np.int32, (n,))
+        hbm("scalarization_int32_multiply", 8 * n, dev.prepared_launch("scalarization_int", "multiply", -1, i_out, i_src, 3))
+        hbm("scalarization_int32_divide", 8 * n, dev.prepared_launch("scalarization_int", "divide", -1, i_out, i_src, 7))
+        dev.free(i_src); dev.free(i_out)
         # permuted [4096,16384] views of row-major [16384,4096]
         from neureka_amd import NDConfiguration
         pv = []

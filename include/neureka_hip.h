@@ -38,7 +38,8 @@ typedef uint64_t nk_buf;
 
 #define NK_MAX_RANK 8
 
-enum { NK_F32 = 0, NK_F64 = 1 };
+enum { NK_F32 = 0, NK_F64 = 1,
+       NK_I32 = 2, NK_I64 = 3, NK_I16 = 4, NK_I8 = 5 };   /* integer types: nk_scalarization_int only */
 
 /* status codes besides hipError_t values */
 enum {
@@ -124,6 +125,18 @@ int nk_elementwise(nk_dev dev, int op_id, int d, int dtype, int rank,
 int nk_scalarization(nk_dev dev, int op_id, int d, int dtype, int rank,
                      nk_buf drn, const int32_t* drn_cfg, nk_buf src, const int32_t* src_cfg,
                      double value, int64_t n);
+
+/* scalarization_<op>_<type> for type in {int, long, short, char}: the integer kernels that
+ * J/backend/main/implementations/broadcast/CLScalarBroadcast.java:40-58 generates beside float and double.
+ * dtype is one of NK_I32, NK_I64, NK_I16, NK_I8; value is narrowed to it (Number.intValue() ...).  The arithmetic
+ * is the CPU device's: J/backend/main/implementations/broadcast/CPUScalarBroadcast.java:83-190 with the operator
+ * classes beside it and the defaults of J/backend/main/implementations/fun/api/CPUBiFun.java:9-27 -- int and long
+ * wrap and truncate like Java, short and byte are evaluated in double and narrowed with Math.round.  A zero
+ * divisor of a forward int or long division or modulo is an argument error ("/ by zero", the CPU device's
+ * ArithmeticException).  d < 0: drain = src op value; d = 0 / 1: derivative by the element / by the value. */
+int nk_scalarization_int(nk_dev dev, int op_id, int d, int dtype, int rank,
+                         nk_buf drn, const int32_t* drn_cfg, nk_buf src, const int32_t* src_cfg,
+                         int64_t value, int64_t n);
 
 /* scalar_broadcast: K/scalar_broadcast.cl:12-23, launched by
  * J/backend/main/algorithms/ScalarBroadcast.java:65-81.  drain[i] = value through the drain's view. */

@@ -423,7 +423,8 @@ def hip_broadcast(op: str):
 def hip_scalar_broadcast(op: str):
     """CLScalarBroadcast<Op>.run (e.g. implementations/broadcast/CLScalarBroadcastAddition.java:15-34)."""
     def run(call: ExecutionCall):
-        value = float(call.input(2).item(0))
+        value = call.input(2).item(0)
+        value = int(value) if np.issubdtype(call.input(0).dtype, np.integer) else float(value)
         call.device.launch_scalarization(op, call.derivIdx, call.input(0), call.input(1), value)
         return call.input(0)
     return run

@@ -16,13 +16,16 @@ from . import _lib
 from .ndim import IllegalArgumentException, IllegalStateException, NDConfiguration
 
 
+_INT_CODES = {np.dtype(np.int32): 2, np.dtype(np.int64): 3, np.dtype(np.int16): 4, np.dtype(np.int8): 5}
+
+
 def _dtype_code(dtype) -> int:
     dt = np.dtype(dtype)
     if dt == np.float32:
         return _lib.F32
     if dt == np.float64:
         return _lib.F64
-    raise IllegalArgumentException(f"HipDevice computes in float32 and float64, not {dt}")
+    raise IllegalArgumentException(f"HipDevice computes in float32 and float64 (integer types: scalar broadcast only), not {dt}")
 
 
 class HipData:
@@ -327,8 +330,15 @@ class HipDevice:
         (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = self._ops(drn, a, b)
         _lib.check(self._lib.nk_elementwise(self.handle, _lib.OP[op], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, drn.ndc.size))
 
-    def launch_scalarization(self, op: str, d: int, drn, src, value: float) -> None:
+    def launch_scalarization(self, op: str, d: int, drn, src, value) -> None:
         (p0, k0, c0), (p1, k1, c1) = self._ops(drn, src)
+        if drn.dtype in _INT_CODES:              # CLScalarBroadcast's "int", "long", "short", "char" kernels
+            if src.dtype != drn.dtype:
+                raise IllegalArgumentException(f"scalarization of {src.dtype} data into a {drn.dtype} drain")
+            wrapped = (int(value) + (1 << 63)) % (1 << 64) - (1 << 63)
+            _lib.check(self._lib.nk_scalarization_int(self.handle, _lib.OP[op], d, _INT_CODES[drn.dtype], drn.ndc.rank, p0, c0, p1, c1,
+                                                      wrapped, drn.ndc.size))
+            return
         _lib.check(self._lib.nk_scalarization(self.handle, _lib.OP[op], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, float(value), drn.ndc.size))
 
     def launch_scalar_fill(self, drn, value: float) -> None:
@@ -387,7 +397,7 @@ class HipDevice:
 
     def prepared_launch(self, kind: str, *a):
         """kind: 'broadcast' | 'elementwise' (op, d, drn, x, y) | 'activation' (fun, d, drn, x) |
-        'fused' (program, consts, drn, srcs) | 'convolution' (d, drn, x, y) | 'matmul' (row_major, M, K, N, x, y, z)"""
+        'scalarization_int' (op, d, drn, x, value) | 'fused' (program, consts, drn, srcs) | 'convolution' (d, drn, x, y) | 'matmul' (row_major, M, K, N, x, y, z)"""
         h = C.c_uint64(self.handle)
         if kind in ("broadcast", "elementwise"):
             op, d, drn, x, y = a
@@ -397,6 +407,11 @@ class HipDevice:
             fun, d, drn, x = a
             (p0, k0, c0), (p1, k1, c1) = ops = self._ops(drn, x)
             call = self.prepared("nk_activation", h, _lib.FUN[fun], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, C.c_int64(drn.ndc.size))
+        elif kind == "scalarization_int":
+            op, d, drn, x, value = a
+            (p0, k0, c0), (p1, k1, c1) = ops = self._ops(drn, x)
+            call = self.prepared("nk_scalarization_int", h, _lib.OP[op], d, _INT_CODES[drn.dtype], drn.ndc.rank, p0, c0, p1, c1,
+                                 C.c_int64(int(value)), C.c_int64(drn.ndc.size))
         elif kind == "convolution":
             d, drn, x, y = a
             (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = ops = self._ops(drn, x, y)

@@ -219,7 +219,7 @@ class Tensor:
     def _bin(self, op: str, other) -> "Tensor":
         from .function import execute
         if not isinstance(other, Tensor):
-            other = Tensor.of(self.dtype, (1,), float(other))
+            other = Tensor.of(self.dtype, (1,), int(other) if np.issubdtype(self.dtype, np.integer) else float(other))
         return execute(op, [self, other])
 
     def plus(self, o): return self._bin("add", o)

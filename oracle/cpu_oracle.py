@@ -62,6 +62,8 @@ def lib() -> C.CDLL:
         l.orc_reduce_index.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int]
         l.orc_dot.restype = C.c_double
         l.orc_dot.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int]
+        l.orc_scalarization_int.restype = C.c_int
+        l.orc_scalarization_int.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_int]
         l.orc_simple_conv2d.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = l
     return _lib
@@ -136,6 +138,26 @@ def elementwise(op: str, d: int, drn, drn_cfg, a, a_cfg, b, b_cfg, **kw):
 
 def scalarization(op: str, d: int, drn, drn_cfg, src, src_cfg, value: float, **kw):
     return run("scalarization", OP[op], d, drn, drn_cfg, src, src_cfg, value=value, **kw)
+
+
+ITYPE = {np.dtype(np.int32): 2, np.dtype(np.int64): 3, np.dtype(np.int16): 4, np.dtype(np.int8): 5}
+
+
+class JavaArithmeticException(ArithmeticError):
+    """Where the CPU device throws java.lang.ArithmeticException (integer division by zero)."""
+
+
+def scalarization_int(op: str, d: int, drn: np.ndarray, drn_cfg, src: np.ndarray, src_cfg, value: int) -> np.ndarray:
+    """CPUScalarBroadcast on int32 / int64 / int16 / int8 data; `value` is narrowed to the element type."""
+    drn_cfg, src_cfg = _cfg(drn_cfg), _cfg(src_cfg)
+    assert drn.dtype == src.dtype and drn.dtype in ITYPE
+    value = int(value)
+    value = (value + (1 << 63)) % (1 << 64) - (1 << 63)
+    thrown = lib().orc_scalarization_int(ITYPE[drn.dtype], OP[op], d, len(drn_cfg) // 5, _p(drn), _p(drn_cfg), _p(src), _p(src_cfg),
+                                         value, 0, _size(drn_cfg))
+    if thrown:
+        raise JavaArithmeticException("/ by zero")
+    return drn
 
 
 def scalar_fill(drn, drn_cfg, value: float):

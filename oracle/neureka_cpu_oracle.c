@@ -348,6 +348,106 @@ void orc_scalarization(int op, int d, int is_f64, int rank, void* drn, const int
     }
 }
 
+/* ---- integer scalarization --------------------------------------------------------------------------------
+ * java.lang.Math.round(double): "the closest long to the argument, with ties rounding to positive infinity";
+ * NaN -> 0, at or beyond the ends of long -> Long.MIN_VALUE / Long.MAX_VALUE. */
+static int64_t java_math_round(double a) {
+    if (isnan(a)) return 0;
+    if (a <= -9223372036854775808.0) return INT64_MIN;
+    if (a >= 9223372036854775807.0) return INT64_MAX;
+    double below = floor(a);
+    if (a - below < 0.5) return (int64_t)below;       /* the difference is exact */
+    return (int64_t)below + 1;
+}
+/* Java's narrowing primitive conversions (JLS 5.1.3) keep the low-order bits */
+static int32_t to_int(int64_t v) { return (int32_t)(uint32_t)(uint64_t)v; }
+static int16_t to_short(int64_t v) { return (int16_t)(uint16_t)(uint64_t)v; }
+static int8_t to_byte(int64_t v) { return (int8_t)(uint8_t)(uint64_t)v; }
+static int32_t int_neg(int32_t a) { return (int32_t)(0u - (uint32_t)a); }
+static int64_t long_neg(int64_t a) { return (int64_t)(0ull - (uint64_t)a); }
+
+/* the double overloads of the seven operator classes (family "scalar broadcast"): function, deriveAt0, deriveAt1.
+ * CPUScalarBroadcastAddition.java, ...Subtraction, ...Multiplication, ...Division, ...Modulo, ...Identity,
+ * CPUScalaBroadcastPower.java */
+static double scalar_fun_f64(int op, int d, double a, double b) {
+    switch (op) {
+        case 0: return d < 0 ? a + b : 1;
+        case 1: return d < 0 ? a - b : (d == 0 ? 1 : -1);
+        case 2: return d < 0 ? a * b : (d == 0 ? b : a);
+        case 3: return d < 0 ? a / b : (d == 0 ? 1 / b : -(a / pow(b, 2)));
+        case 4: return d < 0 ? fmod(a, b) : (d == 0 ? 1 / b : -(a / pow(b, 2)));
+        case 5: return d < 0 ? pow(a, b) : (d == 0 ? b * pow(a, b - 1) : pow(a, b) * log(a));
+        default: return b;
+    }
+}
+/* invoke(int, int) of the same classes; returns 0 and sets *div_by_zero where Java throws ArithmeticException */
+static int32_t scalar_fun_i32(int op, int d, int32_t a, int32_t b, int* div_by_zero) {
+    switch (op) {
+        case 0: return d < 0 ? (int32_t)((uint32_t)a + (uint32_t)b) : 1;
+        case 1: return d < 0 ? (int32_t)((uint32_t)a - (uint32_t)b) : (d == 0 ? 1 : -1);
+        case 2: return d < 0 ? (int32_t)((uint32_t)a * (uint32_t)b) : (d == 0 ? b : a);
+        case 3: case 4:
+            if (d < 0) {
+                if (b == 0) { *div_by_zero = 1; return 0; }
+                if (b == -1) return op == 3 ? int_neg(a) : 0;          /* JLS 15.17.2: MIN_VALUE / -1 overflows to MIN_VALUE */
+                return op == 3 ? a / b : a % b;
+            }
+            if (d == 0) return to_int(java_math_round(1.0 / b));
+            return to_int(java_math_round(int_neg(a) / pow(b, 2)));
+        case 5:
+            if (d < 0) return to_int(java_math_round(pow(a, b)));
+            if (d == 0) return to_int(java_math_round(b * pow(a, (int32_t)((uint32_t)b - 1u))));
+            return to_int(java_math_round(pow(a, b) * log(a)));
+        default: return b;
+    }
+}
+static int64_t scalar_fun_i64(int op, int d, int64_t a, int64_t b, int* div_by_zero) {
+    switch (op) {
+        case 0: return d < 0 ? (int64_t)((uint64_t)a + (uint64_t)b) : 1;
+        case 1: return d < 0 ? (int64_t)((uint64_t)a - (uint64_t)b) : (d == 0 ? 1 : -1);
+        case 2: return d < 0 ? (int64_t)((uint64_t)a * (uint64_t)b) : (d == 0 ? b : a);
+        case 3: case 4:
+            if (d < 0) {
+                if (b == 0) { *div_by_zero = 1; return 0; }
+                if (b == -1) return op == 3 ? long_neg(a) : 0;
+                return op == 3 ? a / b : a % b;
+            }
+            if (d == 0) return java_math_round(1.0 / (double)b);
+            return java_math_round((double)long_neg(a) / pow((double)b, 2));
+        case 5:
+            if (d < 0) return java_math_round(pow((double)a, (double)b));
+            if (d == 0) return java_math_round((double)b * pow((double)a, (double)(int64_t)((uint64_t)b - 1ull)));
+            return java_math_round(pow((double)a, (double)b) * log((double)a));
+        default: return b;
+    }
+}
+
+/* CPUScalarBroadcast._workloadFor for Integer / Long / Short / Byte (CPUScalarBroadcast.java:83-162).  Short has no
+ * overload in any operator class and Byte only Identity's, so both run CPUBiFun's defaults (CPUBiFun.java:21-27):
+ * (short) Math.round(invoke((double) a, (double) b)).  itype: 2 int, 3 long, 4 short, 5 byte.
+ * Returns 1 where the CPU device throws ArithmeticException (nothing defined is written from there on). */
+int orc_scalarization_int(int itype, int op, int d, int rank, void* drn, const int32_t* drn_cfg, const void* src,
+                          const int32_t* src_cfg, int64_t number, int start, int end) {
+    view_t v0 = view_of(drn_cfg, rank), v1 = view_of(src_cfg, rank);
+    int i0[ORC_MAX_RANK], i1[ORC_MAX_RANK];
+    int thrown = 0;
+    indices_of_index(&v0, start, i0);
+    indices_of_index(&v1, start, i1);
+    for (int i = start; i < end && !thrown; i++) {
+        int to = index_of_indices(&v0, i0), from = index_of_indices(&v1, i1);
+        switch (itype) {
+            case 2: ((int32_t*)drn)[to] = scalar_fun_i32(op, d, ((const int32_t*)src)[from], to_int(number), &thrown); break;
+            case 3: ((int64_t*)drn)[to] = scalar_fun_i64(op, d, ((const int64_t*)src)[from], number, &thrown); break;
+            case 4: ((int16_t*)drn)[to] = to_short(java_math_round(scalar_fun_f64(op, d, ((const int16_t*)src)[from], to_short(number)))); break;
+            default: ((int8_t*)drn)[to] = op == 6 ? to_byte(number)
+                                                  : to_byte(java_math_round(scalar_fun_f64(op, d, ((const int8_t*)src)[from], to_byte(number)))); break;
+        }
+        increment(i0, v0.shape, rank);
+        increment(i1, v1.shape, rank);
+    }
+    return thrown;
+}
+
 /* CPUScalarBroadcastFunction (J/backend/main/implementations/scalar/CPUScalarBroadcastFunction.java:18-132):
  * drain[i] = value through the drain's view */
 void orc_scalar_fill(int is_f64, int rank, void* drn, const int32_t* drn_cfg, double value, int start, int end) {

@@ -696,6 +696,62 @@ def test_conv2d_config1_shape(device, orc):
     assert_bits(y.items, want, "SimpleCPUConvolution order")
 
 
+# ---- integer scalarization ----------------------------------------------------------------------------------------
+INT_OPS = ["add", "subtract", "multiply", "divide", "modulo", "power", "idy"]
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.int16, np.int8])
+def test_integer_scalarization_bit_exact(device, orc, golden, dt):
+    """drain = src op value on int / long / short / byte data: every operator, the function and both derivatives,
+    dense data (16-byte path with a ragged tail) and views, against the oracle's Java arithmetic."""
+    rng = np.random.default_rng(81)
+    info = np.iinfo(dt)
+    n = 4099
+    edge = np.array([info.min, info.max, 0, 1, -1, 2, -2, 7, -7, info.min + 1], dtype=dt)
+    small = rng.integers(-9, 10, n, dtype=dt)                                  # keeps powers in range
+    wide = np.concatenate([edge, rng.integers(info.min, info.max, n - edge.size, dtype=dt, endpoint=True)])
+    for op in INT_OPS:
+        for d in (-1, 0, 1):
+            for value in ((3, -2, 0) if op == "power" else (3, -7, 1, -1, 0, int(info.max), int(info.min))):
+                data = small if op == "power" else wide
+                if value == 0 and d < 0 and op in ("divide", "modulo") and dt in (np.int32, np.int64):
+                    say("int scalarization / by zero", dt.__name__, op)
+                    with pytest.raises(Exception, match="by zero"):
+                        device.launch_scalarization(op, d, Tensor._on_device(device, dt, (n,)), on(device, data), value)
+                    with pytest.raises(orc.JavaArithmeticException):
+                        orc.scalarization_int(op, d, np.zeros_like(data), orc.dense_cfg([n]), data, orc.dense_cfg([n]), value)
+                    continue
+                out = Tensor._on_device(device, dt, (n,))
+                device.launch_scalarization(op, d, out, on(device, data), value)
+                assert _lib.last_path() == "int_flat"
+                want = orc.scalarization_int(op, d, np.zeros_like(data), orc.dense_cfg([n]), data, orc.dense_cfg([n]), value)
+                got = out.getData()
+                assert (got == want).all(), (dt.__name__, op, d, value, data[got != want][:5], got[got != want][:5], want[got != want][:5])
+    say("int scalarization on views", dt.__name__)
+    parent = on(device, rng.integers(-100, 100, (40, 66), dtype=dt))
+    src = parent[1:39:2, 3:63:3].T()                                           # [20,19] -> transposed [20? ...]
+    out_parent = on(device, np.zeros((30, 30), dtype=dt))
+    drn = out_parent[2:2 + src.shape[0], 5:5 + src.shape[1]]
+    before = out_parent.getData().copy()
+    for op, value in (("multiply", 5), ("subtract", -3), ("divide", 4)):
+        device.launch_scalarization(op, -1, drn, src, value)
+        assert _lib.last_path() == "int_indexed"
+        want = orc.scalarization_int(op, -1, before.copy(), cfg(drn), parent.getData(), cfg(src), value)
+        assert (out_parent.getData() == want).all(), (dt.__name__, op)
+    if dt == np.int32:
+        say("Tensor_Operation_Spec integer rows on the device")
+        g = golden["int_scalarization"]
+        i0 = on(device, np.array(g["tempeh_i0_recovered"], dtype=np.int32), (2, 3))
+        times10 = i0 * 10
+        assert (np.abs(times10.items) == np.abs(np.array(g["tempeh_i0_recovered"], dtype=np.int32) * np.int32(10))).all()
+        assert (on(device, np.abs(times10.items), (2, 3)) % 3).items.tolist() == g["tempeh_abs_i0_times_10_mod_3"]
+    if dt in (np.int32, np.int64):
+        s = golden["int_scalarization"]["scalar_broadcast_add"]
+        a = on(device, np.array(s["a"], dtype=dt), (3, 2))
+        b = on(device, np.array([s["b"]], dtype=dt), (1, 1))
+        assert (a + b).items.tolist() == s["c"]                                   # 'Scalar broadcasting works across devices'
+
+
 # ---- matmul ---------------------------------------------------------------------------------------------------
 def test_matmul_hash_known_answers_on_device(device, golden):
     g = golden["matmul_hashes"]

@@ -419,3 +419,92 @@ def test_dot_reproduces_the_dot_product_spec(golden, orc):
         s[i % 4] = s[i % 4] + a[i] * b[i]
     s[0] = s[0] + a[1000] * b[1000]
     assert orc.dot(a, b) == ((s[0] + s[1]) + s[2]) + s[3]
+
+
+# ---- integer scalarization (CPUScalarBroadcast on Integer / Long / Short / Byte) ---------------------------------
+def _iscal(orc, op, d, data, value, dtype):
+    src = np.asarray(data, dtype=dtype)
+    cfg = orc.dense_cfg([src.size])
+    return orc.scalarization_int(op, d, np.zeros_like(src), cfg, src, cfg, value)
+
+
+def test_int_scalarization_reproduces_the_integer_rows_of_the_operation_spec(golden, orc):
+    """Tensor_Operation_Spec.groovy:560-636, Integer rows: 'abs(i0*10)%3', 'relu(-i0-5)+i0*3' and 'relu(-i0)+i0' on
+    the tensor seeded with "Tempeh".  The tensor itself follows from two more rows of the same table
+    (relu(i0) and relu(i0)-i0); relu on Integer is CPUFun's default, (int) Math.round(relu((double) x))."""
+    g = golden["int_scalarization"]
+    i0 = np.array(g["tempeh_i0_recovered"], dtype=np.int32)
+
+    def relu(x):
+        return np.where(x >= 0, x, np.floor(x.astype(np.float64) * .01 + 0.5).astype(np.int64)).astype(np.int32)
+    assert relu(i0).tolist() == g["tempeh_relu_i0"]
+    times10 = _iscal(orc, "multiply", -1, i0, 10, np.int32)                      # wraps
+    assert _iscal(orc, "modulo", -1, np.abs(times10), 3, np.int32).tolist() == g["tempeh_abs_i0_times_10_mod_3"]
+    neg = (-i0.astype(np.int64)).astype(np.int32)
+    with np.errstate(over="ignore"):
+        got = relu(_iscal(orc, "subtract", -1, neg, 5, np.int32)) + _iscal(orc, "multiply", -1, i0, 3, np.int32)
+        assert got.tolist() == g["tempeh_relu_neg_i0_minus_5_plus_i0_times_3"]
+        assert (relu(neg) + i0).tolist() == g["tempeh_relu_neg_i0_plus_i0"]
+    s = g["scalar_broadcast_add"]
+    for dt in (np.int32, np.int64):
+        assert _iscal(orc, "add", -1, s["a"], s["b"], dt).tolist() == s["c"]
+
+
+def test_int_scalarization_follows_the_java_language_rules(orc):
+    """Known answers worked out by hand from the Java Language Specification (15.17 integer division and remainder,
+    5.1.3 narrowing) and the contract of Math.round (ties towards positive infinity, NaN -> 0, saturation)."""
+    i32, i64, i16, i8 = np.int32, np.int64, np.int16, np.int8
+    IMIN, IMAX, LMIN, LMAX = -2**31, 2**31 - 1, -2**63, 2**63 - 1
+    rows = [
+        # int: integer overloads
+        (i32, "add", -1, [IMAX, 5], 1, [IMIN, 6]), (i32, "subtract", -1, [IMIN], 1, [IMAX]), (i32, "multiply", -1, [IMAX, -3], 2, [-2, -6]),
+        (i32, "divide", -1, [7, -7, IMIN], 2, [3, -3, -2**30]), (i32, "divide", -1, [IMIN, 5], -1, [IMIN, -5]),
+        (i32, "modulo", -1, [-7, 7, 6], 3, [-1, 1, 0]), (i32, "modulo", -1, [7, -7], -3, [1, -1]), (i32, "modulo", -1, [IMIN], -1, [0]),
+        (i32, "power", -1, [10], 10, [1410065408]), (i32, "power", -1, [-2, 0, 3], 3, [-8, 0, 27]), (i32, "power", -1, [2, -2, 4], -1, [1, 0, 0]),
+        (i32, "power", -1, [0, 7], 0, [1, 1]), (i32, "idy", -1, [4, 5], 9, [9, 9]),
+        (i32, "add", 0, [3], 4, [1]), (i32, "add", 1, [3], 4, [1]), (i32, "subtract", 0, [3], 4, [1]), (i32, "subtract", 1, [3], 4, [-1]),
+        (i32, "multiply", 0, [3], 4, [4]), (i32, "multiply", 1, [3], 4, [3]),
+        (i32, "divide", 0, [9], 2, [1]), (i32, "divide", 0, [9], -2, [0]), (i32, "divide", 0, [9], 3, [0]), (i32, "divide", 0, [9], 0, [-1]),
+        (i32, "divide", 1, [7, -7, 5, 6], 2, [-2, 2, -1, -1]), (i32, "modulo", 0, [9], 1, [1]), (i32, "modulo", 1, [8], 2, [-2]),
+        (i32, "power", 0, [3], 2, [6]), (i32, "power", 0, [2], 0, [0]), (i32, "power", 1, [2], 3, [6]), (i32, "power", 1, [-2, 0], 2, [0, 0]),
+        (i32, "power", 1, [0], 0, [0]),
+        # long
+        (i64, "add", -1, [LMAX], 1, [LMIN]), (i64, "multiply", -1, [2**62], 2, [LMIN]), (i64, "divide", -1, [LMIN, -9], -1, [LMIN, 9]),
+        (i64, "divide", -1, [-9, 9], 2, [-4, 4]), (i64, "modulo", -1, [-9, LMIN], -1, [0, 0]), (i64, "power", -1, [3], 40, [LMAX]),
+        (i64, "power", -1, [2, 10], 18, [2**18, 10**18]), (i64, "power", -1, [2], 62, [2**62]), (i64, "divide", 0, [1], 0, [LMAX]),
+        (i64, "divide", 1, [7], 2, [-2]), (i64, "power", 1, [0], 0, [LMIN]),
+        # short: no overloads, everything through double and (short) Math.round
+        (i16, "divide", -1, [7, -7, 1, -1, 0], 2, [4, -3, 1, 0, 0]), (i16, "divide", -1, [7, -7, 0], 0, [-1, 0, 0]),
+        (i16, "modulo", -1, [-7, 7], 3, [-1, 1]), (i16, "modulo", -1, [7], 0, [0]), (i16, "multiply", -1, [300], 300, [24464]),
+        (i16, "add", -1, [32767], 1, [-32768]), (i16, "power", -1, [2], 15, [-32768]), (i16, "power", -1, [2], 16, [0]),
+        (i16, "divide", 0, [5], 2, [1]), (i16, "divide", 1, [6], 2, [-1]), (i16, "idy", -1, [1], 70000, [4464]),
+        # byte
+        (i8, "add", -1, [100], 100, [-56]), (i8, "multiply", -1, [90], 2, [-76]), (i8, "divide", -1, [7], 2, [4]), (i8, "subtract", -1, [-128], 1, [127]),
+        (i8, "idy", -1, [0], 300, [44]), (i8, "power", 1, [2], 3, [6]),
+    ]
+    for dt, op, d, data, value, want in rows:
+        assert _iscal(orc, op, d, data, value, dt).tolist() == want, (dt.__name__, op, d, data, value)
+    for dt in (i32, i64):
+        for op in ("divide", "modulo"):
+            with pytest.raises(orc.JavaArithmeticException):
+                _iscal(orc, op, -1, [1, 2], 0, dt)
+
+
+def test_int_scalarization_matches_exact_integer_arithmetic_and_views(orc):
+    """Random data against Python's exact integers (wrapped), through a strided source view into a permuted drain."""
+    rng = np.random.default_rng(77)
+    for dt, bits in ((np.int32, 32), (np.int64, 64)):
+        lo, hi = -2**(bits - 1), 2**(bits - 1) - 1
+        data = rng.integers(lo, hi, 500, dtype=dt, endpoint=True)
+        wrap = lambda v: (v - lo) % 2**bits + lo
+        for value in (3, -7, hi, lo + 1):
+            for op, f in (("add", lambda a, b: a + b), ("subtract", lambda a, b: a - b), ("multiply", lambda a, b: a * b),
+                          ("divide", lambda a, b: abs(a) // abs(b) * (1 if (a < 0) == (b < 0) else -1)),
+                          ("modulo", lambda a, b: (abs(a) % abs(b)) * (-1 if a < 0 else 1))):
+                want = [wrap(f(int(a), value)) for a in data]
+                assert _iscal(orc, op, -1, data, value, dt).tolist() == want, (dt.__name__, op, value)
+    base = np.arange(4 * 6, dtype=np.int16)
+    src_cfg = [3, 3, 6, 1, 3, 1, 0, 1, 1, 2]                     # shape | strides | indicesMap | offset | spread: rows 0..2, columns 1, 3, 5
+    drn_cfg = [3, 3, 1, 3, 3, 1, 0, 0, 1, 1]                     # column-major strides
+    out = orc.scalarization_int("multiply", -1, np.zeros(9, dtype=np.int16), drn_cfg, base, src_cfg, 5)
+    assert out.reshape(3, 3).T.tolist() == (base.reshape(4, 6)[0:3, 1::2] * 5).tolist()
