@@ -13,22 +13,6 @@ namespace nk {
 int broadcast_forward(nk_dev dev, int op_id, int dtype, int rank, nk_buf drn, const int32_t* drn_cfg,
                       nk_buf a, const int32_t* a_cfg, nk_buf b, const int32_t* b_cfg, int64_t n);
 
-// CPUBroadcast<Op>.java _getDeriveAt0 / _getDeriveAt1 (these differ from the same-shape elementwise
-// derivatives: the backward of + and - adds the operands because src1 is a zero tensor there).
-template <typename T>
-__device__ __forceinline__ T bcast_derive(int op, int d, T a, T b) {
-    using N = Num<T>;
-    switch (op) {
-        case NK_OP_ADD: return a + b;
-        case NK_OP_SUB: return d == 0 ? a + b : a - b;
-        case NK_OP_MUL: return d == 0 ? b : a;
-        case NK_OP_DIV:
-        case NK_OP_MOD: return d == 0 ? T(1) / b : ddiv_db_ref(a, b);
-        case NK_OP_POW: return d == 0 ? bcast_dpow_da_ref(a, b) : dpow_db_ref(a, b);
-    }
-    return T(NAN);
-}
-
 // Physical offsets are linear in the nd-index (phys = sum (idx*spread + offset) * stride), so per launch the host
 // reduces the three descriptors to: a base offset and one effective stride per axis for each operand as it
 // follows the drain's index, plus the list of reduced axes (axis 0 first = fastest, the reference's order) with
@@ -46,7 +30,34 @@ struct BcastBwdArgs {
     int64_t red1[NK_MAX_RANK], red2[NK_MAX_RANK];
 };
 
-template <typename T, int V>
+// The eight forms the backward term takes: CPUBroadcast<Op>.java _getDeriveAt0 / _getDeriveAt1 (these differ from
+// the same-shape elementwise derivatives: the backward of + and - adds the operands because src1 is a zero tensor
+// there).  The form is a template parameter, so the inner loop carries no operator dispatch, and an operand that
+// is not part of the term is not read.
+enum { G_SUM = 0, G_DIFF = 1, G_SECOND = 2, G_FIRST = 3, G_RCP = 4, G_DDIV = 5, G_DPOW_A = 6, G_DPOW_B = 7 };
+static int derive_form(int op, int d) {
+    switch (op) {
+        case NK_OP_ADD: return G_SUM;
+        case NK_OP_SUB: return d == 0 ? G_SUM : G_DIFF;
+        case NK_OP_MUL: return d == 0 ? G_SECOND : G_FIRST;
+        case NK_OP_DIV:
+        case NK_OP_MOD: return d == 0 ? G_RCP : G_DDIV;
+        default:        return d == 0 ? G_DPOW_A : G_DPOW_B;
+    }
+}
+template <typename T, int G>
+__device__ __forceinline__ T derive_term(T a, T b) {
+    if constexpr (G == G_SUM) return a + b;
+    if constexpr (G == G_DIFF) return a - b;
+    if constexpr (G == G_SECOND) return b;
+    if constexpr (G == G_FIRST) return a;
+    if constexpr (G == G_RCP) return T(1) / b;
+    if constexpr (G == G_DDIV) return ddiv_db_ref(a, b);
+    if constexpr (G == G_DPOW_A) return bcast_dpow_da_ref(a, b);
+    return dpow_db_ref(a, b);
+}
+
+template <typename T, int V, int G>
 __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* __restrict__ drn,
                                                             const T* __restrict__ s1, const T* __restrict__ s2) {
     constexpr int UNROLL = 8;
@@ -57,50 +68,74 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
     nd_of_flat(A.c0, A.rank, (int)(t * V), o);
     int64_t o1 = A.base1, o2 = A.base2;
     for (int k = 0; k < A.rank; k++) { o1 += o[k] * A.keep1[k]; o2 += o[k] * A.keep2[k]; }
-    const int64_t last1 = A.keep1[A.rank - 1];       // V > 1: 1 (contiguous) or 0 (pinned); src2 is contiguous there
-    auto load1 = [&](int64_t at, T (&dst)[V]) {
-        if (V == 1) dst[0] = s1[at];
-        else if (last1 == 0) { const T x = s1[at]; for (int v = 0; v < V; v++) dst[v] = x; }
-        else { const Vec x = *(const Vec*)(s1 + at); for (int v = 0; v < V; v++) dst[v] = ((const T*)&x)[v]; }
-    };
-    auto load2 = [&](int64_t at, T (&dst)[V]) {
-        if (V == 1) dst[0] = s2[at];
-        else { const Vec x = __builtin_nontemporal_load((const Vec*)(s2 + at)); for (int v = 0; v < V; v++) dst[v] = ((const T*)&x)[v]; }
-    };
     T value[V];
 #pragma unroll
     for (int v = 0; v < V; v++) value[v] = T(0);
-    int r[NK_MAX_RANK];
-    for (int k = 0; k < NK_MAX_RANK; k++) r[k] = 0;
     const int n0 = A.nred > 0 ? A.red_extent[0] : 1;
     const int64_t st1 = A.nred > 0 ? A.red1[0] : 0, st2 = A.nred > 0 ? A.red2[0] : 0;
-    for (;;) {
-        int j = 0;
-        for (; j + UNROLL <= n0; j += UNROLL) {
-            T a[UNROLL][V], b[UNROLL][V];
+
+    // PINNED: src1 does not move along the last axis (V > 1 only): one element serves the thread's V neighbours
+    auto reduce = [&](auto pinned_tag) {
+        constexpr bool PINNED = decltype(pinned_tag)::value;
+        auto load1 = [&](int64_t at, T (&dst)[V]) {
+            if constexpr (G == G_SECOND || G == G_RCP) { for (int v = 0; v < V; v++) dst[v] = T(0); }      // src1 is not part of the term
+            else if constexpr (V == 1) dst[0] = s1[at];
+            else if constexpr (PINNED) { const T x = s1[at]; for (int v = 0; v < V; v++) dst[v] = x; }
+            else { const Vec x = *(const Vec*)(s1 + at); for (int v = 0; v < V; v++) dst[v] = ((const T*)&x)[v]; }
+        };
+        auto load2 = [&](int64_t at, T (&dst)[V]) {
+            if constexpr (G == G_FIRST) { for (int v = 0; v < V; v++) dst[v] = T(0); }                     // src2 is not part of the term
+            else if constexpr (V == 1) dst[0] = s2[at];
+            else { const Vec x = __builtin_nontemporal_load((const Vec*)(s2 + at)); for (int v = 0; v < V; v++) dst[v] = ((const T*)&x)[v]; }
+        };
+        int r[NK_MAX_RANK];
+        for (int k = 0; k < NK_MAX_RANK; k++) r[k] = 0;
+        for (;;) {
+            // the loads of the next UNROLL terms are issued before the current ones are added, so a wavefront
+            // always has requests in flight; the order of the additions is the reference's
+            int j = 0;
+            const int batches = n0 / UNROLL;
+            if (batches > 0) {
+                T a[UNROLL][V], b[UNROLL][V], an[UNROLL][V], bn[UNROLL][V];
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++) { load1(o1 + (j + u) * st1, a[u]); load2(o2 + (j + u) * st2, b[u]); }
+                for (int u = 0; u < UNROLL; u++) { load1(o1 + u * st1, a[u]); load2(o2 + u * st2, b[u]); }
+                for (int bi = 0; bi < batches; bi++) {
+                    if (bi + 1 < batches) {
+                        const int64_t jn = (int64_t)(bi + 1) * UNROLL;
 #pragma unroll
-            for (int u = 0; u < UNROLL; u++)
+                        for (int u = 0; u < UNROLL; u++) { load1(o1 + (jn + u) * st1, an[u]); load2(o2 + (jn + u) * st2, bn[u]); }
+                    }
 #pragma unroll
-                for (int v = 0; v < V; v++) value[v] = value[v] + bcast_derive<T>(A.op, A.d, a[u][v], b[u][v]);
+                    for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                        for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[u][v], b[u][v]);
+#pragma unroll
+                    for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                        for (int v = 0; v < V; v++) { a[u][v] = an[u][v]; b[u][v] = bn[u][v]; }
+                }
+                j = batches * UNROLL;
+            }
+            for (; j < n0; j++) {
+                T a[V], b[V];
+                load1(o1 + j * st1, a); load2(o2 + j * st2, b);
+#pragma unroll
+                for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[v], b[v]);
+            }
+            // carry into the slower reduced axes
+            int k = 1;
+            for (; k < A.nred; k++) {
+                r[k]++; o1 += A.red1[k]; o2 += A.red2[k];
+                if (r[k] < A.red_extent[k]) break;
+                o1 -= (int64_t)A.red_extent[k] * A.red1[k]; o2 -= (int64_t)A.red_extent[k] * A.red2[k];
+                r[k] = 0;
+            }
+            if (k >= A.nred) break;
         }
-        for (; j < n0; j++) {
-            T a[V], b[V];
-            load1(o1 + j * st1, a); load2(o2 + j * st2, b);
-#pragma unroll
-            for (int v = 0; v < V; v++) value[v] = value[v] + bcast_derive<T>(A.op, A.d, a[v], b[v]);
-        }
-        // carry into the slower reduced axes
-        int k = 1;
-        for (; k < A.nred; k++) {
-            r[k]++; o1 += A.red1[k]; o2 += A.red2[k];
-            if (r[k] < A.red_extent[k]) break;
-            o1 -= (int64_t)A.red_extent[k] * A.red1[k]; o2 -= (int64_t)A.red_extent[k] * A.red2[k];
-            r[k] = 0;
-        }
-        if (k >= A.nred) break;
-    }
+    };
+    if (V > 1 && A.keep1[A.rank - 1] == 0) reduce(std::true_type{});
+    else reduce(std::false_type{});
+
     const int at = phys_of_nd(A.c0, A.rank, o);
     if (V == 1) drn[at] = value[0];
     else {
@@ -170,12 +205,25 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
     A.n_threads = (unsigned)(vec ? n / V : n);
     const unsigned blocks = (A.n_threads + 255) / 256;
     set_path(vec ? "broadcast_backward_vec" : "broadcast_backward");
-    if (dtype == NK_F32) {
-        if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<float, 4>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
-        else     hipLaunchKernelGGL((broadcast_bwd_kernel<float, 1>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
-    } else {
-        if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<double, 2>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
-        else     hipLaunchKernelGGL((broadcast_bwd_kernel<double, 1>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+    auto go = [&](auto form) {
+        constexpr int G = decltype(form)::value;
+        if (dtype == NK_F32) {
+            if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<float, 4, G>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
+            else     hipLaunchKernelGGL((broadcast_bwd_kernel<float, 1, G>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
+        } else {
+            if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<double, 2, G>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+            else     hipLaunchKernelGGL((broadcast_bwd_kernel<double, 1, G>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+        }
+    };
+    switch (derive_form(op_id, d)) {
+        case G_SUM: go(std::integral_constant<int, G_SUM>{}); break;
+        case G_DIFF: go(std::integral_constant<int, G_DIFF>{}); break;
+        case G_SECOND: go(std::integral_constant<int, G_SECOND>{}); break;
+        case G_FIRST: go(std::integral_constant<int, G_FIRST>{}); break;
+        case G_RCP: go(std::integral_constant<int, G_RCP>{}); break;
+        case G_DDIV: go(std::integral_constant<int, G_DDIV>{}); break;
+        case G_DPOW_A: go(std::integral_constant<int, G_DPOW_A>{}); break;
+        default: go(std::integral_constant<int, G_DPOW_B>{}); break;
     }
     NK_HIP(hipGetLastError());
     return NK_OK;
