@@ -110,6 +110,79 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     }
 }
 
+// The last levels in one launch: once at most 256 tiles are left, one block finishes the tree.  Thread t reduces
+// tile t straight from memory (a whole tile is requested at once, then combined front to back), the tile results
+// go to LDS, and the following levels -- at most 256 values, then at most 4 -- are reduced there the same way.
+template <typename T, int RTS, int MODE>
+__global__ __launch_bounds__(256) void tail_reduce_kernel(const T* __restrict__ in, const T* __restrict__ in2,
+                                                          const int* __restrict__ idx_in, int m,
+                                                          T* __restrict__ out, int* __restrict__ idx_out) {
+    constexpr int VEC = 16 / sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));      // partial results start at any element
+    constexpr bool INDEXED = MODE == STAT_MIN || MODE == STAT_MAX;
+    __shared__ T vals[2][256];
+    __shared__ int idxs[2][256];
+    const int t = threadIdx.x;
+    int count = (m + RTS - 1) / RTS;                 // <= 256, checked by the host
+    auto combine = [&](T& value, int& found, T x, int pos) {
+        if (MODE == STAT_SUM || MODE == STAT_DOT) value = value + x;
+        else {
+            const bool better = MODE == STAT_MIN ? x < value : x > value;
+            if (pos == 0 || better) { value = x; found = pos; }
+        }
+    };
+    if (t < count) {
+        const int first = t * RTS;
+        const int limit = m - first < RTS ? m - first : RTS;
+        T value = T(0);
+        int found = 0;
+        if (limit == RTS) {
+            Vec v[RTS / VEC], w[RTS / VEC];
+#pragma unroll
+            for (int k = 0; k < RTS / VEC; k++) {
+                v[k] = ((const Vec*)(in + first))[k];
+                if (MODE == STAT_DOT) w[k] = ((const Vec*)(in2 + first))[k];
+            }
+#pragma unroll
+            for (int k = 0; k < RTS / VEC; k++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) combine(value, found, MODE == STAT_DOT ? v[k][e] * w[k][e] : v[k][e], k * VEC + e);
+        } else {
+            for (int i = 0; i < limit; i++) combine(value, found, MODE == STAT_DOT ? in[first + i] * in2[first + i] : in[first + i], i);
+        }
+        vals[0][t] = value;
+        if (INDEXED) idxs[0][t] = idx_in ? idx_in[first + found] : first + found;
+    }
+    __syncthreads();
+    int cur = 0;
+    while (count > 1) {
+        const int next = (count + RTS - 1) / RTS;
+        if (t < next) {
+            const int first = t * RTS;
+            const int limit = count - first < RTS ? count - first : RTS;
+            T value = T(0);
+            int found = 0;
+            for (int i = 0; i < limit; i++) {
+                const T x = vals[cur][first + i];
+                if (MODE == STAT_SUM || MODE == STAT_DOT) value = value + x;
+                else {
+                    const bool better = MODE == STAT_MIN ? x < value : x > value;
+                    if (i == 0 || better) { value = x; found = i; }
+                }
+            }
+            vals[cur ^ 1][t] = value;
+            if (INDEXED) idxs[cur ^ 1][t] = idxs[cur][first + found];
+        }
+        __syncthreads();
+        cur ^= 1;
+        count = next;
+    }
+    if (t == 0) {
+        out[0] = vals[cur][0];
+        if (INDEXED) idx_out[0] = idxs[cur][0];
+    }
+}
+
 template <typename T, int RTS, int MODE>
 static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* out_value, int* out_index) {
     constexpr bool indexed = MODE == STAT_MIN || MODE == STAT_MAX;
@@ -131,9 +204,17 @@ static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* o
     int level = 0;
     do {
         const int64_t tiles = (m + RTS - 1) / RTS;
-        const bool last = tiles == 1;
-        T* dst = last && out_value ? out_value : vals + used;
-        int* dst_idx = !indexed ? nullptr : (last && out_index ? out_index : idxs + used);
+        if (tiles <= 256) {                         // one block finishes the tree
+            T* dst = out_value ? out_value : vals + used;
+            int* dst_idx = !indexed ? nullptr : (out_index ? out_index : idxs + used);
+            if (MODE == STAT_DOT && level > 0)
+                hipLaunchKernelGGL((tail_reduce_kernel<T, RTS, STAT_SUM>), dim3(1), dim3(256), 0, dev->stream, cur, cur, cur_idx, (int)m, dst, dst_idx);
+            else
+                hipLaunchKernelGGL((tail_reduce_kernel<T, RTS, MODE>), dim3(1), dim3(256), 0, dev->stream, cur, cur2, cur_idx, (int)m, dst, dst_idx);
+            break;
+        }
+        T* dst = vals + used;
+        int* dst_idx = indexed ? idxs + used : nullptr;
         const unsigned blocks = (unsigned)((tiles + 255) / 256);
         if (MODE == STAT_DOT && level > 0)
             hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, STAT_SUM>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur, cur_idx, m, dst, dst_idx);

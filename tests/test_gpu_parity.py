@@ -944,7 +944,7 @@ def test_stats_autograd_golden(device, golden):
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_sum_is_bit_identical_to_the_cpu_tree(device, orc, dt):
     rng = np.random.default_rng(61)
-    for n in (1, 2, 31, 127, 128, 129, 8191, 8192, 16385, 100003, (1 << 21) + 77):
+    for n in (1, 2, 31, 127, 128, 129, 8191, 8192, 16385, 32767, 32768, 32769, 100003, (1 << 21) + 77):
         say("sum", dt, n)
         x = rng.standard_normal(n).astype(F[dt])
         got = on(device, x).sum()
@@ -960,7 +960,7 @@ def test_sum_is_bit_identical_to_the_cpu_tree(device, orc, dt):
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_min_max_return_the_reference_index(device, orc, dt):
     rng = np.random.default_rng(62)
-    for n in (1, 2, 63, 64, 65, 4095, 4096, 4097, 70001, (1 << 20) + 3):
+    for n in (1, 2, 63, 64, 65, 4095, 4096, 4097, 16383, 16384, 16385, 70001, (1 << 20) + 3):
         say("min/max", dt, n)
         x = rng.integers(-40, 40, n).astype(F[dt])                 # many ties: the first one must win
         t = on(device, x)
@@ -978,7 +978,7 @@ def test_min_max_return_the_reference_index(device, orc, dt):
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_dot_product(device, orc, dt):
     rng = np.random.default_rng(63)
-    for n in (1, 5, 128, 129, 100003):
+    for n in (1, 5, 128, 129, 32768, 32769, 100003):
         say("dot", dt, n)
         a, b = rng.standard_normal(n).astype(F[dt]), rng.standard_normal(n).astype(F[dt])
         got = on(device, a).dot(on(device, b)).items
