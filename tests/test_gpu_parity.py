@@ -739,7 +739,7 @@ def test_integer_scalarization_bit_exact(device, orc, golden, dt):
         want = orc.scalarization_int(op, -1, before.copy(), cfg(drn), parent.getData(), cfg(src), value)
         assert (out_parent.getData() == want).all(), (dt.__name__, op)
     if dt == np.int32:
-        say("Tensor_Operation_Spec integer rows on the device")
+        say("recorded (unenforced) integer rows of Tensor_Operation_Spec on the device")
         g = golden["int_scalarization"]
         i0 = on(device, np.array(g["tempeh_i0_recovered"], dtype=np.int32), (2, 3))
         times10 = i0 * 10
