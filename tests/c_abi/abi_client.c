@@ -104,6 +104,24 @@ int main(void) {
     CHECK(nk_d2h(dev, &where, dwhere, 0, 4));
     EXPECT(where == 8);
 
+    /* integer scalarization: Java's int arithmetic (wrapping multiply, truncating division), / by zero is an error */
+    const int32_t iv[5] = {2147483647, -7, 7, 0, -2147483647 - 1};
+    int32_t ir[5];
+    const int five[1] = {5};
+    int32_t ci[5];
+    dense_cfg(ci, five, 1);
+    nk_buf di, dr;
+    CHECK(nk_alloc(dev, sizeof iv, &di)); CHECK(nk_alloc(dev, sizeof ir, &dr));
+    CHECK(nk_h2d(dev, di, 0, iv, sizeof iv));
+    CHECK(nk_scalarization_int(dev, NK_OP_MUL, -1, NK_I32, 1, dr, ci, di, ci, 2, 5));
+    CHECK(nk_d2h(dev, ir, dr, 0, sizeof ir));
+    EXPECT(ir[0] == -2 && ir[1] == -14 && ir[2] == 14 && ir[3] == 0 && ir[4] == 0);
+    CHECK(nk_scalarization_int(dev, NK_OP_DIV, -1, NK_I32, 1, dr, ci, di, ci, 2, 5));
+    CHECK(nk_d2h(dev, ir, dr, 0, sizeof ir));
+    EXPECT(ir[0] == 1073741823 && ir[1] == -3 && ir[2] == 3 && ir[3] == 0 && ir[4] == -1073741824);
+    EXPECT(nk_scalarization_int(dev, NK_OP_DIV, -1, NK_I32, 1, dr, ci, di, ci, 0, 5) != 0);
+    CHECK(nk_free(dev, di)); CHECK(nk_free(dev, dr));
+
     /* a descriptor that reaches outside its buffer is an error, not a launch */
     const int too_big[2] = {4, 4};
     int32_t cbad[10];
