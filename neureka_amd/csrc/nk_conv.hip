@@ -115,7 +115,12 @@ __global__ __launch_bounds__(256) void conv_split(ConvArgs A, T* __restrict__ dr
     const int tid = threadIdx.x;
     const int rank = RANK ? RANK : A.rank;          // RANK = 0: any rank up to NK_MAX_RANK
     constexpr int NR = RANK ? RANK : NK_MAX_RANK;
-    for (unsigned i = blockIdx.x; i < A.n; i += gridDim.x) {
+    // consecutive block ids go round-robin to the 8 XCDs: give every XCD one contiguous eighth of the drain, so that
+    // neighbouring drain elements, whose terms overlap, share that XCD's L2 (the grid is 8 * ceil(n / 8) blocks)
+    const unsigned per_xcd = gridDim.x >> 3;
+    {
+        const unsigned i = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
+        if (i >= A.n) return;
         int o[NR], lo[NR], ext[NR], b1[NR], j[NR], d[NR];
         nd_of_flat(A.c0, rank, (int)i, o);
         unsigned terms = 1;
@@ -167,7 +172,6 @@ __global__ __launch_bounds__(256) void conv_split(ConvArgs A, T* __restrict__ dr
             __syncthreads();
         }
         if (tid == 0) drn[phys_of_nd(A.c0, rank, o)] = part[0];
-        __syncthreads();
     }
 }
 
@@ -733,7 +737,7 @@ static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, n
     }
     if (terms >= 1024 && n <= ((int64_t)1 << 18)) {
         set_path(d < 0 ? "split_fwd" : "split_bwd");
-        const unsigned grid = (unsigned)n;
+        const unsigned grid = 8u * (unsigned)((n + 7) / 8);
         auto go = [&](auto R) {
             constexpr int RANK = decltype(R)::value;
             if (d < 0) hipLaunchKernelGGL((conv_split<T, false, RANK>), dim3(grid), dim3(256), 0, dev->stream, A, out, s1, s2);
