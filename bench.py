@@ -49,6 +49,63 @@ def event_times_ms(dev, launch, reps):
     return [dev.elapsed_ms(events[i], events[i + 1]) for i in range(reps)]
 
 
+def cpu_side_of_the_other_configs(cores):
+    """The oracle (the reference's CPU kernels restated in C, split like JVMExecutor over `cores` threads) on bounded
+    samples of the configurations besides the headline one; every entry says what was timed."""
+    from oracle import cpu_oracle as orc
+    f32 = np.float32
+    rng = np.random.default_rng(3)
+    out = {}
+
+    def timed(fn, reps):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    x = rng.uniform(-1, 1, 4096).astype(f32); k = rng.uniform(-1, 1, 9).astype(f32)
+    sec = timed(lambda: orc.simple_conv2d(x, k, 64, 64, 3, 3), 200)
+    out["conv2d_64x64_3x3"] = {"ms": round(sec * 1e3, 4), "GFLOP/s": round(69192 / sec / 1e9, 3), "cores": 1,
+                               "sample": "the whole configuration (SimpleCPUConvolution.ImplF32, one image)"}
+    n = 1 << 24
+    a, b, c = [rng.standard_normal(n).astype(f32) for _ in range(3)]
+    cf = orc.dense_cfg([n]); tmp = np.zeros(n, f32); o = np.zeros(n, f32)
+
+    def chain():
+        orc.activation("sig", -1, tmp, cf, a, cf, workers=cores); orc.elementwise("multiply", -1, o, cf, tmp, cf, b, cf, workers=cores)
+        orc.elementwise("add", -1, tmp, cf, o, cf, c, cf, workers=cores); orc.activation("tanh", -1, o, cf, tmp, cf, workers=cores)
+    sec = timed(chain, 3)
+    out["chain_unfused_4_kernels"] = {"ms": round(sec * 1e3, 2), "GB/s": round(40 * n / sec / 1e9, 2), "cores": cores,
+                                      "sample": "2^24 of the 2^26 elements, the four kernels the reference runs (10 arrays, 40 B per element)"}
+    del a, b, c, tmp, o
+    M, K, N = 512, 4096, 4096
+    A = rng.uniform(-1, 1, M * K).astype(f32); B = rng.uniform(-1, 1, K * N).astype(f32)
+    sec = timed(lambda: orc.gemm(True, A, B, M, K, N, workers=cores), 1)
+    out["matmul_4096"] = {"ms": round(sec * 1e3 * 4096 / M, 1), "GFLOP/s": round(2.0 * M * K * N / sec / 1e9, 2), "cores": cores,
+                          "sample": "the first 512 of the 4096 rows of A (GEMM.threaded_F32_MxN_RM splits rows), time scaled by 8"}
+    M, K, N = 65536, 256, 256
+    A = rng.uniform(-1, 1, M * K).astype(f32); B = rng.uniform(-1, 1, K * N).astype(f32)
+    sec = timed(lambda: orc.gemm(True, A, B, M, K, N, workers=cores), 1)
+    out["matmul_tall_skinny"] = {"ms": round(sec * 1e3, 1), "GFLOP/s": round(2.0 * M * K * N / sec / 1e9, 2), "cores": cores, "sample": "the whole configuration"}
+    del A, B
+    xs, ks, ys = [64, 256, 256], [64, 5, 5], [1, 252, 252]
+    x5 = (rng.standard_normal(64 * 256 * 256) * 0.1).astype(f32); k5 = (rng.standard_normal(1600) * 0.1).astype(f32)
+    e5 = rng.standard_normal(252 * 252).astype(f32)
+    y = np.zeros(252 * 252, f32)
+    sec = timed(lambda: orc.convolve(y, orc.dense_cfg(ys), x5, orc.dense_cfg(xs), k5, orc.dense_cfg(ks), workers=cores), 3)
+    out["conv_c5_forward"] = {"ms": round(sec * 1e3, 2), "GFLOP/s": round(203212800 / sec / 1e9, 3), "cores": cores, "sample": "the whole configuration (_convolve32)"}
+    dk = np.zeros(1600, f32)
+    sec = timed(lambda: orc.deconvolve(dk, orc.dense_cfg(ks), x5, orc.dense_cfg(xs), e5, orc.dense_cfg(ys), workers=cores), 2)
+    out["conv_c5_grad_kernel"] = {"ms": round(sec * 1e3, 2), "GFLOP/s": round(203212800 / sec / 1e9, 3), "cores": cores, "sample": "the whole configuration (_deConvolve32)"}
+    dx = np.zeros(64 * 256 * 256, f32)
+    part = dx.size // 1024
+    sec = timed(lambda: orc.run("deconvolve", 0, 0, dx, orc.dense_cfg(xs), k5, orc.dense_cfg(ks), e5, orc.dense_cfg(ys), workers=cores, first=0, limit=part), 1)
+    out["conv_c5_grad_input"] = {"ms": round(sec * 1e3 * 1024, 0), "GFLOP/s": round(203212800 / (sec * 1024) / 1e9, 4), "cores": cores,
+                                 "sample": "the first 1/1024 of the drain, time scaled by 1024: _deConvolve32 visits every entry of the error for every drain element"}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -276,6 +333,11 @@ def main():
         flops("conv_c5_grad_input_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", 0, dx5, k5, e5), f64=True)
         flops("conv_c5_grad_kernel_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", 0, dk5, x5, e5), f64=True)
 
+    # ---- the reference's CPU path beside the other configurations (oracle, bounded samples) -----------------------
+    cpu_others = None
+    if not args.no_cpu and not args.no_others:
+        cpu_others = cpu_side_of_the_other_configs(min(16, len(os.sched_getaffinity(0))))
+
     result = {
         "metric": "GB/s & % HBM peak (broadcast/elementwise)",
         "value": round(value, 1),
@@ -294,6 +356,7 @@ def main():
                    "device": dev.name(), "compute_units": dev.maxComputeUnits()},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "cpu_others": cpu_others,
         "others": others,
     }
     print(json.dumps(result))
