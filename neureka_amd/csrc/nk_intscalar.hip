@@ -76,9 +76,7 @@ __device__ inline I int_apply(I a, I b) {
     return (I)0;
 }
 
-constexpr int INT_MODES = 7 * 3;
-
-template <typename I, typename Body>
+template <typename Body>
 __device__ inline void for_mode(int mode, Body body) {
     switch (mode) {
 #define NK_MODE(M) case M: body(std::integral_constant<int, M>{}); break;
@@ -98,7 +96,7 @@ __global__ __launch_bounds__(256) void int_scalar_flat(int mode, I value, int64_
     const int64_t n_vec = n / VEC;
     const int64_t step = (int64_t)gridDim.x * blockDim.x;
     const int64_t first = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    for_mode<I>(mode, [&](auto M) {
+    for_mode(mode, [&](auto M) {
         constexpr int MODE = decltype(M)::value;
         for (int64_t p = first; p < n_vec; p += step) {
             const Vec v = __builtin_nontemporal_load((const Vec*)src + p);
@@ -117,7 +115,7 @@ __global__ __launch_bounds__(256) void int_scalar_indexed(int mode, I value, int
                                                           const I* __restrict__ src) {
     const unsigned step = gridDim.x * blockDim.x;
     const unsigned first = blockIdx.x * blockDim.x + threadIdx.x;
-    for_mode<I>(mode, [&](auto M) {
+    for_mode(mode, [&](auto M) {
         constexpr int MODE = decltype(M)::value;
         for (unsigned i = first; i < n; i += step)
             drn[phys_of_flat(c0, rank, (int)i)] = int_apply<I, MODE>(src[phys_of_flat(c1, rank, (int)i)], value);
