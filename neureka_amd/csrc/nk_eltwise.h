@@ -252,6 +252,7 @@ struct RowsArgs {
     unsigned const_last;       // bit j: source j has stride 0 along the innermost axis
     int simple_loads;          // every source register is filled by a plain vector load
     int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
+    int ragged;                // L is not a multiple of vec: the last vector of a row is moved back to end with the row
     int streaming;             // non-temporal stores for the drain
     int nt_loads;              // every source element is read exactly once: the host picks the non-temporal-load variant
     FastDiv chunk_div;
@@ -279,6 +280,7 @@ __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsign
     R.live = row_ok && R.col < A.L;
     if (!row_ok) row = 0;                                           // dead lanes get a valid address:
     if (!R.live) R.col = 0;                                         // loads need no predicate
+    if (A.ragged && R.col + (unsigned)A.vec > A.L) R.col = A.L - (unsigned)A.vec;
     auto resolve = [&](unsigned r) {
 #pragma unroll
         for (int o = 0; o < NOPS; o++) R.off[o] = A.base[o];

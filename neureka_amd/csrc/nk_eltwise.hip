@@ -204,8 +204,30 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     }
     if (rows_ok) {
         constexpr int VMAX = 16 / sizeof(T);
-        // 16 bytes per lane whenever a row is a whole number of vectors (no alignment requirement)
-        const bool vec = cn.shape[last] % VMAX == 0;
+        // 16 bytes per lane whenever a row is a whole number of vectors (no alignment requirement).  A ragged row
+        // (length not a multiple of the vector) also runs on vectors: the last vector of a row is moved back so
+        // that it ends with the row and overlaps its neighbour, whose elements are then computed and written twice
+        // with the same values -- which is only the same thing when no source shares memory with the drain.
+        bool ragged = cn.shape[last] % VMAX != 0 && cn.shape[last] >= VMAX && env_flag("NK_RAGGED_VECTORS", true);
+        if (ragged) {
+            auto span = [&](int o, int64_t& lo, int64_t& hi) {
+                const int64_t ptr = o == 0 ? (int64_t)c.drn : (int64_t)c.src[o - 1];
+                lo = hi = cn.base[o];
+                for (int k = 0; k < cn.rank; k++) {
+                    const int64_t sp = (cn.shape[k] - 1) * cn.stride[o][k];
+                    if (sp < 0) lo += sp; else hi += sp;
+                }
+                lo = ptr + lo * (int64_t)sizeof(T); hi = ptr + (hi + 1) * (int64_t)sizeof(T);
+            };
+            int64_t dlo, dhi;
+            span(0, dlo, dhi);
+            for (int j = 0; j < c.nsrc && ragged; j++) {
+                int64_t slo, shi;
+                span(j + 1, slo, shi);
+                if (slo < dhi && dlo < shi) ragged = false;
+            }
+        }
+        const bool vec = cn.shape[last] % VMAX == 0 || ragged;
         RowsArgs& A = plan.rows;
         const int V = vec ? VMAX : 1;
         int passes = rows_passes(funset, funset >= 2 ? NK_FUSE_MAX_SRC : (c.nsrc <= 1 ? 1 : c.nsrc));
@@ -238,6 +260,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             for (int k = 0; k < last; k++) A.stride[o][k] = (int)cn.stride[o][last - 1 - k];
         }
         A.vec = V;
+        A.ragged = ragged ? 1 : 0;
         A.simple_loads = (funset < 2 && A.const_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel

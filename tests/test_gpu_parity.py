@@ -369,6 +369,39 @@ def test_broadcast_forward_bit_exact(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_ragged_rows_run_on_vectors_and_stay_bit_exact(device, orc, dt):
+    """Rows whose length is not a multiple of the 16-byte vector: the last vector of a row is moved back to end with the
+    row (its neighbour's elements are computed twice).  Broadcast, same-shape elementwise, an activation and a fused
+    chain, bit for bit; and in place (the drain is one of the sources), where computing twice would not be the
+    same thing, the element-wise path must be taken."""
+    rng = np.random.default_rng(23)
+    T = F[dt]
+    V = 16 // np.dtype(T).itemsize
+    for s1, s2 in (([37, 1, 511], [1, 9, 511]), ([5, 1, 7], [1, 6, 7]), ([3, 1023], [3, 1023]), ([64, 1, 5], [1, 33, 5]), ([2, 1, V + 1], [1, 3, V + 1])):
+        so = [q if p == 1 else p for p, q in zip(s1, s2)]
+        a = rng.uniform(-1, 1, s1).astype(T); b = rng.uniform(-1, 1, s2).astype(T)
+        ta, tb = on(device, a), on(device, b)
+        for op, f in (("add", np.add), ("multiply", np.multiply), ("divide", np.divide)):
+            say("ragged broadcast", s1, s2, op, dt)
+            out = Tensor._on_device(device, T, so)
+            device.launch_broadcast(op, -1, out, ta, tb)
+            assert _lib.last_path() == "rows_vec_binary", _lib.last_path()
+            assert_bits(out.getData().reshape(so), f(a, b), f"{op} {s1} {s2}")
+    n = [7, 333]
+    x = rng.uniform(-2, 2, n).astype(T); y = rng.uniform(-2, 2, n).astype(T)
+    tx, ty = on(device, x), on(device, y)
+    say("ragged activation", dt)
+    out = Tensor._on_device(device, T, n)
+    device.launch_activation("softsign", -1, out, tx)
+    assert _lib.last_path() == "rows_vec"
+    assert_bits(out.getData(), orc.activation("softsign", -1, np.zeros(x.size, dtype=T), orc.dense_cfg(n), x.reshape(-1), orc.dense_cfg(n)), "softsign")
+    say("ragged in place", dt)
+    device.launch_elementwise("add", -1, tx, tx, ty)                       # x += y
+    assert _lib.last_path() == "rows_binary", _lib.last_path()
+    assert_bits(tx.getData().reshape(n), x + y, "in place")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_broadcast_backward_bit_exact(device, orc, dt):
     rng = np.random.default_rng(22)
     full = [6, 5, 7]
