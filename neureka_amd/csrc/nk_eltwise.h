@@ -234,9 +234,12 @@ __device__ __forceinline__ void store_vec(T* p, const T (&src)[V], bool streamin
 // that an operand which does not change along the rows is the same piece of memory in every pass.  A thread
 // issues the loads of all its passes, runs the program once over all of them, then stores.  When a row spans at least a wavefront (tpr >= 64) the row index is wave-uniform:
 // the nd-index arithmetic then runs on the scalar unit.  Element offsets are 32-bit (the host checks),
-// at most ROWS_MAX_OUTER outer axes (more fall to the canon kernel); the argument block is small and
+// at most ROWS_MAX_OUTER outer axes (more fall to the canon kernel; kernels take MAXO of them); the argument block is small and
 // fixed-size so that it is fetched with a few wide scalar loads at kernel start.
-constexpr int ROWS_MAX_OUTER = 3;
+constexpr int ROWS_MAX_OUTER = 5;
+// The kernels resolve ROWS_FAST_OUTER outer axes unless instantiated for more: two further (unused) steps in the
+// address arithmetic of every pass cost the broadcast of [1024,1,512] o [1,2048,512] five per cent.
+constexpr int ROWS_FAST_OUTER = 3;
 // units per block of rows_kernel: enough loads in flight to cover latency, few enough registers to keep
 // several wavefronts per SIMD (three sources x 16 values already costs half the occupancy)
 constexpr int rows_passes(int funset, int nsrc) { return funset >= 2 ? 1 : (nsrc >= 3 ? 2 : 4); }
@@ -268,7 +271,7 @@ struct RowsAddr {
     unsigned col;
     bool live;
 };
-template <int NOPS>
+template <int NOPS, int MAXO = ROWS_FAST_OUTER>
 __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsigned rg, unsigned chunk) {
     const unsigned tpr = 1u << A.tpr_log2;
     const unsigned rows_per_pass = 256u >> A.tpr_log2;
@@ -285,7 +288,7 @@ __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsign
 #pragma unroll
         for (int o = 0; o < NOPS; o++) R.off[o] = A.base[o];
 #pragma unroll
-        for (int k = 0; k < ROWS_MAX_OUTER; k++) {
+        for (int k = 0; k < MAXO; k++) {
             if (k < A.nouter) {
                 const unsigned q = A.outer[k].div(r);
                 const int idx = (int)(r - q * A.outer[k].d);
@@ -315,7 +318,7 @@ __device__ __forceinline__ void rows_unit(const RowsArgs& A, int passes, int p, 
     }
 }
 
-template <typename T, int V, int NSRC, int FUNSET, int PASSES, bool NT = false>
+template <typename T, int V, int NSRC, int FUNSET, int PASSES, bool NT = false, int MAXO = ROWS_FAST_OUTER>
 __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg LP, T* __restrict__ drn, Ptrs srcs) {
     T x[NSRC][PASSES * V];
     int doff[PASSES];
@@ -326,7 +329,7 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
         for (int p = 0; p < PASSES; p++) {
             unsigned rg, chunk;
             rows_unit(A, PASSES, p, rg, chunk);
-            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, rg, chunk);
+            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1, MAXO>(A, rg, chunk);
             live[p] = R.live;
             doff[p] = R.off[0] + (int)R.col;
 #pragma unroll
@@ -340,7 +343,7 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
         for (int p = 0; p < PASSES; p++) {
             unsigned rg, chunk;
             rows_unit(A, PASSES, p, rg, chunk);
-            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1>(A, rg, chunk);
+            const RowsAddr<NSRC + 1> R = rows_address<NSRC + 1, MAXO>(A, rg, chunk);
             live[p] = R.live;
             doff[p] = R.off[0] + (int)R.col;
 #pragma unroll
@@ -377,7 +380,8 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
 // (same-shape elementwise and forward broadcast).  The operator is resolved once, outside the passes,
 // and each pass is stored as soon as its operands have arrived.
 // HOIST bit j: source j does not change along the rows a block covers (forward broadcast): it is loaded once.
-template <typename T, int V, int PASSES, bool NT = false, int HOIST = 0>
+// CONST bit j: source j does not change along a row (one element per row, e.g. a per-row scale or an outer product).
+template <typename T, int V, int PASSES, bool NT = false, int HOIST = 0, int CONST = 0, int MAXO = ROWS_FAST_OUTER>
 __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T* __restrict__ drn, const T* __restrict__ s0,
                                                           const T* __restrict__ s1) {
     T x0[PASSES][V], x1[PASSES][V];
@@ -387,11 +391,13 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
     for (int p = 0; p < PASSES; p++) {
         unsigned rg, chunk;
         rows_unit(A, PASSES, p, rg, chunk);
-        const RowsAddr<3> R = rows_address<3>(A, rg, chunk);
+        const RowsAddr<3> R = rows_address<3, MAXO>(A, rg, chunk);
         live[p] = R.live;
         doff[p] = R.off[0] + (int)R.col;
-        if (p == 0 || !(HOIST & 1)) load_vec<T, V, NT>(x0[p], s0 + R.off[1] + R.col);
-        if (p == 0 || !(HOIST & 2)) load_vec<T, V, NT>(x1[p], s1 + R.off[2] + R.col);
+        if (CONST & 1) { const T c = s0[R.off[1]]; _Pragma("unroll") for (int v = 0; v < V; v++) x0[p][v] = c; }
+        else if (p == 0 || !(HOIST & 1)) load_vec<T, V, NT>(x0[p], s0 + R.off[1] + R.col);
+        if (CONST & 2) { const T c = s1[R.off[2]]; _Pragma("unroll") for (int v = 0; v < V; v++) x1[p][v] = c; }
+        else if (p == 0 || !(HOIST & 2)) load_vec<T, V, NT>(x1[p], s1 + R.off[2] + R.col);
     }
     if (HOIST) {
 #pragma unroll

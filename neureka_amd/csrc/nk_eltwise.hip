@@ -238,6 +238,8 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
         for (int j = 0; j < c.nsrc && once; j++)
             for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) once = false;
+        const bool deep = last > ROWS_FAST_OUTER;           // more outer axes than the tuned variants resolve: plain variants
+        if (deep) once = false;
         A.nt_loads = once ? 1 : 0;
         A.const_last = 0;
         for (int j = 0; j < c.nsrc; j++) if (cn.stride[j + 1][last] == 0) A.const_last |= 1u << j;
@@ -264,13 +266,15 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         A.simple_loads = (funset < 2 && A.const_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel
-        if (A.simple_loads && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
+        // (sources that are constant along a row are handled by that kernel's vector variant only)
+        const bool loads_ok = A.simple_loads || (A.const_last != 0 && vec && env_flag("NK_BINARY_ROW_CONSTANT", true));
+        if (loads_ok && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
             prog.op[1] == I_BIN && prog.src[1] == 1 && prog.arg[1] <= NK_OP_DIV) {
             plan.kind = PLAN_ROWS_BINARY;
             plan.binary_op = prog.arg[1];
             if (vec) {
                 static const int env_passes = [] { const char* v = getenv("NK_BINARY_PASSES"); return v && *v ? atoi(v) : 8; }();
-                passes = env_passes == 2 || env_passes == 4 ? env_passes : 8;
+                passes = (env_passes == 2 || env_passes == 4) && A.const_last == 0 && !deep ? env_passes : 8;
             }
             plan.passes = passes;
         }
@@ -285,7 +289,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             if (constant) A.pass_rows = 1;
             // measured at steady state: loading the constant source once gains 2..14 % when a row fills the block
             // (256 threads) and loses 4..14 % when a block covers several rows per pass
-            if (constant && env_flag("NK_HOIST", true) && vec && passes == 8 && !A.nt_loads && rpp == 1 &&
+            if (constant && env_flag("NK_HOIST", true) && vec && passes == 8 && !A.nt_loads && rpp == 1 && A.const_last == 0 && !deep &&
                 cn.shape[last - 1] % ((int64_t)passes * rpp) == 0)
                 plan.hoist = constant;
         }

@@ -402,6 +402,45 @@ def test_ragged_rows_run_on_vectors_and_stay_bit_exact(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_deep_index_spaces_and_row_constant_sources(device, orc, dt):
+    """Four and five outer axes that do not merge (alternating broadcast axes, slices on every axis) and sources that
+    are constant along a row (outer products, per-row scales): the vector kernels with every outer axis resolved,
+    bit for bit against numpy / the oracle."""
+    rng = np.random.default_rng(24)
+    T = F[dt]
+    for s1, s2 in (([6, 1, 5, 1, 8], [1, 4, 1, 3, 8]), ([3, 1, 4, 1, 2, 12], [1, 2, 1, 3, 1, 12]), ([6, 1, 5, 1, 3], [1, 4, 1, 3, 3]),
+                   ([40, 9, 1], [1, 1, 64]), ([7, 1], [1, 36]), ([1, 36], [7, 1]), ([5, 3, 16], [5, 3, 1]), ([5, 3, 1], [5, 1, 1])):
+        so = [max(p, q) for p, q in zip(s1, s2)]
+        a = rng.uniform(-1, 1, s1).astype(T); b = rng.uniform(-1, 1, s2).astype(T)
+        ta, tb = on(device, a), on(device, b)
+        for op, f in (("add", np.add), ("subtract", np.subtract), ("multiply", np.multiply), ("divide", np.divide)):
+            say("deep / row-constant broadcast", s1, s2, op, dt)
+            out = Tensor._on_device(device, T, so)
+            device.launch_broadcast(op, -1, out, ta, tb)
+            assert _lib.last_path() in ("rows_vec_binary", "rows_binary", "rows_vec", "rows"), _lib.last_path()
+            assert_bits(out.getData().reshape(so), f(a, b), f"{op} {s1} {s2}")
+    say("activation and fused chain on a view with five live axes", dt)
+    parent = rng.uniform(-2, 2, (5, 6, 7, 5, 40)).astype(T)
+    tp = on(device, parent)
+    view = tp[1:4, 0:6:2, 2:7, 1:5:3, 4:36]
+    want_items = parent[1:4, 0:6:2, 2:7, 1:5:3, 4:36]
+    out = Tensor._on_device(device, T, view.shape)
+    device.launch_activation("softsign", -1, out, view)
+    assert _lib.last_path() == "rows_vec", _lib.last_path()
+    dense = orc.dense_cfg(list(view.shape))
+    want = orc.activation("softsign", -1, np.zeros(out.size, dtype=T), dense, np.ascontiguousarray(want_items).reshape(-1), dense)
+    assert_bits(out.getData(), want, "softsign on a deep view")
+    from neureka_amd.function import Function
+    fused = device.optimizedFunctionOf(Function.of("tanh(sig(I[0])*I[1]+I[2])"), "chain")
+    got = fused(view, view, view)
+    x = np.ascontiguousarray(want_items).reshape(-1)
+    t1 = orc.activation("sig", -1, np.zeros_like(x), dense, x, dense)
+    t2 = orc.elementwise("multiply", -1, np.zeros_like(x), dense, t1, dense, x, dense)
+    t3 = orc.elementwise("add", -1, np.zeros_like(x), dense, t2, dense, x, dense)
+    assert_close(got.items, orc.activation("tanh", -1, np.zeros_like(x), dense, t3, dense), "fused chain on a deep view")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_broadcast_backward_bit_exact(device, orc, dt):
     rng = np.random.default_rng(22)
     full = [6, 5, 7]
