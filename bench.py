@@ -240,6 +240,11 @@ def main():
             g_t = Tensor._on_device(dev, f32, tgt); z_t = Tensor._on_device(dev, f32, oth)
             hbm(f"broadcast_backward_grad{d}", 4 * (err.size + g_t.size + z_t.size), dev.prepared_launch("broadcast", "add", d, g_t, z_t, err))
             dev.free(g_t); dev.free(z_t)
+        # a bias gradient (few outputs, long sums) and the sum over the innermost axis of the same 4 GiB of error
+        for name, tgt in (("broadcast_backward_bias", (1, 1, 512)), ("broadcast_backward_per_slab", (1024, 1, 1))):
+            g_t = Tensor._on_device(dev, f32, tgt); z_t = Tensor._on_device(dev, f32, tuple(1 if t > 1 else f for t, f in zip(tgt, (1024, 2048, 512))))
+            hbm(name, 4 * (err.size + g_t.size + z_t.size), dev.prepared_launch("broadcast", "add", 0, g_t, z_t, err))
+            dev.free(g_t); dev.free(z_t)
         dev.free(err)
 
         # C3: tanh(sig(a)*b+c) on 2^26 elements: fused, and the reference's 4-kernel sequence

@@ -145,6 +145,145 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
     }
 }
 
+// ---- few outputs, long sums ---------------------------------------------------------------------------------
+// One thread per drain element cannot feed the machine when a gradient has few elements (a bias: 512 sums of
+// 131 072 terms) or when the reduced axis is the contiguous one (every thread would walk its own row).  Here a
+// block owns OT neighbouring drain elements and one segment of their sums: its 256 threads are TL = 256 / OT lanes
+// per element; the lanes of an element take every TL-th term of the segment -- terms enumerated with the last
+// reduced axis fastest, the order memory runs in -- and meet in LDS.
+//   ROWS = false (the drain keeps the innermost axis): OT = 64, neighbouring threads own neighbouring drain elements,
+//                so a wavefront reads 64 neighbouring elements of the error per term;
+//   ROWS = true  (the innermost axis is reduced): neighbouring threads own neighbouring terms, VT of them each
+//                through one 16-byte load when the axis allows it; TL = 64 or 256 by the length of the sums.
+// Several segments write partial sums that a second launch adds in segment order.  The terms are the
+// reference's; their order is not: results agree norm-wise (1e-5 / 1e-12).
+struct BwdSplitArgs {
+    unsigned n_out, out_blocks;          // drain elements, blocks of OT of them
+    unsigned terms, seg_terms;           // term units (VT terms each) per drain element and per segment
+    int segments;
+    int splat1;                          // VT > 1: src1 does not move along the innermost reduced axis
+};
+
+template <typename T, int G, int OT, bool ROWS, int VW>
+__global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A, BwdSplitArgs S, T* __restrict__ drn, T* __restrict__ partial,
+                                                                  const T* __restrict__ s1, const T* __restrict__ s2) {
+    // VW: width of the 16-byte accesses -- ROWS: VW neighbouring terms of one drain element per load;
+    // otherwise VW neighbouring drain elements per thread
+    constexpr int TL = 256 / OT;                                 // term lanes per drain element (group)
+    constexpr int U = 4;                                         // loads in flight per lane
+    constexpr int NV = ROWS ? 1 : VW;                            // running sums per thread
+    typedef typename std::conditional<VW == 1, T, T __attribute__((ext_vector_type(VW == 1 ? 2 : VW), aligned(sizeof(T))))>::type Vec;
+    __shared__ T part[NV][256];
+    const int tid = threadIdx.x;
+    const unsigned ob = blockIdx.x % S.out_blocks, seg = blockIdx.x / S.out_blocks;
+    const unsigned oi = ROWS ? (unsigned)tid / TL : (unsigned)tid % OT;
+    const unsigned tl = ROWS ? (unsigned)tid % TL : (unsigned)tid / OT;
+    const unsigned out = (ob * OT + oi) * NV;                     // first (or only) drain element of the thread
+    const bool live = out < S.n_out;
+    int o[NK_MAX_RANK];
+    nd_of_flat(A.c0, A.rank, (int)(live ? out : 0), o);
+    int64_t o1 = A.base1, o2 = A.base2;
+    for (int k = 0; k < A.rank; k++) { o1 += o[k] * A.keep1[k]; o2 += o[k] * A.keep2[k]; }
+    const unsigned first = seg * S.seg_terms;
+    unsigned end = first + S.seg_terms;
+    if (end > S.terms) end = S.terms;
+    // mixed-radix position of the lane's first term unit and of the step TL, last reduced axis fastest
+    int idx[NK_MAX_RANK], step[NK_MAX_RANK];
+    {
+        unsigned r = first + tl, q = (unsigned)TL;
+        for (int k = A.nred - 1; k >= 0; k--) {
+            const unsigned e = (unsigned)A.red_extent[k];
+            idx[k] = (int)(r % e); r /= e;
+            step[k] = (int)(q % e); q /= e;
+        }
+    }
+    auto advance = [&]() {
+        int carry = 0;
+        for (int k = A.nred - 1; k >= 0; k--) {
+            idx[k] += step[k] + carry;
+            carry = idx[k] >= A.red_extent[k];
+            if (carry) idx[k] -= A.red_extent[k];
+        }
+    };
+    auto fetch = [&](T (&a)[VW], T (&b)[VW]) {
+        int64_t a1 = o1, a2 = o2;
+        for (int k = 0; k < A.nred; k++) { a1 += idx[k] * A.red1[k]; a2 += idx[k] * A.red2[k]; }
+#pragma unroll
+        for (int v = 0; v < VW; v++) { a[v] = T(0); b[v] = T(0); }
+        if constexpr (G != G_SECOND && G != G_RCP) {
+            if (VW == 1) a[0] = s1[a1];
+            else if (S.splat1) { const T x = s1[a1]; for (int v = 0; v < VW; v++) a[v] = x; }
+            else { const Vec x = *(const Vec*)(s1 + a1); for (int v = 0; v < VW; v++) a[v] = ((const T*)&x)[v]; }
+        }
+        if constexpr (G != G_FIRST) {
+            if (VW == 1) b[0] = s2[a2];
+            else { const Vec x = *(const Vec*)(s2 + a2); for (int v = 0; v < VW; v++) b[v] = ((const T*)&x)[v]; }
+        }
+    };
+    T value[NV];
+#pragma unroll
+    for (int v = 0; v < NV; v++) value[v] = T(0);
+    auto add = [&](const T (&a)[VW], const T (&b)[VW]) {
+#pragma unroll
+        for (int v = 0; v < VW; v++) {
+            T& sum = value[ROWS ? 0 : v];
+            sum = sum + derive_term<T, G>(a[v], b[v]);
+        }
+    };
+    unsigned t = first + tl;
+    for (; t + (U - 1) * TL < end; t += U * TL) {                // U loads in flight, added in the order they were requested
+        T a[U][VW], b[U][VW];
+#pragma unroll
+        for (int u = 0; u < U; u++) { fetch(a[u], b[u]); advance(); }
+#pragma unroll
+        for (int u = 0; u < U; u++) add(a[u], b[u]);
+    }
+    for (; t < end; t += TL) {
+        T a[VW], b[VW];
+        fetch(a, b); advance();
+        add(a, b);
+    }
+#pragma unroll
+    for (int v = 0; v < NV; v++) part[v][tid] = live ? value[v] : T(0);
+    __syncthreads();
+    if (ROWS) {
+        for (int w = TL / 2; w >= 1; w >>= 1) {
+            if ((int)tl < w) part[0][tid] = part[0][tid] + part[0][tid + w];
+            __syncthreads();
+        }
+    } else {
+        for (int w = 128; w >= OT; w >>= 1) {
+            if (tid < w)
+#pragma unroll
+                for (int v = 0; v < NV; v++) part[v][tid] = part[v][tid] + part[v][tid + w];
+            __syncthreads();
+        }
+    }
+    if (tl == 0 && live) {
+        T* dst = S.segments == 1 ? drn + phys_of_nd(A.c0, A.rank, o) : partial + (int64_t)seg * S.n_out + out;
+#pragma unroll
+        for (int v = 0; v < NV; v++) dst[v] = part[v][tid];      // NV > 1: the drain is contiguous along these elements
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void broadcast_bwd_segments_kernel(Cfg c0, int rank, unsigned n_out, int segments, const T* __restrict__ partial,
+                                                                     T* __restrict__ drn) {
+    const unsigned out = blockIdx.x * blockDim.x + threadIdx.x;
+    if (out >= n_out) return;
+    T s = T(0);
+    int k = 0;
+    for (; k + 8 <= segments; k += 8) {             // eight loads in flight, added in segment order
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = partial[(int64_t)(k + u) * n_out + out];
+#pragma unroll
+        for (int u = 0; u < 8; u++) s = s + v[u];
+    }
+    for (; k < segments; k++) s = s + partial[(int64_t)k * n_out + out];
+    drn[phys_of_flat(c0, rank, (int)out)] = s;
+}
+
 }  // namespace nk
 
 using namespace nk;
@@ -203,6 +342,81 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                      A.c0.shape[last] >= c1.shape[last] && A.keep2[last] == 1 && (A.keep1[last] == 1 || A.keep1[last] == 0) &&
                      env_vec_ok();
     A.n_threads = (unsigned)(vec ? n / V : n);
+    // few outputs with long sums, or the innermost axis reduced: the kernel that splits the sums (another order of
+    // the same terms, see above); everything else keeps the reference's order bit for bit
+    int64_t terms = 1;
+    for (int k = 0; k < A.nred; k++) terms *= A.red_extent[k];
+    const bool last_reduced = A.c0.shape[last] < c1.shape[last];
+    static const bool split_on = [] { const char* v = getenv("NK_BWD_SPLIT"); return !(v && v[0] == '0'); }();
+    if (split_on && terms >= 1024 && terms < ((int64_t)1 << 31) && (last_reduced || A.n_threads < 16384)) {
+        // innermost reduced axis in 16-byte pieces when it is contiguous in the error and contiguous or constant in src1
+        int VT = 1;
+        if (last_reduced) {
+            const int lr = A.nred - 1;
+            if (A.red_extent[lr] % V == 0 && A.red2[lr] == 1 && (A.red1[lr] == 1 || A.red1[lr] == 0)) VT = V;
+        }
+        const int64_t units = terms / VT;
+        const int VO = !last_reduced && vec ? V : 1;                               // neighbouring drain elements per thread
+        // lanes per drain element: by the length of the sums when the innermost axis is reduced; otherwise more lanes
+        // the fewer drain elements there are, so that the blocks of at most 64 segments still fill the machine
+        const int64_t out_threads = n / VO;
+        const int TL = last_reduced ? (units >= 2048 ? 256 : 64) : (out_threads >= 1024 ? 4 : (out_threads >= 256 ? 16 : 64));
+        const int OT = 256 / TL;
+        BwdSplitArgs S{};
+        S.n_out = (unsigned)n; S.terms = (unsigned)units;
+        S.splat1 = last_reduced ? (VT > 1 && A.red1[A.nred - 1] == 0) : (A.keep1[last] == 0);
+        if (VT > 1) { A.red_extent[A.nred - 1] /= VT; A.red1[A.nred - 1] *= VT; A.red2[A.nred - 1] *= VT; }
+        S.out_blocks = (unsigned)((n / VO + OT - 1) / OT);
+        int64_t segs = (2048 + S.out_blocks - 1) / S.out_blocks;                  // enough blocks to fill the machine ...
+        const int64_t most = units / (TL * 8) > 0 ? units / (TL * 8) : 1;         // ... with at least 8 term units per lane
+        if (segs > most) segs = most;
+        if (segs > 64) segs = 64;                                                  // the second launch adds them one after the other
+        if (segs < 1) segs = 1;
+        S.seg_terms = (unsigned)((units + segs - 1) / segs);
+        S.segments = (int)((units + S.seg_terms - 1) / S.seg_terms);
+        void* ws = nullptr;
+        if (S.segments > 1)
+            if (int e = workspace(dev, (uint64_t)S.segments * S.n_out * eb, &ws)) return e;
+        const unsigned grid = S.out_blocks * (unsigned)S.segments;
+        set_path(last_reduced ? (VT > 1 ? "broadcast_backward_split_rows_vec" : "broadcast_backward_split_rows")
+                              : (VO > 1 ? "broadcast_backward_split_vec" : "broadcast_backward_split"));
+        auto split = [&](auto form) {
+            constexpr int G = decltype(form)::value;
+            auto typed = [&](auto zero) {
+                using T = decltype(zero);
+                constexpr int VM = 16 / sizeof(T);
+                T* d_ = (T*)drn; T* w_ = (T*)ws; const T* a_ = (const T*)a; const T* b_ = (const T*)b;
+                if (!last_reduced) {
+                    auto keep = [&](auto ot, auto vw) {
+                        hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, false, decltype(vw)::value>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                    };
+                    using one = std::integral_constant<int, 1>; using wide = std::integral_constant<int, VM>;
+                    if (OT == 64) { if (VO > 1) keep(std::integral_constant<int, 64>{}, wide{}); else keep(std::integral_constant<int, 64>{}, one{}); }
+                    else if (OT == 16) { if (VO > 1) keep(std::integral_constant<int, 16>{}, wide{}); else keep(std::integral_constant<int, 16>{}, one{}); }
+                    else { if (VO > 1) keep(std::integral_constant<int, 4>{}, wide{}); else keep(std::integral_constant<int, 4>{}, one{}); }
+                }
+                else if (TL == 256 && VT > 1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else if (TL == 256)          hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else if (VT > 1)             hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else                         hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                if (S.segments > 1)
+                    hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((S.n_out + 255) / 256), dim3(256), 0, dev->stream, A.c0, rank, S.n_out, S.segments, (const T*)ws, d_);
+            };
+            if (dtype == NK_F32) typed(0.0f); else typed(0.0);
+        };
+        switch (derive_form(op_id, d)) {
+            case G_SUM: split(std::integral_constant<int, G_SUM>{}); break;
+            case G_DIFF: split(std::integral_constant<int, G_DIFF>{}); break;
+            case G_SECOND: split(std::integral_constant<int, G_SECOND>{}); break;
+            case G_FIRST: split(std::integral_constant<int, G_FIRST>{}); break;
+            case G_RCP: split(std::integral_constant<int, G_RCP>{}); break;
+            case G_DDIV: split(std::integral_constant<int, G_DDIV>{}); break;
+            case G_DPOW_A: split(std::integral_constant<int, G_DPOW_A>{}); break;
+            default: split(std::integral_constant<int, G_DPOW_B>{}); break;
+        }
+        NK_HIP(hipGetLastError());
+        return NK_OK;
+    }
     const unsigned blocks = (A.n_threads + 255) / 256;
     set_path(vec ? "broadcast_backward_vec" : "broadcast_backward");
     auto go = [&](auto form) {

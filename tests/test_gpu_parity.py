@@ -459,6 +459,60 @@ def test_broadcast_backward_bit_exact(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_broadcast_backward_split_sums(device, orc, dt):
+    """Gradients with few elements and long sums (a bias, a row sum, a full reduction) or with the innermost axis
+    reduced: blocks split the sums.  Same terms as the reference, another order: |delta| <= tol * sum |terms| against the
+    oracle's sequential sums (tol 1e-5 / 1e-12), exact on integer-valued data."""
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    rng = np.random.default_rng(25)
+    cases = [([48, 40, 128], [1, 1, 128], "broadcast_backward_split_vec"), ([48, 40, 128], [48, 1, 1], "broadcast_backward_split_rows_vec"),
+             ([48, 40, 128], [1, 40, 1], "broadcast_backward_split_rows_vec"), ([48, 40, 128], [1, 1, 1], "broadcast_backward_split_rows_vec"),
+             ([6, 10, 2048], [6, 10, 1], "broadcast_backward_split_rows_vec"), ([5, 3, 1027], [5, 3, 1], "broadcast_backward_split_rows"),
+             ([1100, 700], [1, 700], "broadcast_backward_split_vec"), ([1100, 701], [1, 701], "broadcast_backward_split"),
+             ([30, 2100], [30, 1], "broadcast_backward_split_rows_vec"), ([1100, 2000], [1, 2000], "broadcast_backward_split_vec"),
+             ([19, 300, 1, 70], [1, 300, 1, 1], "broadcast_backward_split_rows")]
+    for full, tgt, path in cases:
+        for integer in (True, False):
+            for op, d in (("add", 0), ("subtract", 1), ("multiply", 0), ("multiply", 1), ("divide", 1)):
+                if integer and op == "divide":
+                    continue
+                if op == "divide":      # the error is the divisor here: keep it away from zero, or single terms dwarf the sum
+                    e = (rng.uniform(0.5, 1.5, full) * rng.choice([-1.0, 1.0], full)).astype(T)
+                else:
+                    e = (rng.integers(-3, 4, full) if integer else rng.uniform(-1, 1, full)).astype(T)
+                te = on(device, e)
+                say("broadcast bwd split", full, tgt, op, d, dt, "integer" if integer else "uniform")
+                if op in ("multiply", "divide"):
+                    other = (rng.integers(1, 4, full) if integer else rng.uniform(0.5, 1.5, full)).astype(T)
+                else:
+                    other = np.zeros(full, dtype=T)
+                drn = Tensor._on_device(device, T, tgt)
+                device.launch_broadcast(op, d, drn, on(device, other), te)
+                assert _lib.last_path().startswith(path), (_lib.last_path(), path)
+                dense_t, dense_f = orc.dense_cfg(tgt), orc.dense_cfg(full)
+                want = orc.broadcast(op, d, np.zeros(drn.size, dtype=T), dense_t, other.reshape(-1), dense_f, e.reshape(-1), dense_f)
+                if integer:
+                    assert_bits(drn.getData(), want, f"{full} {tgt} {op} {d}")
+                else:
+                    # the same sum over the absolute values of the terms bounds the rounding error of any order
+                    mag = orc.broadcast(op, d, np.zeros(drn.size), dense_t, np.abs(other).astype(np.float64).reshape(-1), dense_f,
+                                        np.abs(e).astype(np.float64).reshape(-1), dense_f)
+                    err_abs = np.abs(drn.getData().astype(np.float64) - want)
+                    worst = int(np.argmax(err_abs / (np.abs(mag) + 1e-300)))
+                    assert (err_abs <= tol * np.abs(mag) + 1e-30).all(), (full, tgt, op, d, worst, float(drn.getData()[worst]), float(want[worst]), float(mag[worst]))
+    say("broadcast bwd split on a sliced error and a transposed drain", dt)
+    parent = rng.integers(-3, 4, (50, 44, 140)).astype(T)
+    err = on(device, parent)[1:49, 2:42, 6:134]
+    for tgt in ([1, 1, 128], [48, 1, 1]):
+        drn = Tensor._on_device(device, T, tgt)
+        device.launch_broadcast("add", 0, drn, on(device, np.zeros([48, 40, 128], dtype=T)), err)
+        assert _lib.last_path().startswith("broadcast_backward_split")
+        axes = tuple(k for k in range(3) if tgt[k] == 1)
+        assert_bits(drn.getData().reshape(tgt), parent[1:49, 2:42, 6:134].sum(axis=axes, keepdims=True).astype(T), f"sliced error {tgt}")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_broadcast_backward_vector_path_and_views(device, orc, dt):
     """Drains whose last axis is kept and a multiple of the vector width (16-byte accesses, several drain
     elements per thread), one and two reduced axes, sources of the operands' own shapes as autograd passes
