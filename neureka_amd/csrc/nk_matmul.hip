@@ -9,6 +9,8 @@
 //   mfma_edge  the same kernel for f32 shapes that are not whole tiles, from 2^24 multiply-adds on: clamped
 //            edges, zeroed k tail, element-wise stores along the edges.
 //   mfma_f64 / mfma_f64_edge  f64 from 2^24 multiply-adds on: v_mfma_f64_16x16x4_f64, same tiling.
+//   ..._split  the same kernels for products with fewer tiles than compute units: the k range cut into parts,
+//            partial tiles in the device workspace, added in order by a second launch.
 //   simple   everything else (small products): one thread per element of C, the k loop in the
 //            reference's order with the product rounded before the add, which makes it bit-identical
 //            to GEMM.partial_F32_MxN_RM + AXPY (J/backend/main/operations/linear/internal/blas/GEMM.java:282-304,
@@ -45,13 +47,14 @@ struct MfmaArgs {
     int M, K, N;
     int tiles_m, tiles_n;
     int group_rows;      // tile rows per group of the block-id regrouping
+    int splits;          // SPLIT kernels: parts the k range is cut into (grid = tiles * splits) ...
+    int split_slices;    // ... and k-slices per part
 };
 
-__device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int bid, int& tm, int& tn) {
     // hardware deals consecutive block ids round-robin to the 8 XCDs: give XCD x the x-th contiguous
     // eighth of a grouped ordering (groups of `group_rows` tile rows, walked column by column)
     const int nblk = g.tiles_m * g.tiles_n;
-    int bid = blockIdx.x;
     int logical = bid;
     if (nblk % 8 == 0) logical = (bid % 8) * (nblk / 8) + bid / 8;
     const int per_group = g.group_rows * g.tiles_n;
@@ -79,15 +82,19 @@ constexpr int LDS_FLOATS = LDS_FLOATS_AB > LDS_FLOATS_C ? LDS_FLOATS_AB : LDS_FL
 // matrices (nothing past their end is touched, the range check returns 0 there), rows and columns past the
 // edge are clamped or left as they come (they only feed results that are not stored), and the k tail is zeroed
 // in both operands so that it adds exactly nothing; the epilogue stores element-wise along the edges.
-template <bool EDGE>
+// SPLIT: few tiles (small or thin products): the k range is cut into g.splits parts, block (tile, part) stores its
+// partial tile to P[part] instead of adding it to C, and matmul_add_parts_kernel adds the parts in order.
+template <bool EDGE, bool SPLIT = false>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const float* __restrict__ A,
-                                                          const float* __restrict__ B, float* __restrict__ C) {
+                                                          const float* __restrict__ B, float* __restrict__ C, float* __restrict__ P = nullptr) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     float* const As0 = lds;                                   // [2][BM * A_PITCH]
     float* const Bs0 = lds + 2 * BM * A_PITCH;                // [2][BK * B_PITCH]
 
     int tm, tn;
-    tile_of_block(g, tm, tn);
+    const int n_tiles = g.tiles_m * g.tiles_n;
+    const int part = SPLIT ? (int)blockIdx.x / n_tiles : 0;
+    tile_of_block(g, SPLIT ? (int)blockIdx.x - part * n_tiles : (int)blockIdx.x, tm, tn);
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;     // wave's sub-tile origin inside the block tile
@@ -170,15 +177,19 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     // A buffer is rewritten only after a barrier that every wavefront reaches with all its reads of that
     // buffer complete.
     static_assert(BK == 32, "the pipeline below is written for four depth-8 chunks per slice");
-    const int nk = (g.K + BK - 1) / BK;
+    const int all_slices = (g.K + BK - 1) / BK;
+    const int slice0 = SPLIT ? part * g.split_slices : 0;                           // first k-slice of this block
+    int nk = all_slices;                                                             // ... and how many it takes
+    if (SPLIT) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
+    const int kbase = slice0 * BK;
     Frag f0, f1;
-    load_global(0);
+    load_global(kbase);
     store_lds(0);
     __syncthreads();
     read_frag(f0, 0, 0);
     for (int kt = 0; kt + 1 < nk; kt++) {                  // branch-free body; the last slice is peeled off below
         const int cur = kt & 1;
-        load_global((kt + 1) * BK);
+        load_global(kbase + (kt + 1) * BK);
         read_frag(f1, cur, 1);
         mma(f0);
         read_frag(f0, cur, 2);
@@ -215,7 +226,7 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
                 cs[row * C_PITCH + wn + 32 * j + l32] = acc[i][j][v];
             }
     __syncthreads();
-    float* Cg = C + (int64_t)tm * BM * g.N + tn * BN;
+    float* Cg = (SPLIT ? P + (int64_t)part * g.M * g.N : C) + (int64_t)tm * BM * g.N + tn * BN;
     const int c_col = (tid & 31) * 4, c_row = tid >> 5;
     if (EDGE) {
         const int rows = g.M - tm * BM, cols = g.N - tn * BN;          // what is left of C from this tile's origin
@@ -226,9 +237,15 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
                 const float* add = &cs[r * C_PITCH + c_col];
                 float* dst = Cg + (int64_t)r * g.N + c_col;
 #pragma unroll
-                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = dst[e] + add[e];
+                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = SPLIT ? add[e] : dst[e] + add[e];
             }
         }
+        return;
+    }
+    if (SPLIT) {
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            *(f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col) = *(const f32x4*)(&cs[(c_row + 8 * i) * C_PITCH + c_col]);
         return;
     }
     f32x4 old[16];
@@ -239,6 +256,16 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
         const f32x4 add = *(const f32x4*)(&cs[(c_row + 8 * i) * C_PITCH + c_col]);
         *(f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col) = old[i] + add;
     }
+}
+
+// C[i] += part_0[i] + part_1[i] + ... in that order (the parts of a SPLIT product)
+template <typename T>
+__global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int parts, const T* __restrict__ P, T* __restrict__ C) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    T s = P[i];
+    for (int k = 1; k < parts; k++) s = s + P[(int64_t)k * n + i];
+    C[i] = C[i] + s;
 }
 
 // ---- f64 on the matrix cores ----------------------------------------------------------------------------------
@@ -255,15 +282,17 @@ constexpr int DB_PITCH = BN + 2;
 constexpr int LDS_DOUBLES = 2 * BM * DA_PITCH + 2 * DK * DB_PITCH;
 }
 
-template <bool EDGE>
+template <bool EDGE, bool SPLIT = false>
 __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, const double* __restrict__ A,
-                                                              const double* __restrict__ B, double* __restrict__ C) {
+                                                              const double* __restrict__ B, double* __restrict__ C, double* __restrict__ P = nullptr) {
     using namespace d64;
     __shared__ __attribute__((aligned(16))) double lds[LDS_DOUBLES];
     double* const As0 = lds;                                   // [2][BM * DA_PITCH]
     double* const Bs0 = lds + 2 * BM * DA_PITCH;                // [2][DK * DB_PITCH]
     int tm, tn;
-    tile_of_block(g, tm, tn);
+    const int n_tiles = g.tiles_m * g.tiles_n;
+    const int part = SPLIT ? (int)blockIdx.x / n_tiles : 0;
+    tile_of_block(g, SPLIT ? (int)blockIdx.x - part * n_tiles : (int)blockIdx.x, tm, tn);
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
@@ -312,14 +341,18 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0};
 
-    const int nk = (g.K + DK - 1) / DK;
-    load_global(0);
+    const int all_slices = (g.K + DK - 1) / DK;
+    const int slice0 = SPLIT ? part * g.split_slices : 0;
+    int nk = all_slices;
+    if (SPLIT) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
+    const int kbase = slice0 * DK;
+    load_global(kbase);
     store_lds(0);
     __syncthreads();
     for (int kt = 0; kt < nk; kt++) {
         const int cur = kt & 1;
         const bool more = kt + 1 < nk;
-        if (more) load_global((kt + 1) * DK);
+        if (more) load_global(kbase + (kt + 1) * DK);
         const double* as = As0 + cur * (BM * DA_PITCH);
         const double* bs = Bs0 + cur * (DK * DB_PITCH);
 #pragma unroll
@@ -342,7 +375,7 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
 
     // epilogue: C is accumulated into; a quarter-wavefront covers 16 consecutive doubles of a row
     const int rows = g.M - tm * BM, cols = g.N - tn * BN;
-    double* Cg = C + (int64_t)tm * BM * g.N + tn * BN;
+    double* Cg = (SPLIT ? P + (int64_t)part * g.M * g.N : C) + (int64_t)tm * BM * g.N + tn * BN;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -352,7 +385,7 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
                 const int row = wm + 16 * i + 4 * v + q, col = wn + 16 * j + l16;
                 if (!EDGE || (row < rows && col < cols)) {
                     double* p = Cg + (int64_t)row * g.N + col;
-                    *p = *p + acc[i][j][v];
+                    *p = SPLIT ? acc[i][j][v] : *p + acc[i][j][v];
                 }
             }
 }
@@ -367,25 +400,63 @@ static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* 
     return NK_OK;
 }
 
+// Few tiles cannot fill 256 compute units (a 512^3 product has 16, a matrix-vector product a single row of them):
+// the k range is then cut into parts until there are about two blocks per unit, each part at least four
+// k-slices long; the parts are written to the device workspace and added in order by a second launch.
+static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes) {
+    static const bool on = [] { const char* v = getenv("NK_MATMUL_SPLIT_K"); return !(v && v[0] == '0'); }();
+    const int tiles = g.tiles_m * g.tiles_n, cus = dev->props.multiProcessorCount;
+    const int slices = (g.K + slice - 1) / slice;
+    g.splits = 1; g.split_slices = slices;
+    if (!on || tiles >= cus || slices < 8) return 1;
+    int parts = (2 * cus + tiles - 1) / tiles;
+    if (parts > slices / 4) parts = slices / 4;
+    if (parts > 64) parts = 64;
+    // bound the workspace: parts * M * N elements
+    while (parts > 1 && (uint64_t)parts * g.M * g.N * elem_bytes > ((uint64_t)1 << 30)) parts--;
+    if (parts < 2) return 1;
+    g.split_slices = (slices + parts - 1) / parts;
+    g.splits = (slices + g.split_slices - 1) / g.split_slices;
+    return g.splits;
+}
+
+template <typename T, typename Launch>
+static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch) {
+    const int tiles = g.tiles_m * g.tiles_n;
+    void* ws = nullptr;
+    if (split_plan(dev, g, slice, sizeof(T)) > 1) {
+        const int64_t mn = (int64_t)g.M * g.N;
+        if (int e = workspace(dev, (uint64_t)g.splits * mn * sizeof(T), &ws)) return e;
+        launch(true, dim3((unsigned)(tiles * g.splits)), (T*)ws);
+        hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, dev->stream, mn, g.splits, (const T*)ws, Cp);
+    } else {
+        launch(false, dim3((unsigned)tiles), (T*)nullptr);
+    }
+    NK_HIP(hipGetLastError());
+    return NK_OK;
+}
+
 static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
     static const int64_t mfma_from = [] { const char* v = getenv("NK_MFMA_EDGE_FROM"); return v && *v ? atoll(v) : (int64_t)1 << 24; }();
+    MfmaArgs g{};
+    g.M = (int)M; g.K = (int)K; g.N = (int)N;
+    g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
+    g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
     if (dtype == NK_F64) {
         // from 2^24 multiply-adds on the matrix cores take over (sums re-ordered, within 1e-12 of the reference);
         // smaller products keep the reference's summation order bit for bit
         const bool fits = M * K * 8 < ((int64_t)1 << 32) && K * N * 8 < ((int64_t)1 << 32);
         if (M * K * N >= mfma_from && fits) {
             const bool whole = (A % 16 == 0) && (B % 16 == 0) && M % BM == 0 && N % BN == 0 && K % d64::DK == 0;
-            MfmaArgs g{};
-            g.M = (int)M; g.K = (int)K; g.N = (int)N;
-            g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
-            g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
-            set_path(whole ? "mfma_f64" : "mfma_f64_edge");
-            if (whole) hipLaunchKernelGGL(matmul_mfma_f64_kernel<false>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
-                                          (const double*)A, (const double*)B, (double*)C);
-            else       hipLaunchKernelGGL(matmul_mfma_f64_kernel<true>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
-                                          (const double*)A, (const double*)B, (double*)C);
-            NK_HIP(hipGetLastError());
-            return NK_OK;
+            const double* Ap = (const double*)A; const double* Bp = (const double*)B; double* Cp = (double*)C;
+            const int rc = launch_mfma<double>(dev, g, d64::DK, Cp, [&](bool split, dim3 grid, double* P) {
+                if (whole && split)       hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+                else if (whole)           hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+                else if (split)           hipLaunchKernelGGL((matmul_mfma_f64_kernel<true, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+                else                      hipLaunchKernelGGL((matmul_mfma_f64_kernel<true, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+            });
+            set_path(whole ? (g.splits > 1 ? "mfma_f64_split" : "mfma_f64") : (g.splits > 1 ? "mfma_f64_edge_split" : "mfma_f64_edge"));
+            return rc;
         }
         return launch_simple<double>(dev, M, K, N, (const double*)A, (const double*)B, (double*)C);
     }
@@ -393,22 +464,17 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
     const bool whole_tiles = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
     // Small products stay on the simple kernel, which keeps the reference's summation order bit for bit; from
     // 2^24 multiply-adds on, shapes that are not whole tiles take the matrix cores through the edge variant.
-    const int64_t edge_from = mfma_from;
-    const bool edge = !whole_tiles && M * K * N >= edge_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
+    const bool edge = !whole_tiles && M * K * N >= mfma_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
     if (whole_tiles || edge) {
-        MfmaArgs g{};
-        g.M = (int)M; g.K = (int)K; g.N = (int)N;
-        g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
-        g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
-        set_path(whole_tiles ? "mfma" : "mfma_edge");
-        if (whole_tiles)
-            hipLaunchKernelGGL(matmul_mfma_kernel<false>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
-                               (const float*)A, (const float*)B, (float*)C);
-        else
-            hipLaunchKernelGGL(matmul_mfma_kernel<true>, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(256), 0, dev->stream, g,
-                               (const float*)A, (const float*)B, (float*)C);
-        NK_HIP(hipGetLastError());
-        return NK_OK;
+        const float* Ap = (const float*)A; const float* Bp = (const float*)B; float* Cp = (float*)C;
+        const int rc = launch_mfma<float>(dev, g, BK, Cp, [&](bool split, dim3 grid, float* P) {
+            if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+            else if (whole_tiles)     hipLaunchKernelGGL((matmul_mfma_kernel<false, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+            else if (split)           hipLaunchKernelGGL((matmul_mfma_kernel<true, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+            else                      hipLaunchKernelGGL((matmul_mfma_kernel<true, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+        });
+        set_path(whole_tiles ? (g.splits > 1 ? "mfma_split" : "mfma") : (g.splits > 1 ? "mfma_edge_split" : "mfma_edge"));
+        return rc;
     }
     return launch_simple<float>(dev, M, K, N, (const float*)A, (const float*)B, (float*)C);
 }
