@@ -10,8 +10,8 @@
 //   literal        any rank / layout / view: one thread per drain element, the sum in the reference's
 //                  order with rounded products, bit-identical to the CPU device.  The gradient only
 //                  visits the e-range that can pass the bounds test (skipped terms add +0).
-//   split          the same terms for few drain elements with long sums (at least 1024 terms, at most 2^18
-//                  elements): a block per element, re-ordered sum.
+//   split          the same terms where one thread per drain element would leave the machine idle (long sums into few
+//                  elements): a wavefront or a block per element, in segments if need be; re-ordered sum.
 //   chan_fwd/dx/dk rank 3, dense row-major f32, full reduction over axis 0 (channels), square taps of extent
 //                  2, 3, 4, 5 or 7: [C,H,W] x [C,k,k] -> [1,H-k+1,W-k+1] and its two gradients, register
 //                  sliding-window kernels (see below); sums are re-ordered, results agree with the reference
@@ -108,71 +108,96 @@ __global__ __launch_bounds__(256) void conv_bwd_literal(ConvArgs A, T* __restric
 // order memory runs in for row-major operands -- and their partial sums meet in a fixed LDS tree.  Each thread
 // steps its nd term index by 256 with a mixed-radix add (no division inside the loop).  Same terms as the
 // literal kernels, another order: results agree with the reference norm-wise, not bit for bit.
-template <typename T, bool BWD, int RANK>
-__global__ __launch_bounds__(256) void conv_split(ConvArgs A, T* __restrict__ drn, const T* __restrict__ s1,
-                                                  const T* __restrict__ s2) {
+// GS lanes per drain element: 256 (a block) or 64 (a wavefront, four elements per block) for sums that are only a
+// few hundred terms long.  SEG: the terms of an element are cut into gridDim.y segments whose partial sums go to
+// `partial` and are added in order by conv_split_finish (very few elements, very long sums: a tap gradient).
+struct SplitArgs {
+    unsigned per_xcd;        // element groups per XCD (the grid's x extent is 8 * per_xcd)
+    unsigned seg_terms;      // SEG: terms per segment
+};
+
+template <typename T, bool BWD, int RANK, int GS, bool SEG>
+__global__ __launch_bounds__(256) void conv_split(ConvArgs A, SplitArgs S, T* __restrict__ drn, T* __restrict__ partial,
+                                                  const T* __restrict__ s1, const T* __restrict__ s2) {
+    constexpr int EPB = 256 / GS;                   // drain elements per block
     __shared__ T part[256];
     const int tid = threadIdx.x;
+    const unsigned lane = (unsigned)tid % GS, sub = (unsigned)tid / GS;
     const int rank = RANK ? RANK : A.rank;          // RANK = 0: any rank up to NK_MAX_RANK
     constexpr int NR = RANK ? RANK : NK_MAX_RANK;
     // consecutive block ids go round-robin to the 8 XCDs: give every XCD one contiguous eighth of the drain, so that
-    // neighbouring drain elements, whose terms overlap, share that XCD's L2 (the grid is 8 * ceil(n / 8) blocks)
-    const unsigned per_xcd = gridDim.x >> 3;
-    {
-        const unsigned i = (blockIdx.x & 7u) * per_xcd + (blockIdx.x >> 3);
-        if (i >= A.n) return;
-        int o[NR], lo[NR], ext[NR], b1[NR], j[NR], d[NR];
-        nd_of_flat(A.c0, rank, (int)i, o);
-        unsigned terms = 1;
-        for (int k = 0; k < rank; k++) {
-            const int e0 = A.c0.shape[k], e1 = A.c1.shape[k], e2 = A.c2.shape[k];
-            if (!BWD) {
-                b1[k] = e1 >= e2 ? o[k] : 0;
-                lo[k] = e1 <= e2 ? o[k] : 0;                 // start in src2
-                ext[k] = e1 < e2 ? e1 : e2;
-            } else {
-                int l, h;
-                if (e0 > e1) { l = o[k] - e1 + 1; if (l < 0) l = 0; h = o[k] + 1; if (h > e2) h = e2; }
-                else         { l = 0; h = e1 - o[k]; if (h > e2) h = e2; }
-                lo[k] = l;
-                ext[k] = h > l ? h - l : 0;
-                b1[k] = 0;
-            }
-            terms *= (unsigned)ext[k];
+    // neighbouring drain elements, whose terms overlap, share that XCD's L2
+    const unsigned group = (blockIdx.x & 7u) * S.per_xcd + (blockIdx.x >> 3);
+    const unsigned i = group * EPB + sub;
+    const bool live = i < A.n;
+    int o[NR], lo[NR], ext[NR], b1[NR], j[NR], d[NR];
+    nd_of_flat(A.c0, rank, (int)(live ? i : 0), o);
+    unsigned terms = 1;
+    for (int k = 0; k < rank; k++) {
+        const int e0 = A.c0.shape[k], e1 = A.c1.shape[k], e2 = A.c2.shape[k];
+        if (!BWD) {
+            b1[k] = e1 >= e2 ? o[k] : 0;
+            lo[k] = e1 <= e2 ? o[k] : 0;                 // start in src2
+            ext[k] = e1 < e2 ? e1 : e2;
+        } else {
+            int l, h;
+            if (e0 > e1) { l = o[k] - e1 + 1; if (l < 0) l = 0; h = o[k] + 1; if (h > e2) h = e2; }
+            else         { l = 0; h = e1 - o[k]; if (h > e2) h = e2; }
+            lo[k] = l;
+            ext[k] = h > l ? h - l : 0;
+            b1[k] = 0;
         }
-        T value = T(0);
-        if (terms) {
-            unsigned r = (unsigned)tid, q = 256u;
-            for (int k = rank - 1; k >= 0; k--) {
-                j[k] = (int)(r % (unsigned)ext[k]); r /= (unsigned)ext[k];
-                d[k] = (int)(q % (unsigned)ext[k]); q /= (unsigned)ext[k];
-            }
-#pragma unroll 4
-            for (unsigned t = (unsigned)tid; t < terms; t += 256u) {
-                int i1[NR], i2[NR];
-                for (int k = 0; k < rank; k++) {
-                    i2[k] = lo[k] + j[k];
-                    if (!BWD) i1[k] = b1[k] + j[k];
-                    else      i1[k] = A.c0.shape[k] > A.c1.shape[k] ? o[k] - i2[k] : o[k] + i2[k];
-                }
-                const T prod = s1[phys_of_nd(A.c1, rank, i1)] * s2[phys_of_nd(A.c2, rank, i2)];
-                value = value + prod;
-                int carry = 0;
-                for (int k = rank - 1; k >= 0; k--) {
-                    j[k] += d[k] + carry;
-                    carry = j[k] >= ext[k];
-                    if (carry) j[k] -= ext[k];
-                }
-            }
-        }
-        part[tid] = value;
-        __syncthreads();
-        for (int w = 128; w > 0; w >>= 1) {
-            if (tid < w) part[tid] = part[tid] + part[tid + w];
-            __syncthreads();
-        }
-        if (tid == 0) drn[phys_of_nd(A.c0, rank, o)] = part[0];
+        terms *= (unsigned)ext[k];
     }
+    unsigned first = 0, end = terms;
+    if (SEG) {
+        first = blockIdx.y * S.seg_terms;
+        end = first + S.seg_terms < terms ? first + S.seg_terms : terms;
+    }
+    T value = T(0);
+    if (live && first < end) {
+        unsigned r = first + lane, q = (unsigned)GS;
+        for (int k = rank - 1; k >= 0; k--) {
+            j[k] = (int)(r % (unsigned)ext[k]); r /= (unsigned)ext[k];
+            d[k] = (int)(q % (unsigned)ext[k]); q /= (unsigned)ext[k];
+        }
+#pragma unroll 4
+        for (unsigned t = first + lane; t < end; t += (unsigned)GS) {
+            int i1[NR], i2[NR];
+            for (int k = 0; k < rank; k++) {
+                i2[k] = lo[k] + j[k];
+                if (!BWD) i1[k] = b1[k] + j[k];
+                else      i1[k] = A.c0.shape[k] > A.c1.shape[k] ? o[k] - i2[k] : o[k] + i2[k];
+            }
+            const T prod = s1[phys_of_nd(A.c1, rank, i1)] * s2[phys_of_nd(A.c2, rank, i2)];
+            value = value + prod;
+            int carry = 0;
+            for (int k = rank - 1; k >= 0; k--) {
+                j[k] += d[k] + carry;
+                carry = j[k] >= ext[k];
+                if (carry) j[k] -= ext[k];
+            }
+        }
+    }
+    part[tid] = value;
+    __syncthreads();
+    for (int w = GS / 2; w > 0; w >>= 1) {
+        if ((int)lane < w) part[tid] = part[tid] + part[tid + w];
+        __syncthreads();
+    }
+    if (lane == 0 && live) {
+        if (SEG) partial[(int64_t)blockIdx.y * A.n + i] = part[tid];
+        else drn[phys_of_nd(A.c0, rank, o)] = part[tid];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void conv_split_finish(Cfg c0, int rank, unsigned n, int segments, const T* __restrict__ partial, T* __restrict__ drn) {
+    const unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    T s = T(0);
+    for (int k = 0; k < segments; k++) s = s + partial[(int64_t)k * n + i];
+    drn[phys_of_flat(c0, rank, (int)i)] = s;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -735,17 +760,47 @@ static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, n
         for (int k = 0; k < rank; k++) window *= c1.shape[k] < c2.shape[k] ? c1.shape[k] : c2.shape[k];
         if (window < terms) terms = window;
     }
-    if (terms >= 1024 && n <= ((int64_t)1 << 18)) {
+    // one thread per drain element feeds the machine only with many elements or short sums; otherwise a wavefront
+    // (sums of a few hundred terms) or a block per element, and segments when even that gives too few blocks
+    const bool few = n < ((int64_t)1 << 17) && terms >= 128;
+    if ((terms >= 1024 && n <= ((int64_t)1 << 18)) || few) {
+        const int GS = terms >= 2048 ? 256 : 64;
+        const int EPB = 256 / GS;
+        const int64_t groups = (n + EPB - 1) / EPB;
+        SplitArgs S{};
+        S.per_xcd = (unsigned)((groups + 7) / 8);
+        int64_t segs = 1;
+        if (groups < 1024) {
+            segs = (2048 + groups - 1) / groups;
+            const int64_t most = terms / ((int64_t)GS * 8);
+            if (segs > most) segs = most;
+            if (segs > 256) segs = 256;
+            if (segs < 1) segs = 1;
+        }
+        S.seg_terms = (unsigned)((terms + segs - 1) / segs);
+        segs = (terms + S.seg_terms - 1) / S.seg_terms;
+        void* ws = nullptr;
+        if (segs > 1)
+            if (int e = workspace(dev, (uint64_t)segs * n * sizeof(T), &ws)) return e;
         set_path(d < 0 ? "split_fwd" : "split_bwd");
-        const unsigned grid = 8u * (unsigned)((n + 7) / 8);
+        const dim3 grid(8u * S.per_xcd, (unsigned)segs);
         auto go = [&](auto R) {
             constexpr int RANK = decltype(R)::value;
-            if (d < 0) hipLaunchKernelGGL((conv_split<T, false, RANK>), dim3(grid), dim3(256), 0, dev->stream, A, out, s1, s2);
-            else       hipLaunchKernelGGL((conv_split<T, true, RANK>), dim3(grid), dim3(256), 0, dev->stream, A, out, s1, s2);
+            auto sized = [&](auto gs, auto seg) {
+                constexpr int G = decltype(gs)::value;
+                constexpr bool SEG = decltype(seg)::value;
+                if (d < 0) hipLaunchKernelGGL((conv_split<T, false, RANK, G, SEG>), grid, dim3(256), 0, dev->stream, A, S, out, (T*)ws, s1, s2);
+                else       hipLaunchKernelGGL((conv_split<T, true, RANK, G, SEG>), grid, dim3(256), 0, dev->stream, A, S, out, (T*)ws, s1, s2);
+            };
+            if (GS == 256) { if (segs > 1) sized(std::integral_constant<int, 256>{}, std::true_type{}); else sized(std::integral_constant<int, 256>{}, std::false_type{}); }
+            else           { if (segs > 1) sized(std::integral_constant<int, 64>{}, std::true_type{}); else sized(std::integral_constant<int, 64>{}, std::false_type{}); }
         };
         if (rank == 2) go(std::integral_constant<int, 2>{});
         else if (rank == 3) go(std::integral_constant<int, 3>{});
+        else if (rank == 4) go(std::integral_constant<int, 4>{});
         else go(std::integral_constant<int, 0>{});
+        if (segs > 1)
+            hipLaunchKernelGGL(conv_split_finish<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, dev->stream, c0, rank, (unsigned)n, (int)segs, (const T*)ws, out);
         NK_HIP(hipGetLastError());
         return NK_OK;
     }
@@ -759,6 +814,7 @@ static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, n
     };
     if (rank == 2) go(std::integral_constant<int, 2>{});
     else if (rank == 3) go(std::integral_constant<int, 3>{});
+    else if (rank == 4) go(std::integral_constant<int, 4>{});
     else go(std::integral_constant<int, 0>{});
     NK_HIP(hipGetLastError());
     return NK_OK;

@@ -728,7 +728,8 @@ def test_channel_convolution_fast_paths(device, orc, shape):
     e = rng.standard_normal(ys).astype(np.float32)
     tx, tk, te = on(device, x), on(device, k), on(device, e)
     square = ks[1] == ks[2]          # the register-window kernels exist for square taps of extent 2, 3, 4, 5, 7
-    fwd, dxp, dkp = ("chan_fwd", "chan_dx", "chan_dk") if square else ("literal_fwd", "literal_bwd", "literal_bwd")
+    # other tap shapes take the general kernels: one thread per element, or (sums of 128 terms and more into few elements) split sums
+    fwd, dxp, dkp = ("chan_fwd", "chan_dx", "chan_dk") if square else ("literal_fwd", "literal_bwd", "split_bwd")
     say("chan_fwd", xs, ks)
     out = Tensor._on_device(device, np.float32, ys)
     device.launch_convolution(-1, out, tx, tk)
@@ -758,7 +759,8 @@ def test_channel_convolution_fast_paths(device, orc, shape):
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 @pytest.mark.parametrize("shape", [([48, 40, 44], [48, 5, 5]), ([200, 20, 21], [200, 4, 2]), ([4, 60, 70], [4, 4, 2]),
-                                   ([80, 90], [40, 45]), ([30, 1100, 1], [1, 1100, 20]), ([2, 3, 44, 34], [2, 3, 6, 5])])
+                                   ([80, 90], [40, 45]), ([30, 1100, 1], [1, 1100, 20]), ([2, 3, 44, 34], [2, 3, 6, 5]),
+                                   ([300, 310], [5, 5]), ([3, 8, 20, 20], [1, 8, 5, 5]), ([6, 40, 40], [1, 3, 3])])
 def test_convolution_split_sums(device, orc, shape, dt):
     """Few drain elements with sums of 1024 terms or more: a block per element adds the reference's terms in another
     order.  Norm-wise |delta| <= tol * sum|a||b| per output (tol 1e-5 / 1e-12), exact on integer-valued data; every
