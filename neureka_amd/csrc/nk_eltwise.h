@@ -253,6 +253,7 @@ struct RowsArgs {
     unsigned row_groups;       // groups of (256 >> tpr_log2) rows
     int pass_rows;             // a block's passes walk down the rows (same chunk) instead of along the chunks
     unsigned const_last;       // bit j: source j has stride 0 along the innermost axis
+    unsigned strided_last;     // bit j: source j has a stride other than 0 or 1 along the innermost axis (every n-th column)
     int simple_loads;          // every source register is filled by a plain vector load
     int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
     int ragged;                // L is not a multiple of vec: the last vector of a row is moved back to end with the row
@@ -262,6 +263,7 @@ struct RowsArgs {
     FastDiv outer[ROWS_MAX_OUTER];           // outer[0] is the innermost outer axis
     int base[MAX_OPERANDS];
     int stride[MAX_OPERANDS][ROWS_MAX_OUTER];
+    int last_stride[MAX_OPERANDS];           // innermost stride of every operand (1 for the drain)
 };
 
 // addressing shared by the rows kernels: unit -> (row, col), row -> element offset of every operand
@@ -355,6 +357,10 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
                         const T c = *sp;
 #pragma unroll
                         for (int v = 0; v < V; v++) xj[v] = c;
+                    } else if ((A.strided_last >> j) & 1u) {
+                        const int ls = A.last_stride[j + 1];
+#pragma unroll
+                        for (int v = 0; v < V; v++) xj[v] = sp[(int)(R.col + v) * ls];
                     } else {
                         load_vec<T, V>(xj, sp + R.col);
                     }

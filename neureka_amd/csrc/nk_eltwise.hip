@@ -187,7 +187,11 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     if (cn.rank == 0) { cn.rank = 1; cn.shape[0] = 1; for (int o = 0; o <= c.nsrc; o++) cn.stride[o][0] = 1; }
     const int last = cn.rank - 1;
     bool rows_ok = cn.stride[0][last] == 1 && cn.rank - 1 <= ROWS_MAX_OUTER;
-    for (int j = 0; j < c.nsrc; j++) rows_ok = rows_ok && (cn.stride[j + 1][last] == 0 || cn.stride[j + 1][last] == 1);
+    // sources may also take every n-th column (a gather per element; the drain is still written in whole vectors)
+    static const bool strided_ok = env_flag("NK_ROWS_STRIDED_SOURCES", true);
+    for (int j = 0; j < c.nsrc; j++)
+        rows_ok = rows_ok && (cn.stride[j + 1][last] == 0 || cn.stride[j + 1][last] == 1 ||
+                              (strided_ok && cn.stride[j + 1][last] > 1 && cn.stride[j + 1][last] <= 8));
     bool done = false;
 
     // the rows kernel keeps element offsets in 32 bits: every reachable offset must fit
@@ -242,7 +246,13 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         if (deep) once = false;
         A.nt_loads = once ? 1 : 0;
         A.const_last = 0;
-        for (int j = 0; j < c.nsrc; j++) if (cn.stride[j + 1][last] == 0) A.const_last |= 1u << j;
+        A.strided_last = 0;
+        for (int j = 0; j < c.nsrc; j++) {
+            if (cn.stride[j + 1][last] == 0) A.const_last |= 1u << j;
+            else if (cn.stride[j + 1][last] != 1) A.strided_last |= 1u << j;
+            A.last_stride[j + 1] = (int)cn.stride[j + 1][last];
+        }
+        A.last_stride[0] = 1;
         uint64_t n_rows = 1;
         // kernel axis k counts outward from the innermost outer axis
         for (int k = 0; k < last; k++) { n_rows *= cn.shape[k]; A.outer[k] = FastDiv((unsigned)cn.shape[last - 1 - k]); }
@@ -263,11 +273,11 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         }
         A.vec = V;
         A.ragged = ragged ? 1 : 0;
-        A.simple_loads = (funset < 2 && A.const_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
+        A.simple_loads = (funset < 2 && A.const_last == 0 && A.strided_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel
         // (sources that are constant along a row are handled by that kernel's vector variant only)
-        const bool loads_ok = A.simple_loads || (A.const_last != 0 && vec && env_flag("NK_BINARY_ROW_CONSTANT", true));
+        const bool loads_ok = A.simple_loads || (A.const_last != 0 && A.strided_last == 0 && vec && env_flag("NK_BINARY_ROW_CONSTANT", true));
         if (loads_ok && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
             prog.op[1] == I_BIN && prog.src[1] == 1 && prog.arg[1] <= NK_OP_DIV) {
             plan.kind = PLAN_ROWS_BINARY;

@@ -402,6 +402,29 @@ def test_ragged_rows_run_on_vectors_and_stay_bit_exact(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_sources_that_take_every_nth_column(device, orc, dt):
+    """Step slices along the innermost axis: the rows kernels gather the source element by element and still write the
+    drain in whole vectors."""
+    rng = np.random.default_rng(26)
+    T = F[dt]
+    a = rng.uniform(-2, 2, (33, 200)).astype(T); b = rng.uniform(-2, 2, (33, 200)).astype(T)
+    ta, tb = on(device, a), on(device, b)
+    for sl in (np.s_[:, ::2], np.s_[1:30, 1::3], np.s_[::2, 4:196:8]):
+        va, vb = ta[sl], tb[sl]
+        say("every n-th column", sl, dt)
+        out = Tensor._on_device(device, T, va.shape)
+        device.launch_activation("softsign", -1, out, va)
+        assert _lib.last_path() in ("rows_vec", "rows"), _lib.last_path()
+        x = np.ascontiguousarray(a[sl]); dense = orc.dense_cfg(list(x.shape))
+        assert_bits(out.getData(), orc.activation("softsign", -1, np.zeros(x.size, dtype=T), dense, x.reshape(-1), dense), "softsign")
+        device.launch_elementwise("multiply", -1, out, va, vb)
+        assert _lib.last_path() in ("rows_vec", "rows"), _lib.last_path()
+        assert_bits(out.getData().reshape(x.shape), a[sl] * b[sl], "multiply")
+        device.launch_elementwise("subtract", -1, out, va, on(device, np.ascontiguousarray(b[sl])))     # one strided, one dense
+        assert_bits(out.getData().reshape(x.shape), a[sl] - b[sl], "subtract")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_deep_index_spaces_and_row_constant_sources(device, orc, dt):
     """Four and five outer axes that do not merge (alternating broadcast axes, slices on every axis) and sources that
     are constant along a row (outer products, per-row scales): the vector kernels with every outer axis resolved,
