@@ -348,7 +348,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
     for (int k = 0; k < A.nred; k++) terms *= A.red_extent[k];
     const bool last_reduced = A.c0.shape[last] < c1.shape[last];
     static const bool split_on = [] { const char* v = getenv("NK_BWD_SPLIT"); return !(v && v[0] == '0'); }();
-    if (split_on && terms >= 1024 && terms < ((int64_t)1 << 31) && (last_reduced || A.n_threads < 16384)) {
+    if (split_on && terms < ((int64_t)1 << 31) && ((last_reduced && terms >= 512) || (terms >= 1024 && A.n_threads < 16384))) {
         // innermost reduced axis in 16-byte pieces when it is contiguous in the error and contiguous or constant in src1
         int VT = 1;
         if (last_reduced) {
@@ -360,7 +360,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         // lanes per drain element: by the length of the sums when the innermost axis is reduced; otherwise more lanes
         // the fewer drain elements there are, so that the blocks of at most 64 segments still fill the machine
         const int64_t out_threads = n / VO;
-        const int TL = last_reduced ? (units >= 2048 ? 256 : 64) : (out_threads >= 1024 ? 4 : (out_threads >= 256 ? 16 : 64));
+        const int TL = last_reduced ? (units >= 2048 ? 256 : (units >= 512 ? 64 : 16)) : (out_threads >= 1024 ? 4 : (out_threads >= 256 ? 16 : 64));
         const int OT = 256 / TL;
         BwdSplitArgs S{};
         S.n_out = (unsigned)n; S.terms = (unsigned)units;
@@ -397,8 +397,10 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                 }
                 else if (TL == 256 && VT > 1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                 else if (TL == 256)          hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else if (VT > 1)             hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else                         hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else if (TL == 64 && VT > 1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else if (TL == 64)           hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else if (VT > 1)             hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 16, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else                         hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 16, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                 if (S.segments > 1)
                     hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((S.n_out + 255) / 256), dim3(256), 0, dev->stream, A.c0, rank, S.n_out, S.segments, (const T*)ws, d_);
             };

@@ -491,7 +491,8 @@ def test_broadcast_backward_split_sums(device, orc, dt):
     rng = np.random.default_rng(25)
     cases = [([48, 40, 128], [1, 1, 128], "broadcast_backward_split_vec"), ([48, 40, 128], [48, 1, 1], "broadcast_backward_split_rows_vec"),
              ([48, 40, 128], [1, 40, 1], "broadcast_backward_split_rows_vec"), ([48, 40, 128], [1, 1, 1], "broadcast_backward_split_rows_vec"),
-             ([6, 10, 2048], [6, 10, 1], "broadcast_backward_split_rows_vec"), ([5, 3, 1027], [5, 3, 1], "broadcast_backward_split_rows"),
+             ([6, 10, 2048], [6, 10, 1], "broadcast_backward_split_rows_vec"), ([6, 10, 512], [6, 10, 1], "broadcast_backward_split_rows_vec"),
+             ([7, 9, 515], [7, 9, 1], "broadcast_backward_split_rows"), ([5, 3, 1027], [5, 3, 1], "broadcast_backward_split_rows"),
              ([1100, 700], [1, 700], "broadcast_backward_split_vec"), ([1100, 701], [1, 701], "broadcast_backward_split"),
              ([30, 2100], [30, 1], "broadcast_backward_split_rows_vec"), ([1100, 2000], [1, 2000], "broadcast_backward_split_vec"),
              ([19, 300, 1, 70], [1, 300, 1, 1], "broadcast_backward_split_rows")]
