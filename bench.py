@@ -316,6 +316,12 @@ def main():
         k1 = Tensor.of(f32, (3, 3), rng.uniform(-1, 1, 9).astype(f32)).to(dev)
         y1 = Tensor._on_device(dev, f32, (62, 62))
         flops("conv2d_64x64_3x3", 69192, 31796, dev.prepared_launch("convolution", -1, y1, x1, k1))
+        # the same operation on an image large enough to fill the machine
+        xl = Tensor.of(f32, (2048, 2048), rng.uniform(-1, 1, 2048 * 2048).astype(f32)).to(dev)
+        kl = Tensor.of(f32, (5, 5), rng.uniform(-1, 1, 25).astype(f32)).to(dev)
+        yl = Tensor._on_device(dev, f32, (2044, 2044))
+        flops("conv2d_2048x2048_5x5", 2.0 * 2044 * 2044 * 25, 4 * (2048 * 2048 + 25 + 2044 * 2044), dev.prepared_launch("convolution", -1, yl, xl, kl))
+        for t in (xl, kl, yl): dev.free(t)
         x5 = Tensor.of(f32, (64, 256, 256), (rng.standard_normal(64 * 256 * 256) * 0.1).astype(f32)).to(dev)
         k5 = Tensor.of(f32, (64, 5, 5), (rng.standard_normal(1600) * 0.1).astype(f32)).to(dev)
         y5 = Tensor._on_device(dev, f32, (1, 252, 252))

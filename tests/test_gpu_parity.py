@@ -836,6 +836,23 @@ def test_convolution_split_sums(device, orc, shape, dt):
         assert_bits(dk.getData(), want, "transposed operand")
 
 
+@pytest.mark.parametrize("shape", [([300, 523], [5, 5]), ([3, 200, 300], [1, 3, 3]), ([130, 700], [7, 7]), ([260, 257], [2, 2]), ([2, 190, 261], [1, 4, 4])])
+def test_conv2d_large_images_bit_exact(device, orc, shape):
+    """Large f32 images with square taps take the register-window kernel: the same products, rounded and added in
+    SimpleCPUConvolution's order (ky outer, kx inner) -- bit for bit."""
+    xs, ks = shape
+    rng = np.random.default_rng(45)
+    x = rng.uniform(-1, 1, xs).astype(np.float32); k = rng.uniform(-1, 1, ks).astype(np.float32)
+    say("conv2d window", xs, ks)
+    y = on(device, x).conv(on(device, k))
+    assert _lib.last_path() == "simple2d_window", _lib.last_path()
+    B = xs[0] if len(xs) == 3 else 1
+    want = orc.simple_conv2d(x.reshape(-1), k.reshape(-1), xs[-1], xs[-2], ks[-1], ks[-2], batch=B)
+    assert_bits(y.items, want, f"{xs} x {ks}")
+    y2 = on(device, k).conv(on(device, x))                        # taps first
+    assert_bits(y2.items, want, "operand order")
+
+
 def test_conv2d_config1_shape(device, orc):
     """[64,64] x [3,3] -> [62,62] (the reference runs this on SimpleCPUConvolution: ky outer, kx inner)."""
     say("conv2d 64x64 x 3x3")
