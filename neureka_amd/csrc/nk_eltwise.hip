@@ -451,7 +451,11 @@ int nk_scalarization(nk_dev dev, int op_id, int d, int dtype, int rank, nk_buf d
     ProgBuilder b;
     b.p.consts[0] = value;
     b.emit(I_SET, 0, 0);
-    if (d < 0) b.emit(I_BIN, op_id, SRC_CONST0);
+    // x ** 2 is the correctly rounded product (exact in double for a float x, what Math.pow returns) and x ** 1 is x by
+    // Math.pow's specification: both leave the heavy power kernels for the streaming ones
+    if (d < 0 && op_id == NK_OP_POW && value == 2.0) b.emit(I_BIN, NK_OP_MUL, 0);
+    else if (d < 0 && op_id == NK_OP_POW && value == 1.0) { /* a copy */ }
+    else if (d < 0) b.emit(I_BIN, op_id, SRC_CONST0);
     else b.emit(I_DBIN, op_id * 2 + d, SRC_CONST0);
     EltCall c{};
     c.name = "nk_scalarization"; c.dtype = dtype; c.rank = rank; c.nsrc = 1;

@@ -52,15 +52,25 @@ template <> struct Num<double> {
 // double; implementations/elementwise/CPUBiElementWisePower.java:11,21,31, CPUBiElementWiseDivision.java:31,
 // CPUBiElementWiseModulo.java:31 and the broadcast twins): the intermediates neither overflow nor underflow
 // where float ones would.
-__device__ __forceinline__ double pow_ref(double a, double b) { return ::pow(a, b); }
-__device__ __forceinline__ float pow_ref(float a, float b) { return (float)::pow((double)a, (double)b); }
-__device__ __forceinline__ double dpow_da_ref(double a, double b) { return b * ::pow(a, b - 1); }
-__device__ __forceinline__ float dpow_da_ref(float a, float b) { return (float)((double)b * ::pow((double)a, (double)(b - 1.0f))); }
+// The exponents that dominate in practice have exact answers that need no general pow (which costs some hundred
+// double-precision instructions): Math.pow returns its first argument for an exponent of 1 and 1.0 for an exponent
+// of zero by specification, and a square is the correctly rounded product (exact in double for a float base) --
+// what a correctly rounded pow returns and what HotSpot substitutes for pow(x, 2.0).
+__device__ __forceinline__ double pow_double(double a, double b) {
+    if (b == 2.0) return a * a;
+    if (b == 1.0) return a;
+    if (b == 0.0) return 1.0;
+    return ::pow(a, b);
+}
+__device__ __forceinline__ double pow_ref(double a, double b) { return pow_double(a, b); }
+__device__ __forceinline__ float pow_ref(float a, float b) { return (float)pow_double((double)a, (double)b); }
+__device__ __forceinline__ double dpow_da_ref(double a, double b) { return b * pow_double(a, b - 1); }
+__device__ __forceinline__ float dpow_da_ref(float a, float b) { return (float)((double)b * pow_double((double)a, (double)(b - 1.0f))); }
 // the broadcast twin multiplies by a, not by b (implementations/broadcast/CPUBroadcastPower.java:20-21)
-__device__ __forceinline__ double bcast_dpow_da_ref(double a, double b) { return a * ::pow(a, b - 1); }
-__device__ __forceinline__ float bcast_dpow_da_ref(float a, float b) { return (float)((double)a * ::pow((double)a, (double)(b - 1.0f))); }
-__device__ __forceinline__ double dpow_db_ref(double a, double b) { return ::pow(a, b) * ::log(a); }
-__device__ __forceinline__ float dpow_db_ref(float a, float b) { return (float)(::pow((double)a, (double)b) * ::log((double)a)); }
+__device__ __forceinline__ double bcast_dpow_da_ref(double a, double b) { return a * pow_double(a, b - 1); }
+__device__ __forceinline__ float bcast_dpow_da_ref(float a, float b) { return (float)((double)a * pow_double((double)a, (double)(b - 1.0f))); }
+__device__ __forceinline__ double dpow_db_ref(double a, double b) { return pow_double(a, b) * ::log(a); }
+__device__ __forceinline__ float dpow_db_ref(float a, float b) { return (float)(pow_double((double)a, (double)b) * ::log((double)a)); }
 __device__ __forceinline__ double ddiv_db_ref(double a, double b) { return -(a / (b * b)); }
 __device__ __forceinline__ float ddiv_db_ref(float a, float b) { return (float)-((double)a / ((double)b * (double)b)); }   // b*b is exact in double
 

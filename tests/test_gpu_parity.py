@@ -402,6 +402,29 @@ def test_ragged_rows_run_on_vectors_and_stay_bit_exact(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_square_and_first_power_are_exact_products(device, orc, dt):
+    """x ** 2 and x ** 1 with a scalar exponent leave the power kernels: the square is the correctly rounded product
+    (what Math.pow returns: the exact product of two floats fits a double), the first power is x itself
+    (Math.pow's specification).  Special values included; other exponents still go through pow."""
+    T = F[dt]
+    rng = np.random.default_rng(27)
+    x = np.concatenate([rng.uniform(-3, 3, 1000), [0.0, -0.0, np.inf, -np.inf, np.nan, 1e30, -1e30, 1e-30, 3e-39]]).astype(T)
+    tx = on(device, x)
+    cfg1 = orc.dense_cfg([x.size])
+    for value in (2.0, 1.0, 3.0, 0.0, -1.0):
+        say("x **", value, dt)
+        out = Tensor._on_device(device, T, (x.size,))
+        device.launch_scalarization("power", -1, out, tx, value)
+        with np.errstate(all="ignore"):
+            want = orc.scalarization("power", -1, np.zeros_like(x), cfg1, x, cfg1, value)
+            if value == 2.0:
+                assert_bits(out.getData(), x * x, "square")
+            if value == 1.0:
+                assert_bits(out.getData(), x, "first power")
+        assert_close(out.getData(), want, f"x ** {value}")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_sources_that_take_every_nth_column(device, orc, dt):
     """Step slices along the innermost axis: the rows kernels gather the source element by element and still write the
     drain in whole vectors."""
