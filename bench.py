@@ -109,8 +109,8 @@ def cpu_side_of_the_other_configs(cores):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the figures of the other configurations")
     ap.add_argument("--calibrate", action="store_true",
@@ -206,7 +206,7 @@ def main():
     # ---- the other configurations: kernel figures only ------------------------------------------------------
     others = {}
     if not args.no_others:
-        reps = max(50, args.steps)                             # after 10 warm-up launches each
+        reps = max(50, min(args.steps, 100))                   # after 10 warm-up launches each
 
         def warm(launch):
             for _ in range(10):
