@@ -209,8 +209,11 @@ def main():
         reps = max(50, min(args.steps, 100))                   # after 10 warm-up launches each
 
         def warm(launch):
-            for _ in range(10):
+            # at least 10 launches and about 5 ms of queued work: the clock needs a few milliseconds of load to settle
+            t0, count = time.perf_counter(), 0
+            while count < 10 or (time.perf_counter() - t0 < 0.005 and count < 2000):
                 launch()
+                count += 1
             dev.sync()
 
         def hbm(name, nbytes, launch):
