@@ -266,22 +266,23 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
     }
 }
 
+// partial[segment][element] -> drain: sixteen lanes per element take every sixteenth segment and meet in LDS
 template <typename T>
 __global__ __launch_bounds__(256) void broadcast_bwd_segments_kernel(Cfg c0, int rank, unsigned n_out, int segments, const T* __restrict__ partial,
                                                                      T* __restrict__ drn) {
-    const unsigned out = blockIdx.x * blockDim.x + threadIdx.x;
-    if (out >= n_out) return;
+    __shared__ T part[256];
+    const int tid = threadIdx.x;
+    const unsigned lane = (unsigned)tid & 15u, out = blockIdx.x * 16u + ((unsigned)tid >> 4);
     T s = T(0);
-    int k = 0;
-    for (; k + 8 <= segments; k += 8) {             // eight loads in flight, added in segment order
-        T v[8];
-#pragma unroll
-        for (int u = 0; u < 8; u++) v[u] = partial[(int64_t)(k + u) * n_out + out];
-#pragma unroll
-        for (int u = 0; u < 8; u++) s = s + v[u];
+    if (out < n_out)
+        for (int k = (int)lane; k < segments; k += 16) s = s + partial[(int64_t)k * n_out + out];
+    part[tid] = s;
+    __syncthreads();
+    for (int w = 8; w >= 1; w >>= 1) {
+        if ((int)lane < w) part[tid] = part[tid] + part[tid + w];
+        __syncthreads();
     }
-    for (; k < segments; k++) s = s + partial[(int64_t)k * n_out + out];
-    drn[phys_of_flat(c0, rank, (int)out)] = s;
+    if (lane == 0 && out < n_out) drn[phys_of_flat(c0, rank, (int)out)] = part[tid];
 }
 
 }  // namespace nk
@@ -358,9 +359,9 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         const int64_t units = terms / VT;
         const int VO = !last_reduced && vec ? V : 1;                               // neighbouring drain elements per thread
         // lanes per drain element: by the length of the sums when the innermost axis is reduced; otherwise more lanes
-        // the fewer drain elements there are, so that the blocks of at most 64 segments still fill the machine
+        // the fewer drain elements there are, so that the blocks of at most 256 segments still fill the machine
         const int64_t out_threads = n / VO;
-        const int TL = last_reduced ? (units >= 2048 ? 256 : (units >= 512 ? 64 : 16)) : (out_threads >= 1024 ? 4 : (out_threads >= 256 ? 16 : 64));
+        const int TL = last_reduced ? (units >= 2048 ? 256 : (units >= 512 ? 64 : 16)) : (out_threads >= 1024 ? 4 : 16);
         const int OT = 256 / TL;
         BwdSplitArgs S{};
         S.n_out = (unsigned)n; S.terms = (unsigned)units;
@@ -370,7 +371,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         int64_t segs = (2048 + S.out_blocks - 1) / S.out_blocks;                  // enough blocks to fill the machine ...
         const int64_t most = units / (TL * 8) > 0 ? units / (TL * 8) : 1;         // ... with at least 8 term units per lane
         if (segs > most) segs = most;
-        if (segs > 64) segs = 64;                                                  // the second launch adds them one after the other
+        if (segs > 256) segs = 256;
         if (segs < 1) segs = 1;
         S.seg_terms = (unsigned)((units + segs - 1) / segs);
         S.segments = (int)((units + S.seg_terms - 1) / S.seg_terms);
@@ -392,8 +393,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                     };
                     using one = std::integral_constant<int, 1>; using wide = std::integral_constant<int, VM>;
                     if (OT == 64) { if (VO > 1) keep(std::integral_constant<int, 64>{}, wide{}); else keep(std::integral_constant<int, 64>{}, one{}); }
-                    else if (OT == 16) { if (VO > 1) keep(std::integral_constant<int, 16>{}, wide{}); else keep(std::integral_constant<int, 16>{}, one{}); }
-                    else { if (VO > 1) keep(std::integral_constant<int, 4>{}, wide{}); else keep(std::integral_constant<int, 4>{}, one{}); }
+                    else { if (VO > 1) keep(std::integral_constant<int, 16>{}, wide{}); else keep(std::integral_constant<int, 16>{}, one{}); }
                 }
                 else if (TL == 256 && VT > 1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                 else if (TL == 256)          hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
@@ -402,7 +402,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                 else if (VT > 1)             hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 16, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                 else                         hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 16, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                 if (S.segments > 1)
-                    hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((S.n_out + 255) / 256), dim3(256), 0, dev->stream, A.c0, rank, S.n_out, S.segments, (const T*)ws, d_);
+                    hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((S.n_out + 15) / 16), dim3(256), 0, dev->stream, A.c0, rank, S.n_out, S.segments, (const T*)ws, d_);
             };
             if (dtype == NK_F32) typed(0.0f); else typed(0.0);
         };
