@@ -149,8 +149,8 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
 // One thread per drain element cannot feed the machine when a gradient has few elements (a bias: 512 sums of
 // 131 072 terms) or when the reduced axis is the contiguous one (every thread would walk its own row).  Here a
 // block owns OT neighbouring drain elements and one segment of their sums: its 256 threads are TL = 256 / OT lanes
-// per element; the lanes of an element take every TL-th term of the segment -- terms enumerated with the last
-// reduced axis fastest, the order memory runs in -- and meet in LDS.
+// per element; lane l of segment s takes the terms s * TL + l, then every (segments * TL)-th -- terms enumerated
+// with the last reduced axis fastest, the order memory runs in -- and the lanes meet in LDS.
 //   ROWS = false (the drain keeps the innermost axis): OT = 64, neighbouring threads own neighbouring drain elements,
 //                so a wavefront reads 64 neighbouring elements of the error per term;
 //   ROWS = true  (the innermost axis is reduced): neighbouring threads own neighbouring terms, VT of them each
@@ -159,18 +159,21 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
 // reference's; their order is not: results agree norm-wise (1e-5 / 1e-12).
 struct BwdSplitArgs {
     unsigned n_out, out_blocks;          // drain elements, blocks of OT of them
-    unsigned terms, seg_terms;           // term units (VT terms each) per drain element and per segment
+    unsigned terms, seg_terms;           // term units (VT terms each) per drain element and (host side) per segment
     int segments;
     int splat1;                          // VT > 1: src1 does not move along the innermost reduced axis
 };
 
-template <typename T, int G, int OT, bool ROWS, int VW>
+template <typename T, int G, int OT, bool ROWS, int VW, bool SPLAT = false>
 __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A, BwdSplitArgs S, T* __restrict__ drn, T* __restrict__ partial,
                                                                   const T* __restrict__ s1, const T* __restrict__ s2) {
     // VW: width of the 16-byte accesses -- ROWS: VW neighbouring terms of one drain element per load;
     // otherwise VW neighbouring drain elements per thread
     constexpr int TL = 256 / OT;                                 // term lanes per drain element (group)
     constexpr int U = 4;                                         // loads in flight per lane
+    constexpr int VA = SPLAT ? 1 : VW;                           // values kept per term of src1: one serves all VW when it
+                                                                 // does not move along the vector (a template parameter: a
+                                                                 // run-time test in the term loop costs a quarter of the rate)
     constexpr int NV = ROWS ? 1 : VW;                            // running sums per thread
     typedef typename std::conditional<VW == 1, T, T __attribute__((ext_vector_type(VW == 1 ? 2 : VW), aligned(sizeof(T))))>::type Vec;
     __shared__ T part[NV][256];
@@ -184,62 +187,72 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
     nd_of_flat(A.c0, A.rank, (int)(live ? out : 0), o);
     int64_t o1 = A.base1, o2 = A.base2;
     for (int k = 0; k < A.rank; k++) { o1 += o[k] * A.keep1[k]; o2 += o[k] * A.keep2[k]; }
-    const unsigned first = seg * S.seg_terms;
-    unsigned end = first + S.seg_terms;
-    if (end > S.terms) end = S.terms;
-    // mixed-radix position of the lane's first term unit and of the step TL, last reduced axis fastest
+    // the segments interleave: segment s takes the term units s * TL + tl, then those segments * TL further on, so
+    // that the blocks running at one time read one window of memory together
+    const unsigned first = seg * TL, stride = (unsigned)S.segments * TL, end = S.terms;
+    // mixed-radix position of the lane's first term unit and of its step, last reduced axis fastest; the two
+    // offsets follow it by additions only: a step adds the offset of that many units, a carry out of axis k takes
+    // the axis back to its start and moves axis k - 1 on by one (no multiplication in the term loop)
     int idx[NK_MAX_RANK], step[NK_MAX_RANK];
+    int64_t fix1[NK_MAX_RANK], fix2[NK_MAX_RANK];
+    int64_t a1 = o1, a2 = o2, delta1 = 0, delta2 = 0;
     {
-        unsigned r = first + tl, q = (unsigned)TL;
+        unsigned r = first + tl, q = stride;
         for (int k = A.nred - 1; k >= 0; k--) {
             const unsigned e = (unsigned)A.red_extent[k];
             idx[k] = (int)(r % e); r /= e;
             step[k] = (int)(q % e); q /= e;
+            a1 += idx[k] * A.red1[k]; a2 += idx[k] * A.red2[k];
+            delta1 += step[k] * A.red1[k]; delta2 += step[k] * A.red2[k];
+            fix1[k] = (k > 0 ? A.red1[k - 1] : 0) - (int64_t)e * A.red1[k];
+            fix2[k] = (k > 0 ? A.red2[k - 1] : 0) - (int64_t)e * A.red2[k];
         }
     }
     auto advance = [&]() {
         int carry = 0;
+        a1 += delta1; a2 += delta2;
         for (int k = A.nred - 1; k >= 0; k--) {
             idx[k] += step[k] + carry;
             carry = idx[k] >= A.red_extent[k];
-            if (carry) idx[k] -= A.red_extent[k];
+            if (carry) { idx[k] -= A.red_extent[k]; a1 += fix1[k]; a2 += fix2[k]; }
         }
     };
-    auto fetch = [&](T (&a)[VW], T (&b)[VW]) {
-        int64_t a1 = o1, a2 = o2;
-        for (int k = 0; k < A.nred; k++) { a1 += idx[k] * A.red1[k]; a2 += idx[k] * A.red2[k]; }
+    auto fetch = [&](T (&a)[VA], T (&b)[VW]) {
 #pragma unroll
-        for (int v = 0; v < VW; v++) { a[v] = T(0); b[v] = T(0); }
+        for (int v = 0; v < VA; v++) a[v] = T(0);
+#pragma unroll
+        for (int v = 0; v < VW; v++) b[v] = T(0);
         if constexpr (G != G_SECOND && G != G_RCP) {
-            if (VW == 1) a[0] = s1[a1];
-            else if (S.splat1) { const T x = s1[a1]; for (int v = 0; v < VW; v++) a[v] = x; }
+            if constexpr (VA == 1) a[0] = s1[a1];
             else { const Vec x = *(const Vec*)(s1 + a1); for (int v = 0; v < VW; v++) a[v] = ((const T*)&x)[v]; }
         }
         if constexpr (G != G_FIRST) {
             if (VW == 1) b[0] = s2[a2];
-            else { const Vec x = *(const Vec*)(s2 + a2); for (int v = 0; v < VW; v++) b[v] = ((const T*)&x)[v]; }
+            else { const Vec x = __builtin_nontemporal_load((const Vec*)(s2 + a2)); for (int v = 0; v < VW; v++) b[v] = ((const T*)&x)[v]; }
         }
     };
     T value[NV];
 #pragma unroll
     for (int v = 0; v < NV; v++) value[v] = T(0);
-    auto add = [&](const T (&a)[VW], const T (&b)[VW]) {
+    auto add = [&](const T (&a)[VA], const T (&b)[VW]) {
 #pragma unroll
         for (int v = 0; v < VW; v++) {
             T& sum = value[ROWS ? 0 : v];
-            sum = sum + derive_term<T, G>(a[v], b[v]);
+            sum = sum + derive_term<T, G>(a[VA == 1 ? 0 : v], b[v]);
         }
     };
-    unsigned t = first + tl;
-    for (; t + (U - 1) * TL < end; t += U * TL) {                // U loads in flight, added in the order they were requested
-        T a[U][VW], b[U][VW];
+    const unsigned t = first + tl;
+    const unsigned mine = t < end ? (end - t + stride - 1) / stride : 0;   // term units of this lane
+    unsigned i = 0;
+    for (; i + U <= mine; i += U) {                                  // U loads requested together, added in that order
+        T a[U][VA], b[U][VW];
 #pragma unroll
         for (int u = 0; u < U; u++) { fetch(a[u], b[u]); advance(); }
 #pragma unroll
         for (int u = 0; u < U; u++) add(a[u], b[u]);
     }
-    for (; t < end; t += TL) {
-        T a[VW], b[VW];
+    for (; i < mine; i++) {
+        T a[VA], b[VW];
         fetch(a, b); advance();
         add(a, b);
     }
@@ -389,18 +402,27 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                 T* d_ = (T*)drn; T* w_ = (T*)ws; const T* a_ = (const T*)a; const T* b_ = (const T*)b;
                 if (!last_reduced) {
                     auto keep = [&](auto ot, auto vw) {
-                        hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, false, decltype(vw)::value>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        constexpr int O = decltype(ot)::value, W = decltype(vw)::value;
+                        if (W > 1 && S.splat1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, O, false, W, true>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        else hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, O, false, W, false>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                     };
                     using one = std::integral_constant<int, 1>; using wide = std::integral_constant<int, VM>;
                     if (OT == 64) { if (VO > 1) keep(std::integral_constant<int, 64>{}, wide{}); else keep(std::integral_constant<int, 64>{}, one{}); }
                     else { if (VO > 1) keep(std::integral_constant<int, 16>{}, wide{}); else keep(std::integral_constant<int, 16>{}, one{}); }
                 }
-                else if (TL == 256 && VT > 1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else if (TL == 256)          hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else if (TL == 64 && VT > 1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else if (TL == 64)           hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 4, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else if (VT > 1)             hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 16, true, VM>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                else                         hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 16, true, 1>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                else {
+                    auto rows = [&](auto ot, auto vw, auto splat) {
+                        hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                    };
+                    auto lanes = [&](auto ot) {
+                        if (VT > 1 && S.splat1) rows(ot, std::integral_constant<int, VM>{}, std::true_type{});
+                        else if (VT > 1) rows(ot, std::integral_constant<int, VM>{}, std::false_type{});
+                        else rows(ot, std::integral_constant<int, 1>{}, std::false_type{});
+                    };
+                    if (TL == 256) lanes(std::integral_constant<int, 1>{});
+                    else if (TL == 64) lanes(std::integral_constant<int, 4>{});
+                    else lanes(std::integral_constant<int, 16>{});
+                }
                 if (S.segments > 1)
                     hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((S.n_out + 15) / 16), dim3(256), 0, dev->stream, A.c0, rank, S.n_out, S.segments, (const T*)ws, d_);
             };
