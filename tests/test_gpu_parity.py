@@ -548,6 +548,31 @@ def test_broadcast_backward_split_sums(device, orc, dt):
                     err_abs = np.abs(drn.getData().astype(np.float64) - want)
                     worst = int(np.argmax(err_abs / (np.abs(mag) + 1e-300)))
                     assert (err_abs <= tol * np.abs(mag) + 1e-30).all(), (full, tgt, op, d, worst, float(drn.getData()[worst]), float(want[worst]), float(mag[worst]))
+    # a source that does not move along the 16-byte vector has its own instantiations: the other operand in its own
+    # shape, as autograd passes it (extent 1 where the drain keeps the innermost axis), and a virtual tensor (one
+    # element, all-zero tables) where the innermost axis is reduced
+    for full, tgt, oth, path in (([48, 40, 128], [1, 1, 128], [48, 40, 1], "broadcast_backward_split_vec"),
+                                 ([1100, 700], [1, 700], [1100, 1], "broadcast_backward_split_vec"),
+                                 ([48, 40, 128], [48, 1, 1], None, "broadcast_backward_split_rows_vec"),
+                                 ([30, 2100], [30, 1], None, "broadcast_backward_split_rows_vec")):
+        e = rng.integers(-3, 4, full).astype(T)
+        te = on(device, e)
+        for op, d in (("add", 0), ("subtract", 1), ("multiply", 0), ("multiply", 1)):
+            say("broadcast bwd split, constant source", full, tgt, oth, op, d, dt)
+            if oth is None:
+                other = np.full(full, 3, dtype=T)
+                tother = Tensor.of(T, full, 3.0).to(device)
+                assert tother.isVirtual()
+                other_cfg = orc.dense_cfg(full)
+            else:
+                other = rng.integers(1, 4, oth).astype(T)
+                tother = on(device, other)
+                other_cfg = orc.dense_cfg(oth)
+            drn = Tensor._on_device(device, T, tgt)
+            device.launch_broadcast(op, d, drn, tother, te)
+            assert _lib.last_path().startswith(path), (_lib.last_path(), path)
+            want = orc.broadcast(op, d, np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt), other.reshape(-1), other_cfg, e.reshape(-1), orc.dense_cfg(full))
+            assert_bits(drn.getData(), want, f"constant source {full} {tgt} {oth} {op} {d}")
     say("broadcast bwd split on a sliced error and a transposed drain", dt)
     parent = rng.integers(-3, 4, (50, 44, 140)).astype(T)
     err = on(device, parent)[1:49, 2:42, 6:134]
