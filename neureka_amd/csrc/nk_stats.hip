@@ -11,7 +11,9 @@
 // the piece through LDS 32 columns at a time -- 16-byte buffer loads that run along memory, rows of 33
 // elements in LDS -- and lane t then walks front to back through the 32 values of tile t (conflict-free).  The
 // loads of the next 32 columns are in flight while the current ones are reduced.  Elements past the end of the
-// data read as zero through the buffer range check and are skipped by the tile's own limit.
+// data read as zero through the buffer range check and are skipped by the tile's own limit.  A block's 256 tile
+// results are whole tiles of the next level (256 = 2 x 128 = 4 x 64), which the block reduces itself: one launch
+// covers two levels of the tree.
 #include "nk_internal.h"
 
 namespace nk {
@@ -34,8 +36,8 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int64_t tile0 = ((int64_t)blockIdx.x * 4 + wave) * 64;          // first tile of the wavefront
     const int64_t elem0 = tile0 * RTS;
-    if (elem0 >= n) return;                                              // whole wavefronts leave together
-    const int64_t left = n - elem0;
+    const bool active = elem0 < n;                                       // wave-uniform; idle wavefronts only join the block's last step
+    const int64_t left = active ? n - elem0 : 0;
     const unsigned bytes = left * (int64_t)sizeof(T) > 0xffffffffll ? 0xffffffffu : (unsigned)(left * sizeof(T));
     const BufRsrc r1 = __builtin_amdgcn_make_buffer_rsrc((void*)(in + elem0), 0, bytes, 0x00020000);
     const BufRsrc r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == STAT_DOT ? in2 : in) + elem0), 0, bytes, 0x00020000);
@@ -69,9 +71,9 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     T value = T(0);
     int found = 0;
 
-    request(0);
+    if (active) request(0);
 #pragma unroll
-    for (int c = 0; c < NCH; c++) {
+    for (int c = 0; active && c < NCH; c++) {
 #pragma unroll
         for (int k = 0; k < LOADS; k++) {
             typedef T Vec __attribute__((ext_vector_type(VEC)));
@@ -100,12 +102,35 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
         }
         __builtin_amdgcn_wave_barrier();
     }
-    if (limit > 0) {
-        const int64_t tile = tile0 + lane;
-        out[tile] = value;
-        if (MODE == STAT_MIN || MODE == STAT_MAX) {
-            const int64_t at = my_first + found;                      // position in this level's input
-            idx_out[tile] = idx_in ? idx_in[at] : (int)at;            // ... mapped back to the original data
+    // The next level of the tree in the same launch: the block's 256 tile results are 256 / RTS whole tiles of the
+    // next level; one thread each reduces them front to back out of LDS and only those results are written.
+    constexpr bool INDEXED = MODE == STAT_MIN || MODE == STAT_MAX;
+    constexpr int NEXT = 256 / RTS;                  // next-level tiles per block
+    __shared__ T level_val[256];
+    __shared__ int level_idx[INDEXED ? 256 : 1];
+    level_val[threadIdx.x] = value;
+    if (INDEXED && limit > 0) {
+        const int64_t at = my_first + found;                          // position in this level's input
+        level_idx[threadIdx.x] = idx_in ? idx_in[at] : (int)at;       // ... mapped back to the original data
+    }
+    __syncthreads();
+    if (threadIdx.x < NEXT) {
+        const int64_t results = (n + RTS - 1) / RTS;                  // tile results of this level in the whole grid
+        const int64_t first = (int64_t)blockIdx.x * 256 + (int64_t)threadIdx.x * RTS;
+        if (first < results) {
+            const int count = results - first < RTS ? (int)(results - first) : RTS;
+            T v = T(0);
+            int at = 0;
+            for (int i = 0; i < count; i++) {
+                const T x = level_val[threadIdx.x * RTS + i];
+                if (!INDEXED) v = v + x;
+                else {
+                    const bool better = MODE == STAT_MIN ? x < v : x > v;
+                    if (i == 0 || better) { v = x; at = i; }
+                }
+            }
+            out[(int64_t)blockIdx.x * NEXT + threadIdx.x] = v;
+            if (INDEXED) idx_out[(int64_t)blockIdx.x * NEXT + threadIdx.x] = level_idx[threadIdx.x * RTS + at];
         }
     }
 }
@@ -221,9 +246,10 @@ static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* o
         else
             hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, MODE>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur2, cur_idx, m, dst, dst_idx);
         cur = dst; cur2 = dst; cur_idx = dst_idx;
-        used += tiles;
-        m = tiles;
-        level++;
+        const int64_t written = (tiles + RTS - 1) / RTS;           // the launch covers two levels of the tree
+        used += written;
+        m = written;
+        level += 2;
     } while (m > 1);
     NK_HIP(hipGetLastError());
     return NK_OK;
