@@ -884,6 +884,79 @@ def test_convolution_split_sums(device, orc, shape, dt):
         assert_bits(dk.getData(), want, "transposed operand")
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_random_convolutions_through_every_plan(device, orc, dt):
+    """Random shapes of rank 1 to 4 (every axis either slides, in either operand, or is reduced), biased towards the
+    shapes the specialised kernels take and towards their edges (widths around a wavefront's 256 columns, heights
+    that are no multiple of a strip, channel counts that are no multiple of a group), sometimes through a transposed
+    or sliced operand.  The data are small integers, so every order of the sums is exact: forward and both gradients
+    must equal the oracle's state machines bit for bit on whichever kernel the planner picks."""
+    T = F[dt]
+    rng = np.random.default_rng(46)
+    seen = set()
+
+    def operand(shape, view):
+        """A device tensor of the given shape and (its parent's data, its descriptor) for the oracle."""
+        if view == "transposed" and len(shape) >= 2:
+            parent = rng.integers(-3, 4, shape[:-2] + [shape[-1], shape[-2]]).astype(T)
+            axes = list(range(len(shape) - 2)) + [len(shape) - 1, len(shape) - 2]
+            t = on(device, parent).permute(*axes)
+        elif view == "sliced":
+            parent = rng.integers(-3, 4, [s + 2 for s in shape]).astype(T)
+            t = on(device, parent)[tuple(slice(1, 1 + s) for s in shape)]
+        else:
+            parent = rng.integers(-3, 4, shape).astype(T)
+            t = on(device, parent)
+        assert list(t.shape) == list(shape)
+        return t, parent.reshape(-1), cfg(t)
+
+    for case in range(70):
+        kind = ("channels", "image", "any")[case % 3]
+        if kind == "channels":          # [C,H,W] x [C,k,k]
+            c = int(rng.choice([2, 3, 5, 8, 13, 16, 33]))
+            kk = int(rng.choice([2, 3, 4, 5, 7, 6, 1]))
+            h = int(rng.integers(kk, 40)); w = int(rng.choice([kk, 17, 64, 255, 256, 257, 258, 259, 263, 300, 515]))
+            w = max(w, kk)
+            xs, ks = [c, h, w], [c, kk, kk if rng.random() < 0.85 else max(1, kk - 1)]
+        elif kind == "image":           # [H,W] x [k,k] and [B,H,W] x [1,k,k]
+            kk = int(rng.choice([2, 3, 4, 5, 7]))
+            h = int(rng.choice([kk, 9, 64, 200, 270])); w = int(rng.choice([kk, 33, 257, 300, 520]))
+            xs, ks = [h, w], [kk, kk]
+            if rng.random() < 0.4:
+                xs, ks = [int(rng.integers(1, 4))] + xs, [1] + ks
+        else:
+            rank = int(rng.integers(1, 5))
+            xs, ks = [], []
+            for _ in range(rank):
+                a, b = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+                mode = rng.random()
+                if mode < 0.3: b = a                      # reduced axis
+                elif mode < 0.7: a, b = max(a, b), min(a, b)
+                xs.append(a); ks.append(b)
+        ys = [abs(p - q) + 1 for p, q in zip(xs, ks)]
+        views = [str(rng.choice(["dense", "dense", "transposed", "sliced"])) for _ in range(3)]
+        say("random convolution", case, kind, xs, ks, views, dt)
+        (tx, dx_, cx), (tk, dk_, ck), (te, de_, ce) = operand(xs, views[0]), operand(ks, views[1]), operand(ys, views[2])
+        out = Tensor._on_device(device, T, ys)
+        if rng.random() < 0.5:
+            device.launch_convolution(-1, out, tx, tk)
+            want = orc.convolve(np.zeros(out.size, dtype=T), orc.dense_cfg(ys), dx_, cx, dk_, ck)
+        else:                                             # taps first
+            device.launch_convolution(-1, out, tk, tx)
+            want = orc.convolve(np.zeros(out.size, dtype=T), orc.dense_cfg(ys), dk_, ck, dx_, cx)
+        seen.add(_lib.last_path())
+        assert_bits(out.getData(), want, f"case {case} forward {xs} x {ks} {views} on {_lib.last_path()}")
+        for name, tgt_shape, other, other_data, other_cfg in (("dx", xs, tk, dk_, ck), ("dk", ks, tx, dx_, cx)):
+            drn = Tensor._on_device(device, T, tgt_shape)
+            device.launch_convolution(0, drn, other, te)
+            seen.add(_lib.last_path())
+            want = orc.deconvolve(np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt_shape), other_data, other_cfg, de_, ce, fast=True)
+            assert_bits(drn.getData(), want, f"case {case} {name} {xs} x {ks} {views} on {_lib.last_path()}")
+    say("plans seen", sorted(seen))
+    want_plans = {"literal_fwd", "literal_bwd", "simple2d"} | ({"chan_fwd", "chan_dx", "chan_dk", "simple2d_window"} if dt == "f32" else set())
+    assert want_plans <= seen, (sorted(want_plans - seen), sorted(seen))
+
+
 @pytest.mark.parametrize("shape", [([300, 523], [5, 5]), ([3, 200, 300], [1, 3, 3]), ([130, 700], [7, 7]), ([260, 257], [2, 2]), ([2, 190, 261], [1, 4, 4])])
 def test_conv2d_large_images_bit_exact(device, orc, shape):
     """Large f32 images with square taps take the register-window kernel: the same products, rounded and added in
