@@ -617,6 +617,56 @@ def test_broadcast_backward_vector_path_and_views(device, orc, dt):
         assert_bits(drn.getData(), want, f"sliced error {tgt}")
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_random_broadcast_gradients_through_every_plan(device, orc, dt):
+    """Random ranks, shapes, reduced axes, operators and derivative indices; the other operand in the full shape, in
+    its own shape (extent 1 where the drain keeps an axis) or virtual; the error sometimes a slice of a larger
+    tensor.  Small integers make every order of the sums exact, so whichever kernel the planner picks -- a thread
+    per element, vectors, split sums along or across the rows -- must equal the oracle bit for bit."""
+    T = F[dt]
+    rng = np.random.default_rng(47)
+    seen = set()
+    for case in range(120):
+        rank = int(rng.integers(1, 5))
+        big = case % 3 == 0                                # long sums: the split kernels
+        full = [int(rng.choice([1, 2, 3, 5, 8, 16, 31, 64] if not big else [1, 4, 20, 33, 64, 130, 512])) for _ in range(rank)]
+        while int(np.prod(full)) > 300000:
+            full[int(np.argmax(full))] //= 2
+        tgt = [s if rng.random() < 0.5 else 1 for s in full]
+        style = str(rng.choice(["full", "own", "virtual"]))
+        if style == "own":
+            oth = [s if t == 1 else 1 for s, t in zip(full, tgt)]
+            if all(o == 1 for o in oth) and int(np.prod(full)) > 1:
+                style, oth = "full", list(full)
+        else:
+            oth = list(full)
+        op = str(rng.choice(["add", "subtract", "multiply"]))
+        d = int(rng.integers(0, 2))
+        sliced = rng.random() < 0.3
+        say("random broadcast gradient", case, full, tgt, oth, style, op, d, "sliced error" if sliced else "", dt)
+        if sliced:
+            parent = rng.integers(-3, 4, [s + 3 for s in full]).astype(T)
+            te = on(device, parent)[tuple(slice(2, 2 + s) for s in full)]
+            e_data, e_cfg = parent.reshape(-1), cfg(te)
+        else:
+            e = rng.integers(-3, 4, full).astype(T)
+            te, e_data, e_cfg = on(device, e), e.reshape(-1), orc.dense_cfg(full)
+        if style == "virtual":
+            other = np.full(oth, 2, dtype=T)
+            tother = Tensor.of(T, oth, 2.0).to(device)
+        else:
+            other = rng.integers(-3, 4, oth).astype(T)
+            tother = on(device, other)
+        drn = Tensor._on_device(device, T, tgt)
+        device.launch_broadcast(op, d, drn, tother, te)
+        seen.add(_lib.last_path())
+        want = orc.broadcast(op, d, np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt), other.reshape(-1), orc.dense_cfg(oth), e_data, e_cfg)
+        assert_bits(drn.getData(), want, f"case {case} {full} -> {tgt}, other {oth} ({style}), {op} d={d} on {_lib.last_path()}")
+    say("plans seen", sorted(seen))
+    assert {"broadcast_backward", "broadcast_backward_vec", "broadcast_backward_split_vec",
+            "broadcast_backward_split_rows", "broadcast_backward_split_rows_vec"} <= seen, sorted(seen)
+
+
 def test_broadcast_autograd_golden(device, golden):
     g = golden["broadcast_autograd"]
     for row in g["rows"]:
