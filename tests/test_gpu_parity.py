@@ -1252,6 +1252,39 @@ def test_matmul_split_k(device, orc, mkn, dt):
     assert (np.abs(tc.getData().reshape(N, M).T.astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_random_products_through_every_plan(device, dt):
+    """Random extents around the edges of the tilings (1, 2, just below / at / above 128, 256 and the split and
+    matrix-core thresholds), both layouts, accumulation into a non-zero C.  Small integers keep every order of the
+    sums exact, so each kernel -- the reference's order, matrix-core tiles whole and partial, inner dimension in
+    parts -- must equal the integer product."""
+    T = F[dt]
+    rng = np.random.default_rng(57)
+    sizes = [1, 2, 3, 31, 64, 127, 128, 129, 200, 255, 256, 257, 384, 511, 513, 1024]
+    seen = set()
+    for case in range(60):
+        M, K, N = (int(rng.choice(sizes)) for _ in range(3))
+        if case % 6 == 0:
+            K = int(rng.choice([2048, 4096, 5000, 8192]))       # few tiles, long inner dimension
+            M, N = int(rng.choice([64, 128, 130, 256])), int(rng.choice([64, 128, 130, 256]))
+        row_major = bool(rng.random() < 0.6)
+        say("random product", case, (M, K, N), "row major" if row_major else "column major", dt)
+        A = rng.integers(-3, 4, (M, K)).astype(T); B = rng.integers(-3, 4, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
+        want = A.astype(np.float64) @ B.astype(np.float64) + C0
+        if row_major:
+            tc = on(device, C0)
+            device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+            got = tc.getData().reshape(M, N)
+        else:
+            tc = on(device, C0.T.copy())
+            device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+            got = tc.getData().reshape(N, M).T
+        seen.add(_lib.last_path())
+        assert (got == want).all(), (case, M, K, N, row_major, _lib.last_path())
+    say("plans seen", sorted(seen))
+    assert "simple" in seen and any(p.endswith("_split") for p in seen) and any("edge" in p for p in seen), sorted(seen)
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
