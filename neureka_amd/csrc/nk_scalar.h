@@ -56,10 +56,13 @@ template <> struct Num<double> {
 // double-precision instructions): Math.pow returns its first argument for an exponent of 1 and 1.0 for an exponent
 // of zero by specification, and a square is the correctly rounded product (exact in double for a float base) --
 // what a correctly rounded pow returns and what HotSpot substitutes for pow(x, 2.0).
+// Where java.lang.Math.pow differs from C99's pow the reference's answer is kept: a NaN exponent gives NaN whatever
+// the base (C: pow(1, NaN) = 1) and a base of magnitude 1 with an infinite exponent gives NaN (C: 1).
 __device__ __forceinline__ double pow_double(double a, double b) {
     if (b == 2.0) return a * a;
     if (b == 1.0) return a;
     if (b == 0.0) return 1.0;
+    if (b != b || (fabs(a) == 1.0 && isinf(b))) return __builtin_nan("");
     return ::pow(a, b);
 }
 __device__ __forceinline__ double pow_ref(double a, double b) { return pow_double(a, b); }

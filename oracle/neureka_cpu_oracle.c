@@ -31,6 +31,18 @@
 #include <stdlib.h>
 #include <string.h>
 
+/* java.lang.Math.pow where it differs from C99's pow: a NaN exponent gives NaN whatever the base (C: pow(1, NaN) = 1)
+ * and a base of magnitude 1 with an infinite exponent gives NaN (C: 1).  Every other special case of the Javadoc
+ * table (x^0 = 1 also for NaN, negative base with a non-integer exponent = NaN, signed zeros and infinities) is C99's
+ * Annex F behaviour.  Exported for the tests that check the table. */
+double orc_java_pow(double a, double b) {
+    if (b == 0.0) return 1.0;
+    if (b != b) return (double)NAN;
+    if (fabs(a) == 1.0 && isinf(b)) return (double)NAN;
+    return pow(a, b);
+}
+
+
 #define ORC_MAX_RANK 8
 
 /* ------------------------------------------------------------------------------------------------
@@ -170,7 +182,7 @@ double orc_fun_f64(int id, int derive, double x) {
         case FUN_ABS: return (x < 0.0 ? -1.0 : 1.0);
         case FUN_COS: return -sin(x);
         case FUN_GASU: { double x2 = x * x, x6 = x2 * x2 * x2; return 3.0 * x2 / (2.0 * x2 * fabs(x) + x6 + 1.0); }
-        case FUN_GATU: { double x2 = x * x, x3 = x2 * x, temp = 3 * x2, t2 = pow(tanh64(x3), 2); return -temp * t2 + temp; }
+        case FUN_GATU: { double x2 = x * x, x3 = x2 * x, temp = 3 * x2, t2 = orc_java_pow(tanh64(x3), 2); return -temp * t2 + temp; }
         case FUN_GAUS: return -2 * x * exp(-(x * x));
         case FUN_FAST_GAUS: { double x2 = x * x; return -2 * x / (x2 * x2 + 2 * x2 + 1); }
         case FUN_GELU: { double s = sig64(x * 1.702), ds = s * (1.0 - s); return s + ds * x * 1.702; }
@@ -184,12 +196,12 @@ double orc_fun_f64(int id, int derive, double x) {
         case FUN_SIN: return cos(x);
         case FUN_SOFTPLUS: return 1.0 / (1.0 + exp(-x));
         case FUN_SOFTSIGN: return 1.0 / (2.0 * fabs(x) + x * x + 1.0);
-        case FUN_TANH: return 1 - pow(tanh64(x), 2);
+        case FUN_TANH: return 1 - orc_java_pow(tanh64(x), 2);
         case FUN_FAST_TANH: { double t1 = x * x, t2 = sqrt(1 + t1); return 1 / (t1 * t2 + t2); }
         case FUN_EXP: return exp(x);
         case FUN_LOG10: return 1 / (x * log(10));
         case FUN_SQRT: return 0.5 * inv_sqrt_f64(x);
-        case FUN_CBRT: return 1 / (3 * pow(x, 2.0 / 3.0));
+        case FUN_CBRT: return 1 / (3 * orc_java_pow(x, 2.0 / 3.0));
     }
     return (double)NAN;
 }
@@ -209,10 +221,10 @@ float orc_fun_f32(int id, int derive, float x) {
         default: return (float)orc_fun_f64(id, 0, (double)x);     /* CPUFun default and the (float) Math.f(x) overrides */
     } else switch (id) {
         case FUN_ABS: return (x < 0.0f ? -1.0f : 1.0f);
-        case FUN_CBRT: return 1 / (3 * (float)pow((double)x, (double)(2.0f / 3.0f)));
+        case FUN_CBRT: return 1 / (3 * (float)orc_java_pow((double)x, (double)(2.0f / 3.0f)));
         case FUN_EXP: return (float)exp((double)x);
         case FUN_GASU: { float x2 = x * x, x6 = x2 * x2 * x2; return 3.0f * x2 / (2.0f * x2 * fabsf(x) + x6 + 1.0f); }
-        case FUN_GATU: { float x2 = x * x, x3 = x2 * x, temp = 3 * x2, t2 = (float)pow((double)tanh32(x3), 2); return -temp * t2 + temp; }
+        case FUN_GATU: { float x2 = x * x, x3 = x2 * x, temp = 3 * x2, t2 = (float)orc_java_pow((double)tanh32(x3), 2); return -temp * t2 + temp; }
         case FUN_FAST_GAUS: { float x2 = x * x; return -2 * x / (x2 * x2 + 2 * x2 + 1); }
         case FUN_GELU: { float s = (float)sig64((double)x * 1.702), ds = s * (1.0f - s); return s + ds * x * 1.702f; }
         case FUN_IDY: return 1;
@@ -225,7 +237,7 @@ float orc_fun_f32(int id, int derive, float x) {
         case FUN_SILU: { float s = (float)sig64((double)x); return s + (x * s * (1.0f - s)); }
         case FUN_SOFTSIGN: return 1.0f / (2.0f * fabsf(x) + x * x + 1.0f);
         case FUN_SQRT: return 0.5f * inv_sqrt_f32(x);
-        case FUN_TANH: return (float)(1 - pow((double)tanh32(x), 2));
+        case FUN_TANH: return (float)(1 - orc_java_pow((double)tanh32(x), 2));
         case FUN_FAST_TANH: { float t1 = x * x, t2 = (float)sqrt((double)(1 + t1)); return 1 / (t1 * t2 + t2); }
         default: return (float)orc_fun_f64(id, 1, (double)x);
     }
@@ -236,6 +248,7 @@ float orc_fun_f32(int id, int derive, float x) {
  * d < 0: the operator; d = 0/1: _getDeriveAt0/_getDeriveAt1 of that family. */
 enum { OP_ADD = 0, OP_SUB, OP_MUL, OP_DIV, OP_MOD, OP_POW, OP_IDY };
 
+
 double orc_bin_f64(int family, int op, int d, double a, double b) {
     if (d < 0) switch (op) {
         case OP_ADD: return a + b;
@@ -243,22 +256,22 @@ double orc_bin_f64(int family, int op, int d, double a, double b) {
         case OP_MUL: return a * b;
         case OP_DIV: return a / b;
         case OP_MOD: return fmod(a, b);           /* Java % on doubles */
-        case OP_POW: return pow(a, b);
+        case OP_POW: return orc_java_pow(a, b);
         case OP_IDY: return b;
     }
     if (family == 2) switch (op) {
         case OP_ADD: return a + b;
         case OP_SUB: return d == 0 ? a + b : a - b;
         case OP_MUL: return d == 0 ? b : a;
-        case OP_DIV: case OP_MOD: return d == 0 ? 1 / b : -(a / pow(b, 2));
-        case OP_POW: return d == 0 ? a * pow(a, b - 1) : pow(a, b) * log(a);
+        case OP_DIV: case OP_MOD: return d == 0 ? 1 / b : -(a / orc_java_pow(b, 2));
+        case OP_POW: return d == 0 ? a * orc_java_pow(a, b - 1) : orc_java_pow(a, b) * log(a);
     }
     switch (op) {
         case OP_ADD: return 1;
         case OP_SUB: return d == 0 ? 1 : -1;
         case OP_MUL: return d == 0 ? b : a;
-        case OP_DIV: case OP_MOD: return d == 0 ? 1.0 / b : -a / pow(b, 2);
-        case OP_POW: return d == 0 ? b * pow(a, b - 1) : pow(a, b) * log(a);
+        case OP_DIV: case OP_MOD: return d == 0 ? 1.0 / b : -a / orc_java_pow(b, 2);
+        case OP_POW: return d == 0 ? b * orc_java_pow(a, b - 1) : orc_java_pow(a, b) * log(a);
         case OP_IDY: return d == 0 ? 0 : 1;
     }
     return (double)NAN;
@@ -271,22 +284,22 @@ float orc_bin_f32(int family, int op, int d, float a, float b) {
         case OP_MUL: return a * b;
         case OP_DIV: return a / b;
         case OP_MOD: return fmodf(a, b);
-        case OP_POW: return (float)pow((double)a, (double)b);
+        case OP_POW: return (float)orc_java_pow((double)a, (double)b);
         case OP_IDY: return b;
     }
     if (family == 2) switch (op) {
         case OP_ADD: return a + b;
         case OP_SUB: return d == 0 ? a + b : a - b;
         case OP_MUL: return d == 0 ? b : a;
-        case OP_DIV: case OP_MOD: return d == 0 ? 1 / b : (float)-((double)a / pow((double)b, 2));
-        case OP_POW: return d == 0 ? (float)((double)a * pow((double)a, (double)(b - 1))) : (float)(pow((double)a, (double)b) * log((double)a));
+        case OP_DIV: case OP_MOD: return d == 0 ? 1 / b : (float)-((double)a / orc_java_pow((double)b, 2));
+        case OP_POW: return d == 0 ? (float)((double)a * orc_java_pow((double)a, (double)(b - 1))) : (float)(orc_java_pow((double)a, (double)b) * log((double)a));
     }
     switch (op) {
         case OP_ADD: return 1;
         case OP_SUB: return d == 0 ? 1 : -1;
         case OP_MUL: return d == 0 ? b : a;
-        case OP_DIV: case OP_MOD: return d == 0 ? 1.0f / b : (float)-((double)a / pow((double)b, 2));
-        case OP_POW: return d == 0 ? (float)((double)b * pow((double)a, (double)(b - 1))) : (float)(pow((double)a, (double)b) * log((double)a));
+        case OP_DIV: case OP_MOD: return d == 0 ? 1.0f / b : (float)-((double)a / orc_java_pow((double)b, 2));
+        case OP_POW: return d == 0 ? (float)((double)b * orc_java_pow((double)a, (double)(b - 1))) : (float)(orc_java_pow((double)a, (double)b) * log((double)a));
         case OP_IDY: return d == 0 ? 0 : 1;
     }
     return NAN;
@@ -374,9 +387,9 @@ static double scalar_fun_f64(int op, int d, double a, double b) {
         case 0: return d < 0 ? a + b : 1;
         case 1: return d < 0 ? a - b : (d == 0 ? 1 : -1);
         case 2: return d < 0 ? a * b : (d == 0 ? b : a);
-        case 3: return d < 0 ? a / b : (d == 0 ? 1 / b : -(a / pow(b, 2)));
-        case 4: return d < 0 ? fmod(a, b) : (d == 0 ? 1 / b : -(a / pow(b, 2)));
-        case 5: return d < 0 ? pow(a, b) : (d == 0 ? b * pow(a, b - 1) : pow(a, b) * log(a));
+        case 3: return d < 0 ? a / b : (d == 0 ? 1 / b : -(a / orc_java_pow(b, 2)));
+        case 4: return d < 0 ? fmod(a, b) : (d == 0 ? 1 / b : -(a / orc_java_pow(b, 2)));
+        case 5: return d < 0 ? orc_java_pow(a, b) : (d == 0 ? b * orc_java_pow(a, b - 1) : orc_java_pow(a, b) * log(a));
         default: return b;
     }
 }
@@ -393,11 +406,11 @@ static int32_t scalar_fun_i32(int op, int d, int32_t a, int32_t b, int* div_by_z
                 return op == 3 ? a / b : a % b;
             }
             if (d == 0) return to_int(java_math_round(1.0 / b));
-            return to_int(java_math_round(int_neg(a) / pow(b, 2)));
+            return to_int(java_math_round(int_neg(a) / orc_java_pow(b, 2)));
         case 5:
-            if (d < 0) return to_int(java_math_round(pow(a, b)));
-            if (d == 0) return to_int(java_math_round(b * pow(a, (int32_t)((uint32_t)b - 1u))));
-            return to_int(java_math_round(pow(a, b) * log(a)));
+            if (d < 0) return to_int(java_math_round(orc_java_pow(a, b)));
+            if (d == 0) return to_int(java_math_round(b * orc_java_pow(a, (int32_t)((uint32_t)b - 1u))));
+            return to_int(java_math_round(orc_java_pow(a, b) * log(a)));
         default: return b;
     }
 }
@@ -413,11 +426,11 @@ static int64_t scalar_fun_i64(int op, int d, int64_t a, int64_t b, int* div_by_z
                 return op == 3 ? a / b : a % b;
             }
             if (d == 0) return java_math_round(1.0 / (double)b);
-            return java_math_round((double)long_neg(a) / pow((double)b, 2));
+            return java_math_round((double)long_neg(a) / orc_java_pow((double)b, 2));
         case 5:
-            if (d < 0) return java_math_round(pow((double)a, (double)b));
-            if (d == 0) return java_math_round((double)b * pow((double)a, (double)(int64_t)((uint64_t)b - 1ull)));
-            return java_math_round(pow((double)a, (double)b) * log((double)a));
+            if (d < 0) return java_math_round(orc_java_pow((double)a, (double)b));
+            if (d == 0) return java_math_round((double)b * orc_java_pow((double)a, (double)(int64_t)((uint64_t)b - 1ull)));
+            return java_math_round(orc_java_pow((double)a, (double)b) * log((double)a));
         default: return b;
     }
 }

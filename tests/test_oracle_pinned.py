@@ -511,3 +511,36 @@ def test_int_scalarization_matches_exact_integer_arithmetic_and_views(orc):
     drn_cfg = [3, 3, 1, 3, 3, 1, 0, 0, 1, 1]                     # column-major strides
     out = orc.scalarization_int("multiply", -1, np.zeros(9, dtype=np.int16), drn_cfg, base, src_cfg, 5)
     assert out.reshape(3, 3).T.tolist() == (base.reshape(4, 6)[0:3, 1::2] * 5).tolist()
+
+
+def test_power_follows_the_special_cases_of_java_math_pow(orc):
+    """The operator ** is Math.pow (CPUBiElementWisePower.java:11): its documented special cases, including the two
+    where C's pow answers differently (a NaN exponent with base 1; a base of magnitude 1 with an infinite exponent)."""
+    inf, nan = np.inf, np.nan
+    rows = [  # (base, exponent, Math.pow)
+        (3.0, 0.0, 1.0), (nan, 0.0, 1.0), (inf, -0.0, 1.0), (-2.5, 1.0, -2.5), (nan, 1.0, nan),
+        (1.0, nan, nan), (0.0, nan, nan), (inf, nan, nan), (nan, 2.5, nan), (nan, -1.0, nan),
+        (2.0, inf, inf), (-2.0, inf, inf), (0.5, -inf, inf), (-0.5, -inf, inf),
+        (2.0, -inf, 0.0), (-2.0, -inf, 0.0), (0.5, inf, 0.0), (-0.5, inf, 0.0),
+        (1.0, inf, nan), (-1.0, inf, nan), (1.0, -inf, nan), (-1.0, -inf, nan),
+        (0.0, 2.5, 0.0), (inf, -3.0, 0.0), (0.0, -2.5, inf), (inf, 3.0, inf),
+        (-0.0, 2.0, 0.0), (-0.0, 2.5, 0.0), (-inf, -2.0, 0.0), (-inf, -2.5, 0.0),
+        (-0.0, 3.0, -0.0), (-inf, -3.0, -0.0),
+        (-0.0, -2.0, inf), (-0.0, -2.5, inf), (-inf, 2.0, inf), (-inf, 2.5, inf),
+        (-0.0, -3.0, -inf), (-inf, 3.0, -inf),
+        (-2.0, 2.0, 4.0), (-2.0, 3.0, -8.0), (-2.0, -2.0, 0.25), (-2.0, 0.5, nan), (-8.0, 1.0 / 3.0, nan),
+        (2.0, 10.0, 1024.0), (4.0, 0.5, 2.0), (10.0, -2.0, 0.01), (2.0, 0.5, np.sqrt(2.0)),
+    ]
+    a = np.array([r[0] for r in rows]); b = np.array([r[1] for r in rows]); want = np.array([r[2] for r in rows])
+    c = orc.dense_cfg([a.size])
+    for T in (np.float64, np.float32):
+        with np.errstate(all="ignore"):
+            got = orc.elementwise("power", -1, np.zeros(a.size, dtype=T), c, a.astype(T), c, b.astype(T), c)
+            expect = want.astype(T)
+            if T is np.float32:      # the float form is (float) Math.pow((double) a, (double) b) on the rounded arguments
+                expect[rows.index((-8.0, 1.0 / 3.0, nan))] = nan
+        for i, r in enumerate(rows):
+            g, w = got[i], expect[i]
+            ok = (np.isnan(g) and np.isnan(w)) or (g == w and np.signbit(g) == np.signbit(w)) or \
+                 (np.isfinite(w) and w != 0 and abs(g - w) <= 4 * np.finfo(T).eps * abs(w))
+            assert ok, (T.__name__, r, float(g))
