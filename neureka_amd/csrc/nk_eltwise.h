@@ -481,10 +481,11 @@ struct TileArgs {
     unsigned P, L;                          // extents of pax and of the innermost axis
     unsigned tiles_p, tiles_l;
     unsigned n_blocks;
-    int group_log2;                         // blocks are numbered through G x G groups of tiles, G = 1 << group_log2
+    int group_log2, group_p_log2;           // blocks are numbered through groups of (1 << group_p_log2) x (1 << group_log2) tiles
     int streaming;
     int nt_loads;                           // every source element is read exactly once: the host picks the non-temporal-load variant
     int careful;                            // some direct operand is constant along the innermost axis: no vector path
+    int xcd_regions;                        // XCD x (blocks x, x + 8, ...) takes the x-th eighth of the tile order
     FastDiv div_tiles_l, div_tiles_p;
     FastDiv outer[NK_MAX_RANK];             // extents of the remaining axes
     int64_t base[MAX_OPERANDS];
@@ -507,17 +508,19 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
     __shared__ T tiles[NSRC][TILE_L][TILE_P + 1];
     const int last = A.rank - 1;
 
-    // Consecutive blocks run at the same time.  Numbering them through G x G groups of tiles makes the pieces
-    // that neighbouring blocks read (along pax) and write (along the innermost axis) add up to longer
-    // contiguous runs on both sides.
+    // Blocks that run at the same time behind one L2 should be neighbours: the hardware deals consecutive block ids
+    // round-robin to the 8 XCDs, so XCD x (blocks x, x + 8, ...) takes the x-th eighth of the tile order, and that
+    // order runs through groups of GP x GL tiles -- the pieces one L2 reads (along pax) and writes (along the
+    // innermost axis) at a time then add up to long contiguous runs on both sides.
     unsigned rest = blockIdx.x;
-    const unsigned G = 1u << A.group_log2;
-    const unsigned local = rest & (G * G - 1);
-    rest >>= 2 * A.group_log2;
-    unsigned d = A.div_tiles_l.div(rest);                  // divisors are the group counts tiles_l / G and tiles_p / G
-    const unsigned tl = (rest - d * A.div_tiles_l.d) * G + (local & (G - 1)); rest = d;
+    if (A.xcd_regions) rest = (blockIdx.x & 7u) * (A.n_blocks >> 3) + (blockIdx.x >> 3);
+    const unsigned GL = 1u << A.group_log2, GP = 1u << A.group_p_log2;
+    const unsigned local = rest & (GL * GP - 1);
+    rest >>= A.group_log2 + A.group_p_log2;
+    unsigned d = A.div_tiles_l.div(rest);                  // divisors are the group counts tiles_l / GL and tiles_p / GP
+    const unsigned tl = (rest - d * A.div_tiles_l.d) * GL + (local & (GL - 1)); rest = d;
     d = A.div_tiles_p.div(rest);
-    const unsigned tp = (rest - d * A.div_tiles_p.d) * G + (local >> A.group_log2); rest = d;
+    const unsigned tp = (rest - d * A.div_tiles_p.d) * GP + (local >> A.group_log2); rest = d;
     int64_t off[NSRC + 1];
 #pragma unroll
     for (int o = 0; o <= NSRC; o++) off[o] = A.base[o];

@@ -346,17 +346,26 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             }
             if (nb < ((uint64_t)1 << 31)) {
                 A.n_blocks = (unsigned)nb;
+                // groups of 4 (pax) x 8 (innermost) tiles: 1 KiB runs on both sides (f32); measured optimum of the sweep
                 static const int env_group = [] { const char* v = getenv("NK_TILE_GROUP_LOG2"); return v && *v ? atoi(v) : 3; }();
-                int gl = env_group < 0 ? 0 : (env_group > 4 ? 4 : env_group);
-                while (gl > 0 && (A.tiles_l % (1u << gl) || A.tiles_p % (1u << gl))) gl--;
-                A.group_log2 = gl;
-                A.div_tiles_l = FastDiv(A.tiles_l >> gl); A.div_tiles_p = FastDiv(A.tiles_p >> gl);
+                static const int env_group_p = [] { const char* v = getenv("NK_TILE_GROUP_P_LOG2"); return v && *v ? atoi(v) : 2; }();
+                int gl = env_group < 0 ? 0 : (env_group > 6 ? 6 : env_group);
+                int gp = env_group_p < 0 ? 0 : (env_group_p > 6 ? 6 : env_group_p);
+                while (gl > 0 && A.tiles_l % (1u << gl)) gl--;
+                while (gp > 0 && A.tiles_p % (1u << gp)) gp--;
+                A.group_log2 = gl; A.group_p_log2 = gp;
+                A.div_tiles_l = FastDiv(A.tiles_l >> gl); A.div_tiles_p = FastDiv(A.tiles_p >> gp);
                 for (int o = 0; o <= c.nsrc; o++) {
                     A.base[o] = cn.base[o];
                     for (int k = 0; k < cn.rank; k++) A.stride[o][k] = cn.stride[o][k];
                 }
                 plan.kind = PLAN_TILE;
                 plan.grid = (unsigned)nb;                    // one block per tile
+                // The hardware deals consecutive block ids round-robin to the 8 XCDs, each with its own L2.  XCD x takes the
+                // x-th eighth of the tile order, so the tiles one L2 serves at a time are neighbours in both directions:
+                // its reads (along pax) and its writes (along the innermost axis) add up to long runs
+                static const bool xcd_regions = env_flag("NK_TILE_XCD_REGIONS", true);
+                A.xcd_regions = xcd_regions && nb % 8 == 0;
                 set_path("tile_transpose");
                 done = true;
             }
