@@ -640,7 +640,7 @@ static bool for_taps(int KH, int KW, F&& f) {
 
 // the three channel kernels for dense f32 operands; returns NK_OK with *taken = true when one was launched
 static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, const float* s1, const Cfg& c1,
-                              const float* s2, const Cfg& c2, bool* taken) {
+                              const float* s2, const Cfg& c2, bool* taken, bool one_plane = false) {
     using T = float;
     *taken = false;
     static const long waves_per_cu = [] { const char* v = getenv("NK_CONV_WAVES_PER_CU"); return v && *v ? atol(v) : 8L; }();
@@ -699,7 +699,7 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
         *taken = true;
         return NK_OK;
     }
-    if (d >= 0 && c2.shape[0] == 1 && c0.shape[0] == c1.shape[0] && c0.shape[0] > 1) {
+    if (d >= 0 && c2.shape[0] == 1 && c0.shape[0] == c1.shape[0] && (c0.shape[0] > 1 || one_plane)) {
         const int OH = c2.shape[1], OW = c2.shape[2];      // src2 = error [1,OH,OW]
         // dx: the drain is the big operand, src1 the taps
         if (c0.shape[1] == OH + c1.shape[1] - 1 && c0.shape[2] == OW + c1.shape[2] - 1 &&
@@ -835,6 +835,13 @@ static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, n
         if (rank == 3 && dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank)) {
             bool taken = false;
             if (int e = conv_channel_paths(dev, d, out, c0, s1, c1, s2, c2, &taken)) return e;
+            if (taken) return NK_OK;
+        }
+        // both gradients of a 2-D image convolution [H,W] x [kh,kw] are the one-channel case of the same kernels
+        if (rank == 2 && d >= 0 && dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank)) {
+            auto plane = [](const Cfg& c) { Cfg p{}; p.shape[0] = 1; p.shape[1] = c.shape[0]; p.shape[2] = c.shape[1]; return p; };
+            bool taken = false;
+            if (int e = conv_channel_paths(dev, d, out, plane(c0), s1, plane(c1), s2, plane(c2), &taken, true)) return e;
             if (taken) return NK_OK;
         }
     }

@@ -920,6 +920,8 @@ def test_convolution_split_sums(device, orc, shape, dt):
                 assert (np.abs(drn.getData().astype(np.float64) - want) <= tol * babs + 1e-30).all(), name
     if dt == "f32" and ks == [48, 5, 5]:
         assert seen == {"chan_fwd", "chan_dx", "chan_dk"}, seen          # the register-window kernels take dense f32 square taps
+    elif dt == "f32" and ks == [5, 5]:
+        assert seen == {"simple2d_window", "chan_dx", "chan_dk"}, seen   # ... and a 2-D image as their one-channel case
     else:
         assert seen & {"split_fwd", "split_bwd"}, seen
     if len(xs) == 2:
