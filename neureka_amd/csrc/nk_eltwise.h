@@ -214,16 +214,17 @@ __device__ __forceinline__ void load_vec(T (&dst)[V], const T* p) {
         for (int i = 0; i < V; i++) dst[i] = v[i];
     }
 }
+// Plain stores.  Non-temporal stores were measured on these kernels (several units per block) and lose 5..8 %;
+// they pay only together with one unit per block (rows_binary_lean_kernel).  Such a choice has to be made at compile
+// time: a store that is non-temporal in one branch and plain in the other is merged into one plain store.
 template <typename T, int V>
-__device__ __forceinline__ void store_vec(T* p, const T (&src)[V], bool streaming) {
-    if constexpr (V == 1) {
-        if (streaming) __builtin_nontemporal_store(src[0], p); else *p = src[0];
-    } else {
+__device__ __forceinline__ void store_vec(T* p, const T (&src)[V]) {
+    if constexpr (V == 1) *p = src[0];
+    else {
         typename VecOf<T, V>::type v;
 #pragma unroll
         for (int i = 0; i < V; i++) v[i] = src[i];
-        if (streaming) __builtin_nontemporal_store(v, (typename VecOf<T, V>::type*)p);
-        else *(typename VecOf<T, V>::type*)p = v;
+        *(typename VecOf<T, V>::type*)p = v;
     }
 }
 
@@ -257,7 +258,6 @@ struct RowsArgs {
     int simple_loads;          // every source register is filled by a plain vector load
     int vec;                   // elements per thread and pass (1 or 16 / sizeof(T))
     int ragged;                // L is not a multiple of vec: the last vector of a row is moved back to end with the row
-    int streaming;             // non-temporal stores for the drain
     int nt_loads;              // every source element is read exactly once: the host picks the non-temporal-load variant
     FastDiv chunk_div;
     FastDiv outer[ROWS_MAX_OUTER];           // outer[0] is the innermost outer axis
@@ -377,7 +377,7 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
     for (int p = 0; p < PASSES; p++) {
         if (live[p]) {
             T (&op)[V] = *reinterpret_cast<T (*)[V]>(&out[p * V]);
-            store_vec<T, V>(drn + doff[p], op, A.streaming != 0);
+            store_vec<T, V>(drn + doff[p], op);
         }
     }
 }
@@ -418,7 +418,7 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
     _Pragma("unroll") for (int p = 0; p < PASSES; p++) {                              \
         T out[V];                                                                     \
         _Pragma("unroll") for (int v = 0; v < V; v++) { const T a = x0[p][v], b = x1[p][v]; out[v] = (EXPR); } \
-        if (live[p]) store_vec<T, V>(drn + doff[p], out, A.streaming != 0);           \
+        if (live[p]) store_vec<T, V>(drn + doff[p], out);                                     \
     }
     switch (op) {
         case NK_OP_ADD: NK_BINARY_PASSES(a + b) break;
@@ -427,6 +427,58 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
         default: NK_BINARY_PASSES(a / b) break;
     }
 #undef NK_BINARY_PASSES
+}
+
+// Large outputs (the write stream dominates): one unit per block and non-temporal stores.  Measured with a plain
+// fill of 4 GiB, blocks that write 4 KiB each in dispatch order reach 6.9 TB/s where blocks of 32 KiB reach 5.8: the
+// window of memory that is being written at one time stays small and moves front to back.  Non-temporal stores
+// keep the output from displacing the (re-used) sources in L2, so the short blocks' loads return quickly; the
+// prologue is kept short for the same reason -- a compact argument block read at once, the number of outer axes a
+// template parameter, rows resolved on the scalar unit.
+struct LeanArgs {
+    unsigned n_rows, L;
+    int tpr_log2;              // threads per row, log2 (>= 6: a row index is wave-uniform)
+    unsigned chunks;           // column chunks per row
+    int op;
+    FastDiv chunk_div;
+    FastDiv outer[ROWS_FAST_OUTER];          // outer[0] is the innermost outer axis
+    int base[3];
+    int stride[3][ROWS_FAST_OUTER];
+};
+template <typename T, int V, int NOUT, bool NT>
+__global__ __launch_bounds__(256) void rows_binary_lean_kernel(LeanArgs A, T* __restrict__ drn, const T* __restrict__ s0, const T* __restrict__ s1) {
+    const unsigned tpr = 1u << A.tpr_log2, rpp = 256u >> A.tpr_log2;
+    const unsigned rg = A.chunk_div.div(blockIdx.x), chunk = blockIdx.x - rg * A.chunks;
+    const unsigned sub = threadIdx.x >> A.tpr_log2, lane = threadIdx.x & (tpr - 1);
+    unsigned row = rg * rpp + sub, col = (chunk * tpr + lane) * (unsigned)V;
+    const bool row_ok = row < A.n_rows;
+    const bool live = row_ok && col < A.L;
+    if (!row_ok) row = 0;                        // dead lanes get a valid address: the loads need no predicate
+    if (!live) col = 0;
+    unsigned r = __builtin_amdgcn_readfirstlane(row);
+    int off0 = A.base[0], off1 = A.base[1], off2 = A.base[2];
+#pragma unroll
+    for (int k = 0; k < NOUT; k++) {
+        const unsigned q = A.outer[k].div(r);
+        const int idx = (int)(r - q * A.outer[k].d);
+        r = q;
+        off0 += idx * A.stride[0][k]; off1 += idx * A.stride[1][k]; off2 += idx * A.stride[2][k];
+    }
+    T a[V], b[V], out[V];
+    load_vec<T, V, NT>(a, s0 + off1 + col);
+    load_vec<T, V, NT>(b, s1 + off2 + col);
+    switch (A.op) {
+        case NK_OP_ADD: _Pragma("unroll") for (int v = 0; v < V; v++) out[v] = a[v] + b[v]; break;
+        case NK_OP_SUB: _Pragma("unroll") for (int v = 0; v < V; v++) out[v] = a[v] - b[v]; break;
+        case NK_OP_MUL: _Pragma("unroll") for (int v = 0; v < V; v++) out[v] = a[v] * b[v]; break;
+        default:        _Pragma("unroll") for (int v = 0; v < V; v++) out[v] = a[v] / b[v]; break;
+    }
+    if (live) {
+        typename VecOf<T, V>::type w;
+#pragma unroll
+        for (int v = 0; v < V; v++) w[v] = out[v];
+        __builtin_nontemporal_store(w, (typename VecOf<T, V>::type*)(drn + off0 + col));
+    }
 }
 
 // ---- canon kernel: arbitrary strides, one element per thread -------------------------------------------
@@ -482,7 +534,6 @@ struct TileArgs {
     unsigned tiles_p, tiles_l;
     unsigned n_blocks;
     int group_log2, group_p_log2;           // blocks are numbered through groups of (1 << group_p_log2) x (1 << group_log2) tiles
-    int streaming;
     int nt_loads;                           // every source element is read exactly once: the host picks the non-temporal-load variant
     int careful;                            // some direct operand is constant along the innermost axis: no vector path
     int xcd_regions;                        // XCD x (blocks x, x + 8, ...) takes the x-th eighth of the tile order
@@ -585,7 +636,7 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
 #pragma unroll
         for (int it = 0; it < W_NIT; it++) {
             T (&ov)[VEC] = *reinterpret_cast<T (*)[VEC]>(&out[it * VEC]);
-            store_vec<T, VEC>(dp + (int64_t)(p0 + wr + W_RPI * it) * dP, ov, A.streaming != 0);
+            store_vec<T, VEC>(dp + (int64_t)(p0 + wr + W_RPI * it) * dP, ov);
         }
         return;
     }
@@ -634,7 +685,7 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
         const unsigned p = p0 + dy + D_RPI * it, l = l0 + dx;
         if (p < A.P && l < A.L) {
             T* dst = drn + off[0] + (int64_t)p * dP + l;
-            if (A.streaming) __builtin_nontemporal_store(out[it], dst); else *dst = out[it];
+            *dst = out[it];
         }
     }
 }
@@ -687,6 +738,7 @@ struct Plan {
     int hoist = 0;             // rows_binary_kernel: bit j = source j is loaded once per block
     int binary_op;             // PLAN_ROWS_BINARY
     int passes;                // PLAN_ROWS_BINARY: units per block (2, 4 or 8)
+    bool lean = false;         // PLAN_ROWS_BINARY: rows_binary_lean_kernel (one unit per block, non-temporal stores)
     int nsrc;
     unsigned grid;
     RowsArgs rows;

@@ -170,7 +170,8 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         for (int i = 0; i < LIGHT_CONST; i++) plan.light.consts[i] = prog.consts[i];
     }
     // outputs far larger than the last-level cache are written with non-temporal stores
-    const bool streaming = env_flag("NK_STREAMING_STORES", true) && (uint64_t)c.n * sizeof(T) >= ((uint64_t)64 << 20);
+    // an output far larger than the caches: sources read once are loaded past them, re-used ones take the lean kernel
+    const bool streaming = (uint64_t)c.n * sizeof(T) >= ((uint64_t)64 << 20);
 
     Canon cn;
     const bool canon_ok = canonicalize(cn, c.rank, cfgs[0].shape, c.nsrc + 1, cfgp, axis_on, own_unravel);
@@ -237,7 +238,6 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         int passes = rows_passes(funset, funset >= 2 ? NK_FUSE_MAX_SRC : (c.nsrc <= 1 ? 1 : c.nsrc));
         A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
-        A.streaming = streaming ? 1 : 0;
         // sources at least as large as the drain's threshold whose every element is read once stream past the caches
         bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
         for (int j = 0; j < c.nsrc && once; j++)
@@ -306,8 +306,16 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // one block per `passes` units, no grid-stride loop
         plan.grid = A.pass_rows ? (unsigned)(((row_groups + passes - 1) / passes) * A.chunks)
                                 : (unsigned)((row_groups * A.chunks + passes - 1) / passes);
-        set_path(plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary")
-                                               : vec ? "rows_vec" : "rows");
+        // large outputs of the binary kernel: one unit per block, non-temporal stores
+        static const int lean_mode = [] { const char* v = getenv("NK_BINARY_LEAN"); return v && *v ? atoi(v) : 1; }();
+        if (plan.kind == PLAN_ROWS_BINARY && vec && streaming && !deep && !ragged && A.const_last == 0 && A.strided_last == 0 && A.tpr_log2 >= 6 &&
+            lean_mode != 0 && (lean_mode == 2 || !A.nt_loads)) {
+            plan.lean = true;
+            plan.hoist = 0;
+            plan.grid = (unsigned)(row_groups * A.chunks);
+        }
+        set_path(plan.lean ? "rows_vec_binary_lean"
+                           : plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary") : vec ? "rows_vec" : "rows");
         done = true;
     }
 
@@ -328,7 +336,6 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         if (ok && pax >= 0) {
             TileArgs& A = plan.tile;
             A.rank = cn.rank; A.nsrc = c.nsrc; A.pax = pax; A.turned = turned;
-            A.streaming = streaming ? 1 : 0;
             bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
             for (int j = 0; j < c.nsrc && once; j++)
                 for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) once = false;

@@ -52,7 +52,7 @@ def test_config2_broadcast_full_size(device, orc, dt, s1, s2):
     out = Tensor._on_device(device, T, so)
     for op, f in (("add", np.add), ("multiply", np.multiply)):
         device.launch_broadcast(op, -1, out, ta, tb)
-        assert _lib.last_path() == "rows_vec_binary"
+        assert _lib.last_path() == "rows_vec_binary_lean"      # 64 MiB and more with re-used sources: one unit per block
         got = out.getData().reshape(so)
         # slabs against the oracle (bit for bit) ...
         for o0 in (0, 1, so[0] // 2, so[0] - 1):
@@ -233,3 +233,48 @@ def test_reductions_over_2_pow_26_elements(device, orc):
     assert_bits(got, np.array([orc.sum_tree(a * b)], dtype=f32), "dot as multiply + sum")
     assert abs(float(got[0]) - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) <= 1e-5 * float(np.abs(a * b).sum(dtype=np.float64))
     free(device, ta, tb)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_large_broadcast_outputs_one_unit_per_block(device, orc, dt):
+    """Outputs of 64 MiB and more whose sources are re-used take the binary kernel's variant with one unit per block and
+    non-temporal stores: rows longer than a block (several column chunks), row counts that leave the last block half
+    empty, one to three outer axes, a source that is a slice of a larger tensor, all four operators -- every result
+    bit for bit the oracle's (numpy's single IEEE operation per element for + - * /)."""
+    T = np.dtype(dt.replace("f", "float"))
+    scale = 1 if dt == "f32" else 2                      # the same number of bytes in f64
+    rng = np.random.default_rng(9)
+    cases = [("add", (4096 // scale, 4100), (1, 4100), None),
+             ("subtract", (4099 // scale, 1, 512), (1, 9, 512), None),
+             ("multiply", (70 // scale, 1, 17, 256), (1, 61, 1, 256), None),
+             ("divide", (4096 // scale, 1, 260), (1, 17, 260), None),
+             ("add", (4096 // scale, 4100), (1, 4100), "sliced"),
+             ("multiply", (1, 4100), (4096 // scale, 4100), None)]
+    for op, sa, sb, view in cases:
+        so = tuple(max(p, q) for p, q in zip(sa, sb))
+        say("large broadcast", op, sa, sb, view or "", dt)
+        assert int(np.prod(so)) * T.itemsize >= 64 << 20
+        b = rng.uniform(0.5, 1.5, sb).astype(T)
+        tb = on(device, b)
+        if view == "sliced":                              # rows of a wider parent, starting 16 bytes in
+            pad = 16 // T.itemsize
+            parent = rng.uniform(-1, 1, (sa[0] + 2, sa[1] + 2 * pad)).astype(T)
+            ta = on(device, parent)[1:1 + sa[0], pad:pad + sa[1]]
+            a = parent[1:1 + sa[0], pad:pad + sa[1]]
+        else:
+            a = rng.uniform(-1, 1, sa).astype(T)
+            ta = on(device, a)
+        out = Tensor._on_device(device, T, so)
+        device.launch_broadcast(op, -1, out, ta, tb)
+        assert _lib.last_path() == "rows_vec_binary_lean", _lib.last_path()
+        f = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide}[op]
+        assert_bits(out.getData().reshape(so), f(a, b).astype(T), f"{op} {sa} {sb}")
+        # ... and a slab through the oracle's own state machine
+        rows = 3
+        first = tuple(slice(0, min(rows, s)) if k == 0 else slice(None) for k, s in enumerate(so))
+        ssa = tuple(min(rows, s) if k == 0 else s for k, s in enumerate(sa)); ssb = tuple(min(rows, s) if k == 0 else s for k, s in enumerate(sb))
+        sso = tuple(max(p, q) for p, q in zip(ssa, ssb))
+        want = orc.broadcast(op, -1, np.zeros(int(np.prod(sso)), dtype=T), orc.dense_cfg(sso), np.ascontiguousarray(a[first[:len(sa)]] if sa[0] > 1 else a).reshape(-1),
+                             orc.dense_cfg(ssa), np.ascontiguousarray(b[first[:len(sb)]] if sb[0] > 1 else b).reshape(-1), orc.dense_cfg(ssb))
+        assert_bits(out.getData().reshape(so)[first].reshape(-1), want, f"oracle slab {op}")
+        free(device, ta, tb, out)

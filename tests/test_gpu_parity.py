@@ -61,6 +61,23 @@ def test_memory_roundtrip_fill_and_accounting(device):
             small.release()
 
 
+def test_large_fills_every_pattern_size(device):
+    """Fills of a MiB and more go through 16-byte stores with the pattern repeated, the rest of the last 16 bytes
+    through the element kernel; a start that is not on a 16-byte boundary keeps the element kernel.  Every element
+    type's pattern, the elements before and after the filled range untouched."""
+    say("large fills")
+    for dt, value in ((np.int8, -7), (np.int16, -12345), (np.float32, -0.0), (np.float32, 3.25), (np.float64, -1e-300), (np.int64, -(2 ** 62) - 5)):
+        n = (3 << 20) // np.dtype(dt).itemsize + 37
+        for start, count in ((0, n), (16 // np.dtype(dt).itemsize, n - 2 * (16 // np.dtype(dt).itemsize) - 3), (1, n - 2)):
+            data = device.allocate(dt, n)
+            device._fill(data, 0, n, 1)
+            device._fill(data, start, count, value)
+            got = device._read_all(data)
+            want = np.ones(n, dtype=dt); want[start:start + count] = value
+            assert got.tobytes() == want.tobytes(), (np.dtype(dt).name, start, count)
+            data.release()
+
+
 def test_store_restore_free_virtual_and_slices(device):
     say("device contract")
     stored, objs = device.numberOfStored(), device.numberOfDataObjects()
