@@ -25,7 +25,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
 FP64_PEAK_TFLOPS = 78.6        # MI355X dense fp64 matrix, published
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
-# against a plain 1 GiB copy): profiles/rows_binary_kernel_broadcast_c2.md
+# against a plain 1 GiB copy): profiles/rows_binary_lean_kernel_broadcast_c2.md
 C2_TRAFFIC_BYTES = 4316386969
 
 
@@ -168,7 +168,7 @@ def main():
     singles = sorted(event_times_ms(dev, launch_add, 50) + event_times_ms(dev, launch_mul, 50))
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_TRAFFIC_BYTES if path == "rows_vec_binary_lean" else None,
-                "kernel": f"nk::rows_binary_lean_kernel<float, 4, 2, false> ({path})",
+                "kernel": f"nk::rows_binary_lean_kernel<float, 4, 2, 0, true> ({path})",
                 "launch_ms": round(k_ms, 4), "algorithmic_bytes": bytes_per_launch,
                 "single_launch_ms": {"p10": round(singles[len(singles) // 10], 4), "median": round(singles[len(singles) // 2], 4),
                                      "p90": round(singles[(len(singles) * 9) // 10], 4), "launches": len(singles)}}

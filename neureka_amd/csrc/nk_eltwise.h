@@ -445,7 +445,9 @@ struct LeanArgs {
     int base[3];
     int stride[3][ROWS_FAST_OUTER];
 };
-template <typename T, int V, int NOUT, bool NT>
+// CONST bit j: source j does not change along a row (one element per row).  WIDE: a row spans at least a wavefront, so
+// its index is wave-uniform and is resolved on the scalar unit.
+template <typename T, int V, int NOUT, int CONST, bool WIDE>
 __global__ __launch_bounds__(256) void rows_binary_lean_kernel(LeanArgs A, T* __restrict__ drn, const T* __restrict__ s0, const T* __restrict__ s1) {
     const unsigned tpr = 1u << A.tpr_log2, rpp = 256u >> A.tpr_log2;
     const unsigned rg = A.chunk_div.div(blockIdx.x), chunk = blockIdx.x - rg * A.chunks;
@@ -455,7 +457,7 @@ __global__ __launch_bounds__(256) void rows_binary_lean_kernel(LeanArgs A, T* __
     const bool live = row_ok && col < A.L;
     if (!row_ok) row = 0;                        // dead lanes get a valid address: the loads need no predicate
     if (!live) col = 0;
-    unsigned r = __builtin_amdgcn_readfirstlane(row);
+    unsigned r = WIDE ? (unsigned)__builtin_amdgcn_readfirstlane(row) : row;
     int off0 = A.base[0], off1 = A.base[1], off2 = A.base[2];
 #pragma unroll
     for (int k = 0; k < NOUT; k++) {
@@ -465,8 +467,10 @@ __global__ __launch_bounds__(256) void rows_binary_lean_kernel(LeanArgs A, T* __
         off0 += idx * A.stride[0][k]; off1 += idx * A.stride[1][k]; off2 += idx * A.stride[2][k];
     }
     T a[V], b[V], out[V];
-    load_vec<T, V, NT>(a, s0 + off1 + col);
-    load_vec<T, V, NT>(b, s1 + off2 + col);
+    if constexpr (CONST & 1) { const T c = s0[off1]; _Pragma("unroll") for (int v = 0; v < V; v++) a[v] = c; }
+    else load_vec<T, V>(a, s0 + off1 + col);
+    if constexpr (CONST & 2) { const T c = s1[off2]; _Pragma("unroll") for (int v = 0; v < V; v++) b[v] = c; }
+    else load_vec<T, V>(b, s1 + off2 + col);
     switch (A.op) {
         case NK_OP_ADD: _Pragma("unroll") for (int v = 0; v < V; v++) out[v] = a[v] + b[v]; break;
         case NK_OP_SUB: _Pragma("unroll") for (int v = 0; v < V; v++) out[v] = a[v] - b[v]; break;

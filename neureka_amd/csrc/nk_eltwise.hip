@@ -308,8 +308,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
                                 : (unsigned)((row_groups * A.chunks + passes - 1) / passes);
         // large outputs of the binary kernel: one unit per block, non-temporal stores
         static const int lean_mode = [] { const char* v = getenv("NK_BINARY_LEAN"); return v && *v ? atoi(v) : 1; }();
-        if (plan.kind == PLAN_ROWS_BINARY && vec && streaming && !deep && !ragged && A.const_last == 0 && A.strided_last == 0 && A.tpr_log2 >= 6 &&
-            lean_mode != 0 && (lean_mode == 2 || !A.nt_loads)) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && streaming && !deep && !ragged && A.strided_last == 0 && lean_mode != 0 && !A.nt_loads) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);

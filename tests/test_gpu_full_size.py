@@ -249,7 +249,11 @@ def test_large_broadcast_outputs_one_unit_per_block(device, orc, dt):
              ("multiply", (70 // scale, 1, 17, 256), (1, 61, 1, 256), None),
              ("divide", (4096 // scale, 1, 260), (1, 17, 260), None),
              ("add", (4096 // scale, 4100), (1, 4100), "sliced"),
-             ("multiply", (1, 4100), (4096 // scale, 4100), None)]
+             ("multiply", (1, 4100), (4096 // scale, 4100), None),
+             ("multiply", (8192 // scale, 1), (1, 4096), None),              # an outer product: both sources constant along a row or a column
+             ("add", ((1 << 20) // scale, 1), (1, 32), None),               # short rows: several rows per wavefront
+             ("subtract", ((1 << 19) // scale, 64), (1, 64), None),
+             ("divide", (300 // scale, 1, 70, 1), (1, 50, 1, 64), None)]
     for op, sa, sb, view in cases:
         so = tuple(max(p, q) for p, q in zip(sa, sb))
         say("large broadcast", op, sa, sb, view or "", dt)
