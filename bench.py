@@ -26,7 +26,7 @@ FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
 FP64_PEAK_TFLOPS = 78.6        # MI355X dense fp64 matrix, published
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
 # against a plain 1 GiB copy): profiles/rows_binary_lean_kernel_broadcast_c2.md
-C2_TRAFFIC_BYTES = 4316386969
+C2_TRAFFIC_BYTES = 4316437187
 
 
 def event_time_ms(dev, launch, reps):
