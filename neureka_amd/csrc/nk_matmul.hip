@@ -258,6 +258,146 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     }
 }
 
+// Whole tiles, no split, more tiles than resident blocks: blocks that stay.  A block walks the tiles blockIdx.x,
+// + gridDim.x, ... and the software pipeline over the k-slices runs on across them: the first slice of the next
+// tile is fetched and written to the free LDS buffer during the last slice of the current one, so only the
+// block's very first slice is waited for.  The result leaves straight from the accumulators (32 lanes cover 128
+// contiguous bytes of a row of C), which needs neither LDS nor a barrier and so does not disturb the pipeline.
+__global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, const float* __restrict__ A,
+                                                                 const float* __restrict__ B, float* __restrict__ C) {
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS_AB];
+    float* const As0 = lds;
+    float* const Bs0 = lds + 2 * BM * A_PITCH;
+    const int n_tiles = g.tiles_m * g.tiles_n;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int a_row = tid >> 3, a_col = (tid & 7) * 4;
+    const int b_row = tid >> 5, b_col = (tid & 31) * 4;
+    f32x4 ra[4], rb[4];
+    auto load_global = [&](int tm, int tn, int k0) {
+        const float* Ag = A + (int64_t)tm * BM * g.K;
+        const float* Bg = B + (int64_t)tn * BN;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 8 * i) * g.N + b_col);
+        }
+    };
+    auto store_lds = [&](int buf) {
+        float* as = As0 + buf * (BM * A_PITCH);
+        float* bs = Bs0 + buf * (BK * B_PITCH);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            *(f32x4*)(&as[(a_row + 32 * i) * A_PITCH + a_col]) = ra[i];
+            *(f32x4*)(&bs[(b_row + 8 * i) * B_PITCH + b_col]) = rb[i];
+        }
+    };
+    auto read_frag = [&](Frag& f, int buf, int c) {
+        const float* as = As0 + buf * (BM * A_PITCH);
+        const float* bs = Bs0 + buf * (BK * B_PITCH);
+        f.a0 = *(const f32x4*)(&as[(wm + l32) * A_PITCH + 8 * c + 4 * h]);
+        f.a1 = *(const f32x4*)(&as[(wm + 32 + l32) * A_PITCH + 8 * c + 4 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            f.b0[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + l32];
+            f.b1[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + 32 + l32];
+        }
+    };
+    f32x16 acc[2][2];
+    auto clear = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    };
+    auto mma = [&](const Frag& f) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b0[t], acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b1[t], acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b0[t], acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b1[t], acc[1][1], 0, 0, 0);
+        }
+    };
+    static_assert(BK == 32, "the pipeline below is written for four depth-8 chunks per slice");
+    const int nk = g.K / BK;
+
+    int tile = blockIdx.x;
+    if (tile >= n_tiles) return;
+    int tm, tn;
+    tile_of_block(g, tile, tm, tn);
+    Frag f0, f1;
+    clear();
+    load_global(tm, tn, 0);
+    store_lds(0);
+    __syncthreads();
+    read_frag(f0, 0, 0);
+    int phase = 0;                                         // LDS buffer that holds slice 0 of the current tile
+    for (;;) {
+        for (int kt = 0; kt + 1 < nk; kt++) {              // as in matmul_mfma_kernel
+            const int cur = (kt + phase) & 1;
+            load_global(tm, tn, (kt + 1) * BK);
+            read_frag(f1, cur, 1);
+            mma(f0);
+            read_frag(f0, cur, 2);
+            mma(f1);
+            store_lds(cur ^ 1);
+            read_frag(f1, cur, 3);
+            mma(f0);
+            __syncthreads();
+            read_frag(f0, cur ^ 1, 0);
+            mma(f1);
+        }
+        // last slice of this tile; the first slice of the next tile takes the place of "slice kt + 1"
+        const int cur = (nk - 1 + phase) & 1;
+        const int next = tile + (int)gridDim.x;
+        const bool more = next < n_tiles;                  // the same for the whole block
+        int nm = tm, nn = tn;
+        if (more) { tile_of_block(g, next, nm, nn); load_global(nm, nn, 0); }
+        // C += the tile: accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4, column l32.  Addresses are a
+        // wave-uniform part (tile, sub-tile, accumulator: scalar registers) plus one 32-bit offset per lane.  The old
+        // values of the upper two sub-tiles are requested before the last multiply-adds, those of the lower two
+        // while the upper two are stored.
+        float* const Cg = C + (int64_t)tm * BM * g.N + tn * BN;
+        const unsigned lane_off = (unsigned)((wm + 4 * h) * g.N + wn + l32);
+        float old[2][16];
+        auto fetch_old = [&](int i) {
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) old[j][v] = (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off];
+        };
+        auto store_new = [&](int i) {
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off] = old[j][v] + acc[i][j][v];
+        };
+        fetch_old(0);
+        read_frag(f1, cur, 1);
+        mma(f0);
+        read_frag(f0, cur, 2);
+        mma(f1);
+        if (more) store_lds(cur ^ 1);
+        read_frag(f1, cur, 3);
+        mma(f0);
+        __syncthreads();
+        if (more) read_frag(f0, cur ^ 1, 0);
+        mma(f1);
+        store_new(0);
+        fetch_old(1);
+        store_new(1);
+        if (!more) break;
+        clear();
+        tile = next; tm = nm; tn = nn;
+        phase = cur ^ 1;
+    }
+}
+
 // C[i] += part_0[i] + part_1[i] + ... in that order (the parts of a SPLIT product)
 template <typename T>
 __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int parts, const T* __restrict__ P, T* __restrict__ C) {
@@ -467,13 +607,27 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
     const bool edge = !whole_tiles && M * K * N >= mfma_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
     if (whole_tiles || edge) {
         const float* Ap = (const float*)A; const float* Bp = (const float*)B; float* Cp = (float*)C;
+        bool streamed = false;
         const int rc = launch_mfma<float>(dev, g, BK, Cp, [&](bool split, dim3 grid, float* P) {
             if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
-            else if (whole_tiles)     hipLaunchKernelGGL((matmul_mfma_kernel<false, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+            else if (whole_tiles) {
+                // more tiles than blocks that fit the machine at one time: the blocks stay and walk the tiles
+                static const int stream_mode = [] { const char* v = getenv("NK_MATMUL_STREAM"); return v && *v ? atoi(v) : 1; }();
+                const unsigned resident = 2u * (unsigned)dev->props.multiProcessorCount;
+                const unsigned tiles = (unsigned)(g.tiles_m * g.tiles_n);
+                // (pays while a tile has few k-slices, i.e. while its first fetch and its write-back weigh: measured
+                // +4 % at 8 slices, +1 % at 16, -1 % at 128)
+                if (stream_mode && g.K / BK <= 16 && tiles >= 2 * resident && tiles % 8 == 0 && resident % 8 == 0) {
+                    hipLaunchKernelGGL(matmul_mfma_stream_kernel, dim3(resident), dim3(256), 0, dev->stream, g, Ap, Bp, Cp);
+                    streamed = true;
+                }
+                else
+                    hipLaunchKernelGGL((matmul_mfma_kernel<false, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
+            }
             else if (split)           hipLaunchKernelGGL((matmul_mfma_kernel<true, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
             else                      hipLaunchKernelGGL((matmul_mfma_kernel<true, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
         });
-        set_path(whole_tiles ? (g.splits > 1 ? "mfma_split" : "mfma") : (g.splits > 1 ? "mfma_edge_split" : "mfma_edge"));
+        set_path(streamed ? "mfma_stream" : whole_tiles ? (g.splits > 1 ? "mfma_split" : "mfma") : (g.splits > 1 ? "mfma_edge_split" : "mfma_edge"));
         return rc;
     }
     return launch_simple<float>(dev, M, K, N, (const float*)A, (const float*)B, (float*)C);

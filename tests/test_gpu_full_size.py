@@ -165,7 +165,7 @@ def test_config4_matmul_full_size(device, mkn):
     A = rng.integers(-3, 4, (M, K)).astype(f32); B = rng.integers(-3, 4, (K, N)).astype(f32)
     ta, tb = on(device, A), on(device, B)
     c = ta.matMul(tb)
-    assert _lib.last_path() == "mfma"
+    assert _lib.last_path() == ("mfma" if K == 4096 else "mfma_stream")      # few k-slices per tile: the blocks walk the tiles
     got = c.items.reshape(M, N)
     rows = rng.choice(M, 48, replace=False)
     assert (got[rows] == A[rows].astype(np.float64) @ B.astype(np.float64)).all()

@@ -1304,6 +1304,35 @@ def test_random_products_through_every_plan(device, dt):
     assert "simple" in seen and any(p.endswith("_split") for p in seen) and any("edge" in p for p in seen), sorted(seen)
 
 
+@pytest.mark.parametrize("mkn", [(16384, 64, 1024), (8192, 96, 2048), (65536, 32, 256), (4096, 160, 4096), (12288, 512, 1536)])
+def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
+    """Whole-tile f32 products with few k-slices per tile and at least four tiles per compute unit: the blocks stay,
+    walk the tiles and keep the k-slice pipeline running across them (an odd and an even number of slices per tile
+    alternate the LDS buffers differently; one slice per tile leaves only the hand-over).  Exact on integer-valued
+    data with accumulation into a non-zero C, both layouts; within 1e-5 norm-wise on uniform data."""
+    M, K, N = mkn
+    rng = np.random.default_rng(58)
+    say("matmul walking blocks, integers", mkn)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float32); B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    C0 = rng.integers(-9, 10, (M, N)).astype(np.float32)
+    want = A.astype(np.float64) @ B.astype(np.float64) + C0
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == "mfma_stream"
+    assert (tc.getData().reshape(M, N) == want).all()
+    say("matmul walking blocks, column major", mkn)
+    tc = on(device, C0.T.copy())
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+    assert (tc.getData().reshape(N, M).T == want).all()
+    say("matmul walking blocks, uniform", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    tc = on(device, np.zeros((M, N), dtype=np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
