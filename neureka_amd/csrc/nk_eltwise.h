@@ -437,7 +437,7 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
 // template parameter, rows resolved on the scalar unit.
 struct LeanArgs {
     unsigned n_rows, L;
-    int tpr_log2;              // threads per row, log2 (>= 6: a row index is wave-uniform)
+    int tpr_log2;              // threads per row, log2
     unsigned chunks;           // column chunks per row
     int op;
     FastDiv chunk_div;
