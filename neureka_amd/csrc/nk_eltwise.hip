@@ -308,12 +308,23 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
                                 : (unsigned)((row_groups * A.chunks + passes - 1) / passes);
         // large outputs of the binary kernel: one unit per block, non-temporal stores
         static const int lean_mode = [] { const char* v = getenv("NK_BINARY_LEAN"); return v && *v ? atoi(v) : 1; }();
-        if (plan.kind == PLAN_ROWS_BINARY && vec && streaming && !deep && !ragged && A.strided_last == 0 && lean_mode != 0 && !A.nt_loads) {
+        // (only for a drain without gaps: the gain comes from the write front that moves through memory in order; a
+        // drain that is a slice of a wider tensor measured 5 % slower this way)
+        bool drain_dense = cn.stride[0][last] == 1;
+        for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
+        if (plan.kind == PLAN_ROWS_BINARY && vec && streaming && drain_dense && !deep && !ragged && A.strided_last == 0 && lean_mode != 0 && !A.nt_loads) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
-        set_path(plan.lean ? "rows_vec_binary_lean"
+        // ... and of a program that is one constant
+        if (plan.kind == PLAN_ROWS && c.nsrc == 0 && prog.n == 1 && prog.op[0] == I_SET && prog.src[0] == SRC_CONST0 && funset == 0 &&
+            vec && streaming && drain_dense && !deep && !ragged && lean_mode != 0) {
+            plan.lean_fill = true;
+            plan.fill_value = prog.consts[0];
+            plan.grid = (unsigned)(row_groups * A.chunks);
+        }
+        set_path(plan.lean_fill ? "rows_vec_fill_lean" : plan.lean ? "rows_vec_binary_lean"
                            : plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary") : vec ? "rows_vec" : "rows");
         done = true;
     }

@@ -282,3 +282,30 @@ def test_large_broadcast_outputs_one_unit_per_block(device, orc, dt):
                              orc.dense_cfg(ssa), np.ascontiguousarray(b[first[:len(sb)]] if sb[0] > 1 else b).reshape(-1), orc.dense_cfg(ssb))
         assert_bits(out.getData().reshape(so)[first].reshape(-1), want, f"oracle slab {op}")
         free(device, ta, tb, out)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_large_scalar_fills_one_unit_per_block(device, dt):
+    """Fills of 64 MiB and more through the elementwise engine: dense tensors take the variant with one unit per block,
+    slices of larger tensors the general rows kernel; every element of the view takes the value, everything around a
+    sliced view stays as it was."""
+    T = np.dtype(dt.replace("f", "float"))
+    scale = 1 if dt == "f32" else 2
+    say("large fill, dense", dt)
+    t = Tensor._on_device(device, T, (4099 // scale, 4100))
+    device.launch_scalar_fill(t, -2.5)
+    assert _lib.last_path() == "rows_vec_fill_lean", _lib.last_path()
+    assert (t.getData() == T.type(-2.5)).all()
+    free(device, t)
+    for shape, sl in (((4100 // scale, 4200), (slice(1, 4097 // scale), slice(8, 4108))),
+                      ((70 // scale, 61, 17, 272), (slice(None), slice(2, 60), slice(None), slice(8, 264)))):
+        say("large fill, sliced", shape, dt)
+        parent = Tensor._on_device(device, T, shape)
+        device.launch_scalar_fill(parent, 1.0)
+        view = parent[sl]
+        assert view.size * T.itemsize >= 64 << 20
+        device.launch_scalar_fill(view, 7.25)
+        assert _lib.last_path() == "rows_vec", _lib.last_path()              # a drain with gaps keeps the kernel with several units per block
+        want = np.ones(shape, dtype=T); want[sl] = 7.25
+        assert parent.getData().tobytes() == want.tobytes()
+        free(device, parent)
