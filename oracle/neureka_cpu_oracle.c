@@ -17,6 +17,12 @@
  *   convolution fwd/bwd    literal vectors of Tensor_Convolution_Spec, CrossDeviceSystemTest;
  *                          scipy.signal.correlate; the state machines against the closed forms
  *   matmul                 hash known-answers of InternalMatMulTest; numpy matmul on integer data
+ *   power                  the table of special cases in the Javadoc of Math.pow (where C's pow differs the
+ *                          reference's answer is kept)
+ *   reductions             the literal results of Tensor_Stats_Spec / Tensor_Dot_Product_Spec; the tree against
+ *                          its own definition and numpy on integer data
+ *   integer scalar         the enforced Integer / Long rows of Tensor_Operation_Spec, the Java language rules
+ *   broadcast              (wrapping, truncating division, Math.round) against exact integer arithmetic
  *   JVMExecutor split      leaf-count / coverage properties (no golden vector exists: "parity
  *                          unpinned" beyond those properties; it only affects baseline timing)
  *
