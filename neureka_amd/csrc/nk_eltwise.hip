@@ -172,6 +172,9 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     // outputs far larger than the last-level cache are written with non-temporal stores
     // an output far larger than the caches: sources read once are loaded past them, re-used ones take the lean kernel
     const bool streaming = (uint64_t)c.n * sizeof(T) >= ((uint64_t)64 << 20);
+    // the kernels with one unit per block: from 16 MiB of output on (measured: 32 MiB 8.8 -> 7.9 us; at 8 MiB no difference)
+    static const uint64_t lean_from = [] { const char* v = getenv("NK_LEAN_FROM_MIB"); return (uint64_t)(v && *v ? atoll(v) : 16) << 20; }();
+    const bool large = (uint64_t)c.n * sizeof(T) >= lean_from;
 
     Canon cn;
     const bool canon_ok = canonicalize(cn, c.rank, cfgs[0].shape, c.nsrc + 1, cfgp, axis_on, own_unravel);
@@ -239,9 +242,10 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
         // sources at least as large as the drain's threshold whose every element is read once stream past the caches
-        bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
-        for (int j = 0; j < c.nsrc && once; j++)
-            for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) once = false;
+        bool reused = false;                                // some source is read more than once (a broadcast)
+        for (int j = 0; j < c.nsrc; j++)
+            for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) reused = true;
+        bool once = streaming && env_flag("NK_STREAMING_LOADS", true) && !reused;
         const bool deep = last > ROWS_FAST_OUTER;           // more outer axes than the tuned variants resolve: plain variants
         if (deep) once = false;
         A.nt_loads = once ? 1 : 0;
@@ -312,14 +316,14 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // drain that is a slice of a wider tensor measured 5 % slower this way)
         bool drain_dense = cn.stride[0][last] == 1;
         for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
-        if (plan.kind == PLAN_ROWS_BINARY && vec && streaming && drain_dense && !deep && !ragged && A.strided_last == 0 && lean_mode != 0 && !A.nt_loads) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && !ragged && A.strided_last == 0 && lean_mode != 0 && reused) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
         // ... and of a program that is one constant
         if (plan.kind == PLAN_ROWS && c.nsrc == 0 && prog.n == 1 && prog.op[0] == I_SET && prog.src[0] == SRC_CONST0 && funset == 0 &&
-            vec && streaming && drain_dense && !deep && !ragged && lean_mode != 0) {
+            vec && large && drain_dense && !deep && !ragged && lean_mode != 0) {
             plan.lean_fill = true;
             plan.fill_value = prog.consts[0];
             plan.grid = (unsigned)(row_groups * A.chunks);
