@@ -440,6 +440,7 @@ struct LeanArgs {
     int tpr_log2;              // threads per row, log2
     unsigned chunks;           // column chunks per row
     int op;
+    int ragged;                // L is not a multiple of V: the last vector of a row is moved back to end with the row
     FastDiv chunk_div;
     FastDiv outer[ROWS_FAST_OUTER];          // outer[0] is the innermost outer axis
     int base[3];
@@ -457,6 +458,7 @@ __global__ __launch_bounds__(256) void rows_binary_lean_kernel(LeanArgs A, T* __
     const bool live = row_ok && col < A.L;
     if (!row_ok) row = 0;                        // dead lanes get a valid address: the loads need no predicate
     if (!live) col = 0;
+    if (A.ragged && col + (unsigned)V > A.L) col = A.L - (unsigned)V;
     unsigned r = WIDE ? (unsigned)__builtin_amdgcn_readfirstlane(row) : row;
     int off0 = A.base[0], off1 = A.base[1], off2 = A.base[2];
 #pragma unroll
@@ -492,8 +494,10 @@ __global__ __launch_bounds__(256) void rows_fill_lean_kernel(LeanArgs A, T value
     const unsigned tpr = 1u << A.tpr_log2, rpp = 256u >> A.tpr_log2;
     const unsigned rg = A.chunk_div.div(blockIdx.x), chunk = blockIdx.x - rg * A.chunks;
     const unsigned sub = threadIdx.x >> A.tpr_log2, lane = threadIdx.x & (tpr - 1);
-    const unsigned row = rg * rpp + sub, col = (chunk * tpr + lane) * (unsigned)V;
+    const unsigned row = rg * rpp + sub;
+    unsigned col = (chunk * tpr + lane) * (unsigned)V;
     if (row >= A.n_rows || col >= A.L) return;
+    if (A.ragged && col + (unsigned)V > A.L) col = A.L - (unsigned)V;
     unsigned r = WIDE ? (unsigned)__builtin_amdgcn_readfirstlane(row) : row;
     int off0 = A.base[0];
 #pragma unroll

@@ -316,14 +316,14 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // drain that is a slice of a wider tensor measured 5 % slower this way)
         bool drain_dense = cn.stride[0][last] == 1;
         for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
-        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && !ragged && A.strided_last == 0 && lean_mode != 0 && reused) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && lean_mode != 0 && reused) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
         // ... and of a program that is one constant
         if (plan.kind == PLAN_ROWS && c.nsrc == 0 && prog.n == 1 && prog.op[0] == I_SET && prog.src[0] == SRC_CONST0 && funset == 0 &&
-            vec && large && drain_dense && !deep && !ragged && lean_mode != 0) {
+            vec && large && drain_dense && !deep && lean_mode != 0) {
             plan.lean_fill = true;
             plan.fill_value = prog.consts[0];
             plan.grid = (unsigned)(row_groups * A.chunks);

@@ -254,6 +254,8 @@ def test_large_broadcast_outputs_one_unit_per_block(device, orc, dt):
              ("add", ((1 << 20) // scale, 1), (1, 32), None),               # short rows: several rows per wavefront
              ("subtract", ((1 << 19) // scale, 64), (1, 64), None),
              ("divide", (300 // scale, 1, 70, 1), (1, 50, 1, 64), None),
+             ("add", (4096 // scale, 4099), (1, 4099), None),                # rows that are no multiple of a vector
+             ("subtract", (1, 9, 515), (4099 // scale, 1, 515), None),
              ("add", (33 // scale + 1, 1, 1021, 64), (1, 9, 1, 64), None),   # three outer axes above rows of 64 elements
              ("multiply", (524289 // scale, 32), (524289 // scale, 1), None)]  # an odd number of short rows, a per-row scale
     for op, sa, sb, view in cases:
