@@ -386,7 +386,9 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
                 // x-th eighth of the tile order, so the tiles one L2 serves at a time are neighbours in both directions:
                 // its reads (along pax) and its writes (along the innermost axis) add up to long runs
                 static const bool xcd_regions = env_flag("NK_TILE_XCD_REGIONS", true);
-                A.xcd_regions = xcd_regions && nb % 8 == 0;
+                // (with fewer than 8 tiles in a plane the order is ruled by the outer axes and an eighth per XCD is an eighth of
+                // the output per XCD, which a write stream does not like: measured 5.5 -> 4.7 TB/s on a fully reversed rank-4 view)
+                A.xcd_regions = xcd_regions && nb % 8 == 0 && (uint64_t)A.tiles_p * A.tiles_l >= 8;
                 set_path("tile_transpose");
                 done = true;
             }
