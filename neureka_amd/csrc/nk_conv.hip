@@ -821,13 +821,57 @@ static bool conv2d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& 
     return true;
 }
 
+// Forward 1-D convolution of dense vectors, out[j] = sum_k x[j + k] * w[k]: a block owns 256 * R neighbouring outputs,
+// stages the 256 * R + K - 1 inputs they read in LDS once, and every thread adds its R sums tap by tap (k ascending,
+// product rounded before the add) -- the order of _convolve32 / _convolve64 for rank 1, so the result is theirs bit for
+// bit.  The taps come through scalar loads (the index is the same for the whole block).
+template <typename T, int R>
+__global__ __launch_bounds__(256) void conv1d_direct(int N, int K, const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv1d_lds[];
+    T* tile = (T*)conv1d_lds;
+    const int n_out = N - K + 1;
+    const int j0 = blockIdx.x * (256 * R);
+    const int span = 256 * R + K - 1;
+    for (int e = threadIdx.x; e < span; e += 256) tile[e] = j0 + e < N ? x[j0 + e] : T(0);
+    __syncthreads();
+    T acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = T(0);
+    for (int k = 0; k < K; k++) {
+        const T wk = w[k];
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = acc[r] + tile[r * 256 + threadIdx.x + k] * wk;
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int j = j0 + r * 256 + (int)threadIdx.x;
+        if (j < n_out) out[j] = acc[r];
+    }
+}
+
+template <typename T>
+static bool conv1d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& c0, const T* s1, const Cfg& c1, const T* s2, const Cfg& c2) {
+    if (rank != 1 || d >= 0 || !dense_rm(c0, 1) || !dense_rm(c1, 1) || !dense_rm(c2, 1)) return false;
+    const bool first_long = c1.shape[0] >= c2.shape[0];
+    const int N = first_long ? c1.shape[0] : c2.shape[0], K = first_long ? c2.shape[0] : c1.shape[0];
+    constexpr int R = 4;
+    if (K < 2 || K > 4096 || N - K + 1 < 4096) return false;          // short vectors stay on the general kernel
+    const T* x = first_long ? s1 : s2;
+    const T* w = first_long ? s2 : s1;
+    const unsigned blocks = (unsigned)((N - K + 1 + 256 * R - 1) / (256 * R));
+    const size_t lds = (size_t)(256 * R + K - 1) * sizeof(T);
+    hipLaunchKernelGGL((conv1d_direct<T, R>), dim3(blocks), dim3(256), lds, dev->stream, N, K, x, w, out);
+    set_path("simple1d");
+    return true;
+}
+
 template <typename T>
 static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, nk_buf a, const Cfg& c1, nk_buf b,
                       const Cfg& c2, int64_t n) {
     T* out = (T*)drn;
     const T* s1 = (const T*)a;
     const T* s2 = (const T*)b;
-    if (conv2d_direct_path<T>(dev, d, rank, out, c0, s1, c1, s2, c2)) {
+    if (conv2d_direct_path<T>(dev, d, rank, out, c0, s1, c1, s2, c2) || conv1d_direct_path<T>(dev, d, rank, out, c0, s1, c1, s2, c2)) {
         NK_HIP(hipGetLastError());
         return NK_OK;
     }

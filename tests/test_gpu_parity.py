@@ -1043,6 +1043,36 @@ def test_conv2d_large_images_bit_exact(device, orc, shape):
     assert_bits(y2.items, want, "operand order")
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_conv1d_long_vectors_bit_exact(device, orc, dt):
+    """Dense vectors with at least 4096 outputs and 2 to 4096 taps take the 1-D kernel (inputs staged in LDS, sums tap
+    by tap in the reference's order): bit for bit the oracle's general state machine, either operand order; shorter
+    vectors, longer tap sets and views keep the general kernel -- and agree with it too."""
+    T = F[dt]
+    rng = np.random.default_rng(48)
+    for n, k, path in ((5000, 2, "simple1d"), (70001, 64, "simple1d"), (4096 + 4095, 4096, "simple1d"), (100000, 333, "simple1d"),
+                       (4000, 64, "literal_fwd"), (9000, 5000, None), (70001, 1, "literal_fwd")):
+        say("conv1d", n, k, dt)
+        if path is None:        # whichever general kernel takes it (sums may be split): integer data, exact in any order
+            x = rng.integers(-3, 4, n).astype(T); w = rng.integers(-3, 4, k).astype(T)
+        else:
+            x = rng.uniform(-1, 1, n).astype(T); w = rng.uniform(-1, 1, k).astype(T)
+        want = orc.convolve(np.zeros(n - k + 1, dtype=T), orc.dense_cfg([n - k + 1]), x, orc.dense_cfg([n]), w, orc.dense_cfg([k]))
+        for first, second in ((x, w), (w, x)):
+            out = Tensor._on_device(device, T, [n - k + 1])
+            device.launch_convolution(-1, out, on(device, first), on(device, second))
+            if path is not None:
+                assert _lib.last_path() == path, (_lib.last_path(), n, k)
+            assert_bits(out.getData(), want, f"conv1d {n} {k}")
+    say("conv1d on a strided view stays general", dt)
+    big = rng.uniform(-1, 1, 20000).astype(T); w = rng.uniform(-1, 1, 9).astype(T)
+    view = on(device, big)[::2]
+    out = Tensor._on_device(device, T, [10000 - 8])
+    device.launch_convolution(-1, out, view, on(device, w))
+    assert _lib.last_path() == "literal_fwd"
+    assert_bits(out.getData(), orc.convolve(np.zeros(9992, dtype=T), orc.dense_cfg([9992]), big, cfg(view), w, orc.dense_cfg([9])), "strided view")
+
+
 def test_conv2d_config1_shape(device, orc):
     """[64,64] x [3,3] -> [62,62] (the reference runs this on SimpleCPUConvolution: ky outer, kx inner)."""
     say("conv2d 64x64 x 3x3")
