@@ -849,9 +849,55 @@ __global__ __launch_bounds__(256) void conv1d_direct(int N, int K, const T* __re
     }
 }
 
+// Gradient of the same convolution by the long operand: dx[i] = sum_e w[i - e] * err[e] over the error entries that
+// pass the bounds test, e ascending (_deConvolve32 / _deConvolve64 for rank 1).  The same staging; entries outside the
+// error are skipped by a predicate, not replaced by zeros (a zero times an infinite tap would not be nothing).
+template <typename T, int R>
+__global__ __launch_bounds__(256) void conv1d_grad_long(int N, int K, const T* __restrict__ w, const T* __restrict__ err, T* __restrict__ dx) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv1d_lds[];
+    T* tile = (T*)conv1d_lds;
+    const int n_err = N - K + 1;
+    const int i0 = blockIdx.x * (256 * R);
+    const int first = i0 - (K - 1);                              // error index of tile[0]
+    const int span = 256 * R + K - 1;
+    for (int s = threadIdx.x; s < span; s += 256) {
+        const int e = first + s;
+        tile[s] = e >= 0 && e < n_err ? err[e] : T(0);
+    }
+    __syncthreads();
+    T acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = T(0);
+    for (int s = 0; s < K; s++) {                                 // tap K - 1 - s meets error entry i - (K - 1) + s
+        const T wk = w[K - 1 - s];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int local = r * 256 + (int)threadIdx.x;
+            const int e = first + local + s;
+            if (e >= 0 && e < n_err) acc[r] = acc[r] + wk * tile[local + s];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        const int i = i0 + r * 256 + (int)threadIdx.x;
+        if (i < N) dx[i] = acc[r];
+    }
+}
+
 template <typename T>
 static bool conv1d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& c0, const T* s1, const Cfg& c1, const T* s2, const Cfg& c2) {
-    if (rank != 1 || d >= 0 || !dense_rm(c0, 1) || !dense_rm(c1, 1) || !dense_rm(c2, 1)) return false;
+    if (rank != 1 || !dense_rm(c0, 1) || !dense_rm(c1, 1) || !dense_rm(c2, 1)) return false;
+    if (d >= 0) {
+        // drain = the long operand, src1 = the taps, src2 = the error [N - K + 1]
+        const int N = c0.shape[0], K = c1.shape[0];
+        constexpr int R = 4;
+        if (K < 2 || K > 4096 || N <= K || c2.shape[0] != N - K + 1 || N < 4096) return false;
+        const unsigned blocks = (unsigned)((N + 256 * R - 1) / (256 * R));
+        const size_t lds = (size_t)(256 * R + K - 1) * sizeof(T);
+        hipLaunchKernelGGL((conv1d_grad_long<T, R>), dim3(blocks), dim3(256), lds, dev->stream, N, K, s1, s2, out);
+        set_path("simple1d_grad");
+        return true;
+    }
     const bool first_long = c1.shape[0] >= c2.shape[0];
     const int N = first_long ? c1.shape[0] : c2.shape[0], K = first_long ? c2.shape[0] : c1.shape[0];
     constexpr int R = 4;

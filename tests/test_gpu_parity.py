@@ -1064,6 +1064,16 @@ def test_conv1d_long_vectors_bit_exact(device, orc, dt):
             if path is not None:
                 assert _lib.last_path() == path, (_lib.last_path(), n, k)
             assert_bits(out.getData(), want, f"conv1d {n} {k}")
+    for n, k in ((5000, 2), (70001, 64), (8200, 4096), (100000, 333)):
+        say("conv1d gradient by the long operand", n, k, dt)
+        w = rng.uniform(-1, 1, k).astype(T); e = rng.uniform(-1, 1, n - k + 1).astype(T)
+        w[0] = np.inf if k == 64 else w[0]                       # an infinite tap must not meet entries outside the error
+        dx = Tensor._on_device(device, T, [n])
+        device.launch_convolution(0, dx, on(device, w), on(device, e))
+        assert _lib.last_path() == "simple1d_grad", _lib.last_path()
+        with np.errstate(all="ignore"):
+            want = orc.deconvolve(np.zeros(n, dtype=T), orc.dense_cfg([n]), w, orc.dense_cfg([k]), e, orc.dense_cfg([n - k + 1]), fast=True)
+        assert_bits(dx.getData(), want, f"conv1d dx {n} {k}")
     say("conv1d on a strided view stays general", dt)
     big = rng.uniform(-1, 1, 20000).astype(T); w = rng.uniform(-1, 1, 9).astype(T)
     view = on(device, big)[::2]
