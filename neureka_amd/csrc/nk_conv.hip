@@ -884,11 +884,47 @@ __global__ __launch_bounds__(256) void conv1d_grad_long(int N, int K, const T* _
     }
 }
 
+// ... and by the taps: dk[k] = sum_e x[k + e] * err[e].  Few outputs with long sums: a block takes 1024 entries of the
+// error, stages them and the inputs they meet in LDS, thread t adds the partial sums of the taps t, t + 256, ...;
+// conv_partial_reduce_wide adds the blocks' partial sums.  The terms are the reference's, their order is not
+// (norm-wise 1e-5 / 1e-12, like the other split sums).
+constexpr int CONV1D_SEG = 1024;
+template <typename T>
+__global__ __launch_bounds__(256) void conv1d_grad_taps(int N, int K, const T* __restrict__ x, const T* __restrict__ err, T* __restrict__ partial) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv1d_lds[];
+    T* xt = (T*)conv1d_lds;                                       // CONV1D_SEG + K - 1 inputs
+    T* et = xt + CONV1D_SEG + K - 1;                              // CONV1D_SEG error entries
+    const int n_err = N - K + 1;
+    const int e0 = blockIdx.x * CONV1D_SEG;
+    const int count = n_err - e0 < CONV1D_SEG ? n_err - e0 : CONV1D_SEG;
+    for (int s = threadIdx.x; s < CONV1D_SEG + K - 1; s += 256) xt[s] = e0 + s < N ? x[e0 + s] : T(0);
+    for (int s = threadIdx.x; s < CONV1D_SEG; s += 256) et[s] = s < count ? err[e0 + s] : T(0);
+    __syncthreads();
+    for (int k = threadIdx.x; k < K; k += 256) {
+        T acc = T(0);
+        for (int e = 0; e < count; e++) acc = acc + xt[k + e] * et[e];
+        partial[(int64_t)blockIdx.x * K + k] = acc;
+    }
+}
+
 template <typename T>
 static bool conv1d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& c0, const T* s1, const Cfg& c1, const T* s2, const Cfg& c2) {
     if (rank != 1 || !dense_rm(c0, 1) || !dense_rm(c1, 1) || !dense_rm(c2, 1)) return false;
     if (d >= 0) {
         // drain = the long operand, src1 = the taps, src2 = the error [N - K + 1]
+        if (c0.shape[0] < c1.shape[0]) {
+            // drain = the taps [K], src1 = the long operand [N], src2 = the error [N - K + 1]
+            const int K = c0.shape[0], N = c1.shape[0], n_err = N - K + 1;
+            if (K < 2 || K > 4096 || c2.shape[0] != n_err || n_err < 4096) return false;
+            const int parts = (n_err + CONV1D_SEG - 1) / CONV1D_SEG;
+            void* ws = nullptr;
+            if (workspace(dev, (uint64_t)parts * K * sizeof(T), &ws)) return false;
+            const size_t lds = (size_t)(2 * CONV1D_SEG + K - 1) * sizeof(T);
+            hipLaunchKernelGGL(conv1d_grad_taps<T>, dim3(parts), dim3(256), lds, dev->stream, N, K, s1, s2, (T*)ws);
+            hipLaunchKernelGGL(conv_partial_reduce_wide<T>, dim3((K + 3) / 4), dim3(256), 0, dev->stream, parts, K, (const T*)ws, out);
+            set_path("simple1d_grad_taps");
+            return true;
+        }
         const int N = c0.shape[0], K = c1.shape[0];
         constexpr int R = 4;
         if (K < 2 || K > 4096 || N <= K || c2.shape[0] != N - K + 1 || N < 4096) return false;

@@ -1074,6 +1074,22 @@ def test_conv1d_long_vectors_bit_exact(device, orc, dt):
         with np.errstate(all="ignore"):
             want = orc.deconvolve(np.zeros(n, dtype=T), orc.dense_cfg([n]), w, orc.dense_cfg([k]), e, orc.dense_cfg([n - k + 1]), fast=True)
         assert_bits(dx.getData(), want, f"conv1d dx {n} {k}")
+    tol = 1e-5 if dt == "f32" else 1e-12
+    for n, k in ((5000, 2), (70001, 64), (8200, 4096), (100000, 333)):
+        for integer in (True, False):
+            say("conv1d gradient by the taps", n, k, dt, "integer" if integer else "uniform")
+            x = (rng.integers(-3, 4, n) if integer else rng.uniform(-1, 1, n)).astype(T)
+            e = (rng.integers(-3, 4, n - k + 1) if integer else rng.uniform(-1, 1, n - k + 1)).astype(T)
+            dk = Tensor._on_device(device, T, [k])
+            device.launch_convolution(0, dk, on(device, x), on(device, e))
+            assert _lib.last_path() == "simple1d_grad_taps", _lib.last_path()
+            want = orc.deconvolve(np.zeros(k, dtype=T), orc.dense_cfg([k]), x, orc.dense_cfg([n]), e, orc.dense_cfg([n - k + 1]), fast=True)
+            if integer:
+                assert_bits(dk.getData(), want, f"conv1d dk {n} {k}")
+            else:       # the same terms in another order: bounded by the sum of their magnitudes
+                mag = orc.deconvolve(np.zeros(k), orc.dense_cfg([k]), np.abs(x).astype(np.float64), orc.dense_cfg([n]),
+                                     np.abs(e).astype(np.float64), orc.dense_cfg([n - k + 1]), fast=True)
+                assert (np.abs(dk.getData().astype(np.float64) - want) <= tol * mag + 1e-30).all()
     say("conv1d on a strided view stays general", dt)
     big = rng.uniform(-1, 1, 20000).astype(T); w = rng.uniform(-1, 1, 9).astype(T)
     view = on(device, big)[::2]
