@@ -250,6 +250,8 @@ __global__ __launch_bounds__(256) void conv_partial_reduce_wide(int parts, int n
 
 constexpr int CX = 4;                       // columns per lane
 typedef float f32x4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef double f64x2u __attribute__((ext_vector_type(2), aligned(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 // one fused multiply-add in the operand's own precision (the bare builtin is the double one)
 __device__ __forceinline__ float fused_mad(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
@@ -259,7 +261,7 @@ __device__ __forceinline__ double fused_mad(double a, double b, double c) { retu
 // offset for the row and one 32-bit per-lane byte offset -- no 64-bit vector arithmetic per access.  The
 // extent must stay below 2^32 bytes (checked on the host).
 typedef __amdgpu_buffer_rsrc_t BufRsrc;
-__device__ __forceinline__ BufRsrc buffer_of(const float* base, unsigned bytes) {
+__device__ __forceinline__ BufRsrc buffer_of(const void* base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, bytes, 0x00020000);      // raw buffer, 32-bit data format
 }
 __device__ __forceinline__ float buffer_load(BufRsrc r, unsigned lane_off, unsigned row_off) {
@@ -274,36 +276,77 @@ __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? l
 // Rows are addressed through one buffer descriptor per row (base = first element of the row, extent = the row):
 // the hardware range check then returns 0 for every dword left or right of the row (negative lane offsets wrap to
 // huge unsigned ones) and, with an extent of 0, for a whole row that does not exist.  No clamp, no mask.
-__device__ __forceinline__ BufRsrc row_of(const float* base, int64_t row, int width, bool exists) {
-    return buffer_of(base + (exists ? row * width : 0), exists ? (unsigned)width * 4u : 0u);
+template <typename T>
+__device__ __forceinline__ BufRsrc row_of(const T* base, int64_t row, int width, bool exists) {
+    return buffer_of(base + (exists ? row * width : 0), exists ? (unsigned)width * (unsigned)sizeof(T) : 0u);
+}
+
+// the CX columns col .. col+CX-1 of a row (col is a multiple of CX and may lie left or right of the row): one
+// 16-byte load in f32, two in f64
+__device__ __forceinline__ void load_cols(BufRsrc row, int col, float* dst) {
+    const f32x4u q = buffer_load4(row, (unsigned)col * 4u, 0);
+#pragma unroll
+    for (int e = 0; e < CX; e++) dst[e] = q[e];
+}
+__device__ __forceinline__ void load_cols(BufRsrc row, int col, double* dst) {
+    const unsigned off = (unsigned)col * 8u;
+    const f64x2u lo = __builtin_bit_cast(f64x2u, __builtin_amdgcn_raw_buffer_load_b128(row, off, 0, 0));
+    const f64x2u hi = __builtin_bit_cast(f64x2u, __builtin_amdgcn_raw_buffer_load_b128(row, off + 16u, 0, 0));
+    dst[0] = lo[0]; dst[1] = lo[1]; dst[2] = hi[0]; dst[3] = hi[1];
+}
+// CX adjacent results that nothing reads again soon
+__device__ __forceinline__ void store_cols(float* dst, const float* v) {
+    f32x4u o; o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+    __builtin_nontemporal_store(o, (f32x4u*)dst);
+}
+__device__ __forceinline__ void store_cols(double* dst, const double* v) {
+    f64x2u lo, hi; lo[0] = v[0]; lo[1] = v[1]; hi[0] = v[2]; hi[1] = v[3];
+    __builtin_nontemporal_store(lo, (f64x2u*)dst);
+    __builtin_nontemporal_store(hi, (f64x2u*)dst + 1);
 }
 
 // A lane holds CX adjacent columns; the KW - 1 further columns its window needs are the first (forward) or last
 // (gradients) registers of its neighbours.  They arrive through wavefront shifts of the registers instead of
-// through more loads: one 16-byte load per lane and row is all the memory traffic a window costs.  Only the
+// through more loads: one load of CX columns per lane and row is all the memory traffic a window costs.  Only the
 // lane at the end (start) of the wavefront, which has no neighbour, loads its extra columns itself; the shift
-// leaves that lane's registers as they are.
+// leaves that lane's registers as they are.  A double moves as its two halves.
 __device__ __forceinline__ float from_next_lane(float keep, float v) {     // lane i <- lane i + 1, lane 63 keeps `keep`
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, v), 0x130, 0xf, 0xf, false));
 }
 __device__ __forceinline__ float from_prev_lane(float keep, float v) {     // lane i <- lane i - 1, lane 0 keeps `keep`
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, v), 0x138, 0xf, 0xf, false));
 }
+__device__ __forceinline__ double from_next_lane(double keep, double v) {
+    const i32x2 k = __builtin_bit_cast(i32x2, keep), s = __builtin_bit_cast(i32x2, v);
+    i32x2 r;
+    r[0] = __builtin_amdgcn_update_dpp(k[0], s[0], 0x130, 0xf, 0xf, false);
+    r[1] = __builtin_amdgcn_update_dpp(k[1], s[1], 0x130, 0xf, 0xf, false);
+    return __builtin_bit_cast(double, r);
+}
+__device__ __forceinline__ double from_prev_lane(double keep, double v) {
+    const i32x2 k = __builtin_bit_cast(i32x2, keep), s = __builtin_bit_cast(i32x2, v);
+    i32x2 r;
+    r[0] = __builtin_amdgcn_update_dpp(k[0], s[0], 0x138, 0xf, 0xf, false);
+    r[1] = __builtin_amdgcn_update_dpp(k[1], s[1], 0x138, 0xf, 0xf, false);
+    return __builtin_bit_cast(double, r);
+}
 constexpr int WAVE_COLS = 64 * CX;          // columns per wavefront
 
 // window[0 .. CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[CX .. CX+EXTRA-1] with the
 // columns to the right of them
-template <int EXTRA>
-__device__ __forceinline__ void extend_right(float (&window)[CX + EXTRA], BufRsrc row, unsigned xoff, int lane) {
-    static_assert(EXTRA <= 2 * CX, "at most two further 16-byte pieces");
+template <int EXTRA, typename T>
+__device__ __forceinline__ void extend_right(T (&window)[CX + EXTRA], BufRsrc row, int x, int lane) {
+    static_assert(EXTRA <= 2 * CX, "at most two further pieces of CX columns");
 #pragma unroll
-    for (int e = CX; e < CX + EXTRA; e++) window[e] = 0.0f;
+    for (int e = CX; e < CX + EXTRA; e++) window[e] = T(0);
     if (lane == 63) {
-        const f32x4u a = buffer_load4(row, xoff + 16u, 0);
+        T a[CX];
+        load_cols(row, x + CX, a);
 #pragma unroll
         for (int e = 0; e < CX && e < EXTRA; e++) window[CX + e] = a[e];
         if (EXTRA > CX) {
-            const f32x4u b = buffer_load4(row, xoff + 32u, 0);
+            T b[CX];
+            load_cols(row, x + 2 * CX, b);
 #pragma unroll
             for (int e = CX; e < EXTRA; e++) window[CX + e] = b[e - CX];
         }
@@ -313,18 +356,20 @@ __device__ __forceinline__ void extend_right(float (&window)[CX + EXTRA], BufRsr
 }
 
 // window[EXTRA .. EXTRA+CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[0 .. EXTRA-1] with
-// the columns x-EXTRA .. x-1 to the left of them (lane offsets below the row start read as zero)
-template <int EXTRA>
-__device__ __forceinline__ void extend_left(float (&window)[CX + EXTRA], BufRsrc row, unsigned xoff, int lane) {
-    static_assert(EXTRA <= 2 * CX, "at most two further 16-byte pieces");
+// the columns x-EXTRA .. x-1 to the left of them (columns left of the row start read as zero)
+template <int EXTRA, typename T>
+__device__ __forceinline__ void extend_left(T (&window)[CX + EXTRA], BufRsrc row, int x, int lane) {
+    static_assert(EXTRA <= 2 * CX, "at most two further pieces of CX columns");
 #pragma unroll
-    for (int i = 0; i < EXTRA; i++) window[i] = 0.0f;
+    for (int i = 0; i < EXTRA; i++) window[i] = T(0);
     if (lane == 0) {
-        const f32x4u a = buffer_load4(row, xoff - 16u, 0);                 // columns x-4 .. x-1
+        T a[CX];
+        load_cols(row, x - CX, a);                                         // columns x-4 .. x-1
 #pragma unroll
         for (int e = 0; e < CX; e++) if (EXTRA - CX + e >= 0) window[EXTRA - CX + e] = a[e];
         if (EXTRA > CX) {
-            const f32x4u b = buffer_load4(row, xoff - 32u, 0);             // columns x-8 .. x-5
+            T b[CX];
+            load_cols(row, x - 2 * CX, b);                                 // columns x-8 .. x-5
 #pragma unroll
             for (int e = 0; e < CX; e++) if (EXTRA - 2 * CX + e >= 0) window[EXTRA - 2 * CX + e] = b[e];
         }
@@ -343,7 +388,6 @@ __global__ __launch_bounds__(NW * 64) void conv_chan_fwd(ChanArgs g, const T* __
     __shared__ T red[NW][R][64 * CX];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int x = blockIdx.x * COLS + lane * CX;                 // first of the lane's CX columns
-    const unsigned xoff = (unsigned)x * 4u;
     const int y0 = blockIdx.y * R;
     const int c0 = blockIdx.z * g.cg;
     int c1 = c0 + g.cg; if (c1 > g.C) c1 = g.C;
@@ -362,14 +406,11 @@ __global__ __launch_bounds__(NW * 64) void conv_chan_fwd(ChanArgs g, const T* __
         const T* plane = in + (int64_t)c * g.H * g.W;
         T v[R + KH - 1][CX + KW - 1];
 #pragma unroll
-        for (int yy = 0; yy < R + KH - 1; yy++) {                // all loads of the window first: one wait for the lot
-            const f32x4u head = buffer_load4(row_of(plane, y0 + yy, g.W, y0 + yy < g.H), xoff, 0);
-#pragma unroll
-            for (int e = 0; e < CX; e++) v[yy][e] = head[e];
-        }
+        for (int yy = 0; yy < R + KH - 1; yy++)                  // all loads of the window first: one wait for the lot
+            load_cols(row_of(plane, y0 + yy, g.W, y0 + yy < g.H), x, v[yy]);
 #pragma unroll
         for (int yy = 0; yy < R + KH - 1; yy++)
-            extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, g.W, y0 + yy < g.H), xoff, lane);
+            extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, g.W, y0 + yy < g.H), x, lane);
 #pragma unroll
         for (int yy = 0; yy < R + KH - 1; yy++)
 #pragma unroll
@@ -417,14 +458,12 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
 #pragma unroll
     for (int rr = 0; rr < R + KH - 1; rr++) {
         const int ey = y0 - (KH - 1) + rr;
-        const f32x4u own = buffer_load4(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), (unsigned)x * 4u, 0);
-#pragma unroll
-        for (int j = 0; j < CX; j++) E[rr][KW - 1 + j] = own[j];
+        load_cols(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), x, &E[rr][KW - 1]);
     }
 #pragma unroll
     for (int rr = 0; rr < R + KH - 1; rr++) {
         const int ey = y0 - (KH - 1) + rr;
-        extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), (unsigned)x * 4u, lane);
+        extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), x, lane);
     }
     const bool stores = x < g.W;
     const bool vec_ok = x + CX <= g.W;
@@ -450,8 +489,7 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
             if (stores && y0 + r < g.H) {
                 T* dst = plane + (int64_t)(y0 + r) * g.W + x;
                 if (vec_ok) {
-                    f32x4u o; o[0] = acc[0]; o[1] = acc[1]; o[2] = acc[2]; o[3] = acc[3];
-                    __builtin_nontemporal_store(o, (f32x4u*)dst);
+                    store_cols(dst, acc);
                 } else {
 #pragma unroll
                     for (int j = 0; j < CX; j++) if (x + j < g.W) dst[j] = acc[j];
@@ -473,7 +511,6 @@ __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstri
     const int strip = blockIdx.y * 4 + wave;
     if (strip >= nstrips) return;                                 // whole wavefronts leave together
     const int xx = blockIdx.x * WAVE_COLS + lane * CX;
-    const unsigned eoff = (unsigned)xx * 4u, voff = eoff;
     const int yy0 = strip * S;
     int yy1 = yy0 + S; if (yy1 > g.H) yy1 = g.H;
     const int c = blockIdx.z;
@@ -487,22 +524,16 @@ __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstri
         T E[R + KH - 1][CX + KW - 1];                             // E[rr][i] = err[y - (KH-1) + rr][xx - (KW-1) + i], zero outside err
         T V[R][CX];                                               // V[r] = input row y + r, zero past the strip
 #pragma unroll
-        for (int r = 0; r < R; r++) {
-            const f32x4u q = buffer_load4(row_of(plane, y + r, g.W, y + r < yy1), voff, 0);
+        for (int r = 0; r < R; r++) load_cols(row_of(plane, y + r, g.W, y + r < yy1), xx, V[r]);
 #pragma unroll
-            for (int j = 0; j < CX; j++) V[r][j] = q[j];
+        for (int rr = 0; rr < R + KH - 1; rr++) {
+            const int ey = y - (KH - 1) + rr;
+            load_cols(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, &E[rr][KW - 1]);
         }
 #pragma unroll
         for (int rr = 0; rr < R + KH - 1; rr++) {
             const int ey = y - (KH - 1) + rr;
-            const f32x4u own = buffer_load4(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), eoff, 0);
-#pragma unroll
-            for (int j = 0; j < CX; j++) E[rr][KW - 1 + j] = own[j];
-        }
-#pragma unroll
-        for (int rr = 0; rr < R + KH - 1; rr++) {
-            const int ey = y - (KH - 1) + rr;
-            extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), eoff, lane);
+            extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, lane);
         }
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -566,7 +597,6 @@ __global__ __launch_bounds__(256) void conv2d_window(int H, int W, const float* 
     const int OH = H - KH + 1, OW = W - KW + 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int x = blockIdx.x * WAVE_COLS + lane * CX;
-    const unsigned xoff = (unsigned)x * 4u;
     const int y0 = (blockIdx.y * 4 + wave) * R;
     if (y0 >= OH) return;                                        // whole wavefronts leave together
     const float* plane = img + (int64_t)blockIdx.z * H * W;
@@ -577,14 +607,10 @@ __global__ __launch_bounds__(256) void conv2d_window(int H, int W, const float* 
         for (int kx = 0; kx < KW; kx++) wt[ky][kx] = taps[ky * KW + kx];
     float v[R + KH - 1][CX + KW - 1];
 #pragma unroll
-    for (int yy = 0; yy < R + KH - 1; yy++) {
-        const f32x4u head = buffer_load4(row_of(plane, y0 + yy, W, y0 + yy < H), xoff, 0);
-#pragma unroll
-        for (int e = 0; e < CX; e++) v[yy][e] = head[e];
-    }
+    for (int yy = 0; yy < R + KH - 1; yy++) load_cols(row_of(plane, y0 + yy, W, y0 + yy < H), x, v[yy]);
 #pragma unroll
     for (int yy = 0; yy < R + KH - 1; yy++)
-        extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, W, y0 + yy < H), xoff, lane);
+        extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, W, y0 + yy < H), x, lane);
     float acc[R][CX];
 #pragma unroll
     for (int r = 0; r < R; r++)
@@ -638,10 +664,12 @@ static bool for_taps(int KH, int KW, F&& f) {
     }
 }
 
-// the three channel kernels for dense f32 operands; returns NK_OK with *taken = true when one was launched
-static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, const float* s1, const Cfg& c1,
-                              const float* s2, const Cfg& c2, bool* taken, bool one_plane = false) {
-    using T = float;
+// the three channel kernels for dense f32 or f64 operands; returns NK_OK with *taken = true when one was launched.
+// A double takes two registers, so the f64 instantiations work on half as many rows per wavefront.
+template <typename T>
+static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T* s1, const Cfg& c1,
+                              const T* s2, const Cfg& c2, bool* taken, bool one_plane = false) {
+    constexpr bool F32 = sizeof(T) == 4;
     *taken = false;
     static const long waves_per_cu = [] { const char* v = getenv("NK_CONV_WAVES_PER_CU"); return v && *v ? atol(v) : 8L; }();
     const int64_t want_waves = (int64_t)dev->props.multiProcessorCount * waves_per_cu;
@@ -669,17 +697,21 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
             int tall_r = 0;
             if (g.C >= 16)
                 for (int r : {8, 4})
-                    if ((int64_t)g.col_blocks * ((g.OH + r - 1) / r) >= cus) { tall_r = r; break; }
+                    if ((F32 || r == 4) && (int64_t)g.col_blocks * ((g.OH + r - 1) / r) >= cus) { tall_r = r; break; }
             if (tall_r) {
                 g.cg = g.C;
                 dim3 grid(g.col_blocks, (g.OH + tall_r - 1) / tall_r, 1);
-                if (tall_r == 8) hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 8, 16>), grid, dim3(1024), 0, dev->stream, g, bigp, smallp, out);
-                else             hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 4, 16>), grid, dim3(1024), 0, dev->stream, g, bigp, smallp, out);
+                if constexpr (F32) {
+                    if (tall_r == 8) hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 8, 16>), grid, dim3(1024), 0, dev->stream, g, bigp, smallp, out);
+                    else             hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 4, 16>), grid, dim3(1024), 0, dev->stream, g, bigp, smallp, out);
+                } else {            // eight wavefronts: 256 registers each for the window, 64 KiB of LDS for their sums
+                    hipLaunchKernelGGL((conv_chan_fwd<T, KK, KK, 4, 8>), grid, dim3(512), 0, dev->stream, g, bigp, smallp, out);
+                }
                 return;
             }
             // Small planes: parallelism has to come from the channels.  Blocks of four wavefronts take groups of
             // channels (multiples of 4), a second pass adds the partial planes in a fixed order.
-            constexpr int R = 8;
+            constexpr int R = F32 ? 8 : 4;
             const int strips = (g.OH + R - 1) / R;
             g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips * 4, want_waves);
             g.cg = (g.cg + 3) / 4 * 4;
@@ -728,7 +760,7 @@ static int conv_channel_paths(Device* dev, int d, float* out, const Cfg& c0, con
             ChanArgs g{};
             g.C = c0.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2]; g.OH = OH; g.OW = OW;
             g.cg = 1;
-            constexpr int R = 8;
+            constexpr int R = F32 ? 8 : 4;
             int rc = NK_OK;
             const bool ok = for_taps(c0.shape[1], c0.shape[2], [&](auto K) {
                 constexpr int KK = decltype(K)::value;
@@ -957,17 +989,17 @@ static int conv_typed(Device* dev, int d, int rank, nk_buf drn, const Cfg& c0, n
         NK_HIP(hipGetLastError());
         return NK_OK;
     }
-    if constexpr (sizeof(T) == 4) {
+    if constexpr (std::is_floating_point<T>::value) {
         if (rank == 3 && dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank)) {
             bool taken = false;
-            if (int e = conv_channel_paths(dev, d, out, c0, s1, c1, s2, c2, &taken)) return e;
+            if (int e = conv_channel_paths<T>(dev, d, out, c0, s1, c1, s2, c2, &taken)) return e;
             if (taken) return NK_OK;
         }
         // both gradients of a 2-D image convolution [H,W] x [kh,kw] are the one-channel case of the same kernels
         if (rank == 2 && d >= 0 && dense_rm(c0, rank) && dense_rm(c1, rank) && dense_rm(c2, rank)) {
             auto plane = [](const Cfg& c) { Cfg p{}; p.shape[0] = 1; p.shape[1] = c.shape[0]; p.shape[2] = c.shape[1]; return p; };
             bool taken = false;
-            if (int e = conv_channel_paths(dev, d, out, plane(c0), s1, plane(c1), s2, plane(c2), &taken, true)) return e;
+            if (int e = conv_channel_paths<T>(dev, d, out, plane(c0), s1, plane(c1), s2, plane(c2), &taken, true)) return e;
             if (taken) return NK_OK;
         }
     }

@@ -856,44 +856,48 @@ def _abs_bound(orc, xs, ks, x, k, dt):
                                    ([3, 130, 200], [3, 7, 7]), ([9, 17, 300], [9, 2, 2]), ([2, 12, 12], [2, 4, 4]),
                                    ([3, 10, 71], [3, 3, 3]), ([5, 9, 302], [5, 2, 2]), ([70, 30, 261], [70, 5, 5]),
                                    ([16, 520, 1030], [16, 3, 3]), ([16, 300, 1100], [16, 7, 7])])
-def test_channel_convolution_fast_paths(device, orc, shape):
-    """[C,H,W] x [C,kh,kw] forward and both gradients on the register-window kernels: re-ordered f32 sums, compared
-    norm-wise: |delta| <= 1e-5 * sum|a||b| per output.  Covers ragged widths, several column blocks per row, taps
-    that reach two lanes to the side, and planes large enough for the 16-wavefront forward blocks."""
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_channel_convolution_fast_paths(device, orc, shape, dt):
+    """[C,H,W] x [C,kh,kw] forward and both gradients on the register-window kernels: re-ordered sums, compared
+    norm-wise: |delta| <= tol * sum|a||b| per output (tol 1e-5 in f32, 1e-12 in f64).  Covers ragged widths, several
+    column blocks per row, taps that reach two lanes to the side, and planes large enough for the forward blocks
+    that reduce all channels themselves."""
     xs, ks = shape
+    T = F[dt]
+    tol = RTOL[np.dtype(T)]
     ys = [1, xs[1] - ks[1] + 1, xs[2] - ks[2] + 1]
     rng = np.random.default_rng(43)
-    x = (rng.standard_normal(xs) * 0.1).astype(np.float32); k = (rng.standard_normal(ks) * 0.1).astype(np.float32)
-    e = rng.standard_normal(ys).astype(np.float32)
+    x = (rng.standard_normal(xs) * 0.1).astype(T); k = (rng.standard_normal(ks) * 0.1).astype(T)
+    e = rng.standard_normal(ys).astype(T)
     tx, tk, te = on(device, x), on(device, k), on(device, e)
     square = ks[1] == ks[2]          # the register-window kernels exist for square taps of extent 2, 3, 4, 5, 7
     # other tap shapes take the general kernels: one thread per element, or (sums of 128 terms and more into few elements) split sums
     fwd, dxp, dkp = ("chan_fwd", "chan_dx", "chan_dk") if square else ("literal_fwd", "literal_bwd", "split_bwd")
-    say("chan_fwd", xs, ks)
-    out = Tensor._on_device(device, np.float32, ys)
+    say("chan_fwd", xs, ks, dt)
+    out = Tensor._on_device(device, T, ys)
     device.launch_convolution(-1, out, tx, tk)
     assert _lib.last_path() == fwd
-    want = orc.convolve(np.zeros(out.size, dtype=np.float32), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
-    bound = RTOL[np.dtype(np.float32)] * _abs_bound(orc, xs, ks, x, k, np.float32) + 1e-30
+    want = orc.convolve(np.zeros(out.size, dtype=T), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
+    bound = tol * _abs_bound(orc, xs, ks, x, k, T) + 1e-30
     assert (np.abs(out.getData().astype(np.float64) - want) <= bound).all(), "chan_fwd"
-    out2 = Tensor._on_device(device, np.float32, ys)
+    out2 = Tensor._on_device(device, T, ys)
     device.launch_convolution(-1, out2, tk, tx)                       # kernel first
     assert _lib.last_path() == fwd
     assert_bits(out2.getData(), out.getData(), "operand order")
-    say("chan_dx", xs, ks)
-    dx = Tensor._on_device(device, np.float32, xs)
+    say("chan_dx", xs, ks, dt)
+    dx = Tensor._on_device(device, T, xs)
     device.launch_convolution(0, dx, tk, te)
     assert _lib.last_path() == dxp
-    want = orc.deconvolve(np.zeros(dx.size, dtype=np.float32), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks), e.reshape(-1), orc.dense_cfg(ys), fast=True)
+    want = orc.deconvolve(np.zeros(dx.size, dtype=T), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks), e.reshape(-1), orc.dense_cfg(ys), fast=True)
     babs = orc.deconvolve(np.zeros(dx.size), orc.dense_cfg(xs), np.abs(k).astype(np.float64).reshape(-1), orc.dense_cfg(ks), np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
-    assert (np.abs(dx.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dx"
-    say("chan_dk", xs, ks)
-    dk = Tensor._on_device(device, np.float32, ks)
+    assert (np.abs(dx.getData().astype(np.float64) - want) <= tol * babs + 1e-30).all(), "chan_dx"
+    say("chan_dk", xs, ks, dt)
+    dk = Tensor._on_device(device, T, ks)
     device.launch_convolution(0, dk, tx, te)
     assert _lib.last_path() == dkp
-    want = orc.deconvolve(np.zeros(dk.size, dtype=np.float32), orc.dense_cfg(ks), x.reshape(-1), orc.dense_cfg(xs), e.reshape(-1), orc.dense_cfg(ys), fast=True)
+    want = orc.deconvolve(np.zeros(dk.size, dtype=T), orc.dense_cfg(ks), x.reshape(-1), orc.dense_cfg(xs), e.reshape(-1), orc.dense_cfg(ys), fast=True)
     babs = orc.deconvolve(np.zeros(dk.size), orc.dense_cfg(ks), np.abs(x).astype(np.float64).reshape(-1), orc.dense_cfg(xs), np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
-    assert (np.abs(dk.getData().astype(np.float64) - want) <= 1e-5 * babs + 1e-30).all(), "chan_dk"
+    assert (np.abs(dk.getData().astype(np.float64) - want) <= tol * babs + 1e-30).all(), "chan_dk"
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
@@ -935,10 +939,10 @@ def test_convolution_split_sums(device, orc, shape, dt):
                 babs = orc.deconvolve(np.zeros(drn.size), orc.dense_cfg(tgt_shape), np.abs(other_arr).astype(np.float64).reshape(-1), orc.dense_cfg(other_shape),
                                       np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
                 assert (np.abs(drn.getData().astype(np.float64) - want) <= tol * babs + 1e-30).all(), name
-    if dt == "f32" and ks == [48, 5, 5]:
-        assert seen == {"chan_fwd", "chan_dx", "chan_dk"}, seen          # the register-window kernels take dense f32 square taps
-    elif dt == "f32" and ks == [5, 5]:
-        assert seen == {"simple2d_window", "chan_dx", "chan_dk"}, seen   # ... and a 2-D image as their one-channel case
+    if ks == [48, 5, 5]:
+        assert seen == {"chan_fwd", "chan_dx", "chan_dk"}, seen          # the register-window kernels take dense square taps
+    elif ks == [5, 5]:                                                   # ... and a 2-D image as their one-channel case
+        assert seen == {"simple2d_window" if dt == "f32" else "simple2d", "chan_dx", "chan_dk"}, seen
     else:
         assert seen & {"split_fwd", "split_bwd"}, seen
     if len(xs) == 2:
@@ -1022,7 +1026,7 @@ def test_random_convolutions_through_every_plan(device, orc, dt):
             want = orc.deconvolve(np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt_shape), other_data, other_cfg, de_, ce, fast=True)
             assert_bits(drn.getData(), want, f"case {case} {name} {xs} x {ks} {views} on {_lib.last_path()}")
     say("plans seen", sorted(seen))
-    want_plans = {"literal_fwd", "literal_bwd", "simple2d"} | ({"chan_fwd", "chan_dx", "chan_dk", "simple2d_window"} if dt == "f32" else set())
+    want_plans = {"literal_fwd", "literal_bwd", "simple2d", "chan_fwd", "chan_dx", "chan_dk"} | ({"simple2d_window"} if dt == "f32" else set())
     assert want_plans <= seen, (sorted(want_plans - seen), sorted(seen))
 
 
