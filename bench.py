@@ -335,7 +335,7 @@ def main():
         flops("conv_c5_grad_input", 203212800, 17037632, dev.prepared_launch("convolution", 0, dx5, k5, e5))
         flops("conv_c5_grad_kernel", 203212800, 17037632, dev.prepared_launch("convolution", 0, dk5, x5, e5))
         for t in (x5, k5, y5, e5, dx5, dk5): dev.free(t)
-        # the same shapes in f64 take the general kernels (any rank, layout and view)
+        # the same shapes in f64: the channel kernels instantiated for double
         f64 = np.float64
         x5 = Tensor.of(f64, (64, 256, 256), rng.standard_normal(64 * 256 * 256) * 0.1).to(dev)
         k5 = Tensor.of(f64, (64, 5, 5), rng.standard_normal(1600) * 0.1).to(dev)

@@ -332,6 +332,17 @@ __device__ __forceinline__ double from_prev_lane(double keep, double v) {
 }
 constexpr int WAVE_COLS = 64 * CX;          // columns per wavefront
 
+// CX adjacent results through ordinary 16-byte stores
+__device__ __forceinline__ void write_cols(float* dst, const float* v) {
+    f32x4u o; o[0] = v[0]; o[1] = v[1]; o[2] = v[2]; o[3] = v[3];
+    *(f32x4u*)dst = o;
+}
+__device__ __forceinline__ void write_cols(double* dst, const double* v) {
+    f64x2u lo, hi; lo[0] = v[0]; lo[1] = v[1]; hi[0] = v[2]; hi[1] = v[3];
+    *(f64x2u*)dst = lo;
+    *((f64x2u*)dst + 1) = hi;
+}
+
 // window[0 .. CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[CX .. CX+EXTRA-1] with the
 // columns to the right of them
 template <int EXTRA, typename T>
@@ -586,36 +597,36 @@ static int channels_per_group(int C, int64_t waves_per_group_set, int64_t want) 
     return (int)((C + groups - 1) / groups);
 }
 
-// 2-D valid cross-correlation of large images, f32, square taps: the register-window scheme of the channel kernels
+// 2-D valid cross-correlation of large images, square taps: the register-window scheme of the channel kernels
 // for one plane.  A wavefront owns R output rows x 256 columns, loads the R + KH - 1 window rows once and reuses
 // them for every tap.  For an output element the contributions arrive with ky ascending and kx ascending inside,
 // and every product is rounded before it is added (no fused multiply-add): the summation order of
 // SimpleCPUConvolution, so the result is bit-identical to conv2d_direct's.
-template <int KH, int KW, int R>
-__global__ __launch_bounds__(256) void conv2d_window(int H, int W, const float* __restrict__ img, const float* __restrict__ taps,
-                                                     float* __restrict__ out) {
+template <typename T, int KH, int KW, int R>
+__global__ __launch_bounds__(256) void conv2d_window(int H, int W, const T* __restrict__ img, const T* __restrict__ taps,
+                                                     T* __restrict__ out) {
     const int OH = H - KH + 1, OW = W - KW + 1;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int x = blockIdx.x * WAVE_COLS + lane * CX;
     const int y0 = (blockIdx.y * 4 + wave) * R;
     if (y0 >= OH) return;                                        // whole wavefronts leave together
-    const float* plane = img + (int64_t)blockIdx.z * H * W;
-    float wt[KH][KW];
+    const T* plane = img + (int64_t)blockIdx.z * H * W;
+    T wt[KH][KW];
 #pragma unroll
     for (int ky = 0; ky < KH; ky++)
 #pragma unroll
         for (int kx = 0; kx < KW; kx++) wt[ky][kx] = taps[ky * KW + kx];
-    float v[R + KH - 1][CX + KW - 1];
+    T v[R + KH - 1][CX + KW - 1];
 #pragma unroll
     for (int yy = 0; yy < R + KH - 1; yy++) load_cols(row_of(plane, y0 + yy, W, y0 + yy < H), x, v[yy]);
 #pragma unroll
     for (int yy = 0; yy < R + KH - 1; yy++)
         extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, W, y0 + yy < H), x, lane);
-    float acc[R][CX];
+    T acc[R][CX];
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
-        for (int j = 0; j < CX; j++) acc[r][j] = 0.0f;
+        for (int j = 0; j < CX; j++) acc[r][j] = T(0);
 #pragma unroll
     for (int yy = 0; yy < R + KH - 1; yy++)
 #pragma unroll
@@ -626,22 +637,19 @@ __global__ __launch_bounds__(256) void conv2d_window(int H, int W, const float* 
                 for (int j = 0; j < CX; j++)
 #pragma unroll
                     for (int kx = 0; kx < KW; kx++) {
-                        const float prod = v[yy][j + kx] * wt[ky][kx];
+                        const T prod = v[yy][j + kx] * wt[ky][kx];
                         acc[r][j] = acc[r][j] + prod;
                     }
             }
         }
-    float* dst = out + (int64_t)blockIdx.z * OH * OW;
+    T* dst = out + (int64_t)blockIdx.z * OH * OW;
 #pragma unroll
     for (int r = 0; r < R; r++) {
         const int yo = y0 + r;
         if (yo < OH) {
-            float* p = dst + (int64_t)yo * OW + x;
+            T* p = dst + (int64_t)yo * OW + x;
             if (x + CX <= OW) {
-                f32x4u o4;
-#pragma unroll
-                for (int j = 0; j < CX; j++) o4[j] = acc[r][j];
-                *(f32x4u*)p = o4;
+                write_cols(p, acc[r]);
             } else {
 #pragma unroll
                 for (int j = 0; j < CX; j++) if (x + j < OW) p[j] = acc[r][j];
@@ -828,19 +836,19 @@ static bool conv2d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& 
     const int B = rank == 3 ? (int)img.shape[0] : 1;
     const int64_t n = (int64_t)B * (img.shape[o] - tap.shape[o] + 1) * (img.shape[o + 1] - tap.shape[o + 1] + 1);
     if (n >= ((int64_t)1 << 31)) return false;
-    if constexpr (sizeof(T) == 4) {
-        // large f32 images with square taps: the register-window kernel (same sums, same order)
+    {
+        // large images with square taps: the register-window kernel (same sums, same order); half the rows in f64
         const int H = (int)img.shape[o], W = (int)img.shape[o + 1];
         static const bool window_on = [] { const char* v = getenv("NK_CONV2D_WINDOW"); return !(v && v[0] == '0'); }();
-        if (window_on && n >= 65536 && (int64_t)H * W * 4 < ((int64_t)1 << 31) && B <= 65535) {
-            constexpr int R = 8;
+        if (window_on && n >= 65536 && (int64_t)H * W * (int64_t)sizeof(T) < ((int64_t)1 << 31) && B <= 65535) {
+            constexpr int R = sizeof(T) == 4 ? 8 : 4;
             const int OH = H - (int)tap.shape[o] + 1, OW = W - (int)tap.shape[o + 1] + 1;
             const dim3 grid((unsigned)((OW + WAVE_COLS - 1) / WAVE_COLS), (unsigned)(((OH + R - 1) / R + 3) / 4), (unsigned)B);
-            const float* ip = (const float*)(a_img ? s1 : s2);
-            const float* tp = (const float*)(a_img ? s2 : s1);
+            const T* ip = a_img ? s1 : s2;
+            const T* tp = a_img ? s2 : s1;
             if (grid.y <= 65535 && for_taps((int)tap.shape[o], (int)tap.shape[o + 1], [&](auto K) {
                     constexpr int KK = decltype(K)::value;
-                    hipLaunchKernelGGL((conv2d_window<KK, KK, R>), grid, dim3(256), 0, dev->stream, H, W, ip, tp, (float*)out);
+                    hipLaunchKernelGGL((conv2d_window<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, H, W, ip, tp, out);
                 })) {
                 set_path("simple2d_window");
                 return true;

@@ -818,7 +818,7 @@ def test_convolution_literal_kernels_bit_exact(device, orc, dt):
         want = orc.convolve(np.zeros(out.size, dtype=F[dt]), orc.dense_cfg(ys), x.reshape(-1), orc.dense_cfg(xs), k.reshape(-1), orc.dense_cfg(ks))
         if _lib.last_path().startswith("literal"):
             assert_bits(out.getData(), want, f"fwd {xs} {ks}")
-        elif _lib.last_path() == "simple2d":        # what the reference hands to SimpleCPUConvolution: its order, bit for bit
+        elif _lib.last_path() in ("simple2d", "simple2d_window"):        # what the reference hands to SimpleCPUConvolution: its order, bit for bit
             img, tap, ishape, tshape = (x, k, xs, ks) if xs[-1] >= ks[-1] else (k, x, ks, xs)
             assert len(xs) == 2 or tshape[0] == 1
             simple = orc.simple_conv2d(img.reshape(-1), tap.reshape(-1), ishape[-1], ishape[-2], tshape[-1], tshape[-2], batch=ishape[0] if len(xs) == 3 else 1)
@@ -942,7 +942,7 @@ def test_convolution_split_sums(device, orc, shape, dt):
     if ks == [48, 5, 5]:
         assert seen == {"chan_fwd", "chan_dx", "chan_dk"}, seen          # the register-window kernels take dense square taps
     elif ks == [5, 5]:                                                   # ... and a 2-D image as their one-channel case
-        assert seen == {"simple2d_window" if dt == "f32" else "simple2d", "chan_dx", "chan_dk"}, seen
+        assert seen == {"simple2d_window", "chan_dx", "chan_dk"}, seen
     else:
         assert seen & {"split_fwd", "split_bwd"}, seen
     if len(xs) == 2:
@@ -1026,18 +1026,19 @@ def test_random_convolutions_through_every_plan(device, orc, dt):
             want = orc.deconvolve(np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt_shape), other_data, other_cfg, de_, ce, fast=True)
             assert_bits(drn.getData(), want, f"case {case} {name} {xs} x {ks} {views} on {_lib.last_path()}")
     say("plans seen", sorted(seen))
-    want_plans = {"literal_fwd", "literal_bwd", "simple2d", "chan_fwd", "chan_dx", "chan_dk"} | ({"simple2d_window"} if dt == "f32" else set())
+    want_plans = {"literal_fwd", "literal_bwd", "simple2d", "chan_fwd", "chan_dx", "chan_dk", "simple2d_window"}
     assert want_plans <= seen, (sorted(want_plans - seen), sorted(seen))
 
 
 @pytest.mark.parametrize("shape", [([300, 523], [5, 5]), ([3, 200, 300], [1, 3, 3]), ([130, 700], [7, 7]), ([260, 257], [2, 2]), ([2, 190, 261], [1, 4, 4])])
-def test_conv2d_large_images_bit_exact(device, orc, shape):
-    """Large f32 images with square taps take the register-window kernel: the same products, rounded and added in
-    SimpleCPUConvolution's order (ky outer, kx inner) -- bit for bit."""
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_conv2d_large_images_bit_exact(device, orc, shape, dt):
+    """Large images with square taps take the register-window kernel: the same products, rounded and added in
+    SimpleCPUConvolution's order (ky outer, kx inner) -- bit for bit, in f32 and f64."""
     xs, ks = shape
     rng = np.random.default_rng(45)
-    x = rng.uniform(-1, 1, xs).astype(np.float32); k = rng.uniform(-1, 1, ks).astype(np.float32)
-    say("conv2d window", xs, ks)
+    x = rng.uniform(-1, 1, xs).astype(F[dt]); k = rng.uniform(-1, 1, ks).astype(F[dt])
+    say("conv2d window", xs, ks, dt)
     y = on(device, x).conv(on(device, k))
     assert _lib.last_path() == "simple2d_window", _lib.last_path()
     B = xs[0] if len(xs) == 3 else 1
