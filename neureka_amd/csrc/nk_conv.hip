@@ -217,6 +217,8 @@ struct ChanArgs {
     int C, H, W, OH, OW;
     int cg;              // channels per group (grid z)
     int col_blocks;      // 256-column blocks across the lane axis
+    int err_plane;       // gradients: elements between the error planes of two channels (0: one plane for all)
+    int tap_plane;       // gradients: elements between the taps of two channels (0: one set for all)
 };
 
 template <typename T>
@@ -464,6 +466,7 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
     if (y0 >= g.H) return;                                        // whole wavefronts leave together
     const int c0 = blockIdx.z * g.cg;
     int c1 = c0 + g.cg; if (c1 > g.C) c1 = g.C;
+    err += (int64_t)c0 * g.err_plane;                             // one error plane per channel: groups of one channel
     // E[rr][i] = err[y0 - (KH-1) + rr][x - (KW-1) + i], zero outside err
     T E[R + KH - 1][CX + KW - 1];
 #pragma unroll
@@ -479,7 +482,7 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
     const bool stores = x < g.W;
     const bool vec_ok = x + CX <= g.W;
     for (int c = c0; c < c1; c++) {
-        const T* wc = w + (int64_t)c * (KH * KW);
+        const T* wc = w + (int64_t)c * g.tap_plane;
         T wt[KH][KW];
 #pragma unroll
         for (int ky = 0; ky < KH; ky++)
@@ -531,6 +534,7 @@ __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstri
 #pragma unroll
         for (int kx = 0; kx < KW; kx++) acc[ky][kx] = T(0);
     const T* plane = in + (int64_t)c * g.H * g.W;
+    err += (int64_t)c * g.err_plane;
     for (int y = yy0; y < yy1; y += R) {
         T E[R + KH - 1][CX + KW - 1];                             // E[rr][i] = err[y - (KH-1) + rr][xx - (KW-1) + i], zero outside err
         T V[R][CX];                                               // V[r] = input row y + r, zero past the strip
@@ -739,10 +743,15 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
         *taken = true;
         return NK_OK;
     }
-    if (d >= 0 && c2.shape[0] == 1 && c0.shape[0] == c1.shape[0] && (c0.shape[0] > 1 || one_plane)) {
-        const int OH = c2.shape[1], OW = c2.shape[2];      // src2 = error [1,OH,OW]
+    // gradients, src2 = the error: one plane [1,OH,OW] shared by the channels of [C,H,W] x [C,k,k], or -- a batch of
+    // images under one set of taps, [B,H,W] x [1,k,k] -- one plane per image [B,OH,OW]
+    const bool shared_err = c2.shape[0] == 1 && c0.shape[0] == c1.shape[0] && (c0.shape[0] > 1 || one_plane);
+    const bool batch_dx = c2.shape[0] > 1 && c0.shape[0] == c2.shape[0] && c1.shape[0] == 1;
+    const bool batch_dk = c2.shape[0] > 1 && c1.shape[0] == c2.shape[0] && c0.shape[0] == 1;
+    if (d >= 0 && (shared_err || batch_dx || batch_dk)) {
+        const int OH = c2.shape[1], OW = c2.shape[2];
         // dx: the drain is the big operand, src1 the taps
-        if (c0.shape[1] == OH + c1.shape[1] - 1 && c0.shape[2] == OW + c1.shape[2] - 1 &&
+        if ((shared_err || batch_dx) && c0.shape[1] == OH + c1.shape[1] - 1 && c0.shape[2] == OW + c1.shape[2] - 1 &&
             (c0.shape[1] > c1.shape[1] || c1.shape[1] == 1) && (c0.shape[2] > c1.shape[2] || c1.shape[2] == 1)) {
             constexpr int R = 4;
             ChanArgs g{};
@@ -751,8 +760,11 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
             const bool ok = for_taps(c1.shape[1], c1.shape[2], [&](auto K) {
                 constexpr int KK = decltype(K)::value;
                 g.col_blocks = (g.W + WAVE_COLS - 1) / WAVE_COLS;
+                g.err_plane = batch_dx ? OH * OW : 0;
+                g.tap_plane = batch_dx ? 0 : KK * KK;
                 g.cg = channels_per_group(g.C, (int64_t)g.col_blocks * strips, want_waves);
                 if (g.cg < 2 && g.C >= 2) g.cg = 2;          // amortise the err window over at least two channels
+                if (batch_dx) g.cg = 1;                      // every image has its own err window
                 const int groups = (g.C + g.cg - 1) / g.cg;
                 dim3 grid(g.col_blocks, (strips + 3) / 4, groups);
                 hipLaunchKernelGGL((conv_chan_dx<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, s2, s1, out);
@@ -764,9 +776,10 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
             return NK_OK;
         }
         // dk: the drain is the taps, src1 the big operand
-        if (c1.shape[1] == OH + c0.shape[1] - 1 && c1.shape[2] == OW + c0.shape[2] - 1 && c0.shape[1] < c1.shape[1] && c0.shape[2] < c1.shape[2]) {
+        if ((shared_err || batch_dk) && c1.shape[1] == OH + c0.shape[1] - 1 && c1.shape[2] == OW + c0.shape[2] - 1 && c0.shape[1] < c1.shape[1] && c0.shape[2] < c1.shape[2]) {
             ChanArgs g{};
-            g.C = c0.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2]; g.OH = OH; g.OW = OW;
+            g.err_plane = batch_dk ? OH * OW : 0;
+            g.C = c1.shape[0]; g.H = c1.shape[1]; g.W = c1.shape[2]; g.OH = OH; g.OW = OW;
             g.cg = 1;
             constexpr int R = F32 ? 8 : 4;
             int rc = NK_OK;
@@ -785,7 +798,9 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
                 if ((rc = workspace(dev, (uint64_t)parts * on * sizeof(T), &ws))) return;
                 dim3 grid(g.col_blocks, (nstrips + 3) / 4, g.C);
                 hipLaunchKernelGGL((conv_chan_dk<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, S, nstrips, s1, s2, (T*)ws);
-                hipLaunchKernelGGL(conv_partial_reduce_wide<T>, dim3((on + 3) / 4), dim3(256), 0, dev->stream, parts, on, (const T*)ws, out);
+                // a batch sums the images' tap gradients as well: [parts][C][k*k] read as [parts * C][k*k]
+                const int sums = batch_dk ? parts * g.C : parts, outs = batch_dk ? KK * KK : on;
+                hipLaunchKernelGGL(conv_partial_reduce_wide<T>, dim3((outs + 3) / 4), dim3(256), 0, dev->stream, sums, outs, (const T*)ws, out);
             });
             if (!ok) return NK_OK;
             if (rc) return rc;

@@ -824,18 +824,18 @@ def test_convolution_literal_kernels_bit_exact(device, orc, dt):
             simple = orc.simple_conv2d(img.reshape(-1), tap.reshape(-1), ishape[-1], ishape[-2], tshape[-1], tshape[-2], batch=ishape[0] if len(xs) == 3 else 1)
             assert_bits(out.getData(), simple, f"fwd simple {xs} {ks}")
             np.testing.assert_allclose(out.getData(), want, rtol=1e-5 if dt == "f32" else 1e-12, atol=1e-5 if dt == "f32" else 1e-12)
-        else:       # dense f32 [C,H,W] x [C,kh,kw] takes the channel kernel: same sums in another order
-            assert dt == "f32" and len(xs) == 3
-            np.testing.assert_allclose(out.getData(), want, rtol=1e-5, atol=1e-5)
+        else:       # dense [C,H,W] x [C,kh,kw] takes the channel kernel: same sums in another order
+            assert len(xs) == 3
+            np.testing.assert_allclose(out.getData(), want, rtol=1e-5 if dt == "f32" else 1e-12, atol=1e-5 if dt == "f32" else 1e-12)
         for tgt, tgt_shape, other, other_arr, other_shape in ((tx, xs, tk, k, ks), (tk, ks, tx, x, xs)):
             drn = Tensor._on_device(device, F[dt], tgt_shape)
             device.launch_convolution(0, drn, other, te)
             want = orc.deconvolve(np.zeros(drn.size, dtype=F[dt]), orc.dense_cfg(tgt_shape), other_arr.reshape(-1), orc.dense_cfg(other_shape), e.reshape(-1), orc.dense_cfg(ys))
             if _lib.last_path().startswith("literal"):
                 assert_bits(drn.getData(), want, f"bwd {tgt_shape} {other_shape}")
-            else:
-                assert dt == "f32" and len(xs) == 3
-                np.testing.assert_allclose(drn.getData(), want, rtol=1e-5, atol=1e-5)
+            else:       # ... and so do its gradients, and those of a batch of images under one set of taps
+                assert len(xs) == 3
+                np.testing.assert_allclose(drn.getData(), want, rtol=1e-5 if dt == "f32" else 1e-12, atol=1e-5 if dt == "f32" else 1e-12)
     say("conv literal on a transposed operand", dt)
     x = rng.uniform(-1, 1, (8, 10)).astype(F[dt]); k = rng.uniform(-1, 1, (3, 3)).astype(F[dt])
     tx, tk = on(device, x), on(device, k)
@@ -943,6 +943,8 @@ def test_convolution_split_sums(device, orc, shape, dt):
         assert seen == {"chan_fwd", "chan_dx", "chan_dk"}, seen          # the register-window kernels take dense square taps
     elif ks == [5, 5]:                                                   # ... and a 2-D image as their one-channel case
         assert seen == {"simple2d_window", "chan_dx", "chan_dk"}, seen
+    elif ks == [1, 3, 3]:                                                # ... and a batch of images under one set of taps
+        assert seen == {"simple2d", "chan_dx", "chan_dk"}, seen
     else:
         assert seen & {"split_fwd", "split_bwd"}, seen
     if len(xs) == 2:
@@ -955,6 +957,35 @@ def test_convolution_split_sums(device, orc, shape, dt):
         assert _lib.last_path() == "split_bwd"
         want = orc.deconvolve(np.zeros(dk.size, dtype=T), orc.dense_cfg(ks), x.reshape(-1), cfg(vx), e.reshape(-1), orc.dense_cfg(ys))
         assert_bits(dk.getData(), want, "transposed operand")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("shape", [([6, 40, 300], [1, 5, 5]), ([3, 33, 65], [1, 3, 3]), ([40, 70, 70], [1, 7, 7]), ([2, 9, 520], [1, 2, 2]),
+                                   ([130, 12, 12], [1, 4, 4])])
+def test_batched_image_gradients_on_the_channel_kernels(device, orc, shape, dt):
+    """[B,H,W] x [1,k,k]: the error has one plane per image.  The input gradient convolves every image's plane with the
+    one set of taps, the tap gradient also sums over the images: exact on integer-valued data, norm-wise otherwise."""
+    xs, ks = shape
+    T = F[dt]
+    tol = RTOL[np.dtype(T)]
+    ys = [xs[0], xs[1] - ks[1] + 1, xs[2] - ks[2] + 1]
+    rng = np.random.default_rng(49)
+    for integer in (True, False):
+        draw = (lambda sh: rng.integers(-3, 4, sh).astype(T)) if integer else (lambda sh: rng.uniform(-1, 1, sh).astype(T))
+        x, k, e = draw(xs), draw(ks), draw(ys)
+        tx, tk, te = on(device, x), on(device, k), on(device, e)
+        for name, tgt_shape, other, other_arr, other_shape in (("dx", xs, tk, k, ks), ("dk", ks, tx, x, xs)):
+            say("batched conv gradient", name, xs, ks, dt, "integer" if integer else "uniform")
+            drn = Tensor._on_device(device, T, tgt_shape)
+            device.launch_convolution(0, drn, other, te)
+            assert _lib.last_path() == "chan_" + name, _lib.last_path()
+            want = orc.deconvolve(np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt_shape), other_arr.reshape(-1), orc.dense_cfg(other_shape), e.reshape(-1), orc.dense_cfg(ys), fast=True)
+            if integer:
+                assert_bits(drn.getData(), want, name + " on integers")
+            else:
+                babs = orc.deconvolve(np.zeros(drn.size), orc.dense_cfg(tgt_shape), np.abs(other_arr).astype(np.float64).reshape(-1), orc.dense_cfg(other_shape),
+                                      np.abs(e).astype(np.float64).reshape(-1), orc.dense_cfg(ys), fast=True)
+                assert (np.abs(drn.getData().astype(np.float64) - want) <= tol * babs + 1e-30).all(), name
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
