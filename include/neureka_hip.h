@@ -166,6 +166,15 @@ int nk_convolution(nk_dev dev, int d, int dtype, int rank,
  * result is bit-identical to the CPU device's. */
 int nk_sum(nk_dev dev, int dtype, nk_buf in, int64_t n, nk_buf out);
 
+/* nk_sum for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same result as nk_sum, bit for bit; the partial results
+ * of the tree live in a 1 MiB array that is part of the library's device image (one copy per GPU, held until the
+ * process ends) instead of the grow-on-demand device workspace, so the call neither allocates nor frees.
+ * n <= NK_SUM_STATIC_MAX_N, larger inputs are an argument error.  Calls that overlap in time on one GPU share the
+ * array and race; nothing in it has to be cleared between calls (every slot is written before it is read). */
+#define NK_SUM_STATIC_MAX_N ((int64_t)1 << 30)
+int nk_sum_static(nk_dev dev, int dtype, nk_buf in, int64_t n, nk_buf out);
+
 /* CLReduce (min / max): J/backend/main/operations/linear/internal/opencl/CLReduce.java, registered in
  * J/backend/main/operations/other/Min.java:72-73 and Max.java:72-73.  Writes to out_index[0] (int32) the index of
  * the minimum or maximum of the n elements of `in`, found as the CPU device finds it: tiles of 64, strict

@@ -52,6 +52,7 @@ SYMBOLS = {
     "nk_matmul": (_i32, [_u64, _i32, _i32, _i64, _i64, _i64, _u64, _u64, _u64]),
     "nk_scalarization_int": (_i32, [_u64, _i32, _i32, _i32, _i32, _u64, _cfg, _u64, _cfg, _i64, _i64]),
     "nk_sum": (_i32, [_u64, _i32, _u64, _i64, _u64]),
+    "nk_sum_static": (_i32, [_u64, _i32, _u64, _i64, _u64]),
     "nk_reduce_index": (_i32, [_u64, _i32, _i32, _u64, _i64, _u64]),
     "nk_dot": (_i32, [_u64, _i32, _u64, _u64, _i64, _u64]),
     "nk_fused": (_i32, [_u64, C.POINTER(C.c_int32), _i32, C.POINTER(C.c_double), _i32, _i32, _i32, _u64, _cfg, _i32,

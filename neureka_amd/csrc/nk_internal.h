@@ -21,12 +21,15 @@ struct Device {
     // grow-only scratch for two-pass kernels (partial sums); owned by the device, freed on close
     void* workspace = nullptr;
     uint64_t workspace_bytes = 0;
+    // this device's copy of the file-scope array nk_sum_static keeps its partial results in
+    void* sum_static_scratch = nullptr;
 };
 
 int set_error(int code, const char* fmt, ...);
 void set_path(const char* name);
 Device* device_of(nk_dev h);            // nullptr (and error set) if unknown
 int workspace(Device* dev, uint64_t bytes, void** out);
+int stats_static_init(Device* dev);     // resolves sum_static_scratch; the device must be current
 
 #define NK_HIP(expr)                                                                         \
     do {                                                                                     \

@@ -194,6 +194,7 @@ int nk_device_open(int index, nk_dev* dev) {
     NK_HIP(hipSetDevice(index));
     NK_HIP(hipGetDeviceProperties(&d->props, index));
     NK_HIP(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+    if (int e = stats_static_init(d.get())) { (void)hipStreamDestroy(d->stream); return e; }
     std::lock_guard<std::mutex> lock(g_devices_mu);
     g_devices.push_back(std::move(d));
     *dev = g_devices.size();

@@ -208,18 +208,33 @@ __global__ __launch_bounds__(256) void tail_reduce_kernel(const T* __restrict__ 
     }
 }
 
+// Partial results reduce_levels keeps for n elements: what every launch but the last writes (a launch covers two
+// levels of the tree) plus one slot for the last; values first, then, from the next 16-byte boundary, their indices.
+template <int RTS>
+static int64_t partial_slots(int64_t n) {
+    int64_t total = 1, m = n;
+    while ((m + RTS - 1) / RTS > 256) { m = ((m + RTS - 1) / RTS + RTS - 1) / RTS; total += m; }
+    return total;
+}
+template <typename T, int RTS>
+static uint64_t partials_bytes(int64_t n) {
+    const uint64_t total = (uint64_t)partial_slots<RTS>(n);
+    return ((total * sizeof(T) + 15) & ~(uint64_t)15) + total * sizeof(int);
+}
+
+// `scratch` (of at least partials_bytes<T, RTS>(n) bytes) holds the partial results; nullptr takes the device
+// workspace, which is grown (allocated) on demand.
 template <typename T, int RTS, int MODE>
-static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* out_value, int* out_index) {
+static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* out_value, int* out_index,
+                         void* scratch = nullptr) {
     constexpr bool indexed = MODE == STAT_MIN || MODE == STAT_MAX;
     if (MODE == STAT_SUM && n == 1) {               // CPUSum returns a single element as it is (keeps a -0)
         NK_HIP(hipMemcpyAsync(out_value, in, sizeof(T), hipMemcpyDeviceToDevice, dev->stream));
         return NK_OK;
     }
-    // partial results of all levels but the last live in the device workspace: values first, then indices
-    int64_t total = 0;
-    { int64_t m = n; do { m = (m + RTS - 1) / RTS; total += m; } while (m > 1); }
-    void* ws = nullptr;
-    if (int e = workspace(dev, (uint64_t)total * (sizeof(T) + sizeof(int)) + 64, &ws)) return e;
+    const int64_t total = partial_slots<RTS>(n);
+    void* ws = scratch;
+    if (!ws) if (int e = workspace(dev, partials_bytes<T, RTS>(n), &ws)) return e;
     T* vals = (T*)ws;
     int* idxs = (int*)((char*)ws + (((uint64_t)total * sizeof(T) + 15) & ~(uint64_t)15));
     const T* cur = in;
@@ -273,6 +288,36 @@ extern "C" int nk_sum(nk_dev h, int dtype, nk_buf in, int64_t n, nk_buf out) {
     set_path("tile_tree_128");
     return dtype == NK_F32 ? reduce_levels<float, 128, STAT_SUM>(dev, (const float*)in, nullptr, n, (float*)out, nullptr)
                            : reduce_levels<double, 128, STAT_SUM>(dev, (const double*)in, nullptr, n, (double*)out, nullptr);
+}
+
+// nk_sum for callers that cannot allocate: the partial results live in a file-scope device array instead of the
+// device workspace.  The array's name is a host-side stand-in, not a device address; the address is asked for once
+// per opened device (with that device current) and only that pointer is handed to the kernels.
+constexpr uint64_t SUM_STATIC_BYTES = 1u << 20;
+static __device__ __align__(256) unsigned char scratch[SUM_STATIC_BYTES];
+
+int nk::stats_static_init(Device* dev) {
+    void* ptr = nullptr;
+    NK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    dev->sum_static_scratch = ptr;
+    return NK_OK;
+}
+
+extern "C" int nk_sum_static(nk_dev h, int dtype, nk_buf in, int64_t n, nk_buf out) {
+    NK_DEVICE(dev, h);
+    NK_REQUIRE(n <= NK_SUM_STATIC_MAX_N, "nk_sum_static: n = %lld exceeds the maximum of %lld elements this entry point "
+               "holds partial results for; use nk_sum", (long long)n, (long long)NK_SUM_STATIC_MAX_N);
+    if (int e = check_vector(dev, "nk_sum_static(in)", dtype, in, n)) return e;
+    if (int e = check_range(dev, "nk_sum_static(out)", out, 0, dtype_bytes(dtype))) return e;
+    const uint64_t need = dtype == NK_F32 ? partials_bytes<float, 128>(n) : partials_bytes<double, 128>(n);
+    NK_REQUIRE(need <= SUM_STATIC_BYTES, "nk_sum_static: %llu bytes of partial results exceed the static scratch",
+               (unsigned long long)need);
+    NK_REQUIRE(dev->sum_static_scratch != nullptr, "nk_sum_static: the static scratch of this device was not resolved");
+    set_path("tile_tree_128_static");
+    // every partial slot a launch reads was written by the launch before it, so nothing has to start at zero
+    return dtype == NK_F32
+        ? reduce_levels<float, 128, STAT_SUM>(dev, (const float*)in, nullptr, n, (float*)out, nullptr, dev->sum_static_scratch)
+        : reduce_levels<double, 128, STAT_SUM>(dev, (const double*)in, nullptr, n, (double*)out, nullptr, dev->sum_static_scratch);
 }
 
 extern "C" int nk_reduce_index(nk_dev h, int kind, int dtype, nk_buf in, int64_t n, nk_buf out_index) {
