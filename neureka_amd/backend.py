@@ -21,7 +21,7 @@ from .device import HipDevice
 from .ndim import IllegalArgumentException, IllegalStateException, Layout
 
 # suitability scores: backend/api/fun/SuitabilityPredicate.java:21-29
-VERY_GOOD, GOOD, BAD, UNSUITABLE = 0.75, 0.625, 0.25, 0.0
+PERFECT, EXCELLENT, VERY_GOOD, GOOD, BAD, UNSUITABLE = 1.0, 0.875, 0.75, 0.625, 0.25, 0.0
 
 ACTIVATIONS = ["abs", "cos", "gasu", "gatu", "gaus", "fast_gaus", "gelu", "idy", "ln", "quad", "relu", "selu", "sig",
                "silu", "sin", "softplus", "softsign", "tanh", "fast_tanh", "exp", "log10", "sqrt", "cbrt"]
@@ -180,6 +180,82 @@ class ElementwiseAlgorithm(Algorithm):
         if call.input(0) is None:
             call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape))
         return call
+
+
+def _two_slots(call: ExecutionCall) -> List[Optional[object]]:
+    """(drain or None, source): the activation calls arrive with one input or with an empty drain slot in front."""
+    return [None] + list(call.inputs) if call.arity == 1 else list(call.inputs)
+
+
+class ScalarAlgorithm(Algorithm):
+    """"scalar activation": a function of a virtual tensor is a virtual tensor (algorithms/ScalarAlgorithm.java:15-58)."""
+    name = "scalar activation"
+
+    def isSuitableFor(self, call):       # ScalarAlgorithm.java:24-34
+        ts = _two_slots(call)
+        if len(ts) != 2 or ts[1] is None or not ts[1].isVirtual():
+            return UNSUITABLE
+        if ts[0] is not None and (not ts[0].isVirtual() or ts[0].shape != ts[1].shape):
+            return UNSUITABLE
+        return EXCELLENT
+
+    def prepare(self, call):             # ScalarAlgorithm.java:36-46: a virtual output of the source's shape and type
+        from .tensor import Tensor
+        ts = _two_slots(call)
+        if ts[0] is None:
+            out = Tensor.of(ts[1].dtype, ts[1].shape, 0.0).to(call.device)
+            out._intermediate = True
+            ts[0] = out
+        return call.withInputs(ts)
+
+
+class ScalarBroadcast(Algorithm):
+    """"scalar broadcast": a function of a virtual tensor written to every element of a full drain
+    (algorithms/ScalarBroadcast.java:21-82)."""
+    name = "scalar broadcast"
+
+    def isSuitableFor(self, call):       # ScalarBroadcast.java:32-42
+        ts = _two_slots(call)
+        if len(ts) != 2 or ts[1] is None or not ts[1].isVirtual():
+            return UNSUITABLE
+        if ts[0] is not None and (ts[0].isVirtual() or ts[0].shape != ts[1].shape):
+            return UNSUITABLE
+        return VERY_GOOD
+
+    def prepare(self, call):             # ScalarBroadcast.java:44-58: a full (actual) output of the source's shape
+        ts = _two_slots(call)
+        if ts[0] is None:
+            ts[0] = _new_output(call.device, ts[1].dtype, ts[1].shape)
+        return call.withInputs(ts)
+
+
+class AssignScalar(BiScalarBroadcast):
+    """The BiScalarBroadcast of AssignLeft (operations/other/AssignLeft.java:32-71): the last operand is one value
+    (virtual or of size 1) that is written to every element of the drain's view."""
+
+    def isSuitableFor(self, call):       # AssignLeft.java:35-51
+        if call.arity > 3:
+            raise IllegalArgumentException("AssignLeft operation only supports up to 3 arguments!")
+        if call.arity < 2:
+            raise IllegalArgumentException("AssignLeft operation needs at least 2 arguments!")
+        last = call.input(call.arity - 1)
+        return PERFECT if last.isVirtual() or last.size == 1 else UNSUITABLE
+
+    def prepare(self, call):             # AssignLeft.java:59-68
+        offset = 1 if call.input(0) is None else 0
+        call.input(offset).setIsVirtual(False)
+        return replace(call, inputs=[call.input(offset), call.input(offset + 1)], derivIdx=-1)
+
+
+class AssignElementwise(ElementwiseAlgorithm):
+    """The ElementwiseAlgorithm of AssignLeft (AssignLeft.java:74-98): drain view <- source view, element by element."""
+
+    def isSuitableFor(self, call):       # AssignLeft.java:76-81
+        return EXCELLENT if call.arity in (2, 3) else UNSUITABLE
+
+    def prepare(self, call):             # AssignLeft.java:88-95
+        offset = 1 if call.input(0) is None else 0
+        return replace(call, inputs=[call.input(offset), call.input(offset + 1)], derivIdx=-1)
 
 
 class NDConvolution(Algorithm):
@@ -358,8 +434,10 @@ class BackendContext:
         self.operations["min"] = Operation("min", "min", [ReduceAlgorithm()])
         self.operations["max"] = Operation("max", "max", [ReduceAlgorithm()])
         self.operations["dot"] = Operation("dot", "dot", [DotProductAlgorithm()])
-        for f in ACTIVATIONS:
-            self.operations[f] = Operation(f, f, [ElementwiseAlgorithm()])
+        for f in ACTIVATIONS:      # functions/AbstractActivationOperation.java:38-50
+            self.operations[f] = Operation(f, f, [ElementwiseAlgorithm(), ScalarBroadcast(), ScalarAlgorithm()])
+        self.operations["left_inline"] = Operation("left_inline", "<", [AssignScalar(), AssignElementwise()])
+        self.operations["random"] = Operation("random", "rand", [ElementwiseAlgorithm()])
         self.extensions: List[object] = []
 
     def getOperation(self, identifier: str) -> Operation:
@@ -436,6 +514,58 @@ def hip_elementwise_function(fun: str):
         call.device.launch_activation(fun, call.derivIdx, call.input(0), call.input(1))
         return call.input(0)
     return run
+
+
+def hip_scalar_function(fun: str):
+    """CLScalarFunction (implementations/scalar/CLScalarFunction.java:11-29): drain item 0 = f(source item 0), both
+    tensors virtual.  The reference evaluates f on the host and writes the item; here the one stored element goes
+    through the activation kernel on the device, so no value crosses the bus and f is the device's f."""
+    def run(call: ExecutionCall):
+        call.device.launch_activation_item(fun, call.derivIdx, call.input(0), call.input(1))
+        return call.input(0)
+    return run
+
+
+def hip_scalar_broadcast_function(fun: str):
+    """The OpenCLDevice lambda of ScalarBroadcast (algorithms/ScalarBroadcast.java:64-81): value = f(source item 0),
+    then the scalar_broadcast kernel writes it through the drain's view."""
+    def run(call: ExecutionCall):
+        dev, drn, src = call.device, call.input(0), call.input(1)
+        slot = dev.allocate(drn.dtype, 1)
+        try:
+            dev.launch_activation_item(fun, call.derivIdx, slot, src)
+            value = float(dev._read(slot, 0, 1)[0])         # the reference reads the item too (blocking)
+        finally:
+            slot.release()
+        dev.launch_scalar_fill(drn, value)
+        return drn
+    return run
+
+
+def hip_scalar_broadcast_identity(call: ExecutionCall):
+    """CLScalarBroadcastIdentity (implementations/broadcast/CLScalarBroadcastIdentity.java:18-32): the drain is passed
+    as drain and as source, the kernel writes the value."""
+    drn = call.input(0)
+    value = call.input(1).item(0)
+    value = int(value) if np.issubdtype(drn.dtype, np.integer) else float(value)
+    call.device.launch_scalarization("idy", call.derivIdx, drn, drn, value)
+    return drn
+
+
+def hip_assign_elementwise(call: ExecutionCall):
+    """CLElementwiseFunction(ScalarFun.IDENTITY) as AssignLeft registers it (backend/ocl/CLBackend.java:232-234); the
+    drain is made actual first as CPUElementwiseAssignFun does (implementations/elementwise/CPUElementwiseAssignFun.java:30)."""
+    drn, src = call.input(0), call.input(1)
+    if drn.shape != src.shape:
+        raise IllegalArgumentException(f"cannot assign a tensor of shape {list(src.shape)} to one of shape {list(drn.shape)}")
+    drn.setIsVirtual(False)
+    call.device.launch_activation("idy", -1, drn, src)
+    return drn
+
+
+def hip_randomization(call: ExecutionCall):
+    """CLRandomization (implementations/elementwise/CLRandomization.java:8-13) is a stub that throws; so is this."""
+    raise IllegalStateException("Not yet implemented")
 
 
 def hip_convolution(call: ExecutionCall):
@@ -525,8 +655,22 @@ class HipBackend:
         registry.forOperation("min").set(ReduceAlgorithm, hip_reduce("min"))
         registry.forOperation("max").set(ReduceAlgorithm, hip_reduce("max"))
         registry.forOperation("dot").set(DotProductAlgorithm, hip_dot)
-        for f in ACTIVATIONS:
-            registry.forOperation(f).set(ElementwiseAlgorithm, hip_elementwise_function(f))
+        (registry.forOperation("left_inline")                                    # CLBackend.java:232-234
+            .set(BiScalarBroadcast, hip_scalar_broadcast_identity)
+            .set(ElementwiseAlgorithm, hip_assign_elementwise))
+        registry.forOperation("random").set(ElementwiseAlgorithm, hip_randomization)     # CLBackend.java:252-253
+        for f in ACTIVATIONS:                                                    # CLBackend.java:255-324
+            (registry.forOperation(f)
+                .set(ElementwiseAlgorithm, hip_elementwise_function(f))
+                .set(ScalarAlgorithm, hip_scalar_function(f)))
+            # ScalarBroadcast carries its device implementation itself (ScalarBroadcast.java:64-81): it is attached
+            # to the algorithm object, not through a registry row
+            self.context_operation(registry, f).getAlgorithm(ScalarBroadcast).setImplementationFor(
+                HipDevice, hip_scalar_broadcast_function(f))
+
+    @staticmethod
+    def context_operation(registry: _Registry, identifier: str) -> "Operation":
+        return registry.ctx.getOperation(identifier)
 
     def dispose(self) -> None:
         for dev in list(HipDevice._open.values()):

@@ -338,8 +338,8 @@ __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b
         case NK_OP_SUB * 2 + 1: NK_EACH2(T(-1));
         case NK_OP_MUL * 2 + 0: NK_EACH2(y);
         case NK_OP_MUL * 2 + 1: NK_EACH2(x);
-        case NK_OP_IDY * 2 + 0: NK_EACH2(T(0));
-        case NK_OP_IDY * 2 + 1: NK_EACH2(T(1));
+        case NK_OP_IDY * 2 + 0:
+        case NK_OP_IDY * 2 + 1: NK_EACH2(y);      // CPUScalarBroadcastIdentity.java:25-33: both derivatives are the function itself
         default:
             if constexpr (FUNSET >= 2) {
                 switch (op * 2 + d) {

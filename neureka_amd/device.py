@@ -8,6 +8,7 @@ the C ABI of ``libneureka_hip.so``.  Method names follow ``neureka.devices.Devic
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -98,7 +99,10 @@ class HipDevice:
         self.index = index
         self._disposed = False
         self._data_objects = 0
-        self._stored: List[object] = []          # tensors currently outsourced to this device
+        # tensors currently outsourced to this device, held weakly (id -> weak reference): a tensor nobody holds any
+        # more leaves the table by itself and its HipData releases the buffer once no tensor shares it -- the role of
+        # the DeviceCleaner on weak reachability (devices/AbstractDevice.java:59,109; OpenCLDevice.java:301)
+        self._stored: Dict[int, weakref.ref] = {}
         name = C.create_string_buffer(256)
         cu, mhz, lds, wave = C.c_int(0), C.c_int(0), C.c_int(0), C.c_int(0)
         mem = C.c_uint64(0)
@@ -126,7 +130,17 @@ class HipDevice:
         return not self._stored
 
     def has(self, tensor) -> bool:
-        return any(t is tensor for t in self._stored)
+        ref = self._stored.get(id(tensor))
+        return ref is not None and ref() is tensor
+
+    def _register(self, tensor) -> None:
+        key = id(tensor)
+        stored = self._stored
+
+        def gone(ref, key=key, stored=stored):
+            if stored.get(key) is ref:       # the id may have been taken by a younger tensor meanwhile
+                del stored[key]
+        stored[key] = weakref.ref(tensor, gone)
 
     def contains(self, tensor) -> bool:
         return self.has(tensor)
@@ -148,12 +162,12 @@ class HipDevice:
             if isinstance(host, HipData):
                 if host.device is self:
                     tensor._set_data(host, self)
-                    self._stored.append(tensor)
+                    self._register(tensor)
                     return self
                 raise IllegalStateException("tensor already lives on another device")
             data = self._upload(host, tensor.dtype, tensor.isVirtual())
             tensor._set_data(data, self)
-        self._stored.append(tensor)
+        self._register(tensor)
         return self
 
     def restore(self, tensor) -> "HipDevice":
@@ -167,12 +181,9 @@ class HipDevice:
 
     def free(self, tensor) -> "HipDevice":
         """Drops the device's claim on the tensor (OpenCLDevice.java:609-620)."""
-        for i, t in enumerate(self._stored):
-            if t is tensor:
-                del self._stored[i]
-                break
-        else:
+        if not self.has(tensor):
             raise IllegalArgumentException("tensor is not stored on this device")
+        del self._stored[id(tensor)]
         data = tensor._data
         tensor._data = None
         tensor._device = None
@@ -194,9 +205,11 @@ class HipDevice:
         """OpenCLDevice.dispose (OpenCLDevice.java:299-304): finishes the queue and drops every buffer."""
         if self._disposed:
             return
-        for t in list(self._stored):
-            t._data = None
-            t._device = None
+        for ref in list(self._stored.values()):
+            t = ref()
+            if t is not None:
+                t._data = None
+                t._device = None
         self._stored.clear()
         _lib.check(self._lib.nk_device_close(self.handle))
         self._disposed = True
@@ -325,6 +338,15 @@ class HipDevice:
     def launch_activation(self, fun: str, d: int, drn, src) -> None:
         (p0, k0, c0), (p1, k1, c1) = self._ops(drn, src)
         _lib.check(self._lib.nk_activation(self.handle, _lib.FUN[fun], d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, drn.ndc.size))
+
+    def launch_activation_item(self, fun: str, d: int, drn, src) -> None:
+        """f (or f') of the one element a virtual tensor keeps on the device, written to the drain's one element.
+        `drn` / `src` are virtual tensors or bare one-element buffers."""
+        one = NDConfiguration.ofShape((1,)).asInlineArray()
+        dt = drn.dtype
+        p0 = C.c_uint64(drn.ptr if isinstance(drn, HipData) else drn._data.ptr)
+        p1 = C.c_uint64(src.ptr if isinstance(src, HipData) else src._data.ptr)
+        _lib.check(self._lib.nk_activation(self.handle, _lib.FUN[fun], d, _dtype_code(dt), 1, p0, _lib.cfg_ptr(one), p1, _lib.cfg_ptr(one), 1))
 
     def launch_elementwise(self, op: str, d: int, drn, a, b) -> None:
         (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = self._ops(drn, a, b)

@@ -18,8 +18,8 @@ import numpy as np
 from typing import List, Optional, Sequence, Union
 
 from . import _lib
-from .backend import (ACTIVATIONS, BiElementwise, BiScalarBroadcast, Broadcast, ExecutionCall, backend,
-                      execute_device_algorithm, execute_on_common_device)
+from .backend import (ACTIVATIONS, BiElementwise, BiScalarBroadcast, Broadcast, ExecutionCall, ScalarAlgorithm,
+                      ScalarBroadcast, backend, execute_device_algorithm, execute_on_common_device)
 from .ndim import IllegalArgumentException, IllegalStateException
 from .tensor import GraphNode, Tensor, make_fit
 
@@ -36,6 +36,10 @@ def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = Tr
     ctx = backend()
     operation = ctx.getOperation(op_id)
     device = _device_for(inputs)
+    if op_id == "left_inline":               # operations/other/AssignLeft.java:103-114: inline, no autograd
+        if d >= 0:
+            raise IllegalArgumentException("Assignment does not support autograd!")
+        record = False
     parents = list(inputs)                   # the tensors the caller holds: gradients attach to these
     if len(inputs) > 1 and len({t.rank for t in inputs}) > 1 and op_id != "dot":
         inputs = make_fit(list(inputs))      # FunctionNode.execute pads ranks first (FunctionNode.java:92-93)
@@ -45,7 +49,7 @@ def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = Tr
     def run(c: ExecutionCall):
         c = c.algorithm.prepare(c)
         for t in c.inputs[1:]:
-            if t.isVirtual() and not isinstance(c.algorithm, BiScalarBroadcast):
+            if t.isVirtual() and not isinstance(c.algorithm, (BiScalarBroadcast, ScalarAlgorithm, ScalarBroadcast)):
                 t.setIsVirtual(False)       # sources are de-virtualised before the kernels (CPUBiElementWise.java:103-104)
         return execute_device_algorithm(c), c
 
@@ -153,8 +157,8 @@ class Node:
         return f"({self.children[0]!r} {self.value} {self.children[1]!r})"
 
 
-_TOKEN = re.compile(r"\s*(?:(\d+\.\d*(?:[eE][-+]?\d+)?|\d+(?:[eE][-+]?\d+)?)|([iI]\[?\s*\d+\s*\]?)|([A-Za-z_][A-Za-z_0-9]*)|(\*\*|[-+*/%^()@,]))")
-_BIN_OPS = {"+": ("add", 1), "-": ("subtract", 1), "*": ("multiply", 2), "/": ("divide", 2), "%": ("modulo", 2),
+_TOKEN = re.compile(r"\s*(?:(\d+\.\d*(?:[eE][-+]?\d+)?|\d+(?:[eE][-+]?\d+)?)|([iI]\[?\s*\d+\s*\]?)|([A-Za-z_][A-Za-z_0-9]*)|(\*\*|<-|[-+*/%^()@,]))")
+_BIN_OPS = {"<-": ("left_inline", 0), "+": ("add", 1), "-": ("subtract", 1), "*": ("multiply", 2), "/": ("divide", 2), "%": ("modulo", 2),
             "x": ("mul_conv", 2), "@": ("matMul", 2), "^": ("power", 3), "**": ("power", 3)}
 
 
@@ -179,7 +183,7 @@ class _Parser:
     def peek(self): return self.t[self.i] if self.i < len(self.t) else (None, None)
     def next(self): tok = self.peek(); self.i += 1; return tok
 
-    def expr(self, min_prec: int = 1) -> Node:
+    def expr(self, min_prec: int = 0) -> Node:
         left = self.atom()
         while True:
             kind, val = self.peek()
@@ -188,7 +192,7 @@ class _Parser:
                 return left
             self.next()
             op, prec = _BIN_OPS[sym]
-            right = self.expr(prec + 1)
+            right = self.expr(prec if op == "left_inline" else prec + 1)     # a <- b <- c nests to the right
             left = Node("op", op, [left, right])
 
     def atom(self) -> Node:
@@ -310,6 +314,8 @@ def derivative_of(n: Node, index: int) -> Node:
         first = _mul(_mul(v, Node("op", "power", [u, Node("op", "subtract", [v, _const(1.0)])])), du)
         second = _mul(_mul(Node("op", "power", [u, v]), Node("fun", "ln", [u])), dv)
         return _add(first, second)
+    if n.value == "modulo":          # operator/Modulo.java:183-185: the derivative of the first operand
+        return du
     raise IllegalArgumentException(f"operator '{n.value}' has no fused derivative")
 
 
@@ -354,13 +360,31 @@ class OptimizedFunction:
             self._derivatives[index] = (program, consts)
         return self._derivatives[index]
 
+    def _with_guests(self, srcs: List[Tensor], run):
+        """Operands that are not on the device are stored for the call and restored afterwards
+        (AbstractDeviceAlgorithm.executeOnCommonDevice, AbstractDeviceAlgorithm.java:427-449)."""
+        guests = [t for t in srcs if not t.isOutsourced()]
+        for t in guests:
+            self.device.store(t)
+        try:
+            for t in srcs:
+                t.setIsVirtual(False)
+            return run()
+        finally:
+            for t in guests:
+                if self.device.has(t):
+                    self.device.restore(t)
+
     def derive(self, inputs: Sequence[Tensor], index: int) -> Tensor:
         """d f / d I[index] at the inputs, in one launch."""
         srcs = list(inputs[: self.n_src])
         program, consts = self.derivative_program(index)
-        out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
-        self.device.launch_fused(program, consts, out, srcs)
-        return out
+
+        def run():
+            out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
+            self.device.launch_fused(program, consts, out, srcs)
+            return out
+        return self._with_guests(srcs, run)
 
     def call(self, *inputs: Tensor) -> Tensor:
         if len(inputs) == 1 and isinstance(inputs[0], (list, tuple)):
@@ -371,22 +395,18 @@ class OptimizedFunction:
         for t in srcs:
             if t.shape != srcs[0].shape:
                 raise IllegalArgumentException("operands of a fused function must share one shape")
-        guests = [t for t in srcs if not t.isOutsourced()]
-        for t in guests:
-            self.device.store(t)
-        try:
-            for t in srcs:
-                t.setIsVirtual(False)
+
+        def run():
             out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
             self.device.launch_fused(self.program, self.consts, out, srcs)
-            if self.function.doAD and not guests and any(t.rqsGradient() or t._node is not None for t in srcs):
-                # reverse mode: error * (d f / d I[d]), the derivative in one fused launch
-                def action(d):
-                    return lambda error: execute("multiply", [error, self.derive(srcs, d)], record=False)
-                out._node = GraphNode(srcs, [action(d) if (t.rqsGradient() or t._node is not None) else None for d, t in enumerate(srcs)])
             return out
-        finally:
-            for t in guests:
-                self.device.restore(t)
+        out = self._with_guests(srcs, run)
+        if self.function.doAD and any(t.rqsGradient() or t._node is not None for t in srcs):
+            # reverse mode: error * (d f / d I[d]), the derivative in one fused launch (operands that live on the
+            # host are stored again for that launch)
+            def action(d):
+                return lambda error: execute("multiply", [error, self.derive(srcs, d)], record=False)
+            out._node = GraphNode(srcs, [action(d) if (t.rqsGradient() or t._node is not None) else None for d, t in enumerate(srcs)])
+        return out
 
     __call__ = call

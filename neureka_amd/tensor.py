@@ -66,7 +66,7 @@ class Tensor:
         t = Tensor(dtype, ndc, None)
         data = device.allocateFromOne(dtype, ndc.size, 0)
         t._set_data(data, device)
-        device._stored.append(t)
+        device._register(t)
         return t
 
     # ---- shape -----------------------------------------------------------------------------------
@@ -101,6 +101,17 @@ class Tensor:
             data.incrementUsageCount()
         if isinstance(old, HipData) and old is not data:
             old.decrementUsageCount()
+
+    def __del__(self):
+        # a tensor that is dropped without Device.free gives up its share of the buffer (the usage count the
+        # DeviceCleaner decrements in the reference: OpenCLDevice.java:950-966)
+        try:
+            data = self._data
+            if isinstance(data, HipData):
+                self._data = None
+                data.decrementUsageCount()
+        except Exception:
+            pass
 
     def _replace_data(self, data: HipData) -> None:
         self._set_data(data, self._device)
@@ -165,7 +176,7 @@ class Tensor:
         v._parent = self
         if self._device is not None:
             v._set_data(self._root()._data, self._device)
-            self._device._stored.append(v)
+            self._device._register(v)
         else:
             v._data = self._data
         return v
@@ -229,6 +240,13 @@ class Tensor:
     def mod(self, o): return self._bin("modulo", o)
     def power(self, o): return self._bin("power", o)
     __add__, __sub__, __mul__, __truediv__, __mod__, __pow__ = plus, minus, times, div, mod, power
+
+    def assign(self, other) -> "Tensor":
+        """``mut.assign(other)`` / ``I[0] <- I[1]``: the operation "left_inline" (operations/other/AssignLeft.java)."""
+        from .function import execute
+        if not isinstance(other, Tensor):
+            other = Tensor.of(self.dtype, self.shape, int(other) if np.issubdtype(self.dtype, np.integer) else float(other))
+        return execute("left_inline", [self, other])
 
     def conv(self, k: "Tensor") -> "Tensor":
         from .function import execute

@@ -278,7 +278,7 @@ double orc_bin_f64(int family, int op, int d, double a, double b) {
         case OP_MUL: return d == 0 ? b : a;
         case OP_DIV: case OP_MOD: return d == 0 ? 1.0 / b : -a / orc_java_pow(b, 2);
         case OP_POW: return d == 0 ? b * orc_java_pow(a, b - 1) : orc_java_pow(a, b) * log(a);
-        case OP_IDY: return d == 0 ? 0 : 1;
+        case OP_IDY: return b;   /* CPUScalarBroadcastIdentity.java:25-33: _getDeriveAt0/1 return _getFun() */
     }
     return (double)NAN;
 }
@@ -306,7 +306,7 @@ float orc_bin_f32(int family, int op, int d, float a, float b) {
         case OP_MUL: return d == 0 ? b : a;
         case OP_DIV: case OP_MOD: return d == 0 ? 1.0f / b : (float)-((double)a / orc_java_pow((double)b, 2));
         case OP_POW: return d == 0 ? (float)((double)b * orc_java_pow((double)a, (double)(b - 1))) : (float)(orc_java_pow((double)a, (double)b) * log((double)a));
-        case OP_IDY: return d == 0 ? 0 : 1;
+        case OP_IDY: return b;   /* CPUScalarBroadcastIdentity.java:25-33: _getDeriveAt0/1 return _getFun() */
     }
     return NAN;
 }

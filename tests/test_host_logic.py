@@ -154,3 +154,54 @@ def test_symbolic_derivative_of_fused_expressions():
     # folding: the derivative with respect to an absent input is the constant 0, of I[0]+I[1] the constant 1
     assert repr(derivative_of(Function.of("sig(I[0])*I[1]").root, 2)) == "0.0"
     assert repr(derivative_of(Function.of("I[0]+I[1]").root, 1)) == "1.0"
+
+
+def test_every_registration_row_of_the_opencl_backend_has_a_hip_counterpart():
+    """CLBackend.java:200-325 as data (tests/golden/clbackend_registration_rows.json): every (operation, algorithm) row
+    must resolve to an implementation for HipDevice, and ScalarBroadcast must carry one on every activation."""
+    import json
+    import importlib
+    B = importlib.import_module("neureka_amd.backend")
+    from neureka_amd.device import HipDevice
+    rows = json.load(open(os.path.join(ROOT, "tests", "golden", "clbackend_registration_rows.json")))
+    ctx = B.BackendContext().set(B.HipBackend())           # registration touches no device
+    probe = object.__new__(HipDevice)                      # an instance only for the class lookup
+    for op_id, alg_name in rows["rows"]:
+        alg = ctx.getOperation(op_id).getAlgorithm(getattr(B, alg_name))
+        assert alg is not None, (op_id, alg_name)
+        assert alg.getImplementationFor(probe) is not None, f"no HipDevice implementation for {op_id} x {alg_name}"
+    for f in B.ACTIVATIONS:
+        alg = ctx.getOperation(f).getAlgorithm(B.ScalarBroadcast)
+        assert alg is not None and alg.getImplementationFor(probe) is not None, f
+    # every row must hit an existing (operation, algorithm) pair, as BackendContext.set demands (BackendContext.java:309-318)
+    with pytest.raises(IllegalStateException):
+        B._Registry(ctx, HipDevice).forOperation("add").set(B.NDConvolution, lambda call: None)
+    with pytest.raises(IllegalStateException):
+        B.hip_randomization(None)
+
+
+def test_integration_text_binds_every_export_and_every_registration_row():
+    """INTEGRATION.md is the binding a maintainer copies: it must declare a MethodHandle for every export of the header
+    and name every operation class the OpenCL backend registers."""
+    header = open(os.path.join(ROOT, "include", "neureka_hip.h")).read()
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    declared = sorted(set(re.findall(r"\b(nk_[a-z0-9_]+)\s*\(", header)))
+    bound = set(re.findall(r'MethodHandle\s+(nk_[a-z0-9_]+)\s*=\s*h\("(nk_[a-z0-9_]+)"', text))
+    assert all(a == b for a, b in bound)
+    missing = [n for n in declared if n not in {a for a, _ in bound}]
+    assert not missing, f"exports without a MethodHandle in INTEGRATION.md: {missing}"
+    for cls in ("Addition", "Subtraction", "Multiplication", "Division", "Modulo", "Power", "AssignLeft", "Convolution", "XConvLeft",
+                "XConvRight", "MatMul", "DotProduct", "Sum", "Randomization", "Absolute", "Cosinus", "GaSU", "GaTU", "Gaussian",
+                "GaussianFast", "GeLU", "Identity", "Logarithm", "Quadratic", "ReLU", "SeLU", "Sigmoid", "SiLU", "Sinus", "Softplus",
+                "Softsign", "Tanh", "TanhFast", "Exp", "Cbrt", "Log10", "Sqrt"):
+        assert re.search(rf"\b{cls}\.class", text), f"{cls} is not registered in INTEGRATION.md"
+    for method in ("_readAll", "_readItem", "_readArray", "_writeItem", "_writeArray", "_swap", "_sizeOccupiedBy", "_actualize",
+                   "_virtualize", "_dataTypeOf", "allocateFromOne", "allocateFromAll", "optimizedOperationOf", "dispose"):
+        assert re.search(rf"\b{method}\(", text), f"HipDevice.{method} is missing from INTEGRATION.md"
+
+
+def test_assignment_parses_and_nests_to_the_right():
+    assert repr(Function.of("I[0]<-I[1]").root) == "(I[0] left_inline I[1])"           # Function_Parsing_Spec.groovy:67
+    assert repr(Function.of("I[0] <- (I[0] * -3)").root) == "(I[0] left_inline (I[0] multiply (-1.0 multiply 3.0)))"
+    assert repr(Function.of("I[2]<-I[0]<-I[1]").root) == "(I[2] left_inline (I[0] left_inline I[1]))"
+    assert repr(Function.of("I[0] <- I[1] + I[2]").root) == "(I[0] left_inline (I[1] add I[2]))"
