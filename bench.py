@@ -27,6 +27,8 @@ FP64_PEAK_TFLOPS = 78.6        # MI355X dense fp64 matrix, published
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
 # against a plain 1 GiB copy): profiles/rows_binary_lean_kernel_broadcast_c2.md
 C2_TRAFFIC_BYTES = 4316437187
+SETTLE_MS = 60.0               # untimed load before the warm-up steps, so that the timed steps run at the working clock
+HOST_CORE_SHARE = 16           # host threads one GPU's box grants a job, whatever the machine's core count
 
 
 def event_time_ms(dev, launch, reps):
@@ -149,6 +151,13 @@ def main():
 
     if args.calibrate:
         _lib.check(dev._lib.nk_d2d(dev.handle, out._data.ptr, 0, out._data.ptr, 2 << 30, 1 << 30))
+    # The clock of an idle device takes about 30 ms of load to reach its working frequency (the first steps after
+    # idleness run at 1.5 ms, the 25th at 1.2 ms), more than a handful of warm-up steps: load the device for
+    # SETTLE_MS first, untimed, then run the W warm-up steps, synchronise, and time exactly K steps.
+    t_settle = time.perf_counter()
+    while (time.perf_counter() - t_settle) * 1e3 < SETTLE_MS:
+        step()
+        dev.sync()
     for _ in range(args.warmup):
         step()
     dev.sync()
@@ -181,7 +190,7 @@ def main():
     cpu = None
     if not args.no_cpu:
         from oracle import cpu_oracle as orc
-        cores = min(16, len(os.sched_getaffinity(0)))
+        cores = min(HOST_CORE_SHARE, len(os.sched_getaffinity(0)))
         rows = 256                                             # sample: the first 256 of 1024 slabs of the output
         sample_shape = (rows, 2048, 512)
         drn = np.zeros(int(np.prod(sample_shape)), dtype=f32)
@@ -199,7 +208,10 @@ def main():
         cpu = {"value": round(passes * sample_bytes / spent / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": f"{passes} passes (add, multiply alternating) over the first {rows}/1024 slabs of the output "
                          f"({drn.size} elements per pass, {spent:.1f} s in total): the oracle's restatement of "
-                         "CPUBroadcast._broadcastF32 split like JVMExecutor; no JVM exists on this box"}
+                         "CPUBroadcast._broadcastF32 split like JVMExecutor over min(host cores, "
+                         f"{HOST_CORE_SHARE}) threads ({len(os.sched_getaffinity(0))} cores visible; {HOST_CORE_SHARE} is "
+                         "the CPU share of a one-GPU job on this pool, the reference would take availableProcessors()); "
+                         "no JVM exists on this box"}
         del drn
     dev.free(out)
 
@@ -350,7 +362,7 @@ def main():
     # ---- the reference's CPU path beside the other configurations (oracle, bounded samples) -----------------------
     cpu_others = None
     if not args.no_cpu and not args.no_others:
-        cpu_others = cpu_side_of_the_other_configs(min(16, len(os.sched_getaffinity(0))))
+        cpu_others = cpu_side_of_the_other_configs(min(HOST_CORE_SHARE, len(os.sched_getaffinity(0))))
 
     result = {
         "metric": "GB/s & % HBM peak (broadcast/elementwise)",
@@ -367,7 +379,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "broadcast add + multiply, f32 [1024,1,512] o [1,2048,512] -> [1024,2048,512], "
                                "one step = one add launch + one multiply launch, 4 301 258 752 algorithmic bytes each",
-                   "device": dev.name(), "compute_units": dev.maxComputeUnits()},
+                   "device": dev.name(), "compute_units": dev.maxComputeUnits(),
+                   "clock_settle": f"{SETTLE_MS:.0f} ms of the same steps, untimed, before the warm-up steps"},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "cpu_others": cpu_others,

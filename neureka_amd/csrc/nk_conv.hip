@@ -332,6 +332,32 @@ __device__ __forceinline__ double from_prev_lane(double keep, double v) {
     r[1] = __builtin_amdgcn_update_dpp(k[1], s[1], 0x138, 0xf, 0xf, false);
     return __builtin_bit_cast(double, r);
 }
+// Sum over the 64 lanes of a wavefront, delivered in lane 63, with data-parallel-primitive adds instead of LDS
+// permutes: four shifted adds inside each row of 16 lanes (lane 15 of a row then holds the row's sum), then lane 15
+// of rows 0 and 2 is added into rows 1 and 3, then lane 31 into rows 2 and 3.  Lanes a step does not reach, or
+// whose source lies outside the row, add zero.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_zero(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_or_zero(double v) {
+    const i32x2 s = __builtin_bit_cast(i32x2, v);
+    i32x2 r;
+    r[0] = __builtin_amdgcn_update_dpp(0, s[0], CTRL, ROW_MASK, 0xf, false);
+    r[1] = __builtin_amdgcn_update_dpp(0, s[1], CTRL, ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(double, r);
+}
+template <typename T>
+__device__ __forceinline__ T wave_sum_in_lane63(T v) {
+    v += dpp_or_zero<0x111, 0xf>(v);        // row_shr:1
+    v += dpp_or_zero<0x112, 0xf>(v);        // row_shr:2
+    v += dpp_or_zero<0x114, 0xf>(v);        // row_shr:4
+    v += dpp_or_zero<0x118, 0xf>(v);        // row_shr:8
+    v += dpp_or_zero<0x142, 0xa>(v);        // row_bcast:15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v);        // row_bcast:31 into rows 2 and 3
+    return v;
+}
 constexpr int WAVE_COLS = 64 * CX;          // columns per wavefront
 
 // CX adjacent results through ordinary 16-byte stores
@@ -455,6 +481,103 @@ __global__ __launch_bounds__(NW * 64) void conv_chan_fwd(ChanArgs g, const T* __
     }
 }
 
+// forward on planes too small for the strips above to fill the machine: a block owns a tile of TR output rows x 64
+// columns and reduces ALL channels for it, so the result leaves in one launch with no partial planes.  Its NW
+// wavefronts take every NW-th channel.  A wavefront stages a channel's (TR + K - 1) x (64 + K - 1) input window in
+// its own piece of LDS with 16-byte loads that run along the rows (the next channel's loads are in flight while the
+// current one is multiplied), then every lane reads the K x (TR + K - 1) values above its own output column and
+// multiplies them in: the only vector instructions besides the multiply-adds are the LDS accesses.  The tiles of an
+// XCD form a band of neighbouring strips, so the K - 1 rows two strips share meet in that XCD's L2 and are
+// fetched from memory once.
+template <typename T, int K, int TR, int NW>
+__global__ __launch_bounds__(NW * 64) void conv_chan_fwd_tiles(ChanArgs g, int col_tiles, int n_tiles, int per_xcd,
+                                                               const T* __restrict__ in, const T* __restrict__ w, T* __restrict__ out) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int WR = TR + K - 1;                               // window rows
+    constexpr int PITCH = (64 + K - 1 + VEC - 1) / VEC * VEC;    // window columns, a whole number of 16-byte pieces
+    constexpr int PPR = PITCH / VEC;                             // pieces per window row
+    constexpr int PIECES = WR * PPR;
+    constexpr int LOADS = (PIECES + 63) / 64;
+    constexpr int STAGE = WR * PITCH;
+    constexpr int WORDS = NW * STAGE > NW * TR * 64 ? NW * STAGE : NW * TR * 64;
+    __shared__ __attribute__((aligned(16))) T lds[WORDS];        // the windows; afterwards the wavefronts' sums
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    // blocks are dealt round-robin to the 8 XCDs: XCD k works through tiles [k * per_xcd, (k + 1) * per_xcd)
+    const int tile = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if (tile >= n_tiles) return;                                 // whole blocks leave together
+    const int x0 = (tile % col_tiles) * 64, y0 = (tile / col_tiles) * TR;
+    T* mine = lds + wave * STAGE;
+
+    // piece k of the lane: where it comes from in the plane and where it goes in the window
+    unsigned src_off[LOADS];
+    int dst_at[LOADS];
+#pragma unroll
+    for (int k = 0; k < LOADS; k++) {
+        const int p = lane + 64 * k;
+        const int row = p / PPR, col = (p - row * PPR) * VEC;
+        src_off[k] = (unsigned)(((y0 + row) * g.W + x0 + col) * (int)sizeof(T));
+        dst_at[k] = p < PIECES ? row * PITCH + col : -1;
+    }
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 piece[LOADS];
+    const unsigned plane_bytes = (unsigned)g.H * (unsigned)g.W * (unsigned)sizeof(T);
+    auto request = [&](int c) {                                  // rows past the plane read as zero (range check per dword)
+        const BufRsrc plane = buffer_of(in + (int64_t)c * g.H * g.W, plane_bytes);
+#pragma unroll
+        for (int k = 0; k < LOADS; k++)
+            if (LOADS * 64 == PIECES || dst_at[k] >= 0)
+                piece[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(plane, src_off[k], 0, 0));
+    };
+    T acc[TR];
+#pragma unroll
+    for (int r = 0; r < TR; r++) acc[r] = T(0);
+    // One channel ahead: the next window's loads are in flight while the current one is multiplied.  (More channels
+    // in flight measured slower: 7.1 us with one, 7.4 with two, 7.7 with four on [64,256,256] x [64,5,5].)
+    if (wave < g.C) request(wave);
+    for (int c = wave; c < g.C; c += NW) {
+#pragma unroll
+        for (int k = 0; k < LOADS; k++)
+            if (LOADS * 64 == PIECES || dst_at[k] >= 0) *(u32x4*)(mine + dst_at[k]) = piece[k];
+        __builtin_amdgcn_wave_barrier();                         // LDS operations of a wavefront complete in order
+        if (c + NW < g.C) request(c + NW);
+        T wt[K][K];
+        const T* wc = w + (int64_t)c * (K * K);
+#pragma unroll
+        for (int ky = 0; ky < K; ky++)
+#pragma unroll
+            for (int kx = 0; kx < K; kx++) wt[ky][kx] = wc[ky * K + kx];
+#pragma unroll
+        for (int rr = 0; rr < WR; rr++) {
+            T v[K];
+#pragma unroll
+            for (int kx = 0; kx < K; kx++) v[kx] = mine[rr * PITCH + lane + kx];
+#pragma unroll
+            for (int ky = 0; ky < K; ky++) {
+                const int r = rr - ky;
+                if (r >= 0 && r < TR) {
+#pragma unroll
+                    for (int kx = 0; kx < K; kx++) acc[r] = fused_mad(v[kx], wt[ky][kx], acc[r]);
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();                         // the window is read before the next one overwrites it
+    }
+    __syncthreads();                                             // every wavefront is done with its window
+#pragma unroll
+    for (int r = 0; r < TR; r++) lds[(wave * TR + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < TR * 64; e += NW * 64) {       // wavefronts added in a fixed order
+        const int r = e >> 6, col = e & 63;
+        const int yo = y0 + r, xo = x0 + col;
+        if (yo < g.OH && xo < g.OW) {
+            T s = lds[r * 64 + col];
+#pragma unroll
+            for (int k = 1; k < NW; k++) s = s + lds[(k * TR + r) * 64 + col];
+            out[(int64_t)yo * g.OW + xo] = s;
+        }
+    }
+}
+
 // gradient w.r.t. the big operand: dx[c][y][x] = sum_ky sum_kx w[c][ky][kx] * err[y-ky][x-kx] (zero outside err)
 // wave -> (column block over W, strip of R rows of dx, channel group); the err window of the strip is loaded once
 // (one 16-byte load per row) and reused by every channel of the group.  
@@ -559,28 +682,88 @@ __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstri
 #pragma unroll
                     for (int j = 0; j < CX; j++) acc[ky][kx] = fused_mad(V[r][j], E[r - ky + KH - 1][j - kx + KW - 1], acc[ky][kx]);
     }
-    // lanes -> lane 0: every step moves all KH*KW sums before any of them is added, so the cross-lane
-    // exchanges of one step are in flight together instead of one dependent chain per sum
+    // lanes -> lane 63 with data-parallel-primitive adds
     const int part = strip * gridDim.x + blockIdx.x;
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        T moved[KH][KW];
+    for (int ky = 0; ky < KH; ky++)
 #pragma unroll
-        for (int ky = 0; ky < KH; ky++)
-#pragma unroll
-            for (int kx = 0; kx < KW; kx++) moved[ky][kx] = __shfl_down(acc[ky][kx], off, 64);
-#pragma unroll
-        for (int ky = 0; ky < KH; ky++)
-#pragma unroll
-            for (int kx = 0; kx < KW; kx++) acc[ky][kx] += moved[ky][kx];
-    }
-    if (lane == 0) {
+        for (int kx = 0; kx < KW; kx++) acc[ky][kx] = wave_sum_in_lane63(acc[ky][kx]);
+    if (lane == 63) {
         T* dst = partial + ((int64_t)part * g.C + c) * (KH * KW);
 #pragma unroll
         for (int ky = 0; ky < KH; ky++)
 #pragma unroll
             for (int kx = 0; kx < KW; kx++) dst[ky * KW + kx] = acc[ky][kx];
     }
+}
+
+// The same sums for planes small enough that the channels alone fill the machine: a block is NW wavefronts of one
+// channel that own neighbouring strips; their lanes are reduced with data-parallel-primitive adds, the wavefronts
+// through LDS in a fixed order, and the block writes the channel's KH*KW results -- one launch, no partial sums.
+// (For larger planes the same blocks with their partial sums joined by the block that draws a channel's last
+// ticket were measured: the agent-scope release before the ticket costs more than a second launch, 14.6 us
+// against 11.8 on [64,256,256] x [64,5,5]; blocks of eight wavefronts plus a second launch were no faster than
+// the strips of conv_chan_dk either.)
+template <typename T, int KH, int KW, int R, int NW>
+__global__ __launch_bounds__(NW * 64) void conv_chan_dk_joined(ChanArgs g, int S, int nstrips, const T* __restrict__ in, const T* __restrict__ err,
+                                                               T* __restrict__ dst) {
+    constexpr int KK = KH * KW;
+    __shared__ T red[NW][KK];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int strip = blockIdx.y * NW + wave;
+    const int xx = blockIdx.x * WAVE_COLS + lane * CX;
+    const int yy0 = strip * S;
+    int yy1 = yy0 + S; if (yy1 > g.H) yy1 = g.H;
+    const int c = blockIdx.z;
+    T acc[KH][KW];
+#pragma unroll
+    for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+        for (int kx = 0; kx < KW; kx++) acc[ky][kx] = T(0);
+    const T* plane = in + (int64_t)c * g.H * g.W;
+    for (int y = yy0; y < yy1; y += R) {                          // no trip for a wavefront past the last strip
+        T E[R + KH - 1][CX + KW - 1];                             // E[rr][i] = err[y - (KH-1) + rr][xx - (KW-1) + i], zero outside err
+        T V[R][CX];                                               // V[r] = input row y + r, zero past the strip
+#pragma unroll
+        for (int r = 0; r < R; r++) load_cols(row_of(plane, y + r, g.W, y + r < yy1), xx, V[r]);
+#pragma unroll
+        for (int rr = 0; rr < R + KH - 1; rr++) {
+            const int ey = y - (KH - 1) + rr;
+            load_cols(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, &E[rr][KW - 1]);
+        }
+#pragma unroll
+        for (int rr = 0; rr < R + KH - 1; rr++) {
+            const int ey = y - (KH - 1) + rr;
+            extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, lane);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+                for (int kx = 0; kx < KW; kx++)
+#pragma unroll
+                    for (int j = 0; j < CX; j++) acc[ky][kx] = fused_mad(V[r][j], E[r - ky + KH - 1][j - kx + KW - 1], acc[ky][kx]);
+    }
+#pragma unroll
+    for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+        for (int kx = 0; kx < KW; kx++) acc[ky][kx] = wave_sum_in_lane63(acc[ky][kx]);
+    if (lane == 63) {
+#pragma unroll
+        for (int ky = 0; ky < KH; ky++)
+#pragma unroll
+            for (int kx = 0; kx < KW; kx++) red[wave][ky * KW + kx] = acc[ky][kx];
+    }
+    __syncthreads();
+    if (wave != 0) return;                                        // KK <= 64: the first wavefront finishes
+    const int t = lane;
+    T s = T(0);
+    if (t < KK) {
+#pragma unroll
+        for (int k = 0; k < NW; k++) s = s + red[k][t];           // wavefronts in order
+    }
+    if (t < KK) dst[(int64_t)c * KK + t] = s;
 }
 
 static bool dense_rm(const Cfg& c, int rank) {
@@ -700,6 +883,7 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
         g.OH = g.H - small.shape[1] + 1; g.OW = g.W - small.shape[2] + 1;
         const int cus = dev->props.multiProcessorCount;
         int rc = NK_OK;
+        bool tiled = false;
         const bool ok = for_taps(small.shape[1], small.shape[2], [&](auto K) {
             constexpr int KK = decltype(K)::value;
             g.col_blocks = (g.OW + WAVE_COLS - 1) / WAVE_COLS;
@@ -721,6 +905,25 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
                 }
                 return;
             }
+            // Planes that still give about one (TR rows x 64 columns) tile per compute unit: every block reduces all
+            // channels of its tile, one launch.
+            {
+                constexpr int NW = F32 ? 16 : 8;
+                const int col_tiles = (g.OW + 63) / 64;
+                int tr = 0;
+                for (int r : {8, 4})
+                    if ((int64_t)col_tiles * ((g.OH + r - 1) / r) * 10 >= (int64_t)cus * 9) { tr = r; break; }
+                if (!tr && (int64_t)col_tiles * ((g.OH + 3) / 4) * 2 >= cus) tr = 4;
+                if (tr && g.C >= NW) {
+                    const int n_tiles = col_tiles * ((g.OH + tr - 1) / tr);
+                    const int per_xcd = (n_tiles + 7) / 8;
+                    g.cg = g.C;
+                    if (tr == 8) hipLaunchKernelGGL((conv_chan_fwd_tiles<T, KK, 8, NW>), dim3(8 * per_xcd), dim3(NW * 64), 0, dev->stream, g, col_tiles, n_tiles, per_xcd, bigp, smallp, out);
+                    else         hipLaunchKernelGGL((conv_chan_fwd_tiles<T, KK, 4, NW>), dim3(8 * per_xcd), dim3(NW * 64), 0, dev->stream, g, col_tiles, n_tiles, per_xcd, bigp, smallp, out);
+                    tiled = true;
+                    return;
+                }
+            }
             // Small planes: parallelism has to come from the channels.  Blocks of four wavefronts take groups of
             // channels (multiples of 4), a second pass adds the partial planes in a fixed order.
             constexpr int R = F32 ? 8 : 4;
@@ -739,7 +942,7 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
         if (!ok) return NK_OK;
         if (rc) return rc;
         NK_HIP(hipGetLastError());
-        set_path("chan_fwd");
+        set_path(tiled ? "chan_fwd_tiles" : "chan_fwd");
         *taken = true;
         return NK_OK;
     }
@@ -795,6 +998,13 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
                 const int parts = nstrips * g.col_blocks;
                 const int on = g.C * KK * KK;
                 void* ws = nullptr;
+                constexpr int NW = 8;
+                if (!batch_dk && g.col_blocks == 1 && nstrips <= NW) {
+                    // a channel fits one block of NW wavefronts: finished in one launch
+                    dim3 grid(1, 1, g.C);
+                    hipLaunchKernelGGL((conv_chan_dk_joined<T, KK, KK, R, NW>), grid, dim3(NW * 64), 0, dev->stream, g, S, nstrips, s1, s2, out);
+                    return;
+                }
                 if ((rc = workspace(dev, (uint64_t)parts * on * sizeof(T), &ws))) return;
                 dim3 grid(g.col_blocks, (nstrips + 3) / 4, g.C);
                 hipLaunchKernelGGL((conv_chan_dk<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, g, S, nstrips, s1, s2, (T*)ws);

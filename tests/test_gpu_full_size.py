@@ -195,7 +195,7 @@ def test_config5_conv_forward_and_backward_full_size(device, orc):
     tx = on(device, x).setRqsGradient(True); tk = on(device, k).setRqsGradient(True)
     say("C5 forward")
     y = tx.conv(tk)
-    assert _lib.last_path() == "chan_fwd" and list(y.shape) == ys
+    assert _lib.last_path() == "chan_fwd_tiles" and list(y.shape) == ys      # one launch: every block reduces all channels of its tile
     dc = orc.dense_cfg
     want = orc.convolve(np.zeros(252 * 252, dtype=f32), dc(ys), x.reshape(-1), dc(xs), k.reshape(-1), dc(ks), workers=16)
     babs = orc.convolve(np.zeros(252 * 252), dc(ys), np.abs(x).astype(np.float64).reshape(-1), dc(xs), np.abs(k).astype(np.float64).reshape(-1), dc(ks), workers=16)

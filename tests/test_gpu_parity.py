@@ -336,7 +336,8 @@ def test_exotic_descriptor_falls_back_to_the_literal_formula(device, orc):
     assert phys == physical_indices(ndc).tolist() == [0, 0, 1, 3, 3, 4]
     assert_bits(out.getData(), src[phys] + np.arange(6, dtype=np.float32), "literal")
     # the same descriptor as the drain
-    out2 = Tensor(np.float32, ndc, None); out2._set_data(on(device, np.full(12, -1, dtype=np.float32))._data, device)
+    backing = on(device, np.full(12, -1, dtype=np.float32))             # kept: a dropped tensor gives up its buffer
+    out2 = Tensor(np.float32, ndc, None); out2._set_data(backing._data, device)
     device.launch_activation("idy", -1, out2, dense6)
     # a unary kernel addresses its source with the DRAIN's nd-index (CPUElementwiseFunction.java:103-104):
     # flat 0..5 -> nd (0,0),(0,0),(0,1),(1,0),(1,0),(1,1) -> the dense source's elements 0,0,1,3,3,4
@@ -855,7 +856,11 @@ def _abs_bound(orc, xs, ks, x, k, dt):
 @pytest.mark.parametrize("shape", [([8, 40, 70], [8, 5, 5]), ([6, 33, 65], [6, 3, 3]), ([5, 20, 21], [5, 4, 2]), ([64, 64, 64], [64, 5, 5]),
                                    ([3, 130, 200], [3, 7, 7]), ([9, 17, 300], [9, 2, 2]), ([2, 12, 12], [2, 4, 4]),
                                    ([3, 10, 71], [3, 3, 3]), ([5, 9, 302], [5, 2, 2]), ([70, 30, 261], [70, 5, 5]),
-                                   ([16, 520, 1030], [16, 3, 3]), ([16, 300, 1100], [16, 7, 7])])
+                                   ([16, 520, 1030], [16, 3, 3]), ([16, 300, 1100], [16, 7, 7]),
+                                   # planes that give about one (rows x 64 columns) tile per compute unit: every block reduces all
+                                   # channels of its tile (4-row and 8-row tiles, ragged edges, channel counts that leave wavefronts idle)
+                                   ([20, 130, 520], [20, 3, 3]), ([17, 200, 700], [17, 5, 5]), ([33, 140, 500], [33, 7, 7]),
+                                   ([16, 130, 520], [16, 2, 2]), ([19, 131, 517], [19, 4, 4])])
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_channel_convolution_fast_paths(device, orc, shape, dt):
     """[C,H,W] x [C,kh,kw] forward and both gradients on the register-window kernels: re-ordered sums, compared
@@ -873,6 +878,8 @@ def test_channel_convolution_fast_paths(device, orc, shape, dt):
     square = ks[1] == ks[2]          # the register-window kernels exist for square taps of extent 2, 3, 4, 5, 7
     # other tap shapes take the general kernels: one thread per element, or (sums of 128 terms and more into few elements) split sums
     fwd, dxp, dkp = ("chan_fwd", "chan_dx", "chan_dk") if square else ("literal_fwd", "literal_bwd", "split_bwd")
+    if xs[2] >= 500 and xs[1] <= 200:
+        fwd = "chan_fwd_tiles"
     say("chan_fwd", xs, ks, dt)
     out = Tensor._on_device(device, T, ys)
     device.launch_convolution(-1, out, tx, tk)
