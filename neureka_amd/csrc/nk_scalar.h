@@ -103,20 +103,35 @@ __device__ __forceinline__ float inv_sqrt_ref(float x) {
 // ScalarSigmoid.sig (fun/ScalarSigmoid.java:38): 1/(1+exp(-x)).
 __device__ __forceinline__ double sigmoid(double x) { return 1.0 / (1.0 + ::exp(-x)); }
 // f32 building blocks for the two activations of the bandwidth-critical chain (sig, tanh): the
-// hardware exp2 and reciprocal (about 1 ulp each).  exp(t) = exp2(t * log2 e) carries the rounding of the
-// product into the result as a relative error of |t| * 2^-24, so with |t| clamped to where the functions
-// saturate the results stay within ~5e-6 relative of the reference, inside the 1e-5 contract, at a
-// fraction of the instructions of the library routines.
-__device__ __forceinline__ float fast_exp_neg(float t) {        // exp(-t) for t >= 0
-    return __builtin_amdgcn_exp2f(-1.44269504088896341f * t);
+// hardware exp2 and reciprocal (about 1 ulp each).  exp(-t) = exp2(-t * log2 e); the rounding of that product
+// alone would enter the result as a relative error of t * 2^-24 (5e-6 at t = 87), so the product is carried in two
+// floats -- p and what p lacks -- and the small part is applied to the result to first order.  `dt` is a
+// correction of the argument the caller already knows (the rounding of x * 1.702 in gelu), 0 otherwise.
+// The results stay within a few ulp of the reference's (float) f((double) x) over the whole range.
+__device__ __forceinline__ float fast_exp_neg(float t, float dt = 0.0f) {        // exp(-(t + dt)) for t >= 0
+    const float L = 1.44269502162933349609375f;                  // (float) log2(e)
+    const float L_LO = 1.925963033500947e-8f;                    // log2(e) - L
+    t = t > 128.0f ? 128.0f : t;                                 // exp(-128) is below the smallest float; a NaN stays
+    const float p = t * L;
+    const float lack = __builtin_fmaf(t, L, -p) + (t * L_LO + dt * L);
+    const float e = __builtin_amdgcn_exp2f(-p);
+    return __builtin_fmaf(e * -0.693147182464599609375f, lack, e);               // e * 2^-lack
 }
 // f32: the same quantity as the reference's double evaluation, evaluated on e = exp(-|x|) <= 1 so
-// nothing overflows: x >= 0 -> 1/(1+e), x < 0 -> e/(1+e).
-__device__ __forceinline__ float sigmoid(float x) {
-    const float e = fast_exp_neg(::fabsf(x));
+// nothing overflows: x >= 0 -> 1/(1+e), x < 0 -> e/(1+e).  `dx` as above: sigmoid(x + dx).
+__device__ __forceinline__ float sigmoid(float x, float dx = 0.0f) {
+    const float e = fast_exp_neg(::fabsf(x), x >= 0.0f ? dx : -dx);
     const float r = __builtin_amdgcn_rcpf(1.0f + e);
     return x >= 0.0f ? r : e * r;
 }
+// x * 1.702 in two floats (the reference multiplies in double: fun/ScalarGeLU.java), then the sigmoid of it
+__device__ __forceinline__ float gelu_sigmoid(float x) {
+    const float C = 1.70200002193450927734375f;                  // (float) 1.702
+    const float y = x * C;
+    const float lo = ::fabsf(y) < 1.0e30f ? __builtin_fmaf(x, C, -y) + x * -2.193450927734375e-8f : 0.0f;   // + x * (1.702 - C)
+    return sigmoid(y, lo);
+}
+__device__ __forceinline__ double gelu_sigmoid(double x) { return sigmoid(x * 1.702); }
 
 // ScalarTanh.tanh (fun/ScalarTanh.java:37-38): 2/(1+exp(-2x))-1.
 __device__ __forceinline__ double tanh_ref(double x) { return 2.0 / (1.0 + ::exp(-x * 2.0)) - 1.0; }
@@ -185,9 +200,14 @@ template <typename T> __device__ __forceinline__ T dselu_ref(T x) {
 }
 __device__ __forceinline__ float tanh_f32_via_f64(float x) { return (float)(2.0 / (1.0 + ::exp((double)(-x * 2.0f))) - 1.0); }
 __device__ __forceinline__ float sig_f32_via_f64(float x) { return (float)(1.0 / (1.0 + ::exp(-(double)x))); }
+// log(1 + exp(x)) (fun/ScalarSoftplus.java:18-22).  The reference evaluates exactly this in double, and for x below
+// about -16 the sum 1 + exp(x) keeps only a few bits of exp(x): its result is exp(x) rounded to a multiple of
+// 2^-52 (0 or 2.2e-16 around x = -36.7).  Parity is with those results, so the f32 kernel repeats the double
+// formula there; above, log1p of the float exponential agrees with it to a few ulp.
 template <typename T> __device__ __forceinline__ T softplus_ref(T x) {
     using N = Num<T>;
     if (sizeof(T) == 8) return N::log(T(1) + N::exp(x));
+    if (x < T(-13)) return T(::log(1.0 + ::exp((double)x)));
     return x > T(0) ? x + N::log1p(N::exp(-x)) : N::log1p(N::exp(x));
 }
 template <typename T> __device__ __forceinline__ T dgasu_ref(T x) {
@@ -234,7 +254,7 @@ __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
         case NK_FUN_GATU: NK_EACH(tanh_ref(x * x * x));
         case NK_FUN_GAUS: NK_EACH(gauss(x));
         case NK_FUN_FAST_GAUS: NK_EACH(T(1) / (T(1) + x * x));
-        case NK_FUN_GELU: NK_EACH(x * sigmoid(x * T(1.702)));
+        case NK_FUN_GELU: NK_EACH(x * gelu_sigmoid(x));
         case NK_FUN_IDY: break;
         case NK_FUN_LN: NK_EACH(N::log(x));
         case NK_FUN_QUAD: NK_EACH(x * x);
@@ -242,7 +262,6 @@ __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
         case NK_FUN_SELU: NK_EACH(selu_ref(x));
         case NK_FUN_SIG: NK_EACH(sigmoid(x));
         case NK_FUN_SILU: NK_EACH(x * sigmoid(x));
-        case NK_FUN_SOFTPLUS: NK_EACH(softplus_ref(x));
         case NK_FUN_SOFTSIGN: NK_EACH(softsign(x));
         case NK_FUN_TANH: NK_EACH(tanh_ref(x));
         case NK_FUN_FAST_TANH: NK_EACH(x * inv_sqrt_ref(T(1) + x * x));
@@ -251,6 +270,7 @@ __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
         default:
             if constexpr (FUNSET >= 2) {
                 switch (id) {
+                    case NK_FUN_SOFTPLUS: NK_EACH(softplus_ref(x));
                     case NK_FUN_COS: NK_EACH(N::cos(x));
                     case NK_FUN_SIN: NK_EACH(N::sin(x));
                     case NK_FUN_LOG10: NK_EACH(N::log10(x));
@@ -262,7 +282,7 @@ __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
 }
 
 // does function `id` need the full table?
-inline bool fun_is_heavy(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN || id == NK_FUN_LOG10 || id == NK_FUN_CBRT; }
+inline bool fun_is_heavy(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN || id == NK_FUN_LOG10 || id == NK_FUN_CBRT || id == NK_FUN_SOFTPLUS; }
 
 template <typename T, int V>
 __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {

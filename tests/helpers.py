@@ -4,10 +4,11 @@ import decimal
 import numpy as np
 
 # Tolerances of the parity contract.  + - * and copies are compared bit for bit; transcendental
-# activations and reductions (convolution, matmul) within RTOL relative, with an absolute floor that
-# covers the cancellation noise of the reference's own formulas (2/(1+e^-2x)-1 and e^x-1 near 0).
+# activations and reductions (convolution, matmul) within RTOL relative, with an absolute floor of four rounding
+# quanta of a double near 1: the reference's own formulas 2/(1+e^-2x)-1 and e^x-1 are evaluated in double (also for
+# float tensors) and return multiples of 2^-52 near 0, whatever the true value is.
 RTOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
-ATOL = {np.dtype(np.float32): 1e-10, np.dtype(np.float64): 2.0 ** -50}
+ATOL = {np.dtype(np.float32): 2.0 ** -50, np.dtype(np.float64): 2.0 ** -50}
 
 
 def assert_close(got, want, what=""):

@@ -1,0 +1,99 @@
+"""The f32 activations that go through exp -- the two of the benchmark chain (sig, tanh) and everything built on them --
+swept densely against the oracle's evaluation of the reference's formulas ((float) f((double) x), ScalarSigmoid.java:14-38,
+ScalarTanh.java:20-38, CPUFun.java:7-9): every binade from 2^-30 to 2^7 on both signs, the neighbourhood of the series
+switch of tanh at |x| = 1/8, and the points where the functions saturate or underflow.
+
+Contract: |got - want| <= 1e-5 * |want| + atol for EVERY element.  atol is 1e-30 (it only admits results in the
+subnormal range, where the device flushes to zero), except for the two functions whose reference formula cancels in
+double at arguments this sweep reaches: gatu = tanh(x^3) evaluates 2/(1+exp(-2y))-1 at y = x^3 down to 1e-27, and selu
+evaluates exp(x)-1 at x down to -1e-9; both return multiples of the double rounding quantum there (0, 1.1e-16,
+2.2e-16, ...) where the true value is smaller, so those results are pinned only to within that quantum (4e-16).
+The worst relative error seen per function is printed."""
+import numpy as np
+import pytest
+
+from neureka_amd import Tensor
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-30
+QUANTUM = {"gatu": 4e-16, "selu": 4e-16}       # cancellation quantum of the reference's own double formula, see above
+SWEPT = ["sig", "tanh", "silu", "gelu", "softplus", "gatu", "gaus", "selu", "exp"]
+
+
+def sweep_points() -> np.ndarray:
+    rng = np.random.default_rng(2026)
+    parts = []
+    for e in range(-30, 8):                                   # 38 binades x 2 signs x 140 000 points
+        mag = np.float32(2.0) ** e * (1 + rng.random(140_000, dtype=np.float32))
+        parts += [mag, -mag]
+    dense = lambda lo, hi, n: (lo + (hi - lo) * rng.random(n)).astype(np.float32)
+    sw = dense(0.12, 0.13, 1 << 20)                           # the series switch of tanh, both signs
+    parts += [sw, -sw, np.float32(0.125) + np.arange(-2048, 2048, dtype=np.float32) * np.float32(2.0 ** -27)]
+    for lo, hi in ((8.3, 9.2), (16.0, 18.0), (86.0, 90.0), (100.0, 105.0)):   # tanh -> 1, sig -> 1, exp(-x) underflows, leaves the subnormals
+        s = dense(lo, hi, 1 << 19)
+        parts += [s, -s]
+    specials = np.array([0.0, -0.0, 1e-38, -1e-38, 1e-45, 88.72, -88.72, 87.33, -87.33, -103.97, 128.0, -128.0, 255.9, -255.9], dtype=np.float32)
+    return np.concatenate(parts + [specials]).astype(np.float32)
+
+
+def test_f32_exp_based_activations_dense_sweep(device, orc):
+    x = sweep_points()
+    n = x.size
+    assert n >= 1 << 24, n
+    cfg = orc.dense_cfg([n])
+    tx = Tensor.of(np.float32, (n,), x).to(device)
+    out = Tensor._on_device(device, np.float32, (n,))
+    report = []
+    for name in SWEPT:
+        for d in (-1, 0):
+            print(f"[case] sweep {name} d={d} over {n} points", flush=True)
+            device.launch_activation(name, d, out, tx)
+            got = out.getData().astype(np.float64)
+            with np.errstate(all="ignore"):
+                want32 = orc.activation(name, d, np.zeros(n, dtype=np.float32), cfg, x, cfg, workers=16)
+            want = want32.astype(np.float64)
+            finite = np.isfinite(want)
+            assert (np.isnan(got) == np.isnan(want)).all(), f"{name} d={d}: NaNs differ"
+            inf = np.isinf(want)
+            assert (got[inf] == want[inf]).all(), f"{name} d={d}: infinities differ"
+            err = np.abs(got[finite] - want[finite])
+            atol = QUANTUM.get(name, ATOL) if d < 0 else ATOL
+            bound = RTOL * np.abs(want[finite]) + atol
+            bad = err > bound
+            with np.errstate(all="ignore"):
+                rel = np.where(np.abs(want[finite]) > 1e5 * atol, err / np.abs(want[finite]), 0.0)
+            worst = int(np.argmax(rel))
+            xs = x[finite]
+            report.append((name, d, float(rel[worst]), float(xs[worst])))
+            print(f"[sweep] {name:9s} d={d:2d} worst relative error {rel[worst]:.3e} at x = {xs[worst]!r}", flush=True)
+            assert not bad.any(), (f"{name} d={d}: {int(bad.sum())} of {n} outside rtol {RTOL}; first at x = {xs[np.flatnonzero(bad)[0]]!r}: "
+                                   f"got {got[finite][np.flatnonzero(bad)[0]]!r}, want {want[finite][np.flatnonzero(bad)[0]]!r}")
+    device.free(tx); device.free(out)
+    print("[sweep] summary: " + "; ".join(f"{n_} d={d} {r:.2e}" for n_, d, r, _ in report), flush=True)
+
+
+def test_config3_single_kernels_full_size(device, orc):
+    """The four kernels the reference runs for tanh(sig(a)*b+c), each alone on 2^26 elements: sig and tanh within 1e-5
+    of the oracle element by element, multiply and add bit for bit."""
+    n = 1 << 26
+    rng = np.random.default_rng(33)
+    a = rng.standard_normal(n).astype(np.float32); b = rng.standard_normal(n).astype(np.float32)
+    cfg = orc.dense_cfg([n])
+    ta = Tensor.of(np.float32, (n,), a).to(device); tb = Tensor.of(np.float32, (n,), b).to(device)
+    out = Tensor._on_device(device, np.float32, (n,))
+    for name in ("sig", "tanh"):
+        print(f"[case] full-size {name}", flush=True)
+        device.launch_activation(name, -1, out, ta)
+        got = out.getData().astype(np.float64)
+        want = orc.activation(name, -1, np.zeros(n, dtype=np.float32), cfg, a, cfg, workers=16).astype(np.float64)
+        err = np.abs(got - want)
+        assert (err <= RTOL * np.abs(want) + ATOL).all(), f"{name}: worst relative error {np.max(err / np.abs(want)):.3e}"
+        print(f"[sweep] {name} over 2^26 N(0,1) values: worst relative error {np.max(err / np.maximum(np.abs(want), 1e-300)):.3e}", flush=True)
+    for op in ("multiply", "add"):
+        print(f"[case] full-size {op}", flush=True)
+        device.launch_elementwise(op, -1, out, ta, tb)
+        want = orc.elementwise(op, -1, np.zeros(n, dtype=np.float32), cfg, a, cfg, b, cfg, workers=16)
+        assert out.getData().tobytes() == want.tobytes(), op
+    for t in (ta, tb, out):
+        device.free(t)
