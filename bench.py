@@ -124,7 +124,7 @@ def main():
               "exchange), run it with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
-    from neureka_amd import Function, HipDevice, Tensor, _lib
+    from neureka_amd import Function, HipDevice, NDConfiguration, Tensor, _lib
 
     dev = HipDevice.get(0)
     rng = np.random.default_rng(2)
@@ -281,6 +281,18 @@ def main():
         hbm("activation_sig", 8 * n, dev.prepared_launch("activation", "sig", -1, o, srcs[0]))
         hbm("elementwise_add", 12 * n, dev.prepared_launch("elementwise", "add", -1, o, srcs[0], srcs[1]))
         hbm("elementwise_mul", 12 * n, dev.prepared_launch("elementwise", "multiply", -1, o, srcs[0], srcs[1]))
+        # the slow tails of the elementwise engine, measured so that they are on record: the derivative kernel of the fused
+        # chain (the full function table, one pass per block), general power (the device library's float pow: arithmetic,
+        # not memory, bounds it) and a view no fast path takes (every 16th column of every 2nd row: one element per thread)
+        dprog, dconsts = fused.derivative_program(0)
+        hbm("chain_derivative_by_input0", 16 * n, dev.prepared_launch("fused", dprog, dconsts, o, srcs))
+        pos = Tensor.of(f32, (n,), rng.uniform(0.1, 2.0, n).astype(f32)).to(dev)
+        hbm("power_tensor_exponent", 12 * n, dev.prepared_launch("elementwise", "power", -1, o, pos, srcs[1]))
+        dev.free(pos)
+        wide = Tensor(f32, NDConfiguration.ofShape((4096, 16384)), None); wide._set_data(srcs[0]._data, dev)
+        strided = wide[::2, ::16]
+        small = Tensor(f32, NDConfiguration.ofShape(strided.shape), None); small._set_data(o._data, dev)
+        hbm("tanh_of_every_16th_column", 8 * strided.size, dev.prepared_launch("activation", "tanh", -1, small, strided))
         # whole-tensor reductions of the same 2^26 elements (the operations that follow the hot path in training loops)
         one = Tensor._on_device(dev, f32, (1,))
         slot = dev.allocate(np.int32, 1)
@@ -295,7 +307,6 @@ def main():
         hbm("scalarization_int32_divide", 8 * n, dev.prepared_launch("scalarization_int", "divide", -1, i_out, i_src, 7))
         dev.free(i_src); dev.free(i_out)
         # permuted [4096,16384] views of row-major [16384,4096]
-        from neureka_amd import NDConfiguration
         pv = []
         for t in srcs:
             v = Tensor(f32, NDConfiguration.ofShape((16384, 4096)).newReshaped((1, 0)), None)

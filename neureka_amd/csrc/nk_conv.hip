@@ -1068,12 +1068,18 @@ static bool conv2d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& 
         if (window_on && n >= 65536 && (int64_t)H * W * (int64_t)sizeof(T) < ((int64_t)1 << 31) && B <= 65535) {
             constexpr int R = sizeof(T) == 4 ? 8 : 4;
             const int OH = H - (int)tap.shape[o] + 1, OW = W - (int)tap.shape[o + 1] + 1;
-            const dim3 grid((unsigned)((OW + WAVE_COLS - 1) / WAVE_COLS), (unsigned)(((OH + R - 1) / R + 3) / 4), (unsigned)B);
+            // strips of R rows per wavefront; half as many rows while that still leaves fewer than four wavefronts per
+            // SIMD (more wavefronts overlap their loads with the others' arithmetic: [2048,2048] x [5,5] 11.4 -> 10.4 us,
+            // [1024,1024] x [5,5] 7.1 -> 4.8 us; [4096,4096] x [3,3] keeps R rows, 22.9 against 24.8 us)
+            const int64_t waves_r = (int64_t)((OW + WAVE_COLS - 1) / WAVE_COLS) * ((OH + R - 1) / R) * B;
+            const int RR = (sizeof(T) == 4 && waves_r < 16 * (int64_t)dev->props.multiProcessorCount) ? 4 : R;
+            const dim3 grid((unsigned)((OW + WAVE_COLS - 1) / WAVE_COLS), (unsigned)(((OH + RR - 1) / RR + 3) / 4), (unsigned)B);
             const T* ip = a_img ? s1 : s2;
             const T* tp = a_img ? s2 : s1;
             if (grid.y <= 65535 && for_taps((int)tap.shape[o], (int)tap.shape[o + 1], [&](auto K) {
                     constexpr int KK = decltype(K)::value;
-                    hipLaunchKernelGGL((conv2d_window<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, H, W, ip, tp, out);
+                    if (RR == 4) hipLaunchKernelGGL((conv2d_window<T, KK, KK, 4>), grid, dim3(256), 0, dev->stream, H, W, ip, tp, out);
+                    else hipLaunchKernelGGL((conv2d_window<T, KK, KK, R>), grid, dim3(256), 0, dev->stream, H, W, ip, tp, out);
                 })) {
                 set_path("simple2d_window");
                 return true;
