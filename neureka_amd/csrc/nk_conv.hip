@@ -866,7 +866,7 @@ static int conv_channel_paths(Device* dev, int d, T* out, const Cfg& c0, const T
                               const T* s2, const Cfg& c2, bool* taken, bool one_plane = false) {
     constexpr bool F32 = sizeof(T) == 4;
     *taken = false;
-    static const long waves_per_cu = [] { const char* v = getenv("NK_CONV_WAVES_PER_CU"); return v && *v ? atol(v) : 8L; }();
+    constexpr long waves_per_cu = 8;
     const int64_t want_waves = (int64_t)dev->props.multiProcessorCount * waves_per_cu;
     for (const Cfg* c : {&c0, &c1, &c2})          // a plane is addressed with 32-bit byte offsets; grid y and z are 16-bit
         if ((int64_t)c->shape[1] * c->shape[2] * (int64_t)sizeof(T) >= (int64_t(1) << 31) || c->shape[0] > 65535 || c->shape[1] > 65535) return NK_OK;
@@ -1064,8 +1064,7 @@ static bool conv2d_direct_path(Device* dev, int d, int rank, T* out, const Cfg& 
     {
         // large images with square taps: the register-window kernel (same sums, same order); half the rows in f64
         const int H = (int)img.shape[o], W = (int)img.shape[o + 1];
-        static const bool window_on = [] { const char* v = getenv("NK_CONV2D_WINDOW"); return !(v && v[0] == '0'); }();
-        if (window_on && n >= 65536 && (int64_t)H * W * (int64_t)sizeof(T) < ((int64_t)1 << 31) && B <= 65535) {
+        if (n >= 65536 && (int64_t)H * W * (int64_t)sizeof(T) < ((int64_t)1 << 31) && B <= 65535) {
             constexpr int R = sizeof(T) == 4 ? 8 : 4;
             const int OH = H - (int)tap.shape[o] + 1, OW = W - (int)tap.shape[o + 1] + 1;
             // strips of R rows per wavefront; half as many rows while that still leaves fewer than four wavefronts per

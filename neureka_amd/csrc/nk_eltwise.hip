@@ -122,17 +122,10 @@ struct EltCall {
 static unsigned grid_for(Device* dev, uint64_t work_blocks) {
     // One block per tile: on this part a streaming kernel is fastest when the grid is far larger than the
     // machine (262144 blocks of 256 threads write at 6.3 TB/s, 4096 grid-striding blocks at 4.6 TB/s).
-    // NK_GRID_CAP (blocks per compute unit, 0 = no cap) exists for experiments.
-    static const long cap_per_cu = [] { const char* v = getenv("NK_GRID_CAP"); return v && *v ? atol(v) : 0L; }();
-    uint64_t cap = cap_per_cu > 0 ? (uint64_t)dev->props.multiProcessorCount * cap_per_cu : ((uint64_t)1 << 31) - 1;
+    (void)dev;
+    const uint64_t cap = ((uint64_t)1 << 31) - 1;
     if (work_blocks == 0) work_blocks = 1;
     return (unsigned)(work_blocks < cap ? work_blocks : cap);
-}
-
-static bool env_flag(const char* name, bool dflt) {
-    const char* v = getenv(name);
-    if (!v || !*v) return dflt;
-    return v[0] != '0';
 }
 
 template <typename T>
@@ -173,7 +166,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     // an output far larger than the caches: sources read once are loaded past them, re-used ones take the lean kernel
     const bool streaming = (uint64_t)c.n * sizeof(T) >= ((uint64_t)64 << 20);
     // the kernels with one unit per block: from 16 MiB of output on (measured: 32 MiB 8.8 -> 7.9 us; at 8 MiB no difference)
-    static const uint64_t lean_from = [] { const char* v = getenv("NK_LEAN_FROM_MIB"); return (uint64_t)(v && *v ? atoll(v) : 16) << 20; }();
+    constexpr uint64_t lean_from = (uint64_t)16 << 20;
     const bool large = (uint64_t)c.n * sizeof(T) >= lean_from;
 
     Canon cn;
@@ -192,10 +185,9 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     const int last = cn.rank - 1;
     bool rows_ok = cn.stride[0][last] == 1 && cn.rank - 1 <= ROWS_MAX_OUTER;
     // sources may also take every n-th column (a gather per element; the drain is still written in whole vectors)
-    static const bool strided_ok = env_flag("NK_ROWS_STRIDED_SOURCES", true);
     for (int j = 0; j < c.nsrc; j++)
         rows_ok = rows_ok && (cn.stride[j + 1][last] == 0 || cn.stride[j + 1][last] == 1 ||
-                              (strided_ok && cn.stride[j + 1][last] > 1 && cn.stride[j + 1][last] <= 8));
+                              (cn.stride[j + 1][last] > 1 && cn.stride[j + 1][last] <= 8));
     bool done = false;
 
     // the rows kernel keeps element offsets in 32 bits: every reachable offset must fit
@@ -216,7 +208,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // (length not a multiple of the vector) also runs on vectors: the last vector of a row is moved back so
         // that it ends with the row and overlaps its neighbour, whose elements are then computed and written twice
         // with the same values -- which is only the same thing when no source shares memory with the drain.
-        bool ragged = cn.shape[last] % VMAX != 0 && cn.shape[last] >= VMAX && env_flag("NK_RAGGED_VECTORS", true);
+        bool ragged = cn.shape[last] % VMAX != 0 && cn.shape[last] >= VMAX;
         if (ragged) {
             auto span = [&](int o, int64_t& lo, int64_t& hi) {
                 const int64_t ptr = o == 0 ? (int64_t)c.drn : (int64_t)c.src[o - 1];
@@ -245,7 +237,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         bool reused = false;                                // some source is read more than once (a broadcast)
         for (int j = 0; j < c.nsrc; j++)
             for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) reused = true;
-        bool once = streaming && env_flag("NK_STREAMING_LOADS", true) && !reused;
+        bool once = streaming && !reused;
         const bool deep = last > ROWS_FAST_OUTER;           // more outer axes than the tuned variants resolve: plain variants
         if (deep) once = false;
         A.nt_loads = once ? 1 : 0;
@@ -281,15 +273,12 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel
         // (sources that are constant along a row are handled by that kernel's vector variant only)
-        const bool loads_ok = A.simple_loads || (A.const_last != 0 && A.strided_last == 0 && vec && env_flag("NK_BINARY_ROW_CONSTANT", true));
+        const bool loads_ok = A.simple_loads || (A.const_last != 0 && A.strided_last == 0 && vec);
         if (loads_ok && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
             prog.op[1] == I_BIN && prog.src[1] == 1 && prog.arg[1] <= NK_OP_DIV) {
             plan.kind = PLAN_ROWS_BINARY;
             plan.binary_op = prog.arg[1];
-            if (vec) {
-                static const int env_passes = [] { const char* v = getenv("NK_BINARY_PASSES"); return v && *v ? atoi(v) : 8; }();
-                passes = (env_passes == 2 || env_passes == 4) && A.const_last == 0 && !deep ? env_passes : 8;
-            }
+            if (vec) passes = 8;
             plan.passes = passes;
         }
         plan.vec = vec;
@@ -303,7 +292,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             if (constant) A.pass_rows = 1;
             // measured at steady state: loading the constant source once gains 2..14 % when a row fills the block
             // (256 threads) and loses 4..14 % when a block covers several rows per pass
-            if (constant && env_flag("NK_HOIST", true) && vec && passes == 8 && !A.nt_loads && rpp == 1 && A.const_last == 0 && !deep &&
+            if (constant && vec && passes == 8 && !A.nt_loads && rpp == 1 && A.const_last == 0 && !deep &&
                 cn.shape[last - 1] % ((int64_t)passes * rpp) == 0)
                 plan.hoist = constant;
         }
@@ -311,19 +300,18 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         plan.grid = A.pass_rows ? (unsigned)(((row_groups + passes - 1) / passes) * A.chunks)
                                 : (unsigned)((row_groups * A.chunks + passes - 1) / passes);
         // large outputs of the binary kernel: one unit per block, non-temporal stores
-        static const int lean_mode = [] { const char* v = getenv("NK_BINARY_LEAN"); return v && *v ? atoi(v) : 1; }();
         // (only for a drain without gaps: the gain comes from the write front that moves through memory in order; a
         // drain that is a slice of a wider tensor measured 5 % slower this way)
         bool drain_dense = cn.stride[0][last] == 1;
         for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
-        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && lean_mode != 0 && reused) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && reused) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
         // ... and of a program that is one constant
         if (plan.kind == PLAN_ROWS && c.nsrc == 0 && prog.n == 1 && prog.op[0] == I_SET && prog.src[0] == SRC_CONST0 && funset == 0 &&
-            vec && large && drain_dense && !deep && lean_mode != 0) {
+            vec && large && drain_dense && !deep) {
             plan.lean_fill = true;
             plan.fill_value = prog.consts[0];
             plan.grid = (unsigned)(row_groups * A.chunks);
@@ -350,7 +338,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         if (ok && pax >= 0) {
             TileArgs& A = plan.tile;
             A.rank = cn.rank; A.nsrc = c.nsrc; A.pax = pax; A.turned = turned;
-            bool once = streaming && env_flag("NK_STREAMING_LOADS", true);
+            bool once = streaming;
             for (int j = 0; j < c.nsrc && once; j++)
                 for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) once = false;
             A.nt_loads = once ? 1 : 0;
@@ -368,10 +356,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             if (nb < ((uint64_t)1 << 31)) {
                 A.n_blocks = (unsigned)nb;
                 // groups of 4 (pax) x 8 (innermost) tiles: 1 KiB runs on both sides (f32); measured optimum of the sweep
-                static const int env_group = [] { const char* v = getenv("NK_TILE_GROUP_LOG2"); return v && *v ? atoi(v) : 3; }();
-                static const int env_group_p = [] { const char* v = getenv("NK_TILE_GROUP_P_LOG2"); return v && *v ? atoi(v) : 2; }();
-                int gl = env_group < 0 ? 0 : (env_group > 6 ? 6 : env_group);
-                int gp = env_group_p < 0 ? 0 : (env_group_p > 6 ? 6 : env_group_p);
+                int gl = 3, gp = 2;
                 while (gl > 0 && A.tiles_l % (1u << gl)) gl--;
                 while (gp > 0 && A.tiles_p % (1u << gp)) gp--;
                 A.group_log2 = gl; A.group_p_log2 = gp;
@@ -385,10 +370,9 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
                 // The hardware deals consecutive block ids round-robin to the 8 XCDs, each with its own L2.  XCD x takes the
                 // x-th eighth of the tile order, so the tiles one L2 serves at a time are neighbours in both directions:
                 // its reads (along pax) and its writes (along the innermost axis) add up to long runs
-                static const bool xcd_regions = env_flag("NK_TILE_XCD_REGIONS", true);
                 // (with fewer than 8 tiles in a plane the order is ruled by the outer axes and an eighth per XCD is an eighth of
                 // the output per XCD, which a write stream does not like: measured 5.5 -> 4.7 TB/s on a fully reversed rank-4 view)
-                A.xcd_regions = xcd_regions && nb % 8 == 0 && (uint64_t)A.tiles_p * A.tiles_l >= 8;
+                A.xcd_regions = nb % 8 == 0 && (uint64_t)A.tiles_p * A.tiles_l >= 8;
                 set_path("tile_transpose");
                 done = true;
             }

@@ -544,11 +544,10 @@ static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* 
 // the k range is then cut into parts until there are about two blocks per unit, each part at least four
 // k-slices long; the parts are written to the device workspace and added in order by a second launch.
 static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes) {
-    static const bool on = [] { const char* v = getenv("NK_MATMUL_SPLIT_K"); return !(v && v[0] == '0'); }();
     const int tiles = g.tiles_m * g.tiles_n, cus = dev->props.multiProcessorCount;
     const int slices = (g.K + slice - 1) / slice;
     g.splits = 1; g.split_slices = slices;
-    if (!on || tiles >= cus || slices < 8) return 1;
+    if (tiles >= cus || slices < 8) return 1;
     int parts = (2 * cus + tiles - 1) / tiles;
     if (parts > slices / 4) parts = slices / 4;
     if (parts > 64) parts = 64;
@@ -577,7 +576,7 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
 }
 
 static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
-    static const int64_t mfma_from = [] { const char* v = getenv("NK_MFMA_EDGE_FROM"); return v && *v ? atoll(v) : (int64_t)1 << 24; }();
+    constexpr int64_t mfma_from = (int64_t)1 << 24;
     MfmaArgs g{};
     g.M = (int)M; g.K = (int)K; g.N = (int)N;
     g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
@@ -612,12 +611,11 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
             if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
             else if (whole_tiles) {
                 // more tiles than blocks that fit the machine at one time: the blocks stay and walk the tiles
-                static const int stream_mode = [] { const char* v = getenv("NK_MATMUL_STREAM"); return v && *v ? atoi(v) : 1; }();
                 const unsigned resident = 2u * (unsigned)dev->props.multiProcessorCount;
                 const unsigned tiles = (unsigned)(g.tiles_m * g.tiles_n);
                 // (pays while a tile has few k-slices, i.e. while its first fetch and its write-back weigh: measured
                 // +4 % at 8 slices, +1 % at 16, -1 % at 128)
-                if (stream_mode && g.K / BK <= 16 && tiles >= 2 * resident && tiles % 8 == 0 && resident % 8 == 0) {
+                if (g.K / BK <= 16 && tiles >= 2 * resident && tiles % 8 == 0 && resident % 8 == 0) {
                     hipLaunchKernelGGL(matmul_mfma_stream_kernel, dim3(resident), dim3(256), 0, dev->stream, g, Ap, Bp, Cp);
                     streamed = true;
                 }

@@ -302,11 +302,6 @@ __global__ __launch_bounds__(256) void broadcast_bwd_segments_kernel(Cfg c0, int
 
 using namespace nk;
 
-static bool env_vec_ok() {
-    static const bool on = [] { const char* v = getenv("NK_BWD_VECTOR"); return !(v && v[0] == '0'); }();
-    return on;
-}
-
 extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_buf drn, const int32_t* drn_cfg,
                             nk_buf a, const int32_t* a_cfg, nk_buf b, const int32_t* b_cfg, int64_t n) {
     NK_REQUIRE(op_id >= NK_OP_ADD && op_id <= NK_OP_POW, "nk_broadcast: unknown operator id %d", op_id);
@@ -353,16 +348,14 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
     constexpr int VB = 16;
     const int V = VB / eb, last = rank - 1;
     const bool vec = A.c0.shape[last] % V == 0 && A.c0.imap[last] == 1 && (int64_t)A.c0.spread[last] * A.c0.strides[last] == 1 &&
-                     A.c0.shape[last] >= c1.shape[last] && A.keep2[last] == 1 && (A.keep1[last] == 1 || A.keep1[last] == 0) &&
-                     env_vec_ok();
+                     A.c0.shape[last] >= c1.shape[last] && A.keep2[last] == 1 && (A.keep1[last] == 1 || A.keep1[last] == 0);
     A.n_threads = (unsigned)(vec ? n / V : n);
     // few outputs with long sums, or the innermost axis reduced: the kernel that splits the sums (another order of
     // the same terms, see above); everything else keeps the reference's order bit for bit
     int64_t terms = 1;
     for (int k = 0; k < A.nred; k++) terms *= A.red_extent[k];
     const bool last_reduced = A.c0.shape[last] < c1.shape[last];
-    static const bool split_on = [] { const char* v = getenv("NK_BWD_SPLIT"); return !(v && v[0] == '0'); }();
-    if (split_on && terms < ((int64_t)1 << 31) && ((last_reduced && terms >= 512) || (terms >= 1024 && A.n_threads < 16384))) {
+    if (terms < ((int64_t)1 << 31) && ((last_reduced && terms >= 512) || (terms >= 1024 && A.n_threads < 16384))) {
         // innermost reduced axis in 16-byte pieces when it is contiguous in the error and contiguous or constant in src1
         int VT = 1;
         if (last_reduced) {
