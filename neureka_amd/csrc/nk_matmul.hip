@@ -185,30 +185,61 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     Frag f0, f1;
     load_global(kbase);
     store_lds(0);
+    load_global(kbase + (nk > 1 ? BK : 0));                // slice 1 waits in the staging registers
     __syncthreads();
     read_frag(f0, 0, 0);
+    // The order of issue inside a chunk is pinned with scheduling groups.  Left alone, the compiler sinks the LDS
+    // reads of chunk c + 1 behind the sixteen multiply-adds of chunk c (fewer live registers), and the matrix cores
+    // then sit out an LDS latency at the start of every chunk.  Pinned: the six reads follow the first three
+    // multiply-adds, global requests and LDS writes are dealt out one per multiply-add after them, so every memory
+    // instruction issues in the shadow of a multiply-add and has the rest of the chunk to complete.
+#define NK_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
+#define NK_DS_READ(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
+#define NK_DS_WRITE(n) __builtin_amdgcn_sched_group_barrier(0x200, n, 0)
+#define NK_VMEM_READ(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
+#define NK_FENCE __builtin_amdgcn_sched_barrier(0)
+#define NK_READS_FIRST NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2)
+#define NK_CHUNK_PLAIN NK_READS_FIRST; NK_MFMA(13); NK_FENCE
+#define NK_CHUNK_WITH(GROUP) NK_READS_FIRST; NK_MFMA(1); GROUP(1); NK_MFMA(1); GROUP(1); NK_MFMA(1); GROUP(1); NK_MFMA(1); GROUP(1); \
+                             NK_MFMA(1); GROUP(1); NK_MFMA(1); GROUP(1); NK_MFMA(1); GROUP(1); NK_MFMA(1); GROUP(1); NK_MFMA(5); NK_FENCE
+#define NK_CHUNK_WRITE_AND_REQUEST NK_READS_FIRST; NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); \
+                                   NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); \
+                                   NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); \
+                                   NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(5); NK_FENCE
+    NK_FENCE;
+    // Slice kt + 1 is written to LDS in the third chunk of slice kt from the staging registers, which are then free
+    // for the request of slice kt + 2: a request has a whole slice of multiply-adds to arrive.  (Past the last slice
+    // the request repeats the last one; nothing reads it.)
     for (int kt = 0; kt + 1 < nk; kt++) {                  // branch-free body; the last slice is peeled off below
         const int cur = kt & 1;
-        load_global(kbase + (kt + 1) * BK);
         read_frag(f1, cur, 1);
         mma(f0);
+        NK_CHUNK_PLAIN;
         read_frag(f0, cur, 2);
         mma(f1);
+        NK_CHUNK_PLAIN;
+        read_frag(f1, cur, 3);                             // (before the writes in program order: LDS accesses keep it)
         store_lds(cur ^ 1);
-        read_frag(f1, cur, 3);
+        load_global(kbase + (kt + 2 < nk ? kt + 2 : nk - 1) * BK);
         mma(f0);
+        NK_CHUNK_WRITE_AND_REQUEST;
         __syncthreads();
+        NK_FENCE;
         read_frag(f0, cur ^ 1, 0);
         mma(f1);
+        NK_CHUNK_PLAIN;
     }
     {
         const int cur = (nk - 1) & 1;
         read_frag(f1, cur, 1);
         mma(f0);
+        NK_CHUNK_PLAIN;
         read_frag(f0, cur, 2);
         mma(f1);
+        NK_CHUNK_PLAIN;
         read_frag(f1, cur, 3);
         mma(f0);
+        NK_CHUNK_PLAIN;
         mma(f1);
     }
 
@@ -613,9 +644,9 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
                 // more tiles than blocks that fit the machine at one time: the blocks stay and walk the tiles
                 const unsigned resident = 2u * (unsigned)dev->props.multiProcessorCount;
                 const unsigned tiles = (unsigned)(g.tiles_m * g.tiles_n);
-                // (pays while a tile has few k-slices, i.e. while its first fetch and its write-back weigh: measured
-                // +4 % at 8 slices, +1 % at 16, -1 % at 128)
-                if (g.K / BK <= 16 && tiles >= 2 * resident && tiles % 8 == 0 && resident % 8 == 0) {
+                // (pays while a tile has very few k-slices, i.e. while its first fetch and its write-back weigh: measured
+                // +3 % at 8 slices, -3 % at 16 against the tile kernel)
+                if (g.K / BK <= 8 && tiles >= 2 * resident && tiles % 8 == 0 && resident % 8 == 0) {
                     hipLaunchKernelGGL(matmul_mfma_stream_kernel, dim3(resident), dim3(256), 0, dev->stream, g, Ap, Bp, Cp);
                     streamed = true;
                 }
