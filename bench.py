@@ -328,13 +328,16 @@ def main():
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
             Cm = Tensor._on_device(dev, f32, (M, N))
-            flops(name, 2.0 * M * K * N, 4 * (M * K + K * N + M * N), dev.prepared_launch("matmul", True, M, K, N, A, B, Cm))
+            # what the registered implementation launches: C = A @ B (nk_matmul_set, as CLMatMul's kernel); the accumulating
+            # entry point (C += A @ B, the old C read as well) beside it
+            flops(name, 2.0 * M * K * N, 4 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm))
+            flops(name + "_accumulating", 2.0 * M * K * N, 4 * (M * K + K * N + 2 * M * N), dev.prepared_launch("matmul", True, M, K, N, A, B, Cm))
             for t in (A, B, Cm): dev.free(t)
         M = K = N = 4096
         A = Tensor.of(np.float64, (M, K), rng.uniform(-1, 1, M * K)).to(dev)
         B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)
         Cm = Tensor._on_device(dev, np.float64, (M, N))
-        flops("matmul_4096_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul", True, M, K, N, A, B, Cm), f64=True)
+        flops("matmul_4096_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm), f64=True)
         for t in (A, B, Cm): dev.free(t)
 
         # C1 and C5 convolutions

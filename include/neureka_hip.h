@@ -195,6 +195,14 @@ int nk_dot(nk_dev dev, int dtype, nk_buf a, nk_buf b, int64_t n, nk_buf out);
 int nk_matmul(nk_dev dev, int dtype, int layout, int64_t M, int64_t K, int64_t N,
               nk_buf A, nk_buf B, nk_buf C);
 
+/* simple_matMul as the OpenCL device runs it: J/backend/main/implementations/matmul/CLMatMul.java:35-52, whose kernel
+ * ends in `C[ n + m * N ] = acc` (:50).  C[M,N] = A[M,K] @ B[K,N]: the old contents of C are neither read nor
+ * kept, which saves their trip from memory (a third of the traffic of a product with a short inner dimension).
+ * On a zeroed C -- the only way the reference calls either (MatMulAlgorithm.java:74-85) -- the result equals nk_matmul's
+ * bit for bit.  Same arguments, limits and errors as nk_matmul. */
+int nk_matmul_set(nk_dev dev, int dtype, int layout, int64_t M, int64_t K, int64_t N,
+                  nk_buf A, nk_buf B, nk_buf C);
+
 /* Fused elementwise expression, the device side of Device.optimizedFunctionOf
  * (J/devices/Device.java:216-243; J/devices/opencl/utility/CLFunctionCompiler.java:101-199).
  * `program` is a postfix op-code sequence of `n_ops` int32 words evaluated per drain element on a

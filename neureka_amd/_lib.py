@@ -50,6 +50,7 @@ SYMBOLS = {
     "nk_broadcast": (_i32, [_u64, _i32, _i32, _i32, _i32, _u64, _cfg, _u64, _cfg, _u64, _cfg, _i64]),
     "nk_convolution": (_i32, [_u64, _i32, _i32, _i32, _u64, _cfg, _u64, _cfg, _u64, _cfg, _i64]),
     "nk_matmul": (_i32, [_u64, _i32, _i32, _i64, _i64, _i64, _u64, _u64, _u64]),
+    "nk_matmul_set": (_i32, [_u64, _i32, _i32, _i64, _i64, _i64, _u64, _u64, _u64]),
     "nk_scalarization_int": (_i32, [_u64, _i32, _i32, _i32, _i32, _u64, _cfg, _u64, _cfg, _i64, _i64]),
     "nk_sum": (_i32, [_u64, _i32, _u64, _i64, _u64]),
     "nk_sum_static": (_i32, [_u64, _i32, _u64, _i64, _u64]),

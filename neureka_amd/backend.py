@@ -575,7 +575,8 @@ def hip_convolution(call: ExecutionCall):
 
 
 def hip_matmul(call: ExecutionCall):
-    """CLMatMul / CPUMatMul (implementations/matmul/CPUMatMul.java:17-96): layout check, then the GEMM."""
+    """CLMatMul / CPUMatMul (implementations/matmul/CPUMatMul.java:17-96): layout check, then the product, written
+    over the drain as the OpenCL device's kernel does (CLMatMul.java:50; the drain arrives zeroed: MatMulAlgorithm.java:74-85)."""
     c, a, b = call.input(0), call.input(1), call.input(2)
     la, lb = a.ndc.getLayout(), b.ndc.getLayout()
     if not (la.isCompatible(lb) and la.isCompatible(c.ndc.getLayout()) and lb.isCompatible(c.ndc.getLayout())):
@@ -585,7 +586,7 @@ def hip_matmul(call: ExecutionCall):
     row_major = all(l in (Layout.ROW_MAJOR, Layout.SYMMETRIC) for l in (la, lb))
     if a.shape[1] != b.shape[0]:
         raise IllegalArgumentException(f"'A' matrix rows {a.shape[1]} did not match 'B' matrix columns {b.shape[0]}.")
-    call.device.launch_matmul(row_major, a.shape[0], a.shape[1], b.shape[1], a, b, c)
+    call.device.launch_matmul(row_major, a.shape[0], a.shape[1], b.shape[1], a, b, c, accumulate=False)
     return c
 
 

@@ -22,12 +22,12 @@
 namespace nk {
 
 template <typename T>
-__global__ __launch_bounds__(256) void matmul_simple_kernel(int M, int K, int N, const T* __restrict__ A,
+__global__ __launch_bounds__(256) void matmul_simple_kernel(int M, int K, int N, int overwrite, const T* __restrict__ A,
                                                             const T* __restrict__ B, T* __restrict__ C) {
     const int n = blockIdx.x * 64 + (threadIdx.x & 63);
     const int m = blockIdx.y * 4 + (threadIdx.x >> 6);
     if (m >= M || n >= N) return;
-    T acc = C[(int64_t)m * N + n];
+    T acc = overwrite ? T(0) : C[(int64_t)m * N + n];
     const T* a = A + (int64_t)m * K;
     for (int k = 0; k < K; k++) {
         T prod = a[k] * B[(int64_t)k * N + n];   // rounded product, then add: no contraction
@@ -49,6 +49,7 @@ struct MfmaArgs {
     int group_rows;      // tile rows per group of the block-id regrouping
     int splits;          // SPLIT kernels: parts the k range is cut into (grid = tiles * splits) ...
     int split_slices;    // ... and k-slices per part
+    int overwrite;       // C = A @ B instead of C += A @ B: the old values of C are not read
 };
 
 __device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int bid, int& tm, int& tn) {
@@ -268,12 +269,12 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
                 const float* add = &cs[r * C_PITCH + c_col];
                 float* dst = Cg + (int64_t)r * g.N + c_col;
 #pragma unroll
-                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = SPLIT ? add[e] : dst[e] + add[e];
+                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = (SPLIT || g.overwrite) ? add[e] : dst[e] + add[e];
             }
         }
         return;
     }
-    if (SPLIT) {
+    if (SPLIT || g.overwrite) {                            // the same for every block of a launch
 #pragma unroll
         for (int i = 0; i < 16; i++)
             *(f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col) = *(const f32x4*)(&cs[(c_row + 8 * i) * C_PITCH + c_col]);
@@ -294,6 +295,7 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
 // tile is fetched and written to the free LDS buffer during the last slice of the current one, so only the
 // block's very first slice is waited for.  The result leaves straight from the accumulators (32 lanes cover 128
 // contiguous bytes of a row of C), which needs neither LDS nor a barrier and so does not disturb the pipeline.
+template <bool OVERWRITE>
 __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, const float* __restrict__ A,
                                                                  const float* __restrict__ B, float* __restrict__ C) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS_AB];
@@ -389,10 +391,13 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
         const bool more = next < n_tiles;                  // the same for the whole block
         int nm = tm, nn = tn;
         if (more) { tile_of_block(g, next, nm, nn); load_global(nm, nn, 0); }
-        // C += the tile: accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4, column l32.  Addresses are a
-        // wave-uniform part (tile, sub-tile, accumulator: scalar registers) plus one 32-bit offset per lane.  The old
-        // values of the upper two sub-tiles are requested before the last multiply-adds, those of the lower two
-        // while the upper two are stored.
+        // C (+)= the tile: accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4, column l32, so a store
+        // instruction writes 128 contiguous bytes of two rows.  (With the operands of the multiply-adds swapped a lane
+        // would own four neighbouring columns of one row and C could move 16 bytes per lane, 32 bytes per row and
+        // instruction: measured slower, 76.3 against 72.8 us for 65536 x 256 x 256.)  Addresses are a wave-uniform part
+        // (tile, sub-tile, accumulator: scalar registers) plus one 32-bit offset per lane.  Accumulating, the old values
+        // of the upper two sub-tiles are requested before the last multiply-adds, those of the lower two while the
+        // upper two are stored.
         float* const Cg = C + (int64_t)tm * BM * g.N + tn * BN;
         const unsigned lane_off = (unsigned)((wm + 4 * h) * g.N + wn + l32);
         float old[2][16];
@@ -400,13 +405,13 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) old[j][v] = (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off];
+                for (int v = 0; v < 16; v++) old[j][v] = OVERWRITE ? 0.0f : (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off];
         };
         auto store_new = [&](int i) {
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off] = old[j][v] + acc[i][j][v];
+                for (int v = 0; v < 16; v++) (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off] = OVERWRITE ? acc[i][j][v] : old[j][v] + acc[i][j][v];
         };
         fetch_old(0);
         read_frag(f1, cur, 1);
@@ -429,14 +434,14 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
     }
 }
 
-// C[i] += part_0[i] + part_1[i] + ... in that order (the parts of a SPLIT product)
+// C[i] += (or, overwriting, =) part_0[i] + part_1[i] + ... in that order (the parts of a SPLIT product)
 template <typename T>
-__global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int parts, const T* __restrict__ P, T* __restrict__ C) {
+__global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int parts, int overwrite, const T* __restrict__ P, T* __restrict__ C) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     T s = P[i];
     for (int k = 1; k < parts; k++) s = s + P[(int64_t)k * n + i];
-    C[i] = C[i] + s;
+    C[i] = overwrite ? s : C[i] + s;
 }
 
 // ---- f64 on the matrix cores ----------------------------------------------------------------------------------
@@ -556,17 +561,17 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
                 const int row = wm + 16 * i + 4 * v + q, col = wn + 16 * j + l16;
                 if (!EDGE || (row < rows && col < cols)) {
                     double* p = Cg + (int64_t)row * g.N + col;
-                    *p = SPLIT ? acc[i][j][v] : *p + acc[i][j][v];
+                    *p = (SPLIT || g.overwrite) ? acc[i][j][v] : *p + acc[i][j][v];
                 }
             }
 }
 
 template <typename T>
-static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, const T* A, const T* B, T* C) {
+static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, bool overwrite, const T* A, const T* B, T* C) {
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4));
     NK_REQUIRE(grid.y <= 65535u * 1024u, "nk_matmul: M too large");
     set_path("simple");
-    hipLaunchKernelGGL(matmul_simple_kernel<T>, grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, A, B, C);
+    hipLaunchKernelGGL(matmul_simple_kernel<T>, grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, overwrite ? 1 : 0, A, B, C);
     NK_HIP(hipGetLastError());
     return NK_OK;
 }
@@ -598,7 +603,7 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
         const int64_t mn = (int64_t)g.M * g.N;
         if (int e = workspace(dev, (uint64_t)g.splits * mn * sizeof(T), &ws)) return e;
         launch(true, dim3((unsigned)(tiles * g.splits)), (T*)ws);
-        hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, dev->stream, mn, g.splits, (const T*)ws, Cp);
+        hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, dev->stream, mn, g.splits, g.overwrite, (const T*)ws, Cp);
     } else {
         launch(false, dim3((unsigned)tiles), (T*)nullptr);
     }
@@ -606,12 +611,13 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
     return NK_OK;
 }
 
-static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
     constexpr int64_t mfma_from = (int64_t)1 << 24;
     MfmaArgs g{};
     g.M = (int)M; g.K = (int)K; g.N = (int)N;
     g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
     g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
+    g.overwrite = overwrite ? 1 : 0;
     if (dtype == NK_F64) {
         // from 2^24 multiply-adds on the matrix cores take over (sums re-ordered, within 1e-12 of the reference);
         // smaller products keep the reference's summation order bit for bit
@@ -628,7 +634,7 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
             set_path(whole ? (g.splits > 1 ? "mfma_f64_split" : "mfma_f64") : (g.splits > 1 ? "mfma_f64_edge_split" : "mfma_f64_edge"));
             return rc;
         }
-        return launch_simple<double>(dev, M, K, N, (const double*)A, (const double*)B, (double*)C);
+        return launch_simple<double>(dev, M, K, N, overwrite, (const double*)A, (const double*)B, (double*)C);
     }
     const bool aligned = (A % 16 == 0) && (B % 16 == 0) && (C % 16 == 0);
     const bool whole_tiles = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
@@ -647,7 +653,8 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
                 // (pays while a tile has very few k-slices, i.e. while its first fetch and its write-back weigh: measured
                 // +3 % at 8 slices, -3 % at 16 against the tile kernel)
                 if (g.K / BK <= 8 && tiles >= 2 * resident && tiles % 8 == 0 && resident % 8 == 0) {
-                    hipLaunchKernelGGL(matmul_mfma_stream_kernel, dim3(resident), dim3(256), 0, dev->stream, g, Ap, Bp, Cp);
+                    if (overwrite) hipLaunchKernelGGL(matmul_mfma_stream_kernel<true>, dim3(resident), dim3(256), 0, dev->stream, g, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL(matmul_mfma_stream_kernel<false>, dim3(resident), dim3(256), 0, dev->stream, g, Ap, Bp, Cp);
                     streamed = true;
                 }
                 else
@@ -659,14 +666,14 @@ static int matmul_rm(Device* dev, int dtype, int64_t M, int64_t K, int64_t N, nk
         set_path(streamed ? "mfma_stream" : whole_tiles ? (g.splits > 1 ? "mfma_split" : "mfma") : (g.splits > 1 ? "mfma_edge_split" : "mfma_edge"));
         return rc;
     }
-    return launch_simple<float>(dev, M, K, N, (const float*)A, (const float*)B, (float*)C);
+    return launch_simple<float>(dev, M, K, N, overwrite, (const float*)A, (const float*)B, (float*)C);
 }
 
 }  // namespace nk
 
 using namespace nk;
 
-extern "C" int nk_matmul(nk_dev h, int dtype, int layout, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+static int matmul_entry(nk_dev h, bool overwrite, int dtype, int layout, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
     NK_DEVICE(dev, h);
     NK_REQUIRE(dtype == NK_F32 || dtype == NK_F64, "nk_matmul: unknown dtype %d", dtype);
     NK_REQUIRE(layout == NK_LAYOUT_ROW_MAJOR || layout == NK_LAYOUT_COLUMN_MAJOR, "nk_matmul: unknown layout %d", layout);
@@ -677,7 +684,15 @@ extern "C" int nk_matmul(nk_dev h, int dtype, int layout, int64_t M, int64_t K, 
     if (int e = check_range(dev, "nk_matmul(A)", A, 0, (uint64_t)(M * K) * eb)) return e;
     if (int e = check_range(dev, "nk_matmul(B)", B, 0, (uint64_t)(K * N) * eb)) return e;
     if (int e = check_range(dev, "nk_matmul(C)", C, 0, (uint64_t)(M * N) * eb)) return e;
-    if (layout == NK_LAYOUT_ROW_MAJOR) return matmul_rm(dev, dtype, M, K, N, A, B, C);
+    if (layout == NK_LAYOUT_ROW_MAJOR) return matmul_rm(dev, dtype, overwrite, M, K, N, A, B, C);
     // column-major data of X[r,c] is the row-major data of X^T[c,r]:  C^T[N,M] += B^T[N,K] @ A^T[K,M]
-    return matmul_rm(dev, dtype, N, K, M, B, A, C);
+    return matmul_rm(dev, dtype, overwrite, N, K, M, B, A, C);
+}
+
+extern "C" int nk_matmul(nk_dev h, int dtype, int layout, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+    return matmul_entry(h, false, dtype, layout, M, K, N, A, B, C);
+}
+
+extern "C" int nk_matmul_set(nk_dev h, int dtype, int layout, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+    return matmul_entry(h, true, dtype, layout, M, K, N, A, B, C);
 }

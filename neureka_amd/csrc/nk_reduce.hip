@@ -91,34 +91,37 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
         int r[NK_MAX_RANK];
         for (int k = 0; k < NK_MAX_RANK; k++) r[k] = 0;
         for (;;) {
-            // the loads of the next UNROLL terms are issued before the current ones are added, so a wavefront
-            // always has requests in flight; the order of the additions is the reference's
-            int j = 0;
+            // the loads of the next UNROLL terms are requested before the current ones are added, so a wavefront
+            // always has requests in flight; the order of the additions is the reference's.  Two sets of registers
+            // take turns (no copies), and the offsets of the next term to request move by additions only.
+            int64_t q1 = o1, q2 = o2;
+            auto request = [&](T (&a)[UNROLL][V], T (&b)[UNROLL][V]) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++) { load1(q1, a[u]); load2(q2, b[u]); q1 += st1; q2 += st2; }
+            };
+            auto consume = [&](const T (&a)[UNROLL][V], const T (&b)[UNROLL][V]) {
+#pragma unroll
+                for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+                    for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[u][v], b[u][v]);
+            };
             const int batches = n0 / UNROLL;
             if (batches > 0) {
-                T a[UNROLL][V], b[UNROLL][V], an[UNROLL][V], bn[UNROLL][V];
-#pragma unroll
-                for (int u = 0; u < UNROLL; u++) { load1(o1 + u * st1, a[u]); load2(o2 + u * st2, b[u]); }
-                for (int bi = 0; bi < batches; bi++) {
-                    if (bi + 1 < batches) {
-                        const int64_t jn = (int64_t)(bi + 1) * UNROLL;
-#pragma unroll
-                        for (int u = 0; u < UNROLL; u++) { load1(o1 + (jn + u) * st1, an[u]); load2(o2 + (jn + u) * st2, bn[u]); }
-                    }
-#pragma unroll
-                    for (int u = 0; u < UNROLL; u++)
-#pragma unroll
-                        for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[u][v], b[u][v]);
-#pragma unroll
-                    for (int u = 0; u < UNROLL; u++)
-#pragma unroll
-                        for (int v = 0; v < V; v++) { a[u][v] = an[u][v]; b[u][v] = bn[u][v]; }
+                T a0[UNROLL][V], b0[UNROLL][V], a1[UNROLL][V], b1[UNROLL][V];
+                request(a0, b0);
+                int bi = 0;
+                for (; bi + 2 <= batches; bi += 2) {
+                    request(a1, b1);
+                    consume(a0, b0);
+                    if (bi + 2 < batches) request(a0, b0);
+                    consume(a1, b1);
                 }
-                j = batches * UNROLL;
+                if (bi < batches) consume(a0, b0);
             }
-            for (; j < n0; j++) {
+            for (int j = batches * UNROLL; j < n0; j++) {
                 T a[V], b[V];
-                load1(o1 + j * st1, a); load2(o2 + j * st2, b);
+                load1(q1, a); load2(q2, b);
+                q1 += st1; q2 += st2;
 #pragma unroll
                 for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[v], b[v]);
             }
@@ -162,15 +165,20 @@ struct BwdSplitArgs {
     unsigned terms, seg_terms;           // term units (VT terms each) per drain element and (host side) per segment
     int segments;
     int splat1;                          // VT > 1: src1 does not move along the innermost reduced axis
+    int contiguous;                      // segment s owns the term units [s * seg_terms, (s + 1) * seg_terms) instead of every
+                                         // segments-th group of TL: chosen when a block's step covers a contiguous piece of
+                                         // memory, so that every block walks its own contiguous stretch front to back
 };
 
-template <typename T, int G, int OT, bool ROWS, int VW, bool SPLAT = false>
+template <typename T, int G, int OT, bool ROWS, int VW, bool SPLAT = false, bool FLAT = false>
 __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A, BwdSplitArgs S, T* __restrict__ drn, T* __restrict__ partial,
                                                                   const T* __restrict__ s1, const T* __restrict__ s2) {
     // VW: width of the 16-byte accesses -- ROWS: VW neighbouring terms of one drain element per load;
     // otherwise VW neighbouring drain elements per thread
     constexpr int TL = 256 / OT;                                 // term lanes per drain element (group)
-    constexpr int U = 4;                                         // loads in flight per lane
+    // FLAT: the reduced axes nest in both sources and were merged into one by the host, so a lane's offsets move by a
+    // constant from term to term (no carries) -- the carry chain below costs about 40 vector instructions per load
+    constexpr int U = FLAT ? 8 : 4;                              // loads in flight per lane
     constexpr int VA = SPLAT ? 1 : VW;                           // values kept per term of src1: one serves all VW when it
                                                                  // does not move along the vector (a template parameter: a
                                                                  // run-time test in the term loop costs a quarter of the rate)
@@ -188,8 +196,11 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
     int64_t o1 = A.base1, o2 = A.base2;
     for (int k = 0; k < A.rank; k++) { o1 += o[k] * A.keep1[k]; o2 += o[k] * A.keep2[k]; }
     // the segments interleave: segment s takes the term units s * TL + tl, then those segments * TL further on, so
-    // that the blocks running at one time read one window of memory together
-    const unsigned first = seg * TL, stride = (unsigned)S.segments * TL, end = S.terms;
+    // that the blocks running at one time read one window of memory together -- or, `contiguous`, each its own stretch
+    const unsigned first = S.contiguous ? seg * S.seg_terms : seg * TL;
+    const unsigned stride = S.contiguous ? (unsigned)TL : (unsigned)S.segments * TL;
+    const unsigned seg_end = first + S.seg_terms;
+    const unsigned end = S.contiguous && seg_end < S.terms ? seg_end : S.terms;
     // mixed-radix position of the lane's first term unit and of its step, last reduced axis fastest; the two
     // offsets follow it by additions only: a step adds the offset of that many units, a carry out of axis k takes
     // the axis back to its start and moves axis k - 1 on by one (no multiplication in the term loop)
@@ -211,6 +222,7 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
     auto advance = [&]() {
         int carry = 0;
         a1 += delta1; a2 += delta2;
+        if constexpr (FLAT) return;
         for (int k = A.nred - 1; k >= 0; k--) {
             idx[k] += step[k] + carry;
             carry = idx[k] >= A.red_extent[k];
@@ -367,17 +379,32 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         // lanes per drain element: by the length of the sums when the innermost axis is reduced; otherwise more lanes
         // the fewer drain elements there are, so that the blocks of at most 256 segments still fill the machine
         const int64_t out_threads = n / VO;
-        const int TL = last_reduced ? (units >= 2048 ? 256 : (units >= 512 ? 64 : 16)) : (out_threads >= 1024 ? 4 : 16);
+        // (a drain that is one row of 128 threads gets two rows per block: the block then reads whole rows)
+        const int TL = last_reduced ? (units >= 2048 ? 256 : (units >= 512 ? 64 : 16)) : (out_threads >= 1024 ? 4 : (out_threads == 128 ? 2 : 16));
         const int OT = 256 / TL;
         BwdSplitArgs S{};
         S.n_out = (unsigned)n; S.terms = (unsigned)units;
         S.splat1 = last_reduced ? (VT > 1 && A.red1[A.nred - 1] == 0) : (A.keep1[last] == 0);
         if (VT > 1) { A.red_extent[A.nred - 1] /= VT; A.red1[A.nred - 1] *= VT; A.red2[A.nred - 1] *= VT; }
+        // neighbouring reduced axes that nest in both sources (the slower one's stride is the faster one's whole
+        // length) are one axis to the term enumeration, which runs last axis fastest
+        for (int k = A.nred - 1; k > 0; k--) {
+            if (A.red1[k - 1] == (int64_t)A.red_extent[k] * A.red1[k] && A.red2[k - 1] == (int64_t)A.red_extent[k] * A.red2[k] &&
+                (int64_t)A.red_extent[k - 1] * A.red_extent[k] < ((int64_t)1 << 31)) {
+                A.red_extent[k - 1] *= A.red_extent[k]; A.red1[k - 1] = A.red1[k]; A.red2[k - 1] = A.red2[k];
+                for (int m = k; m + 1 < A.nred; m++) { A.red_extent[m] = A.red_extent[m + 1]; A.red1[m] = A.red1[m + 1]; A.red2[m] = A.red2[m + 1]; }
+                A.nred--;
+            }
+        }
+        const bool flat = A.nred == 1;
+        // a step of the block is one contiguous piece of the error when its lanes take neighbouring 16-byte units of a
+        // contiguous reduced axis (256 of them: 4 KiB), or when the block covers whole rows that follow each other
         S.out_blocks = (unsigned)((n / VO + OT - 1) / OT);
+        S.contiguous = flat && (last_reduced ? (TL == 256 && VT > 1) : (S.out_blocks == 1 && VO > 1 && A.red2[0] == n));
         int64_t segs = (2048 + S.out_blocks - 1) / S.out_blocks;                  // enough blocks to fill the machine ...
         const int64_t most = units / (TL * 8) > 0 ? units / (TL * 8) : 1;         // ... with at least 8 term units per lane
         if (segs > most) segs = most;
-        if (segs > 256) segs = 256;
+        if (segs > (S.contiguous ? 2048 : 256)) segs = S.contiguous ? 2048 : 256;
         if (segs < 1) segs = 1;
         S.seg_terms = (unsigned)((units + segs - 1) / segs);
         S.segments = (int)((units + S.seg_terms - 1) / S.seg_terms);
@@ -396,16 +423,21 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                 if (!last_reduced) {
                     auto keep = [&](auto ot, auto vw) {
                         constexpr int O = decltype(ot)::value, W = decltype(vw)::value;
-                        if (W > 1 && S.splat1) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, O, false, W, true>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
-                        else hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, O, false, W, false>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        auto run = [&](auto splat, auto flat_tag) {
+                            hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, O, false, W, decltype(splat)::value, decltype(flat_tag)::value>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        };
+                        if (W > 1 && S.splat1) { if (flat) run(std::true_type{}, std::true_type{}); else run(std::true_type{}, std::false_type{}); }
+                        else { if (flat) run(std::false_type{}, std::true_type{}); else run(std::false_type{}, std::false_type{}); }
                     };
                     using one = std::integral_constant<int, 1>; using wide = std::integral_constant<int, VM>;
-                    if (OT == 64) { if (VO > 1) keep(std::integral_constant<int, 64>{}, wide{}); else keep(std::integral_constant<int, 64>{}, one{}); }
+                    if (OT == 128) { if (VO > 1) keep(std::integral_constant<int, 128>{}, wide{}); else keep(std::integral_constant<int, 128>{}, one{}); }
+                    else if (OT == 64) { if (VO > 1) keep(std::integral_constant<int, 64>{}, wide{}); else keep(std::integral_constant<int, 64>{}, one{}); }
                     else { if (VO > 1) keep(std::integral_constant<int, 16>{}, wide{}); else keep(std::integral_constant<int, 16>{}, one{}); }
                 }
                 else {
                     auto rows = [&](auto ot, auto vw, auto splat) {
-                        hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        if (flat) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value, true>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        else      hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value, false>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                     };
                     auto lanes = [&](auto ot) {
                         if (VT > 1 && S.splat1) rows(ot, std::integral_constant<int, VM>{}, std::true_type{});

@@ -53,6 +53,7 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
         pcol[k] = (p % PPR) * VEC;
         voff[k] = (unsigned)((prow[k] * RTS + pcol[k]) * sizeof(T));
     }
+    // one chunk ahead (two in flight measured slower: 47.1 against 45.1 us for the sum of 2^26 floats)
     u32x4 cur[LOADS], cur2[LOADS];
     constexpr int NON_TEMPORAL = 2;                 // cache policy of the loads: every element is read exactly once
     auto request = [&](int c) {
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     // next level; one thread each reduces them front to back out of LDS and only those results are written.
     constexpr bool INDEXED = MODE == STAT_MIN || MODE == STAT_MAX;
     constexpr int NEXT = 256 / RTS;                  // next-level tiles per block
-    __shared__ T level_val[256];
+    __shared__ __attribute__((aligned(16))) T level_val[256];
     __shared__ int level_idx[INDEXED ? 256 : 1];
     level_val[threadIdx.x] = value;
     if (INDEXED && limit > 0) {
@@ -121,13 +122,29 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
             const int count = results - first < RTS ? (int)(results - first) : RTS;
             T v = T(0);
             int at = 0;
-            for (int i = 0; i < count; i++) {
-                const T x = level_val[threadIdx.x * RTS + i];
+            auto take = [&](T x, int i) {
                 if (!INDEXED) v = v + x;
                 else {
                     const bool better = MODE == STAT_MIN ? x < v : x > v;
                     if (i == 0 || better) { v = x; at = i; }
                 }
+            };
+            if (count == RTS) {
+                // a whole tile: sixteen values per trip through 16-byte LDS reads that are all requested before the
+                // first is used (one value per trip would wait out an LDS latency RTS times, at the end of every block)
+                constexpr int STEP = 16;
+                typedef T Vec __attribute__((ext_vector_type(VEC)));
+                for (int i0 = 0; i0 < RTS; i0 += STEP) {
+                    Vec q[STEP / VEC];
+#pragma unroll
+                    for (int k = 0; k < STEP / VEC; k++) q[k] = *(const Vec*)(&level_val[threadIdx.x * RTS + i0 + k * VEC]);
+#pragma unroll
+                    for (int k = 0; k < STEP / VEC; k++)
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) take(q[k][e], i0 + k * VEC + e);
+                }
+            } else {
+                for (int i = 0; i < count; i++) take(level_val[threadIdx.x * RTS + i], i);
             }
             out[(int64_t)blockIdx.x * NEXT + threadIdx.x] = v;
             if (INDEXED) idx_out[(int64_t)blockIdx.x * NEXT + threadIdx.x] = level_idx[threadIdx.x * RTS + at];

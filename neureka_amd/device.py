@@ -375,9 +375,12 @@ class HipDevice:
         (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = self._ops(drn, a, b)
         _lib.check(self._lib.nk_convolution(self.handle, d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, drn.ndc.size))
 
-    def launch_matmul(self, row_major: bool, M: int, K: int, N: int, a, b, c) -> None:
-        _lib.check(self._lib.nk_matmul(self.handle, _dtype_code(c.dtype), _lib.ROW_MAJOR if row_major else _lib.COLUMN_MAJOR,
-                                       M, K, N, a._data.ptr, b._data.ptr, c._data.ptr))
+    def launch_matmul(self, row_major: bool, M: int, K: int, N: int, a, b, c, accumulate: bool = True) -> None:
+        """c += a @ b (GEMM.java:282-304), or with accumulate=False c = a @ b, what the OpenCL device's kernel does
+        (CLMatMul.java:50) and what the registered implementation calls: the drain it is handed is freshly zeroed."""
+        fn = self._lib.nk_matmul if accumulate else self._lib.nk_matmul_set
+        _lib.check(fn(self.handle, _dtype_code(c.dtype), _lib.ROW_MAJOR if row_major else _lib.COLUMN_MAJOR,
+                      M, K, N, a._data.ptr, b._data.ptr, c._data.ptr))
 
     def launch_sum(self, src, out) -> None:
         """CLSum.run (operations/linear/internal/opencl/CLSum.java:24-62): out[0] = sum of the dense tensor `src`."""
@@ -438,10 +441,10 @@ class HipDevice:
             d, drn, x, y = a
             (p0, k0, c0), (p1, k1, c1), (p2, k2, c2) = ops = self._ops(drn, x, y)
             call = self.prepared("nk_convolution", h, d, _dtype_code(drn.dtype), drn.ndc.rank, p0, c0, p1, c1, p2, c2, C.c_int64(drn.ndc.size))
-        elif kind == "matmul":
+        elif kind in ("matmul", "matmul_set"):
             rm, M, K, N, x, y, z = a
             ops = None
-            call = self.prepared("nk_matmul", h, _dtype_code(z.dtype), _lib.ROW_MAJOR if rm else _lib.COLUMN_MAJOR, C.c_int64(M), C.c_int64(K), C.c_int64(N),
+            call = self.prepared("nk_matmul" if kind == "matmul" else "nk_matmul_set", h, _dtype_code(z.dtype), _lib.ROW_MAJOR if rm else _lib.COLUMN_MAJOR, C.c_int64(M), C.c_int64(K), C.c_int64(N),
                                  C.c_uint64(x._data.ptr), C.c_uint64(y._data.ptr), C.c_uint64(z._data.ptr))
         elif kind == "fused":
             program, consts, drn, srcs = a

@@ -1431,6 +1431,33 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
     assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("dt,mkn,path", [
+    ("f32", (64, 48, 80), "simple"), ("f32", (512, 512, 512), "mfma_split"), ("f32", (2048, 256, 2048), "mfma"),
+    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (1000, 300, 520), "mfma_edge_split"), ("f32", (2100, 130, 2100), "mfma_edge"),
+    ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
+    ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge")])
+def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mkn, path):
+    """nk_matmul_set (C = A @ B, the OpenCL device's `C[n + m*N] = acc`, CLMatMul.java:50) on every kernel plan, both
+    layouts: the drain starts as NaN everywhere, so a single old value read would show; the result must equal, bit for
+    bit, what nk_matmul (C += A @ B) leaves in a zeroed C."""
+    T = F[dt]
+    M, K, N = mkn
+    rng = np.random.default_rng(59)
+    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
+    for row_major in (True, False):
+        say("matmul set", dt, mkn, "row major" if row_major else "column major")
+        ta, tb = (on(device, A), on(device, B)) if row_major else (on(device, A.T.copy()), on(device, B.T.copy()))
+        acc = on(device, np.zeros((M, N), dtype=T))
+        device.launch_matmul(row_major, M, K, N, ta, tb, acc)
+        if row_major: assert _lib.last_path() == path
+        got = on(device, np.full((M, N), np.nan, dtype=T))
+        device.launch_matmul(row_major, M, K, N, ta, tb, got, accumulate=False)
+        if row_major: assert _lib.last_path() == path
+        a, g = acc.getData(), got.getData()
+        assert not np.isnan(g).any()
+        assert (a.view(np.uint32 if dt == "f32" else np.uint64) == g.view(np.uint32 if dt == "f32" else np.uint64)).all()
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
