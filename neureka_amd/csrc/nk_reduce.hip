@@ -28,6 +28,9 @@ struct BcastBwdArgs {
     int64_t keep1[NK_MAX_RANK], keep2[NK_MAX_RANK];       // stride of src1 / src2 along axis k as the drain's index moves (0: pinned)
     int red_extent[NK_MAX_RANK];
     int64_t red1[NK_MAX_RANK], red2[NK_MAX_RANK];
+    // S = 2: a thread owns the drain elements at index i and i + extent / 2 of one kept axis along which src1 is
+    // pinned, so every value of src1 it loads serves two sums; c0.imap then unravels the halved index space
+    int64_t pair2, pair0;                // what the second element adds to the offset into src2 / into the drain
 };
 
 // The eight forms the backward term takes: CPUBroadcast<Op>.java _getDeriveAt0 / _getDeriveAt1 (these differ from
@@ -57,7 +60,7 @@ __device__ __forceinline__ T derive_term(T a, T b) {
     return dpow_db_ref(a, b);
 }
 
-template <typename T, int V, int G>
+template <typename T, int V, int G, int S = 1>
 __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* __restrict__ drn,
                                                             const T* __restrict__ s1, const T* __restrict__ s2) {
     constexpr int UNROLL = 8;
@@ -68,9 +71,11 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
     nd_of_flat(A.c0, A.rank, (int)(t * V), o);
     int64_t o1 = A.base1, o2 = A.base2;
     for (int k = 0; k < A.rank; k++) { o1 += o[k] * A.keep1[k]; o2 += o[k] * A.keep2[k]; }
-    T value[V];
+    T value[S][V];
 #pragma unroll
-    for (int v = 0; v < V; v++) value[v] = T(0);
+    for (int s = 0; s < S; s++)
+#pragma unroll
+        for (int v = 0; v < V; v++) value[s][v] = T(0);
     const int n0 = A.nred > 0 ? A.red_extent[0] : 1;
     const int64_t st1 = A.nred > 0 ? A.red1[0] : 0, st2 = A.nred > 0 ? A.red2[0] : 0;
 
@@ -95,19 +100,26 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
             // always has requests in flight; the order of the additions is the reference's.  Two sets of registers
             // take turns (no copies), and the offsets of the next term to request move by additions only.
             int64_t q1 = o1, q2 = o2;
-            auto request = [&](T (&a)[UNROLL][V], T (&b)[UNROLL][V]) {
+            auto request = [&](T (&a)[UNROLL][V], T (&b)[S][UNROLL][V]) {
 #pragma unroll
-                for (int u = 0; u < UNROLL; u++) { load1(q1, a[u]); load2(q2, b[u]); q1 += st1; q2 += st2; }
+                for (int u = 0; u < UNROLL; u++) {
+                    load1(q1, a[u]);
+#pragma unroll
+                    for (int s = 0; s < S; s++) load2(q2 + s * A.pair2, b[s][u]);
+                    q1 += st1; q2 += st2;
+                }
             };
-            auto consume = [&](const T (&a)[UNROLL][V], const T (&b)[UNROLL][V]) {
+            auto consume = [&](const T (&a)[UNROLL][V], const T (&b)[S][UNROLL][V]) {
 #pragma unroll
                 for (int u = 0; u < UNROLL; u++)
 #pragma unroll
-                    for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[u][v], b[u][v]);
+                    for (int s = 0; s < S; s++)
+#pragma unroll
+                        for (int v = 0; v < V; v++) value[s][v] = value[s][v] + derive_term<T, G>(a[u][v], b[s][u][v]);
             };
             const int batches = n0 / UNROLL;
             if (batches > 0) {
-                T a0[UNROLL][V], b0[UNROLL][V], a1[UNROLL][V], b1[UNROLL][V];
+                T a0[UNROLL][V], b0[S][UNROLL][V], a1[UNROLL][V], b1[S][UNROLL][V];
                 request(a0, b0);
                 int bi = 0;
                 for (; bi + 2 <= batches; bi += 2) {
@@ -119,11 +131,15 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
                 if (bi < batches) consume(a0, b0);
             }
             for (int j = batches * UNROLL; j < n0; j++) {
-                T a[V], b[V];
-                load1(q1, a); load2(q2, b);
+                T a[V], b[S][V];
+                load1(q1, a);
+#pragma unroll
+                for (int s = 0; s < S; s++) load2(q2 + s * A.pair2, b[s]);
                 q1 += st1; q2 += st2;
 #pragma unroll
-                for (int v = 0; v < V; v++) value[v] = value[v] + derive_term<T, G>(a[v], b[v]);
+                for (int s = 0; s < S; s++)
+#pragma unroll
+                    for (int v = 0; v < V; v++) value[s][v] = value[s][v] + derive_term<T, G>(a[v], b[s][v]);
             }
             // carry into the slower reduced axes
             int k = 1;
@@ -140,11 +156,14 @@ __global__ __launch_bounds__(256) void broadcast_bwd_kernel(BcastBwdArgs A, T* _
     else reduce(std::false_type{});
 
     const int at = phys_of_nd(A.c0, A.rank, o);
-    if (V == 1) drn[at] = value[0];
-    else {
-        Vec out;
-        for (int v = 0; v < V; v++) ((T*)&out)[v] = value[v];
-        *(Vec*)(drn + at) = out;
+#pragma unroll
+    for (int s = 0; s < S; s++) {
+        if (V == 1) drn[at + s * A.pair0] = value[s][0];
+        else {
+            Vec out;
+            for (int v = 0; v < V; v++) ((T*)&out)[v] = value[s][v];
+            *(Vec*)(drn + at + s * A.pair0) = out;
+        }
     }
 }
 
@@ -466,10 +485,38 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         NK_HIP(hipGetLastError());
         return NK_OK;
     }
+    // Two drain elements per thread where src1 is pinned along a kept axis (the forward broadcast repeated it there):
+    // each value of src1 is then loaded once for two sums, which takes a quarter off the requests the vector memory
+    // unit has to serve.  Needs the row-major unravelling of the drain's flat index and enough threads left.
+    A.pair2 = 0; A.pair0 = 0;
+    bool paired = false;
+    const int form_id = derive_form(op_id, d);
+    if (vec && form_id != G_SECOND && form_id != G_RCP && A.n_threads / 2 >= 256u * (unsigned)dev->props.multiProcessorCount) {
+        bool row_major = true;
+        int64_t run = 1;
+        for (int k = rank - 1; k >= 0; k--) { if (A.c0.shape[k] > 1 && A.c0.imap[k] != run) row_major = false; run *= A.c0.shape[k]; }
+        for (int k = 0; row_major && !paired && k < rank - 1; k++) {
+            const int e = A.c0.shape[k];
+            if (e >= 2 && e % 2 == 0 && A.keep1[k] == 0 && A.keep2[k] != 0) {
+                A.pair2 = (int64_t)(e / 2) * A.keep2[k];
+                A.pair0 = (int64_t)(e / 2) * A.c0.spread[k] * A.c0.strides[k];
+                A.c0.shape[k] = e / 2;
+                int64_t m = 1;
+                for (int j = rank - 1; j >= 0; j--) { A.c0.imap[j] = (int)m; m *= A.c0.shape[j]; }
+                A.n_threads /= 2;
+                paired = true;
+            }
+        }
+    }
     const unsigned blocks = (A.n_threads + 255) / 256;
-    set_path(vec ? "broadcast_backward_vec" : "broadcast_backward");
+    set_path(vec ? (paired ? "broadcast_backward_vec_pairs" : "broadcast_backward_vec") : "broadcast_backward");
     auto go = [&](auto form) {
         constexpr int G = decltype(form)::value;
+        if (paired) {
+            if (dtype == NK_F32) hipLaunchKernelGGL((broadcast_bwd_kernel<float, 4, G, 2>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
+            else                 hipLaunchKernelGGL((broadcast_bwd_kernel<double, 2, G, 2>), dim3(blocks), dim3(256), 0, dev->stream, A, (double*)drn, (const double*)a, (const double*)b);
+            return;
+        }
         if (dtype == NK_F32) {
             if (vec) hipLaunchKernelGGL((broadcast_bwd_kernel<float, 4, G>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);
             else     hipLaunchKernelGGL((broadcast_bwd_kernel<float, 1, G>), dim3(blocks), dim3(256), 0, dev->stream, A, (float*)drn, (const float*)a, (const float*)b);

@@ -602,6 +602,43 @@ def test_broadcast_backward_split_sums(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_broadcast_backward_two_drain_elements_per_thread(device, orc, dt):
+    """Large gradients along whose kept axis src1 is pinned (the operand the forward broadcast repeated): a thread owns
+    the drain elements i and i + extent / 2 of that axis and loads every value of src1 once for both sums.  Random,
+    non-zero src1 of the other operand's shape, every form of the term that reads src1, pair axis first, in the middle
+    and next to the vector axis, a drain view with gaps: bit-identical to the CPU state machine."""
+    T = F[dt]
+    rng = np.random.default_rng(26)
+    cases = [([1024, 6, 512], [1024, 1, 512], [1, 6, 512]),            # pair axis 0
+             ([6, 1024, 512], [1, 1024, 512], [6, 1, 512]),            # pair axis 1, reduced axis outermost
+             ([4, 1024, 5, 512], [1, 1024, 1, 512], [4, 1, 5, 1]),     # two reduced axes around the pair axis
+             ([512, 3, 2, 512], [512, 1, 2, 512], [1, 3, 1, 512])]     # the first of two pinned axes pairs
+    for full, tgt, oth in cases:
+        e = rng.uniform(0.5, 1.5, full).astype(T) * rng.choice([-1.0, 1.0], full).astype(T)
+        te = on(device, e)
+        for op, d in (("add", 0), ("subtract", 1), ("multiply", 1), ("divide", 1), ("power", 0)):
+            say("broadcast bwd pairs", full, tgt, op, d, dt)
+            other = rng.uniform(0.5, 1.5, oth).astype(T)
+            drn = Tensor._on_device(device, T, tgt)
+            device.launch_broadcast(op, d, drn, on(device, other), te)
+            assert _lib.last_path() == "broadcast_backward_vec_pairs", _lib.last_path()
+            want = orc.broadcast(op, d, np.zeros(drn.size, dtype=T), orc.dense_cfg(tgt), other.reshape(-1), orc.dense_cfg(oth), e.reshape(-1), orc.dense_cfg(full), workers=8)
+            if op in ("add", "subtract", "multiply"): assert_bits(drn.getData(), want, f"{full} {tgt} {op} {d}")
+            else: assert_close(drn.getData(), want, f"{full} {tgt} {op} {d}")
+    say("broadcast bwd pairs into a drain with gaps", dt)
+    full, oth = [1024, 6, 512], [1, 6, 512]
+    e = rng.uniform(-1, 1, full).astype(T); other = rng.uniform(-1, 1, oth).astype(T)
+    backing = on(device, np.zeros((1024, 2, 1024), dtype=T))
+    view = backing[:, 1:2, 256:768]                                     # shape [1024, 1, 512] inside a wider tensor
+    device.launch_broadcast("add", 0, view, on(device, other), on(device, e))
+    assert _lib.last_path() == "broadcast_backward_vec_pairs", _lib.last_path()
+    want = orc.broadcast("add", 0, np.zeros(1024 * 512, dtype=T), orc.dense_cfg([1024, 1, 512]), other.reshape(-1), orc.dense_cfg(oth), e.reshape(-1), orc.dense_cfg(full), workers=8)
+    got = backing.getData().reshape(1024, 2, 1024)
+    assert_bits(got[:, 1, 256:768].reshape(-1), want, "drain view")
+    assert (got[:, 0, :] == 0).all() and (got[:, 1, :256] == 0).all() and (got[:, 1, 768:] == 0).all()
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_broadcast_backward_vector_path_and_views(device, orc, dt):
     """Drains whose last axis is kept and a multiple of the vector width (16-byte accesses, several drain
     elements per thread), one and two reduced axes, sources of the operands' own shapes as autograd passes
