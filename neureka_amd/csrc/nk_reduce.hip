@@ -189,7 +189,7 @@ struct BwdSplitArgs {
                                          // memory, so that every block walks its own contiguous stretch front to back
 };
 
-template <typename T, int G, int OT, bool ROWS, int VW, bool SPLAT = false, bool FLAT = false>
+template <typename T, int G, int OT, bool ROWS, int VW, bool SPLAT = false, bool FLAT = false, int PAIR = 1>
 __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A, BwdSplitArgs S, T* __restrict__ drn, T* __restrict__ partial,
                                                                   const T* __restrict__ s1, const T* __restrict__ s2) {
     // VW: width of the 16-byte accesses -- ROWS: VW neighbouring terms of one drain element per load;
@@ -201,14 +201,17 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
     constexpr int VA = SPLAT ? 1 : VW;                           // values kept per term of src1: one serves all VW when it
                                                                  // does not move along the vector (a template parameter: a
                                                                  // run-time test in the term loop costs a quarter of the rate)
-    constexpr int NV = ROWS ? 1 : VW;                            // running sums per thread
+    constexpr int NV = ROWS ? PAIR : VW;                         // running sums per thread
+    // PAIR = 2 (ROWS only): the thread also owns the drain element that lies A.pair0 / A.pair2 further on along a kept
+    // axis where src1 is pinned -- the same terms of src1 serve both sums (S.n_out counts the first elements only)
+    static_assert(PAIR == 1 || (ROWS && OT == 1), "pairs of drain elements: one pair per block");
     typedef typename std::conditional<VW == 1, T, T __attribute__((ext_vector_type(VW == 1 ? 2 : VW), aligned(sizeof(T))))>::type Vec;
     __shared__ T part[NV][256];
     const int tid = threadIdx.x;
     const unsigned ob = blockIdx.x % S.out_blocks, seg = blockIdx.x / S.out_blocks;
     const unsigned oi = ROWS ? (unsigned)tid / TL : (unsigned)tid % OT;
     const unsigned tl = ROWS ? (unsigned)tid % TL : (unsigned)tid / OT;
-    const unsigned out = (ob * OT + oi) * NV;                     // first (or only) drain element of the thread
+    const unsigned out = ROWS ? ob * OT + oi : (ob * OT + oi) * NV;   // first (or only) drain element of the thread
     const bool live = out < S.n_out;
     int o[NK_MAX_RANK];
     nd_of_flat(A.c0, A.rank, (int)(live ? out : 0), o);
@@ -248,42 +251,50 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
             if (carry) { idx[k] -= A.red_extent[k]; a1 += fix1[k]; a2 += fix2[k]; }
         }
     };
-    auto fetch = [&](T (&a)[VA], T (&b)[VW]) {
+    auto fetch = [&](T (&a)[VA], T (&b)[PAIR][VW]) {
 #pragma unroll
         for (int v = 0; v < VA; v++) a[v] = T(0);
 #pragma unroll
-        for (int v = 0; v < VW; v++) b[v] = T(0);
+        for (int p = 0; p < PAIR; p++)
+#pragma unroll
+            for (int v = 0; v < VW; v++) b[p][v] = T(0);
         if constexpr (G != G_SECOND && G != G_RCP) {
             if constexpr (VA == 1) a[0] = s1[a1];
             else { const Vec x = *(const Vec*)(s1 + a1); for (int v = 0; v < VW; v++) a[v] = ((const T*)&x)[v]; }
         }
         if constexpr (G != G_FIRST) {
-            if (VW == 1) b[0] = s2[a2];
-            else { const Vec x = __builtin_nontemporal_load((const Vec*)(s2 + a2)); for (int v = 0; v < VW; v++) b[v] = ((const T*)&x)[v]; }
+#pragma unroll
+            for (int p = 0; p < PAIR; p++) {
+                const int64_t at = a2 + p * A.pair2;
+                if (VW == 1) b[p][0] = s2[at];
+                else { const Vec x = __builtin_nontemporal_load((const Vec*)(s2 + at)); for (int v = 0; v < VW; v++) b[p][v] = ((const T*)&x)[v]; }
+            }
         }
     };
     T value[NV];
 #pragma unroll
     for (int v = 0; v < NV; v++) value[v] = T(0);
-    auto add = [&](const T (&a)[VA], const T (&b)[VW]) {
+    auto add = [&](const T (&a)[VA], const T (&b)[PAIR][VW]) {
 #pragma unroll
-        for (int v = 0; v < VW; v++) {
-            T& sum = value[ROWS ? 0 : v];
-            sum = sum + derive_term<T, G>(a[VA == 1 ? 0 : v], b[v]);
-        }
+        for (int p = 0; p < PAIR; p++)
+#pragma unroll
+            for (int v = 0; v < VW; v++) {
+                T& sum = value[ROWS ? p : v];
+                sum = sum + derive_term<T, G>(a[VA == 1 ? 0 : v], b[p][v]);
+            }
     };
     const unsigned t = first + tl;
     const unsigned mine = t < end ? (end - t + stride - 1) / stride : 0;   // term units of this lane
     unsigned i = 0;
     for (; i + U <= mine; i += U) {                                  // U loads requested together, added in that order
-        T a[U][VA], b[U][VW];
+        T a[U][VA], b[U][PAIR][VW];
 #pragma unroll
         for (int u = 0; u < U; u++) { fetch(a[u], b[u]); advance(); }
 #pragma unroll
         for (int u = 0; u < U; u++) add(a[u], b[u]);
     }
     for (; i < mine; i++) {
-        T a[VA], b[VW];
+        T a[VA], b[PAIR][VW];
         fetch(a, b); advance();
         add(a, b);
     }
@@ -292,7 +303,9 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
     __syncthreads();
     if (ROWS) {
         for (int w = TL / 2; w >= 1; w >>= 1) {
-            if ((int)tl < w) part[0][tid] = part[0][tid] + part[0][tid + w];
+            if ((int)tl < w)
+#pragma unroll
+                for (int v = 0; v < NV; v++) part[v][tid] = part[v][tid] + part[v][tid + w];
             __syncthreads();
         }
     } else {
@@ -304,16 +317,26 @@ __global__ __launch_bounds__(256) void broadcast_bwd_split_kernel(BcastBwdArgs A
         }
     }
     if (tl == 0 && live) {
-        T* dst = S.segments == 1 ? drn + phys_of_nd(A.c0, A.rank, o) : partial + (int64_t)seg * S.n_out + out;
+        if (ROWS) {
 #pragma unroll
-        for (int v = 0; v < NV; v++) dst[v] = part[v][tid];      // NV > 1: the drain is contiguous along these elements
+            for (int p = 0; p < PAIR; p++) {     // partial sums: all first elements of a segment, then all second ones
+                if (S.segments == 1) drn[phys_of_nd(A.c0, A.rank, o) + p * A.pair0] = part[p][tid];
+                else partial[((int64_t)seg * PAIR + p) * S.n_out + out] = part[p][tid];
+            }
+        } else {
+            T* dst = S.segments == 1 ? drn + phys_of_nd(A.c0, A.rank, o) : partial + (int64_t)seg * S.n_out + out;
+#pragma unroll
+            for (int v = 0; v < NV; v++) dst[v] = part[v][tid];      // NV > 1: the drain is contiguous along these elements
+        }
     }
 }
 
 // partial[segment][element] -> drain: sixteen lanes per element take every sixteenth segment and meet in LDS
 template <typename T>
 __global__ __launch_bounds__(256) void broadcast_bwd_segments_kernel(Cfg c0, int rank, unsigned n_out, int segments, const T* __restrict__ partial,
-                                                                     T* __restrict__ drn) {
+                                                                     T* __restrict__ drn, unsigned firsts, int64_t pair0) {
+    // n_out = firsts, or 2 * firsts when the blocks summed pairs of drain elements: element e >= firsts is the partner of
+    // e - firsts, pair0 further on in the drain
     __shared__ T part[256];
     const int tid = threadIdx.x;
     const unsigned lane = (unsigned)tid & 15u, out = blockIdx.x * 16u + ((unsigned)tid >> 4);
@@ -326,7 +349,7 @@ __global__ __launch_bounds__(256) void broadcast_bwd_segments_kernel(Cfg c0, int
         if ((int)lane < w) part[tid] = part[tid] + part[tid + w];
         __syncthreads();
     }
-    if (lane == 0 && out < n_out) drn[phys_of_flat(c0, rank, (int)out)] = part[tid];
+    if (lane == 0 && out < n_out) drn[out < firsts ? phys_of_flat(c0, rank, (int)out) : phys_of_flat(c0, rank, (int)(out - firsts)) + pair0] = part[tid];
 }
 
 }  // namespace nk
@@ -418,7 +441,30 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         const bool flat = A.nred == 1;
         // a step of the block is one contiguous piece of the error when its lanes take neighbouring 16-byte units of a
         // contiguous reduced axis (256 of them: 4 KiB), or when the block covers whole rows that follow each other
-        S.out_blocks = (unsigned)((n / VO + OT - 1) / OT);
+        // long sums over a contiguous innermost axis with src1 pinned along a kept axis (per-slab sums of a broadcast
+        // operand): a block owns the two drain elements that lie half that axis apart and reads src1 once for both
+        A.pair2 = 0; A.pair0 = 0;
+        int pairs = 1;
+        const int form_of_term = derive_form(op_id, d);
+        if (flat && last_reduced && TL == 256 && VT > 1 && !S.splat1 && form_of_term != G_SECOND && form_of_term != G_RCP && n >= 512) {
+            bool row_major = true;
+            int64_t run = 1;
+            for (int k = rank - 1; k >= 0; k--) { if (A.c0.shape[k] > 1 && A.c0.imap[k] != run) row_major = false; run *= A.c0.shape[k]; }
+            for (int k = 0; row_major && pairs == 1 && k < rank; k++) {
+                const int e = A.c0.shape[k];
+                if (e >= 2 && e % 2 == 0 && A.keep1[k] == 0 && A.keep2[k] != 0) {
+                    A.pair2 = (int64_t)(e / 2) * A.keep2[k];
+                    A.pair0 = (int64_t)(e / 2) * A.c0.spread[k] * A.c0.strides[k];
+                    A.c0.shape[k] = e / 2;
+                    int64_t m = 1;
+                    for (int j = rank - 1; j >= 0; j--) { A.c0.imap[j] = (int)m; m *= A.c0.shape[j]; }
+                    pairs = 2;
+                }
+            }
+        }
+        const int64_t firsts = n / pairs;                                             // drain elements the blocks enumerate
+        S.n_out = (unsigned)firsts;
+        S.out_blocks = (unsigned)((firsts / VO + OT - 1) / OT);
         S.contiguous = flat && (last_reduced ? (TL == 256 && VT > 1) : (S.out_blocks == 1 && VO > 1 && A.red2[0] == n));
         int64_t segs = (2048 + S.out_blocks - 1) / S.out_blocks;                  // enough blocks to fill the machine ...
         const int64_t most = units / (TL * 8) > 0 ? units / (TL * 8) : 1;         // ... with at least 8 term units per lane
@@ -429,9 +475,9 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         S.segments = (int)((units + S.seg_terms - 1) / S.seg_terms);
         void* ws = nullptr;
         if (S.segments > 1)
-            if (int e = workspace(dev, (uint64_t)S.segments * S.n_out * eb, &ws)) return e;
+            if (int e = workspace(dev, (uint64_t)S.segments * n * eb, &ws)) return e;
         const unsigned grid = S.out_blocks * (unsigned)S.segments;
-        set_path(last_reduced ? (VT > 1 ? "broadcast_backward_split_rows_vec" : "broadcast_backward_split_rows")
+        set_path(last_reduced ? (pairs == 2 ? "broadcast_backward_split_rows_vec_pairs" : VT > 1 ? "broadcast_backward_split_rows_vec" : "broadcast_backward_split_rows")
                               : (VO > 1 ? "broadcast_backward_split_vec" : "broadcast_backward_split"));
         auto split = [&](auto form) {
             constexpr int G = decltype(form)::value;
@@ -455,7 +501,11 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                 }
                 else {
                     auto rows = [&](auto ot, auto vw, auto splat) {
-                        if (flat) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value, true>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        if (pairs == 2) {
+                            if constexpr (decltype(ot)::value == 1 && decltype(vw)::value == VM && !decltype(splat)::value)
+                                hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, 1, true, VM, false, true, 2>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
+                        }
+                        else if (flat) hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value, true>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                         else      hipLaunchKernelGGL((broadcast_bwd_split_kernel<T, G, decltype(ot)::value, true, decltype(vw)::value, decltype(splat)::value, false>), dim3(grid), dim3(256), 0, dev->stream, A, S, d_, w_, a_, b_);
                     };
                     auto lanes = [&](auto ot) {
@@ -468,7 +518,8 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
                     else lanes(std::integral_constant<int, 16>{});
                 }
                 if (S.segments > 1)
-                    hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((S.n_out + 15) / 16), dim3(256), 0, dev->stream, A.c0, rank, S.n_out, S.segments, (const T*)ws, d_);
+                    hipLaunchKernelGGL(broadcast_bwd_segments_kernel<T>, dim3((unsigned)((n + 15) / 16)), dim3(256), 0, dev->stream, A.c0, rank, (unsigned)n, S.segments, (const T*)ws, d_,
+                                       S.n_out, A.pair0);
             };
             if (dtype == NK_F32) typed(0.0f); else typed(0.0);
         };
@@ -490,8 +541,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
     // unit has to serve.  Needs the row-major unravelling of the drain's flat index and enough threads left.
     A.pair2 = 0; A.pair0 = 0;
     bool paired = false;
-    const int form_id = derive_form(op_id, d);
-    if (vec && form_id != G_SECOND && form_id != G_RCP && A.n_threads / 2 >= 256u * (unsigned)dev->props.multiProcessorCount) {
+    if (vec && A.n_threads / 2 >= 256u * (unsigned)dev->props.multiProcessorCount) {
         bool row_major = true;
         int64_t run = 1;
         for (int k = rank - 1; k >= 0; k--) { if (A.c0.shape[k] > 1 && A.c0.imap[k] != run) row_major = false; run *= A.c0.shape[k]; }

@@ -602,6 +602,42 @@ def test_broadcast_backward_split_sums(device, orc, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_broadcast_backward_split_sums_in_pairs(device, orc, dt):
+    """Long sums over a contiguous innermost axis with src1 pinned along a kept axis (per-slab sums of an operand that the
+    forward broadcast repeated over the slabs): a block owns two drain elements half that axis apart and reads src1
+    once for both.  Exact on integer-valued data; norm-wise within 1e-5 / 1e-12 on uniform data; one and several
+    segments per sum; a kept axis in the middle."""
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    rng = np.random.default_rng(27)
+    for full, tgt, oth in (([1024, 16, 512], [1024, 1, 1], [1, 16, 512]),       # four segments per pair of sums
+                           ([4096, 4, 2048], [4096, 1, 1], [1, 4, 2048]),       # one segment: straight into the drain
+                           ([3, 512, 8192], [3, 512, 1], [3, 1, 8192])):        # the second axis pairs
+        for integer in (True, False):
+            for op, d in (("add", 0), ("subtract", 1), ("multiply", 1), ("divide", 1)):
+                if integer and op == "divide":
+                    continue
+                if op == "divide":
+                    e = (rng.uniform(0.5, 1.5, full) * rng.choice([-1.0, 1.0], full)).astype(T)
+                else:
+                    e = (rng.integers(-3, 4, full) if integer else rng.uniform(-1, 1, full)).astype(T)
+                other = (rng.integers(1, 4, oth) if integer else rng.uniform(0.5, 1.5, oth)).astype(T)
+                say("broadcast bwd split pairs", full, tgt, op, d, dt, "integer" if integer else "uniform")
+                drn = Tensor._on_device(device, T, tgt)
+                device.launch_broadcast(op, d, drn, on(device, other), on(device, e))
+                assert _lib.last_path() == "broadcast_backward_split_rows_vec_pairs", _lib.last_path()
+                dense_t, dense_o, dense_f = orc.dense_cfg(tgt), orc.dense_cfg(oth), orc.dense_cfg(full)
+                want = orc.broadcast(op, d, np.zeros(drn.size, dtype=T), dense_t, other.reshape(-1), dense_o, e.reshape(-1), dense_f, workers=8)
+                if integer:
+                    assert_bits(drn.getData(), want, f"{full} {tgt} {op} {d}")
+                else:
+                    mag = orc.broadcast(op, d, np.zeros(drn.size), dense_t, np.abs(other).astype(np.float64).reshape(-1), dense_o,
+                                        np.abs(e).astype(np.float64).reshape(-1), dense_f, workers=8)
+                    err_abs = np.abs(drn.getData().astype(np.float64) - want)
+                    assert (err_abs <= tol * np.abs(mag) + 1e-30).all(), (full, tgt, op, d, float(err_abs.max()))
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_broadcast_backward_two_drain_elements_per_thread(device, orc, dt):
     """Large gradients along whose kept axis src1 is pinned (the operand the forward broadcast repeated): a thread owns
     the drain elements i and i + extent / 2 of that axis and loads every value of src1 once for both sums.  Random,
@@ -616,7 +652,7 @@ def test_broadcast_backward_two_drain_elements_per_thread(device, orc, dt):
     for full, tgt, oth in cases:
         e = rng.uniform(0.5, 1.5, full).astype(T) * rng.choice([-1.0, 1.0], full).astype(T)
         te = on(device, e)
-        for op, d in (("add", 0), ("subtract", 1), ("multiply", 1), ("divide", 1), ("power", 0)):
+        for op, d in (("add", 0), ("subtract", 1), ("multiply", 0), ("multiply", 1), ("divide", 0), ("divide", 1), ("power", 0)):
             say("broadcast bwd pairs", full, tgt, op, d, dt)
             other = rng.uniform(0.5, 1.5, oth).astype(T)
             drn = Tensor._on_device(device, T, tgt)
