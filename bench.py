@@ -260,7 +260,19 @@ def main():
             g_t = Tensor._on_device(dev, f32, tgt); z_t = Tensor._on_device(dev, f32, tuple(1 if t > 1 else f for t, f in zip(tgt, (1024, 2048, 512))))
             hbm(name, 4 * (err.size + g_t.size + z_t.size), dev.prepared_launch("broadcast", "add", 0, g_t, z_t, err))
             dev.free(g_t); dev.free(z_t)
+        # the same 2^30 elements through the whole-tensor reductions: what the fixed tree streams at when its second,
+        # latency-bound launch (about 5 us) no longer weighs (the 2^26 entries below are a tenth tail)
+        one30 = Tensor._on_device(dev, f32, (1,)); slot30 = dev.allocate(np.int32, 1)
+        hbm("sum_2^30", 4 * err.size, dev.prepared("nk_sum", dev.handle, 0, err._data.ptr, err.size, one30._data.ptr))
+        hbm("max_index_2^30", 4 * err.size, dev.prepared("nk_reduce_index", dev.handle, 1, 0, err._data.ptr, err.size, slot30.ptr))
+        dev.free(one30); slot30.release()
         dev.free(err)
+        # rows shorter than a 16-byte vector: [2^20,1,3] + [1,64,3] -> [2^20,64,3] (one element per thread, index arithmetic bound)
+        a3 = Tensor.of(f32, (1 << 20, 1, 3), rng.uniform(-1, 1, 3 << 20).astype(f32)).to(dev)
+        b3 = Tensor.of(f32, (1, 64, 3), rng.uniform(-1, 1, 192).astype(f32)).to(dev)
+        o3s = Tensor._on_device(dev, f32, (1 << 20, 64, 3))
+        hbm("broadcast_add_rows_of_3", 4 * (o3s.size + a3.size + b3.size), dev.prepared_launch("broadcast", "add", -1, o3s, a3, b3))
+        for t in (a3, b3, o3s): dev.free(t)
 
         # C3: tanh(sig(a)*b+c) on 2^26 elements: fused, and the reference's 4-kernel sequence
         n = 1 << 26

@@ -622,7 +622,16 @@ __global__ __launch_bounds__(256) void tile_kernel(TileArgs A, Prog P, LightProg
     // whole tile inside the tensor, every operand either along pax or along the innermost axis:
     // 16-byte accesses on both sides, one barrier
     if (p0 + TILE_P <= A.P && l0 + TILE_L <= A.L && !A.careful) {
-        const unsigned rq = threadIdx.x % R_LPR, rr = threadIdx.x / R_LPR;
+        // Which 16-byte piece of a turned source a lane reads.  The four elements of a piece stay in one LDS row
+        // (tiles[row][pax]), and the 32 lanes that write together should hit 32 different banks.
+        // With 16 lanes side by side in one row (banks 4 * rq + e, rq = 0..15) lanes rq and rq + 8 collide; eight
+        // lanes per row and four rows (row pitch 65: banks 4 * q + row + e) do not.  A wavefront still reads four
+        // whole 256-byte rows per access, only the order of its lanes differs.
+        unsigned rq = threadIdx.x % R_LPR, rr = threadIdx.x / R_LPR;
+        if constexpr (R_LPR == 16 && sizeof(T) == 4) {
+            rq = ((threadIdx.x >> 5) & 1u) * 8u + (threadIdx.x & 7u);
+            rr = (threadIdx.x >> 6) * 4u + ((threadIdx.x >> 3) & 3u);
+        }
         const unsigned wq = threadIdx.x % W_LPR, wr = threadIdx.x / W_LPR;
 #pragma unroll
         for (int j = 0; j < NSRC; j++) {
