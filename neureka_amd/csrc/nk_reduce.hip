@@ -341,8 +341,18 @@ __global__ __launch_bounds__(256) void broadcast_bwd_segments_kernel(Cfg c0, int
     const int tid = threadIdx.x;
     const unsigned lane = (unsigned)tid & 15u, out = blockIdx.x * 16u + ((unsigned)tid >> 4);
     T s = T(0);
-    if (out < n_out)
-        for (int k = (int)lane; k < segments; k += 16) s = s + partial[(int64_t)k * n_out + out];
+    if (out < n_out) {
+        // eight loads requested together: with one at a time 2048 segments cost 128 memory latencies (44 us)
+        int k = (int)lane;
+        for (; k + 7 * 16 < segments; k += 8 * 16) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = partial[(int64_t)(k + 16 * u) * n_out + out];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s = s + v[u];
+        }
+        for (; k < segments; k += 16) s = s + partial[(int64_t)k * n_out + out];
+    }
     part[tid] = s;
     __syncthreads();
     for (int w = 8; w >= 1; w >>= 1) {
@@ -466,10 +476,14 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
         S.n_out = (unsigned)firsts;
         S.out_blocks = (unsigned)((firsts / VO + OT - 1) / OT);
         S.contiguous = flat && (last_reduced ? (TL == 256 && VT > 1) : (S.out_blocks == 1 && VO > 1 && A.red2[0] == n));
-        int64_t segs = (2048 + S.out_blocks - 1) / S.out_blocks;                  // enough blocks to fill the machine ...
+        // enough blocks to fill the machine: eight per compute unit where the segments interleave; where every block
+        // walks its own contiguous stretch, few long-running blocks read fastest (bias gradient of 4 GiB: 2048 blocks
+        // 6.7, 1024 6.9, 512 7.1, 256 7.2 TB/s) ...
+        const int64_t want_blocks = S.contiguous ? 2 * dev->props.multiProcessorCount : 2048;
+        int64_t segs = (want_blocks + S.out_blocks - 1) / S.out_blocks;
         const int64_t most = units / (TL * 8) > 0 ? units / (TL * 8) : 1;         // ... with at least 8 term units per lane
         if (segs > most) segs = most;
-        if (segs > (S.contiguous ? 2048 : 256)) segs = S.contiguous ? 2048 : 256;
+        if (segs > 256) segs = 256;
         if (segs < 1) segs = 1;
         S.seg_terms = (unsigned)((units + segs - 1) / segs);
         S.segments = (int)((units + S.seg_terms - 1) / S.seg_terms);

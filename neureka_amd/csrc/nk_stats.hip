@@ -26,21 +26,28 @@ enum { STAT_SUM = 0, STAT_MIN = 1, STAT_MAX = 2, STAT_DOT = 3 };
 template <typename T, int RTS, int MODE>
 __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ in, const T* __restrict__ in2,
                                                           const int* __restrict__ idx_in, int64_t n,
-                                                          T* __restrict__ out, int* __restrict__ idx_out) {
+                                                          T* __restrict__ out, int* __restrict__ idx_out, int pieces) {
     constexpr int VEC = 16 / sizeof(T);             // elements per 16-byte load
     constexpr int COLS = 32;                        // columns staged at a time
     constexpr int NCH = RTS / COLS;
     constexpr int LOADS = 64 * COLS / VEC / 64;     // 16-byte loads per lane and chunk
     constexpr int PPR = COLS / VEC;                 // 16-byte pieces per tile row of a chunk
     __shared__ T stage[4][64][COLS + 1];
+    constexpr bool INDEXED = MODE == STAT_MIN || MODE == STAT_MAX;
+    constexpr int NEXT = 256 / RTS;                  // next-level tiles per piece
+    __shared__ __attribute__((aligned(16))) T level_val[256];
+    __shared__ int level_idx[INDEXED ? 256 : 1];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int64_t tile0 = ((int64_t)blockIdx.x * 4 + wave) * 64;          // first tile of the wavefront
-    const int64_t elem0 = tile0 * RTS;
-    const bool active = elem0 < n;                                       // wave-uniform; idle wavefronts only join the block's last step
-    const int64_t left = active ? n - elem0 : 0;
-    const unsigned bytes = left * (int64_t)sizeof(T) > 0xffffffffll ? 0xffffffffu : (unsigned)(left * sizeof(T));
-    const BufRsrc r1 = __builtin_amdgcn_make_buffer_rsrc((void*)(in + elem0), 0, bytes, 0x00020000);
-    const BufRsrc r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == STAT_DOT ? in2 : in) + elem0), 0, bytes, 0x00020000);
+    // A block walks `pieces` consecutive pieces of 256 tiles (what used to be one block each): few long-running blocks
+    // that each read one contiguous stretch stream faster than many short ones, and the first chunk of the next piece
+    // is requested while the last chunk of the current one is reduced.  One buffer descriptor per wavefront spans from
+    // its first tile to the end of the data; the piece and the chunk go into the scalar offset of the loads.
+    const int64_t piece0 = (int64_t)blockIdx.x * pieces;
+    const int64_t wave_elem0 = (piece0 * 4 + wave) * 64 * RTS;           // first element of the wavefront in piece 0
+    const int64_t wave_left = wave_elem0 < n ? n - wave_elem0 : 0;       // nothing left: every load reads zeros
+    const unsigned bytes = wave_left * (int64_t)sizeof(T) > 0xffffffffll ? 0xffffffffu : (unsigned)(wave_left * sizeof(T));
+    const BufRsrc r1 = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (wave_left > 0 ? wave_elem0 : 0)), 0, bytes, 0x00020000);
+    const BufRsrc r2 = __builtin_amdgcn_make_buffer_rsrc((void*)((MODE == STAT_DOT ? in2 : in) + (wave_left > 0 ? wave_elem0 : 0)), 0, bytes, 0x00020000);
     T (*mine)[COLS + 1] = stage[wave];
 
     // piece k of the lane inside a chunk: tile row and column of its 16 bytes
@@ -56,14 +63,20 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     // one chunk ahead (two in flight measured slower: 47.1 against 45.1 us for the sum of 2^26 floats)
     u32x4 cur[LOADS], cur2[LOADS];
     constexpr int NON_TEMPORAL = 2;                 // cache policy of the loads: every element is read exactly once
-    auto request = [&](int c) {
+    constexpr unsigned PIECE_BYTES = 256u * RTS * sizeof(T);
+    auto request = [&](int piece_i, int c) {
+        const unsigned soff = (unsigned)piece_i * PIECE_BYTES + (unsigned)(c * COLS * sizeof(T));
 #pragma unroll
         for (int k = 0; k < LOADS; k++) {
-            cur[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r1, voff[k], (unsigned)(c * COLS * sizeof(T)), NON_TEMPORAL));
+            cur[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r1, voff[k], soff, NON_TEMPORAL));
             if (MODE == STAT_DOT)
-                cur2[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r2, voff[k], (unsigned)(c * COLS * sizeof(T)), NON_TEMPORAL));
+                cur2[k] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r2, voff[k], soff, NON_TEMPORAL));
         }
     };
+    request(0, 0);
+    for (int piece_i = 0; piece_i < pieces; piece_i++) {
+    const int64_t piece = piece0 + piece_i;
+    const int64_t elem0 = (piece * 4 + wave) * 64 * RTS;
 
     // the lane's own tile
     const int64_t my_first = elem0 + (int64_t)lane * RTS;
@@ -72,9 +85,8 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     T value = T(0);
     int found = 0;
 
-    if (active) request(0);
 #pragma unroll
-    for (int c = 0; active && c < NCH; c++) {
+    for (int c = 0; c < NCH; c++) {
 #pragma unroll
         for (int k = 0; k < LOADS; k++) {
             typedef T Vec __attribute__((ext_vector_type(VEC)));
@@ -88,7 +100,8 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
                 for (int e = 0; e < VEC; e++) mine[prow[k]][pcol[k] + e] = v[e];
             }
         }
-        if (c + 1 < NCH) request(c + 1);
+        if (c + 1 < NCH) request(piece_i, c + 1);
+        else if (piece_i + 1 < pieces) request(piece_i + 1, 0);
         __builtin_amdgcn_wave_barrier();            // LDS operations of a wavefront complete in order
 #pragma unroll
         for (int i = 0; i < COLS; i++) {
@@ -103,12 +116,8 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
         }
         __builtin_amdgcn_wave_barrier();
     }
-    // The next level of the tree in the same launch: the block's 256 tile results are 256 / RTS whole tiles of the
+    // The next level of the tree in the same launch: the piece's 256 tile results are 256 / RTS whole tiles of the
     // next level; one thread each reduces them front to back out of LDS and only those results are written.
-    constexpr bool INDEXED = MODE == STAT_MIN || MODE == STAT_MAX;
-    constexpr int NEXT = 256 / RTS;                  // next-level tiles per block
-    __shared__ __attribute__((aligned(16))) T level_val[256];
-    __shared__ int level_idx[INDEXED ? 256 : 1];
     level_val[threadIdx.x] = value;
     if (INDEXED && limit > 0) {
         const int64_t at = my_first + found;                          // position in this level's input
@@ -117,7 +126,7 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
     __syncthreads();
     if (threadIdx.x < NEXT) {
         const int64_t results = (n + RTS - 1) / RTS;                  // tile results of this level in the whole grid
-        const int64_t first = (int64_t)blockIdx.x * 256 + (int64_t)threadIdx.x * RTS;
+        const int64_t first = piece * 256 + (int64_t)threadIdx.x * RTS;
         if (first < results) {
             const int count = results - first < RTS ? (int)(results - first) : RTS;
             T v = T(0);
@@ -146,9 +155,11 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const T* __restrict__ 
             } else {
                 for (int i = 0; i < count; i++) take(level_val[threadIdx.x * RTS + i], i);
             }
-            out[(int64_t)blockIdx.x * NEXT + threadIdx.x] = v;
-            if (INDEXED) idx_out[(int64_t)blockIdx.x * NEXT + threadIdx.x] = level_idx[threadIdx.x * RTS + at];
+            out[piece * NEXT + threadIdx.x] = v;
+            if (INDEXED) idx_out[piece * NEXT + threadIdx.x] = level_idx[threadIdx.x * RTS + at];
         }
+    }
+    if (piece_i + 1 < pieces) __syncthreads();       // the next piece overwrites level_val / level_idx
     }
 }
 
@@ -272,11 +283,16 @@ static int reduce_levels(Device* dev, const T* in, const T* in2, int64_t n, T* o
         }
         T* dst = vals + used;
         int* dst_idx = indexed ? idxs + used : nullptr;
-        const unsigned blocks = (unsigned)((tiles + 255) / 256);
+        // pieces of 256 tiles; a block walks several consecutive ones so that about two blocks per compute unit exist
+        // (sum of 2^26 floats: one block per unit 60.6 us, two 43.6, four 45.8, eight 44.2, one piece per block 45.1)
+        const int64_t piece_count = (tiles + 255) / 256;
+        const int64_t two_per_cu = 2 * (int64_t)dev->props.multiProcessorCount;
+        const int pieces = (int)(piece_count > two_per_cu ? (piece_count + two_per_cu - 1) / two_per_cu : 1);
+        const unsigned blocks = (unsigned)((piece_count + pieces - 1) / pieces);
         if (MODE == STAT_DOT && level > 0)
-            hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, STAT_SUM>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur, cur_idx, m, dst, dst_idx);
+            hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, STAT_SUM>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur, cur_idx, m, dst, dst_idx, pieces);
         else
-            hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, MODE>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur2, cur_idx, m, dst, dst_idx);
+            hipLaunchKernelGGL((tile_reduce_kernel<T, RTS, MODE>), dim3(blocks), dim3(256), 0, dev->stream, cur, cur2, cur_idx, m, dst, dst_idx, pieces);
         cur = dst; cur2 = dst; cur_idx = dst_idx;
         const int64_t written = (tiles + RTS - 1) / RTS;           // the launch covers two levels of the tree
         used += written;
