@@ -242,7 +242,10 @@ constexpr int ROWS_MAX_OUTER = 5;
 // address arithmetic of every pass cost the broadcast of [1024,1,512] o [1,2048,512] five per cent.
 constexpr int ROWS_FAST_OUTER = 3;
 // units per block of rows_kernel: enough loads in flight to cover latency, few enough registers to keep
-// several wavefronts per SIMD (three sources x 16 values already costs half the occupancy)
+// several wavefronts per SIMD (three sources x 16 values already costs half the occupancy).  The fused chain
+// tanh(sig(a)*b+c) on 2^26 elements: one pass 6.71, two 6.71, four 6.46 TB/s -- its 62 vector instructions per
+// element (110 us of issue time in a 160 us launch), not the access pattern, hold it below the 7.2 TB/s a bare
+// three-reads-one-write kernel reaches.
 constexpr int rows_passes(int funset, int nsrc) { return funset >= 2 ? 1 : (nsrc >= 3 ? 2 : 4); }
 struct RowsArgs {
     int nouter;                // collapsed outer axes, 0..ROWS_MAX_OUTER
