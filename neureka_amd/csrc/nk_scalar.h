@@ -118,18 +118,27 @@ __device__ __forceinline__ double sigmoid(double x) { return 1.0 / (1.0 + ::exp(
 // correction of the argument the caller already knows (the rounding of x * 1.702 in gelu), 0 otherwise.
 // The results stay within a few ulp of the reference's (float) f((double) x) wherever they are not saturated, and
 // within 1.3e-6 relative at the far ends (|x| towards 87).
-__device__ __forceinline__ float fast_exp_neg(float t, float dt = 0.0f) {        // exp(-(t + dt)) for t >= 0
+template <bool WITH_DT>
+__device__ __forceinline__ float fast_exp_neg_impl(float t, float dt) {           // exp(-(t + dt)) for t >= 0
     const float L = 1.44269502162933349609375f;                  // (float) log2(e); log2(e) - L = 1.9e-8 stays out: t * 1.3e-8
     t = t > 128.0f ? 128.0f : t;                                 // exp(-128) is below the smallest float; a NaN stays
     const float p = t * L;
-    const float lack = __builtin_fmaf(t, L, -p) + dt * L;        // (relative, 1.2e-6 at t = 87) costs less than its two operations
+    float lack = __builtin_fmaf(t, L, -p);                       // (relative, 1.2e-6 at t = 87) costs less than its two operations
+    if constexpr (WITH_DT) lack = lack + dt * L;                 // (adding a zero is not nothing to the compiler: -0 + 0 = +0)
     const float e = __builtin_amdgcn_exp2f(-p);
     return __builtin_fmaf(e * -0.693147182464599609375f, lack, e);               // e * 2^-lack
 }
+__device__ __forceinline__ float fast_exp_neg(float t, float dt) { return fast_exp_neg_impl<true>(t, dt); }
+__device__ __forceinline__ float fast_exp_neg(float t) { return fast_exp_neg_impl<false>(t, 0.0f); }
 // f32: the same quantity as the reference's double evaluation, evaluated on e = exp(-|x|) <= 1 so
 // nothing overflows: x >= 0 -> 1/(1+e), x < 0 -> e/(1+e).  `dx` as above: sigmoid(x + dx).
-__device__ __forceinline__ float sigmoid(float x, float dx = 0.0f) {
+__device__ __forceinline__ float sigmoid(float x, float dx) {
     const float e = fast_exp_neg(::fabsf(x), x >= 0.0f ? dx : -dx);
+    const float r = __builtin_amdgcn_rcpf(1.0f + e);
+    return x >= 0.0f ? r : e * r;
+}
+__device__ __forceinline__ float sigmoid(float x) {              // no correction of the argument: three instructions fewer
+    const float e = fast_exp_neg(::fabsf(x));
     const float r = __builtin_amdgcn_rcpf(1.0f + e);
     return x >= 0.0f ? r : e * r;
 }
@@ -149,7 +158,9 @@ __device__ __forceinline__ float tanh_ref(float x) {
     float r;
     if (ax < 0.125f) {                       // odd series, next term 62/2835 x^9 < 2e-10 relative here
         const float x2 = ax * ax;
-        r = ax * (1.0f + x2 * (-0.333333333f + x2 * (0.133333333f + x2 * -0.0539682540f)));
+        // (an approximation of this library, not one of the reference's float formulas: fused multiply-adds are free to use)
+        const float poly = __builtin_fmaf(x2, __builtin_fmaf(x2, __builtin_fmaf(x2, -0.0539682540f, 0.133333333f), -0.333333333f), 1.0f);
+        r = ax * poly;
     } else {
         // (1 - e)/(1 + e) with 1 - e >= 0.22: no cancellation, and an error of e enters the quotient scaled by 2e, so
         // the plain exp2 (relative error of e: 2|x| * 4e-8, at most 3e-8 in the quotient) needs no correction here
