@@ -26,7 +26,7 @@ FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
 FP64_PEAK_TFLOPS = 78.6        # MI355X dense fp64 matrix, published
 # HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
 # against a plain 1 GiB copy): profiles/rows_binary_lean_kernel_broadcast_c2.md
-C2_TRAFFIC_BYTES = 4316311460
+C2_TRAFFIC_BYTES = 4316335565
 SETTLE_MS = 60.0               # untimed load before the warm-up steps, so that the timed steps run at the working clock
 HOST_CORE_SHARE = 16           # host threads one GPU's box grants a job, whatever the machine's core count
 
