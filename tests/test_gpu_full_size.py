@@ -111,7 +111,11 @@ def _chain_oracle(orc, bases, cfgs, shape, workers=16):
 
 
 def _check_chain(got, want, m, c_view):
-    bound = RTOL[np.dtype(f32)] * (np.abs(m) + np.abs(c_view) + np.abs(want)) + 1e-10
+    """The outer tanh is held to rtol 1e-5 on the output.  What reaches it is p = fl(m + c) with m = sig(a) * b: the inner
+    sigmoid may differ from the reference's by 1e-5 relative, i.e. m by 1e-5 |m|, and where m + c cancels that is no
+    longer small against p -- so 1e-5 |m| enters absolutely (tanh' <= 1), plus one rounding of the sum, 2^-23 (|m| + |c|).
+    Each of the four kernels alone is held to 1e-5 on its own output at this size in test_gpu_transcendental_sweep.py."""
+    bound = RTOL[np.dtype(f32)] * (np.abs(m) + np.abs(want)) + 2.0 ** -23 * (np.abs(m) + np.abs(c_view)) + 1e-10
     bad = np.abs(got - want) > bound
     assert not bad.any(), f"{bad.sum()} of {bad.size} outside the bound; first {np.flatnonzero(bad)[:3]}"
 
