@@ -21,7 +21,9 @@
  *   - `d` is the derivative index of the ExecutionCall (Arg.DerivIdx), -1 = forward.
  *   - `n` is the drain's element count (the OpenCL global work size), < 2^31 like a Java int.
  *   - dtype: NK_F32 or NK_F64.  Slot order follows the reference: drain first, then sources.
- *   - Calls on one device must not overlap in time (one thread at a time per device).
+ *   - Calls on one device handle from several host threads are serialised inside the library (a lock per device
+ *     held for the length of a call), so they are safe but do not overlap; nk_last_error / nk_last_path are per thread.
+ *     A handle closed while another thread waits for it makes that call fail with NK_ERR_HANDLE.
  */
 #ifndef NEUREKA_HIP_H
 #define NEUREKA_HIP_H

@@ -7,6 +7,7 @@
 #include <mutex>
 #include <string>
 #include <map>
+#include <memory>
 #include "../../include/neureka_hip.h"
 
 namespace nk {
@@ -16,6 +17,11 @@ struct Device {
     hipStream_t stream = nullptr;
     hipDeviceProp_t props{};
     std::mutex mu;
+    // Held for the length of every call on this device: the stream, the grow-on-demand workspace and the registry of
+    // live allocations are one thread's at a time, so calls from several host threads (a JVM binding) queue up here
+    // instead of racing.  Recursive because an entry point may use another one on the same device.
+    std::recursive_mutex call_mu;
+    bool closed = false;                 // set by nk_device_close; a caller that waited for call_mu meanwhile gets NK_ERR_HANDLE
     std::map<uint64_t, uint64_t> live;   // device address -> bytes
     uint64_t live_bytes = 0;
     // grow-only scratch for two-pass kernels (partial sums); owned by the device, freed on close
@@ -27,7 +33,7 @@ struct Device {
 
 int set_error(int code, const char* fmt, ...);
 void set_path(const char* name);
-Device* device_of(nk_dev h);            // nullptr (and error set) if unknown
+std::shared_ptr<Device> device_ref(nk_dev h);   // empty (and error set) if unknown; keeps the device alive across a concurrent close
 int workspace(Device* dev, uint64_t bytes, void** out);
 int stats_static_init(Device* dev);     // resolves sum_static_scratch; the device must be current
 
@@ -44,8 +50,11 @@ int stats_static_init(Device* dev);     // resolves sum_static_scratch; the devi
     } while (0)
 
 #define NK_DEVICE(var, handle)                                                               \
-    nk::Device* var = nk::device_of(handle);                                                 \
+    std::shared_ptr<nk::Device> var##_ref = nk::device_ref(handle);                          \
+    nk::Device* var = var##_ref.get();                                                       \
     if (!var) return NK_ERR_HANDLE;                                                          \
+    std::lock_guard<std::recursive_mutex> var##_lock(var->call_mu);                          \
+    if (var->closed) return nk::set_error(NK_ERR_HANDLE, "the device handle was closed");    \
     NK_HIP(hipSetDevice(var->index))
 
 // ---------------------------------------------------------------------------------------------

@@ -21,15 +21,15 @@ int set_error(int code, const char* fmt, ...) {
 void set_path(const char* name) { g_path = name; }
 
 static std::mutex g_devices_mu;
-static std::vector<std::unique_ptr<Device>> g_devices;   // handle = slot + 1
+static std::vector<std::shared_ptr<Device>> g_devices;   // handle = slot + 1
 
-Device* device_of(nk_dev h) {
+std::shared_ptr<Device> device_ref(nk_dev h) {
     std::lock_guard<std::mutex> lock(g_devices_mu);
     if (h == 0 || h > g_devices.size() || !g_devices[h - 1]) {
         set_error(NK_ERR_HANDLE, "unknown device handle %llu", (unsigned long long)h);
         return nullptr;
     }
-    return g_devices[h - 1].get();
+    return g_devices[h - 1];
 }
 
 int workspace(Device* dev, uint64_t bytes, void** out) {
@@ -189,7 +189,7 @@ int nk_device_open(int index, nk_dev* dev) {
     int n = 0;
     NK_HIP(hipGetDeviceCount(&n));
     NK_REQUIRE(index >= 0 && index < n, "nk_device_open: device index %d outside [0, %d)", index, n);
-    auto d = std::make_unique<Device>();
+    auto d = std::make_shared<Device>();
     d->index = index;
     NK_HIP(hipSetDevice(index));
     NK_HIP(hipGetDeviceProperties(&d->props, index));
@@ -208,6 +208,8 @@ int nk_device_close(nk_dev h) {
     dev->live.clear();
     dev->live_bytes = 0;
     if (dev->workspace) (void)hipFree(dev->workspace);
+    dev->workspace = nullptr; dev->workspace_bytes = 0;
+    dev->closed = true;                  // the object itself lives until the last call that holds a reference returns
     NK_HIP(hipStreamDestroy(dev->stream));
     std::lock_guard<std::mutex> lock(g_devices_mu);
     g_devices[h - 1].reset();

@@ -187,6 +187,54 @@ def test_dropped_results_release_their_buffers(device):
     assert device.has(a) and not device.has(Tensor.of(np.float32, (1,), 0.0))
 
 
+def test_calls_from_several_host_threads_are_serialised(device, orc):
+    """Four host threads call the C ABI on one device handle at once -- allocation and release, whole-tensor sums whose
+    partial results share the device's grow-on-demand workspace, matrix products whose parts do, elementwise launches.
+    The library serialises the calls of a handle, so every result is the single-threaded one and the registry of
+    allocations ends where it began."""
+    import ctypes as C
+    import threading
+    say("threads")
+    lib, h = device._lib, device.handle
+    rng = np.random.default_rng(90)
+    live_before = device.liveBuffers()
+    errors = []
+
+    def worker(seed):
+        try:
+            r = np.random.default_rng(seed)
+            for it in range(12):
+                n = int(r.integers(40000, 3000000))
+                x = r.integers(-8, 9, n).astype(np.float32)            # integer-valued: every summation order is exact
+                buf, out = C.c_uint64(), C.c_uint64()
+                _lib.check(lib.nk_alloc(h, 4 * n, C.byref(buf))); _lib.check(lib.nk_alloc(h, 4, C.byref(out)))
+                _lib.check(lib.nk_h2d(h, buf, 0, x.ctypes.data_as(C.c_void_p), 4 * n))
+                _lib.check(lib.nk_sum(h, 0, buf, n, out))
+                got = np.zeros(1, dtype=np.float32)
+                _lib.check(lib.nk_d2h(h, got.ctypes.data_as(C.c_void_p), out, 0, 4))
+                assert got[0] == np.float32(x.astype(np.float64).sum()), (seed, it, n)
+                M, K, N = 128, int(r.choice([2048, 4096, 8192])), 128      # few tiles, long inner dimension: parts in the workspace
+                a = r.integers(-2, 3, (M, K)).astype(np.float32); b = r.integers(-2, 3, (K, N)).astype(np.float32)
+                pa, pb, pc = C.c_uint64(), C.c_uint64(), C.c_uint64()
+                for ptr, arr in ((pa, a), (pb, b)):
+                    _lib.check(lib.nk_alloc(h, arr.nbytes, C.byref(ptr)))
+                    _lib.check(lib.nk_h2d(h, ptr, 0, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
+                _lib.check(lib.nk_alloc(h, 4 * M * N, C.byref(pc)))
+                _lib.check(lib.nk_matmul_set(h, 0, _lib.ROW_MAJOR, M, K, N, pa, pb, pc))
+                c = np.zeros((M, N), dtype=np.float32)
+                _lib.check(lib.nk_d2h(h, c.ctypes.data_as(C.c_void_p), pc, 0, c.nbytes))
+                assert (c == a.astype(np.float64) @ b.astype(np.float64)).all(), (seed, it, K)
+                for ptr in (buf, out, pa, pb, pc): _lib.check(lib.nk_free(h, ptr))
+        except BaseException as e:                                          # reported by the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(100 + i,)) for i in range(4)]
+    for t in threads: t.start()
+    for t in threads: t.join()
+    assert not errors, errors[0]
+    assert device.liveBuffers() == live_before
+
+
 def test_fused_function_on_host_operands_keeps_autograd(device):
     """A fused function whose operands live on the host (stored for the call, restored afterwards) records its graph
     node like the unfused path does: same result, same gradients."""
