@@ -267,6 +267,11 @@ struct RowsArgs {
     int base[MAX_OPERANDS];
     int stride[MAX_OPERANDS][ROWS_MAX_OUTER];
     int last_stride[MAX_OPERANDS];           // innermost stride of every operand (1 for the drain)
+    // bit j: source j repeats along the innermost axis with period[j + 1] elements -- a short innermost axis (rows of
+    // three: channels-last data and a per-channel operand) merged with the axis above it, along which the source was
+    // pinned; its element at column c is the one at c mod period
+    unsigned periodic_last;
+    FastDiv period[MAX_OPERANDS];
 };
 
 // addressing shared by the rows kernels: unit -> (row, col), row -> element offset of every operand
@@ -364,6 +369,16 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
                         const int ls = A.last_stride[j + 1];
 #pragma unroll
                         for (int v = 0; v < V; v++) xj[v] = sp[(int)(R.col + v) * ls];
+                    } else if ((A.periodic_last >> j) & 1u) {
+                        const unsigned period = A.period[j + 1].d;
+                        const unsigned first = R.col - A.period[j + 1].div(R.col) * period;      // col mod period
+#pragma unroll
+                        for (int v = 0; v < V; v++) {
+                            unsigned at = first + v;                   // < period + 4: at most two periods too far
+                            at = at >= period ? at - period : at;
+                            at = at >= period ? at - period : at;
+                            xj[v] = sp[at];                            // (loading the period once and selecting would make
+                        }                                              // the passes wait for one another: measured slower)
                     } else {
                         load_vec<T, V>(xj, sp + R.col);
                     }
@@ -390,7 +405,9 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
 // and each pass is stored as soon as its operands have arrived.
 // HOIST bit j: source j does not change along the rows a block covers (forward broadcast): it is loaded once.
 // CONST bit j: source j does not change along a row (one element per row, e.g. a per-row scale or an outer product).
-template <typename T, int V, int PASSES, bool NT = false, int HOIST = 0, int CONST = 0, int MAXO = ROWS_FAST_OUTER>
+// PERIODIC bit j: source j repeats along the row with a period shorter than a vector (RowsArgs::periodic_last): its
+//                 elements are gathered at column mod period, all gathers of all passes requested before the first use.
+template <typename T, int V, int PASSES, bool NT = false, int HOIST = 0, int CONST = 0, int MAXO = ROWS_FAST_OUTER, int PERIODIC = 0>
 __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T* __restrict__ drn, const T* __restrict__ s0,
                                                           const T* __restrict__ s1) {
     T x0[PASSES][V], x1[PASSES][V];
@@ -403,9 +420,21 @@ __global__ __launch_bounds__(256) void rows_binary_kernel(RowsArgs A, int op, T*
         const RowsAddr<3> R = rows_address<3, MAXO>(A, rg, chunk);
         live[p] = R.live;
         doff[p] = R.off[0] + (int)R.col;
-        if (CONST & 1) { const T c = s0[R.off[1]]; _Pragma("unroll") for (int v = 0; v < V; v++) x0[p][v] = c; }
+        auto gather = [&](T (&x)[V], const T* sp, int operand) {
+            const unsigned period = A.period[operand].d;
+            const unsigned first = R.col - A.period[operand].div(R.col) * period;          // col mod period
+            _Pragma("unroll") for (int v = 0; v < V; v++) {
+                unsigned at = first + v;                                                   // at most two periods too far
+                at = at >= period ? at - period : at;
+                at = at >= period ? at - period : at;
+                x[v] = sp[at];
+            }
+        };
+        if (PERIODIC & 1) gather(x0[p], s0 + R.off[1], 1);
+        else if (CONST & 1) { const T c = s0[R.off[1]]; _Pragma("unroll") for (int v = 0; v < V; v++) x0[p][v] = c; }
         else if (p == 0 || !(HOIST & 1)) load_vec<T, V, NT>(x0[p], s0 + R.off[1] + R.col);
-        if (CONST & 2) { const T c = s1[R.off[2]]; _Pragma("unroll") for (int v = 0; v < V; v++) x1[p][v] = c; }
+        if (PERIODIC & 2) gather(x1[p], s1 + R.off[2], 2);
+        else if (CONST & 2) { const T c = s1[R.off[2]]; _Pragma("unroll") for (int v = 0; v < V; v++) x1[p][v] = c; }
         else if (p == 0 || !(HOIST & 2)) load_vec<T, V, NT>(x1[p], s1 + R.off[2] + R.col);
     }
     if (HOIST) {

@@ -182,6 +182,57 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         return launch_family<T, 2>(dev, plan);
     }
     if (cn.rank == 0) { cn.rank = 1; cn.shape[0] = 1; for (int o = 0; o <= c.nsrc; o++) cn.stride[o][0] = 1; }
+    // An innermost axis shorter than a vector (rows of three: channels-last data with a per-channel operand,
+    // [.., N, 3] o [.., 1, 3]) would run one element per thread, one of up to seven elements on overlapping vectors.  Where the drain and every source are dense
+    // across the innermost axis and the one above it -- or pinned on the upper one, i.e. periodic in the merged axis, or
+    // constant along both -- the two axes become one long row: dense operands move in vectors, periodic ones are gathered
+    // at column mod period.
+    unsigned periodic = 0;
+    int64_t period_of[MAX_OPERANDS] = {};
+    {
+        constexpr int VM = 16 / sizeof(T);
+        Canon m = cn;
+        unsigned per = 0;
+        int64_t per_of[MAX_OPERANDS] = {};
+        bool any = false;
+        const int64_t first_row = m.rank >= 1 ? m.shape[m.rank - 1] : 0;
+        while (m.rank >= 2) {
+            const int l = m.rank - 1;
+            const int64_t L = m.shape[l];
+            if (L >= 2 * VM || L % VM == 0 || L < 2) break;      // longer rows run on (overlapping) vectors as they are
+            bool ok = m.stride[0][l] == 1 && m.stride[0][l - 1] == L;
+            unsigned per_next = per;
+            for (int j = 0; j < c.nsrc && ok; j++) {
+                const int64_t in = m.stride[j + 1][l], up = m.stride[j + 1][l - 1];
+                if ((per >> j) & 1u) ok = up == 0;                                   // stays periodic with its period
+                else if (in == 1 && up == L) {}                                      // dense across both
+                else if (in == 1 && up == 0) { per_next |= 1u << j; per_of[j + 1] = L; }
+                else if (in == 0 && up == 0) {}                                      // one value for the merged row
+                else ok = false;
+            }
+            if (!ok) break;
+            per = per_next;
+            m.shape[l - 1] *= L;
+            for (int o = 0; o <= c.nsrc; o++) m.stride[o][l - 1] = m.stride[o][l];   // 1 (dense or periodic) or 0
+            m.rank--;
+            any = true;
+        }
+        // what the rows kernels need of the merged form (they keep element offsets in 32 bits)
+        // Rows of VM elements and more also run on overlapping vectors as they are; measured, the merged form wins there
+        // only when everything merges into one row ([2^22,5] + [1,5]: 6.4 TB/s merged; [2^20,1,5] o [1,64,5]: 3.0 merged --
+        // rows of 320 leave 48 of 128 lanes idle -- and [4096,1,5] o [1,4096,5] 4.4, against 4.9 on overlapping vectors).
+        bool fits = any && per != 0 && m.rank - 1 <= ROWS_MAX_OUTER && (first_row < VM || m.rank == 1);
+        for (int o = 0; o <= c.nsrc && fits; o++) {
+            int64_t lo = m.base[o], hi = m.base[o];
+            for (int k = 0; k < m.rank; k++) {
+                const int64_t span = (m.shape[k] - 1) * m.stride[o][k];
+                if (span < 0) lo += span; else hi += span;
+                if (m.stride[o][k] > INT32_MAX || m.stride[o][k] < INT32_MIN) fits = false;
+            }
+            if (lo < INT32_MIN || hi > INT32_MAX) fits = false;
+        }
+        if (fits) { cn = m; periodic = per; for (int o = 0; o < MAX_OPERANDS; o++) period_of[o] = per_of[o]; }
+    }
     const int last = cn.rank - 1;
     bool rows_ok = cn.stride[0][last] == 1 && cn.rank - 1 <= ROWS_MAX_OUTER;
     // sources may also take every n-th column (a gather per element; the drain is still written in whole vectors)
@@ -237,6 +288,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         bool reused = false;                                // some source is read more than once (a broadcast)
         for (int j = 0; j < c.nsrc; j++)
             for (int k = 0; k < cn.rank; k++) if (cn.shape[k] > 1 && cn.stride[j + 1][k] == 0) reused = true;
+        if (periodic) reused = true;
         bool once = streaming && !reused;
         const bool deep = last > ROWS_FAST_OUTER;           // more outer axes than the tuned variants resolve: plain variants
         if (deep) once = false;
@@ -249,6 +301,8 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             A.last_stride[j + 1] = (int)cn.stride[j + 1][last];
         }
         A.last_stride[0] = 1;
+        A.periodic_last = periodic;
+        for (int o = 0; o < MAX_OPERANDS; o++) A.period[o] = FastDiv((unsigned)(period_of[o] > 0 ? period_of[o] : 1));
         uint64_t n_rows = 1;
         // kernel axis k counts outward from the innermost outer axis
         for (int k = 0; k < last; k++) { n_rows *= cn.shape[k]; A.outer[k] = FastDiv((unsigned)cn.shape[last - 1 - k]); }
@@ -269,11 +323,12 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         }
         A.vec = V;
         A.ragged = ragged ? 1 : 0;
-        A.simple_loads = (funset < 2 && A.const_last == 0 && A.strided_last == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
+        A.simple_loads = (funset < 2 && A.const_last == 0 && A.strided_last == 0 && periodic == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel
         // (sources that are constant along a row are handled by that kernel's vector variant only)
-        const bool loads_ok = A.simple_loads || (A.const_last != 0 && A.strided_last == 0 && vec);
+        const bool loads_ok = A.simple_loads || (A.const_last != 0 && A.strided_last == 0 && periodic == 0 && vec) ||
+                              ((periodic == 1 || periodic == 2) && A.const_last == 0 && A.strided_last == 0 && vec && !deep);
         if (loads_ok && c.nsrc == 2 && funset == 0 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
             prog.op[1] == I_BIN && prog.src[1] == 1 && prog.arg[1] <= NK_OP_DIV) {
             plan.kind = PLAN_ROWS_BINARY;
@@ -304,7 +359,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // drain that is a slice of a wider tensor measured 5 % slower this way)
         bool drain_dense = cn.stride[0][last] == 1;
         for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
-        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && reused) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && periodic == 0 && reused) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
@@ -317,7 +372,8 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
         set_path(plan.lean_fill ? "rows_vec_fill_lean" : plan.lean ? "rows_vec_binary_lean"
-                           : plan.kind == PLAN_ROWS_BINARY ? (vec ? "rows_vec_binary" : "rows_binary") : vec ? "rows_vec" : "rows");
+                           : plan.kind == PLAN_ROWS_BINARY ? (periodic ? "rows_vec_binary_periodic" : vec ? "rows_vec_binary" : "rows_binary")
+                           : periodic ? (vec ? "rows_vec_periodic" : "rows_periodic") : vec ? "rows_vec" : "rows");
         done = true;
     }
 

@@ -385,6 +385,50 @@ def test_broadcast_forward_bit_exact(device, orc, dt):
             assert_bits(out.getData().reshape(so), f(a, b), f"{op} numpy")
 
 
+def test_rows_shorter_than_a_vector_merge_with_the_axis_above(device, orc):
+    """f32 rows of two or three elements (channels-last data and a per-channel operand): the innermost axis and the one
+    above it become one long row; operands that are dense across both move in vectors, an operand pinned on the upper
+    axis repeats with the short row as its period and is gathered at column mod period.  Broadcast in both operand
+    orders, a bias over a flat image, rank 4, a million rows; + * / bit for bit, power and modulo against the oracle.
+    A drain with gaps, or a source with another stride, keeps the element-wise path."""
+    T = np.float32
+    rng = np.random.default_rng(28)
+    for s1, s2 in (([4096, 1, 3], [1, 64, 3]), ([1, 64, 3], [4096, 1, 3]), ([300, 500, 3], [1, 1, 3]), ([1, 1, 3], [300, 500, 3]),
+                   ([7, 1, 1, 2], [1, 5, 33, 2]), ([5000, 1, 3], [5000, 77, 3]), ([9, 1, 1, 3], [9, 4, 11, 3]), ([1, 3], [1000003, 3])):
+        so = [q if p == 1 else p for p, q in zip(s1, s2)]
+        a = rng.uniform(-1, 1, s1).astype(T); b = rng.uniform(-1, 1, s2).astype(T)
+        ta, tb = on(device, a), on(device, b)
+        for op, f in (("add", np.add), ("multiply", np.multiply), ("divide", np.divide)):
+            say("short rows", s1, s2, op)
+            out = Tensor._on_device(device, T, so)
+            device.launch_broadcast(op, -1, out, ta, tb)
+            assert _lib.last_path() == "rows_vec_binary_periodic", (_lib.last_path(), s1, s2)
+            assert_bits(out.getData().reshape(so), f(a, b), f"{op} {s1} {s2}")
+    say("rows of five and seven merge when the whole tensor becomes one row")
+    for s1, s2, path in (([70001, 5], [1, 5], "rows_vec_binary_periodic"), ([1, 1, 7], [333, 99, 7], "rows_vec_binary_periodic"), ([512, 1, 5], [1, 9, 5], "rows_vec_binary")):
+        so = [q if p == 1 else p for p, q in zip(s1, s2)]
+        a = rng.uniform(-1, 1, s1).astype(T); b = rng.uniform(-1, 1, s2).astype(T)
+        out = Tensor._on_device(device, T, so)
+        device.launch_broadcast("subtract", -1, out, on(device, a), on(device, b))
+        assert _lib.last_path() == path, (_lib.last_path(), s1, s2)
+        assert_bits(out.getData().reshape(so), a - b, f"subtract {s1} {s2}")
+    say("short rows, power and modulo")
+    s1, s2 = [513, 1, 3], [1, 21, 3]
+    so = [513, 21, 3]
+    a = rng.uniform(0.5, 2, s1).astype(T); b = rng.uniform(0.5, 2, s2).astype(T)
+    for op in ("power", "modulo"):
+        out = Tensor._on_device(device, T, so)
+        device.launch_broadcast(op, -1, out, on(device, a), on(device, b))
+        assert _lib.last_path() == "rows_vec_periodic", _lib.last_path()
+        want = orc.broadcast(op, -1, np.zeros(out.size, dtype=T), orc.dense_cfg(so), a.reshape(-1), orc.dense_cfg(s1), b.reshape(-1), orc.dense_cfg(s2))
+        assert_close(out.getData(), want, op)
+    say("short rows that stay element-wise")
+    wide = on(device, np.zeros((64, 8, 4), dtype=T))
+    view = wide[:, :, 0:3]                                                   # a drain with gaps
+    device.launch_broadcast("add", -1, view, on(device, rng.uniform(-1, 1, [64, 1, 3]).astype(T)), on(device, rng.uniform(-1, 1, [1, 8, 3]).astype(T)))
+    assert _lib.last_path() in ("rows_binary", "rows", "canon"), _lib.last_path()
+
+
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_ragged_rows_run_on_vectors_and_stay_bit_exact(device, orc, dt):
     """Rows whose length is not a multiple of the 16-byte vector: the last vector of a row is moved back to end with the
@@ -480,7 +524,7 @@ def test_deep_index_spaces_and_row_constant_sources(device, orc, dt):
             say("deep / row-constant broadcast", s1, s2, op, dt)
             out = Tensor._on_device(device, T, so)
             device.launch_broadcast(op, -1, out, ta, tb)
-            assert _lib.last_path() in ("rows_vec_binary", "rows_binary", "rows_vec", "rows"), _lib.last_path()
+            assert _lib.last_path() in ("rows_vec_binary", "rows_binary", "rows_vec", "rows", "rows_vec_binary_periodic"), _lib.last_path()
             assert_bits(out.getData().reshape(so), f(a, b), f"{op} {s1} {s2}")
     say("activation and fused chain on a view with five live axes", dt)
     parent = rng.uniform(-2, 2, (5, 6, 7, 5, 40)).astype(T)
