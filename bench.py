@@ -363,6 +363,12 @@ def main():
         yl = Tensor._on_device(dev, f32, (2044, 2044))
         flops("conv2d_2048x2048_5x5", 2.0 * 2044 * 2044 * 25, 4 * (2048 * 2048 + 25 + 2044 * 2044), dev.prepared_launch("convolution", -1, yl, xl, kl))
         for t in (xl, kl, yl): dev.free(t)
+        # 3x3 taps on a 4096^2 image: 18 unfused vector operations per output instead of 50, so memory gets a say
+        xl = Tensor.of(f32, (4096, 4096), rng.uniform(-1, 1, 4096 * 4096).astype(f32)).to(dev)
+        kl = Tensor.of(f32, (3, 3), rng.uniform(-1, 1, 9).astype(f32)).to(dev)
+        yl = Tensor._on_device(dev, f32, (4094, 4094))
+        flops("conv2d_4096x4096_3x3", 2.0 * 4094 * 4094 * 9, 4 * (4096 * 4096 + 9 + 4094 * 4094), dev.prepared_launch("convolution", -1, yl, xl, kl))
+        for t in (xl, kl, yl): dev.free(t)
         x5 = Tensor.of(f32, (64, 256, 256), (rng.standard_normal(64 * 256 * 256) * 0.1).astype(f32)).to(dev)
         k5 = Tensor.of(f32, (64, 5, 5), (rng.standard_normal(1600) * 0.1).astype(f32)).to(dev)
         y5 = Tensor._on_device(dev, f32, (1, 252, 252))
