@@ -422,6 +422,17 @@ def test_rows_shorter_than_a_vector_merge_with_the_axis_above(device, orc):
         assert _lib.last_path() == "rows_vec_periodic", _lib.last_path()
         want = orc.broadcast(op, -1, np.zeros(out.size, dtype=T), orc.dense_cfg(so), a.reshape(-1), orc.dense_cfg(s1), b.reshape(-1), orc.dense_cfg(s2))
         assert_close(out.getData(), want, op)
+    say("short rows in place and with a ragged merged row")
+    for n_rows in (7, 1001, 4096):                                       # 21 and 3003 elements: no whole number of vectors
+        x = rng.uniform(-1, 1, [n_rows, 3]).astype(T); bias = rng.uniform(-1, 1, [1, 3]).astype(T)
+        tx = on(device, x)
+        device.launch_broadcast("add", -1, tx, tx, on(device, bias))     # x += bias
+        assert "periodic" in _lib.last_path(), (_lib.last_path(), n_rows)
+        assert_bits(tx.getData().reshape(n_rows, 3), x + bias, f"in place {n_rows}")
+        out = Tensor._on_device(device, T, [n_rows, 3])
+        device.launch_broadcast("multiply", -1, out, on(device, bias), on(device, x))
+        assert "periodic" in _lib.last_path(), (_lib.last_path(), n_rows)
+        assert_bits(out.getData().reshape(n_rows, 3), bias * x, f"ragged {n_rows}")
     say("short rows that stay element-wise")
     wide = on(device, np.zeros((64, 8, 4), dtype=T))
     view = wide[:, :, 0:3]                                                   # a drain with gaps
