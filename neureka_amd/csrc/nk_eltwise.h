@@ -272,6 +272,10 @@ struct RowsArgs {
     // pinned; its element at column c is the one at c mod period
     unsigned periodic_last;
     FastDiv period[MAX_OPERANDS];
+    // Rows of fewer than 256 vectors whose vector count is no power of two would leave lanes idle (48 vectors per row:
+    // 16 of 64): then the threads are numbered through all rows without gaps -- vector f of the launch is vector
+    // f mod flat_vpr of row f / flat_vpr -- and `row_groups` counts units of 256 such vectors.  d == 1: not in use.
+    FastDiv flat_vpr;
 };
 
 // addressing shared by the rows kernels: unit -> (row, col), row -> element offset of every operand
@@ -289,6 +293,11 @@ __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsign
     unsigned row = rg * rows_per_pass + sub;                        // rg and chunk are block-uniform
     RowsAddr<NOPS> R;
     R.col = (chunk * tpr + lane) * (unsigned)A.vec;
+    if (A.flat_vpr.d > 1) {                                         // threads numbered through the rows without gaps
+        const unsigned f = rg * 256u + threadIdx.x;
+        row = A.flat_vpr.div(f);
+        R.col = (f - row * A.flat_vpr.d) * (unsigned)A.vec;
+    }
     const bool row_ok = rg < A.row_groups && row < A.n_rows;        // wave-uniform when a row spans a wavefront
     R.live = row_ok && R.col < A.L;
     if (!row_ok) row = 0;                                           // dead lanes get a valid address:
@@ -309,7 +318,7 @@ __device__ __forceinline__ RowsAddr<NOPS> rows_address(const RowsArgs& A, unsign
         }
     };
     // a row that spans a whole wavefront is wave-uniform: resolve it on the scalar unit
-    if (A.tpr_log2 >= 6) resolve(__builtin_amdgcn_readfirstlane(row));
+    if (A.tpr_log2 >= 6 && A.flat_vpr.d <= 1) resolve(__builtin_amdgcn_readfirstlane(row));
     else resolve(row);
     return R;
 }

@@ -311,9 +311,11 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         int l2 = 0;
         while ((1u << l2) < vec_per_row && l2 < 8) l2++;
         A.tpr_log2 = l2;
-        const unsigned tpr = 1u << l2, rpp = 256u >> l2;
+        const unsigned tpr = 1u << l2;
+        unsigned rpp = 256u >> l2;
         A.chunks = (unsigned)((vec_per_row + tpr - 1) / tpr);
-        const uint64_t row_groups = (n_rows + rpp - 1) / rpp;
+        uint64_t row_groups = (n_rows + rpp - 1) / rpp;
+        A.flat_vpr = FastDiv(1);
         if (row_groups * A.chunks >= ((uint64_t)1 << 31)) return set_error(NK_ERR_UNSUPPORTED, "%s: too many work units", c.name);
         A.row_groups = (unsigned)row_groups;
         A.chunk_div = FastDiv(A.chunks);
@@ -337,6 +339,24 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             plan.passes = passes;
         }
         plan.vec = vec;
+        // Rows of fewer than 256 vectors, no power of two, leave lanes idle (33 vectors per row: 31 of 64).  From a fifth
+        // of the lanes on, the threads are numbered through all rows without gaps (one division per thread instead of a
+        // shift) -- from three tenths on where the launch would otherwise take the one-unit-per-block kernel, which has
+        // its own addressing and is still the faster one below that when its rows end on 128-byte lines ([4096,1,96] o
+        // [1,1024,96], a quarter idle: 6.35 against 5.65 TB/s; [4096,1,132] o [1,1024,132], 48 % idle: 4.17 against 5.65;
+        // [4096,1,100] o [1,1024,100], 22 % idle and rows of 400 bytes: 4.9 against 5.6).
+        bool dense_drain = cn.stride[0][last] == 1;
+        for (int k = last - 1; k >= 0 && dense_drain; k--) dense_drain = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
+        const bool lean_candidate = plan.kind == PLAN_ROWS_BINARY && vec && large && dense_drain && !deep && A.strided_last == 0 && periodic == 0 && reused;
+        const bool whole_lines = ((uint64_t)A.L * sizeof(T)) % 128 == 0;      // rows that end on a 128-byte line
+        const bool flat_rows = vec_per_row < 256 && n_rows * vec_per_row < ((uint64_t)1 << 31) &&
+                               (lean_candidate && whole_lines ? vec_per_row * 10 <= (uint64_t)tpr * 7 : vec_per_row * 5 <= (uint64_t)tpr * 4);
+        if (flat_rows) {
+            A.flat_vpr = FastDiv((unsigned)vec_per_row);
+            row_groups = (n_rows * vec_per_row + 255) / 256;
+            A.row_groups = (unsigned)row_groups;
+            rpp = 0;                                            // no whole number of rows per unit: nothing below may assume one
+        }
         // a source that is constant along the innermost outer axis is the same memory in every pass of a block
         // when the block's rows never straddle that axis: the binary kernel then loads it once
         plan.hoist = 0;
@@ -344,7 +364,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         if (plan.kind == PLAN_ROWS_BINARY && last >= 1 && row_groups >= (uint64_t)passes) {
             int constant = 0;
             for (int j = 0; j < 2; j++) if (cn.stride[j + 1][last - 1] == 0) constant |= 1 << j;
-            if (constant) A.pass_rows = 1;
+            if (constant && !flat_rows) A.pass_rows = 1;
             // measured at steady state: loading the constant source once gains 2..14 % when a row fills the block
             // (256 threads) and loses 4..14 % when a block covers several rows per pass
             if (constant && vec && passes == 8 && !A.nt_loads && rpp == 1 && A.const_last == 0 && !deep &&
@@ -359,14 +379,14 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // drain that is a slice of a wider tensor measured 5 % slower this way)
         bool drain_dense = cn.stride[0][last] == 1;
         for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
-        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && periodic == 0 && reused) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && periodic == 0 && reused && !flat_rows) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
         // ... and of a program that is one constant
         if (plan.kind == PLAN_ROWS && c.nsrc == 0 && prog.n == 1 && prog.op[0] == I_SET && prog.src[0] == SRC_CONST0 && funset == 0 &&
-            vec && large && drain_dense && !deep) {
+            vec && large && drain_dense && !deep && !flat_rows) {
             plan.lean_fill = true;
             plan.fill_value = prog.consts[0];
             plan.grid = (unsigned)(row_groups * A.chunks);

@@ -278,7 +278,9 @@ def test_large_broadcast_outputs_one_unit_per_block(device, orc, dt):
             ta = on(device, a)
         out = Tensor._on_device(device, T, so)
         device.launch_broadcast(op, -1, out, ta, tb)
-        assert _lib.last_path() == "rows_vec_binary_lean", _lib.last_path()
+        # (rows of 65 or 129 vectors would leave half the lanes of the one-unit kernel idle: threads numbered through the rows)
+        flat = sa[-1] == 260 or (sa[-1] == 515 and dt == "f32")
+        assert _lib.last_path() == ("rows_vec_binary" if flat else "rows_vec_binary_lean"), _lib.last_path()
         f = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply, "divide": np.divide}[op]
         assert_bits(out.getData().reshape(so), f(a, b).astype(T), f"{op} {sa} {sb}")
         # ... and a slab through the oracle's own state machine
