@@ -486,6 +486,8 @@ struct LeanArgs {
     FastDiv outer[ROWS_FAST_OUTER];          // outer[0] is the innermost outer axis
     int base[3];
     int stride[3][ROWS_FAST_OUTER];
+    FastDiv flat_vpr;          // d > 1: threads numbered through the rows without gaps (RowsArgs::flat_vpr); the drain is dense,
+                               // so every block still writes one contiguous, aligned unit whatever the row length
 };
 // CONST bit j: source j does not change along a row (one element per row).  WIDE: a row spans at least a wavefront, so
 // its index is wave-uniform and is resolved on the scalar unit.
@@ -495,6 +497,11 @@ __global__ __launch_bounds__(256) void rows_binary_lean_kernel(LeanArgs A, T* __
     const unsigned rg = A.chunk_div.div(blockIdx.x), chunk = blockIdx.x - rg * A.chunks;
     const unsigned sub = threadIdx.x >> A.tpr_log2, lane = threadIdx.x & (tpr - 1);
     unsigned row = rg * rpp + sub, col = (chunk * tpr + lane) * (unsigned)V;
+    if (A.flat_vpr.d > 1) {
+        const unsigned f = blockIdx.x * 256u + threadIdx.x;
+        row = A.flat_vpr.div(f);
+        col = (f - row * A.flat_vpr.d) * (unsigned)V;
+    }
     const bool row_ok = row < A.n_rows;
     const bool live = row_ok && col < A.L;
     if (!row_ok) row = 0;                        // dead lanes get a valid address: the loads need no predicate

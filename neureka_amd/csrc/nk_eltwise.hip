@@ -349,12 +349,30 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         for (int k = last - 1; k >= 0 && dense_drain; k--) dense_drain = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
         const bool lean_candidate = plan.kind == PLAN_ROWS_BINARY && vec && large && dense_drain && !deep && A.strided_last == 0 && periodic == 0 && reused;
         const bool whole_lines = ((uint64_t)A.L * sizeof(T)) % 128 == 0;      // rows that end on a 128-byte line
-        const bool flat_rows = vec_per_row < 256 && n_rows * vec_per_row < ((uint64_t)1 << 31) &&
-                               (lean_candidate && whole_lines ? vec_per_row * 10 <= (uint64_t)tpr * 7 : vec_per_row * 5 <= (uint64_t)tpr * 4);
+        // the one-unit-per-block kernel numbers its threads through the rows as well (its drain is dense, so a block still
+        // writes one contiguous aligned unit): wherever a tenth of its lanes would idle or its rows do not end on a line
+        // (The sources a broadcast re-reads live in the L2 of each XCD.  Numbered by row and column chunk, the blocks an XCD
+        // gets -- every eighth -- keep to the same columns, so it holds an eighth of such a source; numbered through, they
+        // drift across the columns and every XCD ends up cycling through all of it.  With rows of more than a block that
+        // costs more than the idle lanes once the sources exceed what one L2 keeps: [64,1,4092] o [1,1024,4092], 16 MiB
+        // re-read, 5.6 -> 3.7 TB/s; 2 MiB and less, or rows of at most 256 vectors, gain: 5.4 -> 6.0 .. 6.4.)
+        uint64_t reread_bytes = 0;
+        for (int j = 0; j < c.nsrc; j++) {
+            uint64_t elems = 1;
+            bool reread = false;
+            for (int k = 0; k < cn.rank; k++) { if (cn.stride[j + 1][k] != 0) elems *= (uint64_t)cn.shape[k]; else if (cn.shape[k] > 1) reread = true; }
+            if (reread) reread_bytes += elems * sizeof(T);
+        }
+        const bool lean_flat = lean_candidate && !ragged && c.nsrc == 2 && A.const_last == 0 && n_rows * vec_per_row < ((uint64_t)1 << 31) &&
+                               (!whole_lines || vec_per_row * 10 <= (uint64_t)tpr * A.chunks * 9) &&
+                               (vec_per_row <= 256 || reread_bytes <= ((uint64_t)2 << 20));
+        const bool flat_rows = lean_flat || (vec_per_row < 256 && n_rows * vec_per_row < ((uint64_t)1 << 31) &&
+                               (lean_candidate && whole_lines ? vec_per_row * 10 <= (uint64_t)tpr * 7 : vec_per_row * 5 <= (uint64_t)tpr * 4));
         if (flat_rows) {
             A.flat_vpr = FastDiv((unsigned)vec_per_row);
             row_groups = (n_rows * vec_per_row + 255) / 256;
             A.row_groups = (unsigned)row_groups;
+            A.chunks = 1; A.chunk_div = FastDiv(1);             // a unit is 256 vectors of the launch, not a piece of a row
             rpp = 0;                                            // no whole number of rows per unit: nothing below may assume one
         }
         // a source that is constant along the innermost outer axis is the same memory in every pass of a block
@@ -379,7 +397,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         // drain that is a slice of a wider tensor measured 5 % slower this way)
         bool drain_dense = cn.stride[0][last] == 1;
         for (int k = last - 1; k >= 0 && drain_dense; k--) drain_dense = cn.stride[0][k] == cn.stride[0][k + 1] * (int64_t)cn.shape[k + 1];
-        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && periodic == 0 && reused && !flat_rows) {
+        if (plan.kind == PLAN_ROWS_BINARY && vec && large && drain_dense && !deep && A.strided_last == 0 && periodic == 0 && reused && (!flat_rows || lean_flat)) {
             plan.lean = true;
             plan.hoist = 0;
             plan.grid = (unsigned)(row_groups * A.chunks);
