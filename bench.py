@@ -248,6 +248,12 @@ def main():
         o64 = Tensor._on_device(dev, np.float64, (256, 1024, 512))
         hbm("broadcast_add_f64", 8 * (o64.size + a64.size + b64.size), dev.prepared_launch("broadcast", "add", -1, o64, a64, b64))
         for t in (a64, b64, o64): dev.free(t)
+        # the headline operation with an inner extent that is no power of two (rows of 2000 bytes)
+        a5 = Tensor.of(f32, (1024, 1, 500), rng.uniform(-1, 1, 1024 * 500).astype(f32)).to(dev)
+        b5 = Tensor.of(f32, (1, 2048, 500), rng.uniform(-1, 1, 2048 * 500).astype(f32)).to(dev)
+        o5 = Tensor._on_device(dev, f32, (1024, 2048, 500))
+        hbm("broadcast_add_rows_of_500", 4 * (o5.size + a5.size + b5.size), dev.prepared_launch("broadcast", "add", -1, o5, a5, b5))
+        for t in (a5, b5, o5): dev.free(t)
 
         # C2 backward: the reducing kernel, error [1024,2048,512] -> gradient [1024,1,512] (axis 1 summed) and [1,2048,512]
         err = Tensor._on_device(dev, f32, (1024, 2048, 512))
