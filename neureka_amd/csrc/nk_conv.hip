@@ -1338,6 +1338,7 @@ extern "C" int nk_convolution(nk_dev h, int d, int dtype, int rank, nk_buf drn, 
     if (int e = check_extent(dev, "nk_convolution(src2)", b, b_cfg, rank, eb)) return e;
     Cfg c0, c1, c2;
     load_cfg(c0, drn_cfg, rank); load_cfg(c1, a_cfg, rank); load_cfg(c2, b_cfg, rank);
+    tame_unravel(c0, rank, n);              // (the operands are read at positions derived from the drain's nd-index)
     return dtype == NK_F32 ? conv_typed<float>(dev, d, rank, drn, c0, a, c1, b, c2, n)
                            : conv_typed<double>(dev, d, rank, drn, c0, a, c1, b, c2, n);
 }

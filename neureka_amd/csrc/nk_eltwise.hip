@@ -135,6 +135,9 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     load_cfg(cfgs[0], c.drn_cfg, c.rank);
     cfgp[0] = &cfgs[0];
     for (int j = 0; j < c.nsrc; j++) { load_cfg(cfgs[j + 1], c.src_cfg[j], c.rank); cfgp[j + 1] = &cfgs[j + 1]; }
+    // every operand that unravels the flat index itself: a table that would leave its view becomes the row-major one
+    tame_unravel(cfgs[0], c.rank, c.n);
+    for (int j = 0; j < c.nsrc; j++) if (c.own[j]) tame_unravel(cfgs[j + 1], c.rank, c.n);
     bool axis_on[MAX_OPERANDS][NK_MAX_RANK];
     for (int k = 0; k < NK_MAX_RANK; k++) axis_on[0][k] = true;
     for (int j = 0; j < c.nsrc; j++)

@@ -134,6 +134,15 @@ struct Canon {
 bool canonicalize(Canon& out, int rank, const int* iter_shape, int n_operands,
                   const Cfg* const* cfgs, const bool (*axis_on)[NK_MAX_RANK], const bool* own_unravel);
 
+// The reference turns a flat index into an nd-index with idx[k] = i / indicesMap[k]; i %= indicesMap[k], axis 0 first.
+// With a table that does not descend like the row-major one this can leave the view's own shape: the column-major
+// table the reference gives a slice of a transposed (column-major) matrix, [1, rows], makes idx[0] = i
+// (Slice.java:88, NDConfiguration.java:109-132).  There the reference has one defined result, that of a CPU workload
+// which starts every operand at nd-index 0 and advances all of them in row-major order (CPUBiElementWise.java:99-142;
+// a workload that starts elsewhere unravels its start with the broken table) -- i.e. the row-major table.  Replaces
+// the table of `c` by the row-major one of its shape when some flat index below n would leave the shape and says so;
+// a table that stays inside (the row-major one, a virtual one, hand-made ones) is kept and evaluated literally.
+bool tame_unravel(Cfg& c, int rank, int64_t n);
 int check_cfg(const char* what, const int32_t* cfg, int rank);
 // Verifies on the host that every element the view can address lies inside one live allocation of
 // the device that contains `buf`; an out-of-range view is reported instead of faulting the GPU.

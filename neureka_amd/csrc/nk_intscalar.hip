@@ -180,6 +180,7 @@ extern "C" int nk_scalarization_int(nk_dev h, int op_id, int d, int dtype, int r
     }
     Cfg c0, c1;
     load_cfg(c0, drn_cfg, rank); load_cfg(c1, src_cfg, rank);
+    tame_unravel(c0, rank, n); tame_unravel(c1, rank, n);
     const int mode = op_id * 3 + (d + 1);
     switch (dtype) {
         case NK_I32: return int_scalar_typed<int32_t>(dev, mode, value, rank, drn, c0, src, c1, n);

@@ -396,6 +396,7 @@ extern "C" int nk_broadcast(nk_dev h, int op_id, int d, int dtype, int rank, nk_
     A.rank = rank; A.op = op_id; A.d = d;
     Cfg c1, c2;
     load_cfg(A.c0, drn_cfg, rank); load_cfg(c1, a_cfg, rank); load_cfg(c2, b_cfg, rank);
+    tame_unravel(A.c0, rank, n);            // (the sources follow the drain's nd-index: their tables play no role)
     A.base1 = 0; A.base2 = 0; A.nred = 0;
     for (int k = 0; k < rank; k++) {
         const int e0 = A.c0.shape[k], e1 = c1.shape[k], e2 = c2.shape[k];

@@ -86,6 +86,21 @@ int check_extent(Device* dev, const char* what, nk_buf buf, const int32_t* cfg, 
     return check_range(dev, what, buf, 0, (uint64_t)(hi + 1) * elem_bytes);
 }
 
+bool tame_unravel(Cfg& c, int rank, int64_t n) {
+    int64_t range = n;                                   // the index that reaches axis k lies in [0, range)
+    bool inside = true;
+    for (int k = 0; k < rank && inside; k++) {
+        const int64_t m = c.imap[k];
+        if (m == 0) continue;                            // virtual: index 0 on this axis, the flat index passes on whole
+        if (range > 0 && (range - 1) / m > (int64_t)c.shape[k] - 1) inside = false;
+        if (m < range) range = m;
+    }
+    if (inside) return false;
+    int64_t prod = 1;
+    for (int k = rank - 1; k >= 0; k--) { c.imap[k] = (int)prod; prod *= c.shape[k]; }
+    return true;
+}
+
 bool canonicalize(Canon& out, int rank, const int* iter_shape, int n_operands, const Cfg* const* cfgs,
                   const bool (*axis_on)[NK_MAX_RANK], const bool* own_unravel) {
     if (n_operands > MAX_OPERANDS) return false;

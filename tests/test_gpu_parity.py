@@ -314,6 +314,81 @@ def test_views_take_the_fast_paths_and_match(device, orc, dt):
     assert_bits(out.getData(), orc.activation("quad", -1, np.zeros(out.size, dtype=F[dt]), cfg(out), b3.reshape(-1), cfg(v3)), "perm3")
 
 
+def test_slices_of_transposed_tensors_walk_in_row_major_order(device, orc):
+    """A slice of a transposed (column-major) matrix carries the column-major indicesMap [1, rows] (Slice.java:88),
+    with which idx[0] = i / 1 leaves the view for every flat index beyond the first column.  The one result the
+    reference defines there is that of a CPU workload from index 0 (every operand starts at nd-index 0 and advances
+    in row-major order): what the oracle computes in one piece, what numpy computes -- as source, as drain, for every
+    kernel family that unravels a flat index, and never an access outside the view."""
+    rng = np.random.default_rng(77)
+    for dt in ("f32", "f64"):
+        T = F[dt]
+        for R, Cn in ((8, 15), (130, 517), (1024, 2050)):
+            say("slice of a transposed tensor", dt, R, Cn)
+            a = rng.standard_normal((R, Cn)).astype(T); b = rng.standard_normal((Cn, R)).astype(T)
+            ta, tb = on(device, a), on(device, b)
+            va, vb = ta[1::2, 3::2], tb.T()[1::2, 3::2]
+            assert cfg(vb).tolist()[4:6] == [1, va.shape[0]]                      # the column-major table
+            na, nb = a[1::2, 3::2], b.T[1::2, 3::2]
+            so = va.shape
+            n = int(np.prod(so))
+            dense = orc.dense_cfg(list(so))
+            # both kinds of source, dense drain
+            out = Tensor._on_device(device, T, so)
+            device.launch_elementwise("subtract", -1, out, va, vb)
+            assert _lib.last_path() != "literal", _lib.last_path()
+            assert_bits(out.getData().reshape(so), na - nb, "a - b^T, slices")
+            assert_bits(out.getData(), orc.elementwise("subtract", -1, np.zeros(n, dtype=T), dense, a.reshape(-1), cfg(va), b.reshape(-1), cfg(vb)), "oracle")
+            device.launch_scalarization("multiply", -1, out, vb, 3.0)
+            assert_bits(out.getData().reshape(so), nb * T(3.0), "3 b^T")
+            device.launch_activation("relu", -1, out, vb)
+            assert_bits(out.getData(), orc.activation("relu", -1, np.zeros(n, dtype=T), dense, b.reshape(-1), cfg(vb)), "relu")
+            fn = Function.of("I[0]*I[1]+I[0]")
+            got = device.optimizedFunctionOf(fn, "fma")(vb, va)
+            assert_bits(got.getData().reshape(so), nb * na + nb, "fused")
+            # the drain is such a view: only its elements change
+            parent = rng.standard_normal((Cn, R)).astype(T)
+            tp = on(device, parent)
+            drain = tp.T()[1::2, 3::2]
+            device.launch_elementwise("add", -1, drain, va, vb)
+            want = parent.copy(); want.T[1::2, 3::2] = na + nb
+            assert_bits(tp.getData().reshape(Cn, R), want, "drain view")
+            device.launch_scalar_fill(drain, 7.0)
+            want.T[1::2, 3::2] = 7.0
+            assert_bits(tp.getData().reshape(Cn, R), want, "fill of a drain view")
+            # broadcast backward into such a drain: the error [r, c] summed over axis 0 into a row [1, c] of the view
+            e = rng.integers(-3, 4, so).astype(T)
+            te = on(device, e)
+            row = tb.T()[1:2, 3::2]                                                # column-major table [1, 1]
+            assert cfg(row).tolist()[4:6] == [1, 1]
+            zeros = Tensor._on_device(device, T, (so[0], 1))
+            device.launch_broadcast("add", 0, row, zeros, te)
+            want_b = b.copy(); want_b.T[1:2, 3::2] = e.sum(axis=0, keepdims=True)
+            assert_bits(tb.getData().reshape(Cn, R), want_b, "backward into a drain view")
+        # integers: the indexed kernel
+        say("slice of a transposed int32 tensor")
+        x = rng.integers(-1000, 1000, (15, 8)).astype(np.int32)
+        tx = on(device, x)
+        vx = tx.T()[1::2, 3::2]
+        out = Tensor._on_device(device, np.int32, vx.shape)
+        device.launch_scalarization("multiply", -1, out, vx, 3)
+        assert (out.getData().reshape(vx.shape) == x.T[1::2, 3::2] * 3).all()
+    # convolution into a drain view
+    say("convolution into a slice of a transposed tensor")
+    img = rng.integers(-3, 4, (1, 1, 12, 17)).astype(np.float32); ker = rng.integers(-2, 3, (1, 1, 3, 3)).astype(np.float32)
+    ti, tk = on(device, img), on(device, ker)
+    parent = np.zeros((1, 1, 30, 20), dtype=np.float32)
+    tp = on(device, parent)
+    drain = tp.permute(0, 1, 3, 2)[0:1, 0:1, 0:10, 0:15]
+    device.launch_convolution(-1, drain, ti, tk)
+    full = np.zeros((10, 15), dtype=np.float32)
+    for ky in range(3):
+        for kx in range(3):
+            full += img[0, 0, ky:ky + 10, kx:kx + 15] * ker[0, 0, ky, kx]
+    want = parent.copy(); want.transpose(0, 1, 3, 2)[0, 0, 0:10, 0:15] = full
+    assert_bits(tp.getData().reshape(parent.shape), want, "convolution drain view")
+
+
 def test_exotic_descriptor_falls_back_to_the_literal_formula(device, orc):
     """A descriptor whose indicesMap is not the row-major table of its shape cannot be reduced to
     base + strides: the literal kernel evaluates NDConfiguration.indexOfIndex (the formula the 20 rows of
