@@ -236,4 +236,26 @@ def test_convolution_of_an_8_gib_image(device):
         assert float(got.sum(dtype=np.float64)) == total
         free(device, y)
         del got
-    free(device, tx)
+    # 2047 images of [1024, 1024] in one launch: the planes behind byte offset 4 GiB
+    B, S = 2047, 1024
+    say("max size batched convolution", (B, S, S), (1, 3, 3))
+    x3 = x.reshape(-1)[:B * S * S].reshape(B, S, S)
+    O = S - 2
+    full_rows = x3.sum(axis=2, dtype=np.float64)
+    total = 0.0
+    for kx in range(3):
+        rows = full_rows - x3[:, :, :kx].sum(axis=2, dtype=np.float64) - x3[:, :, kx + O:].sum(axis=2, dtype=np.float64)
+        for ky in range(3):
+            total += float(k[ky, kx]) * float(rows[:, ky:ky + O].sum())
+    vx = Tensor(f32, NDConfiguration.ofShape((B, S, S)), None); vx._set_data(tx._data, device)
+    y = vx.conv(on(device, k, (1, 3, 3)))
+    assert _lib.last_path() == "simple2d_window", _lib.last_path()
+    got = y.getData().reshape(B, O, O)
+    for lo, hi in ((0, 2), (1023, 1026), (B - 2, B)):
+        want = np.zeros((hi - lo, O, O), dtype=f32)
+        for ky in range(3):
+            for kx in range(3):
+                want += x3[lo:hi, ky:ky + O, kx:kx + O] * k[ky, kx]
+        same(got[lo:hi], want, f"images {lo}:{hi}")
+    assert float(got.sum(dtype=np.float64)) == total
+    free(device, y, tx)
