@@ -259,3 +259,51 @@ def test_convolution_of_an_8_gib_image(device):
         same(got[lo:hi], want, f"images {lo}:{hi}")
     assert float(got.sum(dtype=np.float64)) == total
     free(device, y, tx)
+
+
+def test_channel_convolution_with_autograd_over_8_gib(device):
+    """[511, 2048, 2048] x [511, 3, 3] -> [1, 2046, 2046] and both gradients: channels behind byte offset 4 GiB, a
+    gradient of 8 GiB.  Small integers keep every sum exact in any order: bands of rows / channels against numpy, and the
+    sum of each whole result against its closed form."""
+    from scipy.signal import convolve2d
+    rng = np.random.default_rng(39)
+    Cc, S, O = 511, 2048, 2046
+    x = big(rng, Cc * S * S, f32, integers=(-3, 3)).reshape(Cc, S, S)
+    k = rng.integers(-2, 3, (Cc, 3, 3)).astype(f32)
+    e = rng.integers(-1, 2, (1, O, O)).astype(f32)
+    tx = on(device, x).setRqsGradient(True); tk = on(device, k).setRqsGradient(True)
+    say("max size channel convolution forward")
+    y = tx.conv(tk)
+    print("[path]", _lib.last_path(), flush=True)
+    assert tuple(y.shape) == (1, O, O)
+    got = y.getData().reshape(O, O)
+    for lo, hi in ((0, 8), (1019, 1027), (O - 8, O)):
+        want = np.zeros((hi - lo, O), dtype=np.float64)
+        for ky in range(3):
+            for kx in range(3):
+                want += np.einsum("cyx,c->yx", x[:, lo + ky:hi + ky, kx:kx + O], k[:, ky, kx], dtype=np.float64)
+        same(got[lo:hi], want.astype(f32), f"forward rows {lo}:{hi}")
+    full_rows = x.sum(axis=2, dtype=np.float64)                          # [c, y]
+    total = 0.0
+    for kx in range(3):
+        rows = full_rows - x[:, :, :kx].sum(axis=2, dtype=np.float64) - x[:, :, kx + O:].sum(axis=2, dtype=np.float64)
+        for ky in range(3):
+            total += float(np.dot(k[:, ky, kx].astype(np.float64), rows[:, ky:ky + O].sum(axis=1)))
+    assert float(got.sum(dtype=np.float64)) == total
+    say("max size channel convolution backward")
+    y.backward(on(device, e))
+    gx, gk = tx.gradient, tk.gradient
+    assert tuple(gx.shape) == (Cc, S, S) and tuple(gk.shape) == (Cc, 3, 3)
+    gxh = gx.getData().reshape(Cc, S, S)
+    for c in (0, 1, 255, 256, 257, Cc - 1):
+        same(gxh[c], convolve2d(e[0].astype(np.float64), k[c].astype(np.float64), mode="full").astype(f32), f"input gradient, channel {c}")
+    assert float(gxh.sum(dtype=np.float64)) == float(e.sum(dtype=np.float64)) * float(k.sum(dtype=np.float64))
+    del gxh
+    gkh = gk.getData().reshape(Cc, 3, 3)
+    e64 = e[0].astype(np.float64)
+    for c in (0, 1, 255, 256, 257, Cc - 1):
+        want = np.array([[float((e64 * x[c, ky:ky + O, kx:kx + O]).sum()) for kx in range(3)] for ky in range(3)])
+        same(gkh[c], want.astype(f32), f"kernel gradient, channel {c}")
+    planes = x.sum(axis=0, dtype=np.float64)
+    assert float(gkh.sum(dtype=np.float64)) == sum(float((e64 * planes[ky:ky + O, kx:kx + O]).sum()) for ky in range(3) for kx in range(3))
+    free(device, y, gx, gk, tx, tk)
