@@ -18,6 +18,7 @@
 //
 // Column-major operands are handled as the transposed row-major problem C^T = B^T A^T.
 #include "nk_internal.h"
+#include <mutex>
 
 namespace nk {
 
@@ -434,6 +435,150 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
     }
 }
 
+// Large products whose 256x256 tiles fill the machine: one block per compute unit, ONE wavefront per SIMD that owns
+// 128x128 of the block's 256x256 tile as 4x4 accumulators (256 accumulation registers) -- the layout the part's 512
+// registers per lane are made for.  Against the 128x128 kernel (two blocks of 64x64 wavefronts per compute unit) a
+// multiply-add needs half the LDS traffic, a slice of depth 32 is 256 multiply-adds per wavefront between barriers
+// instead of 64, and no second block competes for the matrix core in the same phase.  Same fragments, same order of
+// the k steps inside a chunk: the sums are those of matmul_mfma_kernel bit for bit.  LDS: two buffers of
+// A 256 x 36 and B 32 x 260 floats, 137 KiB (dynamic).
+namespace big {
+constexpr int TM = 256, TN = 256;
+constexpr int AP = BK + 4, BP = TN + 4;
+constexpr int LDS_FLOATS = 2 * TM * AP + 2 * BK * BP;
+struct BigFrag {
+    f32x4 a[4];            // rows wm + 32 i + l32, k = 8c + 4h .. + 3
+    float b[4][4];         // [j][t]: column wn + 32 j + l32, k = 8c + 4h + t
+};
+}
+
+template <bool OVERWRITE>
+__global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, const float* __restrict__ A,
+                                                                const float* __restrict__ B, float* __restrict__ C) {
+    using namespace big;
+    extern __shared__ __attribute__((aligned(16))) float big_lds[];
+    float* const As0 = big_lds;                            // [2][TM * AP]
+    float* const Bs0 = big_lds + 2 * TM * AP;              // [2][BK * BP]
+    int tm, tn;
+    tile_of_block(g, (int)blockIdx.x, tm, tn);
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 128, wn = (wave & 1) * 128;
+    const int l32 = lane & 31, h = lane >> 5;
+    const float* Ag = A + (int64_t)tm * TM * g.K;
+    const float* Bg = B + (int64_t)tn * TN;
+    // global -> register staging: A slice 256x32 and B slice 32x256, 8 float4 each per thread
+    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 i
+    const int b_row = tid >> 6, b_col = (tid & 63) * 4;     // rows b_row + 4 i
+    f32x4 ra[8], rb[8];
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 4 * i) * g.N + b_col);
+        }
+    };
+    auto store_lds = [&](int buf) {
+        float* as = As0 + buf * (TM * AP);
+        float* bs = Bs0 + buf * (BK * BP);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            *(f32x4*)(&as[(a_row + 32 * i) * AP + a_col]) = ra[i];
+            *(f32x4*)(&bs[(b_row + 4 * i) * BP + b_col]) = rb[i];
+        }
+    };
+    auto read_frag = [&](BigFrag& f, int buf, int c) {
+        const float* as = As0 + buf * (TM * AP);
+        const float* bs = Bs0 + buf * (BK * BP);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f.a[i] = *(const f32x4*)(&as[(wm + 32 * i + l32) * AP + 8 * c + 4 * h]);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) f.b[j][t] = bs[(8 * c + 4 * h + t) * BP + wn + 32 * j + l32];
+    };
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    auto mma = [&](const BigFrag& f) {
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][t], f.b[j][t], acc[i][j], 0, 0, 0);
+    };
+    // The pipeline of matmul_mfma_kernel with chunks of 64 multiply-adds: the 20 LDS reads of chunk c + 1 follow the
+    // first ten multiply-adds of chunk c in pairs; in the third chunk each of the next sixteen multiply-adds is
+    // followed by one LDS write of the staged slice kt + 1 and one global request for slice kt + 2.
+#define NK_BIG_READS NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); \
+                     NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2)
+#define NK_BIG_PLAIN NK_BIG_READS; NK_MFMA(54); NK_FENCE
+#define NK_BIG_WR4 NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1)
+#define NK_BIG_WRITE_AND_REQUEST NK_BIG_READS; NK_BIG_WR4; NK_BIG_WR4; NK_BIG_WR4; NK_BIG_WR4; NK_MFMA(38); NK_FENCE
+    const int nk = g.K / BK;
+    BigFrag f0, f1;
+    load_global(0);
+    store_lds(0);
+    load_global(nk > 1 ? BK : 0);                          // slice 1 waits in the staging registers
+    __syncthreads();
+    read_frag(f0, 0, 0);
+    NK_FENCE;
+    for (int kt = 0; kt + 1 < nk; kt++) {
+        const int cur = kt & 1;
+        read_frag(f1, cur, 1);
+        mma(f0);
+        NK_BIG_PLAIN;
+        read_frag(f0, cur, 2);
+        mma(f1);
+        NK_BIG_PLAIN;
+        read_frag(f1, cur, 3);
+        store_lds(cur ^ 1);
+        load_global((kt + 2 < nk ? kt + 2 : nk - 1) * BK);
+        mma(f0);
+        NK_BIG_WRITE_AND_REQUEST;
+        __syncthreads();
+        NK_FENCE;
+        read_frag(f0, cur ^ 1, 0);
+        mma(f1);
+        NK_BIG_PLAIN;
+    }
+    {
+        const int cur = (nk - 1) & 1;
+        read_frag(f1, cur, 1);
+        mma(f0);
+        NK_BIG_PLAIN;
+        read_frag(f0, cur, 2);
+        mma(f1);
+        NK_BIG_PLAIN;
+        read_frag(f1, cur, 3);
+        mma(f0);
+        NK_BIG_PLAIN;
+        mma(f1);
+    }
+    // The result leaves straight from the accumulators: accumulator v of a 32x32 tile sits at row 8*(v/4) + 4*h + v%4,
+    // column l32, so a store instruction writes 128 contiguous bytes of two rows; the address is a wave-uniform part
+    // plus one 32-bit offset per lane.  Accumulating, the old values of one row of four sub-tiles are requested together.
+    float* const Cg = C + (int64_t)tm * TM * g.N + tn * TN;
+    const unsigned lane_off = (unsigned)((wm + 4 * h) * g.N + wn + l32);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float old[4][16];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) old[j][v] = OVERWRITE ? 0.0f : (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) (Cg + (int64_t)(32 * i + 8 * (v >> 2) + (v & 3)) * g.N + 32 * j)[lane_off] = OVERWRITE ? acc[i][j][v] : old[j][v] + acc[i][j][v];
+    }
+}
+
 // C[i] += (or, overwriting, =) part_0[i] + part_1[i] + ... in that order (the parts of a SPLIT product)
 template <typename T>
 __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int parts, int overwrite, const T* __restrict__ P, T* __restrict__ C) {
@@ -643,6 +788,31 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
     const bool edge = !whole_tiles && M * K * N >= mfma_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
     if (whole_tiles || edge) {
         const float* Ap = (const float*)A; const float* Bp = (const float*)B; float* Cp = (float*)C;
+        // 256x256 tiles, one block per compute unit, when they fill the machine in whole rounds (or many rounds) and the
+        // tiles are deep enough for the first fetch and the write-back not to weigh
+        if (whole_tiles && M % big::TM == 0 && N % big::TN == 0 && K / BK >= 32) {
+            const int64_t cus = dev->props.multiProcessorCount;
+            const int64_t tiles = (M / big::TM) * (N / big::TN);
+            if (tiles >= cus && (tiles % cus == 0 || tiles >= 4 * cus)) {
+                MfmaArgs gb = g;
+                gb.tiles_m = (int)(M / big::TM); gb.tiles_n = (int)(N / big::TN);
+                gb.group_rows = gb.tiles_m < 4 ? gb.tiles_m : 4;
+                constexpr int lds_bytes = big::LDS_FLOATS * (int)sizeof(float);
+                static std::once_flag big_once;
+                static hipError_t big_attr = hipSuccess;
+                std::call_once(big_once, [&]() {
+                    big_attr = hipFuncSetAttribute((const void*)matmul_mfma_big_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+                    if (big_attr == hipSuccess)
+                        big_attr = hipFuncSetAttribute((const void*)matmul_mfma_big_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+                });
+                NK_HIP(big_attr);
+                if (overwrite) hipLaunchKernelGGL(matmul_mfma_big_kernel<true>, dim3((unsigned)tiles), dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                else           hipLaunchKernelGGL(matmul_mfma_big_kernel<false>, dim3((unsigned)tiles), dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                NK_HIP(hipGetLastError());
+                set_path("mfma_big");
+                return NK_OK;
+            }
+        }
         bool streamed = false;
         const int rc = launch_mfma<float>(dev, g, BK, Cp, [&](bool split, dim3 grid, float* P) {
             if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);

@@ -169,7 +169,7 @@ def test_config4_matmul_full_size(device, mkn):
     A = rng.integers(-3, 4, (M, K)).astype(f32); B = rng.integers(-3, 4, (K, N)).astype(f32)
     ta, tb = on(device, A), on(device, B)
     c = ta.matMul(tb)
-    assert _lib.last_path() == ("mfma" if K == 4096 else "mfma_stream")      # few k-slices per tile: the blocks walk the tiles
+    assert _lib.last_path() == ("mfma_big" if K == 4096 else "mfma_stream")  # 256 tiles of 256 x 256: one per compute unit; few k-slices per tile: the blocks walk the tiles
     got = c.items.reshape(M, N)
     rows = rng.choice(M, 48, replace=False)
     assert (got[rows] == A[rows].astype(np.float64) @ B.astype(np.float64)).all()

@@ -1661,6 +1661,45 @@ def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mk
         assert (a.view(np.uint32 if dt == "f32" else np.uint64) == g.view(np.uint32 if dt == "f32" else np.uint64)).all()
 
 
+@pytest.mark.parametrize("mkn", [(4096, 1024, 4096), (2048, 2048, 8192), (4096, 1056, 4096), (8192, 1024, 8192)])
+def test_matmul_256_tiles_one_wavefront_per_simd(device, mkn):
+    """Large f32 products whose 256 x 256 tiles fill the machine take the kernel with one wavefront per SIMD.  It sums
+    in the order of the 128 x 128 kernel, which computes the left half of the same product (half as many tiles: not
+    enough for the large kernel) -- bit for bit; integer data are exact against numpy; both entry points, both layouts."""
+    M, K, N = mkn
+    rng = np.random.default_rng(61)
+    say("matmul 256 tiles", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    ta, tb = on(device, A), on(device, B)
+    c = on(device, np.full((M, N), np.nan, dtype=np.float32))
+    device.launch_matmul(True, M, K, N, ta, tb, c, accumulate=False)
+    assert _lib.last_path() == "mfma_big", _lib.last_path()
+    got = c.getData().reshape(M, N)
+    assert not np.isnan(got).any()
+    if (M // 256) * (N // 512) < device.maxComputeUnits():       # (four rounds of tiles: the half is a large product itself)
+        half = np.ascontiguousarray(B[:, :N // 2])
+        th = on(device, half)
+        ch = on(device, np.zeros((M, N // 2), dtype=np.float32))
+        device.launch_matmul(True, M, K, N // 2, ta, th, ch)
+        assert _lib.last_path() == "mfma", _lib.last_path()
+        assert_bits(got[:, :N // 2], ch.getData().reshape(M, N // 2), "left half against the 128 x 128 kernel")
+    rows = rng.choice(M, 32, replace=False)
+    ref = A[rows].astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-5 * (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(got[rows] - ref) <= bound).all()
+    # C += A B on top of the result: exactly twice it (the sum is the same, added to itself)
+    device.launch_matmul(True, M, K, N, ta, tb, c)
+    assert _lib.last_path() == "mfma_big"
+    assert_bits(c.getData().reshape(M, N), 2 * got, "accumulating")
+    say("matmul 256 tiles, integer data, column major", mkn)
+    Ai = rng.integers(-3, 4, (M, K)).astype(np.float32); Bi = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    tai, tbi = on(device, Ai.T.copy()), on(device, Bi.T.copy())
+    ci = on(device, np.zeros((N, M), dtype=np.float32))
+    device.launch_matmul(False, M, K, N, tai, tbi, ci, accumulate=False)
+    assert _lib.last_path() == "mfma_big"
+    assert_bits(ci.getData().reshape(N, M), (Ai @ Bi).T.copy(), "column major")
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
