@@ -1,5 +1,7 @@
 // Dense matrix multiplication C[M,N] += A[M,K] @ B[K,N].
 //
+//   mfma_big f32, M % 256 == 0, N % 256 == 0, K % 32 == 0, K >= 1024 and enough 256x256 tiles to fill the compute
+//            units in whole rounds: one block per compute unit, one wavefront per SIMD with 4x4 accumulators.
 //   mfma     f32, M % 128 == 0, N % 128 == 0, K % 32 == 0: 128x128 block tiles, four wavefronts in a
 //            2x2 arrangement, each owning a 64x64 sub-tile as 2x2 v_mfma_f32_32x32x2_f32
 //            accumulators; A and B k-slices of depth 32 are staged through double-buffered LDS with
