@@ -2,6 +2,7 @@
 //
 //   mfma_big f32, M % 256 == 0, N % 256 == 0, K % 32 == 0, K >= 1024 and enough 256x256 tiles to fill the compute
 //            units in whole rounds: one block per compute unit, one wavefront per SIMD with 4x4 accumulators.
+//   mfma_big_edge  the same kernel for large shapes that are not whole tiles: clamped edges, zeroed k tail.
 //   mfma     f32, M % 128 == 0, N % 128 == 0, K % 32 == 0: 128x128 block tiles, four wavefronts in a
 //            2x2 arrangement, each owning a 64x64 sub-tile as 2x2 v_mfma_f32_32x32x2_f32
 //            accumulators; A and B k-slices of depth 32 are staged through double-buffered LDS with
@@ -454,7 +455,10 @@ struct BigFrag {
 };
 }
 
-template <bool OVERWRITE>
+// EDGE: M, N, K need not be multiples of the tile -- as in matmul_mfma_kernel<true>: loads through buffer descriptors
+// over the whole matrices, rows past the edge clamped, columns past it left as they come (both only feed results that
+// are not stored), the k tail zeroed in both operands, element-wise guarded stores.
+template <bool OVERWRITE, bool EDGE = false>
 __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, const float* __restrict__ A,
                                                                 const float* __restrict__ B, float* __restrict__ C) {
     using namespace big;
@@ -473,16 +477,38 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
     const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 i
     const int b_row = tid >> 6, b_col = (tid & 63) * 4;     // rows b_row + 4 i
     f32x4 ra[8], rb[8];
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 4), 0x00020000);
     auto load_global = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 4 * i) * g.N + b_col);
+            if (!EDGE) {
+                ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+                rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 4 * i) * g.N + b_col);
+            } else {
+                int row = tm * TM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
+                const int ka = k0 + a_col;
+                ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * g.K + ka) * 4u, 0, 0)));
+                const int kb = k0 + b_row + 4 * i;
+                const int krow = kb < g.K ? kb : g.K - 1;
+                rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * g.N + tn * TN + b_col) * 4u, 0, 0)));
+            }
         }
     };
-    auto store_lds = [&](int buf) {
+    // k0: the slice the staging registers hold.  The k tail is zeroed here, a slice after the request, and only in the
+    // one slice that has a tail (a block-uniform branch): zeroing at the request would make every slice wait for its loads.
+    auto store_lds = [&](int buf, int k0) {
         float* as = As0 + buf * (TM * AP);
         float* bs = Bs0 + buf * (BK * BP);
+        if (EDGE && k0 + BK > g.K) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (k0 + a_col + e >= g.K) ra[i][e] = 0.0f;
+                if (k0 + b_row + 4 * i >= g.K) rb[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             *(f32x4*)(&as[(a_row + 32 * i) * AP + a_col]) = ra[i];
@@ -522,10 +548,10 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
 #define NK_BIG_PLAIN NK_BIG_READS; NK_MFMA(54); NK_FENCE
 #define NK_BIG_WR4 NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1)
 #define NK_BIG_WRITE_AND_REQUEST NK_BIG_READS; NK_BIG_WR4; NK_BIG_WR4; NK_BIG_WR4; NK_BIG_WR4; NK_MFMA(38); NK_FENCE
-    const int nk = g.K / BK;
+    const int nk = (g.K + BK - 1) / BK;
     BigFrag f0, f1;
     load_global(0);
-    store_lds(0);
+    store_lds(0, 0);
     load_global(nk > 1 ? BK : 0);                          // slice 1 waits in the staging registers
     __syncthreads();
     read_frag(f0, 0, 0);
@@ -539,7 +565,7 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
         mma(f1);
         NK_BIG_PLAIN;
         read_frag(f1, cur, 3);
-        store_lds(cur ^ 1);
+        store_lds(cur ^ 1, (kt + 1) * BK);
         load_global((kt + 2 < nk ? kt + 2 : nk - 1) * BK);
         mma(f0);
         NK_BIG_WRITE_AND_REQUEST;
@@ -567,6 +593,28 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
     // plus one 32-bit offset per lane.  Accumulating, the old values of one row of four sub-tiles are requested together.
     float* const Cg = C + (int64_t)tm * TM * g.N + tn * TN;
     const unsigned lane_off = (unsigned)((wm + 4 * h) * g.N + wn + l32);
+    if (EDGE && ((tm + 1) * TM > g.M || (tn + 1) * TN > g.N)) {       // a tile on the edge (the same for the whole block)
+        const int rows = g.M - tm * TM - (wm + 4 * h), cols = g.N - tn * TN - (wn + l32);   // what is left of C from the lane's first element
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float old[4][16];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = 32 * i + 8 * (v >> 2) + (v & 3);
+                    old[j][v] = (OVERWRITE || r >= rows || 32 * j >= cols) ? 0.0f : (Cg + (int64_t)r * g.N + 32 * j)[lane_off];
+                }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int r = 32 * i + 8 * (v >> 2) + (v & 3);
+                    if (r < rows && 32 * j < cols) (Cg + (int64_t)r * g.N + 32 * j)[lane_off] = OVERWRITE ? acc[i][j][v] : old[j][v] + acc[i][j][v];
+                }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         float old[4][16];
@@ -792,26 +840,34 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         const float* Ap = (const float*)A; const float* Bp = (const float*)B; float* Cp = (float*)C;
         // 256x256 tiles, one block per compute unit, when they fill the machine in whole rounds (or many rounds) and the
         // tiles are deep enough for the first fetch and the write-back not to weigh
-        if (whole_tiles && M % big::TM == 0 && N % big::TN == 0 && K / BK >= 32) {
+        if (K >= 32 * BK) {
+            const bool whole_big = whole_tiles && M % big::TM == 0 && N % big::TN == 0;
             const int64_t cus = dev->props.multiProcessorCount;
-            const int64_t tiles = (M / big::TM) * (N / big::TN);
-            if (tiles >= cus && (tiles % cus == 0 || tiles >= 4 * cus)) {
+            const int64_t tiles = ((M + big::TM - 1) / big::TM) * ((N + big::TN - 1) / big::TN);
+            if ((whole_big || edge) && tiles >= cus && (tiles % cus == 0 || tiles >= 4 * cus)) {
                 MfmaArgs gb = g;
-                gb.tiles_m = (int)(M / big::TM); gb.tiles_n = (int)(N / big::TN);
+                gb.tiles_m = (int)((M + big::TM - 1) / big::TM); gb.tiles_n = (int)((N + big::TN - 1) / big::TN);
                 gb.group_rows = gb.tiles_m < 4 ? gb.tiles_m : 4;
                 constexpr int lds_bytes = big::LDS_FLOATS * (int)sizeof(float);
                 static std::once_flag big_once;
                 static hipError_t big_attr = hipSuccess;
                 std::call_once(big_once, [&]() {
-                    big_attr = hipFuncSetAttribute((const void*)matmul_mfma_big_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-                    if (big_attr == hipSuccess)
-                        big_attr = hipFuncSetAttribute((const void*)matmul_mfma_big_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+                    const void* kernels[4] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
+                                              (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>};
+                    for (const void* k : kernels)
+                        if (big_attr == hipSuccess) big_attr = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
                 });
                 NK_HIP(big_attr);
-                if (overwrite) hipLaunchKernelGGL(matmul_mfma_big_kernel<true>, dim3((unsigned)tiles), dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
-                else           hipLaunchKernelGGL(matmul_mfma_big_kernel<false>, dim3((unsigned)tiles), dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                const dim3 grid((unsigned)tiles);
+                if (whole_big) {
+                    if (overwrite) hipLaunchKernelGGL((matmul_mfma_big_kernel<true, false>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL((matmul_mfma_big_kernel<false, false>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                } else {
+                    if (overwrite) hipLaunchKernelGGL((matmul_mfma_big_kernel<true, true>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL((matmul_mfma_big_kernel<false, true>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                }
                 NK_HIP(hipGetLastError());
-                set_path("mfma_big");
+                set_path(whole_big ? "mfma_big" : "mfma_big_edge");
                 return NK_OK;
             }
         }

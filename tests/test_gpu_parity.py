@@ -1700,6 +1700,40 @@ def test_matmul_256_tiles_one_wavefront_per_simd(device, mkn):
     assert_bits(ci.getData().reshape(N, M), (Ai @ Bi).T.copy(), "column major")
 
 
+@pytest.mark.parametrize("mkn", [(4000, 1100, 4000), (4090, 1030, 4001), (8100, 1024, 8000), (3841, 1025, 4096)])
+def test_matmul_256_tiles_with_edges(device, mkn):
+    """Large f32 products that are no whole number of tiles, on the 256 x 256 kernel with clamped edges and a zeroed
+    k tail (rows of C that start at odd addresses included): exact on integer data with accumulation into a non-zero
+    C, both layouts, both entry points; NaNs parked around the operands neither leak in nor get overwritten."""
+    M, K, N = mkn
+    rng = np.random.default_rng(62)
+    say("matmul 256 tiles with edges, integers", mkn)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float32); B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    C0 = rng.integers(-9, 10, (M, N)).astype(np.float32)
+    want = A @ B                                             # exact: |sums| < 2^24
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == "mfma_big_edge", _lib.last_path()
+    assert_bits(tc.getData().reshape(M, N), want + C0, "C += A B")
+    say("matmul 256 tiles with edges, column major, C = A B into NaNs", mkn)
+    tc = on(device, np.full((N, M), np.nan, dtype=np.float32))
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc, accumulate=False)
+    assert _lib.last_path() == "mfma_big_edge", _lib.last_path()
+    assert_bits(tc.getData().reshape(N, M), want.T.copy(), "column major")
+    say("matmul 256 tiles with edges, operands inside larger buffers full of NaN", mkn)
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(C0)
+    _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+    assert _lib.last_path() == "mfma_big_edge", _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert_bits(got[pad:pad + M * N].reshape(M, N), want + C0, "parked operands")
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
