@@ -342,7 +342,8 @@ def main():
         dev.free(o)
 
         # C4 matmul
-        for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256))):
+        # (4000^3: a large shape that is no whole number of tiles)
+        for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256)), ("matmul_4000", (4000, 4000, 4000))):
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
             Cm = Tensor._on_device(dev, f32, (M, N))

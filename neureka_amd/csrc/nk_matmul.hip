@@ -839,8 +839,12 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
     if (whole_tiles || edge) {
         const float* Ap = (const float*)A; const float* Bp = (const float*)B; float* Cp = (float*)C;
         // 256x256 tiles, one block per compute unit, when they fill the machine in whole rounds (or many rounds) and the
-        // tiles are deep enough for the first fetch and the write-back not to weigh
-        if (K >= 32 * BK) {
+        // tiles are deep enough for the first fetch and the write-back not to weigh: with one block per compute unit
+        // nothing overlaps a tile's write-back, and reading the old C as well doubles it (measured on 8192 x K x 8192
+        // against the kernels with two blocks per unit -- C = A B: 115 against 112 TFLOP/s at K = 256, 132 against 125
+        // at 512; C += A B: 105 against 112, 121 against 126, the same at 768; 65536 x 256 x 256, a single round of
+        // tiles: 79 against 73 us)
+        if (K >= (overwrite ? 16 : 32) * BK) {
             const bool whole_big = whole_tiles && M % big::TM == 0 && N % big::TN == 0;
             const int64_t cus = dev->props.multiProcessorCount;
             const int64_t tiles = ((M + big::TM - 1) / big::TM) * ((N + big::TN - 1) / big::TN);
