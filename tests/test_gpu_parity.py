@@ -1661,7 +1661,7 @@ def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mk
         assert (a.view(np.uint32 if dt == "f32" else np.uint64) == g.view(np.uint32 if dt == "f32" else np.uint64)).all()
 
 
-@pytest.mark.parametrize("mkn", [(4096, 1024, 4096), (2048, 2048, 8192), (4096, 1056, 4096), (8192, 1024, 8192)])
+@pytest.mark.parametrize("mkn", [(4096, 1024, 4096), (2048, 2048, 8192), (4096, 1056, 4096), (8192, 1024, 8192), (4096, 512, 4096)])
 def test_matmul_256_tiles_one_wavefront_per_simd(device, mkn):
     """Large f32 products whose 256 x 256 tiles fill the machine take the kernel with one wavefront per SIMD.  It sums
     in the order of the 128 x 128 kernel, which computes the left half of the same product (half as many tiles: not
@@ -1689,7 +1689,7 @@ def test_matmul_256_tiles_one_wavefront_per_simd(device, mkn):
     assert (np.abs(got[rows] - ref) <= bound).all()
     # C += A B on top of the result: exactly twice it (the sum is the same, added to itself)
     device.launch_matmul(True, M, K, N, ta, tb, c)
-    assert _lib.last_path() == "mfma_big"
+    assert _lib.last_path() == ("mfma_big" if K >= 1024 else "mfma")          # shallow tiles that also read C: two blocks per compute unit
     assert_bits(c.getData().reshape(M, N), 2 * got, "accumulating")
     say("matmul 256 tiles, integer data, column major", mkn)
     Ai = rng.integers(-3, 4, (M, K)).astype(np.float32); Bi = rng.integers(-3, 4, (K, N)).astype(np.float32)
