@@ -108,6 +108,65 @@ def cpu_side_of_the_other_configs(cores):
     return out
 
 
+def torch_yardstick():
+    """--yardstick: the same workloads through PyTorch's own kernels (vendor BLAS, MIOpen, its elementwise and
+    reduction kernels) on this GPU, microseconds per call from torch's events over 50 calls after 20 -- a yardstick
+    printed beside the figures of this library, never part of them."""
+    import torch
+    import torch.nn.functional as F
+    torch.backends.cuda.matmul.allow_tf32 = False
+    torch.backends.cudnn.allow_tf32 = False
+    d = "cuda:0"
+    res = {"torch": torch.__version__}
+
+    def t(name, fn, n=50, warm=20):
+        for _ in range(warm): fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n): fn()
+        e1.record(); torch.cuda.synchronize()
+        res[name] = round(e0.elapsed_time(e1) / n * 1e3, 1)
+
+    a = torch.randn(1024, 1, 512, device=d); b = torch.randn(1, 2048, 512, device=d); o = torch.empty(1024, 2048, 512, device=d)
+    t("broadcast_add_us", lambda: torch.add(a, b, out=o))
+    ga = torch.empty(1024, 1, 512, device=d); gb = torch.empty(1, 2048, 512, device=d)
+    gbias = torch.empty(1, 1, 512, device=d); gs = torch.empty(1024, 1, 1, device=d)
+    t("broadcast_backward_grad0_us", lambda: torch.sum(o, dim=1, keepdim=True, out=ga))
+    t("broadcast_backward_grad1_us", lambda: torch.sum(o, dim=0, keepdim=True, out=gb))
+    t("broadcast_backward_bias_us", lambda: torch.sum(o, dim=(0, 1), keepdim=True, out=gbias))
+    t("broadcast_backward_per_slab_us", lambda: torch.sum(o, dim=(1, 2), keepdim=True, out=gs))
+    t("sum_2^30_us", lambda: torch.sum(o))
+    t("max_index_2^30_us", lambda: torch.argmax(o))
+    del o
+    n = 1 << 26
+    x, y, z = (torch.randn(n, device=d) for _ in range(3)); out = torch.empty(n, device=d)
+
+    def chain(p, q, r, dst):
+        s = torch.sigmoid(p); s.mul_(q); s.add_(r); torch.tanh(s, out=dst)
+    t("chain_unfused_4_kernels_us", lambda: chain(x, y, z, out))
+    xp, yp, zp = (v.view(16384, 4096).t() for v in (x, y, z))
+    t("chain_unfused_permuted_us", lambda: chain(xp, yp, zp, out.view(4096, 16384)))
+    t("tanh_us", lambda: torch.tanh(x, out=out))
+    t("add_us", lambda: torch.add(x, y, out=out))
+    t("sum_2^26_us", lambda: torch.sum(x))
+    t("max_index_2^26_us", lambda: torch.argmax(x))
+    t("dot_2^26_us", lambda: torch.dot(x, y))
+    del x, y, z, out
+    for name, (M, K, N), dt in (("matmul_4096_us", (4096, 4096, 4096), torch.float32), ("matmul_4000_us", (4000, 4000, 4000), torch.float32),
+                                ("matmul_tall_skinny_us", (65536, 256, 256), torch.float32), ("matmul_4096_f64_us", (4096, 4096, 4096), torch.float64)):
+        A = torch.randn(M, K, device=d, dtype=dt); B = torch.randn(K, N, device=d, dtype=dt); C = torch.empty(M, N, device=d, dtype=dt)
+        t(name, lambda: torch.mm(A, B, out=C))
+    xi = torch.randn(1, 64, 256, 256, device=d, requires_grad=True); w = torch.randn(1, 64, 5, 5, device=d, requires_grad=True)
+    t("conv_c5_forward_us", lambda: F.conv2d(xi, w))
+    yv = F.conv2d(xi, w); e = torch.randn_like(yv)
+    t("conv_c5_grad_input_us", lambda: torch.autograd.grad(yv, xi, e, retain_graph=True))
+    t("conv_c5_grad_kernel_us", lambda: torch.autograd.grad(yv, w, e, retain_graph=True))
+    img = torch.randn(1, 1, 4096, 4096, device=d); k3 = torch.randn(1, 1, 3, 3, device=d)
+    t("conv2d_4096x4096_3x3_us", lambda: F.conv2d(img, k3))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -118,7 +177,13 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy (a copy kernel of known size), so that a "
                          "rocprofv3 --pmc run of this command holds a reference for FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--yardstick", action="store_true",
+                    help="also time the same workloads through PyTorch's own kernels (reported under \"yardstick\")")
+    ap.add_argument("--yardstick-only", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
+    if args.yardstick_only:             # the child process of --yardstick: PyTorch brings its own HIP runtime, which
+        print(json.dumps(torch_yardstick()))    # does not find the GPU in a process where the system's is already at work
+        return
     if args.gpus != 1:
         print("bench.py measures one MI355X: this build has no multi-GPU path (every kernel shards without "
               "exchange), run it with --gpus 1", file=sys.stderr)
@@ -425,6 +490,12 @@ def main():
         "cpu_others": cpu_others,
         "others": others,
     }
+    if args.yardstick:
+        import subprocess
+        dev.sync()
+        child = subprocess.run([sys.executable, os.path.abspath(__file__), "--yardstick-only"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        lines = [ln for ln in child.stdout.splitlines() if ln.startswith("{")]
+        result["yardstick"] = json.loads(lines[-1]) if child.returncode == 0 and lines else {"error": child.stderr[-400:]}
     print(json.dumps(result))
 
 
