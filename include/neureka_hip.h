@@ -216,7 +216,8 @@ int nk_matmul_set(nk_dev dev, int dtype, int layout, int64_t M, int64_t K, int64
  *     NK_FUSE_BIN   op  pop b, pop a, push a op b (NK_OP_ADD..NK_OP_POW)
  * The single value left on the stack is stored to the drain.  Each intermediate is rounded to the
  * tensor dtype exactly as the unfused kernels round it, so + - * stay bit-identical to the unfused
- * sequence.  n_src <= NK_FUSE_MAX_SRC, n_ops <= NK_FUSE_MAX_OPS, stack depth <= NK_FUSE_MAX_STACK. */
+ * sequence.  n_src <= NK_FUSE_MAX_SRC, n_ops <= NK_FUSE_MAX_OPS, stack depth <= NK_FUSE_MAX_STACK per launch: the host
+ * cuts a larger expression into several launches through temporaries, which changes no result because of that rounding. */
 enum { NK_FUSE_LOAD = 0, NK_FUSE_CONST = 1, NK_FUSE_FUN = 2, NK_FUSE_DFUN = 3, NK_FUSE_BIN = 4 };
 #define NK_FUSE_MAX_SRC 6
 #define NK_FUSE_MAX_OPS 32

@@ -319,18 +319,100 @@ def derivative_of(n: Node, index: int) -> Node:
     raise IllegalArgumentException(f"operator '{n.value}' has no fused derivative")
 
 
+# what one launch of nk_fused takes (include/neureka_hip.h: NK_FUSE_MAX_*)
+FUSE_MAX_SRC, FUSE_MAX_OPS, FUSE_MAX_STACK, FUSE_MAX_CONST = 6, 32, 8, 8
+
+
+def _fuse_cost(n: Node):
+    """(op-codes, stack depth, leaves, constants) of the postfix program of the tree; leaves are inputs and temporaries."""
+    if n.kind in ("input", "temp"):
+        return 1, 1, {(n.kind, n.value)}, set()
+    if n.kind == "const":
+        return 1, 1, set(), {n.value}
+    if n.kind in ("fun", "dfun"):
+        ops, depth, leaves, consts = _fuse_cost(n.children[0])
+        return ops + 1, depth, leaves, consts
+    o1, d1, l1, c1 = _fuse_cost(n.children[0])
+    o2, d2, l2, c2 = _fuse_cost(n.children[1])
+    return o1 + o2 + 1, max(d1, d2 + 1), l1 | l2, c1 | c2
+
+
+def _fuse_fits(n: Node) -> bool:
+    ops, depth, leaves, consts = _fuse_cost(n)
+    return ops <= FUSE_MAX_OPS and depth <= FUSE_MAX_STACK and len(leaves) <= FUSE_MAX_SRC and len(consts) <= FUSE_MAX_CONST
+
+
+def plan_fused(root: Node):
+    """Cuts an expression that is too large for one launch of nk_fused (more than 6 sources, 32 op-codes, 8 stack
+    entries or 8 constants) into stages: the largest sub-expressions are evaluated into temporaries first, which
+    later stages read as sources.  Every intermediate of a fused program is rounded to the tensor's element type as
+    the unfused kernels round it, so a temporary holds exactly what the single program would have had on its stack
+    (CLFunctionCompiler generates one OpenCL kernel whatever the size, CLFunctionCompiler.java:101-199).
+    Returns [(program, consts, leaves)], leaves = [("input", k) | ("temp", stage)] in source-slot order; the last
+    stage writes the result."""
+    stages = []
+
+    def lower(n: Node):
+        leaves, consts, program = [], [], []
+
+        def walk(m: Node):
+            if m.kind in ("input", "temp"):
+                key = (m.kind, m.value)
+                if key not in leaves:
+                    leaves.append(key)
+                program.extend([_lib.FUSE_LOAD, leaves.index(key)])
+            elif m.kind == "const":
+                if m.value not in consts:
+                    consts.append(m.value)
+                program.extend([_lib.FUSE_CONST, consts.index(m.value)])
+            elif m.kind in ("fun", "dfun"):
+                if m.value not in _lib.FUN:
+                    raise IllegalArgumentException(f"function '{m.value}' cannot be fused into an elementwise kernel")
+                walk(m.children[0])
+                program.extend([_lib.FUSE_FUN if m.kind == "fun" else _lib.FUSE_DFUN, _lib.FUN[m.value]])
+            else:
+                if m.value not in _lib.OP:
+                    raise IllegalArgumentException(f"operator '{m.value}' cannot be fused into an elementwise kernel")
+                walk(m.children[0]); walk(m.children[1])
+                program.extend([_lib.FUSE_BIN, _lib.OP[m.value]])
+        walk(n)
+        return program, consts, leaves
+
+    def reduce(n: Node) -> Node:
+        if not n.children:
+            return n
+        children = [reduce(c) for c in n.children]            # every child fits one launch by itself now
+        m = Node(n.kind, n.value, children)
+        while not _fuse_fits(m):
+            big = max((i for i, c in enumerate(children) if c.children), key=lambda i: _fuse_cost(children[i])[0])
+            stages.append(lower(children[big]))
+            children[big] = Node("temp", len(stages) - 1)
+            m = Node(n.kind, n.value, children)
+        return m
+
+    final = reduce(root)
+    if final.kind == "temp":                                  # (cannot happen: a temporary is only made of a child)
+        final = Node("fun", "idy", [final])
+    stages.append(lower(final))
+    return stages
+
+
 class OptimizedFunction:
     """One fused kernel for a whole elementwise expression (the counterpart of CLFunctionCompiler,
     devices/opencl/utility/CLFunctionCompiler.java:27-238): the expression tree is lowered to the postfix
-    op-codes of ``nk_fused``; operands must share one shape (views are fine)."""
+    op-codes of ``nk_fused``; operands must share one shape (views are fine).  Expressions beyond what one launch
+    takes run as several launches through temporaries (plan_fused)."""
 
     def __init__(self, device, function: Function, name: str):
         self.device, self.function, self.name = device, function, name
+        self.n_src = function.numberOfArgs()
+        self.stages = plan_fused(function.root)
+        # the single-launch form, sources in input order: what callers that prepare the launch themselves use
         self.program: List[int] = []
         self.consts: List[float] = []
-        self._lower(function.root, self.program, self.consts)
-        self.n_src = function.numberOfArgs()
-        self._derivatives = {}               # input index -> (program, consts) of the derivative kernel
+        if len(self.stages) == 1 and self.n_src <= FUSE_MAX_SRC:
+            self._lower(function.root, self.program, self.consts)
+        self._derivatives = {}               # input index -> stages of the derivative kernel
 
     @staticmethod
     def _lower(n: Node, program: List[int], consts: List[float]) -> None:
@@ -352,13 +434,34 @@ class OptimizedFunction:
             OptimizedFunction._lower(n.children[1], program, consts)
             program += [_lib.FUSE_BIN, _lib.OP[n.value]]
 
-    def derivative_program(self, index: int):
-        """Op-codes of the kernel for d f / d I[index] (CLFunctionCompiler compiles it next to the activation)."""
+    def derivative_stages(self, index: int):
+        """Stages of the kernel(s) for d f / d I[index] (CLFunctionCompiler compiles it next to the activation)."""
         if index not in self._derivatives:
-            program, consts = [], []
-            self._lower(derivative_of(self.function.root, index), program, consts)
-            self._derivatives[index] = (program, consts)
+            self._derivatives[index] = plan_fused(derivative_of(self.function.root, index))
         return self._derivatives[index]
+
+    def derivative_program(self, index: int):
+        """Op-codes and constants of d f / d I[index] when it is one launch with the sources in input order."""
+        program, consts = [], []
+        self._lower(derivative_of(self.function.root, index), program, consts)
+        return program, consts
+
+    def _run_stages(self, stages, srcs: List[Tensor]) -> Tensor:
+        temps = {}
+        out = None
+        try:
+            for k, (program, consts, leaves) in enumerate(stages):
+                operands = [srcs[v] if kind == "input" else temps[v] for kind, v in leaves]
+                if not operands:                     # a constant expression: the drain's shape comes from the first input
+                    operands = [srcs[0]]
+                out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
+                self.device.launch_fused(program, consts, out, operands)
+                temps[k] = out
+        finally:
+            for k, t in temps.items():
+                if t is not out and self.device.has(t):
+                    self.device.free(t)
+        return out
 
     def _with_guests(self, srcs: List[Tensor], run):
         """Operands that are not on the device are stored for the call and restored afterwards
@@ -378,13 +481,8 @@ class OptimizedFunction:
     def derive(self, inputs: Sequence[Tensor], index: int) -> Tensor:
         """d f / d I[index] at the inputs, in one launch."""
         srcs = list(inputs[: self.n_src])
-        program, consts = self.derivative_program(index)
-
-        def run():
-            out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
-            self.device.launch_fused(program, consts, out, srcs)
-            return out
-        return self._with_guests(srcs, run)
+        stages = self.derivative_stages(index)
+        return self._with_guests(srcs, lambda: self._run_stages(stages, srcs))
 
     def call(self, *inputs: Tensor) -> Tensor:
         if len(inputs) == 1 and isinstance(inputs[0], (list, tuple)):
@@ -396,11 +494,7 @@ class OptimizedFunction:
             if t.shape != srcs[0].shape:
                 raise IllegalArgumentException("operands of a fused function must share one shape")
 
-        def run():
-            out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
-            self.device.launch_fused(self.program, self.consts, out, srcs)
-            return out
-        out = self._with_guests(srcs, run)
+        out = self._with_guests(srcs, lambda: self._run_stages(self.stages, srcs))
         if self.function.doAD and any(t.rqsGradient() or t._node is not None for t in srcs):
             # reverse mode: error * (d f / d I[d]), the derivative in one fused launch (operands that live on the
             # host are stored again for that launch)

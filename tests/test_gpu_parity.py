@@ -3,6 +3,7 @@ seeded inputs.  Bit-exact for + - * and copies (and every kernel that keeps the 
 order); rtol 1e-5 (f32) / 1e-12 (f64) for transcendental activations; norm-wise 1e-5 / 1e-12 for
 re-ordered reductions.  Every test prints what it is about to run before touching the GPU."""
 import ctypes as C
+import gc
 
 import numpy as np
 import pytest
@@ -939,6 +940,58 @@ def test_fused_chain_equals_unfused_and_oracle(device, orc, dt):
     if dt == "f64":
         x, y, z = bases
         assert_close(f2(*tens).items, ((x * y) + (y - z) * (z / (x * x + 2))).reshape(-1), "nested vs numpy")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_fused_functions_beyond_one_launch(device, dt):
+    """Expressions with more than 6 inputs, 32 op-codes or 8 constants run as several launches through temporaries:
+    the same bits as the unfused graph for + - * (every intermediate is rounded to the element type either way), no
+    buffer left behind, and derivatives -- far larger trees than the functions themselves -- through the same staging,
+    against central differences in f64."""
+    T = F[dt]
+    rng = np.random.default_rng(34)
+    shape = (33, 40)
+    exprs = ["relu(I[0]*I[1]+I[2])*quad(I[3]-I[4])+abs(I[5]*I[6])-I[7]*I[8]+I[9]",
+             "+".join(f"quad(I[{k % 3}]*{k + 1}.5-I[{(k + 1) % 3}])" for k in range(14)),
+             "I[0]" + "".join(f"{'+-'[k % 2]}(I[1]*{k}.25)" for k in range(40))]
+    for expr in exprs:
+        say("fused beyond one launch", dt, expr[:60])
+        fn = Function.of(expr)
+        fused = device.optimizedFunctionOf(fn, "big")
+        assert len(fused.stages) > 1
+        arrays = [rng.uniform(-1.5, 1.5, shape).astype(T) for _ in range(fn.numberOfArgs())]
+        ts = [on(device, a) for a in arrays]
+        got = None                                                     # (drop the result of the expression before)
+        gc.collect()
+        before = device.liveBuffers()
+        got = fused(*ts)
+        gc.collect()
+        assert device.liveBuffers() == before + 1                      # the temporaries are gone
+        assert_bits(got.items, fn(*ts).items, "fused in stages vs unfused")
+    say("derivatives of a large smooth function", dt)
+    expr = "tanh(sig(I[0])*I[1]+I[2])*sin(I[3]*I[0])+exp(I[1]*0.25)*cos(I[2]-I[3])+softplus(I[0]*I[2])*gaus(I[1])"
+    fn = Function.of(expr)
+    fused = device.optimizedFunctionOf(fn, "smooth")
+    arrays = [rng.uniform(0.5, 1.5, shape).astype(T) for _ in range(4)]
+    ts = [on(device, a) for a in arrays]
+    assert any(len(fused.derivative_stages(i)) > 1 for i in range(4))
+    e = rng.uniform(-1, 1, shape).astype(T)
+    grads = []
+    for runner in (fused, fn):
+        gs = [on(device, a).setRqsGradient(True) for a in arrays]
+        runner(*gs).backward(on(device, e))
+        grads.append([t.gradient.items for t in gs])
+    for i in range(4):
+        scale = np.abs(grads[1][i]) + np.abs(e.reshape(-1))
+        assert (np.abs(grads[0][i] - grads[1][i]) <= 50 * RTOL[np.dtype(T)] * scale + ATOL[np.dtype(T)]).all(), i
+    if dt == "f64":
+        for i in range(4):
+            h = 1e-6
+            up, dn = [a.copy() for a in arrays], [a.copy() for a in arrays]
+            up[i] += h; dn[i] -= h
+            numeric = (fused(*[on(device, a) for a in up]).items - fused(*[on(device, a) for a in dn]).items) / (2 * h)
+            got = fused.derive(ts, i).items
+            assert (np.abs(got - numeric) <= 1e-6 * np.maximum(1.0, np.abs(numeric))).all(), i
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])

@@ -113,6 +113,59 @@ def test_parser_and_fused_lowering():
         OptimizedFunction(None, Function.of("i0 x i1"), "conv")
 
 
+def test_expressions_beyond_one_launch_are_cut_into_stages():
+    """plan_fused: more than 6 sources, 32 op-codes, 8 stack entries or 8 constants per launch make several stages
+    through temporaries; each stage respects the limits, and interpreting the stages gives the tree's own value
+    (float32 after every operation, as the kernels round)."""
+    from neureka_amd.function import FUSE_MAX_CONST, FUSE_MAX_OPS, FUSE_MAX_SRC, FUSE_MAX_STACK, plan_fused
+    rng = np.random.default_rng(8)
+    f32 = np.float32
+    inv_fun = {v: k for k, v in _lib.FUN.items()}; inv_op = {v: k for k, v in _lib.OP.items()}
+    np_fun = {"relu": lambda x: np.where(x >= 0, x, x * f32(0.01)), "quad": lambda x: x * x, "abs": np.abs, "idy": lambda x: x}
+    np_op = {"add": np.add, "subtract": np.subtract, "multiply": np.multiply}
+
+    def tree_value(n, xs):
+        if n.kind == "input": return xs[n.value]
+        if n.kind == "const": return np.full_like(xs[0], n.value)
+        if n.kind == "fun": return np_fun[n.value](tree_value(n.children[0], xs)).astype(f32)
+        return np_op[n.value](tree_value(n.children[0], xs), tree_value(n.children[1], xs)).astype(f32)
+
+    def run_stages(stages, xs):
+        temps = {}
+        for k, (program, consts, leaves) in enumerate(stages):
+            ops = len(program) // 2
+            assert ops <= FUSE_MAX_OPS and len(leaves) <= FUSE_MAX_SRC and len(consts) <= FUSE_MAX_CONST
+            srcs = [xs[v] if kind == "input" else temps[v] for kind, v in leaves]
+            stack, deepest = [], 0
+            for code, arg in zip(program[0::2], program[1::2]):
+                if code == _lib.FUSE_LOAD: stack.append(srcs[arg])
+                elif code == _lib.FUSE_CONST: stack.append(np.full_like(xs[0], consts[arg]))
+                elif code == _lib.FUSE_FUN: stack.append(np_fun[inv_fun[arg]](stack.pop()).astype(f32))
+                else:
+                    b = stack.pop(); a = stack.pop()
+                    stack.append(np_op[inv_op[arg]](a, b).astype(f32))
+                deepest = max(deepest, len(stack))
+            assert len(stack) == 1 and deepest <= FUSE_MAX_STACK
+            temps[k] = stack[0]
+        return temps[len(stages) - 1]
+
+    small = Function.of("tanh(sig(I[0])*I[1]+I[2])")
+    assert len(plan_fused(small.root)) == 1
+    cases = ["relu(i0*i1+i2)*quad(i3-i4)+abs(i5*i6)-i7*i8+i9",                                   # ten sources
+             "+".join(f"quad(i{k % 3}*{k + 1}.5-i{(k + 1) % 3})" for k in range(14)),                # 14 constants, ~100 op-codes
+             "i0" + "".join(f"{'+-'[k % 2]}(i1*{k}.25)" for k in range(40)),                           # a long chain
+             "(" * 12 + "i0" + "".join(f"+i{1 + k % 2})*i{k % 3}" for k in range(12)),               # nested to the left
+             "+".join(f"(i{k % 3}*i{(k + 1) % 3}" for k in range(12)) + ")" * 12]                    # nested to the right: a deep stack
+    for expr in cases:
+        fn = Function.of(expr)
+        stages = plan_fused(fn.root)
+        assert len(stages) > 1, expr
+        xs = [rng.uniform(-2, 2, 64).astype(f32) for _ in range(fn.numberOfArgs())]
+        assert run_stages(stages, xs).tobytes() == tree_value(fn.root, xs).tobytes(), expr
+    opt = OptimizedFunction(None, Function.of(cases[0]), "big")
+    assert opt.program == [] and len(opt.stages) > 1                                            # no single-launch form
+
+
 def test_no_host_arithmetic_path():
     a = Tensor.of(np.float32, [2, 2], [1, 2, 3, 4])
     with pytest.raises(IllegalStateException):
