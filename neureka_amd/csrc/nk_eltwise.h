@@ -20,13 +20,15 @@ constexpr int SRC_CONST0 = 16, SRC_POP = 32;
 constexpr int MAX_INSTR = 48;
 constexpr int HW_STACK = 4;
 
-struct Prog {
+struct alignas(32) Prog {
+    unsigned code[MAX_INSTR];      // op | arg << 8 | src << 16, what the device reads: eight words per scalar load
     int n;
-    unsigned char op[MAX_INSTR];   // I_*
+    unsigned char op[MAX_INSTR];   // I_*                                            (the host's view of the same program)
     unsigned char arg[MAX_INSTR];  // fun id | binary op | (binary op)*2 + d
     unsigned char src[MAX_INSTR];  // k | SRC_CONST0 + k | SRC_POP
     double consts[NK_FUSE_MAX_CONST];
 };
+static_assert(MAX_INSTR % 8 == 0, "the interpreter fetches the program in blocks of eight words");
 
 // interpreter: V elements per thread; all control flow is uniform over the grid (it only depends on
 // kernel arguments), so it costs scalar branches, not divergence.
@@ -41,8 +43,20 @@ __device__ __forceinline__ void run_prog(const Prog& P, const T (&src)[NSRC][V],
     for (int v = 0; v < V; v++) acc[v] = T(0);
 #pragma unroll
     for (int v = 0; v < SV; v++) s0[v] = s1[v] = s2[v] = s3[v] = T(0);
-    for (int pc = 0; pc < P.n; pc++) {
-        const int op = P.op[pc], arg = P.arg[pc], s = P.src[pc];
+    // The program is fetched eight instruction words at a time with one wide scalar load and consumed from a shift
+    // register; the next eight are requested before the current ones run.  (One byte-sized scalar load per field and
+    // instruction made every interpreted instruction wait out a trip to the scalar cache: 1.0 ms for the twelve
+    // instructions of the chain's derivative over 2^26 elements.)
+    unsigned n0 = P.code[0], n1 = P.code[1], n2 = P.code[2], n3 = P.code[3], n4 = P.code[4], n5 = P.code[5], n6 = P.code[6], n7 = P.code[7];
+    for (int base = 0; base < P.n; base += 8) {
+      unsigned c0 = n0, c1 = n1, c2 = n2, c3 = n3, c4 = n4, c5 = n5, c6 = n6, c7 = n7;
+      const int nb = base + 8 < MAX_INSTR ? base + 8 : 0;               // (past the end: any block, it is not run)
+      n0 = P.code[nb]; n1 = P.code[nb + 1]; n2 = P.code[nb + 2]; n3 = P.code[nb + 3]; n4 = P.code[nb + 4]; n5 = P.code[nb + 5]; n6 = P.code[nb + 6]; n7 = P.code[nb + 7];
+      const int here = P.n - base < 8 ? P.n - base : 8;
+      for (int i = 0; i < here; i++) {
+        const unsigned code = c0;
+        c0 = c1; c1 = c2; c2 = c3; c3 = c4; c4 = c5; c5 = c6; c6 = c7;
+        const int op = code & 0xff, arg = (code >> 8) & 0xff, s = (code >> 16) & 0xff;
         T x[V];
         if (op == I_PUSH) {
             if constexpr (STACK) {
@@ -96,6 +110,7 @@ __device__ __forceinline__ void run_prog(const Prog& P, const T (&src)[NSRC][V],
                 for (int v = 0; v < V; v++) acc[v] = x[v];
                 break;
         }
+      }
     }
 }
 
@@ -246,6 +261,7 @@ constexpr int ROWS_FAST_OUTER = 3;
 // tanh(sig(a)*b+c) on 2^26 elements: one pass 6.71, two 6.71, four 6.46 TB/s -- its 62 vector instructions per
 // element (110 us of issue time in a 160 us launch), not the access pattern, hold it below the 7.2 TB/s a bare
 // three-reads-one-write kernel reaches.
+// (the full interpreter family keeps one pass: its V = 4 instantiation already holds 190 registers, two passes spill)
 constexpr int rows_passes(int funset, int nsrc) { return funset >= 2 ? 1 : (nsrc >= 3 ? 2 : 4); }
 struct RowsArgs {
     int nouter;                // collapsed outer axes, 0..ROWS_MAX_OUTER

@@ -149,6 +149,8 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     static thread_local Plan plan;         // large (kernel argument blocks): kept off the stack
     plan = Plan{};
     plan.prog = prog;
+    for (int i = 0; i < MAX_INSTR; i++)
+        plan.prog.code[i] = i < prog.n ? (unsigned)prog.op[i] | ((unsigned)prog.arg[i] << 8) | ((unsigned)prog.src[i] << 16) : 0u;
     plan.nsrc = c.nsrc;
     plan.drn = (void*)c.drn;
     for (int j = 0; j < c.nsrc; j++) plan.srcs.p[j] = (const void*)c.src[j];
