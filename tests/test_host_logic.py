@@ -234,23 +234,23 @@ def test_every_registration_row_of_the_opencl_backend_has_a_hip_counterpart():
 
 
 def test_integration_text_binds_every_export_and_every_registration_row():
-    """INTEGRATION.md is the binding a maintainer copies: it must declare a MethodHandle for every export of the header
-    and name every operation class the OpenCL backend registers."""
+    """The Java binding text a maintainer copies must declare a MethodHandle for every export of the header and name
+    every operation class the OpenCL backend registers."""
     header = open(os.path.join(ROOT, "include", "neureka_hip.h")).read()
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     declared = sorted(set(re.findall(r"\b(nk_[a-z0-9_]+)\s*\(", header)))
     bound = set(re.findall(r'MethodHandle\s+(nk_[a-z0-9_]+)\s*=\s*h\("(nk_[a-z0-9_]+)"', text))
     assert all(a == b for a, b in bound)
     missing = [n for n in declared if n not in {a for a, _ in bound}]
-    assert not missing, f"exports without a MethodHandle in INTEGRATION.md: {missing}"
+    assert not missing, f"exports without a MethodHandle in the binding text: {missing}"
     for cls in ("Addition", "Subtraction", "Multiplication", "Division", "Modulo", "Power", "AssignLeft", "Convolution", "XConvLeft",
                 "XConvRight", "MatMul", "DotProduct", "Sum", "Randomization", "Absolute", "Cosinus", "GaSU", "GaTU", "Gaussian",
                 "GaussianFast", "GeLU", "Identity", "Logarithm", "Quadratic", "ReLU", "SeLU", "Sigmoid", "SiLU", "Sinus", "Softplus",
                 "Softsign", "Tanh", "TanhFast", "Exp", "Cbrt", "Log10", "Sqrt"):
-        assert re.search(rf"\b{cls}\.class", text), f"{cls} is not registered in INTEGRATION.md"
+        assert re.search(rf"\b{cls}\.class", text), f"{cls} is not registered in the binding text"
     for method in ("_readAll", "_readItem", "_readArray", "_writeItem", "_writeArray", "_swap", "_sizeOccupiedBy", "_actualize",
                    "_virtualize", "_dataTypeOf", "allocateFromOne", "allocateFromAll", "optimizedOperationOf", "dispose"):
-        assert re.search(rf"\b{method}\(", text), f"HipDevice.{method} is missing from INTEGRATION.md"
+        assert re.search(rf"\b{method}\(", text), f"HipDevice.{method} is missing from the binding text"
 
 
 def test_assignment_parses_and_nests_to_the_right():
