@@ -5,6 +5,8 @@
 // descriptors to one of four access patterns; the kernels here are instantiated per
 //   T        float | double
 //   FUNSET   0: + - * / and copies only   1: + the cheap forward activations   2: the full table
+//            3: set 1 + every derivative, on the packed interpreter (no saved intermediates, no pow / modulo / heavy
+//               forward function): what the backward launch of every activation runs
 //   NSRC     number of source registers the instantiation carries (1, 2, 3 or 6)
 // so that the bandwidth-critical cases (add/mul, broadcast, the sig/tanh chain) run in kernels with a
 // small register footprint, while rarely used functions live in their own, heavier instantiations.
@@ -118,28 +120,46 @@ __device__ __forceinline__ void run_prog(const Prog& P, const T (&src)[NSRC][V],
 // handed to the specialised families in packed form: all instruction words sit in one aligned block of
 // the kernel arguments and are fetched with a single wide scalar load, then consumed from a shift
 // register, so the interpreter never waits for memory between instructions.
-constexpr int LIGHT_INSTR = 8, LIGHT_CONST = 4;
-struct alignas(16) LightProg {
-    unsigned code[LIGHT_INSTR];    // op | arg << 8 | src << 16
+// Set 3 (derivative programs) takes twice as many instructions and one saved intermediate: the derivative of a chain
+// f(g(..)) by an inner operand is f'(g(..)) saved, times g' computed after it.
+constexpr int LIGHT_INSTR = 8, LIGHT_INSTR_D = 16, LIGHT_CONST = 4;
+struct alignas(64) LightProg {
+    unsigned code[LIGHT_INSTR_D];  // op | arg << 8 | src << 16
     double consts[LIGHT_CONST];
     int n;
 };
 
 template <typename T, int V, int NSRC, int FUNSET>
 __device__ __forceinline__ void run_light(const LightProg& P, const T (&src)[NSRC][V], T (&acc)[V]) {
+    constexpr int FS = FUNSET == 3 ? 1 : FUNSET;         // set 3 carries the forward functions and operators of set 1
+    constexpr bool DERIV = FUNSET == 3;
     unsigned c0 = P.code[0], c1 = P.code[1], c2 = P.code[2], c3 = P.code[3], c4 = P.code[4], c5 = P.code[5], c6 = P.code[6], c7 = P.code[7];
+    unsigned c8 = 0, c9 = 0, c10 = 0, c11 = 0, c12 = 0, c13 = 0, c14 = 0, c15 = 0;
+    if constexpr (DERIV) { c8 = P.code[8]; c9 = P.code[9]; c10 = P.code[10]; c11 = P.code[11]; c12 = P.code[12]; c13 = P.code[13]; c14 = P.code[14]; c15 = P.code[15]; }
     T k[LIGHT_CONST];
 #pragma unroll
     for (int i = 0; i < LIGHT_CONST; i++) k[i] = (T)P.consts[i];
+    T saved[DERIV ? V : 1];
+#pragma unroll
+    for (int v = 0; v < (DERIV ? V : 1); v++) saved[v] = T(0);
 #pragma unroll
     for (int v = 0; v < V; v++) acc[v] = T(0);
     for (int pc = 0; pc < P.n; pc++) {
         const unsigned code = c0;
         c0 = c1; c1 = c2; c2 = c3; c3 = c4; c4 = c5; c5 = c6; c6 = c7;
+        if constexpr (DERIV) { c7 = c8; c8 = c9; c9 = c10; c10 = c11; c11 = c12; c12 = c13; c13 = c14; c14 = c15; }
         const int op = code & 0xff, arg = (code >> 8) & 0xff, s = (code >> 16) & 0xff;
         T x[V];
-        if (op != I_FUN) {
-            if (s >= SRC_CONST0) {
+        if (DERIV && op == I_PUSH) {
+#pragma unroll
+            for (int v = 0; v < (DERIV ? V : 1); v++) saved[v] = acc[v];
+            continue;
+        }
+        if (op != I_FUN && op != I_DFUN) {
+            if (DERIV && s == SRC_POP) {
+#pragma unroll
+                for (int v = 0; v < (DERIV ? V : 1); v++) x[v] = saved[v];
+            } else if (s >= SRC_CONST0) {
                 T c = k[0];
 #pragma unroll
                 for (int i = 1; i < LIGHT_CONST; i++) if (s == SRC_CONST0 + i) c = k[i];
@@ -162,11 +182,14 @@ __device__ __forceinline__ void run_light(const LightProg& P, const T (&src)[NSR
                 for (int v = 0; v < V; v++) acc[v] = x[v];
                 break;
             case I_FUN:
-                if constexpr (FUNSET >= 1) apply_fun<T, V, FUNSET>(arg, acc);
+                if constexpr (FUNSET >= 1) apply_fun<T, V, FS>(arg, acc);
                 break;
-            case I_BIN: apply_bin<T, V, FUNSET>(arg, acc, x); break;
+            case I_DFUN:
+                if constexpr (FUNSET == 3) apply_dfun<T, V>(arg, acc);
+                break;
+            case I_BIN: apply_bin<T, V, FS>(arg, acc, x); break;
             case I_RBIN:
-                apply_bin<T, V, FUNSET>(arg, x, acc);
+                apply_bin<T, V, FS>(arg, x, acc);
 #pragma unroll
                 for (int v = 0; v < V; v++) acc[v] = x[v];
                 break;
@@ -183,7 +206,7 @@ __device__ __forceinline__ void run_light(const LightProg& P, const T (&src)[NSR
 // family-independent entry: the full family interprets the long form, the others the packed form
 template <typename T, int V, int NSRC, int FUNSET>
 __device__ __forceinline__ void run_any(const Prog& P, const LightProg& LP, const T (&src)[NSRC][V], T (&acc)[V]) {
-    if constexpr (FUNSET >= 2) run_prog<T, V, NSRC, FUNSET>(P, src, acc);
+    if constexpr (FUNSET == 2) run_prog<T, V, NSRC, FUNSET>(P, src, acc);
     else run_light<T, V, NSRC, FUNSET>(LP, src, acc);
 }
 
@@ -262,7 +285,7 @@ constexpr int ROWS_FAST_OUTER = 3;
 // element (110 us of issue time in a 160 us launch), not the access pattern, hold it below the 7.2 TB/s a bare
 // three-reads-one-write kernel reaches.
 // (the full interpreter family keeps one pass: its V = 4 instantiation already holds 190 registers, two passes spill)
-constexpr int rows_passes(int funset, int nsrc) { return funset >= 2 ? 1 : (nsrc >= 3 ? 2 : 4); }
+constexpr int rows_passes(int funset, int nsrc) { return funset == 2 ? 1 : funset == 3 ? 2 : (nsrc >= 3 ? 2 : 4); }
 struct RowsArgs {
     int nouter;                // collapsed outer axes, 0..ROWS_MAX_OUTER
     int nsrc;

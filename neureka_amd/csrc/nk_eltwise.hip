@@ -26,18 +26,26 @@ struct ProgBuilder {
 
 // smallest function set that can run the program
 static int funset_of(const Prog& p) {
-    int set = 0;
+    bool fun = false, dfun = false, full = false;
+    int saved = 0;
     for (int i = 0; i < p.n; i++) {
+        if (p.op[i] != I_FUN && p.op[i] != I_DFUN && p.op[i] != I_PUSH && p.src[i] == SRC_POP) saved--;
         switch (p.op[i]) {
-            case I_FUN: set = set < 1 ? 1 : set; if (fun_is_heavy(p.arg[i])) set = 2; break;
-            case I_DFUN: set = 2; break;
-            case I_BIN: case I_RBIN: if (bin_is_heavy(p.arg[i])) set = 2; break;
-            case I_DBIN: case I_RDBIN: if (dbin_is_heavy(p.arg[i] >> 1)) set = 2; break;
-            case I_PUSH: set = 2; break;      // saved intermediates: only the full family has the stack
+            case I_FUN: fun = true; if (fun_is_heavy(p.arg[i])) full = true; break;
+            case I_DFUN: dfun = true; break;
+            case I_BIN: case I_RBIN: if (bin_is_heavy(p.arg[i])) full = true; break;
+            case I_DBIN: case I_RDBIN:
+                if (dbin_is_heavy(p.arg[i] >> 1)) full = true;
+                if (dbin_needs_derivative_set(p.arg[i] >> 1)) dfun = true;
+                break;
+            case I_PUSH:                          // one saved intermediate: the derivative family; more: the full one
+                dfun = true;
+                if (++saved > 1) full = true;
+                break;
             default: break;
         }
     }
-    return set;
+    return full ? 2 : dfun ? 3 : fun ? 1 : 0;
 }
 
 // postfix (the public encoding of nk_fused) -> accumulator form
@@ -161,8 +169,10 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     for (int i = 0; i < prog.n; i++)
         if (prog.op[i] != I_FUN && prog.op[i] != I_DFUN && prog.op[i] != I_PUSH && prog.src[i] >= SRC_CONST0 && prog.src[i] < SRC_POP)
             n_consts = n_consts > prog.src[i] - SRC_CONST0 + 1 ? n_consts : prog.src[i] - SRC_CONST0 + 1;
-    if (prog.n > LIGHT_INSTR || n_consts > LIGHT_CONST) funset = 2;
-    if (funset < 2) {
+    // (programs of 9 to 16 instructions without derivatives also fit the derivative family, which carries set 1)
+    if (n_consts > LIGHT_CONST) funset = 2;
+    else if (prog.n > (funset == 3 ? LIGHT_INSTR_D : LIGHT_INSTR)) funset = (funset != 2 && prog.n <= LIGHT_INSTR_D) ? 3 : 2;
+    if (funset != 2) {
         plan.light.n = prog.n;
         for (int i = 0; i < prog.n; i++) plan.light.code[i] = prog.op[i] | (prog.arg[i] << 8) | (prog.src[i] << 16);
         for (int i = 0; i < LIGHT_CONST; i++) plan.light.consts[i] = prog.consts[i];
@@ -286,7 +296,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         const bool vec = cn.shape[last] % VMAX == 0 || ragged;
         RowsArgs& A = plan.rows;
         const int V = vec ? VMAX : 1;
-        int passes = rows_passes(funset, funset >= 2 ? NK_FUSE_MAX_SRC : (c.nsrc <= 1 ? 1 : c.nsrc));
+        int passes = rows_passes(funset, funset == 2 ? NK_FUSE_MAX_SRC : (c.nsrc <= 1 ? 1 : c.nsrc));
         A.nouter = last; A.nsrc = c.nsrc;
         A.L = (unsigned)cn.shape[last];
         // sources at least as large as the drain's threshold whose every element is read once stream past the caches
@@ -330,7 +340,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         }
         A.vec = V;
         A.ragged = ragged ? 1 : 0;
-        A.simple_loads = (funset < 2 && A.const_last == 0 && A.strided_last == 0 && periodic == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
+        A.simple_loads = (funset != 2 && A.const_last == 0 && A.strided_last == 0 && periodic == 0 && c.nsrc >= 1 && c.nsrc <= 3) ? 1 : 0;
         plan.kind = PLAN_ROWS;
         // drain = src0 op src1 with + - * /: the dedicated kernel
         // (sources that are constant along a row are handled by that kernel's vector variant only)
@@ -422,7 +432,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
 
     // tile_transpose: the drain and some operands run along the innermost axis, the others along one
     // common outer axis
-    if (!done && funset < 2 && cn.stride[0][last] == 1 && cn.rank >= 2) {
+    if (!done && funset != 2 && cn.stride[0][last] == 1 && cn.rank >= 2) {
         int pax = -1;
         unsigned turned = 0;
         bool ok = true;
@@ -493,6 +503,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
     switch (funset) {
         case 0: return launch_family<T, 0>(dev, plan);
         case 1: return launch_family<T, 1>(dev, plan);
+        case 3: return launch_family<T, 3>(dev, plan);
         default: return launch_family<T, 2>(dev, plan);
     }
 }
