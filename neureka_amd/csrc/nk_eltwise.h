@@ -5,8 +5,10 @@
 // descriptors to one of four access patterns; the kernels here are instantiated per
 //   T        float | double
 //   FUNSET   0: + - * / and copies only   1: + the cheap forward activations   2: the full table
-//            3: set 1 + every derivative, on the packed interpreter (no saved intermediates, no pow / modulo / heavy
-//               forward function): what the backward launch of every activation runs
+//            3: set 1 + every derivative (of functions, of / and %) on the packed interpreter (at most 16 instructions, one
+//               saved intermediate, 3 sources; no pow, modulo or heavy forward function: with those the f32 kernels need
+//               181-197 registers instead of 147): the backward launch of every activation and of + - * /, the derivatives
+//               of a fused chain
 //   NSRC     number of source registers the instantiation carries (1, 2, 3 or 6)
 // so that the bandwidth-critical cases (add/mul, broadcast, the sig/tanh chain) run in kernels with a
 // small register footprint, while rarely used functions live in their own, heavier instantiations.

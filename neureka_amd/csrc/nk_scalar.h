@@ -193,11 +193,17 @@ __device__ __forceinline__ float gauss(float x) {
 
 // The evaluators below work on V values at once with the switch outside the lane loop: the op-code
 // is uniform over the whole grid, so the dispatch is done once per instruction, not once per value.
+// NK_ONE_BY_ONE (a constant in the function that uses the macro): the elements of a thread are evaluated one after the
+// other, with a scheduling barrier between them.  The double-precision library functions behind the heavy entries need
+// 28-44 registers per element in flight (pow 44, log 36, sin / cos / exp 28); interleaved over the four elements of a
+// thread that alone is 176 and the kernel ends at 190-256 registers, one or two wavefronts per SIMD, and is bound by
+// the few bytes it keeps in flight.
 #define NK_EACH(expr)                                   \
     {                                                   \
         _Pragma("unroll") for (int v = 0; v < V; v++) { \
             const T x = a[v]; (void)x;                  \
             a[v] = (expr);                              \
+            if constexpr (NK_ONE_BY_ONE) __builtin_amdgcn_sched_barrier(0); \
         }                                               \
     }                                                   \
     break
@@ -270,6 +276,7 @@ template <typename T> __device__ __forceinline__ T dfast_tanh_ref(T x) {
 template <typename T, int V, int FUNSET>
 __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
     using N = Num<T>;
+    constexpr bool NK_ONE_BY_ONE = FUNSET >= 2;
     switch (id) {
         case NK_FUN_ABS: NK_EACH(N::abs(x));
         case NK_FUN_GASU: NK_EACH(softsign(x * x * x));
@@ -309,6 +316,7 @@ inline bool fun_is_heavy(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN |
 template <typename T, int V>
 __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
     using N = Num<T>;
+    constexpr bool NK_ONE_BY_ONE = true;
     switch (id) {
         case NK_FUN_ABS: NK_EACH(x < T(0) ? T(-1) : T(1));
         case NK_FUN_COS: NK_EACH(T(-::sin((double)x)));
@@ -344,6 +352,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
         _Pragma("unroll") for (int v = 0; v < V; v++) { \
             const T x = a[v], y = b[v]; (void)x; (void)y; \
             a[v] = (expr);                              \
+            if constexpr (NK_ONE_BY_ONE) __builtin_amdgcn_sched_barrier(0); \
         }                                               \
     }                                                   \
     break
@@ -351,6 +360,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
 template <typename T, int V, int FUNSET>
 __device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
     using N = Num<T>;
+    constexpr bool NK_ONE_BY_ONE = FUNSET >= 2;
     switch (op) {
         case NK_OP_ADD: NK_EACH2(x + y);
         case NK_OP_SUB: NK_EACH2(x - y);
@@ -373,6 +383,7 @@ inline bool bin_is_heavy(int op) { return op == NK_OP_MOD || op == NK_OP_POW; }
 template <typename T, int V, int FUNSET>
 __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b)[V]) {
     using N = Num<T>;
+    constexpr bool NK_ONE_BY_ONE = FUNSET >= 2;
     switch (op * 2 + d) {
         case NK_OP_ADD * 2 + 0:
         case NK_OP_ADD * 2 + 1:
