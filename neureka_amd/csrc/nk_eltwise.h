@@ -5,10 +5,10 @@
 // descriptors to one of four access patterns; the kernels here are instantiated per
 //   T        float | double
 //   FUNSET   0: + - * / and copies only   1: + the cheap forward activations   2: the full table
-//            3: set 1 + every derivative (of functions, of / and %) on the packed interpreter (at most 16 instructions, one
-//               saved intermediate, 3 sources; no pow, modulo or heavy forward function: with those the f32 kernels need
-//               181-197 registers instead of 147): the backward launch of every activation and of + - * /, the derivatives
-//               of a fused chain
+//            3: the full table on the packed interpreter (at most 16 instructions, one saved intermediate, 3 sources):
+//               every derivative and every heavy function of a program that short -- the backward launch of every
+//               activation and operator, the derivatives of a fused chain, sin / cos / log10 / cbrt / softplus / pow /
+//               modulo by themselves; set 2 keeps the long and deep programs and those with more sources
 //   NSRC     number of source registers the instantiation carries (1, 2, 3 or 6)
 // so that the bandwidth-critical cases (add/mul, broadcast, the sig/tanh chain) run in kernels with a
 // small register footprint, while rarely used functions live in their own, heavier instantiations.
@@ -133,7 +133,7 @@ struct alignas(64) LightProg {
 
 template <typename T, int V, int NSRC, int FUNSET>
 __device__ __forceinline__ void run_light(const LightProg& P, const T (&src)[NSRC][V], T (&acc)[V]) {
-    constexpr int FS = FUNSET == 3 ? 1 : FUNSET;         // set 3 carries the forward functions and operators of set 1
+    constexpr int FS = FUNSET == 3 ? 2 : FUNSET;         // set 3 carries the whole function and operator table
     constexpr bool DERIV = FUNSET == 3;
     unsigned c0 = P.code[0], c1 = P.code[1], c2 = P.code[2], c3 = P.code[3], c4 = P.code[4], c5 = P.code[5], c6 = P.code[6], c7 = P.code[7];
     unsigned c8 = 0, c9 = 0, c10 = 0, c11 = 0, c12 = 0, c13 = 0, c14 = 0, c15 = 0;
@@ -195,9 +195,9 @@ __device__ __forceinline__ void run_light(const LightProg& P, const T (&src)[NSR
 #pragma unroll
                 for (int v = 0; v < V; v++) acc[v] = x[v];
                 break;
-            case I_DBIN: apply_dbin<T, V, FUNSET>(arg >> 1, arg & 1, acc, x); break;
+            case I_DBIN: apply_dbin<T, V, FS>(arg >> 1, arg & 1, acc, x); break;
             case I_RDBIN:
-                apply_dbin<T, V, FUNSET>(arg >> 1, arg & 1, x, acc);
+                apply_dbin<T, V, FS>(arg >> 1, arg & 1, x, acc);
 #pragma unroll
                 for (int v = 0; v < V; v++) acc[v] = x[v];
                 break;

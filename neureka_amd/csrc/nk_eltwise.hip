@@ -26,19 +26,16 @@ struct ProgBuilder {
 
 // smallest function set that can run the program
 static int funset_of(const Prog& p) {
-    bool fun = false, dfun = false, full = false;
+    bool fun = false, dfun = false, full = false;         // dfun: needs the full table (derivatives, heavy entries)
     int saved = 0;
     for (int i = 0; i < p.n; i++) {
         if (p.op[i] != I_FUN && p.op[i] != I_DFUN && p.op[i] != I_PUSH && p.src[i] == SRC_POP) saved--;
         switch (p.op[i]) {
-            case I_FUN: fun = true; if (fun_is_heavy(p.arg[i])) full = true; break;
+            case I_FUN: fun = true; if (fun_is_heavy(p.arg[i])) dfun = true; break;
             case I_DFUN: dfun = true; break;
-            case I_BIN: case I_RBIN: if (bin_is_heavy(p.arg[i])) full = true; break;
-            case I_DBIN: case I_RDBIN:
-                if (dbin_is_heavy(p.arg[i] >> 1)) full = true;
-                if (dbin_needs_derivative_set(p.arg[i] >> 1)) dfun = true;
-                break;
-            case I_PUSH:                          // one saved intermediate: the derivative family; more: the full one
+            case I_BIN: case I_RBIN: if (bin_is_heavy(p.arg[i])) dfun = true; break;
+            case I_DBIN: case I_RDBIN: if (dbin_is_heavy(p.arg[i] >> 1)) dfun = true; break;
+            case I_PUSH:                          // one saved intermediate: set 3; more: the long-program family
                 dfun = true;
                 if (++saved > 1) full = true;
                 break;

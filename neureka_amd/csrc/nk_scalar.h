@@ -400,20 +400,14 @@ __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b
                     case NK_OP_MOD * 2 + 0: NK_EACH2(T(1) / y);
                     case NK_OP_DIV * 2 + 1:
                     case NK_OP_MOD * 2 + 1: NK_EACH2(ddiv_db_ref(x, y));
-                    default:
-                        if constexpr (FUNSET == 2) {             // (set 3, the derivative family, leaves pow to the full table)
-                            switch (op * 2 + d) {
-                                case NK_OP_POW * 2 + 0: NK_EACH2(dpow_da_ref(x, y));
-                                case NK_OP_POW * 2 + 1: NK_EACH2(dpow_db_ref(x, y));
-                                default: NK_EACH2(T(NAN) + x + y);
-                            }
-                        } else NK_EACH2(T(NAN) + x + y);
+                    case NK_OP_POW * 2 + 0: NK_EACH2(dpow_da_ref(x, y));
+                    case NK_OP_POW * 2 + 1: NK_EACH2(dpow_db_ref(x, y));
+                    default: NK_EACH2(T(NAN) + x + y);
                 }
             } else NK_EACH2(T(NAN) + x + y);
     }
 }
-inline bool dbin_is_heavy(int op) { return op == NK_OP_POW; }
-inline bool dbin_needs_derivative_set(int op) { return op == NK_OP_DIV || op == NK_OP_MOD; }
+inline bool dbin_is_heavy(int op) { return op == NK_OP_DIV || op == NK_OP_MOD || op == NK_OP_POW; }
 #undef NK_EACH2
 
 }  // namespace nk
