@@ -97,3 +97,60 @@ def test_config3_single_kernels_full_size(device, orc):
         assert out.getData().tobytes() == want.tobytes(), op
     for t in (ta, tb, out):
         device.free(t)
+
+
+def test_backward_and_heavy_kernels_full_size(device, orc):
+    """The launches the backward pass and the heavy functions make, each alone on 2^25 elements (128 MiB: the variants
+    with non-temporal loads): the derivatives of tanh, sig, relu and of a division, sin, log10, softplus, cbrt, modulo and
+    power -- element by element within 1e-5 of the oracle (relu' and modulo bit for bit) -- and the three derivative
+    programs of the fused chain against the product of the oracle's single derivatives."""
+    from neureka_amd import Function
+    n = 1 << 25
+    rng = np.random.default_rng(35)
+    a = rng.uniform(0.25, 3.0, n).astype(np.float32) * rng.choice(np.array([-1, 1], dtype=np.float32), n)
+    b = rng.uniform(0.5, 2.0, n).astype(np.float32)
+    c = rng.standard_normal(n).astype(np.float32)
+    cfg = orc.dense_cfg([n])
+    ta, tb, tc = (Tensor.of(np.float32, (n,), v).to(device) for v in (a, b, c))
+    out = Tensor._on_device(device, np.float32, (n,))
+    zeros = lambda: np.zeros(n, dtype=np.float32)
+
+    def close(got, want, what):
+        err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+        assert (err <= RTOL * np.abs(want.astype(np.float64)) + ATOL).all(), f"{what}: worst relative error {np.max(err / np.maximum(np.abs(want), 1e-300)):.3e}"
+
+    for name, d, src, host in (("tanh", 0, ta, a), ("sig", 0, ta, a), ("relu", 0, ta, a), ("sin", -1, ta, a), ("softplus", -1, ta, a),
+                               ("log10", -1, tb, b), ("cbrt", -1, tb, b), ("sin", 0, ta, a)):
+        print(f"[case] full-size {name} d={d}", flush=True)
+        device.launch_activation(name, d, out, src)
+        want = orc.activation(name, d, zeros(), cfg, host, cfg, workers=16)
+        if name == "relu":
+            assert out.getData().tobytes() == want.tobytes()
+        else:
+            close(out.getData(), want, f"{name} d={d}")
+    for op, d in (("divide", 0), ("divide", 1), ("modulo", -1), ("power", -1)):
+        print(f"[case] full-size {op} d={d}", flush=True)
+        x = tb if op == "power" else ta
+        hx = b if op == "power" else a
+        device.launch_elementwise(op, d, out, x, tb)
+        want = orc.elementwise(op, d, zeros(), cfg, hx, cfg, b, cfg, workers=16)
+        if op == "modulo":
+            assert out.getData().tobytes() == want.tobytes()
+        else:
+            close(out.getData(), want, f"{op} d={d}")
+    print("[case] full-size derivatives of the fused chain", flush=True)
+    fused = device.optimizedFunctionOf(Function.of("tanh(sig(I[0])*I[1]+I[2])"), "chain")
+    # (1 - t^2 is the difference of quantised floats once tanh saturates: it follows the last bit of its argument, so the
+    # argument is built from the forward kernel's own sigmoid, checked against the oracle in the test above)
+    device.launch_activation("sig", -1, out, ta)
+    s = out.getData()
+    p = ((s * b).astype(np.float32) + c).astype(np.float32)
+    dt = orc.activation("tanh", 0, zeros(), cfg, p, cfg, workers=16).astype(np.float64)
+    ds = orc.activation("sig", 0, zeros(), cfg, a, cfg, workers=16).astype(np.float64)
+    wants = (dt * (ds * b), dt * s, dt)
+    for i, want in enumerate(wants):
+        got = fused.derive([ta, tb, tc], i).getData().astype(np.float64)
+        # the program multiplies rounded floats where this reference multiplies doubles: a few roundings on top
+        assert (np.abs(got - want) <= 4 * RTOL * np.abs(want) + ATOL).all(), i
+    for t in (ta, tb, tc, out):
+        device.free(t)
