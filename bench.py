@@ -364,9 +364,14 @@ def main():
         hbm("activation_sig", 8 * n, dev.prepared_launch("activation", "sig", -1, o, srcs[0]))
         hbm("elementwise_add", 12 * n, dev.prepared_launch("elementwise", "add", -1, o, srcs[0], srcs[1]))
         hbm("elementwise_mul", 12 * n, dev.prepared_launch("elementwise", "multiply", -1, o, srcs[0], srcs[1]))
+        # what the backward pass launches for an activation and for a division, and a heavy forward function
+        hbm("activation_tanh_derivative", 8 * n, dev.prepared_launch("activation", "tanh", 0, o, srcs[0]))
+        hbm("activation_relu_derivative", 8 * n, dev.prepared_launch("activation", "relu", 0, o, srcs[0]))
+        hbm("divide_derivative", 12 * n, dev.prepared_launch("elementwise", "divide", 1, o, srcs[0], srcs[1]))
+        hbm("activation_softplus", 8 * n, dev.prepared_launch("activation", "softplus", -1, o, srcs[0]))
         # the slow tails of the elementwise engine, measured so that they are on record: the derivative kernel of the fused
-        # chain (the full function table, one pass per block), general power (the device library's float pow: arithmetic,
-        # not memory, bounds it) and a view no fast path takes (every 16th column of every 2nd row: one element per thread)
+        # chain (double-precision intermediates), general power (the device library's float pow: arithmetic, not memory,
+        # bounds both) and a view no fast path takes (every 16th column of every 2nd row: one element per thread)
         dprog, dconsts = fused.derivative_program(0)
         hbm("chain_derivative_by_input0", 16 * n, dev.prepared_launch("fused", dprog, dconsts, o, srcs))
         pos = Tensor.of(f32, (n,), rng.uniform(0.1, 2.0, n).astype(f32)).to(dev)
