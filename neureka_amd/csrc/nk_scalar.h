@@ -232,11 +232,30 @@ __device__ __forceinline__ float sig_f32_via_f64(float x) { return (float)(1.0 /
 // about -16 the sum 1 + exp(x) keeps only a few bits of exp(x): its result is exp(x) rounded to a multiple of
 // 2^-52 (0 or 2.2e-16 around x = -36.7).  Parity is with those results, so the f32 kernel repeats the double
 // formula there; above, log1p of the float exponential agrees with it to a few ulp.
+// f32 above -13: max(x, 0) + log1p(e), e = exp(-|x|) in (0, 1] -- one evaluation for both signs -- with
+// log1p(e) = 2 atanh(s), s = e / (2 + e) <= 1/3, as the odd series up to s^13 (the next term is 1.3e-8 relative at s = 1/3);
+// e from the hardware exp2 with its argument's rounding error carried along (1.3e-6 relative at the far end).
+__device__ __forceinline__ float softplus_f32(float x) {
+    const float e = fast_exp_neg(::fabsf(x));
+    const float s = e * __builtin_amdgcn_rcpf(2.0f + e);
+    const float s2 = s * s;
+    float p = 0.0769230798f;                                     // 1/13, 1/11, ... 1/3
+    p = __builtin_fmaf(p, s2, 0.0909090936f);
+    p = __builtin_fmaf(p, s2, 0.111111112f);
+    p = __builtin_fmaf(p, s2, 0.142857149f);
+    p = __builtin_fmaf(p, s2, 0.200000003f);
+    p = __builtin_fmaf(p, s2, 0.333333343f);
+    p = __builtin_fmaf(p, s2, 1.0f);
+    const float r = 2.0f * s * p;
+    return (x > 0.0f ? x : 0.0f) + r;                            // (a NaN arrives through r)
+}
 template <typename T> __device__ __forceinline__ T softplus_ref(T x) {
     using N = Num<T>;
-    if (sizeof(T) == 8) return N::log(T(1) + N::exp(x));
-    if (x < T(-13)) return T(::log(1.0 + ::exp((double)x)));
-    return x > T(0) ? x + N::log1p(N::exp(-x)) : N::log1p(N::exp(x));
+    if constexpr (sizeof(T) == 8) return N::log(T(1) + N::exp(x));
+    else {
+        if (x < T(-13)) return T(::log(1.0 + ::exp((double)x)));
+        return softplus_f32(x);
+    }
 }
 template <typename T> __device__ __forceinline__ T dgasu_ref(T x) {
     T x2 = x * x, x6 = x2 * x2 * x2;
