@@ -216,13 +216,16 @@ int nk_matmul_set(nk_dev dev, int dtype, int layout, int64_t M, int64_t K, int64
  *     NK_FUSE_BIN   op  pop b, pop a, push a op b (NK_OP_ADD..NK_OP_POW)
  * The single value left on the stack is stored to the drain.  Each intermediate is rounded to the
  * tensor dtype exactly as the unfused kernels round it, so + - * stay bit-identical to the unfused
- * sequence.  n_src <= NK_FUSE_MAX_SRC, n_ops <= NK_FUSE_MAX_OPS, stack depth <= NK_FUSE_MAX_STACK per launch: the host
- * cuts a larger expression into several launches through temporaries, which changes no result because of that rounding. */
+ * sequence.  n_src <= NK_FUSE_MAX_SRC, n_ops <= NK_FUSE_MAX_OPS, stack depth <= NK_FUSE_MAX_STACK per launch, and at most
+ * NK_FUSE_MAX_SAVED computed operands may wait at once for the evaluation of their right-hand neighbour (a plain source
+ * or constant never waits: it is read where it is used).  The host cuts a larger expression into several launches
+ * through temporaries, which changes no result because of that rounding. */
 enum { NK_FUSE_LOAD = 0, NK_FUSE_CONST = 1, NK_FUSE_FUN = 2, NK_FUSE_DFUN = 3, NK_FUSE_BIN = 4 };
 #define NK_FUSE_MAX_SRC 6
 #define NK_FUSE_MAX_OPS 32
 #define NK_FUSE_MAX_STACK 8
 #define NK_FUSE_MAX_CONST 8
+#define NK_FUSE_MAX_SAVED 4
 int nk_fused(nk_dev dev, const int32_t* program, int n_ops, const double* consts, int n_consts,
              int dtype, int rank, nk_buf drn, const int32_t* drn_cfg,
              int n_src, const nk_buf* srcs, const int32_t* const* src_cfgs, int64_t n);

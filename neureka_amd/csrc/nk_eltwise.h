@@ -22,7 +22,7 @@ namespace nk {
 enum : int { I_SET = 0, I_FUN, I_DFUN, I_BIN, I_RBIN, I_DBIN, I_RDBIN, I_PUSH };
 constexpr int SRC_CONST0 = 16, SRC_POP = 32;
 constexpr int MAX_INSTR = 48;
-constexpr int HW_STACK = 4;
+constexpr int HW_STACK = NK_FUSE_MAX_SAVED;
 
 struct alignas(32) Prog {
     unsigned code[MAX_INSTR];      // op | arg << 8 | src << 16, what the device reads: eight words per scalar load

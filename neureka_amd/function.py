@@ -320,7 +320,7 @@ def derivative_of(n: Node, index: int) -> Node:
 
 
 # what one launch of nk_fused takes (include/neureka_hip.h: NK_FUSE_MAX_*)
-FUSE_MAX_SRC, FUSE_MAX_OPS, FUSE_MAX_STACK, FUSE_MAX_CONST = 6, 32, 8, 8
+FUSE_MAX_SRC, FUSE_MAX_OPS, FUSE_MAX_STACK, FUSE_MAX_CONST, FUSE_MAX_SAVED = 6, 32, 8, 8, 4
 
 
 def _fuse_cost(n: Node):
@@ -337,14 +337,52 @@ def _fuse_cost(n: Node):
     return o1 + o2 + 1, max(d1, d2 + 1), l1 | l2, c1 | c2
 
 
+def _fuse_saved(n: Node) -> int:
+    """How many intermediate results the program of the tree holds at once while it evaluates another sub-expression.
+    The kernel works on one accumulator: an operand that is a plain source or constant is read where it is used,
+    a computed operand that has to wait for the evaluation of its right-hand neighbour is saved (the rule nk_fused
+    applies when it translates the postfix program)."""
+    LAZY, ACC, SAVED = 0, 1, 2
+    stack, saved, peak = [], 0, 0
+
+    def save_acc():
+        nonlocal saved, peak
+        for i, kind in enumerate(stack):
+            if kind == ACC:
+                stack[i] = SAVED
+                saved += 1
+        peak = max(peak, saved)
+
+    def walk(m: Node):
+        nonlocal saved
+        if not m.children:
+            stack.append(LAZY)
+        elif m.kind in ("fun", "dfun"):
+            walk(m.children[0])
+            if stack[-1] == LAZY:
+                save_acc()
+                stack[-1] = ACC
+        else:
+            walk(m.children[0]); walk(m.children[1])
+            rhs, lhs = stack.pop(), stack.pop()
+            if lhs == LAZY and rhs == LAZY:
+                save_acc()
+            elif lhs == SAVED:
+                saved -= 1
+            stack.append(ACC)
+    walk(n)
+    return peak
+
+
 def _fuse_fits(n: Node) -> bool:
     ops, depth, leaves, consts = _fuse_cost(n)
-    return ops <= FUSE_MAX_OPS and depth <= FUSE_MAX_STACK and len(leaves) <= FUSE_MAX_SRC and len(consts) <= FUSE_MAX_CONST
+    return (ops <= FUSE_MAX_OPS and depth <= FUSE_MAX_STACK and len(leaves) <= FUSE_MAX_SRC and len(consts) <= FUSE_MAX_CONST
+            and _fuse_saved(n) <= FUSE_MAX_SAVED)
 
 
 def plan_fused(root: Node):
     """Cuts an expression that is too large for one launch of nk_fused (more than 6 sources, 32 op-codes, 8 stack
-    entries or 8 constants) into stages: the largest sub-expressions are evaluated into temporaries first, which
+    entries, 8 constants or 4 saved intermediates) into stages: the largest sub-expressions are evaluated into temporaries first, which
     later stages read as sources.  Every intermediate of a fused program is rounded to the tensor's element type as
     the unfused kernels round it, so a temporary holds exactly what the single program would have had on its stack
     (CLFunctionCompiler generates one OpenCL kernel whatever the size, CLFunctionCompiler.java:101-199).

@@ -944,7 +944,8 @@ def test_fused_chain_equals_unfused_and_oracle(device, orc, dt):
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
 def test_fused_functions_beyond_one_launch(device, dt):
-    """Expressions with more than 6 inputs, 32 op-codes or 8 constants run as several launches through temporaries:
+    """Expressions with more than 6 inputs, 32 op-codes, 8 constants or 4 waiting intermediates run as several launches
+    through temporaries:
     the same bits as the unfused graph for + - * (every intermediate is rounded to the element type either way), no
     buffer left behind, and derivatives -- far larger trees than the functions themselves -- through the same staging,
     against central differences in f64."""
@@ -953,7 +954,9 @@ def test_fused_functions_beyond_one_launch(device, dt):
     shape = (33, 40)
     exprs = ["relu(I[0]*I[1]+I[2])*quad(I[3]-I[4])+abs(I[5]*I[6])-I[7]*I[8]+I[9]",
              "+".join(f"quad(I[{k % 3}]*{k + 1}.5-I[{(k + 1) % 3}])" for k in range(14)),
-             "I[0]" + "".join(f"{'+-'[k % 2]}(I[1]*{k}.25)" for k in range(40))]
+             "I[0]" + "".join(f"{'+-'[k % 2]}(I[1]*{k}.25)" for k in range(40)),
+             # 27 op-codes, 6 inputs, 8 stack entries, but six products wait for the seventh
+             "I[0]*I[1]+(I[1]*I[2]+(I[2]*I[3]+(I[3]*I[4]+(I[4]*I[5]+(I[5]*I[0]+I[0]*I[2])))))"]
     for expr in exprs:
         say("fused beyond one launch", dt, expr[:60])
         fn = Function.of(expr)

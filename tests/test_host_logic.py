@@ -114,10 +114,10 @@ def test_parser_and_fused_lowering():
 
 
 def test_expressions_beyond_one_launch_are_cut_into_stages():
-    """plan_fused: more than 6 sources, 32 op-codes, 8 stack entries or 8 constants per launch make several stages
+    """plan_fused: more than 6 sources, 32 op-codes, 8 stack entries, 8 constants or 4 waiting results per launch make several stages
     through temporaries; each stage respects the limits, and interpreting the stages gives the tree's own value
     (float32 after every operation, as the kernels round)."""
-    from neureka_amd.function import FUSE_MAX_CONST, FUSE_MAX_OPS, FUSE_MAX_SRC, FUSE_MAX_STACK, plan_fused
+    from neureka_amd.function import FUSE_MAX_CONST, FUSE_MAX_OPS, FUSE_MAX_SAVED, FUSE_MAX_SRC, FUSE_MAX_STACK, plan_fused
     rng = np.random.default_rng(8)
     f32 = np.float32
     inv_fun = {v: k for k, v in _lib.FUN.items()}; inv_op = {v: k for k, v in _lib.OP.items()}
@@ -136,16 +136,20 @@ def test_expressions_beyond_one_launch_are_cut_into_stages():
             ops = len(program) // 2
             assert ops <= FUSE_MAX_OPS and len(leaves) <= FUSE_MAX_SRC and len(consts) <= FUSE_MAX_CONST
             srcs = [xs[v] if kind == "input" else temps[v] for kind, v in leaves]
-            stack, deepest = [], 0
+            stack, computed, deepest, waiting = [], [], 0, 0
             for code, arg in zip(program[0::2], program[1::2]):
-                if code == _lib.FUSE_LOAD: stack.append(srcs[arg])
-                elif code == _lib.FUSE_CONST: stack.append(np.full_like(xs[0], consts[arg]))
-                elif code == _lib.FUSE_FUN: stack.append(np_fun[inv_fun[arg]](stack.pop()).astype(f32))
+                if code == _lib.FUSE_LOAD: stack.append(srcs[arg]); computed.append(False)
+                elif code == _lib.FUSE_CONST: stack.append(np.full_like(xs[0], consts[arg])); computed.append(False)
+                elif code == _lib.FUSE_FUN:
+                    stack.append(np_fun[inv_fun[arg]](stack.pop()).astype(f32)); computed[-1] = True
                 else:
                     b = stack.pop(); a = stack.pop()
                     stack.append(np_op[inv_op[arg]](a, b).astype(f32))
+                    computed.pop(); computed[-1] = True
                 deepest = max(deepest, len(stack))
-            assert len(stack) == 1 and deepest <= FUSE_MAX_STACK
+                if computed[-1]:                         # results under a fresh result wait in the kernel's save slots
+                    waiting = max(waiting, sum(computed[:-1]))
+            assert len(stack) == 1 and deepest <= FUSE_MAX_STACK and waiting <= FUSE_MAX_SAVED, (deepest, waiting)
             temps[k] = stack[0]
         return temps[len(stages) - 1]
 
@@ -155,7 +159,8 @@ def test_expressions_beyond_one_launch_are_cut_into_stages():
              "+".join(f"quad(i{k % 3}*{k + 1}.5-i{(k + 1) % 3})" for k in range(14)),                # 14 constants, ~100 op-codes
              "i0" + "".join(f"{'+-'[k % 2]}(i1*{k}.25)" for k in range(40)),                           # a long chain
              "(" * 12 + "i0" + "".join(f"+i{1 + k % 2})*i{k % 3}" for k in range(12)),               # nested to the left
-             "+".join(f"(i{k % 3}*i{(k + 1) % 3}" for k in range(12)) + ")" * 12]                    # nested to the right: a deep stack
+             "+".join(f"(i{k % 3}*i{(k + 1) % 3}" for k in range(12)) + ")" * 12,                    # nested to the right: a deep stack
+             "i0*i1+(i1*i2+(i2*i3+(i3*i4+(i4*i5+(i5*i0+i0*i2)))))"]                                  # 27 op-codes, 8 deep, six results wait
     for expr in cases:
         fn = Function.of(expr)
         stages = plan_fused(fn.root)
