@@ -774,12 +774,13 @@ static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, bool over
 // Few tiles cannot fill 256 compute units (a 512^3 product has 16, a matrix-vector product a single row of them):
 // the k range is then cut into parts until there are about two blocks per unit, each part at least four
 // k-slices long; the parts are written to the device workspace and added in order by a second launch.
-static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes) {
+// (`force_parts` >= 2: the caller has planned the number of parts itself, see the row bands in matmul_rm)
+static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes, int force_parts = 0) {
     const int tiles = g.tiles_m * g.tiles_n, cus = dev->props.multiProcessorCount;
     const int slices = (g.K + slice - 1) / slice;
     g.splits = 1; g.split_slices = slices;
-    if (tiles >= cus || slices < 8) return 1;
-    int parts = (2 * cus + tiles - 1) / tiles;
+    if (force_parts < 2 && (tiles >= cus || slices < 8)) return 1;
+    int parts = force_parts >= 2 ? force_parts : (2 * cus + tiles - 1) / tiles;
     if (parts > slices / 4) parts = slices / 4;
     if (parts > 64) parts = 64;
     // bound the workspace: parts * M * N elements
@@ -791,10 +792,10 @@ static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes) {
 }
 
 template <typename T, typename Launch>
-static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch) {
+static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch, int force_parts = 0) {
     const int tiles = g.tiles_m * g.tiles_n;
     void* ws = nullptr;
-    if (split_plan(dev, g, slice, sizeof(T)) > 1) {
+    if (split_plan(dev, g, slice, sizeof(T), force_parts) > 1) {
         const int64_t mn = (int64_t)g.M * g.N;
         if (int e = workspace(dev, (uint64_t)g.splits * mn * sizeof(T), &ws)) return e;
         launch(true, dim3((unsigned)(tiles * g.splits)), (T*)ws);
@@ -806,26 +807,59 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
     return NK_OK;
 }
 
-static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C) {
+// `force_parts`, `bands`: how matmul_rm calls itself for the two row bands described below (callers leave them alone)
+static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C,
+                     int force_parts = 0, bool bands = true) {
     constexpr int64_t mfma_from = (int64_t)1 << 24;
     MfmaArgs g{};
     g.M = (int)M; g.K = (int)K; g.N = (int)N;
     g.tiles_m = (int)((M + BM - 1) / BM); g.tiles_n = (int)((N + BN - 1) / BN);
     g.group_rows = g.tiles_m < 8 ? g.tiles_m : 8;
     g.overwrite = overwrite ? 1 : 0;
+    // Row bands.  Two blocks of a 128 x 128 kernel live on a compute unit, so a launch runs in rounds of 2 x units
+    // tiles, and a last round with few tiles costs a whole tile's time on a machine that is mostly idle (f32 3072^3:
+    // 576 tiles = one full round + 64 tiles, 100 TFLOP/s; as bands 119-128).  The product is then computed as two
+    // products over row bands of A and C, which are matrices of their own in row-major storage: the upper band holds
+    // whole rounds of tiles, the lower band's few tiles cut their k range into parts so that they fill one more, short,
+    // round (partial results through the workspace, added in order as for every split product).  Times are in units
+    // of one tile's time on a compute unit of its own.  Returns -1 when the product is better off in one piece.
+    auto run_bands = [&](int elem_bytes, int64_t slices, const char* path) -> int {
+        if (!bands) return -1;
+        const int64_t cus = dev->props.multiProcessorCount, resident = 2 * cus;
+        const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+        if (tiles <= resident || tiles >= 8 * resident) return -1;
+        const int64_t rows_a = (tiles / resident) * resident / g.tiles_n;               // whole tile rows of the upper band
+        const int64_t tiles_a = rows_a * g.tiles_n, tiles_b = tiles - tiles_a;
+        if (rows_a < 1 || tiles_b < 1) return -1;
+        int64_t parts = resident / tiles_b;
+        if (parts > slices / 4) parts = slices / 4;
+        if (parts > 64) parts = 64;
+        const int64_t m_a = rows_a * BM, m_b = M - m_a;
+        const int64_t per16 = 16 / elem_bytes;                                           // the bands keep the alignment of the whole
+        if (parts < 2 || m_b * K * N < mfma_from || (m_a * K) % per16 != 0 || (m_a * N) % per16 != 0) return -1;
+        const double now = (double)((tiles + cus - 1) / cus);
+        const double part_len = (double)((slices + parts - 1) / parts) / (double)slices;
+        const double then = (double)((tiles_a + cus - 1) / cus) + 2.0 * part_len + 0.15;     // + two more launches
+        if (then >= 0.95 * now) return -1;
+        if (int e = matmul_rm(dev, dtype, overwrite, m_a, K, N, A, B, C, 0, false)) return e;
+        if (int e = matmul_rm(dev, dtype, overwrite, m_b, K, N, A + (uint64_t)(m_a * K) * elem_bytes, B, C + (uint64_t)(m_a * N) * elem_bytes, (int)parts, false)) return e;
+        set_path(path);
+        return NK_OK;
+    };
     if (dtype == NK_F64) {
         // from 2^24 multiply-adds on the matrix cores take over (sums re-ordered, within 1e-12 of the reference);
         // smaller products keep the reference's summation order bit for bit
         const bool fits = M * K * 8 < ((int64_t)1 << 32) && K * N * 8 < ((int64_t)1 << 32);
         if (M * K * N >= mfma_from && fits) {
             const bool whole = (A % 16 == 0) && (B % 16 == 0) && M % BM == 0 && N % BN == 0 && K % d64::DK == 0;
+            if (const int rc = run_bands(8, (K + d64::DK - 1) / d64::DK, whole ? "mfma_f64_bands" : "mfma_f64_edge_bands"); rc >= 0) return rc;
             const double* Ap = (const double*)A; const double* Bp = (const double*)B; double* Cp = (double*)C;
             const int rc = launch_mfma<double>(dev, g, d64::DK, Cp, [&](bool split, dim3 grid, double* P) {
                 if (whole && split)       hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
                 else if (whole)           hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
                 else if (split)           hipLaunchKernelGGL((matmul_mfma_f64_kernel<true, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
                 else                      hipLaunchKernelGGL((matmul_mfma_f64_kernel<true, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
-            });
+            }, force_parts);
             set_path(whole ? (g.splits > 1 ? "mfma_f64_split" : "mfma_f64") : (g.splits > 1 ? "mfma_f64_edge_split" : "mfma_f64_edge"));
             return rc;
         }
@@ -875,6 +909,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 return NK_OK;
             }
         }
+        if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;
         bool streamed = false;
         const int rc = launch_mfma<float>(dev, g, BK, Cp, [&](bool split, dim3 grid, float* P) {
             if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
@@ -894,7 +929,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             }
             else if (split)           hipLaunchKernelGGL((matmul_mfma_kernel<true, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
             else                      hipLaunchKernelGGL((matmul_mfma_kernel<true, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
-        });
+        }, force_parts);
         set_path(streamed ? "mfma_stream" : whole_tiles ? (g.splits > 1 ? "mfma_split" : "mfma") : (g.splits > 1 ? "mfma_edge_split" : "mfma_edge"));
         return rc;
     }

@@ -1790,6 +1790,59 @@ def test_matmul_256_tiles_with_edges(device, mkn):
     assert_bits(got[pad:pad + M * N].reshape(M, N), want + C0, "parked operands")
 
 
+@pytest.mark.parametrize("mkn", [(3072, 1024, 3072), (3000, 800, 3100), (1280, 1024, 8192), (2700, 640, 3400)])
+def test_matmul_row_bands(device, mkn):
+    """Products whose 128 x 128 tiles are a few more than whole rounds of the machine run as two row bands, the lower
+    one with its k range cut into parts: exact on integer data, C += A B into a non-zero C and C = A B into NaNs, both
+    layouts, and with the operands parked between NaNs (the bands start inside the buffers)."""
+    M, K, N = mkn
+    rng = np.random.default_rng(63)
+    whole = M % 128 == 0 and N % 128 == 0 and K % 32 == 0
+    path = "mfma_bands" if whole else "mfma_edge_bands"
+    say("matmul row bands, integers", mkn)
+    A = rng.integers(-3, 4, (M, K)).astype(np.float32); B = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    C0 = rng.integers(-9, 10, (M, N)).astype(np.float32)
+    want = A @ B                                             # exact: |sums| < 2^24
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert_bits(tc.getData().reshape(M, N), want + C0, "C += A B")
+    say("matmul row bands, C = A B into NaNs", mkn)
+    tc = on(device, np.full((M, N), np.nan, dtype=np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert_bits(tc.getData().reshape(M, N), want, "C = A B")
+    say("matmul row bands, column major", mkn)
+    tc = on(device, C0.T.copy())
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+    assert_bits(tc.getData().reshape(N, M), (want + C0).T.copy(), "column major")
+    say("matmul row bands, operands inside larger buffers full of NaN", mkn)
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(C0)
+    _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert_bits(got[pad:pad + M * N].reshape(M, N), want + C0, "parked operands")
+    say("matmul row bands, uniform data against float64", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    tc = on(device, np.zeros((M, N), np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    scale = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+    assert (np.abs(tc.getData().reshape(M, N) - ref) <= 1e-5 * scale + 1e-30).all()
+    say("matmul row bands, float64", mkn)
+    A = rng.uniform(-1, 1, (M, K)); B = rng.uniform(-1, 1, (K, N)); C0 = rng.uniform(-1, 1, (M, N))
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == ("mfma_f64_bands" if M % 128 == 0 and N % 128 == 0 and K % 16 == 0 else "mfma_f64_edge_bands"), _lib.last_path()
+    assert (np.abs(tc.getData().reshape(M, N) - (ref_d := A @ B + C0)) <= 1e-12 * (np.abs(A) @ np.abs(B) + np.abs(C0))).all()
+
+
 def test_matmul_through_the_tensor_api(device):
     """a.matMul(b) with transposed and sliced operands (auto-clone), and its backward."""
     say("matmul tensor api")
