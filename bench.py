@@ -154,6 +154,7 @@ def torch_yardstick():
     t("dot_2^26_us", lambda: torch.dot(x, y))
     del x, y, z, out
     for name, (M, K, N), dt in (("matmul_4096_us", (4096, 4096, 4096), torch.float32), ("matmul_4000_us", (4000, 4000, 4000), torch.float32),
+                                ("matmul_3072_us", (3072, 3072, 3072), torch.float32), ("matmul_3072_f64_us", (3072, 3072, 3072), torch.float64),
                                 ("matmul_tall_skinny_us", (65536, 256, 256), torch.float32), ("matmul_4096_f64_us", (4096, 4096, 4096), torch.float64)):
         A = torch.randn(M, K, device=d, dtype=dt); B = torch.randn(K, N, device=d, dtype=dt); C = torch.empty(M, N, device=d, dtype=dt)
         t(name, lambda: torch.mm(A, B, out=C))
@@ -413,7 +414,8 @@ def main():
 
         # C4 matmul
         # (4000^3: a large shape that is no whole number of tiles)
-        for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256)), ("matmul_4000", (4000, 4000, 4000))):
+        for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256)), ("matmul_4000", (4000, 4000, 4000)),
+                                ("matmul_3072", (3072, 3072, 3072))):          # 576 tiles of 128 x 128: a round of the machine and an eighth
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
             Cm = Tensor._on_device(dev, f32, (M, N))
@@ -427,6 +429,12 @@ def main():
         B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)
         Cm = Tensor._on_device(dev, np.float64, (M, N))
         flops("matmul_4096_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm), f64=True)
+        for t in (A, B, Cm): dev.free(t)
+        M = K = N = 3072
+        A = Tensor.of(np.float64, (M, K), rng.uniform(-1, 1, M * K)).to(dev)
+        B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)
+        Cm = Tensor._on_device(dev, np.float64, (M, N))
+        flops("matmul_3072_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm), f64=True)
         for t in (A, B, Cm): dev.free(t)
 
         # C1 and C5 convolutions
