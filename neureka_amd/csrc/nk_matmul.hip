@@ -639,6 +639,108 @@ __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int pa
     C[i] = overwrite ? s : C[i] + s;
 }
 
+// ---- a few rows times a large matrix ----------------------------------------------------------------------------
+// C[M,N] = A[M,K] @ B[K,N] with M <= 16 (a vector or a small batch times a weight matrix): the product reads B once
+// and is bound by that stream; a 128 x 128 tile would spend its matrix cores on rows that do not exist.  A block owns
+// 64 * (16 bytes / element) columns and one part of the k range (at most few_kp(MR) rows), whose piece of A it stages
+// in LDS; each of its four wavefronts takes a quarter of the part -- a row of B is one contiguous kilobyte for a
+// wavefront, eight rows are requested before the first is used and the next eight while these are -- with MR
+// accumulators per column in registers (the elements of A come as 16-byte LDS reads of one address for the whole
+// wavefront), the wavefronts meet in LDS in a fixed order, and the block's partial rows go to P[part];
+// matmul_add_parts_kernel adds the parts in order.
+constexpr int few_kp(int mr) { return mr <= 4 ? 1024 : 256; }          // k rows a block stages of A: 16-32 KiB of LDS
+__device__ __forceinline__ float fma_of(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_of(double a, double b, double c) { return __builtin_fma(a, b, c); }
+template <typename T, int MR>
+__global__ __launch_bounds__(256) void matmul_few_rows_kernel(int M, int K, int N, int k_per_part, int col_blocks, const T* __restrict__ A,
+                                                              const T* __restrict__ B, T* __restrict__ P) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int UNROLL = 8;
+    constexpr int KP = few_kp(MR);
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    typedef T Quad __attribute__((ext_vector_type(4)));
+    constexpr int A_ELEMS = MR * KP, MEET_ELEMS = 3 * MR * 64 * VEC;
+    __shared__ __attribute__((aligned(16))) T lds[A_ELEMS > MEET_ELEMS ? A_ELEMS : MEET_ELEMS];
+    T (*As)[KP] = (T (*)[KP])lds;                                       // [MR][KP], zero past the part's end
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int part = (int)(blockIdx.x / (unsigned)col_blocks), col_block = (int)(blockIdx.x % (unsigned)col_blocks);
+    const int64_t col0 = ((int64_t)col_block * 64 + lane) * VEC;             // N % VEC == 0 (the host checks)
+    const bool live = col0 < N;
+    const int k_begin = part * k_per_part;
+    const int k_count = k_begin + k_per_part < K ? k_per_part : K - k_begin;  // 1 ... KP
+    const T* Bc = B + (live ? col0 : 0);
+    // the wavefront's quarter of the part, a multiple of UNROLL rows long
+    const int quarter = ((k_per_part + 4 * UNROLL - 1) / (4 * UNROLL)) * UNROLL;
+    const int kk_end = (wave + 1) * quarter < k_count ? (wave + 1) * quarter : k_count;
+    auto request = [&](Vec (&b)[UNROLL], int kk) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) {
+            const int row = kk + u < kk_end ? kk + u : kk_end - 1;      // (what a repeated last row brings is dropped below)
+            b[u] = *(const Vec*)(Bc + (int64_t)(k_begin + row) * N);
+        }
+    };
+    Vec b[UNROLL];
+    int kk = wave * quarter;
+    if (kk < kk_end) request(b, kk);                                    // in flight while the piece of A is staged
+    {
+        // thread t stages columns t, t + 256, ... of the piece: independent loads along the rows of A
+        const int t = threadIdx.x;
+        T av[KP / 256][MR];
+#pragma unroll
+        for (int c = 0; c < KP / 256; c++)
+#pragma unroll
+            for (int m = 0; m < MR; m++) av[c][m] = A[(int64_t)(m < M ? m : M - 1) * K + k_begin + (t + 256 * c < k_count ? t + 256 * c : 0)];
+#pragma unroll
+        for (int c = 0; c < KP / 256; c++)
+#pragma unroll
+            for (int m = 0; m < MR; m++) As[m][t + 256 * c] = (m < M && t + 256 * c < k_count) ? av[c][m] : T(0);
+    }
+    __syncthreads();
+    T acc[MR][VEC];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[m][e] = T(0);
+    for (; kk < kk_end; kk += UNROLL) {
+        Vec bn[UNROLL];
+        if (kk + UNROLL < kk_end) request(bn, kk + UNROLL);             // the next rows, while these are used
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++)
+            if (kk + u >= kk_end) b[u] = Vec(T(0));                     // (only at the part's ragged end, where A is zero too)
+#pragma unroll
+        for (int q = 0; q < UNROLL; q += 4)
+#pragma unroll
+            for (int m = 0; m < MR; m++) {
+                const Quad a = *(const Quad*)&As[m][kk + q];
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) acc[m][e] = fma_of(a[u], b[q + u][e], acc[m][e]);
+            }
+#pragma unroll
+        for (int u = 0; u < UNROLL; u++) b[u] = bn[u];
+    }
+    __syncthreads();                                                    // the staged piece of A makes room for the meeting
+    T (*meet)[MR][64 * VEC] = (T (*)[MR][64 * VEC])lds;
+    if (wave > 0) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) *(Vec*)&meet[wave - 1][m][lane * VEC] = *(const Vec*)acc[m];
+    }
+    __syncthreads();
+    if (wave == 0 && live) {
+        T* Pp = P + (int64_t)part * M * N + col0;
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            if (m < M) {
+                Vec v = *(const Vec*)acc[m];
+#pragma unroll
+                for (int w = 0; w < 3; w++) v = v + *(const Vec*)&meet[w][m][lane * VEC];
+                *(Vec*)(Pp + (int64_t)m * N) = v;
+            }
+        }
+    }
+}
+
 // ---- f64 on the matrix cores ----------------------------------------------------------------------------------
 // 128x128 block tile, four wavefronts in a 2x2 arrangement, each owning 64x64 as 4x4 accumulators of
 // v_mfma_f64_16x16x4_f64 (register v of lane l holds row 4*v + l/16 of column l%16 of a 16x16 tile; it feeds A[row l%16]
@@ -846,6 +948,41 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         set_path(path);
         return NK_OK;
     };
+    // a few rows of A: one stream over B (from 2^24 multiply-adds on, where the sums are re-ordered anyway)
+    if (bands && M <= 16 && M * K * N >= mfma_from) {
+        const int eb = dtype == NK_F64 ? 8 : 4, vec = 16 / eb;
+        if (N % vec == 0 && B % 16 == 0 && N >= 64 * vec) {
+            const int64_t col_blocks = (N + 64 * vec - 1) / (64 * vec);
+            // about two blocks per compute unit, a part at least 32 k rows long (eight per wavefront)
+            int64_t parts = (2 * (int64_t)dev->props.multiProcessorCount + col_blocks - 1) / col_blocks;
+            if (parts > K / 32) parts = K / 32;
+            if (parts < 1) parts = 1;
+            int k_per_part = (int)((K + parts - 1) / parts);
+            const int mr = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+            if (k_per_part > few_kp(mr)) k_per_part = few_kp(mr);          // what a block stages of A
+            parts = (K + k_per_part - 1) / k_per_part;
+            void* ws = nullptr;
+            if (int e = workspace(dev, (uint64_t)parts * M * N * eb, &ws)) return e;
+            const dim3 grid((unsigned)(col_blocks * parts));
+            auto launch = [&](auto t, auto mr) {
+                using T = decltype(t);
+                hipLaunchKernelGGL((matmul_few_rows_kernel<T, decltype(mr)::value>), grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, k_per_part, (int)col_blocks,
+                                   (const T*)A, (const T*)B, (T*)ws);
+                hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, dev->stream, M * N, (int)parts, g.overwrite, (const T*)ws, (T*)C);
+            };
+            auto by_rows = [&](auto t) {
+                if (M <= 1) launch(t, std::integral_constant<int, 1>{});
+                else if (M <= 2) launch(t, std::integral_constant<int, 2>{});
+                else if (M <= 4) launch(t, std::integral_constant<int, 4>{});
+                else if (M <= 8) launch(t, std::integral_constant<int, 8>{});
+                else launch(t, std::integral_constant<int, 16>{});
+            };
+            if (dtype == NK_F64) by_rows(double{}); else by_rows(float{});
+            NK_HIP(hipGetLastError());
+            set_path(dtype == NK_F64 ? "few_rows_f64" : "few_rows");
+            return NK_OK;
+        }
+    }
     if (dtype == NK_F64) {
         // from 2^24 multiply-adds on the matrix cores take over (sums re-ordered, within 1e-12 of the reference);
         // smaller products keep the reference's summation order bit for bit

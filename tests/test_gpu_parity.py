@@ -1616,13 +1616,14 @@ def test_matmul_split_k(device, orc, mkn, dt):
     A = rng.integers(-4, 5, (M, K)).astype(T); B = rng.integers(-4, 5, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
     tc = on(device, C0)
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
-    assert _lib.last_path().endswith("_split"), _lib.last_path()
+    few_rows = lambda rows, cols: rows <= 16 and cols % (16 // np.dtype(T).itemsize) == 0 and cols >= 1024 // np.dtype(T).itemsize
+    assert _lib.last_path().endswith("_split") or (few_rows(M, N) and _lib.last_path().startswith("few_rows")), _lib.last_path()
     assert (tc.getData().reshape(M, N) == A.astype(np.float64) @ B.astype(np.float64) + C0).all()
     say("matmul split-k uniform", mkn, dt)
     A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
     tc = on(device, np.zeros((M, N), dtype=T))
     device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)          # column-major operands
-    assert _lib.last_path().endswith("_split"), _lib.last_path()
+    assert _lib.last_path().endswith("_split") or (few_rows(N, M) and _lib.last_path().startswith("few_rows")), _lib.last_path()
     ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
     bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
     assert (np.abs(tc.getData().reshape(N, M).T.astype(np.float64) - ref) <= bound).all()
@@ -1788,6 +1789,57 @@ def test_matmul_256_tiles_with_edges(device, mkn):
     got = pc.getData()
     assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
     assert_bits(got[pad:pad + M * N].reshape(M, N), want + C0, "parked operands")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("mkn", [(1, 4096, 4096), (16, 4096, 4096), (3, 5001, 4100), (8, 2049, 1024), (2, 70000, 256), (5, 33, 131072), (13, 8192, 512)])
+def test_matmul_few_rows(device, orc, mkn, dt):
+    """A vector or a small batch times a large matrix (at most 16 rows, from 2^24 multiply-adds on) runs as one stream
+    over the matrix with the k range in parts: exact on integer data, C += A B into a non-zero C and C = A B into NaNs,
+    column major (a large matrix times a few columns), operands parked between NaNs, uniform data against the oracle."""
+    M, K, N = mkn
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    path = "few_rows" if dt == "f32" else "few_rows_f64"
+    rng = np.random.default_rng(64)
+    say("matmul few rows, integers", mkn, dt)
+    A = rng.integers(-3, 4, (M, K)).astype(T); B = rng.integers(-3, 4, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul few rows, C = A B into NaNs", mkn, dt)
+    tc = on(device, np.full((M, N), np.nan, dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want).all()
+    say("matmul few rows, column major: a large matrix times a few columns", mkn, dt)
+    # column-major [N,K] @ [K,M]: the row-major data of the transposes
+    tc = on(device, C0)
+    device.launch_matmul(False, N, K, M, on(device, B), on(device, A), tc)      # B's row-major data = column-major B^T[N,K], likewise A
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()                      # column-major C^T[N,M] = row-major C[M,N]
+    say("matmul few rows, operands inside larger buffers full of NaN", mkn, dt)
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=T)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(C0)
+    eb = np.dtype(T).itemsize
+    _lib.check(device._lib.nk_matmul(device.handle, 0 if dt == "f32" else 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + eb * pad, pb._data.ptr + eb * pad, pc._data.ptr + eb * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
+    say("matmul few rows, uniform data against the oracle", mkn, dt)
+    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
+    tc = on(device, np.zeros((M, N), dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
 @pytest.mark.parametrize("mkn", [(3072, 1024, 3072), (3000, 800, 3100), (1280, 1024, 8192), (2700, 640, 3400)])
