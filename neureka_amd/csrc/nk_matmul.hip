@@ -741,6 +741,88 @@ __global__ __launch_bounds__(256) void matmul_few_rows_kernel(int M, int K, int 
     }
 }
 
+// ---- a large matrix times a few columns -----------------------------------------------------------------------
+// C[M,NC] = A[M,K] @ B[K,NC] with NC = 1, 2 or 4 (a weight matrix times a vector): one stream over A.  A wavefront owns R rows
+// of A; its lanes walk along k with 16-byte loads (a row is read in contiguous kilobytes), every lane keeps R x NC
+// sums over its own k's -- the few elements of B it needs for them are 16-byte loads of a matrix that stays in the
+// caches -- and the 64 lanes' sums meet through wavefront shuffles at the end.  One launch, no partial results.
+template <typename T, int NC, int R, bool OVERWRITE>
+__global__ __launch_bounds__(256) void matmul_few_cols_kernel(int M, int K, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * R;
+    if (row0 >= M) return;                                              // (whole wavefronts; the kernel has no barrier)
+    const T* rows[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) rows[r] = A + (row0 + r < M ? row0 + r : M - 1) * (int64_t)K;
+    T acc[R][NC];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int n = 0; n < NC; n++) acc[r][n] = T(0);
+    constexpr int STEP = 64 * VEC;                                      // k's per trip of the wavefront
+    // K % VEC == 0 (the host checks): a lane's VEC k's are inside the matrix or all outside
+    auto request = [&](Vec (&a)[R], Vec (&b)[NC], int k0) {
+        const int k = k0 + lane * VEC;
+        const int kc = k < K ? k : 0;
+#pragma unroll
+        for (int r = 0; r < R; r++) a[r] = *(const Vec*)(rows[r] + kc);
+        // elements [k .. k + VEC) x [0 .. NC) of B are VEC * NC contiguous values: NC vectors
+#pragma unroll
+        for (int j = 0; j < NC; j++) b[j] = *(const Vec*)(B + (int64_t)kc * NC + j * VEC);
+        if (k >= K) {
+#pragma unroll
+            for (int r = 0; r < R; r++) a[r] = Vec(T(0));
+#pragma unroll
+            for (int j = 0; j < NC; j++) b[j] = Vec(T(0));
+        }
+    };
+    Vec a[R], b[NC];
+    request(a, b, 0);
+    for (int k0 = 0; k0 < K; k0 += STEP) {
+        Vec an[R], bn[NC];
+        if (k0 + STEP < K) request(an, bn, k0 + STEP);
+        // b as a flat run f[v * NC + n]
+        T f[VEC * NC];
+#pragma unroll
+        for (int j = 0; j < NC; j++)
+#pragma unroll
+            for (int e = 0; e < VEC; e++) f[j * VEC + e] = b[j][e];
+#pragma unroll
+        for (int v = 0; v < VEC; v++)
+#pragma unroll
+            for (int n = 0; n < NC; n++) {
+                const T bv = f[v * NC + n];
+#pragma unroll
+                for (int r = 0; r < R; r++) acc[r][n] = fma_of(a[r][v], bv, acc[r][n]);
+            }
+#pragma unroll
+        for (int r = 0; r < R; r++) a[r] = an[r];
+#pragma unroll
+        for (int j = 0; j < NC; j++) b[j] = bn[j];
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int n = 0; n < NC; n++) {
+            T v = acc[r][n];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
+            acc[r][n] = v;
+        }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (row0 + r < M)
+#pragma unroll
+                for (int n = 0; n < NC; n++) {
+                    T* c = C + (row0 + r) * (int64_t)NC + n;
+                    *c = OVERWRITE ? acc[r][n] : *c + acc[r][n];
+                }
+    }
+}
+
 // ---- f64 on the matrix cores ----------------------------------------------------------------------------------
 // 128x128 block tile, four wavefronts in a 2x2 arrangement, each owning 64x64 as 4x4 accumulators of
 // v_mfma_f64_16x16x4_f64 (register v of lane l holds row 4*v + l/16 of column l%16 of a 16x16 tile; it feeds A[row l%16]
@@ -980,6 +1062,35 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             if (dtype == NK_F64) by_rows(double{}); else by_rows(float{});
             NK_HIP(hipGetLastError());
             set_path(dtype == NK_F64 ? "few_rows_f64" : "few_rows");
+            return NK_OK;
+        }
+    }
+    // a few columns of B: one stream over A
+    if (bands && N <= 4 && M * K * N >= mfma_from) {
+        const int eb = dtype == NK_F64 ? 8 : 4, vec = 16 / eb;
+        if (K % vec == 0 && A % 16 == 0 && B % 16 == 0 && (N == 1 || N == 2 || N == 4)) {
+            auto launch = [&](auto t, auto nc) {
+                using T = decltype(t);
+                constexpr int NC = decltype(nc)::value;
+                // four rows per wavefront while that leaves two blocks per compute unit, else one
+                const bool four = (M + 15) / 16 >= 2 * (int64_t)dev->props.multiProcessorCount;
+                const unsigned blocks = (unsigned)(four ? (M + 15) / 16 : (M + 3) / 4);
+                if (four) {
+                    if (overwrite) hipLaunchKernelGGL((matmul_few_cols_kernel<T, NC, 4, true>), dim3(blocks), dim3(256), 0, dev->stream, (int)M, (int)K, (const T*)A, (const T*)B, (T*)C);
+                    else           hipLaunchKernelGGL((matmul_few_cols_kernel<T, NC, 4, false>), dim3(blocks), dim3(256), 0, dev->stream, (int)M, (int)K, (const T*)A, (const T*)B, (T*)C);
+                } else {
+                    if (overwrite) hipLaunchKernelGGL((matmul_few_cols_kernel<T, NC, 1, true>), dim3(blocks), dim3(256), 0, dev->stream, (int)M, (int)K, (const T*)A, (const T*)B, (T*)C);
+                    else           hipLaunchKernelGGL((matmul_few_cols_kernel<T, NC, 1, false>), dim3(blocks), dim3(256), 0, dev->stream, (int)M, (int)K, (const T*)A, (const T*)B, (T*)C);
+                }
+            };
+            auto by_cols = [&](auto t) {
+                if (N == 1) launch(t, std::integral_constant<int, 1>{});
+                else if (N == 2) launch(t, std::integral_constant<int, 2>{});
+                else launch(t, std::integral_constant<int, 4>{});
+            };
+            if (dtype == NK_F64) by_cols(double{}); else by_cols(float{});
+            NK_HIP(hipGetLastError());
+            set_path(dtype == NK_F64 ? "few_cols_f64" : "few_cols");
             return NK_OK;
         }
     }

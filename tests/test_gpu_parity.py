@@ -1617,13 +1617,17 @@ def test_matmul_split_k(device, orc, mkn, dt):
     tc = on(device, C0)
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
     few_rows = lambda rows, cols: rows <= 16 and cols % (16 // np.dtype(T).itemsize) == 0 and cols >= 1024 // np.dtype(T).itemsize
-    assert _lib.last_path().endswith("_split") or (few_rows(M, N) and _lib.last_path().startswith("few_rows")), _lib.last_path()
+    vec = 16 // np.dtype(T).itemsize
+    few_cols = lambda inner, cols: cols in (1, 2, 4) and inner % vec == 0
+    assert (_lib.last_path().endswith("_split") or (few_rows(M, N) and _lib.last_path().startswith("few_rows"))
+            or (few_cols(K, N) and _lib.last_path().startswith("few_cols"))), _lib.last_path()
     assert (tc.getData().reshape(M, N) == A.astype(np.float64) @ B.astype(np.float64) + C0).all()
     say("matmul split-k uniform", mkn, dt)
     A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
     tc = on(device, np.zeros((M, N), dtype=T))
     device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)          # column-major operands
-    assert _lib.last_path().endswith("_split") or (few_rows(N, M) and _lib.last_path().startswith("few_rows")), _lib.last_path()
+    assert (_lib.last_path().endswith("_split") or (few_rows(N, M) and _lib.last_path().startswith("few_rows"))
+            or (few_cols(K, M) and _lib.last_path().startswith("few_cols"))), _lib.last_path()
     ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
     bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
     assert (np.abs(tc.getData().reshape(N, M).T.astype(np.float64) - ref) <= bound).all()
@@ -1834,6 +1838,57 @@ def test_matmul_few_rows(device, orc, mkn, dt):
     assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
     assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
     say("matmul few rows, uniform data against the oracle", mkn, dt)
+    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
+    tc = on(device, np.zeros((M, N), dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("mkn", [(4096, 4096, 1), (4099, 4096, 1), (10000, 1000, 2), (513, 8192, 4), (70001, 64, 4), (17, 1048576, 1), (2, 2097152, 4)])
+def test_matmul_few_columns(device, orc, mkn, dt):
+    """A large matrix times a vector (1, 2 or 4 columns, from 2^24 multiply-adds on) runs as one stream over the matrix in
+    one launch: exact on integer data, C += A B into a non-zero C and C = A B into NaNs, column major (a vector times a
+    large matrix), operands parked between NaNs, uniform data against the oracle."""
+    M, K, N = mkn
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    few_rows = M <= 16 and N % (16 // np.dtype(T).itemsize) == 0 and N >= 1024 // np.dtype(T).itemsize
+    path = ("few_rows" if few_rows else "few_cols") + ("" if dt == "f32" else "_f64")
+    rng = np.random.default_rng(65)
+    say("matmul few columns, integers", mkn, dt)
+    A = rng.integers(-3, 4, (M, K)).astype(T); B = rng.integers(-3, 4, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul few columns, C = A B into NaNs", mkn, dt)
+    tc = on(device, np.full((M, N), np.nan, dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want).all()
+    say("matmul few columns, column major: a vector times a large matrix", mkn, dt)
+    tc = on(device, C0)
+    device.launch_matmul(False, N, K, M, on(device, B), on(device, A), tc)      # the row-major data of the transposes
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul few columns, operands inside larger buffers full of NaN", mkn, dt)
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=T)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(C0)
+    eb = np.dtype(T).itemsize
+    _lib.check(device._lib.nk_matmul(device.handle, 0 if dt == "f32" else 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + eb * pad, pb._data.ptr + eb * pad, pc._data.ptr + eb * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
+    say("matmul few columns, uniform data against the oracle", mkn, dt)
     A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
     tc = on(device, np.zeros((M, N), dtype=T))
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
