@@ -1699,7 +1699,9 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
     ("f32", (64, 48, 80), "simple"), ("f32", (512, 512, 512), "mfma_split"), ("f32", (2048, 256, 2048), "mfma"),
     ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (1000, 300, 520), "mfma_edge_split"), ("f32", (2100, 130, 2100), "mfma_edge"),
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
-    ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge")])
+    ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
+    ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
+    ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64")])
 def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mkn, path):
     """nk_matmul_set (C = A @ B, the OpenCL device's `C[n + m*N] = acc`, CLMatMul.java:50) on every kernel plan, both
     layouts: the drain starts as NaN everywhere, so a single old value read would show; the result must equal, bit for
