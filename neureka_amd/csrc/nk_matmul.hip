@@ -823,6 +823,60 @@ __global__ __launch_bounds__(256) void matmul_few_cols_kernel(int M, int K, cons
     }
 }
 
+// ---- a short inner dimension ------------------------------------------------------------------------------------
+// C[M,N] (+)= A[M,K] @ B[K,N] with K <= 16 (the gradient of a weight matrix from a small batch: a sum of K outer
+// products): the product writes C once and is bound by that stream.  A thread owns 16 bytes of columns and keeps its
+// K x 16 bytes of B in registers; a block walks FEW_RB rows of A, staged in LDS (zero-padded to KC), and writes one
+// row of its 256 x 16 bytes of columns per step -- four contiguous kilobytes.
+constexpr int FEW_RB = 32;
+template <typename T, int KC, bool OVERWRITE>
+__global__ __launch_bounds__(256) void matmul_short_inner_kernel(int M, int K, int N, int col_blocks, const T* __restrict__ A,
+                                                                 const T* __restrict__ B, T* __restrict__ C) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    typedef T Quad __attribute__((ext_vector_type(4)));
+    static_assert(KC % 4 == 0, "the staged rows of A are read four elements at a time");
+    __shared__ __attribute__((aligned(16))) T As[FEW_RB][KC];
+    const int row_block = (int)(blockIdx.x / (unsigned)col_blocks), col_block = (int)(blockIdx.x % (unsigned)col_blocks);
+    const int64_t row0 = (int64_t)row_block * FEW_RB;
+    const int64_t col0 = ((int64_t)col_block * 256 + threadIdx.x) * VEC;     // N % VEC == 0 (the host checks)
+    const bool live = col0 < N;
+    for (int i = threadIdx.x; i < FEW_RB * KC; i += 256) {
+        const int r = i / KC, k = i % KC;
+        As[r][k] = (k < K && row0 + r < M) ? A[(row0 + r) * K + k] : T(0);
+    }
+    Vec b[KC];
+#pragma unroll
+    for (int k = 0; k < KC; k++) b[k] = (live && k < K) ? *(const Vec*)(B + (int64_t)k * N + col0) : Vec(T(0));
+    __syncthreads();
+    if (!live) return;
+    const int rows = M - row0 < FEW_RB ? (int)(M - row0) : FEW_RB;
+    T* Cp = C + row0 * N + col0;
+    constexpr int RU = 4;                                               // rows in flight (their old values, when they are read)
+    for (int r0 = 0; r0 < rows; r0 += RU) {
+        Vec old[RU];
+        if (!OVERWRITE) {
+#pragma unroll
+            for (int u = 0; u < RU; u++) old[u] = *(const Vec*)(Cp + (int64_t)(r0 + u < rows ? r0 + u : rows - 1) * N);
+        }
+#pragma unroll
+        for (int u = 0; u < RU; u++) {
+            if (r0 + u < rows) {
+                Vec acc = Vec(T(0));
+#pragma unroll
+                for (int q = 0; q < KC; q += 4) {
+                    const Quad a = *(const Quad*)&As[r0 + u][q];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) acc[e] = fma_of(a[j], b[q + j][e], acc[e]);
+                }
+                *(Vec*)(Cp + (int64_t)(r0 + u) * N) = OVERWRITE ? acc : old[u] + acc;
+            }
+        }
+    }
+}
+
 // ---- f64 on the matrix cores ----------------------------------------------------------------------------------
 // 128x128 block tile, four wavefronts in a 2x2 arrangement, each owning 64x64 as 4x4 accumulators of
 // v_mfma_f64_16x16x4_f64 (register v of lane l holds row 4*v + l/16 of column l%16 of a 16x16 tile; it feeds A[row l%16]
@@ -1062,6 +1116,29 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             if (dtype == NK_F64) by_rows(double{}); else by_rows(float{});
             NK_HIP(hipGetLastError());
             set_path(dtype == NK_F64 ? "few_rows_f64" : "few_rows");
+            return NK_OK;
+        }
+    }
+    // a short inner dimension: one stream over C
+    if (bands && K <= 16 && M * K * N >= mfma_from) {
+        const int eb = dtype == NK_F64 ? 8 : 4, vec = 16 / eb;
+        if (N % vec == 0 && N >= 64 * vec && B % 16 == 0 && C % 16 == 0) {
+            const int64_t col_blocks = (N + 256 * vec - 1) / (256 * vec), row_blocks = (M + FEW_RB - 1) / FEW_RB;
+            const dim3 grid((unsigned)(col_blocks * row_blocks));
+            auto launch = [&](auto t, auto kc) {
+                using T = decltype(t);
+                constexpr int KC = decltype(kc)::value;
+                if (overwrite) hipLaunchKernelGGL((matmul_short_inner_kernel<T, KC, true>), grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, (int)col_blocks, (const T*)A, (const T*)B, (T*)C);
+                else           hipLaunchKernelGGL((matmul_short_inner_kernel<T, KC, false>), grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, (int)col_blocks, (const T*)A, (const T*)B, (T*)C);
+            };
+            auto by_depth = [&](auto t) {
+                if (K <= 4) launch(t, std::integral_constant<int, 4>{});
+                else if (K <= 8) launch(t, std::integral_constant<int, 8>{});
+                else launch(t, std::integral_constant<int, 16>{});
+            };
+            if (dtype == NK_F64) by_depth(double{}); else by_depth(float{});
+            NK_HIP(hipGetLastError());
+            set_path(dtype == NK_F64 ? "short_inner_f64" : "short_inner");
             return NK_OK;
         }
     }

@@ -1701,7 +1701,8 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
     ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
-    ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64")])
+    ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64"),
+    ("f32", (4100, 9, 4096), "short_inner"), ("f64", (4096, 16, 2050), "short_inner_f64")])
 def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mkn, path):
     """nk_matmul_set (C = A @ B, the OpenCL device's `C[n + m*N] = acc`, CLMatMul.java:50) on every kernel plan, both
     layouts: the drain starts as NaN everywhere, so a single old value read would show; the result must equal, bit for
@@ -1891,6 +1892,56 @@ def test_matmul_few_columns(device, orc, mkn, dt):
     assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
     assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
     say("matmul few columns, uniform data against the oracle", mkn, dt)
+    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
+    tc = on(device, np.zeros((M, N), dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("mkn", [(4096, 16, 4096), (4096, 1, 4096), (5000, 7, 3332), (33, 13, 40000), (70000, 3, 256), (1025, 16, 1028)])
+def test_matmul_short_inner_dimension(device, orc, mkn, dt):
+    """A sum of at most 16 outer products (the gradient of a weight matrix from a small batch, from 2^24 multiply-adds
+    on) runs as one stream over C: exact on integer data, C += A B into a non-zero C and C = A B into NaNs, column
+    major, operands parked between NaNs, uniform data against the oracle."""
+    M, K, N = mkn
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    path = "short_inner" if dt == "f32" else "short_inner_f64"
+    rng = np.random.default_rng(66)
+    say("matmul short inner dimension, integers", mkn, dt)
+    A = rng.integers(-3, 4, (M, K)).astype(T); B = rng.integers(-3, 4, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul short inner dimension, C = A B into NaNs", mkn, dt)
+    tc = on(device, np.full((M, N), np.nan, dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want).all()
+    say("matmul short inner dimension, column major", mkn, dt)
+    tc = on(device, C0)
+    device.launch_matmul(False, N, K, M, on(device, B), on(device, A), tc)      # the row-major data of the transposes
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul short inner dimension, operands inside larger buffers full of NaN", mkn, dt)
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=T)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(C0)
+    eb = np.dtype(T).itemsize
+    _lib.check(device._lib.nk_matmul(device.handle, 0 if dt == "f32" else 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + eb * pad, pb._data.ptr + eb * pad, pc._data.ptr + eb * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
+    say("matmul short inner dimension, uniform data against the oracle", mkn, dt)
     A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
     tc = on(device, np.zeros((M, N), dtype=T))
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
