@@ -640,7 +640,7 @@ __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int pa
 }
 
 // ---- a few rows times a large matrix ----------------------------------------------------------------------------
-// C[M,N] = A[M,K] @ B[K,N] with M <= 16 (a vector or a small batch times a weight matrix): the product reads B once
+// C[M,N] = A[M,K] @ B[K,N] with M <= 32 (a vector or a small batch times a weight matrix): the product reads B once
 // and is bound by that stream; a 128 x 128 tile would spend its matrix cores on rows that do not exist.  A block owns
 // 64 * (16 bytes / element) columns and one part of the k range (at most few_kp(MR) rows), whose piece of A it stages
 // in LDS; each of its four wavefronts takes a quarter of the part -- a row of B is one contiguous kilobyte for a
@@ -648,7 +648,7 @@ __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int pa
 // accumulators per column in registers (the elements of A come as 16-byte LDS reads of one address for the whole
 // wavefront), the wavefronts meet in LDS in a fixed order, and the block's partial rows go to P[part];
 // matmul_add_parts_kernel adds the parts in order.
-constexpr int few_kp(int mr) { return mr <= 4 ? 1024 : 256; }          // k rows a block stages of A: 16-32 KiB of LDS
+constexpr int few_kp(int mr) { return mr <= 4 ? 1024 : mr <= 16 ? 256 : 128; }     // k rows a block stages of A: 16-32 KiB of LDS
 __device__ __forceinline__ float fma_of(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fma_of(double a, double b, double c) { return __builtin_fma(a, b, c); }
 template <typename T, int MR>
@@ -659,7 +659,8 @@ __global__ __launch_bounds__(256) void matmul_few_rows_kernel(int M, int K, int 
     constexpr int KP = few_kp(MR);
     typedef T Vec __attribute__((ext_vector_type(VEC)));
     typedef T Quad __attribute__((ext_vector_type(4)));
-    constexpr int A_ELEMS = MR * KP, MEET_ELEMS = 3 * MR * 64 * VEC;
+    constexpr int MEET_SLOTS = MR <= 16 ? 3 : 1;                        // 32 rows: the wavefronts meet one after the other
+    constexpr int A_ELEMS = MR * KP, MEET_ELEMS = MEET_SLOTS * MR * 64 * VEC;
     __shared__ __attribute__((aligned(16))) T lds[A_ELEMS > MEET_ELEMS ? A_ELEMS : MEET_ELEMS];
     T (*As)[KP] = (T (*)[KP])lds;                                       // [MR][KP], zero past the part's end
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -685,15 +686,17 @@ __global__ __launch_bounds__(256) void matmul_few_rows_kernel(int M, int K, int 
     {
         // thread t stages columns t, t + 256, ... of the piece: independent loads along the rows of A
         const int t = threadIdx.x;
-        T av[KP / 256][MR];
+        constexpr int CPT = (KP + 255) / 256;                           // columns per thread
+        T av[CPT][MR];
 #pragma unroll
-        for (int c = 0; c < KP / 256; c++)
+        for (int c = 0; c < CPT; c++)
 #pragma unroll
             for (int m = 0; m < MR; m++) av[c][m] = A[(int64_t)(m < M ? m : M - 1) * K + k_begin + (t + 256 * c < k_count ? t + 256 * c : 0)];
 #pragma unroll
-        for (int c = 0; c < KP / 256; c++)
+        for (int c = 0; c < CPT; c++)
 #pragma unroll
-            for (int m = 0; m < MR; m++) As[m][t + 256 * c] = (m < M && t + 256 * c < k_count) ? av[c][m] : T(0);
+            for (int m = 0; m < MR; m++)
+                if (t + 256 * c < KP) As[m][t + 256 * c] = (m < M && t + 256 * c < k_count) ? av[c][m] : T(0);
     }
     __syncthreads();
     T acc[MR][VEC];
@@ -722,22 +725,37 @@ __global__ __launch_bounds__(256) void matmul_few_rows_kernel(int M, int K, int 
     }
     __syncthreads();                                                    // the staged piece of A makes room for the meeting
     T (*meet)[MR][64 * VEC] = (T (*)[MR][64 * VEC])lds;
-    if (wave > 0) {
+    if constexpr (MEET_SLOTS == 3) {
+        if (wave > 0) {
 #pragma unroll
-        for (int m = 0; m < MR; m++) *(Vec*)&meet[wave - 1][m][lane * VEC] = *(const Vec*)acc[m];
+            for (int m = 0; m < MR; m++) *(Vec*)&meet[wave - 1][m][lane * VEC] = *(const Vec*)acc[m];
+        }
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int m = 0; m < MR; m++)
+#pragma unroll
+                for (int w = 0; w < 3; w++) *(Vec*)acc[m] = *(const Vec*)acc[m] + *(const Vec*)&meet[w][m][lane * VEC];
+        }
+    } else {
+        for (int w = 1; w < 4; w++) {
+            if (wave == w) {
+#pragma unroll
+                for (int m = 0; m < MR; m++) *(Vec*)&meet[0][m][lane * VEC] = *(const Vec*)acc[m];
+            }
+            __syncthreads();
+            if (wave == 0) {
+#pragma unroll
+                for (int m = 0; m < MR; m++) *(Vec*)acc[m] = *(const Vec*)acc[m] + *(const Vec*)&meet[0][m][lane * VEC];
+            }
+            __syncthreads();
+        }
     }
-    __syncthreads();
     if (wave == 0 && live) {
         T* Pp = P + (int64_t)part * M * N + col0;
 #pragma unroll
-        for (int m = 0; m < MR; m++) {
-            if (m < M) {
-                Vec v = *(const Vec*)acc[m];
-#pragma unroll
-                for (int w = 0; w < 3; w++) v = v + *(const Vec*)&meet[w][m][lane * VEC];
-                *(Vec*)(Pp + (int64_t)m * N) = v;
-            }
-        }
+        for (int m = 0; m < MR; m++)
+            if (m < M) *(Vec*)(Pp + (int64_t)m * N) = *(const Vec*)acc[m];
     }
 }
 
@@ -1084,8 +1102,8 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         set_path(path);
         return NK_OK;
     };
-    // a few rows of A: one stream over B (from 2^24 multiply-adds on, where the sums are re-ordered anyway)
-    if (bands && M <= 16 && M * K * N >= mfma_from) {
+    // a few rows of A (at most 32): one stream over B (from 2^24 multiply-adds on, where the sums are re-ordered anyway)
+    if (bands && M <= 32 && M * K * N >= mfma_from) {
         const int eb = dtype == NK_F64 ? 8 : 4, vec = 16 / eb;
         if (N % vec == 0 && B % 16 == 0 && N >= 64 * vec) {
             const int64_t col_blocks = (N + 64 * vec - 1) / (64 * vec);
@@ -1094,7 +1112,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             if (parts > K / 32) parts = K / 32;
             if (parts < 1) parts = 1;
             int k_per_part = (int)((K + parts - 1) / parts);
-            const int mr = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+            const int mr = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : M <= 16 ? 16 : 32;
             if (k_per_part > few_kp(mr)) k_per_part = few_kp(mr);          // what a block stages of A
             parts = (K + k_per_part - 1) / k_per_part;
             void* ws = nullptr;
@@ -1111,7 +1129,8 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 else if (M <= 2) launch(t, std::integral_constant<int, 2>{});
                 else if (M <= 4) launch(t, std::integral_constant<int, 4>{});
                 else if (M <= 8) launch(t, std::integral_constant<int, 8>{});
-                else launch(t, std::integral_constant<int, 16>{});
+                else if (M <= 16) launch(t, std::integral_constant<int, 16>{});
+                else launch(t, std::integral_constant<int, 32>{});
             };
             if (dtype == NK_F64) by_rows(double{}); else by_rows(float{});
             NK_HIP(hipGetLastError());

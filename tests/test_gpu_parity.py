@@ -1616,7 +1616,7 @@ def test_matmul_split_k(device, orc, mkn, dt):
     A = rng.integers(-4, 5, (M, K)).astype(T); B = rng.integers(-4, 5, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
     tc = on(device, C0)
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
-    few_rows = lambda rows, cols: rows <= 16 and cols % (16 // np.dtype(T).itemsize) == 0 and cols >= 1024 // np.dtype(T).itemsize
+    few_rows = lambda rows, cols: rows <= 32 and cols % (16 // np.dtype(T).itemsize) == 0 and cols >= 1024 // np.dtype(T).itemsize
     vec = 16 // np.dtype(T).itemsize
     few_cols = lambda inner, cols: cols in (1, 2, 4) and inner % vec == 0
     assert (_lib.last_path().endswith("_split") or (few_rows(M, N) and _lib.last_path().startswith("few_rows"))
@@ -1702,7 +1702,8 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
     ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
     ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64"),
-    ("f32", (4100, 9, 4096), "short_inner"), ("f64", (4096, 16, 2050), "short_inner_f64")])
+    ("f32", (4100, 9, 4096), "short_inner"), ("f64", (4096, 16, 2050), "short_inner_f64"),
+    ("f32", (32, 2048, 2048), "few_rows"), ("f64", (20, 4096, 512), "few_rows_f64")])
 def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mkn, path):
     """nk_matmul_set (C = A @ B, the OpenCL device's `C[n + m*N] = acc`, CLMatMul.java:50) on every kernel plan, both
     layouts: the drain starts as NaN everywhere, so a single old value read would show; the result must equal, bit for
@@ -1799,9 +1800,10 @@ def test_matmul_256_tiles_with_edges(device, mkn):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
-@pytest.mark.parametrize("mkn", [(1, 4096, 4096), (16, 4096, 4096), (3, 5001, 4100), (8, 2049, 1024), (2, 70000, 256), (5, 33, 131072), (13, 8192, 512)])
+@pytest.mark.parametrize("mkn", [(1, 4096, 4096), (16, 4096, 4096), (3, 5001, 4100), (8, 2049, 1024), (2, 70000, 256), (5, 33, 131072), (13, 8192, 512),
+                                 (32, 4096, 4096), (17, 1000, 2052), (25, 8191, 256)])
 def test_matmul_few_rows(device, orc, mkn, dt):
-    """A vector or a small batch times a large matrix (at most 16 rows, from 2^24 multiply-adds on) runs as one stream
+    """A vector or a small batch times a large matrix (at most 32 rows, from 2^24 multiply-adds on) runs as one stream
     over the matrix with the k range in parts: exact on integer data, C += A B into a non-zero C and C = A B into NaNs,
     column major (a large matrix times a few columns), operands parked between NaNs, uniform data against the oracle."""
     M, K, N = mkn
@@ -1858,7 +1860,7 @@ def test_matmul_few_columns(device, orc, mkn, dt):
     M, K, N = mkn
     T = F[dt]
     tol = 1e-5 if dt == "f32" else 1e-12
-    few_rows = M <= 16 and N % (16 // np.dtype(T).itemsize) == 0 and N >= 1024 // np.dtype(T).itemsize
+    few_rows = M <= 32 and N % (16 // np.dtype(T).itemsize) == 0 and N >= 1024 // np.dtype(T).itemsize
     path = ("few_rows" if few_rows else "few_cols") + ("" if dt == "f32" else "_f64")
     rng = np.random.default_rng(65)
     say("matmul few columns, integers", mkn, dt)
