@@ -841,6 +841,112 @@ __global__ __launch_bounds__(256) void matmul_few_cols_kernel(int M, int K, cons
     }
 }
 
+// ---- a large matrix times a batch of columns --------------------------------------------------------------------
+// C[M,N] = A[M,K] @ B[K,N] with 5 <= N <= 16 (or 3), padded to NC = 8 or 16: still one stream over A, but a lane now
+// needs NC elements of B for each of its k's, which come from LDS.  The block's eight wavefronts (two rows of A each)
+// walk along k together; the piece of B for a trip -- 64 x (16 bytes / element) rows, NC columns -- is staged while
+// the trip before it is computed (two buffers, one barrier per trip), laid out [k % VEC][k / VEC][NC + 16 bytes] so
+// that the 64 lanes' 16-byte reads of one column group fall on different banks.
+template <typename T, int NC, bool OVERWRITE>
+__global__ __launch_bounds__(512) void matmul_some_cols_kernel(int M, int K, int N, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int R = 2, THREADS = 512;                                 // eight wavefronts of two rows: sixteen rows per block
+    constexpr int PITCH = NC + VEC;                                     // elements per (k) row in LDS
+    constexpr int STEP = 64 * VEC;                                      // k's per trip
+    constexpr int PIECES = STEP * NC / VEC / THREADS;                   // 16-byte pieces of a trip's B per thread
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    __shared__ __attribute__((aligned(16))) T Bs[2][VEC][64][PITCH];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row0 = ((int64_t)blockIdx.x * (THREADS / 64) + wave) * R;
+    const T* rows[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) rows[r] = A + (row0 + r < M ? row0 + r : M - 1) * (int64_t)K;
+    T acc[R][NC];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int n = 0; n < NC; n++) acc[r][n] = T(0);
+    // K % VEC == 0 (the host checks): a lane's VEC k's are inside the matrix or all outside
+    auto request_a = [&](Vec (&a)[R], int k0) {
+        const int k = k0 + lane * VEC;
+#pragma unroll
+        for (int r = 0; r < R; r++) a[r] = k < K ? *(const Vec*)(rows[r] + k) : Vec(T(0));
+    };
+    // piece p of a trip: VEC columns from n = (p * VEC) % NC of row k0 + (p * VEC) / NC
+    auto request_b = [&](Vec (&s)[PIECES], int k0) {
+#pragma unroll
+        for (int j = 0; j < PIECES; j++) {
+            const int p = (int)threadIdx.x + THREADS * j;
+            const int kl = p * VEC / NC, n = p * VEC % NC;
+            s[j] = Vec(T(0));
+            if (k0 + kl < K) {
+                if (N == NC) s[j] = *(const Vec*)(B + (int64_t)(k0 + kl) * NC + n);        // (B is 16-byte aligned: the host checks)
+                else {
+#pragma unroll
+                    for (int e = 0; e < VEC; e++)
+                        if (n + e < N) s[j][e] = B[(int64_t)(k0 + kl) * N + n + e];
+                }
+            }
+        }
+    };
+    auto put_b = [&](const Vec (&s)[PIECES], int buf) {
+#pragma unroll
+        for (int j = 0; j < PIECES; j++) {
+            const int p = (int)threadIdx.x + THREADS * j;
+            const int kl = p * VEC / NC, n = p * VEC % NC;
+            *(Vec*)&Bs[buf][kl % VEC][kl / VEC][n] = s[j];
+        }
+    };
+    Vec a[R], staged[PIECES];
+    request_a(a, 0);
+    request_b(staged, 0);
+    put_b(staged, 0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += STEP) {
+        Vec an[R];
+        const bool more = k0 + STEP < K;
+        if (more) { request_a(an, k0 + STEP); request_b(staged, k0 + STEP); }
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            T bv[NC];
+#pragma unroll
+            for (int q = 0; q < NC; q += VEC) *(Vec*)&bv[q] = *(const Vec*)&Bs[buf][v][lane][q];
+#pragma unroll
+            for (int n = 0; n < NC; n++)
+#pragma unroll
+                for (int r = 0; r < R; r++) acc[r][n] = fma_of(a[r][v], bv[n], acc[r][n]);
+        }
+        if (more) {
+            put_b(staged, buf ^ 1);
+#pragma unroll
+            for (int r = 0; r < R; r++) a[r] = an[r];
+        }
+        __syncthreads();
+        buf ^= 1;
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int n = 0; n < NC; n++) {
+            T v = acc[r][n];
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
+            acc[r][n] = v;
+        }
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+            if (row0 + r < M)
+#pragma unroll
+                for (int n = 0; n < NC; n++)
+                    if (n < N) {
+                        T* c = C + (row0 + r) * (int64_t)N + n;
+                        *c = OVERWRITE ? acc[r][n] : *c + acc[r][n];
+                    }
+    }
+}
+
 // ---- a short inner dimension ------------------------------------------------------------------------------------
 // C[M,N] (+)= A[M,K] @ B[K,N] with K <= 16 (the gradient of a weight matrix from a small batch: a sum of K outer
 // products): the product writes C once and is bound by that stream.  A thread owns 16 bytes of columns and keeps its
@@ -1135,6 +1241,27 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             if (dtype == NK_F64) by_rows(double{}); else by_rows(float{});
             NK_HIP(hipGetLastError());
             set_path(dtype == NK_F64 ? "few_rows_f64" : "few_rows");
+            return NK_OK;
+        }
+    }
+    // a batch of columns (3, 5 ... 16): one stream over A, B through LDS
+    if (bands && N <= 16 && N != 1 && N != 2 && N != 4 && M * K * N >= mfma_from) {
+        const int eb = dtype == NK_F64 ? 8 : 4, vec = 16 / eb;
+        if (K % vec == 0 && A % 16 == 0 && B % 16 == 0 && M >= 1024) {
+            const dim3 grid((unsigned)((M + 15) / 16));
+            auto launch = [&](auto t, auto nc) {
+                using T = decltype(t);
+                constexpr int NC = decltype(nc)::value;
+                if (overwrite) hipLaunchKernelGGL((matmul_some_cols_kernel<T, NC, true>), grid, dim3(512), 0, dev->stream, (int)M, (int)K, (int)N, (const T*)A, (const T*)B, (T*)C);
+                else           hipLaunchKernelGGL((matmul_some_cols_kernel<T, NC, false>), grid, dim3(512), 0, dev->stream, (int)M, (int)K, (int)N, (const T*)A, (const T*)B, (T*)C);
+            };
+            auto by_cols = [&](auto t) {
+                if (N <= 8) launch(t, std::integral_constant<int, 8>{});
+                else launch(t, std::integral_constant<int, 16>{});
+            };
+            if (dtype == NK_F64) by_cols(double{}); else by_cols(float{});
+            NK_HIP(hipGetLastError());
+            set_path(dtype == NK_F64 ? "some_cols_f64" : "some_cols");
             return NK_OK;
         }
     }

@@ -1952,6 +1952,56 @@ def test_matmul_short_inner_dimension(device, orc, mkn, dt):
     assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("mkn", [(4096, 4096, 16), (4096, 4096, 8), (4099, 2048, 3), (5000, 1000, 5), (1025, 4096, 11), (70001, 64, 16), (2048, 8192, 13)])
+def test_matmul_batch_of_columns(device, orc, mkn, dt):
+    """A large matrix times a batch of 3 or 5 to 16 columns (at least 1024 rows, from 2^24 multiply-adds on) runs as one
+    stream over the matrix with the columns staged in LDS: exact on integer data, C += A B into a non-zero C and C = A B
+    into NaNs, column major, operands parked between NaNs, uniform data against the oracle."""
+    M, K, N = mkn
+    T = F[dt]
+    tol = 1e-5 if dt == "f32" else 1e-12
+    path = "some_cols" if dt == "f32" else "some_cols_f64"
+    rng = np.random.default_rng(67)
+    say("matmul batch of columns, integers", mkn, dt)
+    A = rng.integers(-3, 4, (M, K)).astype(T); B = rng.integers(-3, 4, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    tc = on(device, C0)
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul batch of columns, C = A B into NaNs", mkn, dt)
+    tc = on(device, np.full((M, N), np.nan, dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want).all()
+    say("matmul batch of columns, column major", mkn, dt)
+    tc = on(device, C0)
+    device.launch_matmul(False, N, K, M, on(device, B), on(device, A), tc)      # the row-major data of the transposes
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want + C0).all()
+    say("matmul batch of columns, operands inside larger buffers full of NaN", mkn, dt)
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=T)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(C0)
+    eb = np.dtype(T).itemsize
+    _lib.check(device._lib.nk_matmul(device.handle, 0 if dt == "f32" else 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + eb * pad, pb._data.ptr + eb * pad, pc._data.ptr + eb * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
+    say("matmul batch of columns, uniform data against the oracle", mkn, dt)
+    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
+    tc = on(device, np.zeros((M, N), dtype=T))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
+    bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
 @pytest.mark.parametrize("mkn", [(3072, 1024, 3072), (3000, 800, 3100), (1280, 1024, 8192), (2700, 640, 3400)])
 def test_matmul_row_bands(device, mkn):
     """Products whose 128 x 128 tiles are a few more than whole rounds of the machine run as two row bands, the lower
