@@ -147,6 +147,51 @@ def test_matmul_into_8_gib(device):
         del want
 
 
+def test_matmul_streams_over_8_gib(device):
+    """The kernels that stream one large operand once, at the largest operand the entry point accepts (2^31 - 4096
+    elements): a matrix times a vector, a vector times a matrix, an outer product.  Small integers: every sum is exact."""
+    rng = np.random.default_rng(39)
+    L, S = 524287, 4096                                     # L * S = 2^31 - 4096
+    say("max size matmul: [L,S] @ [S,1]")
+    A = big(rng, L * S, f32, integers=(-3, 3)).reshape(L, S); x = rng.integers(-3, 4, (S, 1)).astype(f32)
+    ta, tx = on(device, A), on(device, x)
+    c = Tensor._on_device(device, f32, (L, 1))
+    device.launch_scalar_fill(c, 1.0)
+    device.launch_matmul(True, L, S, 1, ta, tx, c, accumulate=False)
+    assert _lib.last_path() == "few_cols", _lib.last_path()
+    want = A @ x
+    same(c.getData().reshape(L, 1), want, "C = A x")
+    device.launch_matmul(True, L, S, 1, ta, tx, c, accumulate=True)
+    same(c.getData().reshape(L, 1), want * 2, "C += A x")
+    free(device, tx, c)
+    say("max size matmul: [1,L] @ [L,S] (the same 8 GiB read as a matrix of S columns)")
+    y = rng.integers(-3, 4, (1, L)).astype(f32)
+    ty = on(device, y)
+    c = Tensor._on_device(device, f32, (1, S))
+    device.launch_scalar_fill(c, 1.0)
+    device.launch_matmul(True, 1, L, S, ty, ta, c, accumulate=False)
+    assert _lib.last_path() == "few_rows", _lib.last_path()
+    want = (y.astype(np.float64) @ A.astype(np.float64)).astype(f32)     # |sums| < 2^24: exact either way
+    same(c.getData().reshape(1, S), want, "C = y A")
+    device.launch_matmul(True, 1, L, S, ty, ta, c, accumulate=True)
+    same(c.getData().reshape(1, S), want * 2, "C += y A")
+    free(device, ta, ty, c)
+    del A, want
+    say("max size matmul: [L,2] @ [2,S] into 8 GiB")
+    u = rng.integers(-3, 4, (L, 2)).astype(f32); v = rng.integers(-3, 4, (2, S)).astype(f32)
+    tu, tv = on(device, u), on(device, v)
+    c = Tensor._on_device(device, f32, (L, S))
+    device.launch_scalar_fill(c, 1.0)
+    device.launch_matmul(True, L, 2, S, tu, tv, c, accumulate=False)
+    assert _lib.last_path() == "short_inner", _lib.last_path()
+    want = u @ v
+    same(c.getData().reshape(L, S), want, "C = u v")
+    device.launch_matmul(True, L, 2, S, tu, tv, c, accumulate=True)
+    want *= 2
+    same(c.getData().reshape(L, S), want, "C += u v")
+    free(device, tu, tv, c)
+
+
 def test_int32_scalar_operations_at_2_pow_31_minus_1(device, orc):
     rng = np.random.default_rng(35)
     x = big(rng, NMAX, i32, integers=(0, 1 << 30))
