@@ -22,6 +22,7 @@
 // Column-major operands are handled as the transposed row-major problem C^T = B^T A^T.
 #include "nk_internal.h"
 #include <mutex>
+#include <type_traits>
 
 namespace nk {
 
@@ -1224,9 +1225,9 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             void* ws = nullptr;
             if (int e = workspace(dev, (uint64_t)parts * M * N * eb, &ws)) return e;
             const dim3 grid((unsigned)(col_blocks * parts));
-            auto launch = [&](auto t, auto mr) {
+            auto launch = [&](auto t, auto rows_tag) {
                 using T = decltype(t);
-                hipLaunchKernelGGL((matmul_few_rows_kernel<T, decltype(mr)::value>), grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, k_per_part, (int)col_blocks,
+                hipLaunchKernelGGL((matmul_few_rows_kernel<T, decltype(rows_tag)::value>), grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, k_per_part, (int)col_blocks,
                                    (const T*)A, (const T*)B, (T*)ws);
                 hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, dev->stream, M * N, (int)parts, g.overwrite, (const T*)ws, (T*)C);
             };
