@@ -768,6 +768,8 @@ __global__ __launch_bounds__(256) void matmul_few_rows_kernel(int M, int K, int 
 template <typename T, int NC, int R, bool OVERWRITE>
 __global__ __launch_bounds__(256) void matmul_few_cols_kernel(int M, int K, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C) {
     constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int U = R == 1 ? 4 : 1;                                   // contiguous kilobytes of a row per trip (one row per wavefront: few
+                                                                        // wavefronts, each must keep more in flight)
     typedef T Vec __attribute__((ext_vector_type(VEC)));
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * R;
@@ -780,46 +782,55 @@ __global__ __launch_bounds__(256) void matmul_few_cols_kernel(int M, int K, cons
     for (int r = 0; r < R; r++)
 #pragma unroll
         for (int n = 0; n < NC; n++) acc[r][n] = T(0);
-    constexpr int STEP = 64 * VEC;                                      // k's per trip of the wavefront
+    constexpr int STEP = U * 64 * VEC;                                  // k's per trip of the wavefront
     // K % VEC == 0 (the host checks): a lane's VEC k's are inside the matrix or all outside
-    auto request = [&](Vec (&a)[R], Vec (&b)[NC], int k0) {
-        const int k = k0 + lane * VEC;
-        const int kc = k < K ? k : 0;
+    auto request = [&](Vec (&a)[U][R], Vec (&b)[U][NC], int k0) {
 #pragma unroll
-        for (int r = 0; r < R; r++) a[r] = *(const Vec*)(rows[r] + kc);
-        // elements [k .. k + VEC) x [0 .. NC) of B are VEC * NC contiguous values: NC vectors
+        for (int u = 0; u < U; u++) {
+            const int k = k0 + (u * 64 + lane) * VEC;
+            const int kc = k < K ? k : 0;
 #pragma unroll
-        for (int j = 0; j < NC; j++) b[j] = *(const Vec*)(B + (int64_t)kc * NC + j * VEC);
-        if (k >= K) {
+            for (int r = 0; r < R; r++) a[u][r] = *(const Vec*)(rows[r] + kc);
+            // elements [k .. k + VEC) x [0 .. NC) of B are VEC * NC contiguous values: NC vectors
 #pragma unroll
-            for (int r = 0; r < R; r++) a[r] = Vec(T(0));
+            for (int j = 0; j < NC; j++) b[u][j] = *(const Vec*)(B + (int64_t)kc * NC + j * VEC);
+            if (k >= K) {
 #pragma unroll
-            for (int j = 0; j < NC; j++) b[j] = Vec(T(0));
+                for (int r = 0; r < R; r++) a[u][r] = Vec(T(0));
+#pragma unroll
+                for (int j = 0; j < NC; j++) b[u][j] = Vec(T(0));
+            }
         }
     };
-    Vec a[R], b[NC];
+    Vec a[U][R], b[U][NC];
     request(a, b, 0);
     for (int k0 = 0; k0 < K; k0 += STEP) {
-        Vec an[R], bn[NC];
+        Vec an[U][R], bn[U][NC];
         if (k0 + STEP < K) request(an, bn, k0 + STEP);
-        // b as a flat run f[v * NC + n]
-        T f[VEC * NC];
 #pragma unroll
-        for (int j = 0; j < NC; j++)
+        for (int u = 0; u < U; u++) {
+            // b as a flat run f[v * NC + n]
+            T f[VEC * NC];
 #pragma unroll
-            for (int e = 0; e < VEC; e++) f[j * VEC + e] = b[j][e];
+            for (int j = 0; j < NC; j++)
 #pragma unroll
-        for (int v = 0; v < VEC; v++)
+                for (int e = 0; e < VEC; e++) f[j * VEC + e] = b[u][j][e];
 #pragma unroll
-            for (int n = 0; n < NC; n++) {
-                const T bv = f[v * NC + n];
+            for (int v = 0; v < VEC; v++)
 #pragma unroll
-                for (int r = 0; r < R; r++) acc[r][n] = fma_of(a[r][v], bv, acc[r][n]);
-            }
+                for (int n = 0; n < NC; n++) {
+                    const T bv = f[v * NC + n];
 #pragma unroll
-        for (int r = 0; r < R; r++) a[r] = an[r];
+                    for (int r = 0; r < R; r++) acc[r][n] = fma_of(a[u][r][v], bv, acc[r][n]);
+                }
+        }
 #pragma unroll
-        for (int j = 0; j < NC; j++) b[j] = bn[j];
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int r = 0; r < R; r++) a[u][r] = an[u][r];
+#pragma unroll
+            for (int j = 0; j < NC; j++) b[u][j] = bn[u][j];
+        }
     }
 #pragma unroll
     for (int r = 0; r < R; r++)
