@@ -155,7 +155,9 @@ def torch_yardstick():
     del x, y, z, out
     for name, (M, K, N), dt in (("matmul_4096_us", (4096, 4096, 4096), torch.float32), ("matmul_4000_us", (4000, 4000, 4000), torch.float32),
                                 ("matmul_3072_us", (3072, 3072, 3072), torch.float32), ("matmul_3072_f64_us", (3072, 3072, 3072), torch.float64),
-                                ("matmul_tall_skinny_us", (65536, 256, 256), torch.float32), ("matmul_4096_f64_us", (4096, 4096, 4096), torch.float64)):
+                                ("matmul_tall_skinny_us", (65536, 256, 256), torch.float32), ("matmul_4096_f64_us", (4096, 4096, 4096), torch.float64),
+                                ("matmul_matrix_vector_us", (4096, 4096, 1), torch.float32), ("matmul_batch_of_16_rows_us", (16, 4096, 4096), torch.float32),
+                                ("matmul_16_outer_products_us", (4096, 16, 4096), torch.float32), ("matmul_batch_of_16_columns_us", (4096, 4096, 16), torch.float32)):
         A = torch.randn(M, K, device=d, dtype=dt); B = torch.randn(K, N, device=d, dtype=dt); C = torch.empty(M, N, device=d, dtype=dt)
         t(name, lambda: torch.mm(A, B, out=C))
     xi = torch.randn(1, 64, 256, 256, device=d, requires_grad=True); w = torch.randn(1, 64, 5, 5, device=d, requires_grad=True)
@@ -430,6 +432,14 @@ def main():
         Cm = Tensor._on_device(dev, np.float64, (M, N))
         flops("matmul_4096_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm), f64=True)
         for t in (A, B, Cm): dev.free(t)
+        # the products of a dense layer with a small batch: each streams its large operand once (memory-bound)
+        for name, (M, K, N) in (("matmul_matrix_vector", (4096, 4096, 1)), ("matmul_batch_of_16_rows", (16, 4096, 4096)),
+                                ("matmul_16_outer_products", (4096, 16, 4096)), ("matmul_batch_of_16_columns", (4096, 4096, 16))):
+            A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
+            B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
+            Cm = Tensor._on_device(dev, f32, (M, N))
+            hbm(name, 4 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm))
+            for t in (A, B, Cm): dev.free(t)
         M = K = N = 3072
         A = Tensor.of(np.float64, (M, K), rng.uniform(-1, 1, M * K)).to(dev)
         B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)

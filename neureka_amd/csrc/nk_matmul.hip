@@ -635,8 +635,17 @@ template <typename T>
 __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int parts, int overwrite, const T* __restrict__ P, T* __restrict__ C) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    T s = P[i];
-    for (int k = 1; k < parts; k++) s = s + P[(int64_t)k * n + i];
+    // eight parts are requested before the first is added (one after the other, a thread waits out a trip to memory per part)
+    T s = T(0);
+    int k = 0;
+    for (; k + 8 <= parts; k += 8) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = P[(int64_t)(k + u) * n + i];
+#pragma unroll
+        for (int u = 0; u < 8; u++) s = (k + u == 0) ? v[u] : s + v[u];
+    }
+    for (; k < parts; k++) s = (k == 0) ? P[i] : s + P[(int64_t)k * n + i];
     C[i] = overwrite ? s : C[i] + s;
 }
 
