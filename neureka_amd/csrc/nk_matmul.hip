@@ -1190,7 +1190,8 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
     return NK_OK;
 }
 
-// `force_parts`, `bands`: how matmul_rm calls itself for the two row bands described below (callers leave them alone)
+// `force_parts`, `bands`: how matmul_rm calls itself for the two row bands described below (callers leave them alone: `bands`
+// is true for a caller's product, which may be planned as bands or take one of the streaming kernels, and false for a band)
 static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C,
                      int force_parts = 0, bool bands = true) {
     constexpr int64_t mfma_from = (int64_t)1 << 24;
