@@ -2002,6 +2002,31 @@ def test_matmul_batch_of_columns(device, orc, mkn, dt):
     assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+@pytest.mark.parametrize("mkn", [(4, 4096, 4096), (4096, 4096, 2), (4096, 8, 4096), (4096, 4096, 12), (4, 4096, 4098), (4096, 4095, 2), (4096, 8, 4097), (4096, 4094, 12)])
+def test_matmul_streaming_plans_need_aligned_operands_and_fall_back(device, mkn, dt):
+    """The streaming kernels read 16 bytes at a time: operands that start 4 or 8 bytes off such a boundary, or whose rows
+    do, take the tile kernels instead.  Whatever the plan, the integer product is exact and nothing outside C is written."""
+    M, K, N = mkn
+    T = F[dt]
+    eb = np.dtype(T).itemsize
+    rng = np.random.default_rng(68)
+    A = rng.integers(-3, 4, (M, K)).astype(T); B = rng.integers(-3, 4, (K, N)).astype(T); C0 = rng.integers(-9, 10, (M, N)).astype(T)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    for pad in (1, 64):                                                    # 1 element: 4 or 8 bytes off a 16-byte boundary
+        say("matmul streaming plans, operands", pad, "elements into their buffers", mkn, dt)
+        def parked(x):
+            host = np.full(x.size + 2 * pad, np.nan, dtype=T)
+            host[pad:pad + x.size] = x.reshape(-1)
+            return on(device, host)
+        pa, pb, pc = parked(A), parked(B), parked(C0)
+        _lib.check(device._lib.nk_matmul(device.handle, 0 if dt == "f32" else 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + eb * pad, pb._data.ptr + eb * pad, pc._data.ptr + eb * pad))
+        print("[path]", _lib.last_path(), flush=True)
+        got = pc.getData()
+        assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()
+        assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
+
+
 @pytest.mark.parametrize("mkn", [(3072, 1024, 3072), (3000, 800, 3100), (1280, 1024, 8192), (2700, 640, 3400)])
 def test_matmul_row_bands(device, mkn):
     """Products whose 128 x 128 tiles are a few more than whole rounds of the machine run as two row bands, the lower
