@@ -170,6 +170,159 @@ def torch_yardstick():
     return res
 
 
+def percentiles(xs):
+    xs = sorted(xs)
+    return {"p10": round(xs[len(xs) // 10], 4), "median": round(xs[len(xs) // 2], 4), "p90": round(xs[(len(xs) * 9) // 10], 4)}
+
+
+def wall_ms(dev, call, reps, warm=10):
+    """Host wall clock per call in steady state: `reps` calls queued back to back, one synchronisation at the end."""
+    for _ in range(warm):
+        call()
+    dev.sync()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        call()
+    dev.sync()
+    return (time.perf_counter() - t0) * 1e3 / reps
+
+
+def memory_figures(dev, C, _lib):
+    """What the memory side of an operation costs (the reference pays an allocation and a zero fill per output:
+    Broadcast.java:89-92, OpenCLDevice.java:465,478-486): nk_alloc + nk_free of the headline output from the pool and
+    from the driver, the zero fill of that output, and the host transfers."""
+    lib, h = dev._lib, C.c_uint64(dev.handle)
+    nbytes = 4 << 30
+    buf = C.c_uint64(0)
+    dev.sync(); dev.trimPool()
+    t0 = time.perf_counter()
+    _lib.check(lib.nk_alloc(h, nbytes, C.byref(buf))); _lib.check(lib.nk_free(h, buf))
+    cold = (time.perf_counter() - t0) * 1e3
+
+    def pooled():
+        lib.nk_alloc(h, nbytes, C.byref(buf)); lib.nk_free(h, buf)
+    pool_us = wall_ms(dev, pooled, 2000) * 1e3
+    _lib.check(lib.nk_alloc(h, nbytes, C.byref(buf)))
+    zero = np.zeros(1, np.float32)
+    fill = lambda: lib.nk_fill(h, buf, 0, zero.ctypes.data_as(C.c_void_p), 4, nbytes // 4)
+    for _ in range(10): fill()
+    fill_ms = event_time_ms(dev, fill, 50)
+    _lib.check(lib.nk_free(h, buf))
+    out = {"alloc_free_4GiB_from_pool_us": round(pool_us, 3), "alloc_free_4GiB_from_driver_ms": round(cold, 3),
+           "zero_fill_4GiB_ms": round(fill_ms, 4),
+           "note": "an output of an operation comes from the pool and, where the kernel writes every element, is not filled"}
+    # host transfers: pageable numpy arrays (touched beforehand), blocking calls as the reference's CL_TRUE transfers
+    for label, n in (("6MiB", 6 << 20), ("256MiB", 256 << 20)):
+        host = np.ones(n, np.uint8); back = np.ones(n, np.uint8)
+        _lib.check(lib.nk_alloc(h, n, C.byref(buf)))
+        up = lambda: lib.nk_h2d(h, buf, 0, host.ctypes.data_as(C.c_void_p), n)
+        down = lambda: lib.nk_d2h(h, back.ctypes.data_as(C.c_void_p), buf, 0, n)
+        reps = 30 if n < (64 << 20) else 6
+        for name, fn in (("h2d", up), ("d2h", down)):
+            for _ in range(3): fn()
+            ts = []
+            for _ in range(reps):
+                t0 = time.perf_counter(); fn(); ts.append((time.perf_counter() - t0) * 1e3)
+            med = sorted(ts)[len(ts) // 2]
+            out[f"{name}_{label}_ms"] = round(med, 4)
+            out[f"{name}_{label}_GBs"] = round(n / (med * 1e-3) / 1e9, 2)
+        _lib.check(lib.nk_free(h, buf))
+    out["h2d_GBs"], out["d2h_GBs"] = out["h2d_256MiB_GBs"], out["d2h_256MiB_GBs"]
+    return out
+
+
+def operation_figures(dev, rng, C, _lib, Function, Tensor, reps):
+    """Whole operations beside their kernels: `ms` = wall clock per call through HipBackend (the Python mirror of the
+    reference's call path: algorithm choice, call preparation with the drain's allocation, launch, drop of the result),
+    `abi_ms` = the same C-ABI calls without the interpreter between them (nk_alloc, the launch, nk_free -- what a JVM
+    binding issues), `kernel_ms` = the launch alone into a drain that exists.  Steady state, calls queued back to back."""
+    f32 = np.float32
+    lib, h = dev._lib, C.c_uint64(dev.handle)
+    out = {}
+
+    def record(name, mirror, abi, kernel, n_mirror=None):
+        for _ in range(10): kernel()
+        k = event_time_ms(dev, kernel, reps)
+        e = {"ms": round(wall_ms(dev, mirror, n_mirror or reps), 4)}
+        if abi: e["abi_ms"] = round(wall_ms(dev, abi, reps), 4)
+        e["kernel_ms"] = round(k, 4)
+        e["mirror_over_kernel"] = round(e["ms"] / k, 3)
+        if abi: e["abi_over_kernel"] = round(e["abi_ms"] / k, 3)
+        out[name] = e
+
+    def abi_sequence(nbytes, launch_with):
+        """nk_alloc(nbytes) -> launch_with(buffer) -> nk_free"""
+        buf = C.c_uint64(0)
+        launch = launch_with(buf)
+        def call():
+            lib.nk_alloc(h, nbytes, C.byref(buf)); launch(); lib.nk_free(h, buf)
+        return call
+
+    def cfg_of(t):
+        inline = t.ndc.asInlineArray()
+        return inline, _lib.cfg_ptr(inline)
+
+    # C2: a + b
+    s1, s2, so = (1024, 1, 512), (1, 2048, 512), (1024, 2048, 512)
+    ta = Tensor.of(f32, s1, rng.uniform(-1, 1, s1).astype(f32)).to(dev); tb = Tensor.of(f32, s2, rng.uniform(-1, 1, s2).astype(f32)).to(dev)
+    drn = Tensor._on_device(dev, f32, so, zeroed=False)
+    keep = [cfg_of(drn), cfg_of(ta), cfg_of(tb)]
+    n = drn.size
+    def c2(buf):
+        return lambda: lib.nk_broadcast(h, _lib.OP["add"], -1, _lib.F32, 3, buf, keep[0][1], ta._data.ptr, keep[1][1], tb._data.ptr, keep[2][1], n)
+    record("op_c2_add", lambda: ta + tb, abi_sequence(4 * n, c2), dev.prepared_launch("broadcast", "add", -1, drn, ta, tb))
+    dev.free(drn); dev.free(ta); dev.free(tb)
+
+    # C3: tanh(sig(a)*b+c), operation by operation (four kernels, three temporaries) and as the fused operation
+    n = 1 << 26
+    srcs = [Tensor.of(f32, (n,), rng.standard_normal(n).astype(f32)).to(dev) for _ in range(3)]
+    o = Tensor._on_device(dev, f32, (n,), zeroed=False); tmp = Tensor._on_device(dev, f32, (n,), zeroed=False)
+    fn = Function.of("tanh(sig(I[0])*I[1]+I[2])", doAD=False)
+    fused = dev.optimizedFunctionOf(fn, "chain")
+    four = [dev.prepared_launch("activation", "sig", -1, tmp, srcs[0]), dev.prepared_launch("elementwise", "multiply", -1, o, tmp, srcs[1]),
+            dev.prepared_launch("elementwise", "add", -1, tmp, o, srcs[2]), dev.prepared_launch("activation", "tanh", -1, o, tmp)]
+    record("op_c3_chain", lambda: fn(*srcs), None, lambda: [k() for k in four])
+    record("op_c3_chain_fused", lambda: fused(*srcs), None, dev.prepared_launch("fused", fused.program, fused.consts, o, srcs))
+    for t in srcs + [o, tmp]: dev.free(t)
+
+    # C4: A @ B
+    M = K = N = 4096
+    A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev); B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
+    Cm = Tensor._on_device(dev, f32, (M, N), zeroed=False)
+    def c4(buf):
+        return lambda: lib.nk_matmul_set(h, _lib.F32, _lib.ROW_MAJOR, M, K, N, A._data.ptr, B._data.ptr, buf)
+    record("op_c4_matmul", lambda: A.matMul(B), abi_sequence(4 * M * N, c4), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm))
+    for t in (A, B, Cm): dev.free(t)
+
+    # C5: x conv k, and the backward pass (both gradients) of that operation
+    x5 = Tensor.of(f32, (64, 256, 256), (rng.standard_normal(64 * 256 * 256) * 0.1).astype(f32)).to(dev)
+    k5 = Tensor.of(f32, (64, 5, 5), (rng.standard_normal(1600) * 0.1).astype(f32)).to(dev)
+    e5 = Tensor.of(f32, (1, 252, 252), rng.standard_normal(252 * 252).astype(f32)).to(dev)
+    y5 = Tensor._on_device(dev, f32, (1, 252, 252), zeroed=False)
+    dx5 = Tensor._on_device(dev, f32, (64, 256, 256), zeroed=False); dk5 = Tensor._on_device(dev, f32, (64, 5, 5), zeroed=False)
+    kc = [cfg_of(y5), cfg_of(x5), cfg_of(k5), cfg_of(e5), cfg_of(dx5), cfg_of(dk5)]
+    def c5(buf):
+        return lambda: lib.nk_convolution(h, -1, _lib.F32, 3, buf, kc[0][1], x5._data.ptr, kc[1][1], k5._data.ptr, kc[2][1], y5.size)
+    record("op_c5_conv_forward", lambda: x5.conv(k5), abi_sequence(4 * y5.size, c5), dev.prepared_launch("convolution", -1, y5, x5, k5), n_mirror=2000)
+    bx, bk = C.c_uint64(0), C.c_uint64(0)
+    def c5_backward_abi():
+        lib.nk_alloc(h, 4 * dx5.size, C.byref(bx)); lib.nk_alloc(h, 4 * dk5.size, C.byref(bk))
+        lib.nk_convolution(h, 0, _lib.F32, 3, bx, kc[4][1], k5._data.ptr, kc[2][1], e5._data.ptr, kc[3][1], dx5.size)
+        lib.nk_convolution(h, 0, _lib.F32, 3, bk, kc[5][1], x5._data.ptr, kc[1][1], e5._data.ptr, kc[3][1], dk5.size)
+        lib.nk_free(h, bx); lib.nk_free(h, bk)
+    gx, gk = dev.prepared_launch("convolution", 0, dx5, k5, e5), dev.prepared_launch("convolution", 0, dk5, x5, e5)
+    x5.setRqsGradient(True); k5.setRqsGradient(True)
+    y = x5.conv(k5)
+    def c5_backward():
+        x5.gradient = None; k5.gradient = None
+        y.backward(e5)
+    record("op_c5_backward", c5_backward, c5_backward_abi, lambda: (gx(), gk()), n_mirror=2000)
+    x5.gradient = None; k5.gradient = None
+    del y
+    for t in (x5, k5, e5, y5, dx5, dk5): dev.free(t)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -177,6 +330,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the figures of the other configurations")
+    ap.add_argument("--no-ops", action="store_true", help="skip the whole-operation and memory figures")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB device-to-device copy (a copy kernel of known size), so that a "
                          "rocprofv3 --pmc run of this command holds a reference for FETCH_SIZE / WRITE_SIZE")
@@ -486,6 +640,13 @@ def main():
         flops("conv_c5_grad_input_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", 0, dx5, k5, e5), f64=True)
         flops("conv_c5_grad_kernel_f64", 203212800, 2 * 17037632, dev.prepared_launch("convolution", 0, dk5, x5, e5), f64=True)
 
+    # ---- whole operations through the backend, allocation, fill and host transfers ---------------------------------
+    operations = memory = None
+    if not args.no_ops:
+        import ctypes
+        operations = operation_figures(dev, rng, ctypes, _lib, Function, Tensor, max(50, min(args.steps, 100)))
+        memory = memory_figures(dev, ctypes, _lib)
+
     # ---- the reference's CPU path beside the other configurations (oracle, bounded samples) -----------------------
     cpu_others = None
     if not args.no_cpu and not args.no_others:
@@ -512,6 +673,10 @@ def main():
         "cpu_baseline": cpu,
         "cpu_others": cpu_others,
         "others": others,
+        "operations": operations,
+        "memory": memory,
+        "alloc_ms": None if memory is None else round(memory["alloc_free_4GiB_from_pool_us"] * 1e-3, 6),
+        "zero_fill_ms": None if memory is None else memory["zero_fill_4GiB_ms"],
     }
     if args.yardstick:
         import subprocess

@@ -97,6 +97,18 @@ int nk_d2d(nk_dev dev, nk_buf dst, uint64_t dst_byte_off, nk_buf src, uint64_t s
 /* writes `count` copies of a 1/2/4/8-byte pattern starting at dst + dst_byte_off */
 int nk_fill(nk_dev dev, nk_buf dst, uint64_t dst_byte_off, const void* pattern, int pattern_bytes, uint64_t count);
 
+/* ---- the buffer pool behind nk_alloc / nk_free.  No counterpart in the reference, whose clCreateBuffer and
+ *      clReleaseMemObject go to the driver for every tensor (OpenCLDevice.java:465,957-962).  nk_free keeps the block, by
+ *      size class, for the next nk_alloc and neither call waits for the device: the one in-order stream orders the work of
+ *      a block's successive owners.  nk_alloc returns memory with arbitrary contents, like clCreateBuffer.  Blocks at rest
+ *      go back to the driver when they would exceed the limit (default: half of the device's memory), when the driver
+ *      runs out of memory, on nk_pool_trim and on nk_device_close. */
+int nk_pool_trim(nk_dev dev);
+int nk_pool_stats(nk_dev dev, uint64_t* resting_blocks, uint64_t* resting_bytes, uint64_t* driver_allocations, uint64_t* reuses);
+/* max_resting_bytes: the limit above.  poison != 0: every block is handed out filled with 0xFF bytes (NaN as float or
+ * double), for tests that prove that no operation relies on the contents of a fresh buffer. */
+int nk_pool_config(nk_dev dev, uint64_t max_resting_bytes, int poison);
+
 /* ---- timing on the device stream (no counterpart in the reference, which only measures wall clock
  *      around closures: src/test/java/testutility/Measure.java).  Events are recorded on the device's
  *      own stream so that they bracket exactly the launches made through this library. */

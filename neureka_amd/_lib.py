@@ -35,6 +35,9 @@ SYMBOLS = {
     "nk_device_stats": (_i32, [_u64, C.POINTER(_u64), C.POINTER(_u64)]),
     "nk_alloc": (_i32, [_u64, _u64, C.POINTER(_u64)]),
     "nk_free": (_i32, [_u64, _u64]),
+    "nk_pool_trim": (_i32, [_u64]),
+    "nk_pool_stats": (_i32, [_u64, C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64)]),
+    "nk_pool_config": (_i32, [_u64, _u64, _i32]),
     "nk_h2d": (_i32, [_u64, _u64, _u64, _p, _u64]),
     "nk_d2h": (_i32, [_u64, _p, _u64, _u64, _u64]),
     "nk_d2d": (_i32, [_u64, _u64, _u64, _u64, _u64, _u64]),

@@ -86,11 +86,15 @@ class Algorithm:
         return call
 
 
-def _new_output(device: HipDevice, dtype, shape, layout: Layout = Layout.ROW_MAJOR):
+def _new_output(device: HipDevice, dtype, shape, layout: Layout = Layout.ROW_MAJOR, overwritten: bool = False):
     """``Tensor.of(type).withShape(shape).all(0)`` + ``setIsVirtual(false)`` + ``device.store`` as the call
-    preparations do it (e.g. Broadcast.java:90-94); the zeros are produced by a device fill."""
+    preparations do it (e.g. Broadcast.java:90-94).  The reference fills the fresh drain with zeros (on the OpenCL
+    device: a clEnqueueFillBuffer of the whole output, OpenCLDevice.java:478-486) and the kernel then writes every
+    element.  ``overwritten=True`` says that the implementation the drain goes to does exactly that, so the zeros
+    would never be read and the fill (a second pass over the output, as long as the kernel itself for a broadcast)
+    is left out; the result is the same bit for bit.  Drains a kernel adds to, or writes in part, keep the fill."""
     from .tensor import Tensor
-    t = Tensor._on_device(device, dtype, shape, layout)
+    t = Tensor._on_device(device, dtype, shape, layout, zeroed=not overwritten)
     t._intermediate = True
     return t
 
@@ -108,7 +112,7 @@ class BiElementwise(Algorithm):
         if call.arity < 3:
             call = call.withAddedInputAt(0, None)
         if call.input(0) is None:
-            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape))
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape, overwritten=True))
         return call
 
 
@@ -139,7 +143,8 @@ class Broadcast(Algorithm):
         if call.input(0) is None:
             s1, s2 = call.input(1).shape, call.input(2).shape
             out_shape = tuple(s2[i] if s1[i] == 1 else s1[i] for i in range(len(s1)))
-            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, out_shape))
+            # the forward kernel writes every element; a drain of the reducing backward kernel arrives from the caller
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, out_shape, overwritten=call.derivIdx < 0))
         return call
 
 
@@ -162,7 +167,7 @@ class BiScalarBroadcast(Algorithm):
         if call.arity == 2:
             offset = 0
         src = call.input(offset)
-        out = _new_output(call.device, src.dtype, src.shape)
+        out = _new_output(call.device, src.dtype, src.shape, overwritten=True)
         if call.arity == 3:
             return call.withInputAt(0, out)
         return call.withAddedInputAt(0, out)
@@ -178,7 +183,7 @@ class ElementwiseAlgorithm(Algorithm):
         if call.arity < 2:
             call = call.withAddedInputAt(0, None)
         if call.input(0) is None:
-            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape))
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, call.input(1).shape, overwritten=True))
         return call
 
 
@@ -225,7 +230,7 @@ class ScalarBroadcast(Algorithm):
     def prepare(self, call):             # ScalarBroadcast.java:44-58: a full (actual) output of the source's shape
         ts = _two_slots(call)
         if ts[0] is None:
-            ts[0] = _new_output(call.device, ts[1].dtype, ts[1].shape)
+            ts[0] = _new_output(call.device, ts[1].dtype, ts[1].shape, overwritten=True)
         return call.withInputs(ts)
 
 
@@ -270,7 +275,7 @@ class NDConvolution(Algorithm):
         if call.input(0) is None:
             s1, s2 = call.input(1).shape, call.input(2).shape
             shp = tuple(abs(s1[i] - s2[i]) + 1 for i in range(min(len(s1), len(s2))))
-            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, shp))
+            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, shp, overwritten=True))
         return call
 
 
@@ -301,7 +306,8 @@ class MatMulAlgorithm(Algorithm):
             else:
                 lc = Layout.ROW_MAJOR
                 a, b = a.toLayoutCopy(lc), b.toLayoutCopy(lc)
-            out = _new_output(call.device, a.dtype, (a.shape[0], b.shape[1]), lc)
+            # the registered implementation writes C = A @ B (nk_matmul_set), it does not add to the drain
+            out = _new_output(call.device, a.dtype, (a.shape[0], b.shape[1]), lc, overwritten=True)
             call = call.withInputs([out, a, b])
         # _autoClone: anything that is not a dense RM or CM matrix is copied before the kernel sees it
         inputs = []
@@ -594,7 +600,7 @@ def hip_sum(call: ExecutionCall):
     """CLSum (operations/linear/internal/opencl/CLSum.java:12-62)."""
     from .tensor import Tensor
     src = call.input(0)
-    out = Tensor._on_device(call.device, src.dtype, (1,))
+    out = Tensor._on_device(call.device, src.dtype, (1,), zeroed=False)
     call.device.launch_sum(src, out)
     return out
 
@@ -620,7 +626,7 @@ def hip_dot(call: ExecutionCall):
         raise IllegalArgumentException("Input tensors must be vectors.")
     if a.shape[0] != b.shape[0]:
         raise IllegalArgumentException("Input vectors must have the same length.")
-    out = Tensor._on_device(call.device, a.dtype, (1,))
+    out = Tensor._on_device(call.device, a.dtype, (1,), zeroed=False)
     call.device.launch_dot(a, b, out)
     return out
 

@@ -8,6 +8,7 @@
 #include <string>
 #include <map>
 #include <memory>
+#include <vector>
 #include "../../include/neureka_hip.h"
 
 namespace nk {
@@ -22,8 +23,18 @@ struct Device {
     // instead of racing.  Recursive because an entry point may use another one on the same device.
     std::recursive_mutex call_mu;
     bool closed = false;                 // set by nk_device_close; a caller that waited for call_mu meanwhile gets NK_ERR_HANDLE
-    std::map<uint64_t, uint64_t> live;   // device address -> bytes
+    std::map<uint64_t, uint64_t> live;   // device address -> bytes the caller asked for (the bound every view is checked against)
     uint64_t live_bytes = 0;
+    // The buffer pool.  A block that nk_free returns keeps its device memory and waits, by size class, for the next
+    // nk_alloc of that class: every kernel and copy of this device runs on the one in-order stream, so work that is
+    // queued on a block's next owner starts after the work of its last owner, and neither call has to wait.
+    std::map<uint64_t, uint64_t> capacity;              // device address -> bytes of the block (its size class)
+    std::map<uint64_t, std::vector<void*>> pool;        // size class -> blocks at rest
+    uint64_t pool_bytes = 0, pool_limit = 0;            // bytes at rest, and the bound beyond which a freed block goes back to the driver
+    uint64_t driver_allocs = 0, pool_reuses = 0;
+    bool poison = false;                                // tests: hand out every block filled with 0xFF bytes (NaN)
+    // pinned staging chunks of the host transfers (nk_h2d / nk_d2h), allocated at the first transfer
+    struct Staging* staging = nullptr;
     // grow-only scratch for two-pass kernels (partial sums); owned by the device, freed on close
     void* workspace = nullptr;
     uint64_t workspace_bytes = 0;
@@ -36,6 +47,8 @@ void set_path(const char* name);
 std::shared_ptr<Device> device_ref(nk_dev h);   // empty (and error set) if unknown; keeps the device alive across a concurrent close
 int workspace(Device* dev, uint64_t bytes, void** out);
 int stats_static_init(Device* dev);     // resolves sum_static_scratch; the device must be current
+int memory_release_all(Device* dev);    // nk_device_close: live buffers, blocks at rest and staging chunks go back to the driver
+void launch_fill_bytes(Device* dev, void* dst, uint64_t bytes, uint64_t pattern8);   // 16-byte aligned dst, bytes a multiple of 16
 
 #define NK_HIP(expr)                                                                         \
     do {                                                                                     \

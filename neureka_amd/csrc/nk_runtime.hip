@@ -178,6 +178,17 @@ __global__ __launch_bounds__(256) void fill_wide_kernel(fill_u4* dst, fill_u4 va
     if (i < n_vec) dst[i] = value;
 }
 
+void launch_fill_bytes(Device* dev, void* dst, uint64_t bytes, uint64_t pattern8) {
+    const fill_u4 value = {(unsigned)pattern8, (unsigned)(pattern8 >> 32), (unsigned)pattern8, (unsigned)(pattern8 >> 32)};
+    const uint64_t n_vec = bytes / 16;
+    for (uint64_t done = 0; done < n_vec;) {                     // a grid holds fewer than 2^31 blocks
+        const uint64_t part = n_vec - done < ((uint64_t)1 << 38) ? n_vec - done : (uint64_t)1 << 38;
+        hipLaunchKernelGGL(fill_wide_kernel, dim3((unsigned)((part + 255) / 256)), dim3(256), 0, dev->stream,
+                           (fill_u4*)dst + done, value, part);
+        done += part;
+    }
+}
+
 }  // namespace nk
 
 using namespace nk;
@@ -209,6 +220,7 @@ int nk_device_open(int index, nk_dev* dev) {
     NK_HIP(hipSetDevice(index));
     NK_HIP(hipGetDeviceProperties(&d->props, index));
     NK_HIP(hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking));
+    d->pool_limit = d->props.totalGlobalMem / 2;         // blocks at rest may hold up to half of the device's memory
     if (int e = stats_static_init(d.get())) { (void)hipStreamDestroy(d->stream); return e; }
     std::lock_guard<std::mutex> lock(g_devices_mu);
     g_devices.push_back(std::move(d));
@@ -219,9 +231,7 @@ int nk_device_open(int index, nk_dev* dev) {
 int nk_device_close(nk_dev h) {
     NK_DEVICE(dev, h);
     NK_HIP(hipStreamSynchronize(dev->stream));
-    for (auto& kv : dev->live) (void)hipFree((void*)kv.first);
-    dev->live.clear();
-    dev->live_bytes = 0;
+    (void)memory_release_all(dev);
     if (dev->workspace) (void)hipFree(dev->workspace);
     dev->workspace = nullptr; dev->workspace_bytes = 0;
     dev->closed = true;                  // the object itself lives until the last call that holds a reference returns
@@ -250,63 +260,6 @@ int nk_device_props(nk_dev h, char* name, size_t name_cap, int* compute_units, i
     if (global_mem_bytes) *global_mem_bytes = dev->props.totalGlobalMem;
     if (lds_bytes_per_block) *lds_bytes_per_block = (int)dev->props.sharedMemPerBlock;
     if (wavefront_size) *wavefront_size = dev->props.warpSize;
-    return NK_OK;
-}
-
-int nk_device_stats(nk_dev h, uint64_t* live_buffers, uint64_t* live_bytes) {
-    NK_DEVICE(dev, h);
-    std::lock_guard<std::mutex> lock(dev->mu);
-    if (live_buffers) *live_buffers = dev->live.size();
-    if (live_bytes) *live_bytes = dev->live_bytes;
-    return NK_OK;
-}
-
-int nk_alloc(nk_dev h, uint64_t bytes, nk_buf* buf) {
-    NK_DEVICE(dev, h);
-    NK_REQUIRE(buf != nullptr, "nk_alloc: null output");
-    void* p = nullptr;
-    NK_HIP(hipMalloc(&p, bytes ? bytes : 1));
-    std::lock_guard<std::mutex> lock(dev->mu);
-    dev->live[(uint64_t)p] = bytes;
-    dev->live_bytes += bytes;
-    *buf = (uint64_t)p;
-    return NK_OK;
-}
-
-int nk_free(nk_dev h, nk_buf buf) {
-    NK_DEVICE(dev, h);
-    {
-        std::lock_guard<std::mutex> lock(dev->mu);
-        auto it = dev->live.find(buf);
-        if (it == dev->live.end())
-            return set_error(NK_ERR_HANDLE, "nk_free: 0x%llx is not a live buffer of this device (double free?)",
-                             (unsigned long long)buf);
-        dev->live_bytes -= it->second;
-        dev->live.erase(it);
-    }
-    // kernels still in flight on the device stream may use the buffer
-    NK_HIP(hipStreamSynchronize(dev->stream));
-    NK_HIP(hipFree((void*)buf));
-    return NK_OK;
-}
-
-int nk_h2d(nk_dev h, nk_buf dst, uint64_t off, const void* host, uint64_t bytes) {
-    NK_DEVICE(dev, h);
-    if (bytes == 0) return NK_OK;
-    NK_REQUIRE(host != nullptr, "nk_h2d: null host pointer");
-    if (int e = check_range(dev, "nk_h2d", dst, off, bytes)) return e;
-    NK_HIP(hipMemcpyAsync((char*)dst + off, host, bytes, hipMemcpyHostToDevice, dev->stream));
-    NK_HIP(hipStreamSynchronize(dev->stream));
-    return NK_OK;
-}
-
-int nk_d2h(nk_dev h, void* host, nk_buf src, uint64_t off, uint64_t bytes) {
-    NK_DEVICE(dev, h);
-    if (bytes == 0) return NK_OK;
-    NK_REQUIRE(host != nullptr, "nk_d2h: null host pointer");
-    if (int e = check_range(dev, "nk_d2h", src, off, bytes)) return e;
-    NK_HIP(hipMemcpyAsync(host, (const char*)src + off, bytes, hipMemcpyDeviceToHost, dev->stream));
-    NK_HIP(hipStreamSynchronize(dev->stream));
     return NK_OK;
 }
 

@@ -219,6 +219,20 @@ class HipDevice:
         _lib.check(self._lib.nk_device_stats(self.handle, C.byref(n), C.byref(b)))
         return n.value
 
+    def poolStats(self) -> dict:
+        """The buffer pool behind ``allocate`` / ``HipData.release``: blocks at rest, their bytes, allocations that
+        went to the driver and allocations served from a block at rest."""
+        v = [C.c_uint64(0) for _ in range(4)]
+        _lib.check(self._lib.nk_pool_stats(self.handle, *[C.byref(x) for x in v]))
+        return dict(zip(("resting_blocks", "resting_bytes", "driver_allocations", "reuses"), (x.value for x in v)))
+
+    def trimPool(self) -> None:
+        _lib.check(self._lib.nk_pool_trim(self.handle))
+
+    def configurePool(self, max_resting_bytes: Optional[int] = None, poison: bool = False) -> None:
+        limit = self._mem // 2 if max_resting_bytes is None else int(max_resting_bytes)
+        _lib.check(self._lib.nk_pool_config(self.handle, limit, 1 if poison else 0))
+
     # ---- data access: AbstractDevice._readAll/_readItem/_readArray/_writeItem/_writeArray ------------
     def allocate(self, dtype, size: int) -> HipData:
         """Device.allocate (OpenCLDevice.java:520-530)."""

@@ -80,7 +80,9 @@ def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: in
         other = prepared_in[1 - d]
         target_shape = prepared_in[d].shape
         def act(error: Tensor) -> Tensor:
-            zeros = Tensor._on_device(device, other.dtype, target_shape)
+            # "zeros like the target" in the reference; the gradient kernels assign every element of the drain
+            # (AbstractCPUConvolution.java:319-408 ends each element with t0_value[i] = value), so the fill is left out
+            zeros = Tensor._on_device(device, other.dtype, target_shape, zeroed=False)
             c = ExecutionCall(device, backend().getOperation("inv_convolve_mul_right"), [zeros, other, error], 0)
             c.algorithm = c.operation.algorithms[0]
             return execute_on_common_device(c, lambda cc: execute_device_algorithm(cc))
@@ -120,7 +122,9 @@ def _ad_action(op_id: str, alg, call: ExecutionCall, inputs: List[Tensor], d: in
         # (zeros like operand d, zeros like the other operand, error)
         tgt, other = prepared_in[d], prepared_in[1 - d]
         def act(error: Tensor) -> Tensor:
-            to_be_derived = Tensor._on_device(device, tgt.dtype, tgt.shape)
+            # the reducing kernel assigns every element of the drain (CPUBroadcast.java:209-257); the "derivative"
+            # operand is an input of the kernel and keeps its zeros
+            to_be_derived = Tensor._on_device(device, tgt.dtype, tgt.shape, zeroed=False)
             derivative = Tensor._on_device(device, other.dtype, other.shape)
             c = ExecutionCall(device, call.operation, [to_be_derived, derivative, error], d, alg)
             return execute_on_common_device(c, lambda cc: execute_device_algorithm(cc))
@@ -492,7 +496,7 @@ class OptimizedFunction:
                 operands = [srcs[v] if kind == "input" else temps[v] for kind, v in leaves]
                 if not operands:                     # a constant expression: the drain's shape comes from the first input
                     operands = [srcs[0]]
-                out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape)
+                out = Tensor._on_device(self.device, srcs[0].dtype, srcs[0].shape, zeroed=False)
                 self.device.launch_fused(program, consts, out, operands)
                 temps[k] = out
         finally:

@@ -61,10 +61,12 @@ class Tensor:
         return Tensor(dt, NDConfiguration.ofShape(shape), np.ascontiguousarray(arr))
 
     @staticmethod
-    def _on_device(device: HipDevice, dtype, shape, layout: Layout = Layout.ROW_MAJOR) -> "Tensor":
+    def _on_device(device: HipDevice, dtype, shape, layout: Layout = Layout.ROW_MAJOR, zeroed: bool = True) -> "Tensor":
+        """A dense tensor in device memory.  ``zeroed=False`` leaves the buffer as the pool hands it out: for drains
+        whose every element the next kernel writes, where the zeros of ``all(0)`` would never be read."""
         ndc = NDConfiguration.ofShape(shape, layout)
         t = Tensor(dtype, ndc, None)
-        data = device.allocateFromOne(dtype, ndc.size, 0)
+        data = device.allocateFromOne(dtype, ndc.size, 0) if zeroed else device.allocate(dtype, ndc.size)
         t._set_data(data, device)
         device._register(t)
         return t
@@ -217,7 +219,7 @@ class Tensor:
         if self.ndc.getLayout() is layout:
             return self
         dev = self._require_device()
-        out = Tensor._on_device(dev, self.dtype, self.shape, layout)
+        out = Tensor._on_device(dev, self.dtype, self.shape, layout, zeroed=False)
         dev.launch_activation("idy", -1, out, self)
         return out
 

@@ -32,6 +32,9 @@ def device():
     """The HipDevice under test; a missing library or GPU is an error for a gpu test, never a skip to CPU."""
     from neureka_amd import HipDevice
     dev = HipDevice.get(0)
+    # every buffer is handed out filled with 0xFF bytes (NaN) for the whole session: an operation that relied on the
+    # contents of a fresh drain, which the pool does not define, would show in its own test
+    dev.configurePool(poison=True)
     print(f"[device] {dev!r}", flush=True)
     yield dev
 
