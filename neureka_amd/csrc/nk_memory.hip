@@ -121,7 +121,10 @@ private:
         for (;;) {
             uint64_t gen = ticket_.load(std::memory_order_acquire) >> 32;
             if (gen == seen) {
-                for (int spin = 0; spin < 4000 && gen == seen; spin++) {       // a transfer is a train of jobs: stay close
+                // a transfer is a train of jobs some tens of microseconds apart: stay awake for about a millisecond after
+                // the last one (waking a sleeper costs more than the copy of a piece)
+                const uint64_t until = __builtin_ia32_rdtsc() + 3000000;
+                while (gen == seen && __builtin_ia32_rdtsc() < until) {
                     __builtin_ia32_pause();
                     gen = ticket_.load(std::memory_order_acquire) >> 32;
                 }
@@ -140,44 +143,46 @@ private:
 };
 
 // ---- the staging ring ------------------------------------------------------------------------------------
-// CHUNKS pinned chunks per device; a transfer is cut into pieces that go through them in turn, so that the copy
-// between pageable memory and one chunk runs while the DMA engine moves another.
+// CHUNKS pinned chunks per device, each with a copy stream of its own ("lane"); a transfer is cut into pieces that go
+// through them in turn, so that the copy between pageable memory and one chunk runs while the DMA engine moves
+// another.  The host waits for a piece with hipStreamSynchronize on its lane.  Measured on 256 MiB with 4 MiB pieces:
+// 53.7 GB/s in both directions this way, 45.7 (up) and 47.2 (down) with all pieces on the device's own stream and an
+// event per chunk; the DMA engine alone moves 57.  The lanes start behind the work already queued on the device's
+// stream (an event it records, which they wait for on the device), and a transfer returns when its last piece has
+// arrived, so the next launch on the device's stream comes after it.
 struct Staging {
     static constexpr int CHUNKS = 4;
     static constexpr uint64_t CHUNK_BYTES = 4 << 20;
     void* chunk[CHUNKS] = {};
-    hipEvent_t moved[CHUNKS] = {};
+    hipStream_t lane[CHUNKS] = {};
+    hipEvent_t queued = nullptr;
 };
+
+static void staging_destroy(Staging* s) {
+    for (int k = 0; k < Staging::CHUNKS; k++) {
+        if (s->chunk[k]) (void)hipHostFree(s->chunk[k]);
+        if (s->lane[k]) (void)hipStreamDestroy(s->lane[k]);
+    }
+    if (s->queued) (void)hipEventDestroy(s->queued);
+    delete s;
+}
 
 static int staging_of(Device* dev, Staging** out) {
     if (!dev->staging) {
         auto* s = new Staging();
-        for (int i = 0; i < Staging::CHUNKS; i++) {
-            hipError_t e = hipHostMalloc(&s->chunk[i], Staging::CHUNK_BYTES, hipHostMallocDefault);
-            if (e == hipSuccess) e = hipEventCreateWithFlags(&s->moved[i], hipEventDisableTiming);
-            if (e != hipSuccess) {
-                for (int k = 0; k <= i; k++) {
-                    if (s->chunk[k]) (void)hipHostFree(s->chunk[k]);
-                    if (s->moved[k]) (void)hipEventDestroy(s->moved[k]);
-                }
-                delete s;
-                return set_error((int)e, "pinned staging memory for host transfers: %s", hipGetErrorString(e));
-            }
+        hipError_t e = hipEventCreateWithFlags(&s->queued, hipEventDisableTiming);
+        for (int i = 0; i < Staging::CHUNKS && e == hipSuccess; i++) {
+            e = hipHostMalloc(&s->chunk[i], Staging::CHUNK_BYTES, hipHostMallocDefault);
+            if (e == hipSuccess) e = hipStreamCreateWithFlags(&s->lane[i], hipStreamNonBlocking);
+        }
+        if (e != hipSuccess) {
+            staging_destroy(s);
+            return set_error((int)e, "pinned staging memory for host transfers: %s", hipGetErrorString(e));
         }
         dev->staging = s;
     }
     *out = dev->staging;
     return NK_OK;
-}
-
-// Waits for a piece to have left (or reached) its chunk by polling: hipEventSynchronize sleeps and comes back tens of
-// microseconds late, which is more than the copy of a small piece takes.
-static hipError_t wait_moved(hipEvent_t e) {
-    for (;;) {
-        const hipError_t s = hipEventQuery(e);
-        if (s != hipErrorNotReady) return s;
-        __builtin_ia32_pause();
-    }
 }
 
 // Pieces of a transfer: small transfers are cut finer, so that they too overlap copy and DMA.
@@ -186,6 +191,13 @@ static uint64_t piece_bytes(uint64_t bytes) {
     if (piece < (256 << 10)) piece = 256 << 10;
     if (piece > Staging::CHUNK_BYTES) piece = Staging::CHUNK_BYTES;
     return piece;
+}
+
+// The first `lanes` lanes wait, on the device, for everything queued on the device's stream so far.
+static int lanes_follow_stream(Device* dev, Staging* s, uint64_t lanes) {
+    NK_HIP(hipEventRecord(s->queued, dev->stream));
+    for (uint64_t k = 0; k < lanes && k < (uint64_t)Staging::CHUNKS; k++) NK_HIP(hipStreamWaitEvent(s->lane[k], s->queued, 0));
+    return NK_OK;
 }
 
 int memory_release_all(Device* dev) {
@@ -198,11 +210,7 @@ int memory_release_all(Device* dev) {
     dev->pool.clear();
     dev->pool_bytes = 0;
     if (dev->staging) {
-        for (int i = 0; i < Staging::CHUNKS; i++) {
-            (void)hipHostFree(dev->staging->chunk[i]);
-            (void)hipEventDestroy(dev->staging->moved[i]);
-        }
-        delete dev->staging;
+        staging_destroy(dev->staging);
         dev->staging = nullptr;
     }
     return NK_OK;
@@ -322,19 +330,18 @@ int nk_h2d(nk_dev h, nk_buf dst, uint64_t off, const void* host, uint64_t bytes)
     if (int e = staging_of(dev, &s)) return e;
     CopyCrew& crew = CopyCrew::get();
     const uint64_t piece = piece_bytes(bytes);
+    const uint64_t pieces = (bytes + piece - 1) / piece;
+    if (int e = lanes_follow_stream(dev, s, pieces)) return e;
     char* to = (char*)dst + off;
     const char* from = (const char*)host;
-    int i = 0;
-    for (uint64_t done = 0; done < bytes; i++) {
-        const int slot = i % Staging::CHUNKS;
-        const uint64_t len = bytes - done < piece ? bytes - done : piece;
-        if (i >= Staging::CHUNKS) NK_HIP(wait_moved(s->moved[slot]));     // the chunk's last piece has left it
-        crew.copy(s->chunk[slot], from + done, len);
-        NK_HIP(hipMemcpyAsync(to + done, s->chunk[slot], len, hipMemcpyHostToDevice, dev->stream));
-        NK_HIP(hipEventRecord(s->moved[slot], dev->stream));
-        done += len;
+    for (uint64_t k = 0; k < pieces; k++) {
+        const int slot = (int)(k % Staging::CHUNKS);
+        const uint64_t len = k + 1 < pieces ? piece : bytes - k * piece;
+        if (k >= (uint64_t)Staging::CHUNKS) NK_HIP(hipStreamSynchronize(s->lane[slot]));     // the chunk's last piece has left it
+        crew.copy(s->chunk[slot], from + k * piece, len);
+        NK_HIP(hipMemcpyAsync(to + k * piece, s->chunk[slot], len, hipMemcpyHostToDevice, s->lane[slot]));
     }
-    NK_HIP(hipStreamSynchronize(dev->stream));
+    for (uint64_t k = 0; k < pieces && k < (uint64_t)Staging::CHUNKS; k++) NK_HIP(hipStreamSynchronize(s->lane[k]));
     return NK_OK;
 }
 
@@ -348,18 +355,18 @@ int nk_d2h(nk_dev h, void* host, nk_buf src, uint64_t off, uint64_t bytes) {
     CopyCrew& crew = CopyCrew::get();
     const uint64_t piece = piece_bytes(bytes);
     const uint64_t pieces = (bytes + piece - 1) / piece;
+    if (int e = lanes_follow_stream(dev, s, pieces)) return e;
     const char* from = (const char*)src + off;
     char* to = (char*)host;
     auto length = [&](uint64_t k) { return k + 1 < pieces ? piece : bytes - k * piece; };
-    auto fetch = [&](uint64_t k) -> hipError_t {
+    auto fetch = [&](uint64_t k) {
         const int slot = (int)(k % Staging::CHUNKS);
-        hipError_t e = hipMemcpyAsync(s->chunk[slot], from + k * piece, length(k), hipMemcpyDeviceToHost, dev->stream);
-        return e != hipSuccess ? e : hipEventRecord(s->moved[slot], dev->stream);
+        return hipMemcpyAsync(s->chunk[slot], from + k * piece, length(k), hipMemcpyDeviceToHost, s->lane[slot]);
     };
     for (uint64_t k = 0; k < pieces && k < (uint64_t)Staging::CHUNKS; k++) NK_HIP(fetch(k));
     for (uint64_t k = 0; k < pieces; k++) {
         const int slot = (int)(k % Staging::CHUNKS);
-        NK_HIP(wait_moved(s->moved[slot]));
+        NK_HIP(hipStreamSynchronize(s->lane[slot]));
         crew.copy(to + k * piece, s->chunk[slot], length(k));
         if (k + Staging::CHUNKS < pieces) NK_HIP(fetch(k + Staging::CHUNKS));
     }
