@@ -371,48 +371,56 @@ __device__ __forceinline__ void write_cols(double* dst, const double* v) {
     *((f64x2u*)dst + 1) = hi;
 }
 
-// window[0 .. CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[CX .. CX+EXTRA-1] with the
-// columns to the right of them
+// The KW - 1 columns a lane's window needs beyond its own CX come from its neighbour's registers; only the lane at
+// the end of the wavefront has no neighbour and loads them.  That load carries no branch: every other lane asks for
+// a column far outside the row, which the range check of the row's descriptor answers with 0 without a memory
+// access.  A branch around it (`if (lane == 63)`) makes the compiler close the divergent block with a wait for the
+// load -- one exposed round trip per window row, twelve in a row for a 5 x 5 tap gradient.  Without it the edge
+// loads leave with the row's other loads and one wait covers them all.
+constexpr int FAR_COL = 0x3FFFFFF8;         // times 4 or 8 bytes, and the next 32 bytes, still beyond every row (a plane, so a row, stays below 2 GiB: checked on the host)
+
+// window[0 .. CX-1] holds (or will hold) the lane's own columns x .. x+CX-1 of `row`; requests, in the last lane,
+// the columns to the right of them into window[CX .. CX+EXTRA-1] (0 in every other lane)
 template <int EXTRA, typename T>
-__device__ __forceinline__ void extend_right(T (&window)[CX + EXTRA], BufRsrc row, int x, int lane) {
+__device__ __forceinline__ void request_right(T (&window)[CX + EXTRA], BufRsrc row, int x, int lane) {
     static_assert(EXTRA <= 2 * CX, "at most two further pieces of CX columns");
+    T a[CX];
+    load_cols(row, lane == 63 ? x + CX : FAR_COL, a);
 #pragma unroll
-    for (int e = CX; e < CX + EXTRA; e++) window[e] = T(0);
-    if (lane == 63) {
-        T a[CX];
-        load_cols(row, x + CX, a);
+    for (int e = 0; e < CX && e < EXTRA; e++) window[CX + e] = a[e];
+    if (EXTRA > CX) {
+        T b[CX];
+        load_cols(row, lane == 63 ? x + 2 * CX : FAR_COL, b);
 #pragma unroll
-        for (int e = 0; e < CX && e < EXTRA; e++) window[CX + e] = a[e];
-        if (EXTRA > CX) {
-            T b[CX];
-            load_cols(row, x + 2 * CX, b);
-#pragma unroll
-            for (int e = CX; e < EXTRA; e++) window[CX + e] = b[e - CX];
-        }
+        for (int e = CX; e < EXTRA; e++) window[CX + e] = b[e - CX];
     }
+}
+// after request_right and the loads of the own columns: every lane but the last takes its neighbour's columns
+template <int EXTRA, typename T>
+__device__ __forceinline__ void shift_in_right(T (&window)[CX + EXTRA]) {
 #pragma unroll
     for (int e = CX; e < CX + EXTRA; e++) window[e] = from_next_lane(window[e], window[e - CX]);
 }
 
-// window[EXTRA .. EXTRA+CX-1] holds the lane's own columns x .. x+CX-1 of `row`; fills window[0 .. EXTRA-1] with
-// the columns x-EXTRA .. x-1 to the left of them (columns left of the row start read as zero)
+// window[EXTRA .. EXTRA+CX-1] holds (or will hold) the lane's own columns x .. x+CX-1 of `row`; requests, in the
+// first lane, the columns x-EXTRA .. x-1 to the left of them into window[0 .. EXTRA-1] (columns left of the row
+// start read as zero, as does every other lane)
 template <int EXTRA, typename T>
-__device__ __forceinline__ void extend_left(T (&window)[CX + EXTRA], BufRsrc row, int x, int lane) {
+__device__ __forceinline__ void request_left(T (&window)[CX + EXTRA], BufRsrc row, int x, int lane) {
     static_assert(EXTRA <= 2 * CX, "at most two further pieces of CX columns");
+    T a[CX];
+    load_cols(row, lane == 0 ? x - CX : FAR_COL, a);                       // columns x-4 .. x-1
 #pragma unroll
-    for (int i = 0; i < EXTRA; i++) window[i] = T(0);
-    if (lane == 0) {
-        T a[CX];
-        load_cols(row, x - CX, a);                                         // columns x-4 .. x-1
+    for (int e = 0; e < CX; e++) if (EXTRA - CX + e >= 0) window[EXTRA - CX + e] = a[e];
+    if (EXTRA > CX) {
+        T b[CX];
+        load_cols(row, lane == 0 ? x - 2 * CX : FAR_COL, b);               // columns x-8 .. x-5
 #pragma unroll
-        for (int e = 0; e < CX; e++) if (EXTRA - CX + e >= 0) window[EXTRA - CX + e] = a[e];
-        if (EXTRA > CX) {
-            T b[CX];
-            load_cols(row, x - 2 * CX, b);                                 // columns x-8 .. x-5
-#pragma unroll
-            for (int e = 0; e < CX; e++) if (EXTRA - 2 * CX + e >= 0) window[EXTRA - 2 * CX + e] = b[e];
-        }
+        for (int e = 0; e < CX; e++) if (EXTRA - 2 * CX + e >= 0) window[EXTRA - 2 * CX + e] = b[e];
     }
+}
+template <int EXTRA, typename T>
+__device__ __forceinline__ void shift_in_left(T (&window)[CX + EXTRA]) {
 #pragma unroll
     for (int i = EXTRA - 1; i >= 0; i--) window[i] = from_prev_lane(window[i], window[i + CX]);
 }
@@ -445,11 +453,12 @@ __global__ __launch_bounds__(NW * 64) void conv_chan_fwd(ChanArgs g, const T* __
         const T* plane = in + (int64_t)c * g.H * g.W;
         T v[R + KH - 1][CX + KW - 1];
 #pragma unroll
-        for (int yy = 0; yy < R + KH - 1; yy++)                  // all loads of the window first: one wait for the lot
+        for (int yy = 0; yy < R + KH - 1; yy++) {                // all loads of the window first: one wait for the lot
             load_cols(row_of(plane, y0 + yy, g.W, y0 + yy < g.H), x, v[yy]);
+            request_right<KW - 1>(v[yy], row_of(plane, y0 + yy, g.W, y0 + yy < g.H), x, lane);
+        }
 #pragma unroll
-        for (int yy = 0; yy < R + KH - 1; yy++)
-            extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, g.W, y0 + yy < g.H), x, lane);
+        for (int yy = 0; yy < R + KH - 1; yy++) shift_in_right<KW - 1>(v[yy]);
 #pragma unroll
         for (int yy = 0; yy < R + KH - 1; yy++)
 #pragma unroll
@@ -596,12 +605,10 @@ __global__ __launch_bounds__(256) void conv_chan_dx(ChanArgs g, const T* __restr
     for (int rr = 0; rr < R + KH - 1; rr++) {
         const int ey = y0 - (KH - 1) + rr;
         load_cols(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), x, &E[rr][KW - 1]);
+        request_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), x, lane);
     }
 #pragma unroll
-    for (int rr = 0; rr < R + KH - 1; rr++) {
-        const int ey = y0 - (KH - 1) + rr;
-        extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), x, lane);
-    }
+    for (int rr = 0; rr < R + KH - 1; rr++) shift_in_left<KW - 1>(E[rr]);
     const bool stores = x < g.W;
     const bool vec_ok = x + CX <= g.W;
     for (int c = c0; c < c1; c++) {
@@ -667,12 +674,10 @@ __global__ __launch_bounds__(256) void conv_chan_dk(ChanArgs g, int S, int nstri
         for (int rr = 0; rr < R + KH - 1; rr++) {
             const int ey = y - (KH - 1) + rr;
             load_cols(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, &E[rr][KW - 1]);
+            request_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, lane);
         }
 #pragma unroll
-        for (int rr = 0; rr < R + KH - 1; rr++) {
-            const int ey = y - (KH - 1) + rr;
-            extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, lane);
-        }
+        for (int rr = 0; rr < R + KH - 1; rr++) shift_in_left<KW - 1>(E[rr]);
 #pragma unroll
         for (int r = 0; r < R; r++)
 #pragma unroll
@@ -730,12 +735,10 @@ __global__ __launch_bounds__(NW * 64) void conv_chan_dk_joined(ChanArgs g, int S
         for (int rr = 0; rr < R + KH - 1; rr++) {
             const int ey = y - (KH - 1) + rr;
             load_cols(row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, &E[rr][KW - 1]);
+            request_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, lane);
         }
 #pragma unroll
-        for (int rr = 0; rr < R + KH - 1; rr++) {
-            const int ey = y - (KH - 1) + rr;
-            extend_left<KW - 1>(E[rr], row_of(err, ey, g.OW, ey >= 0 && ey < g.OH), xx, lane);
-        }
+        for (int rr = 0; rr < R + KH - 1; rr++) shift_in_left<KW - 1>(E[rr]);
 #pragma unroll
         for (int r = 0; r < R; r++)
 #pragma unroll
@@ -805,10 +808,12 @@ __global__ __launch_bounds__(256) void conv2d_window(int H, int W, const T* __re
         for (int kx = 0; kx < KW; kx++) wt[ky][kx] = taps[ky * KW + kx];
     T v[R + KH - 1][CX + KW - 1];
 #pragma unroll
-    for (int yy = 0; yy < R + KH - 1; yy++) load_cols(row_of(plane, y0 + yy, W, y0 + yy < H), x, v[yy]);
+    for (int yy = 0; yy < R + KH - 1; yy++) {
+        load_cols(row_of(plane, y0 + yy, W, y0 + yy < H), x, v[yy]);
+        request_right<KW - 1>(v[yy], row_of(plane, y0 + yy, W, y0 + yy < H), x, lane);
+    }
 #pragma unroll
-    for (int yy = 0; yy < R + KH - 1; yy++)
-        extend_right<KW - 1>(v[yy], row_of(plane, y0 + yy, W, y0 + yy < H), x, lane);
+    for (int yy = 0; yy < R + KH - 1; yy++) shift_in_right<KW - 1>(v[yy]);
     T acc[R][CX];
 #pragma unroll
     for (int r = 0; r < R; r++)
