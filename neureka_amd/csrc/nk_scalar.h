@@ -48,6 +48,67 @@ template <> struct Num<double> {
     static __device__ __forceinline__ double fma(double a, double b, double c) { return ::fma(a, b, c); }
 };
 
+// a * b + c with c a wave-uniform constant that stays in scalar registers.  Written as one instruction because the
+// compiler, left to itself, copies every double constant of a polynomial into a pair of vector registers right before
+// its multiply-add (two more vector instructions per step; hoisting them out of the interpreter's loop instead costs
+// the registers of every table entry at once).
+__device__ __forceinline__ double fma_const(double a, double b, double c) {
+    double d;
+    asm("v_fma_f64 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "s"(c));
+    return d;
+}
+// exp(z) in double, sized for its callers here: the float kernels that must repeat the reference's double evaluation
+// ((float) f((double) x), fun/api/CPUFun.java:7-9) because its formulas cancel -- 1 - tanh^2, s (1 - s) -- so that the
+// float they round to has to be the reference's float.  z = n ln2 + r with |r| <= ln2 / 2 (ln2 in two parts, n ln2_hi
+// exact), e^r as the Taylor polynomial of degree 13 (the next term is below 2^-57), the power of two applied by ldexp:
+// two dozen full-rate instructions, no table, no branch, an error of about one unit in the last place.  The device
+// library's exp spends three times that on cases these callers never reach.
+__device__ __forceinline__ double exp_reduced(double z) {        // -746 <= z <= 710, or NaN
+    const double n = __builtin_rint(z * 1.4426950408889634074);
+    double r = __builtin_fma(n, -6.93147180369123816490e-01, z);
+    r = __builtin_fma(n, -1.90821492927058770002e-10, r);
+    double p = fma_const(r, 1.6059043836821613e-10, 2.08767569878681e-09);      // 1/13!, 1/12!, ... 1/2!
+    p = fma_const(p, r, 2.505210838544172e-08);
+    p = fma_const(p, r, 2.755731922398589e-07);
+    p = fma_const(p, r, 2.7557319223985893e-06);
+    p = fma_const(p, r, 2.48015873015873e-05);
+    p = fma_const(p, r, 1.984126984126984e-04);
+    p = fma_const(p, r, 1.3888888888888889e-03);
+    p = fma_const(p, r, 8.333333333333333e-03);
+    p = fma_const(p, r, 4.1666666666666664e-02);
+    p = fma_const(p, r, 1.6666666666666666e-01);
+    p = __builtin_fma(p, r, 0.5);
+    p = __builtin_fma(p, r, 1.0);
+    p = __builtin_fma(p, r, 1.0);
+    return __builtin_ldexp(p, (int)n);
+}
+// Arguments are clamped to where the result saturates (0 below -746, infinity above 710); a NaN fails both
+// comparisons, passes through and comes out as NaN.
+__device__ __forceinline__ double exp_fast(double z) {
+    z = z < -746.0 ? -746.0 : z;
+    z = z > 710.0 ? 710.0 : z;
+    return exp_reduced(z);
+}
+// 1 / d for 1 <= d < 1e305 (the 1 + e^z of a logistic function): the hardware estimate and two Newton steps, a
+// relative error of about 2^-52, a third of the instructions of the correctly rounded division.
+__device__ __forceinline__ double rcp_fast(double d) {
+    double r = __builtin_amdgcn_rcp(d);
+    r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
+    r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
+    return r;
+}
+// 1 / (1 + e^(k x)) for a float x, |k| <= 2.  The argument stays within +-700, so that 1 + e^z stays finite for the
+// Newton steps (the answers there, 1 and 1e-304, are the saturated ones), by one float instruction on x instead of two
+// double comparisons with their selects.  That clamp turns a NaN into a number: the caller puts the NaN back into its
+// float result (`x != x ? x : result`).
+template <int K1000>                                              // k in thousandths: -2000, -1000, -1702
+__device__ __forceinline__ double logistic_of_float(float x) {
+    constexpr double k = K1000 / 1000.0;
+    constexpr float bound = (float)(700.0 / (K1000 < 0 ? -k : k));
+    const float xc = __builtin_amdgcn_fmed3f(x, -bound, bound);
+    return rcp_fast(1.0 + exp_reduced((double)xc * k));
+}
+
 // Binary operators whose f32 form the reference evaluates through double (Math.pow / Math.log take and return
 // double; implementations/elementwise/CPUBiElementWisePower.java:11,21,31, CPUBiElementWiseDivision.java:31,
 // CPUBiElementWiseModulo.java:31 and the broadcast twins): the intermediates neither overflow nor underflow
@@ -69,11 +130,39 @@ __device__ __forceinline__ double pow_ref(double a, double b) { return pow_doubl
 // f32: the reference evaluates (float) Math.pow((double) a, (double) b).  The float routine of the device library works
 // on a two-float logarithm and is within 2 ulp of that (far inside 1e-5) at a fraction of the cost of the double one
 // (f32 tensors: 0.6 -> 3 TB/s); Math.pow's special cases that C answers differently are taken out first, as above.
+// A positive finite base and a finite exponent -- the bulk of every tensor -- take a path of about forty full-rate
+// instructions: log2 of the base in double (a = m 2^e with m in [sqrt(1/2), sqrt 2), log m = 2 atanh((m - 1)/(m + 1)) as
+// the odd series up to s^13, relative error 2^-34), the product with the exponent in double, and 2^p as the hardware's
+// float exp2 of the fractional part scaled by ldexp.  The error of the product enters the result as p 2^-34 ln 2 <
+// 1e-8 and the float conversion of the fraction as 2e-8, so the result is within 3 ulp of (float) Math.pow.
+__device__ __forceinline__ float pow_positive(float a, float b) {
+    int e;
+    double m = __builtin_frexp((double)a, &e);                   // [0.5, 1)
+    const bool low = m < 0.70710678118654752;
+    m = low ? m + m : m;
+    e = low ? e - 1 : e;
+    const double s = (m - 1.0) * rcp_fast(m + 1.0);
+    const double s2 = s * s;
+    double q = fma_const(s2, 0.076923076923076927, 0.090909090909090912);       // 1/13, 1/11, ... 1/3
+    q = fma_const(q, s2, 0.1111111111111111);
+    q = fma_const(q, s2, 0.14285714285714285);
+    q = fma_const(q, s2, 0.2);
+    q = fma_const(q, s2, 0.33333333333333331);
+    const double ln_m_half = __builtin_fma(s * s2, q, s);        // atanh(s)
+    const double l2 = __builtin_fma(ln_m_half, 2.8853900817779268, (double)e);     // e + 2 atanh(s) log2(e)
+    double p = (double)b * l2;
+    p = p < -320.0 ? -320.0 : p;                                 // 2^-320 and 2^320 are 0 and infinity in float
+    p = p > 320.0 ? 320.0 : p;
+    const double n = __builtin_rint(p);
+    const float r = __builtin_amdgcn_exp2f((float)(p - n));
+    return __builtin_ldexpf(r, (int)n);
+}
 __device__ __forceinline__ float pow_ref(float a, float b) {
     if (b == 2.0f) return a * a;
     if (b == 1.0f) return a;
     if (b == 0.0f) return 1.0f;
     if (b != b || (::fabsf(a) == 1.0f && ::isinf(b))) return __builtin_nanf("");
+    if (a > 0.0f && a < __builtin_inff() && ::fabsf(b) < __builtin_inff()) return pow_positive(a, b);
     return ::powf(a, b);
 }
 __device__ __forceinline__ double dpow_da_ref(double a, double b) { return b * pow_double(a, b - 1); }
@@ -223,11 +312,11 @@ template <typename T> __device__ __forceinline__ T selu_ref(T x) {
 template <typename T> __device__ __forceinline__ T dselu_ref(T x) {
     const double ALPHA = 1.6732632423543772848170429916717, SCALE = 1.0507009873554804934193349852946;
     if (x > T(0)) return T(SCALE);
-    if (x <= T(0)) return T(SCALE * ALPHA * ::exp((double)x));
+    if (x <= T(0)) return T(SCALE * ALPHA * exp_fast((double)x));
     return T(NAN);
 }
-__device__ __forceinline__ float tanh_f32_via_f64(float x) { return (float)(2.0 / (1.0 + ::exp((double)(-x * 2.0f))) - 1.0); }
-__device__ __forceinline__ float sig_f32_via_f64(float x) { return (float)(1.0 / (1.0 + ::exp(-(double)x))); }
+__device__ __forceinline__ float tanh_f32_via_f64(float x) { const float t = (float)(2.0 * logistic_of_float<-2000>(x) - 1.0); return x != x ? x : t; }
+__device__ __forceinline__ float sig_f32_via_f64(float x) { const float s = (float)logistic_of_float<-1000>(x); return x != x ? x : s; }
 // log(1 + exp(x)) (fun/ScalarSoftplus.java:18-22).  The reference evaluates exactly this in double, and for x below
 // about -16 the sum 1 + exp(x) keeps only a few bits of exp(x): its result is exp(x) rounded to a multiple of
 // 2^-52 (0 or 2.2e-16 around x = -36.7).  Parity is with those results, so the f32 kernel repeats the double
@@ -272,7 +361,7 @@ template <typename T> __device__ __forceinline__ T dfast_gaus_ref(T x) {
 }
 template <typename T> __device__ __forceinline__ T dgelu_ref(T x) {      // fun/ScalarGeLU.java
     T sig;
-    if constexpr (sizeof(T) == 8) sig = sigmoid(x * 1.702); else sig = (float)(1.0 / (1.0 + ::exp(-((double)x * 1.702))));
+    if constexpr (sizeof(T) == 8) sig = sigmoid(x * 1.702); else { sig = (float)logistic_of_float<-1702>(x); sig = x != x ? x : sig; }
     T ds = sig * (T(1) - sig);
     return sig + ds * x * T(1.702);
 }
@@ -341,7 +430,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
         case NK_FUN_COS: NK_EACH(T(-::sin((double)x)));
         case NK_FUN_GASU: NK_EACH(dgasu_ref(x));
         case NK_FUN_GATU: NK_EACH(dgatu_ref(x));
-        case NK_FUN_GAUS: NK_EACH(T(-2.0 * (double)x * ::exp(-((double)x * (double)x))));
+        case NK_FUN_GAUS: NK_EACH(T(-2.0 * (double)x * exp_fast(-((double)x * (double)x))));
         case NK_FUN_FAST_GAUS: NK_EACH(dfast_gaus_ref(x));
         case NK_FUN_GELU: NK_EACH(dgelu_ref(x));
         case NK_FUN_IDY: NK_EACH(T(1));
@@ -352,11 +441,11 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
         case NK_FUN_SIG: NK_EACH(dsig_ref(x));
         case NK_FUN_SILU: NK_EACH(dsilu_ref(x));
         case NK_FUN_SIN: NK_EACH(T(::cos((double)x)));
-        case NK_FUN_SOFTPLUS: NK_EACH(T(1.0 / (1.0 + ::exp(-(double)x))));
+        case NK_FUN_SOFTPLUS: NK_EACH(sig_as_ref(x));                   // the logistic function itself
         case NK_FUN_SOFTSIGN: NK_EACH(T(1) / (T(2) * N::abs(x) + x * x + T(1)));
         case NK_FUN_TANH: NK_EACH(dtanh_as_ref(x));
         case NK_FUN_FAST_TANH: NK_EACH(dfast_tanh_ref(x));
-        case NK_FUN_EXP: NK_EACH(T(::exp((double)x)));
+        case NK_FUN_EXP: NK_EACH(T(exp_fast((double)x)));
         case NK_FUN_LOG10: NK_EACH(T(1) / (x * T(2.302585092994046)));   // x * ln(10)
         case NK_FUN_SQRT: NK_EACH(T(0.5) * inv_sqrt_ref(x));
         case NK_FUN_CBRT: NK_EACH(T(1) / (T(3) * T(::pow((double)x, (double)(T(2.0) / T(3.0))))));

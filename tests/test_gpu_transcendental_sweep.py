@@ -73,6 +73,54 @@ def test_f32_exp_based_activations_dense_sweep(device, orc):
     print("[sweep] summary: " + "; ".join(f"{n_} d={d} {r:.2e}" for n_, d, r, _ in report), flush=True)
 
 
+def test_f32_power_dense_sweep(device, orc):
+    """a ** b in f32 against the oracle's (float) pow((double) a, (double) b) (CPUBiElementWisePower.java:11-31), every
+    element within 1e-5 relative: bases over every binade from 2^-40 to 2^40 with exponents in [-12, 12], bases within
+    2^-12 of 1 with exponents up to 3e6 (the logarithm's relative accuracy decides), results that overflow, underflow
+    or land in the subnormals, negative bases with whole and fractional exponents, zeros and infinities."""
+    rng = np.random.default_rng(2027)
+    A, B = [], []
+    for e in range(-40, 41):
+        A.append((np.float32(2.0) ** e * (1 + rng.random(100_000, dtype=np.float32))).astype(np.float32))
+        B.append(rng.uniform(-12, 12, 100_000).astype(np.float32))
+    near = (1 + rng.uniform(-2.0 ** -12, 2.0 ** -12, 1 << 21)).astype(np.float32)
+    A.append(near); B.append((rng.uniform(-3e6, 3e6, near.size)).astype(np.float32))
+    big = rng.uniform(0.5, 2.0, 1 << 20).astype(np.float32)
+    A.append(big); B.append(rng.uniform(-260, 260, big.size).astype(np.float32))         # results from 2^-260 to 2^260
+    neg = -rng.uniform(0.1, 10, 1 << 18).astype(np.float32)
+    A.append(neg); B.append(np.rint(rng.uniform(-9, 9, neg.size)).astype(np.float32))
+    A.append(neg); B.append(rng.uniform(-3, 3, neg.size).astype(np.float32))
+    sp = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, 3.4e38, 0.5, 2.0, 3.0, -2.0, 1e-38], dtype=np.float32)
+    A.append(np.repeat(sp, sp.size)); B.append(np.tile(sp, sp.size))
+    a, b = np.concatenate(A), np.concatenate(B)
+    n = a.size
+    assert n >= 11_000_000
+    print(f"[case] sweep power over {n} pairs", flush=True)
+    cfg = orc.dense_cfg([n])
+    ta, tb = Tensor.of(np.float32, (n,), a).to(device), Tensor.of(np.float32, (n,), b).to(device)
+    out = Tensor._on_device(device, np.float32, (n,))
+    device.launch_elementwise("power", -1, out, ta, tb)
+    got = out.getData().astype(np.float64)
+    with np.errstate(all="ignore"):
+        want = orc.elementwise("power", -1, np.zeros(n, dtype=np.float32), cfg, a, cfg, b, cfg, workers=16).astype(np.float64)
+    assert (np.isnan(got) == np.isnan(want)).all(), "NaNs differ"
+    inf = np.isinf(want)
+    assert (got[inf] == want[inf]).all(), "infinities differ"
+    finite = np.isfinite(want)
+    err = np.abs(got[finite] - want[finite])
+    # results below the smallest normal float are rounded to a multiple of 2^-149 by both sides: one such step apart at most
+    bound = RTOL * np.abs(want[finite]) + 1.5e-45
+    bad = err > bound
+    with np.errstate(all="ignore"):
+        rel = np.where(np.abs(want[finite]) > 1.2e-38, err / np.abs(want[finite]), 0.0)
+    w = int(np.argmax(rel))
+    print(f"[sweep] power worst relative error {rel[w]:.3e} at a = {a[finite][w]!r}, b = {b[finite][w]!r}", flush=True)
+    assert not bad.any(), (f"{int(bad.sum())} of {n} outside rtol {RTOL}; first at a = {a[finite][np.flatnonzero(bad)[0]]!r}, "
+                           f"b = {b[finite][np.flatnonzero(bad)[0]]!r}: got {got[finite][np.flatnonzero(bad)[0]]!r}, want {want[finite][np.flatnonzero(bad)[0]]!r}")
+    for t in (ta, tb, out):
+        device.free(t)
+
+
 def test_config3_single_kernels_full_size(device, orc):
     """The four kernels the reference runs for tanh(sig(a)*b+c), each alone on 2^26 elements: sig and tanh within 1e-5
     of the oracle element by element, multiply and add bit for bit."""
