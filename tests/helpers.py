@@ -75,3 +75,44 @@ def fill_it(n, seed, dtype):
     """InternalMatMulTest._fillIt32/_fillIt64: data[i] = ((i + (32**seed) % 11) % 11) - 5"""
     h = (32 ** seed) % 11
     return (((np.arange(n, dtype=np.int64) + h) % 11) - 5).astype(dtype)
+
+
+VIEW_DTYPES = {"f64": np.float64, "f32": np.float32, "i32": np.int32, "i8": np.int8}
+
+
+def view_row_parent(row):
+    """The parent array of a row of tests/golden/reference_views.json: listed values, a Groovy range cycled through the
+    shape (Tensor.of(shape, -3d..7d)) or a cycle of given values (andFill)."""
+    dt = VIEW_DTYPES[row["dtype"]]
+    size = int(np.prod(row["shape"]))
+    if "values" in row:
+        src = np.asarray(row["values"], dtype=dt)
+    elif "range" in row:
+        src = np.arange(row["range"][0], row["range"][1] + 1).astype(dt)
+    else:
+        src = np.asarray(row["cycle"], dtype=dt)
+    return np.resize(src, size).astype(dt)
+
+
+def apply_view_chain(t, chain):
+    """Applies the chain of a row of tests/golden/reference_views.json to a Tensor."""
+    for step in chain:
+        kind = step[0]
+        if kind == "slice":
+            keys = []
+            for r in step[1:]:
+                if isinstance(r, int):
+                    keys.append(r)
+                else:
+                    first, last = r[0], r[1]
+                    keys.append(slice(first, last + 1, r[2] if len(r) > 2 else 1))
+            t = t.getAt(*keys)
+        elif kind == "all":
+            t = t.getAt(*[slice(None)] * t.rank)
+        elif kind == "T":
+            t = t.T()
+        elif kind == "pad_front":
+            t = t.permute(-1, *range(t.rank))
+        else:
+            raise ValueError(kind)
+    return t

@@ -110,14 +110,23 @@ def _chain_oracle(orc, bases, cfgs, shape, workers=16):
     return want, m
 
 
-def _check_chain(got, want, m, c_view):
-    """The outer tanh is held to rtol 1e-5 on the output.  What reaches it is p = fl(m + c) with m = sig(a) * b: the inner
-    sigmoid may differ from the reference's by 1e-5 relative, i.e. m by 1e-5 |m|, and where m + c cancels that is no
-    longer small against p -- so 1e-5 |m| enters absolutely (tanh' <= 1), plus one rounding of the sum, 2^-23 (|m| + |c|).
-    Each of the four kernels alone is held to 1e-5 on its own output at this size in test_gpu_transcendental_sweep.py."""
-    bound = RTOL[np.dtype(f32)] * (np.abs(m) + np.abs(want)) + 2.0 ** -23 * (np.abs(m) + np.abs(c_view)) + 1e-10
-    bad = np.abs(got - want) > bound
-    assert not bad.any(), f"{bad.sum()} of {bad.size} outside the bound; first {np.flatnonzero(bad)[:3]}"
+def _check_chain(got, want, m, c_view, what=""):
+    """Where the sum p = m + c (m = sig(a) * b) does not cancel, |m + c| >= (|m| + |c|) / 2, the fused output is held to
+    plain rtol 1e-5 of the oracle's.  Elsewhere the inner sigmoid's own tolerance is no longer small against p: it may differ
+    from the reference's by 1e-5 relative, i.e. m by 1e-5 |m|, which enters p absolutely (tanh' <= 1), plus one rounding
+    of the sum, 2^-23 (|m| + |c|) -- the propagated bound.  The share of elements under each bound is printed."""
+    c_view = c_view.astype(np.float64); m64 = m.astype(np.float64)
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    plain = np.abs(m64 + c_view) >= 0.5 * (np.abs(m64) + np.abs(c_view))
+    bad = plain & (err > RTOL[np.dtype(f32)] * np.abs(want) + 1e-30)
+    assert not bad.any(), f"{what}: {bad.sum()} of {plain.sum()} elements without cancellation outside plain rtol 1e-5; first {np.flatnonzero(bad)[:3]}"
+    bound = RTOL[np.dtype(f32)] * (np.abs(m64) + np.abs(want)) + 2.0 ** -23 * (np.abs(m64) + np.abs(c_view)) + 1e-10
+    bad = ~plain & (err > bound)
+    assert not bad.any(), f"{what}: {bad.sum()} of {(~plain).sum()} cancelling elements outside the propagated bound; first {np.flatnonzero(bad)[:3]}"
+    with np.errstate(all="ignore"):
+        worst = float(np.max(np.where(plain & (np.abs(want) > 0), err / np.abs(want), 0.0)))
+    print(f"[chain] {what}: {plain.mean() * 100:.2f} % of {plain.size} elements under plain rtol 1e-5 (worst relative error {worst:.2e}), "
+          f"{(~plain).mean() * 100:.2f} % under the propagated bound", flush=True)
 
 
 def test_config3_chain_contiguous_permuted_sliced(device, orc):
@@ -136,7 +145,7 @@ def test_config3_chain_contiguous_permuted_sliced(device, orc):
     assert _lib.last_path() == "rows_vec"
     cfg1 = orc.dense_cfg([n])
     want, m = _chain_oracle(orc, bases, [cfg1] * 3, (n,))
-    _check_chain(got.items, want, m, bases[2])
+    _check_chain(got.items, want, m, bases[2], "contiguous")
     free(device, got)
     say("C3 permuted")
     views = [t.T() for t in tens]
@@ -144,7 +153,7 @@ def test_config3_chain_contiguous_permuted_sliced(device, orc):
     assert _lib.last_path() == "tile_transpose" and got.shape == (4096, 16384)
     cfgs = [v.ndc.asInlineArray() for v in views]
     want, m = _chain_oracle(orc, bases, cfgs, (4096, 16384))
-    _check_chain(got.items, want, m, bases[2].reshape(16384, 4096).T.reshape(-1))
+    _check_chain(got.items, want, m, bases[2].reshape(16384, 4096).T.reshape(-1), "permuted")
     unf = fn(*views)                                                     # the reference's four launches
     assert_bits(unf.items, got.items, "fused vs unfused, permuted")
     free(device, got, unf, *views, *tens)
@@ -157,12 +166,12 @@ def test_config3_chain_contiguous_permuted_sliced(device, orc):
     assert _lib.last_path() == "rows_vec" and got.shape == (4096, 8192)
     cfgs = [v.ndc.asInlineArray() for v in views]
     want, m = _chain_oracle(orc, parents, cfgs, (4096, 8192))
-    _check_chain(got.items, want, m, parents[2].reshape(8192, 16384)[::2, 1:8193].reshape(-1))
+    _check_chain(got.items, want, m, parents[2].reshape(8192, 16384)[::2, 1:8193].reshape(-1), "sliced")
     free(device, got, *views, *ptens)
 
 
 @pytest.mark.parametrize("mkn", [(4096, 4096, 4096), (65536, 256, 256)])
-def test_config4_matmul_full_size(device, mkn):
+def test_config4_matmul_full_size(device, orc, mkn):
     M, K, N = mkn
     rng = np.random.default_rng(4)
     say("C4 matmul integer data (exact)", mkn)
@@ -184,6 +193,13 @@ def test_config4_matmul_full_size(device, mkn):
     ref = A[rows].astype(np.float64) @ B.astype(np.float64)
     bound = 1e-5 * (np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64))
     assert (np.abs(got[rows] - ref) <= bound).all()
+    # the whole product against the oracle's GEMM (GEMM.threaded_F32_MxN_RM restated, float sums in k order), every
+    # element within 1e-5 sum_k |a_ik| |b_kj| (that sum from a float product: the bound needs two digits, not seven)
+    want = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=16).reshape(M, N)
+    whole = 1e-5 * (np.abs(A) @ np.abs(B)).astype(np.float64)
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    assert (err <= whole).all(), f"{(err > whole).sum()} of {M * N} elements outside the norm-wise bound"
+    print(f"[matmul] {mkn}: worst |delta| / sum|a||b| over all {M * N} elements {float(np.max(err / whole)) * 1e-5:.2e}", flush=True)
     # linearity: (2A) B == 2 (A B) bit for bit (scaling by a power of two is exact)
     c2 = on(device, 2 * A).matMul(tb)
     assert_bits(c2.items, 2 * c.items, "linearity")

@@ -390,6 +390,51 @@ def test_slices_of_transposed_tensors_walk_in_row_major_order(device, orc):
     assert_bits(tp.getData().reshape(parent.shape), want, "convolution drain view")
 
 
+def test_reference_view_chains_on_device(device, orc, golden):
+    """tests/golden/reference_views.json on the device: every view chain of Tensor_Slice_Permute_Spec and Tensor_Slicing_Spec
+    (slices, transposed slices -- whose descriptors carry the column-major unravel table --, padded reshapes) read
+    through the kernels: a copy through the view (the identity activation), the view times two (scalarization), the view
+    as drain of an assignment, and the product of the two transposed blocks through the operator x."""
+    import json
+    import os
+    from helpers import apply_view_chain, view_row_parent
+    data = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_views.json")))
+    views = []
+    for row in data["rows"]:
+        say("view chain", row["name"])
+        parent = view_row_parent(row)
+        t = Tensor.of(parent.dtype, row["shape"], parent).to(device)
+        v = apply_view_chain(t, row["chain"])
+        views.append(v)
+        assert list(v.shape) == row["want_shape"]
+        want = np.asarray(row["want"], dtype=parent.dtype)
+        if np.issubdtype(parent.dtype, np.integer):
+            out = Tensor._on_device(device, parent.dtype, v.shape)
+            device.launch_scalarization("multiply", -1, out, v, 2)
+            assert out.getData().tolist() == (want * 2).tolist(), row["name"]
+            continue
+        assert_bits(v.deepCopy().getData(), want, row["name"] + ": copy through the view")
+        out = Tensor._on_device(device, parent.dtype, v.shape)
+        device.launch_scalarization("multiply", -1, out, v, 2.0)
+        assert_bits(out.getData(), want * 2, row["name"] + ": twice the view")
+        dense = orc.dense_cfg(list(v.shape))
+        assert_bits(orc.activation("idy", -1, np.zeros(v.size, dtype=parent.dtype), dense, parent, cfg(v)), want, row["name"] + ": oracle")
+        # the view as a drain: only its elements change
+        fresh = Tensor.of(parent.dtype, v.shape, -want).to(device)
+        v.assign(fresh)
+        after = parent.copy()
+        orc.activation("idy", -1, after, cfg(v), -want, dense)
+        assert_bits(t.getData(), after, row["name"] + ": assignment into the view")
+        assert_bits(v.items, -want, row["name"] + ": items after the assignment")
+    for prod in data["products"]:
+        say("product of transposed slices")
+        rows = data["rows"]
+        ta = apply_view_chain(on(device, view_row_parent(rows[prod["left_row"]]).reshape(rows[prod["left_row"]]["shape"])), rows[prod["left_row"]]["chain"])
+        tb = apply_view_chain(on(device, view_row_parent(rows[prod["right_row"]]).reshape(rows[prod["right_row"]]["shape"])), rows[prod["right_row"]]["chain"])
+        c = ta.permute(0, 1, -1).conv(tb.permute(-1, 0, 1))          # convDot: [2,2,1] x [1,2,2] (Tensor.java:1949-1966)
+        assert list(c.shape) == prod["want_shape"] and c.items.tolist() == prod["want"]
+
+
 def test_exotic_descriptor_falls_back_to_the_literal_formula(device, orc):
     """A descriptor whose indicesMap is not the row-major table of its shape cannot be reduced to
     base + strides: the literal kernel evaluates NDConfiguration.indexOfIndex (the formula the 20 rows of

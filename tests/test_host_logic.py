@@ -96,6 +96,20 @@ def test_slice_then_transpose_matches_reference_string():
     assert physical_indices(v.ndc).tolist()[:4] == [12, 20, 28, 13]
 
 
+def test_view_chains_give_the_items_the_reference_prints():
+    """tests/golden/reference_views.json: slices, transposed slices and padded reshapes of Tensor_Slice_Permute_Spec and
+    Tensor_Slicing_Spec; the descriptors this package builds must address exactly the items those specifications print."""
+    import json
+    from helpers import apply_view_chain, view_row_parent
+    rows = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_views.json")))["rows"]
+    assert len(rows) >= 12
+    for row in rows:
+        parent = view_row_parent(row)
+        v = apply_view_chain(Tensor.of(parent.dtype, row["shape"], parent), row["chain"])
+        assert list(v.shape) == row["want_shape"], row["name"]
+        assert v.items.tolist() == row["want"], row["name"]
+
+
 def test_parser_and_fused_lowering():
     f = Function.of("tanh(sig(I[0])*I[1]+I[2])")
     assert repr(f.root) == "tanh(((sig(I[0]) multiply I[1]) add I[2]))"
