@@ -270,6 +270,21 @@ def test_integration_text_binds_every_export_and_every_registration_row():
     for method in ("_readAll", "_readItem", "_readArray", "_writeItem", "_writeArray", "_swap", "_sizeOccupiedBy", "_actualize",
                    "_virtualize", "_dataTypeOf", "allocateFromOne", "allocateFromAll", "optimizedOperationOf", "dispose"):
         assert re.search(rf"\b{method}\(", text), f"HipDevice.{method} is missing from the binding text"
+    # the Java sources exist as files, and the document prints them as they are
+    blocks = dict(re.findall(r"`(java/[A-Za-z/]+\.java)`\n\n```java\n(.*?)\n```", text, re.S))
+    files = []
+    for folder, _, names in os.walk(os.path.join(ROOT, "java")):
+        files += [os.path.relpath(os.path.join(folder, n), ROOT) for n in names if n.endswith(".java")]
+    assert sorted(files) == sorted(blocks) and len(files) == 5, (sorted(files), sorted(blocks))
+    for path in files:
+        assert open(os.path.join(ROOT, path)).read().rstrip("\n") == blocks[path], f"{path} differs from its block in INTEGRATION.md"
+    compiler = open(os.path.join(ROOT, "java", "neureka", "devices", "hip", "HipFunctionCompiler.java")).read()
+    for piece in ("static Node treeOf(", "static Node derivativeOf(", "static List<Stage> plan(", "private static Stage lower(", "public Operation optimize()",
+                  "setImplementationFor( HipDevice.class"):
+        assert piece in compiler, piece
+    # the limits and op-codes of the Java planner are the header's
+    for name, value in re.findall(r"#define (NK_FUSE_MAX_[A-Z]+) (\d+)", header):
+        assert re.search(rf"\b{name[len('NK_FUSE_'):]} = {value}\b", compiler), name
 
 
 def test_assignment_parses_and_nests_to_the_right():
