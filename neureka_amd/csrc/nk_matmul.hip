@@ -295,6 +295,116 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     }
 }
 
+// Products with fewer 128 x 128 tiles than compute units (1024^3 has 64) but enough 64 x 64 tiles to give every unit
+// one: 64 x 64 block tiles over the whole k range, four wavefronts in a 2 x 2 arrangement with one 32 x 32 accumulator
+// each.  One launch and no partial tiles, where cutting the k range of the large tiles into parts pays for a second launch
+// and for writing and re-reading the parts.  A lane feeds a multiply-add two registers per 64 cycles, so a single
+// wavefront per SIMD keeps its matrix core busy through the loads and the one barrier of a k-slice.  Whole tiles only
+// (M % 64 == 0, N % 64 == 0, K % 32 == 0, 16-byte aligned operands); the result leaves straight from the accumulators
+// (32 lanes cover 128 contiguous bytes of a row of C).
+namespace t64 {
+constexpr int TM = 64, TN = 64;
+constexpr int A_P = BK + 4, B_P = TN + 4;                    // floats; rows stay 16-byte aligned
+constexpr int STAGE = TM * A_P + BK * B_P;                   // one k-slice of A and of B
+constexpr int LDS_FLOATS = 3 * STAGE;
+}
+template <bool OVERWRITE>
+__global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C) {
+    using namespace t64;
+    __shared__ __attribute__((aligned(16))) float lds[t64::LDS_FLOATS];
+    int tm, tn;
+    tile_of_block(g, (int)blockIdx.x, tm, tn);
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    const int l32 = lane & 31, h = lane >> 5;
+    const float* Ag = A + (int64_t)tm * TM * g.K;
+    const float* Bg = B + (int64_t)tn * TN;
+    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 * i
+    const int b_row = tid >> 4, b_col = (tid & 15) * 4;     // rows b_row + 16 * i
+    f32x4 ra[2], rb[2];
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 16 * i) * g.N + b_col);
+        }
+    };
+    auto store_lds = [&](int stage) {
+        float* as = lds + stage * STAGE;
+        float* bs = as + TM * A_P;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            *(f32x4*)(&as[(a_row + 32 * i) * A_P + a_col]) = ra[i];
+            *(f32x4*)(&bs[(b_row + 16 * i) * B_P + b_col]) = rb[i];
+        }
+    };
+    // operands of one depth-8 chunk: lane half h owns k = 8c + 4h .. + 3; the four multiply-adds pair (k, k + 4) in both operands
+    struct Chunk { f32x4 a; float b[4]; };
+    auto read_chunk = [&](Chunk& f, int stage, int c) {
+        const float* as = lds + stage * STAGE;
+        const float* bs = as + TM * A_P;
+        f.a = *(const f32x4*)(&as[(wm + l32) * A_P + 8 * c + 4 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; t++) f.b[t] = bs[(8 * c + 4 * h + t) * B_P + wn + l32];
+    };
+    // two accumulators that take the multiply-adds of a pair of chunks in turn: no multiply-add waits for the one before it
+    f32x16 acc0, acc1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) { acc0[v] = 0.0f; acc1[v] = 0.0f; }
+    auto mma = [&](const Chunk& even, const Chunk& odd) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(even.a[t], even.b[t], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(odd.a[t], odd.b[t], acc1, 0, 0, 0);
+        }
+    };
+    // Three stages of LDS.  During slice kt the block writes slice kt + 2 and reads slice kt; the barrier at the end of a
+    // slice publishes the writes one slice before anybody reads them, so the first chunks of slice kt + 1 are read before
+    // that barrier, behind the last multiply-adds of slice kt: no wavefront starts a slice by waiting for LDS, which the
+    // single wavefront of a SIMD could hide behind nothing.
+    const int nk = g.K / BK;
+    auto clamped = [&](int slice) { return (slice < nk ? slice : nk - 1) * BK; };     // past the end: the last slice again, read by nobody
+    load_global(0);
+    store_lds(0);
+    load_global(clamped(1));
+    store_lds(1);
+    load_global(clamped(2));                                  // slice 2 waits in the staging registers
+    __syncthreads();
+    Chunk f0, f1, f2, f3;
+    read_chunk(f0, 0, 0);
+    read_chunk(f1, 0, 1);
+    int cur = 0;                                              // stage of slice kt
+    // The body is branch-free, and the write of slice kt + 2 with the request of slice kt + 3 sits in the middle of the
+    // slice: at its top the wait for the request would hold up the multiply-adds behind it.  (Measured and not kept:
+    // requests four slices ahead in four register sets behind a barrier that waits for LDS only -- 74 against 78 TFLOP/s
+    // at 1024^3; the compiler's placement of the LDS reads between the multiply-adds decides, not the distance.)
+    for (int kt = 0; kt < nk; kt++) {
+        const int next = cur == 2 ? 0 : cur + 1, write = next == 2 ? 0 : next + 1;      // stages of slices kt + 1, kt + 2
+        read_chunk(f2, cur, 2);
+        read_chunk(f3, cur, 3);
+        mma(f0, f1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_lds(write);
+        load_global(clamped(kt + 3));
+        read_chunk(f0, next, 0);
+        read_chunk(f1, next, 1);
+        mma(f2, f3);
+        __syncthreads();
+        cur = next;
+    }
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = acc0[v] + acc1[v];
+    // accumulator v sits at row 8 * (v / 4) + 4 * h + v % 4, column l32 of the wavefront's 32 x 32 tile
+    float* Cg = C + (int64_t)(tm * TM + wm) * g.N + tn * TN + wn + l32;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        float* p = Cg + (int64_t)(8 * (v >> 2) + 4 * h + (v & 3)) * g.N;
+        *p = OVERWRITE ? acc[v] : *p + acc[v];
+    }
+}
+
 // Whole tiles, no split, more tiles than resident blocks: blocks that stay.  A block walks the tiles blockIdx.x,
 // + gridDim.x, ... and the software pipeline over the k-slices runs on across them: the first slice of the next
 // tile is fetched and written to the free LDS buffer during the last slice of the current one, so only the
@@ -1163,7 +1273,18 @@ static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes, in
     const int slices = (g.K + slice - 1) / slice;
     g.splits = 1; g.split_slices = slices;
     if (force_parts < 2 && (tiles >= cus || slices < 8)) return 1;
-    int parts = force_parts >= 2 ? force_parts : (2 * cus + tiles - 1) / tiles;
+    int parts = force_parts;
+    if (parts < 2) {
+        // The number of parts that finishes first, in units of one k-slice of one tile on a compute unit of its own: the
+        // blocks a unit ends up with times the slices of a part, plus what a part costs in writing and re-reading its
+        // partial tiles.  (Measured: 1024^3, 64 tiles: 4 parts 69 TFLOP/s, 8 parts 59; 1536^3, 144 tiles: 3 parts 89, 4 parts 81.)
+        int most = slices / 4 < 64 ? slices / 4 : 64;
+        double best = 0;
+        for (int p = 2; p <= most; p++) {
+            const double cost = (double)(((int64_t)tiles * p + cus - 1) / cus) * ((slices + p - 1) / p) + 0.75 * p;
+            if (parts < 2 || cost < best) { parts = p; best = cost; }
+        }
+    }
     if (parts > slices / 4) parts = slices / 4;
     if (parts > 64) parts = 64;
     // bound the workspace: parts * M * N elements
@@ -1246,6 +1367,9 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             if (k_per_part > few_kp(mr)) k_per_part = few_kp(mr);          // what a block stages of A
             parts = (K + k_per_part - 1) / k_per_part;
             void* ws = nullptr;
+            // the partial rows stay below the 1 GiB every split plan keeps its workspace under; a product beyond that
+            // (32 rows against an inner dimension of tens of thousands) goes to the tile kernels below
+            if ((uint64_t)parts * M * N * eb <= ((uint64_t)1 << 30)) {
             if (int e = workspace(dev, (uint64_t)parts * M * N * eb, &ws)) return e;
             const dim3 grid((unsigned)(col_blocks * parts));
             auto launch = [&](auto t, auto rows_tag) {
@@ -1266,6 +1390,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             NK_HIP(hipGetLastError());
             set_path(dtype == NK_F64 ? "few_rows_f64" : "few_rows");
             return NK_OK;
+            }
         }
     }
     // a batch of columns (3, 5 ... 16): one stream over A, B through LDS
@@ -1382,25 +1507,48 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 gb.tiles_m = (int)((M + big::TM - 1) / big::TM); gb.tiles_n = (int)((N + big::TN - 1) / big::TN);
                 gb.group_rows = gb.tiles_m < 4 ? gb.tiles_m : 4;
                 constexpr int lds_bytes = big::LDS_FLOATS * (int)sizeof(float);
-                static std::once_flag big_once;
-                static hipError_t big_attr = hipSuccess;
-                std::call_once(big_once, [&]() {
-                    const void* kernels[4] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
-                                              (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>};
-                    for (const void* k : kernels)
-                        if (big_attr == hipSuccess) big_attr = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-                });
-                NK_HIP(big_attr);
-                const dim3 grid((unsigned)tiles);
-                if (whole_big) {
-                    if (overwrite) hipLaunchKernelGGL((matmul_mfma_big_kernel<true, false>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
-                    else           hipLaunchKernelGGL((matmul_mfma_big_kernel<false, false>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
-                } else {
-                    if (overwrite) hipLaunchKernelGGL((matmul_mfma_big_kernel<true, true>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
-                    else           hipLaunchKernelGGL((matmul_mfma_big_kernel<false, true>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                // the kernel needs more LDS than a launch gets by default: asked for once per device; a device that does not
+                // grant it (or has less) keeps to the plans below
+                if (dev->big_tiles == 0) {
+                    dev->big_tiles = -1;
+                    if ((int64_t)dev->props.sharedMemPerBlockOptin >= lds_bytes) {
+                        const void* kernels[4] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
+                                                  (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>};
+                        hipError_t attr = hipSuccess;
+                        for (const void* k : kernels)
+                            if (attr == hipSuccess) attr = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+                        if (attr == hipSuccess) dev->big_tiles = 1; else (void)hipGetLastError();
+                    }
                 }
+                if (dev->big_tiles > 0) {
+                    const dim3 grid((unsigned)tiles);
+                    if (whole_big) {
+                        if (overwrite) hipLaunchKernelGGL((matmul_mfma_big_kernel<true, false>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                        else           hipLaunchKernelGGL((matmul_mfma_big_kernel<false, false>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                    } else {
+                        if (overwrite) hipLaunchKernelGGL((matmul_mfma_big_kernel<true, true>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                        else           hipLaunchKernelGGL((matmul_mfma_big_kernel<false, true>), grid, dim3(256), lds_bytes, dev->stream, gb, Ap, Bp, Cp);
+                    }
+                    NK_HIP(hipGetLastError());
+                    set_path(whole_big ? "mfma_big" : "mfma_big_edge");
+                    return NK_OK;
+                }
+            }
+        }
+        // fewer large tiles than compute units, but whole 64 x 64 tiles, at least one per unit: the small-tile kernel in one launch
+        if (bands && force_parts < 2 && aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0 && K >= 4 * BK) {
+            const int64_t cus = dev->props.multiProcessorCount;
+            const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = (M / t64::TM) * (N / t64::TN);
+            // (against the k range of the large tiles cut into parts: 1024^3 78 against 69 TFLOP/s; with more large tiles or a
+            // long k range the parts win: 1536^3 83 against 89, 1024 x 4096 x 1024 89 against 104)
+            if (large <= cus / 4 && small >= cus && K <= 2048) {
+                MfmaArgs gs = g;
+                gs.tiles_m = (int)(M / t64::TM); gs.tiles_n = (int)(N / t64::TN);
+                gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
+                if (overwrite) hipLaunchKernelGGL(matmul_mfma64_kernel<true>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                else           hipLaunchKernelGGL(matmul_mfma64_kernel<false>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
                 NK_HIP(hipGetLastError());
-                set_path(whole_big ? "mfma_big" : "mfma_big_edge");
+                set_path("mfma_tiles_of_64");
                 return NK_OK;
             }
         }
