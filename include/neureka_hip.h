@@ -83,6 +83,10 @@ int nk_device_sync(nk_dev dev);
 /* device properties: J/devices/opencl/OpenCLDevice.java:738-809 (name, globalMemSize, maxComputeUnits, ...) */
 int nk_device_props(nk_dev dev, char* name, size_t name_cap, int* compute_units, int* clock_mhz,
                     uint64_t* global_mem_bytes, int* lds_bytes_per_block, int* wavefront_size);
+/* memory of the device that is free right now, and all of it (the latter is CL_DEVICE_GLOBAL_MEM_SIZE,
+ * J/devices/opencl/OpenCLDevice.java:770-774; the former has no counterpart in the reference).  Blocks at rest in
+ * the pool count as used: the driver does not know they are free. */
+int nk_device_memory(nk_dev dev, uint64_t* free_bytes, uint64_t* total_bytes);
 /* live-allocation accounting, what numberOfDataObjects()-style leak tests observe
  * (J/devices/AbstractDeviceData.java:24-56) */
 int nk_device_stats(nk_dev dev, uint64_t* live_buffers, uint64_t* live_bytes);
@@ -205,7 +209,13 @@ int nk_dot(nk_dev dev, int dtype, nk_buf a, nk_buf b, int64_t n, nk_buf out);
  * J/backend/main/operations/linear/internal/opencl/CLGEMM.java:11-100.
  * C[M,N] += A[M,K] @ B[K,N] on dense matrices of one layout; C is accumulated into, as the reference
  * does (J/backend/main/operations/linear/internal/blas/GEMM.java:282-304; C is pre-zeroed by
- * J/backend/main/algorithms/MatMulAlgorithm.java:74-85). */
+ * J/backend/main/algorithms/MatMulAlgorithm.java:74-85).
+ * Below 2^24 multiply-adds, and for an inner dimension of at most 16 (with more than 16 columns), every element is
+ * the reference's own sum, term by term in k order with rounded products: bit-identical to the CPU device.  From
+ * 2^24 multiply-adds on the sum is re-ordered (matrix cores, or fused multiply-adds in the plans for a few rows or
+ * columns) and agrees within 1e-5 (f32) / 1e-12 (f64) of sum_k |a_ik| |b_kj|; WHICH plan runs depends on the shape
+ * and on whether A, B and C start on 16-byte boundaries, so the same product taken from a view at an odd offset may
+ * differ in its last bits from the one taken from the start of a buffer. */
 int nk_matmul(nk_dev dev, int dtype, int layout, int64_t M, int64_t K, int64_t N,
               nk_buf A, nk_buf B, nk_buf C);
 

@@ -25,6 +25,7 @@ public final class Nk {
     public static final MethodHandle nk_device_close      = h("nk_device_close", I, J);
     public static final MethodHandle nk_device_sync       = h("nk_device_sync", I, J);
     public static final MethodHandle nk_device_props      = h("nk_device_props", I, J, P, J, P, P, P, P, P);
+    public static final MethodHandle nk_device_memory     = h("nk_device_memory", I, J, P, P);
     public static final MethodHandle nk_device_stats      = h("nk_device_stats", I, J, P, P);
     // memory: nk_alloc hands out a block of the pool with arbitrary contents, nk_free gives it back without a wait
     public static final MethodHandle nk_alloc             = h("nk_alloc", I, J, J, P);

@@ -32,6 +32,7 @@ SYMBOLS = {
     "nk_device_sync": (_i32, [_u64]),
     "nk_device_props": (_i32, [_u64, C.c_char_p, C.c_size_t, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(_u64),
                                C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "nk_device_memory": (_i32, [_u64, C.POINTER(_u64), C.POINTER(_u64)]),
     "nk_device_stats": (_i32, [_u64, C.POINTER(_u64), C.POINTER(_u64)]),
     "nk_alloc": (_i32, [_u64, _u64, C.POINTER(_u64)]),
     "nk_free": (_i32, [_u64, _u64]),

@@ -533,8 +533,12 @@ def hip_scalar_function(fun: str):
 
 
 def hip_scalar_broadcast_function(fun: str):
-    """The OpenCLDevice lambda of ScalarBroadcast (algorithms/ScalarBroadcast.java:64-81): value = f(source item 0),
-    then the scalar_broadcast kernel writes it through the drain's view."""
+    """ScalarBroadcast (algorithms/ScalarBroadcast.java:21-82): value = f(source item 0), written through the drain's view.
+    f is evaluated by the device's own activation kernel on the one stored element, in the drain's type: what the CPU
+    device does (CPUScalarBroadcastFunction.java:43-67: ``f.invoke(double)`` for Double, ``f.invoke(float)`` for Float
+    tensors), which is the parity target.  The OpenCL device's lambda (ScalarBroadcast.java:64-81) evaluates f in double
+    on the host and hands ``(float) value`` to its kernel for every type, so it drops digits of an f64 result; that
+    rounding is an oddity of that lambda, not of the operation, and is not repeated here."""
     def run(call: ExecutionCall):
         dev, drn, src = call.device, call.input(0), call.input(1)
         slot = dev.allocate(drn.dtype, 1)

@@ -1117,16 +1117,21 @@ __global__ __launch_bounds__(256) void matmul_short_inner_kernel(int M, int K, i
 #pragma unroll
         for (int u = 0; u < RU; u++) {
             if (r0 + u < rows) {
-                Vec acc = Vec(T(0));
+                // the reference's own order and rounding (GEMM.java:282-304): the old value, then one rounded product after the
+                // other in k order -- the same bits as the simple kernel gives, wherever the operands happen to lie.  (The
+                // stream over C bounds this kernel; the second instruction per term costs nothing.)
+                Vec acc = OVERWRITE ? Vec(T(0)) : old[u];
 #pragma unroll
                 for (int q = 0; q < KC; q += 4) {
                     const Quad a = *(const Quad*)&As[r0 + u][q];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
+                        if (q + j < K) {
 #pragma unroll
-                        for (int e = 0; e < VEC; e++) acc[e] = fma_of(a[j], b[q + j][e], acc[e]);
+                            for (int e = 0; e < VEC; e++) { const T prod = a[j] * b[q + j][e]; acc[e] = acc[e] + prod; }
+                        }
                 }
-                *(Vec*)(Cp + (int64_t)(r0 + u) * N) = OVERWRITE ? acc : old[u] + acc;
+                *(Vec*)(Cp + (int64_t)(r0 + u) * N) = acc;
             }
         }
     }
@@ -1436,6 +1441,10 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             set_path(dtype == NK_F64 ? "short_inner_f64" : "short_inner");
             return NK_OK;
         }
+        // not aligned, or rows shorter than a wavefront of vectors: the simple kernel, which gives the same bits (a
+        // matrix-core plan would re-order sixteen terms for nothing); a few columns have their own plan below
+        if (N > 16) return dtype == NK_F64 ? launch_simple<double>(dev, M, K, N, overwrite, (const double*)A, (const double*)B, (double*)C)
+                               : launch_simple<float>(dev, M, K, N, overwrite, (const float*)A, (const float*)B, (float*)C);
     }
     // a few columns of B: one stream over A
     if (bands && N <= 4 && M * K * N >= mfma_from) {

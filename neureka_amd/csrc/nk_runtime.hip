@@ -263,6 +263,15 @@ int nk_device_props(nk_dev h, char* name, size_t name_cap, int* compute_units, i
     return NK_OK;
 }
 
+int nk_device_memory(nk_dev h, uint64_t* free_bytes, uint64_t* total_bytes) {
+    NK_DEVICE(dev, h);
+    size_t f = 0, t = 0;
+    NK_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return NK_OK;
+}
+
 int nk_d2d(nk_dev h, nk_buf dst, uint64_t dst_off, nk_buf src, uint64_t src_off, uint64_t bytes) {
     NK_DEVICE(dev, h);
     if (bytes == 0) return NK_OK;

@@ -219,6 +219,12 @@ class HipDevice:
         _lib.check(self._lib.nk_device_stats(self.handle, C.byref(n), C.byref(b)))
         return n.value
 
+    def freeMemory(self) -> int:
+        """Bytes of device memory the driver reports as free (blocks at rest in the pool count as used)."""
+        f, t = C.c_uint64(0), C.c_uint64(0)
+        _lib.check(self._lib.nk_device_memory(self.handle, C.byref(f), C.byref(t)))
+        return f.value
+
     def poolStats(self) -> dict:
         """The buffer pool behind ``allocate`` / ``HipData.release``: blocks at rest, their bytes, allocations that
         went to the driver and allocations served from a block at rest."""

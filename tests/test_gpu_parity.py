@@ -1988,13 +1988,20 @@ def test_matmul_short_inner_dimension(device, orc, mkn, dt):
     got = pc.getData()
     assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
     assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
-    say("matmul short inner dimension, uniform data against the oracle", mkn, dt)
-    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T)
-    tc = on(device, np.zeros((M, N), dtype=T))
+    say("matmul short inner dimension, uniform data bit for bit against the oracle", mkn, dt)
+    # the kernel keeps the reference's order and rounding (old value, then the rounded products in k order): the bits of
+    # GEMM.partial_F32_MxN_RM, into a non-zero C as well, and the same bits when the operands are moved off the
+    # 16-byte boundary (another plan takes them then)
+    A = rng.uniform(-1, 1, (M, K)).astype(T); B = rng.uniform(-1, 1, (K, N)).astype(T); C1 = rng.uniform(-1, 1, (M, N)).astype(T)
+    tc = on(device, C1)
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
-    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N)
-    bound = tol * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
-    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+    assert _lib.last_path() == path, _lib.last_path()
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, C_init=C1.reshape(-1).copy(), workers=8).reshape(M, N)
+    assert_bits(tc.getData().reshape(M, N), ref, "C += A B, uniform data")
+    pa, pb, pc = (on(device, np.concatenate([np.zeros(1, dtype=T), x.reshape(-1)])) for x in (A, B, C1))
+    _lib.check(device._lib.nk_matmul(device.handle, 0 if dt == "f32" else 1, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + eb, pb._data.ptr + eb, pc._data.ptr + eb))
+    assert _lib.last_path() != path
+    assert_bits(pc.getData()[1:].reshape(M, N), ref, "the same product from operands off a 16-byte boundary")
 
 
 @pytest.mark.parametrize("dt", ["f32", "f64"])
@@ -2070,6 +2077,29 @@ def test_matmul_streaming_plans_need_aligned_operands_and_fall_back(device, mkn,
         got = pc.getData()
         assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()
         assert (got[pad:pad + M * N].reshape(M, N) == want + C0).all()
+
+
+@pytest.mark.parametrize("mkn,path", [((16, 4096, 4096), "few_rows"), ((4096, 4096, 16), "some_cols"), ((4096, 4096, 1), "few_cols")])
+def test_matmul_streaming_plans_depend_on_alignment_only_within_tolerance(device, orc, mkn, path):
+    """few_rows, few_cols and some_cols add their terms with fused multiply-adds in an order of their own and are chosen
+    by the operands' 16-byte alignment as well as by shape: the same product from a view one element into its buffer
+    takes another plan and may differ in the last bits.  Both stay within the norm-wise 1e-5 of the oracle (from 2^24
+    multiply-adds on every plan re-orders the sum), and so within 2e-5 of each other."""
+    M, K, N = mkn
+    rng = np.random.default_rng(69)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    ref = orc.gemm(True, A.reshape(-1), B.reshape(-1), M, K, N, workers=8).reshape(M, N).astype(np.float64)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    results = []
+    for pad in (0, 1):
+        say("matmul plan against alignment", mkn, "operands", pad, "elements into their buffers")
+        pa, pb, pc = (on(device, np.concatenate([np.zeros(pad, dtype=np.float32), x.reshape(-1)])) for x in (A, B, np.zeros((M, N), dtype=np.float32)))
+        _lib.check(device._lib.nk_matmul_set(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+        assert (_lib.last_path() == path) == (pad == 0), _lib.last_path()
+        got = pc.getData()[pad:].reshape(M, N).astype(np.float64)
+        assert (np.abs(got - ref) <= bound).all(), _lib.last_path()
+        results.append(got)
+    assert (np.abs(results[0] - results[1]) <= 2 * bound).all()
 
 
 @pytest.mark.parametrize("mkn", [(3072, 1024, 3072), (3000, 800, 3100), (1280, 1024, 8192), (2700, 640, 3400)])
