@@ -760,7 +760,8 @@ __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int pa
 }
 
 // ---- a few rows times a large matrix ----------------------------------------------------------------------------
-// C[M,N] = A[M,K] @ B[K,N] with M <= 32 (a vector or a small batch times a weight matrix): the product reads B once
+// C[M,N] = A[M,K] @ B[K,N] with M <= 4 (a vector or a handful of rows times a weight matrix; 5 to 32 rows take
+// matmul_few_rows_mfma_kernel further down, which shares this kernel's launch shape): the product reads B once
 // and is bound by that stream; a 128 x 128 tile would spend its matrix cores on rows that do not exist.  A block owns
 // 64 * (16 bytes / element) columns and one part of the k range (at most few_kp(MR) rows), whose piece of A it stages
 // in LDS; each of its four wavefronts takes a quarter of the part -- a row of B is one contiguous kilobyte for a
@@ -768,7 +769,7 @@ __global__ __launch_bounds__(256) void matmul_add_parts_kernel(int64_t n, int pa
 // accumulators per column in registers (the elements of A come as 16-byte LDS reads of one address for the whole
 // wavefront), the wavefronts meet in LDS in a fixed order, and the block's partial rows go to P[part];
 // matmul_add_parts_kernel adds the parts in order.
-constexpr int few_kp(int mr) { return mr <= 4 ? 1024 : mr <= 16 ? 256 : 128; }     // k rows a block stages of A: 16-32 KiB of LDS
+constexpr int few_kp(int mr) { return mr <= 4 ? 1024 : mr <= 16 ? 256 : 128; }     // k rows a block stages of A: at most 16 KiB of LDS
 __device__ __forceinline__ float fma_of(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 __device__ __forceinline__ double fma_of(double a, double b, double c) { return __builtin_fma(a, b, c); }
 template <typename T, int MR>
@@ -973,108 +974,163 @@ __global__ __launch_bounds__(256) void matmul_few_cols_kernel(int M, int K, cons
 }
 
 // ---- a large matrix times a batch of columns --------------------------------------------------------------------
-// C[M,N] = A[M,K] @ B[K,N] with 5 <= N <= 16 (or 3), padded to NC = 8 or 16: still one stream over A, but a lane now
-// needs NC elements of B for each of its k's, which come from LDS.  The block's eight wavefronts (two rows of A each)
-// walk along k together; the piece of B for a trip -- 64 x (16 bytes / element) rows, NC columns -- is staged while
-// the trip before it is computed (two buffers, one barrier per trip), laid out [k % VEC][k / VEC][NC + 16 bytes] so
-// that the 64 lanes' 16-byte reads of one column group fall on different banks.
-template <typename T, int NC, bool OVERWRITE>
+// C[M,N] = A[M,K] @ B[K,N] with 3 <= N <= 16: one stream over A.  A block owns 16 rows of A, its eight wavefronts an
+// eighth of the k range each, and a wavefront multiplies its 16 x (k range) piece of A into 16 columns on the matrix
+// core (v_mfma_f32_16x16x4_f32, v_mfma_f64_16x16x4_f64): lane (row i, quarter q) loads 16 bytes of row i -- the four
+// lanes of a row cover 64 contiguous bytes -- and the elements of B for the same k's with plain loads (a step's piece
+// of B is 16 x VEC rows of N columns, contiguous, and stays in the caches: B is K x N, a few hundred KiB).  Multiply-add
+// e of a step takes element e of every lane, i.e. k = k0 + VEC q + e for q = 0..3: any assignment of k's to the four
+// slots of the instruction works as long as A and B use the same one.  Columns from N on are fed zeros.  Nothing
+// goes through LDS until the eight partial 16 x 16 results meet there, in wavefront order, at the end: no barrier per
+// trip, which is what held the kernel this replaces (B staged through LDS, a barrier per 256 k's) at 33 us for
+// [4096,4096] @ [4096,16].
+template <typename T> struct Mfma16;
+template <> struct Mfma16<float> {
+    typedef float Acc __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ int row_of(int q, int v) { return 4 * q + v; }      // accumulator v of lane quarter q
+};
+template <> struct Mfma16<double> {
+    typedef double Acc __attribute__((ext_vector_type(4)));
+    static __device__ __forceinline__ Acc mma(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ int row_of(int q, int v) { return 4 * v + q; }
+};
+template <typename T, bool OVERWRITE>
 __global__ __launch_bounds__(512) void matmul_some_cols_kernel(int M, int K, int N, const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C) {
     constexpr int VEC = 16 / (int)sizeof(T);
-    constexpr int R = 2, THREADS = 512;                                 // eight wavefronts of two rows: sixteen rows per block
-    constexpr int PITCH = NC + VEC;                                     // elements per (k) row in LDS
-    constexpr int STEP = 64 * VEC;                                      // k's per trip
-    constexpr int PIECES = STEP * NC / VEC / THREADS;                   // 16-byte pieces of a trip's B per thread
+    constexpr int STEP = 4 * VEC;                                       // k's per step of a wavefront
+    constexpr int NW = 8, AHEAD = 4;                                    // wavefronts per block; steps requested together
     typedef T Vec __attribute__((ext_vector_type(VEC)));
-    __shared__ __attribute__((aligned(16))) T Bs[2][VEC][64][PITCH];
+    typedef typename Mfma16<T>::Acc Acc;
+    __shared__ T part[NW][16][17];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int64_t row0 = ((int64_t)blockIdx.x * (THREADS / 64) + wave) * R;
-    const T* rows[R];
-#pragma unroll
-    for (int r = 0; r < R; r++) rows[r] = A + (row0 + r < M ? row0 + r : M - 1) * (int64_t)K;
-    T acc[R][NC];
-#pragma unroll
-    for (int r = 0; r < R; r++)
-#pragma unroll
-        for (int n = 0; n < NC; n++) acc[r][n] = T(0);
+    const int i = lane & 15, q = lane >> 4;
+    const int64_t row0 = (int64_t)blockIdx.x * 16;
+    const T* row = A + (row0 + i < M ? row0 + i : M - 1) * (int64_t)K;
+    const int steps = (K + STEP - 1) / STEP, per = (steps + NW - 1) / NW;
+    const int s0 = wave * per, s1 = s0 + per < steps ? s0 + per : steps;
+    const bool col_live = i < N;
+    Acc acc = {T(0), T(0), T(0), T(0)};
     // K % VEC == 0 (the host checks): a lane's VEC k's are inside the matrix or all outside
-    auto request_a = [&](Vec (&a)[R], int k0) {
-        const int k = k0 + lane * VEC;
+    auto request = [&](Vec (&a)[AHEAD], T (&b)[AHEAD][VEC], int s) {
 #pragma unroll
-        for (int r = 0; r < R; r++) a[r] = k < K ? *(const Vec*)(rows[r] + k) : Vec(T(0));
+        for (int u = 0; u < AHEAD; u++) {
+            const int k = (s + u) * STEP + q * VEC;
+            const bool in = s + u < s1 && k < K;
+            a[u] = in ? *(const Vec*)(row + k) : Vec(T(0));
+#pragma unroll
+            for (int e = 0; e < VEC; e++) b[u][e] = (in && col_live) ? B[(int64_t)(k + e) * N + i] : T(0);
+        }
     };
-    // piece p of a trip: VEC columns from n = (p * VEC) % NC of row k0 + (p * VEC) / NC
-    auto request_b = [&](Vec (&s)[PIECES], int k0) {
+    // the next AHEAD steps are on their way while these are multiplied in
+    Vec a[AHEAD], an[AHEAD];
+    T b[AHEAD][VEC], bn[AHEAD][VEC];
+    request(a, b, s0);
+    for (int s = s0; s < s1; s += AHEAD) {
+        request(an, bn, s + AHEAD);                                     // (past the end: zeros, no memory access)
 #pragma unroll
-        for (int j = 0; j < PIECES; j++) {
-            const int p = (int)threadIdx.x + THREADS * j;
-            const int kl = p * VEC / NC, n = p * VEC % NC;
-            s[j] = Vec(T(0));
-            if (k0 + kl < K) {
-                if (N == NC) s[j] = *(const Vec*)(B + (int64_t)(k0 + kl) * NC + n);        // (B is 16-byte aligned: the host checks)
-                else {
+        for (int u = 0; u < AHEAD; u++)
 #pragma unroll
-                    for (int e = 0; e < VEC; e++)
-                        if (n + e < N) s[j][e] = B[(int64_t)(k0 + kl) * N + n + e];
+            for (int e = 0; e < VEC; e++) acc = Mfma16<T>::mma(a[u][e], b[u][e], acc);
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++) {
+            a[u] = an[u];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) b[u][e] = bn[u][e];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[wave][Mfma16<T>::row_of(q, v)][i] = acc[v];
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        const int r = threadIdx.x >> 4, c = threadIdx.x & 15;
+        if (row0 + r < M && c < N) {
+            T sum = part[0][r][c];
+#pragma unroll
+            for (int w = 1; w < NW; w++) sum = sum + part[w][r][c];     // wavefronts in order
+            T* dst = C + (row0 + r) * (int64_t)N + c;
+            *dst = OVERWRITE ? sum : *dst + sum;
+        }
+    }
+}
+
+// ---- five to 32 rows times a large matrix, on the matrix cores ----------------------------------------------------------
+// The same product as matmul_few_rows_kernel computes, C[M,N] = A[M,K] @ B[K,N] with one stream over B, for 5 <= M <= 32:
+// with 16 or 32 rows a lane of that kernel issues 64 or 128 multiply-adds per 16 bytes of B, and the vector unit, not the
+// stream, sets the pace ([16,4096] @ [4096,4096]: 19 us for 64 MiB).  Here a wavefront owns 16 x VEC columns and
+// multiplies its k range into them as 16 x 16 x 4 matrix instructions: lane (j, q) loads 16 bytes of row k0 + VEC q + e'
+// of B -- the sixteen lanes j cover 256 contiguous bytes of that row -- and element e of the load belongs to column
+// 4 j + e, i.e. to accumulator e; the A operand of the instruction is A[i][k0 + VEC q + e'] out of the block's staged
+// piece of A (lane (i, q), one 16-byte LDS read per step).  The four wavefronts of a block sit side by side on 64 x VEC
+// columns and walk the same part of the k range, so they never meet; partial rows go to P[part] and
+// matmul_add_parts_kernel adds the parts in order.  RG: groups of 16 rows (1 or 2).
+template <typename T, int RG>
+__global__ __launch_bounds__(256) void matmul_few_rows_mfma_kernel(int M, int K, int N, int k_per_part, int col_blocks, const T* __restrict__ A,
+                                                                   const T* __restrict__ B, T* __restrict__ P) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int STEP = 4 * VEC;                                       // k's per step
+    constexpr int KP = 256, AP = KP + VEC;                              // k's a block stages of A; row pitch in LDS
+    constexpr int AHEAD = 4;                                            // steps whose rows of B are requested together
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    typedef typename Mfma16<T>::Acc Acc;
+    __shared__ __attribute__((aligned(16))) T As[RG * 16][AP];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int j = lane & 15, q = lane >> 4;
+    const int part = (int)(blockIdx.x / (unsigned)col_blocks), col_block = (int)(blockIdx.x % (unsigned)col_blocks);
+    const int64_t col0 = (((int64_t)col_block * 4 + wave) * 16 + j) * VEC;     // N % VEC == 0 (the host checks)
+    const bool live = col0 < N;
+    const int k_begin = part * k_per_part;
+    const int k_count = k_begin + k_per_part < K ? k_per_part : K - k_begin;     // 1 ... KP
+    for (int idx = threadIdx.x; idx < RG * 16 * KP; idx += 256) {
+        const int m = idx / KP, kk = idx % KP;
+        As[m][kk] = (m < M && kk < k_count) ? A[(int64_t)m * K + k_begin + kk] : T(0);
+    }
+    Acc acc[RG][VEC];
+#pragma unroll
+    for (int g = 0; g < RG; g++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[g][e] = Acc{T(0), T(0), T(0), T(0)};
+    const T* Bc = B + (live ? col0 : 0) + (int64_t)k_begin * N;
+    const int steps = (k_count + STEP - 1) / STEP;
+    __syncthreads();                                                    // the staged piece of A is complete
+    // (requesting the next AHEAD steps while these are multiplied in changed nothing here: 21.4 against 22.7 us for 16 rows)
+    for (int s = 0; s < steps; s += AHEAD) {
+        Vec b[AHEAD][VEC];
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++)
+#pragma unroll
+            for (int r = 0; r < VEC; r++) {
+                const int kk = (s + u) * STEP + VEC * q + r;
+                b[u][r] = (live && kk < k_count) ? *(const Vec*)(Bc + (int64_t)kk * N) : Vec(T(0));
+            }
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++) {
+            if (s + u < steps) {                                        // (uniform; past the end b is zero anyway, this saves the LDS reads)
+#pragma unroll
+                for (int g = 0; g < RG; g++) {
+                    const Vec a = *(const Vec*)&As[16 * g + j][(s + u) * STEP + VEC * q];
+#pragma unroll
+                    for (int r = 0; r < VEC; r++)
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) acc[g][e] = Mfma16<T>::mma(a[r], b[u][r][e], acc[g][e]);
                 }
             }
         }
-    };
-    auto put_b = [&](const Vec (&s)[PIECES], int buf) {
-#pragma unroll
-        for (int j = 0; j < PIECES; j++) {
-            const int p = (int)threadIdx.x + THREADS * j;
-            const int kl = p * VEC / NC, n = p * VEC % NC;
-            *(Vec*)&Bs[buf][kl % VEC][kl / VEC][n] = s[j];
-        }
-    };
-    Vec a[R], staged[PIECES];
-    request_a(a, 0);
-    request_b(staged, 0);
-    put_b(staged, 0);
-    __syncthreads();
-    int buf = 0;
-    for (int k0 = 0; k0 < K; k0 += STEP) {
-        Vec an[R];
-        const bool more = k0 + STEP < K;
-        if (more) { request_a(an, k0 + STEP); request_b(staged, k0 + STEP); }
-#pragma unroll
-        for (int v = 0; v < VEC; v++) {
-            T bv[NC];
-#pragma unroll
-            for (int q = 0; q < NC; q += VEC) *(Vec*)&bv[q] = *(const Vec*)&Bs[buf][v][lane][q];
-#pragma unroll
-            for (int n = 0; n < NC; n++)
-#pragma unroll
-                for (int r = 0; r < R; r++) acc[r][n] = fma_of(a[r][v], bv[n], acc[r][n]);
-        }
-        if (more) {
-            put_b(staged, buf ^ 1);
-#pragma unroll
-            for (int r = 0; r < R; r++) a[r] = an[r];
-        }
-        __syncthreads();
-        buf ^= 1;
     }
+    if (live) {
+        T* Pp = P + (int64_t)part * M * N + col0;
 #pragma unroll
-    for (int r = 0; r < R; r++)
+        for (int g = 0; g < RG; g++)
 #pragma unroll
-        for (int n = 0; n < NC; n++) {
-            T v = acc[r][n];
+            for (int v = 0; v < 4; v++) {
+                const int row = 16 * g + Mfma16<T>::row_of(q, v);
+                if (row < M) {
+                    Vec out;
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
-            acc[r][n] = v;
-        }
-    if (lane == 0) {
-#pragma unroll
-        for (int r = 0; r < R; r++)
-            if (row0 + r < M)
-#pragma unroll
-                for (int n = 0; n < NC; n++)
-                    if (n < N) {
-                        T* c = C + (row0 + r) * (int64_t)N + n;
-                        *c = OVERWRITE ? acc[r][n] : *c + acc[r][n];
-                    }
+                    for (int e = 0; e < VEC; e++) out[e] = acc[g][e][v];
+                    *(Vec*)(Pp + (int64_t)row * N) = out;
+                }
+            }
     }
 }
 
@@ -1369,7 +1425,9 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             if (parts < 1) parts = 1;
             int k_per_part = (int)((K + parts - 1) / parts);
             const int mr = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : M <= 16 ? 16 : 32;
-            if (k_per_part > few_kp(mr)) k_per_part = few_kp(mr);          // what a block stages of A
+            const bool on_matrix_cores = M > 4;                         // 5 ... 32 rows: 16 x 16 x 4 matrix instructions
+            const int staged = on_matrix_cores ? 256 : few_kp(mr);
+            if (k_per_part > staged) k_per_part = staged;               // what a block stages of A
             parts = (K + k_per_part - 1) / k_per_part;
             void* ws = nullptr;
             // the partial rows stay below the 1 GiB every split plan keeps its workspace under; a product beyond that
@@ -1383,13 +1441,18 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                                    (const T*)A, (const T*)B, (T*)ws);
                 hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, dev->stream, M * N, (int)parts, g.overwrite, (const T*)ws, (T*)C);
             };
+            auto launch_mfma = [&](auto t, auto groups_tag) {
+                using T = decltype(t);
+                hipLaunchKernelGGL((matmul_few_rows_mfma_kernel<T, decltype(groups_tag)::value>), grid, dim3(256), 0, dev->stream, (int)M, (int)K, (int)N, k_per_part, (int)col_blocks,
+                                   (const T*)A, (const T*)B, (T*)ws);
+                hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, dev->stream, M * N, (int)parts, g.overwrite, (const T*)ws, (T*)C);
+            };
             auto by_rows = [&](auto t) {
                 if (M <= 1) launch(t, std::integral_constant<int, 1>{});
                 else if (M <= 2) launch(t, std::integral_constant<int, 2>{});
                 else if (M <= 4) launch(t, std::integral_constant<int, 4>{});
-                else if (M <= 8) launch(t, std::integral_constant<int, 8>{});
-                else if (M <= 16) launch(t, std::integral_constant<int, 16>{});
-                else launch(t, std::integral_constant<int, 32>{});
+                else if (M <= 16) launch_mfma(t, std::integral_constant<int, 1>{});
+                else launch_mfma(t, std::integral_constant<int, 2>{});
             };
             if (dtype == NK_F64) by_rows(double{}); else by_rows(float{});
             NK_HIP(hipGetLastError());
@@ -1398,22 +1461,17 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             }
         }
     }
-    // a batch of columns (3, 5 ... 16): one stream over A, B through LDS
+    // a batch of columns (3, 5 ... 16): one stream over A on the matrix cores
     if (bands && N <= 16 && N != 1 && N != 2 && N != 4 && M * K * N >= mfma_from) {
         const int eb = dtype == NK_F64 ? 8 : 4, vec = 16 / eb;
         if (K % vec == 0 && A % 16 == 0 && B % 16 == 0 && M >= 1024) {
             const dim3 grid((unsigned)((M + 15) / 16));
-            auto launch = [&](auto t, auto nc) {
+            auto launch = [&](auto t) {
                 using T = decltype(t);
-                constexpr int NC = decltype(nc)::value;
-                if (overwrite) hipLaunchKernelGGL((matmul_some_cols_kernel<T, NC, true>), grid, dim3(512), 0, dev->stream, (int)M, (int)K, (int)N, (const T*)A, (const T*)B, (T*)C);
-                else           hipLaunchKernelGGL((matmul_some_cols_kernel<T, NC, false>), grid, dim3(512), 0, dev->stream, (int)M, (int)K, (int)N, (const T*)A, (const T*)B, (T*)C);
+                if (overwrite) hipLaunchKernelGGL((matmul_some_cols_kernel<T, true>), grid, dim3(512), 0, dev->stream, (int)M, (int)K, (int)N, (const T*)A, (const T*)B, (T*)C);
+                else           hipLaunchKernelGGL((matmul_some_cols_kernel<T, false>), grid, dim3(512), 0, dev->stream, (int)M, (int)K, (int)N, (const T*)A, (const T*)B, (T*)C);
             };
-            auto by_cols = [&](auto t) {
-                if (N <= 8) launch(t, std::integral_constant<int, 8>{});
-                else launch(t, std::integral_constant<int, 16>{});
-            };
-            if (dtype == NK_F64) by_cols(double{}); else by_cols(float{});
+            if (dtype == NK_F64) launch(double{}); else launch(float{});
             NK_HIP(hipGetLastError());
             set_path(dtype == NK_F64 ? "some_cols_f64" : "some_cols");
             return NK_OK;
