@@ -24,9 +24,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X dense fp32 matrix, published
 FP64_PEAK_TFLOPS = 78.6        # MI355X dense fp64 matrix, published
-# HBM bytes per launch of the headline kernel from two rocprofv3 --pmc runs (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000
-# against a plain 1 GiB copy): profiles/rows_binary_lean_kernel_broadcast_c2.md
-C2_TRAFFIC_BYTES = 4316335565
+# HBM bytes per launch of the headline kernel come from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE, each
+# scaled by what the same counter reads for a plain 1 GiB copy); the command that writes the profile summaries writes
+# the figure, the kernel it belongs to and a digest of that kernel's sources into this file.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "rows_binary_lean_kernel_broadcast_c2.json")
 SETTLE_MS = 60.0               # untimed load before the warm-up steps, so that the timed steps run at the working clock
 HOST_CORE_SHARE = 16           # host threads one GPU's box grants a job, whatever the machine's core count
 
@@ -168,6 +169,21 @@ def torch_yardstick():
     img = torch.randn(1, 1, 4096, 4096, device=d); k3 = torch.randn(1, 1, 3, 3, device=d)
     t("conv2d_4096x4096_3x3_us", lambda: F.conv2d(img, k3))
     return res
+
+
+def counted_traffic(path):
+    """(bytes, note): the counter-measured HBM traffic per launch of the headline kernel, or (None, why not) when the
+    record is missing, belongs to another kernel plan, or was taken from other sources than the library was built from."""
+    from neureka_amd.profile_summary import kernel_sources_digest
+    if not os.path.exists(TRAFFIC_FILE):
+        return None, "no counter record beside the profile"
+    with open(TRAFFIC_FILE) as f:
+        rec = json.load(f)
+    if rec.get("path") != path:
+        return None, f"the counter record is of plan {rec.get('path')}, this run took {path}"
+    if rec.get("sources_sha256") != kernel_sources_digest():
+        return None, "the kernel's sources changed since the counters were read"
+    return int(rec["traffic_bytes"]), f"FETCH_SIZE x {rec['fetch_scale']} + WRITE_SIZE x {rec['write_scale']}, {rec['dispatches']} dispatches"
 
 
 def percentiles(xs):
@@ -400,8 +416,9 @@ def main():
     k_ms = 0.5 * (k_add + k_mul)
     achieved = bytes_per_launch / (k_ms * 1e-3) / 1e9
     singles = sorted(event_times_ms(dev, launch_add, 50) + event_times_ms(dev, launch_mul, 50))
+    traffic, traffic_note = counted_traffic(path)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": C2_TRAFFIC_BYTES if path == "rows_vec_binary_lean" else None,
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_note,
                 "kernel": f"nk::rows_binary_lean_kernel<float, 4, 2, 0, true> ({path})",
                 "launch_ms": round(k_ms, 4), "algorithmic_bytes": bytes_per_launch,
                 "single_launch_ms": {"p10": round(singles[len(singles) // 10], 4), "median": round(singles[len(singles) // 2], 4),
@@ -453,19 +470,28 @@ def main():
                 count += 1
             dev.sync()
 
-        def hbm(name, nbytes, launch):
+        def spread(launch):
+            # `ms` is the mean of `reps` launches queued back to back between one pair of events; the spread comes from
+            # 30 launches with an event after each (an event between two launches costs them their overlap of tail and
+            # start, a microsecond or two: these are upper figures for kernels of a few microseconds)
+            return percentiles(event_times_ms(dev, launch, 30))
+
+        def hbm(name, nbytes, launch, note=None):
             warm(launch)
             ms = event_time_ms(dev, launch, reps)
             gbs = nbytes / (ms * 1e-3) / 1e9
-            others[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "path": _lib.last_path()}
+            others[name] = {"ms": round(ms, 4), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4), "path": _lib.last_path(),
+                            "single_launch_ms": spread(launch)}
+            if note: others[name]["note"] = note
 
-        def flops(name, nflop, nbytes, launch, f64=False):
+        def flops(name, nflop, nbytes, launch, f64=False, note=None):
             warm(launch)
             ms = event_time_ms(dev, launch, reps)
             tf = nflop / (ms * 1e-3) / 1e12
             frac = {"frac_fp64": round(tf / FP64_PEAK_TFLOPS, 4)} if f64 else {"frac_fp32": round(tf / FP32_PEAK_TFLOPS, 4)}
             others[name] = {"ms": round(ms, 4), "GFLOP/s": round(tf * 1e3, 1), **frac,
-                            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "path": _lib.last_path()}
+                            "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1), "path": _lib.last_path(), "single_launch_ms": spread(launch)}
+            if note: others[name]["note"] = note
 
         # C2 f64
         a64 = Tensor.of(np.float64, (256, 1, 512), rng.uniform(-1, 1, 256 * 512)).to(dev)
@@ -574,7 +600,9 @@ def main():
         # C4 matmul
         # (4000^3: a large shape that is no whole number of tiles)
         for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256)), ("matmul_4000", (4000, 4000, 4000)),
-                                ("matmul_3072", (3072, 3072, 3072))):          # 576 tiles of 128 x 128: a round of the machine and an eighth
+                                ("matmul_3072", (3072, 3072, 3072)),           # 576 tiles of 128 x 128: a round of the machine and an eighth
+                                ("matmul_2048", (2048, 2048, 2048)), ("matmul_1536", (1536, 1536, 1536)),   # a round of tiles, and less
+                                ("matmul_1024", (1024, 1024, 1024))):
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
             Cm = Tensor._on_device(dev, f32, (M, N))
@@ -591,6 +619,7 @@ def main():
         for t in (A, B, Cm): dev.free(t)
         # the products of a dense layer with a small batch: each streams its large operand once (memory-bound)
         for name, (M, K, N) in (("matmul_matrix_vector", (4096, 4096, 1)), ("matmul_batch_of_16_rows", (16, 4096, 4096)),
+                                ("matmul_batch_of_32_rows", (32, 4096, 4096)), ("matmul_batch_of_4_rows", (4, 4096, 4096)),
                                 ("matmul_16_outer_products", (4096, 16, 4096)), ("matmul_batch_of_16_columns", (4096, 4096, 16))):
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
@@ -613,7 +642,10 @@ def main():
         xl = Tensor.of(f32, (2048, 2048), rng.uniform(-1, 1, 2048 * 2048).astype(f32)).to(dev)
         kl = Tensor.of(f32, (5, 5), rng.uniform(-1, 1, 25).astype(f32)).to(dev)
         yl = Tensor._on_device(dev, f32, (2044, 2044))
-        flops("conv2d_2048x2048_5x5", 2.0 * 2044 * 2044 * 25, 4 * (2048 * 2048 + 25 + 2044 * 2044), dev.prepared_launch("convolution", -1, yl, xl, kl))
+        flops("conv2d_2048x2048_5x5", 2.0 * 2044 * 2044 * 25, 4 * (2048 * 2048 + 25 + 2044 * 2044), dev.prepared_launch("convolution", -1, yl, xl, kl),
+              note="a parity decision, not a slow kernel: every tap is a rounded multiply followed by a rounded add, as "
+                   "SimpleCPUConvolution computes it, so that the result has the reference's bits; 50 vector "
+                   "instructions per output bound the kernel, a fused multiply-add would halve them and change the bits")
         for t in (xl, kl, yl): dev.free(t)
         # 3x3 taps on a 4096^2 image: 18 unfused vector operations per output instead of 50, so memory gets a say
         xl = Tensor.of(f32, (4096, 4096), rng.uniform(-1, 1, 4096 * 4096).astype(f32)).to(dev)

@@ -450,6 +450,38 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
     }
 }
 
+// drain = f(src) or f'(src) for ONE function of the table, known at compile time: what nk_activation launches.  The data
+// path is rows_kernel's (plain vector loads, two units per block); the function is inlined instead of interpreted, so a
+// thread spends its instructions on the function alone.  That matters where the function, not memory, bounds the kernel:
+// the f32 derivatives that repeat the reference's double-precision formula (tanh', 2^26 elements: 56 vector instructions
+// per element and 0.49 of the HBM rate through the interpreter, 0.66 here) -- and the light functions lose nothing.
+constexpr int SINGLE_PASSES = 2;
+template <typename T, int V, bool NT, bool DERIV, int FID>
+__global__ __launch_bounds__(256) void rows_single_kernel(RowsArgs A, T* __restrict__ drn, const T* __restrict__ src) {
+    T x[SINGLE_PASSES * V];
+    int doff[SINGLE_PASSES];
+    bool live[SINGLE_PASSES];
+#pragma unroll
+    for (int p = 0; p < SINGLE_PASSES; p++) {
+        unsigned rg, chunk;
+        rows_unit(A, SINGLE_PASSES, p, rg, chunk);
+        const RowsAddr<2> R = rows_address<2>(A, rg, chunk);
+        live[p] = R.live;
+        doff[p] = R.off[0] + (int)R.col;
+        T (&xp)[V] = *reinterpret_cast<T (*)[V]>(&x[p * V]);
+        load_vec<T, V, NT>(xp, src + R.off[1] + R.col);
+    }
+    if constexpr (DERIV) apply_dfun<T, SINGLE_PASSES * V, dfun_calls_library(FID)>(FID, x);
+    else apply_fun<T, SINGLE_PASSES * V, (fun_is_heavy(FID) ? 2 : 1)>(FID, x);
+#pragma unroll
+    for (int p = 0; p < SINGLE_PASSES; p++) {
+        if (live[p]) {
+            T (&op)[V] = *reinterpret_cast<T (*)[V]>(&x[p * V]);
+            store_vec<T, V>(drn + doff[p], op);
+        }
+    }
+}
+
 // drain = src0 op src1 with op in {+, -, *, /} and plain aligned loads: the bandwidth-critical case
 // (same-shape elementwise and forward broadcast).  The operator is resolved once, outside the passes,
 // and each pass is stored as soon as its operands have arrived.
@@ -869,6 +901,9 @@ struct Plan {
     int passes;                // PLAN_ROWS_BINARY: units per block (2, 4 or 8)
     bool lean = false;         // PLAN_ROWS_BINARY: rows_binary_lean_kernel (one unit per block, non-temporal stores)
     bool lean_fill = false;    // PLAN_ROWS: rows_fill_lean_kernel (the program is one constant)
+    bool single = false;       // PLAN_ROWS: rows_single_kernel (the program is one function, or one derivative, of source 0)
+    bool single_deriv = false;
+    int single_fun = 0;
     double fill_value = 0;
     int nsrc;
     unsigned grid;
@@ -883,5 +918,6 @@ struct Plan {
 };
 
 template <typename T, int FUNSET> int launch_family(Device* dev, const Plan& plan);
+template <typename T> int launch_single(Device* dev, const Plan& plan);
 
 }  // namespace nk

@@ -421,7 +421,16 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             plan.fill_value = prog.consts[0];
             plan.grid = (unsigned)(row_groups * A.chunks);
         }
-        set_path(plan.lean_fill ? "rows_vec_fill_lean" : plan.lean ? "rows_vec_binary_lean"
+        // ... and of a program that is one function (or one derivative) of its one source: the kernel with that function
+        // compiled in.  Its blocks take two units each, whatever the interpreter family of the program would take.
+        if (plan.kind == PLAN_ROWS && c.nsrc == 1 && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
+            (prog.op[1] == I_FUN || prog.op[1] == I_DFUN) && prog.arg[1] < NK_FUN_COUNT && vec && A.simple_loads && !deep) {
+            plan.single = true;
+            plan.single_deriv = prog.op[1] == I_DFUN;
+            plan.single_fun = prog.arg[1];
+            plan.grid = (unsigned)((row_groups * A.chunks + SINGLE_PASSES - 1) / SINGLE_PASSES);
+        }
+        set_path(plan.single ? "rows_vec_single" : plan.lean_fill ? "rows_vec_fill_lean" : plan.lean ? "rows_vec_binary_lean"
                            : plan.kind == PLAN_ROWS_BINARY ? (periodic ? "rows_vec_binary_periodic" : vec ? "rows_vec_binary" : "rows_binary")
                            : periodic ? (vec ? "rows_vec_periodic" : "rows_periodic") : vec ? "rows_vec" : "rows");
         done = true;
@@ -497,6 +506,7 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
         plan.grid = grid_for(dev, (cn.n + 255) / 256);
         set_path("canon");
     }
+    if (plan.single) return launch_single<T>(dev, plan);
     switch (funset) {
         case 0: return launch_family<T, 0>(dev, plan);
         case 1: return launch_family<T, 1>(dev, plan);

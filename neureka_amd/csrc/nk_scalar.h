@@ -419,12 +419,15 @@ __device__ __forceinline__ void apply_fun(int id, T (&a)[V]) {
 }
 
 // does function `id` need the full table?
-inline bool fun_is_heavy(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN || id == NK_FUN_LOG10 || id == NK_FUN_CBRT || id == NK_FUN_SOFTPLUS; }
+constexpr bool fun_is_heavy(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN || id == NK_FUN_LOG10 || id == NK_FUN_CBRT || id == NK_FUN_SOFTPLUS; }
 
-template <typename T, int V>
+// derivatives that call a double-precision routine of the device library (registers: evaluated one element at a time)
+constexpr bool dfun_calls_library(int id) { return id == NK_FUN_COS || id == NK_FUN_SIN || id == NK_FUN_CBRT || id == NK_FUN_GASU || id == NK_FUN_GATU; }
+
+template <typename T, int V, bool ONE_BY_ONE = true>
 __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
     using N = Num<T>;
-    constexpr bool NK_ONE_BY_ONE = true;
+    constexpr bool NK_ONE_BY_ONE = ONE_BY_ONE;
     switch (id) {
         case NK_FUN_ABS: NK_EACH(x < T(0) ? T(-1) : T(1));
         case NK_FUN_COS: NK_EACH(T(-::sin((double)x)));
