@@ -482,6 +482,42 @@ __global__ __launch_bounds__(256) void rows_single_kernel(RowsArgs A, T* __restr
     }
 }
 
+// drain = src0 op b, or a partial derivative of it, for ONE heavy operator known at compile time (modulo, power, and
+// the derivatives of division, modulo and power -- the operators the four-operator kernel below does not carry); b is
+// source 1 or a constant (scalarization).  Same data path as rows_single_kernel.
+// KIND 0: the operator; 1, 2: its derivative by operand 0, 1.
+template <typename T, int V, bool NT, int KIND, int OP, bool CONST_B>
+__global__ __launch_bounds__(256) void rows_pair_kernel(RowsArgs A, T* __restrict__ drn, const T* __restrict__ s0, const T* __restrict__ s1, T k) {
+    T x[SINGLE_PASSES * V], y[SINGLE_PASSES * V];
+    int doff[SINGLE_PASSES];
+    bool live[SINGLE_PASSES];
+#pragma unroll
+    for (int p = 0; p < SINGLE_PASSES; p++) {
+        unsigned rg, chunk;
+        rows_unit(A, SINGLE_PASSES, p, rg, chunk);
+        const RowsAddr<3> R = rows_address<3>(A, rg, chunk);
+        live[p] = R.live;
+        doff[p] = R.off[0] + (int)R.col;
+        T (&xp)[V] = *reinterpret_cast<T (*)[V]>(&x[p * V]);
+        T (&yp)[V] = *reinterpret_cast<T (*)[V]>(&y[p * V]);
+        load_vec<T, V, NT>(xp, s0 + R.off[1] + R.col);
+        if constexpr (CONST_B) {
+#pragma unroll
+            for (int v = 0; v < V; v++) yp[v] = k;
+        } else load_vec<T, V, NT>(yp, s1 + R.off[2] + R.col);
+    }
+    constexpr bool ONE = sizeof(T) == 8;       // the double-precision library routines: one element at a time (registers)
+    if constexpr (KIND == 0) apply_bin<T, SINGLE_PASSES * V, 2, ONE>(OP, x, y);
+    else apply_dbin<T, SINGLE_PASSES * V, 2, ONE>(OP, KIND - 1, x, y);
+#pragma unroll
+    for (int p = 0; p < SINGLE_PASSES; p++) {
+        if (live[p]) {
+            T (&op)[V] = *reinterpret_cast<T (*)[V]>(&x[p * V]);
+            store_vec<T, V>(drn + doff[p], op);
+        }
+    }
+}
+
 // drain = src0 op src1 with op in {+, -, *, /} and plain aligned loads: the bandwidth-critical case
 // (same-shape elementwise and forward broadcast).  The operator is resolved once, outside the passes,
 // and each pass is stored as soon as its operands have arrived.
@@ -904,6 +940,10 @@ struct Plan {
     bool single = false;       // PLAN_ROWS: rows_single_kernel (the program is one function, or one derivative, of source 0)
     bool single_deriv = false;
     int single_fun = 0;
+    int pair_kind = -1;        // PLAN_ROWS: rows_pair_kernel (one heavy operator of source 0 and source 1 or a constant): 0 the
+    int pair_op = 0;           // operator, 1 / 2 its derivative by operand 0 / 1
+    bool pair_const = false;
+    double pair_value = 0;
     double fill_value = 0;
     int nsrc;
     unsigned grid;

@@ -430,7 +430,21 @@ static int launch_typed(Device* dev, const EltCall& c, const Prog& prog) {
             plan.single_fun = prog.arg[1];
             plan.grid = (unsigned)((row_groups * A.chunks + SINGLE_PASSES - 1) / SINGLE_PASSES);
         }
-        set_path(plan.single ? "rows_vec_single" : plan.lean_fill ? "rows_vec_fill_lean" : plan.lean ? "rows_vec_binary_lean"
+        // ... and of one heavy operator (or its derivative) of source 0 and either source 1 or a constant
+        if (plan.kind == PLAN_ROWS && (c.nsrc == 1 || c.nsrc == 2) && prog.n == 2 && prog.op[0] == I_SET && prog.src[0] == 0 &&
+            (prog.op[1] == I_BIN || prog.op[1] == I_DBIN) && vec && A.simple_loads && !deep &&
+            (prog.src[1] == SRC_CONST0 || (prog.src[1] == 1 && c.nsrc == 2)) && (prog.src[1] == 1) == (c.nsrc == 2)) {
+            const int op = prog.op[1] == I_BIN ? prog.arg[1] : prog.arg[1] >> 1;
+            const int kind = prog.op[1] == I_BIN ? 0 : 1 + (prog.arg[1] & 1);
+            if (kind == 0 ? bin_is_heavy(op) : dbin_is_heavy(op)) {
+                plan.single = true;
+                plan.pair_kind = kind; plan.pair_op = op;
+                plan.pair_const = prog.src[1] == SRC_CONST0;
+                plan.pair_value = prog.consts[0];
+                plan.grid = (unsigned)((row_groups * A.chunks + SINGLE_PASSES - 1) / SINGLE_PASSES);
+            }
+        }
+        set_path(plan.single ? (plan.pair_kind >= 0 ? "rows_vec_pair" : "rows_vec_single") : plan.lean_fill ? "rows_vec_fill_lean" : plan.lean ? "rows_vec_binary_lean"
                            : plan.kind == PLAN_ROWS_BINARY ? (periodic ? "rows_vec_binary_periodic" : vec ? "rows_vec_binary" : "rows_binary")
                            : periodic ? (vec ? "rows_vec_periodic" : "rows_periodic") : vec ? "rows_vec" : "rows");
         done = true;

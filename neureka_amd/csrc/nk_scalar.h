@@ -468,10 +468,10 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
     }                                                   \
     break
 
-template <typename T, int V, int FUNSET>
+template <typename T, int V, int FUNSET, bool ONE_BY_ONE = (FUNSET >= 2)>
 __device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
     using N = Num<T>;
-    constexpr bool NK_ONE_BY_ONE = FUNSET >= 2;
+    constexpr bool NK_ONE_BY_ONE = ONE_BY_ONE;
     switch (op) {
         case NK_OP_ADD: NK_EACH2(x + y);
         case NK_OP_SUB: NK_EACH2(x - y);
@@ -488,13 +488,13 @@ __device__ __forceinline__ void apply_bin(int op, T (&a)[V], const T (&b)[V]) {
             } else NK_EACH2(T(NAN) + x + y);
     }
 }
-inline bool bin_is_heavy(int op) { return op == NK_OP_MOD || op == NK_OP_POW; }
+constexpr bool bin_is_heavy(int op) { return op == NK_OP_MOD || op == NK_OP_POW; }
 
 // partial derivatives: CPUBiElementWise*.java (_getDeriveAt0 / _getDeriveAt1).  a = d(a op b)/d(operand d).
-template <typename T, int V, int FUNSET>
+template <typename T, int V, int FUNSET, bool ONE_BY_ONE = (FUNSET >= 2)>
 __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b)[V]) {
     using N = Num<T>;
-    constexpr bool NK_ONE_BY_ONE = FUNSET >= 2;
+    constexpr bool NK_ONE_BY_ONE = ONE_BY_ONE;
     switch (op * 2 + d) {
         case NK_OP_ADD * 2 + 0:
         case NK_OP_ADD * 2 + 1:
@@ -518,7 +518,7 @@ __device__ __forceinline__ void apply_dbin(int op, int d, T (&a)[V], const T (&b
             } else NK_EACH2(T(NAN) + x + y);
     }
 }
-inline bool dbin_is_heavy(int op) { return op == NK_OP_DIV || op == NK_OP_MOD || op == NK_OP_POW; }
+constexpr bool dbin_is_heavy(int op) { return op == NK_OP_DIV || op == NK_OP_MOD || op == NK_OP_POW; }
 #undef NK_EACH2
 
 }  // namespace nk

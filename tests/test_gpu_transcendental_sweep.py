@@ -12,7 +12,7 @@ The worst relative error seen per function is printed."""
 import numpy as np
 import pytest
 
-from neureka_amd import Tensor
+from neureka_amd import Tensor, _lib
 
 pytestmark = pytest.mark.gpu
 
@@ -49,6 +49,7 @@ def test_f32_exp_based_activations_dense_sweep(device, orc):
         for d in (-1, 0):
             print(f"[case] sweep {name} d={d} over {n} points", flush=True)
             device.launch_activation(name, d, out, tx)
+            assert _lib.last_path() == "rows_vec_single", _lib.last_path()
             got = out.getData().astype(np.float64)
             with np.errstate(all="ignore"):
                 want32 = orc.activation(name, d, np.zeros(n, dtype=np.float32), cfg, x, cfg, workers=16)
@@ -100,6 +101,7 @@ def test_f32_power_dense_sweep(device, orc):
     ta, tb = Tensor.of(np.float32, (n,), a).to(device), Tensor.of(np.float32, (n,), b).to(device)
     out = Tensor._on_device(device, np.float32, (n,))
     device.launch_elementwise("power", -1, out, ta, tb)
+    assert _lib.last_path() == "rows_vec_pair", _lib.last_path()        # one heavy operator: compiled in, not interpreted
     got = out.getData().astype(np.float64)
     with np.errstate(all="ignore"):
         want = orc.elementwise("power", -1, np.zeros(n, dtype=np.float32), cfg, a, cfg, b, cfg, workers=16).astype(np.float64)
@@ -171,6 +173,7 @@ def test_backward_and_heavy_kernels_full_size(device, orc):
                                ("log10", -1, tb, b), ("cbrt", -1, tb, b), ("sin", 0, ta, a)):
         print(f"[case] full-size {name} d={d}", flush=True)
         device.launch_activation(name, d, out, src)
+        assert _lib.last_path() == "rows_vec_single", _lib.last_path()      # one function: compiled in, not interpreted
         want = orc.activation(name, d, zeros(), cfg, host, cfg, workers=16)
         if name == "relu":
             assert out.getData().tobytes() == want.tobytes()
@@ -181,6 +184,7 @@ def test_backward_and_heavy_kernels_full_size(device, orc):
         x = tb if op == "power" else ta
         hx = b if op == "power" else a
         device.launch_elementwise(op, d, out, x, tb)
+        assert _lib.last_path() == "rows_vec_pair", _lib.last_path()
         want = orc.elementwise(op, d, zeros(), cfg, hx, cfg, b, cfg, workers=16)
         if op == "modulo":
             assert out.getData().tobytes() == want.tobytes()
