@@ -1134,6 +1134,106 @@ __global__ __launch_bounds__(256) void matmul_few_rows_mfma_kernel(int M, int K,
     }
 }
 
+// The same product where A's rows are whole 16-byte vectors (K a multiple of the vector, A aligned): nothing is staged.
+// A block of eight wavefronts owns 16 x VEC columns and a part of the k range; the wavefronts split that part, each
+// streams its rows of B as above and reads its piece of A straight from memory (one more 16-byte load per lane, group of
+// rows and step: A is a few hundred kilobytes that live in the L2), and they meet once, at the end, in LDS, where the
+// first wavefront adds the eight accumulators in order.  With one part the block writes C itself (MODE 1: C = sum,
+// 2: C += sum) and the product is one launch; with more (MODE 0) the partial rows go to P[part] as before.
+// [16,4096] @ [4096,4096]: 64 column blocks x 4 parts, 16.7 us with the addition of the parts (the staged kernel above:
+// 21.2); one part (64 blocks): 31.5, two: 21.3, eight: 17.2.  32 rows: 22.5 (28.8); f64, 16 rows: 24.7 (31.6).
+constexpr int FEW_NW = 8;
+template <typename T, int RG, int MODE>
+__global__ __launch_bounds__(64 * FEW_NW) void matmul_few_rows_split_kernel(int M, int K, int N, int k_per_part, int col_blocks, const T* __restrict__ A,
+                                                                           const T* __restrict__ B, T* __restrict__ P) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int STEP = 4 * VEC;                                       // k's per step
+    constexpr int AHEAD = 2;                                            // steps whose rows of B are requested together
+    constexpr int PITCH = 16 * VEC + VEC;
+    typedef T Vec __attribute__((ext_vector_type(VEC)));
+    typedef typename Mfma16<T>::Acc Acc;
+    __shared__ __attribute__((aligned(16))) T meet[FEW_NW - 1][RG * 16][PITCH];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int j = lane & 15, q = lane >> 4;
+    const int part = (int)(blockIdx.x / (unsigned)col_blocks), col_block = (int)(blockIdx.x % (unsigned)col_blocks);
+    const int64_t col0 = ((int64_t)col_block * 16 + j) * VEC;           // N % VEC == 0 (the host checks)
+    const bool live = col0 < N;
+    const int k_begin = part * k_per_part;
+    const int k_end = k_begin + k_per_part < K ? k_begin + k_per_part : K;
+    const int steps = (k_end - k_begin + STEP - 1) / STEP;
+    const int per_wave = (steps + FEW_NW - 1) / FEW_NW;
+    const int s_begin = wave * per_wave, s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
+    Acc acc[RG][VEC];
+#pragma unroll
+    for (int g = 0; g < RG; g++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[g][e] = Acc{T(0), T(0), T(0), T(0)};
+    const T* Bc = B + (live ? col0 : 0);
+    Vec b[2][AHEAD][VEC], a[2][AHEAD][RG];
+    auto request = [&](int s, Vec (&bb)[AHEAD][VEC], Vec (&aa)[AHEAD][RG]) {
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++) {
+            const int k0 = k_begin + (s + u) * STEP + VEC * q;          // this lane's k's of step s + u: k0 ... k0 + VEC - 1
+            const bool step_live = s + u < s_end;
+#pragma unroll
+            for (int r = 0; r < VEC; r++)
+                bb[u][r] = (live && step_live && k0 + r < k_end) ? *(const Vec*)(Bc + (int64_t)(k0 + r) * N) : Vec(T(0));
+#pragma unroll
+            for (int g = 0; g < RG; g++)                                // (k0 < k_end: the whole vector is, K being a multiple of VEC)
+                aa[u][g] = (16 * g + j < M && step_live && k0 < k_end) ? *(const Vec*)(A + (int64_t)(16 * g + j) * K + k0) : Vec(T(0));
+        }
+    };
+    auto multiply = [&](const Vec (&bb)[AHEAD][VEC], const Vec (&aa)[AHEAD][RG]) {
+#pragma unroll
+        for (int u = 0; u < AHEAD; u++)
+#pragma unroll
+            for (int g = 0; g < RG; g++)
+#pragma unroll
+                for (int r = 0; r < VEC; r++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) acc[g][e] = Mfma16<T>::mma(aa[u][g][r], bb[u][r][e], acc[g][e]);
+    };
+    // two sets of registers: the next AHEAD steps are on their way while these are multiplied in ([16,4096] @ [4096,4096]:
+    // 16.7 us; four steps at a time in one set 17.0, eight 17.7, four in two sets 19.0)
+    request(s_begin, b[0], a[0]);
+    for (int s = s_begin; s < s_end; s += 2 * AHEAD) {
+        request(s + AHEAD, b[1], a[1]);
+        multiply(b[0], a[0]);
+        request(s + 2 * AHEAD, b[0], a[0]);
+        multiply(b[1], a[1]);
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int g = 0; g < RG; g++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                Vec out;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) out[e] = acc[g][e][v];
+                *(Vec*)&meet[wave - 1][16 * g + Mfma16<T>::row_of(q, v)][j * VEC] = out;
+            }
+    }
+    __syncthreads();
+    if (wave == 0 && live) {
+        T* Pp = P + (MODE == 0 ? (int64_t)part * M * N : (int64_t)0) + col0;
+#pragma unroll
+        for (int g = 0; g < RG; g++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = 16 * g + Mfma16<T>::row_of(q, v);
+                if (row < M) {
+                    Vec sum;
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) sum[e] = acc[g][e][v];
+#pragma unroll
+                    for (int w = 0; w < FEW_NW - 1; w++) sum = sum + *(const Vec*)&meet[w][row][j * VEC];     // wavefronts in order
+                    Vec* dst = (Vec*)(Pp + (int64_t)row * N);
+                    *dst = MODE == 2 ? *dst + sum : sum;
+                }
+            }
+    }
+}
+
 // ---- a short inner dimension ------------------------------------------------------------------------------------
 // C[M,N] (+)= A[M,K] @ B[K,N] with K <= 16 (the gradient of a weight matrix from a small batch: a sum of K outer
 // products): the product writes C once and is bound by that stream.  A thread owns 16 bytes of columns and keeps its
@@ -1426,6 +1526,40 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             int k_per_part = (int)((K + parts - 1) / parts);
             const int mr = M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : M <= 16 ? 16 : 32;
             const bool on_matrix_cores = M > 4;                         // 5 ... 32 rows: 16 x 16 x 4 matrix instructions
+            // ... whose wavefronts split the k range inside the block where A's rows are whole vectors: blocks of 16 x vec
+            // columns, as many parts as fill the compute units, none shorter than two rounds of requests per wavefront
+            if (on_matrix_cores && K % vec == 0 && A % 16 == 0 && N >= 16 * vec) {
+                const int64_t blocks_n = (N + 16 * vec - 1) / (16 * vec);
+                int64_t split = (int64_t)dev->props.multiProcessorCount / blocks_n;
+                const int64_t shortest = (int64_t)FEW_NW * 4 * vec * 8;          // eight steps per wavefront
+                if (split > K / shortest) split = K / shortest;
+                if (split < 1) split = 1;
+                int kpp = (int)((K + split - 1) / split);
+                kpp = (kpp + 4 * vec - 1) / (4 * vec) * (4 * vec);                          // whole steps
+                split = (K + kpp - 1) / kpp;
+                void* wsp = nullptr;
+                if (split > 1 && (uint64_t)split * M * N * eb > ((uint64_t)1 << 30)) split = 0;     // (to the kernels below)
+                if (split > 1) if (int e = workspace(dev, (uint64_t)split * M * N * eb, &wsp)) return e;
+                if (split >= 1) {
+                    const dim3 grid((unsigned)(blocks_n * split));
+                    auto go = [&](auto t, auto groups_tag) {
+                        using T = decltype(t);
+                        constexpr int RG = decltype(groups_tag)::value;
+                        if (split == 1) {
+                            if (g.overwrite) hipLaunchKernelGGL((matmul_few_rows_split_kernel<T, RG, 1>), grid, dim3(64 * FEW_NW), 0, dev->stream, (int)M, (int)K, (int)N, kpp, (int)blocks_n, (const T*)A, (const T*)B, (T*)C);
+                            else             hipLaunchKernelGGL((matmul_few_rows_split_kernel<T, RG, 2>), grid, dim3(64 * FEW_NW), 0, dev->stream, (int)M, (int)K, (int)N, kpp, (int)blocks_n, (const T*)A, (const T*)B, (T*)C);
+                        } else {
+                            hipLaunchKernelGGL((matmul_few_rows_split_kernel<T, RG, 0>), grid, dim3(64 * FEW_NW), 0, dev->stream, (int)M, (int)K, (int)N, kpp, (int)blocks_n, (const T*)A, (const T*)B, (T*)wsp);
+                            hipLaunchKernelGGL(matmul_add_parts_kernel<T>, dim3((unsigned)((M * N + 255) / 256)), dim3(256), 0, dev->stream, M * N, (int)split, g.overwrite, (const T*)wsp, (T*)C);
+                        }
+                    };
+                    auto by_groups = [&](auto t) { if (M <= 16) go(t, std::integral_constant<int, 1>{}); else go(t, std::integral_constant<int, 2>{}); };
+                    if (dtype == NK_F64) by_groups(double{}); else by_groups(float{});
+                    NK_HIP(hipGetLastError());
+                    set_path(dtype == NK_F64 ? "few_rows_f64" : "few_rows");
+                    return NK_OK;
+                }
+            }
             const int staged = on_matrix_cores ? 256 : few_kp(mr);
             if (k_per_part > staged) k_per_part = staged;               // what a block stages of A
             parts = (K + k_per_part - 1) / k_per_part;
