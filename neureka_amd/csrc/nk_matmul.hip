@@ -1237,7 +1237,7 @@ __global__ __launch_bounds__(64 * FEW_NW) void matmul_few_rows_split_kernel(int 
 // ---- a short inner dimension ------------------------------------------------------------------------------------
 // C[M,N] (+)= A[M,K] @ B[K,N] with K <= 16 (the gradient of a weight matrix from a small batch: a sum of K outer
 // products): the product writes C once and is bound by that stream.  A thread owns 16 bytes of columns and keeps its
-// K x 16 bytes of B in registers; a block walks FEW_RB rows of A, staged in LDS (zero-padded to KC), and writes one
+// K x 16 bytes of B in registers; a block walks FEW_RB rows of A, staged in LDS (padded to KC with -0), and writes one
 // row of its 256 x 16 bytes of columns per step -- four contiguous kilobytes.
 constexpr int FEW_RB = 32;
 template <typename T, int KC, bool OVERWRITE>
@@ -1254,7 +1254,7 @@ __global__ __launch_bounds__(256) void matmul_short_inner_kernel(int M, int K, i
     const bool live = col0 < N;
     for (int i = threadIdx.x; i < FEW_RB * KC; i += 256) {
         const int r = i / KC, k = i % KC;
-        As[r][k] = (k < K && row0 + r < M) ? A[(row0 + r) * K + k] : T(0);
+        As[r][k] = (k < K && row0 + r < M) ? A[(row0 + r) * K + k] : T(-0.0);     // the padding: products of -0, see below
     }
     Vec b[KC];
 #pragma unroll
@@ -1274,18 +1274,17 @@ __global__ __launch_bounds__(256) void matmul_short_inner_kernel(int M, int K, i
         for (int u = 0; u < RU; u++) {
             if (r0 + u < rows) {
                 // the reference's own order and rounding (GEMM.java:282-304): the old value, then one rounded product after the
-                // other in k order -- the same bits as the simple kernel gives, wherever the operands happen to lie.  (The
-                // stream over C bounds this kernel; the second instruction per term costs nothing.)
+                // other in k order -- the same bits as the simple kernel gives, wherever the operands happen to lie.  The terms
+                // beyond K are (-0) x (+0) = -0, and adding -0 changes no float, a zero of either sign included: the loop needs
+                // no test on k (with one, sixteen scalar branches per row: 24.9 against 14 us for [4096,16] @ [16,4096]).
                 Vec acc = OVERWRITE ? Vec(T(0)) : old[u];
 #pragma unroll
                 for (int q = 0; q < KC; q += 4) {
                     const Quad a = *(const Quad*)&As[r0 + u][q];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
-                        if (q + j < K) {
 #pragma unroll
-                            for (int e = 0; e < VEC; e++) { const T prod = a[j] * b[q + j][e]; acc[e] = acc[e] + prod; }
-                        }
+                        for (int e = 0; e < VEC; e++) { const T prod = a[j] * b[q + j][e]; acc[e] = acc[e] + prod; }
                 }
                 *(Vec*)(Cp + (int64_t)(r0 + u) * N) = acc;
             }
