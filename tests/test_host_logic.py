@@ -292,3 +292,23 @@ def test_assignment_parses_and_nests_to_the_right():
     assert repr(Function.of("I[0] <- (I[0] * -3)").root) == "(I[0] left_inline (I[0] multiply (-1.0 multiply 3.0)))"
     assert repr(Function.of("I[2]<-I[0]<-I[1]").root) == "(I[2] left_inline (I[0] left_inline I[1]))"
     assert repr(Function.of("I[0] <- I[1] + I[2]").root) == "(I[0] left_inline (I[1] add I[2]))"
+
+
+def test_the_counted_traffic_record_belongs_to_the_sources_in_the_tree():
+    """bench.py reports `roofline.traffic` from profiles/rows_binary_lean_kernel_broadcast_c2.json only while the digest
+    in that record is the digest of the headline kernel's sources: a change to those sources without a new counter run
+    fails here, not silently in the driver's bench line."""
+    import json
+    import os
+    from neureka_amd.profile_summary import HEADLINE_PATH, kernel_sources_digest
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with open(os.path.join(root, "profiles", "rows_binary_lean_kernel_broadcast_c2.json")) as f:
+        rec = json.load(f)
+    assert rec["path"] == HEADLINE_PATH
+    assert rec["sources_sha256"] == kernel_sources_digest(), "the headline kernel's sources changed: regenerate profiles/ (neureka_amd/profile_summary.py)"
+    algorithmic = 4 * (1024 * 2048 * 512 + 1024 * 512 + 2048 * 512)
+    assert algorithmic <= rec["traffic_bytes"] <= 1.05 * algorithmic
+    import bench
+    traffic, note = bench.counted_traffic(HEADLINE_PATH)
+    assert traffic == rec["traffic_bytes"] and "FETCH_SIZE" in note
+    assert bench.counted_traffic("some_other_plan")[0] is None
