@@ -73,11 +73,94 @@ __device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int bid, int& t
     tn = in_grp / rows;
 }
 
-// operands of one depth-8 chunk of a k-slice for the wave's 64x64 sub-tile
-struct Frag {
-    f32x4 a0, a1;          // rows wm + l32 and wm + 32 + l32, k = 8c + 4h .. + 3
-    float b0[4], b1[4];    // columns wn + l32 and wn + 32 + l32, same k
+// ---- what the f32 tile kernels share ---------------------------------------------------------------------------------
+// A block of 256 threads stages one k-slice (depth BK = 32) of a TM x TN tile -- A as TM rows of BK floats, B as BK rows
+// of TN floats, N_STAGED 16-byte pieces of each per thread -- through registers into LDS; a wavefront owns RI x RJ tiles
+// of 32 x 32 and reads the operands of a chunk of depth 8 as RI 16-byte pieces of A and RJ x 4 floats of B.  Lane half h
+// owns k = 8c + 4h ... + 3 of chunk c; the four multiply-adds of a chunk pair (k, k + 4): any pairing works as long as A
+// and B use the same one.  Row pitches in LDS keep every row 16-byte aligned and the operand reads free of bank conflicts.
+// The kernels differ in their pipelines (how far ahead a slice is requested, where the barrier sits, the pinned order
+// of issue), not in any of this.  (matmul_mfma64_kernel, whose order of issue is left to the compiler, keeps its own copy
+// of the staging: through this helper the compiler's schedule changed and 1024^3 ran 3 % slower.)
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+template <int TM, int TN, int RI, int RJ>
+struct TileF32 {
+    static_assert(TM == TN, "one thread stages as many pieces of A as of B");
+    static constexpr int A_P = BK + 4, B_P = TN + 4;
+    static constexpr int N_STAGED = TM * BK / 1024;
+    static constexpr int B_STEP = 1024 / TN;                 // rows of B between two pieces of one thread
+    static constexpr int A_FLOATS = TM * A_P, B_FLOATS = BK * B_P;
+    struct Staged { f32x4 a[N_STAGED], b[N_STAGED]; };
+    struct Frag {
+        f32x4 a[RI];           // rows wm + 32 i + l32, k = 8c + 4h .. + 3
+        float b[RJ][4];        // [j][t]: column wn + 32 j + l32, k = 8c + 4h + t
+    };
+    int a_row, a_col, b_row, b_col;      // a thread's pieces: rows a_row + 32 i of A, rows b_row + B_STEP i of B
+    __device__ __forceinline__ explicit TileF32(int tid) : a_row(tid >> 3), a_col((tid & 7) * 4), b_row(tid / (TN / 4)), b_col((tid % (TN / 4)) * 4) {}
+    // whole tiles: Ag = the tile's first row of A, Bg = its first column of B
+    __device__ __forceinline__ void request(Staged& s, const float* Ag, const float* Bg, int K, int N, int k0) const {
+#pragma unroll
+        for (int i = 0; i < N_STAGED; i++) {
+            s.a[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * K + k0 + a_col);
+            s.b[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + B_STEP * i) * N + b_col);
+        }
+    }
+    // any shape: through buffer descriptors over the whole matrices (nothing past their end is touched, the range check
+    // returns 0 there); rows past the edge and k rows past the end are clamped, columns past the edge left as they come:
+    // all of these only feed results that are not stored, once zero_tail has cleared the k tail
+    __device__ __forceinline__ void request_edge(Staged& s, __amdgpu_buffer_rsrc_t Abuf, __amdgpu_buffer_rsrc_t Bbuf, int M, int K, int N,
+                                                 int row0, int col0, int k0) const {
+#pragma unroll
+        for (int i = 0; i < N_STAGED; i++) {
+            int row = row0 + a_row + 32 * i; if (row > M - 1) row = M - 1;
+            s.a[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * K + k0 + a_col) * 4u, 0, 0)));
+            const int kb = k0 + b_row + B_STEP * i;
+            const int krow = kb < K ? kb : K - 1;
+            s.b[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * N + col0 + b_col) * 4u, 0, 0)));
+        }
+    }
+    __device__ __forceinline__ void zero_tail(Staged& s, int K, int k0) const {
+#pragma unroll
+        for (int i = 0; i < N_STAGED; i++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (k0 + a_col + e >= K) s.a[i][e] = 0.0f;
+            if (k0 + b_row + B_STEP * i >= K) s.b[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    __device__ __forceinline__ void store(const Staged& s, float* as, float* bs) const {
+#pragma unroll
+        for (int i = 0; i < N_STAGED; i++) {
+            *(f32x4*)(&as[(a_row + 32 * i) * A_P + a_col]) = s.a[i];
+            *(f32x4*)(&bs[(b_row + B_STEP * i) * B_P + b_col]) = s.b[i];
+        }
+    }
+    static __device__ __forceinline__ void read(Frag& f, const float* as, const float* bs, int wm, int wn, int l32, int h, int c) {
+#pragma unroll
+        for (int i = 0; i < RI; i++) f.a[i] = *(const f32x4*)(&as[(wm + 32 * i + l32) * A_P + 8 * c + 4 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int j = 0; j < RJ; j++) f.b[j][t] = bs[(8 * c + 4 * h + t) * B_P + wn + 32 * j + l32];
+    }
+    static __device__ __forceinline__ void clear(f32x16 (&acc)[RI][RJ]) {
+#pragma unroll
+        for (int i = 0; i < RI; i++)
+#pragma unroll
+            for (int j = 0; j < RJ; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    }
+    static __device__ __forceinline__ void mma(f32x16 (&acc)[RI][RJ], const Frag& f) {
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int i = 0; i < RI; i++)
+#pragma unroll
+                for (int j = 0; j < RJ; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][t], f.b[j][t], acc[i][j], 0, 0, 0);
+    }
 };
+using Tile128 = TileF32<BM, BN, 2, 2>;       // matmul_mfma_kernel, matmul_mfma_stream_kernel: 64 x 64 per wavefront
+static_assert(Tile128::A_P == A_PITCH && Tile128::B_P == B_PITCH, "one LDS layout");
 
 constexpr int C_PITCH = BN + 4;
 constexpr int LDS_FLOATS_AB = 2 * BM * A_PITCH + 2 * BK * B_PITCH;
@@ -109,72 +192,20 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     const float* Ag = A + (int64_t)tm * BM * g.K;
     const float* Bg = B + (int64_t)tn * BN;
 
-    // global -> register staging: A slice 128x32, B slice 32x128, 4 float4 each per thread
-    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32*i
-    const int b_row = tid >> 5, b_col = (tid & 31) * 4;     // rows b_row + 8*i
-    f32x4 ra[4], rb[4];
-
-    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    const Tile128 tile(tid);
+    Tile128::Staged staged;
     const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 4), 0x00020000);
     auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            if (!EDGE) {
-                ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-                rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 8 * i) * g.N + b_col);
-            } else {
-                int row = tm * BM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
-                const int ka = k0 + a_col;
-                ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * g.K + ka) * 4u, 0, 0)));
-#pragma unroll
-                for (int e = 0; e < 4; e++) if (ka + e >= g.K) ra[i][e] = 0.0f;
-                const int kb = k0 + b_row + 8 * i;
-                const int krow = kb < g.K ? kb : g.K - 1;
-                rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * g.N + tn * BN + b_col) * 4u, 0, 0)));
-                if (kb >= g.K) rb[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            }
-        }
+        if (!EDGE) tile.request(staged, Ag, Bg, g.K, g.N, k0);
+        else { tile.request_edge(staged, Abuf, Bbuf, g.M, g.K, g.N, tm * BM, tn * BN, k0); tile.zero_tail(staged, g.K, k0); }
     };
-    auto store_lds = [&](int buf) {
-        float* as = As0 + buf * (BM * A_PITCH);
-        float* bs = Bs0 + buf * (BK * B_PITCH);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *(f32x4*)(&as[(a_row + 32 * i) * A_PITCH + a_col]) = ra[i];
-            *(f32x4*)(&bs[(b_row + 8 * i) * B_PITCH + b_col]) = rb[i];
-        }
-    };
-    // lane half h owns k = 8c + 4h .. 8c + 4h + 3 of chunk c; the four MFMA steps pair (k, k + 4):
-    // any pairing works as long as A and B use the same one
-    auto read_frag = [&](Frag& f, int buf, int c) {
-        const float* as = As0 + buf * (BM * A_PITCH);
-        const float* bs = Bs0 + buf * (BK * B_PITCH);
-        f.a0 = *(const f32x4*)(&as[(wm + l32) * A_PITCH + 8 * c + 4 * h]);
-        f.a1 = *(const f32x4*)(&as[(wm + 32 + l32) * A_PITCH + 8 * c + 4 * h]);
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            f.b0[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + l32];
-            f.b1[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + 32 + l32];
-        }
-    };
-
+    auto store_lds = [&](int buf) { tile.store(staged, As0 + buf * Tile128::A_FLOATS, Bs0 + buf * Tile128::B_FLOATS); };
+    using Frag = Tile128::Frag;
+    auto read_frag = [&](Frag& f, int buf, int c) { Tile128::read(f, As0 + buf * Tile128::A_FLOATS, Bs0 + buf * Tile128::B_FLOATS, wm, wn, l32, h, c); };
     f32x16 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-    auto mma = [&](const Frag& f) {
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b0[t], acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b1[t], acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b0[t], acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b1[t], acc[1][1], 0, 0, 0);
-        }
-    };
+    Tile128::clear(acc);
+    auto mma = [&](const Frag& f) { Tile128::mma(acc, f); };
 
     // Software pipeline over the k-slices.  While the matrix cores work on chunk c of the current slice the
     // operands of chunk c + 1 are read from LDS; the next slice (fetched from global memory at the top of
@@ -421,56 +452,15 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
     const int l32 = lane & 31, h = lane >> 5;
-    const int a_row = tid >> 3, a_col = (tid & 7) * 4;
-    const int b_row = tid >> 5, b_col = (tid & 31) * 4;
-    f32x4 ra[4], rb[4];
-    auto load_global = [&](int tm, int tn, int k0) {
-        const float* Ag = A + (int64_t)tm * BM * g.K;
-        const float* Bg = B + (int64_t)tn * BN;
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 8 * i) * g.N + b_col);
-        }
-    };
-    auto store_lds = [&](int buf) {
-        float* as = As0 + buf * (BM * A_PITCH);
-        float* bs = Bs0 + buf * (BK * B_PITCH);
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *(f32x4*)(&as[(a_row + 32 * i) * A_PITCH + a_col]) = ra[i];
-            *(f32x4*)(&bs[(b_row + 8 * i) * B_PITCH + b_col]) = rb[i];
-        }
-    };
-    auto read_frag = [&](Frag& f, int buf, int c) {
-        const float* as = As0 + buf * (BM * A_PITCH);
-        const float* bs = Bs0 + buf * (BK * B_PITCH);
-        f.a0 = *(const f32x4*)(&as[(wm + l32) * A_PITCH + 8 * c + 4 * h]);
-        f.a1 = *(const f32x4*)(&as[(wm + 32 + l32) * A_PITCH + 8 * c + 4 * h]);
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            f.b0[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + l32];
-            f.b1[t] = bs[(8 * c + 4 * h + t) * B_PITCH + wn + 32 + l32];
-        }
-    };
+    const Tile128 stage(tid);
+    Tile128::Staged staged;
+    auto load_global = [&](int tm, int tn, int k0) { stage.request(staged, A + (int64_t)tm * BM * g.K, B + (int64_t)tn * BN, g.K, g.N, k0); };
+    auto store_lds = [&](int buf) { stage.store(staged, As0 + buf * Tile128::A_FLOATS, Bs0 + buf * Tile128::B_FLOATS); };
+    using Frag = Tile128::Frag;
+    auto read_frag = [&](Frag& f, int buf, int c) { Tile128::read(f, As0 + buf * Tile128::A_FLOATS, Bs0 + buf * Tile128::B_FLOATS, wm, wn, l32, h, c); };
     f32x16 acc[2][2];
-    auto clear = [&]() {
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-    };
-    auto mma = [&](const Frag& f) {
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b0[t], acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a0[t], f.b1[t], acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b0[t], acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a1[t], f.b1[t], acc[1][1], 0, 0, 0);
-        }
-    };
+    auto clear = [&]() { Tile128::clear(acc); };
+    auto mma = [&](const Frag& f) { Tile128::mma(acc, f); };
     static_assert(BK == 32, "the pipeline below is written for four depth-8 chunks per slice");
     const int nk = g.K / BK;
 
@@ -558,12 +548,9 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
 // A 256 x 36 and B 32 x 260 floats, 137 KiB (dynamic).
 namespace big {
 constexpr int TM = 256, TN = 256;
-constexpr int AP = BK + 4, BP = TN + 4;
-constexpr int LDS_FLOATS = 2 * TM * AP + 2 * BK * BP;
-struct BigFrag {
-    f32x4 a[4];            // rows wm + 32 i + l32, k = 8c + 4h .. + 3
-    float b[4][4];         // [j][t]: column wn + 32 j + l32, k = 8c + 4h + t
-};
+using Tile = TileF32<TM, TN, 4, 4>;                      // 128 x 128 per wavefront
+constexpr int LDS_FLOATS = 2 * Tile::A_FLOATS + 2 * Tile::B_FLOATS;
+using BigFrag = Tile::Frag;
 }
 
 // EDGE: M, N, K need not be multiples of the tile -- as in matmul_mfma_kernel<true>: loads through buffer descriptors
@@ -574,8 +561,8 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
                                                                 const float* __restrict__ B, float* __restrict__ C) {
     using namespace big;
     extern __shared__ __attribute__((aligned(16))) float big_lds[];
-    float* const As0 = big_lds;                            // [2][TM * AP]
-    float* const Bs0 = big_lds + 2 * TM * AP;              // [2][BK * BP]
+    float* const As0 = big_lds;                            // [2][Tile::A_FLOATS]
+    float* const Bs0 = big_lds + 2 * Tile::A_FLOATS;       // [2][Tile::B_FLOATS]
     int tm, tn;
     tile_of_block(g, (int)blockIdx.x, tm, tn);
     const int tid = threadIdx.x;
@@ -584,73 +571,24 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
     const int l32 = lane & 31, h = lane >> 5;
     const float* Ag = A + (int64_t)tm * TM * g.K;
     const float* Bg = B + (int64_t)tn * TN;
-    // global -> register staging: A slice 256x32 and B slice 32x256, 8 float4 each per thread
-    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 i
-    const int b_row = tid >> 6, b_col = (tid & 63) * 4;     // rows b_row + 4 i
-    f32x4 ra[8], rb[8];
-    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    const Tile tile(tid);
+    Tile::Staged staged;
     const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 4), 0x00020000);
     const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 4), 0x00020000);
     auto load_global = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            if (!EDGE) {
-                ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-                rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 4 * i) * g.N + b_col);
-            } else {
-                int row = tm * TM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
-                const int ka = k0 + a_col;
-                ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * g.K + ka) * 4u, 0, 0)));
-                const int kb = k0 + b_row + 4 * i;
-                const int krow = kb < g.K ? kb : g.K - 1;
-                rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * g.N + tn * TN + b_col) * 4u, 0, 0)));
-            }
-        }
+        if (!EDGE) tile.request(staged, Ag, Bg, g.K, g.N, k0);
+        else tile.request_edge(staged, Abuf, Bbuf, g.M, g.K, g.N, tm * TM, tn * TN, k0);
     };
     // k0: the slice the staging registers hold.  The k tail is zeroed here, a slice after the request, and only in the
     // one slice that has a tail (a block-uniform branch): zeroing at the request would make every slice wait for its loads.
     auto store_lds = [&](int buf, int k0) {
-        float* as = As0 + buf * (TM * AP);
-        float* bs = Bs0 + buf * (BK * BP);
-        if (EDGE && k0 + BK > g.K) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-#pragma unroll
-                for (int e = 0; e < 4; e++) if (k0 + a_col + e >= g.K) ra[i][e] = 0.0f;
-                if (k0 + b_row + 4 * i >= g.K) rb[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            *(f32x4*)(&as[(a_row + 32 * i) * AP + a_col]) = ra[i];
-            *(f32x4*)(&bs[(b_row + 4 * i) * BP + b_col]) = rb[i];
-        }
+        if (EDGE && k0 + BK > g.K) tile.zero_tail(staged, g.K, k0);
+        tile.store(staged, As0 + buf * Tile::A_FLOATS, Bs0 + buf * Tile::B_FLOATS);
     };
-    auto read_frag = [&](BigFrag& f, int buf, int c) {
-        const float* as = As0 + buf * (TM * AP);
-        const float* bs = Bs0 + buf * (BK * BP);
-#pragma unroll
-        for (int i = 0; i < 4; i++) f.a[i] = *(const f32x4*)(&as[(wm + 32 * i + l32) * AP + 8 * c + 4 * h]);
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int t = 0; t < 4; t++) f.b[j][t] = bs[(8 * c + 4 * h + t) * BP + wn + 32 * j + l32];
-    };
+    auto read_frag = [&](BigFrag& f, int buf, int c) { Tile::read(f, As0 + buf * Tile::A_FLOATS, Bs0 + buf * Tile::B_FLOATS, wm, wn, l32, h, c); };
     f32x16 acc[4][4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < 4; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
-    auto mma = [&](const BigFrag& f) {
-#pragma unroll
-        for (int t = 0; t < 4; t++)
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(f.a[i][t], f.b[j][t], acc[i][j], 0, 0, 0);
-    };
+    Tile::clear(acc);
+    auto mma = [&](const BigFrag& f) { Tile::mma(acc, f); };
     // The pipeline of matmul_mfma_kernel with chunks of 64 multiply-adds: the 20 LDS reads of chunk c + 1 follow the
     // first ten multiply-adds of chunk c in pairs; in the third chunk each of the next sixteen multiply-adds is
     // followed by one LDS write of the staged slice kt + 1 and one global request for slice kt + 2.
