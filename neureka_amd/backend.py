@@ -50,15 +50,15 @@ class ExecutionCall:
     def withInputAt(self, i: int, t) -> "ExecutionCall":
         inputs = list(self.inputs)
         inputs[i] = t
-        return replace(self, inputs=inputs)
+        return ExecutionCall(self.device, self.operation, inputs, self.derivIdx, self.algorithm)
 
     def withAddedInputAt(self, i: int, t) -> "ExecutionCall":
         inputs = list(self.inputs)
         inputs.insert(i, t)
-        return replace(self, inputs=inputs)
+        return ExecutionCall(self.device, self.operation, inputs, self.derivIdx, self.algorithm)
 
     def withInputs(self, inputs: Sequence) -> "ExecutionCall":
-        return replace(self, inputs=list(inputs))
+        return ExecutionCall(self.device, self.operation, list(inputs), self.derivIdx, self.algorithm)
 
 
 class Algorithm:

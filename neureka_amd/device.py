@@ -20,7 +20,13 @@ from .ndim import IllegalArgumentException, IllegalStateException, NDConfigurati
 _INT_CODES = {np.dtype(np.int32): 2, np.dtype(np.int64): 3, np.dtype(np.int16): 4, np.dtype(np.int8): 5}
 
 
+_FLOAT_CODES = {np.float32: _lib.F32, np.float64: _lib.F64, np.dtype(np.float32): _lib.F32, np.dtype(np.float64): _lib.F64}
+
+
 def _dtype_code(dtype) -> int:
+    code = _FLOAT_CODES.get(dtype)
+    if code is not None:
+        return code
     dt = np.dtype(dtype)
     if dt == np.float32:
         return _lib.F32
@@ -347,12 +353,13 @@ class HipDevice:
     @staticmethod
     def _ops(*tensors):
         out = []
-        if len({t.rank for t in tensors}) > 1:
-            raise IllegalArgumentException(f"operands of one kernel must have one rank, got {[t.rank for t in tensors]}")
+        rank = len(tensors[0].ndc.shape)
         for t in tensors:
+            if len(t.ndc.shape) != rank:
+                raise IllegalArgumentException(f"operands of one kernel must have one rank, got {[t.rank for t in tensors]}")
             # a virtual tensor keeps one element on the device and is addressed through all-zero tables
-            inline = (NDConfiguration.virtualOf(t.shape) if t.isVirtual() else t.ndc).asInlineArray()
-            out.append((C.c_uint64(t._data.ptr), inline, _lib.cfg_ptr(inline)))
+            inline, pointer = (NDConfiguration.virtualOf(t.shape) if t._virtual else t.ndc).inlineArguments()
+            out.append((t._data.ptr, inline, pointer))
         return out
 
     def launch_activation(self, fun: str, d: int, drn, src) -> None:
@@ -425,7 +432,7 @@ class HipDevice:
         ops = self._ops(drn, *srcs)
         prog = (C.c_int32 * len(program))(*program)
         cs = (C.c_double * max(1, len(consts)))(*consts)
-        ptrs = (C.c_uint64 * max(1, len(srcs)))(*[o[0].value for o in ops[1:]])
+        ptrs = (C.c_uint64 * max(1, len(srcs)))(*[o[0] for o in ops[1:]])
         cfgs = (C.POINTER(C.c_int32) * max(1, len(srcs)))(*[o[2] for o in ops[1:]])
         _lib.check(self._lib.nk_fused(self.handle, prog, len(program) // 2, cs, len(consts), _dtype_code(drn.dtype), drn.ndc.rank,
                                       ops[0][0], ops[0][2], len(srcs), ptrs, cfgs, drn.ndc.size))
@@ -471,7 +478,7 @@ class HipDevice:
             ops = self._ops(drn, *srcs)
             prog = (C.c_int32 * len(program))(*program)
             cs = (C.c_double * max(1, len(consts)))(*consts)
-            ptrs = (C.c_uint64 * max(1, len(srcs)))(*[o[0].value for o in ops[1:]])
+            ptrs = (C.c_uint64 * max(1, len(srcs)))(*[o[0] for o in ops[1:]])
             cfgs = (C.POINTER(C.c_int32) * max(1, len(srcs)))(*[o[2] for o in ops[1:]])
             call = self.prepared("nk_fused", h, prog, len(program) // 2, cs, len(consts), _dtype_code(drn.dtype), drn.ndc.rank,
                                  ops[0][0], ops[0][2], len(srcs), ptrs, cfgs, C.c_int64(drn.ndc.size))

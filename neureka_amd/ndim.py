@@ -13,6 +13,8 @@ import enum
 from dataclasses import dataclass
 from typing import Sequence, Tuple
 
+import ctypes as C
+import functools
 import numpy as np
 
 MAX_RANK = 8
@@ -92,12 +94,12 @@ class NDConfiguration:
 
     @staticmethod
     def ofShape(shape: Sequence[int], layout: Layout = Layout.ROW_MAJOR) -> "NDConfiguration":
-        """A fresh dense tensor: ``NDConstructor.of(shape)`` (ndim/NDConstructor.java)."""
-        shape = tuple(int(s) for s in shape)
-        strides = layout.newStridesFor(shape)
-        # the flat->nd table is always the row-major one for RM and CM tensors (NDConfiguration.getLayout :157-173)
-        imap = Layout.ROW_MAJOR.newStridesFor(shape)
-        return NDConfiguration.of(shape, strides, imap, (1,) * len(shape), (0,) * len(shape))
+        """A fresh dense tensor: ``NDConstructor.of(shape)`` (ndim/NDConstructor.java).  Configurations are immutable and,
+        as in the reference (``AbstractNDC._cached``, ndim/config/AbstractNDC.java:39-66), one instance serves every
+        tensor of a shape and layout."""
+        if type(shape) is not tuple:
+            shape = tuple(int(s) for s in shape)
+        return _dense_configuration(shape, layout)
 
     @staticmethod
     def virtualOf(shape: Sequence[int]) -> "NDConfiguration":
@@ -185,8 +187,19 @@ class NDConfiguration:
         return self.indexOfIndices(self.indicesOfIndex(index))
 
     def asInlineArray(self) -> np.ndarray:
-        """``shape | strides | indicesMap | offset | spread`` (NDConfiguration.java:335-345)."""
-        return np.array(self.shape + self.strides + self.indicesMap + self.offset + self.spread, dtype=np.int32)
+        """``shape | strides | indicesMap | offset | spread`` (NDConfiguration.java:335-345).  The array is built once
+        per configuration and handed out read-only."""
+        return self.inlineArguments()[0]
+
+    def inlineArguments(self):
+        """(the inline array, a ctypes ``int32*`` to it): what a kernel launch passes for this configuration."""
+        cached = self.__dict__.get("_inline")
+        if cached is None:
+            arr = np.array(self.shape + self.strides + self.indicesMap + self.offset + self.spread, dtype=np.int32)
+            arr.flags.writeable = False
+            cached = (arr, arr.ctypes.data_as(C.POINTER(C.c_int32)))
+            object.__setattr__(self, "_inline", cached)      # a cache beside the (frozen) fields, not one of them
+        return cached
 
     # ---- derived views ---------------------------------------------------------------------
     def newReshaped(self, newForm: Sequence[int]) -> "NDConfiguration":
@@ -226,3 +239,12 @@ class IllegalStateException(RuntimeError):
 
 class IllegalArgumentException(ValueError):
     """Stands for ``java.lang.IllegalArgumentException`` where the reference throws one."""
+
+
+@functools.lru_cache(maxsize=4096)
+def _dense_configuration(shape: Tuple[int, ...], layout: Layout) -> NDConfiguration:
+    shape = tuple(int(s) for s in shape)
+    strides = layout.newStridesFor(shape)
+    # the flat->nd table is always the row-major one for RM and CM tensors (NDConfiguration.getLayout :157-173)
+    imap = Layout.ROW_MAJOR.newStridesFor(shape)
+    return NDConfiguration.of(shape, strides, imap, (1,) * len(shape), (0,) * len(shape))
