@@ -271,6 +271,47 @@ def test_scalarization_and_fill(device, orc, dt):
     assert np.count_nonzero(want) == 15
 
 
+@pytest.mark.parametrize("dt", ["f32", "f64"])
+def test_compiled_in_functions_and_operators_on_row_views(device, orc, dt):
+    """One function, or one heavy operator, of a source runs in a kernel with it compiled in ("rows_vec_single",
+    "rows_vec_pair") -- also on views whose rows are dense but lie apart (row slices, rows of a length that is no
+    multiple of the vector) and into a drain that is such a view: every function and derivative, every heavy operator
+    with a tensor and with a constant as its second operand, against the oracle on the same descriptors."""
+    T = F[dt]
+    rng = np.random.default_rng(77)
+    parent = rng.uniform(0.05, 2.0, (37, 203)).astype(T)
+    other = rng.uniform(0.05, 2.0, (37, 203)).astype(T)
+    tp, to = on(device, parent), on(device, other)
+    sl = np.s_[3:33, :]
+    vp, vo = tp[sl], to[sl]
+    hp, ho = np.ascontiguousarray(parent[sl]).reshape(-1), np.ascontiguousarray(other[sl]).reshape(-1)
+    dense = orc.dense_cfg([30, 203])
+    for name in ACTS:
+        for d in (-1, 0):
+            say("compiled-in function on a row view", name, d, dt)
+            drain_parent = on(device, np.full((37, 203), -7.0, dtype=T))
+            drain = drain_parent[sl]
+            device.launch_activation(name, d, drain, vp)
+            assert _lib.last_path() == "rows_vec_single", _lib.last_path()
+            want = orc.activation(name, d, np.zeros(hp.size, dtype=T), dense, hp, dense)
+            got = drain_parent.getData().reshape(37, 203)
+            assert (got[:3] == -7.0).all() and (got[33:] == -7.0).all(), "rows outside the view changed"
+            assert_close(got[sl].reshape(-1), want, f"{name} d={d}")
+    for op, ds in (("modulo", (-1, 0, 1)), ("power", (-1, 0, 1)), ("divide", (0, 1))):
+        for d in ds:
+            say("compiled-in operator on row views", op, d, dt)
+            out = Tensor._on_device(device, T, (30, 203))
+            device.launch_elementwise(op, d, out, vp, vo)
+            assert _lib.last_path() == "rows_vec_pair", _lib.last_path()
+            want = orc.elementwise(op, d, np.zeros(hp.size, dtype=T), dense, hp, dense, ho, dense)
+            (assert_bits if op == "modulo" and d < 0 else assert_close)(out.getData(), want, f"{op} d={d}")
+            say("compiled-in operator with a constant", op, d, dt)
+            device.launch_scalarization(op, d, out, vp, 1.75)
+            assert _lib.last_path() == "rows_vec_pair", _lib.last_path()
+            want = orc.scalarization(op, d, np.zeros(hp.size, dtype=T), dense, hp, dense, 1.75)
+            (assert_bits if op == "modulo" and d < 0 else assert_close)(out.getData(), want, f"{op} d={d} with a constant")
+
+
 VIEWS = {
     "permuted": lambda t: t.T(),
     "sliced": lambda t: t[::2, 1:t.shape[1] // 2 + 1],
