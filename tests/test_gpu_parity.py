@@ -555,12 +555,19 @@ def test_rows_shorter_than_a_vector_merge_with_the_axis_above(device, orc):
     A drain with gaps, or a source with another stride, keeps the element-wise path."""
     T = np.float32
     rng = np.random.default_rng(28)
-    for s1, s2 in (([4096, 1, 3], [1, 64, 3]), ([1, 64, 3], [4096, 1, 3]), ([300, 500, 3], [1, 1, 3]), ([1, 1, 3], [300, 500, 3]),
-                   ([7, 1, 1, 2], [1, 5, 33, 2]), ([5000, 1, 3], [5000, 77, 3]), ([9, 1, 1, 3], [9, 4, 11, 3]), ([1, 3], [1000003, 3])):
+    for s1, s2 in (([4096, 1, 3], [1, 64, 3]), ([1, 64, 3], [4096, 1, 3]),            # rows of 192
+                         ([300, 500, 3], [1, 1, 3]), ([1, 1, 3], [300, 500, 3]),            # one row of 450 000
+                         ([7, 1, 1, 2], [1, 5, 33, 2]),                                            # rows of 330, period 2
+                         ([5000, 1, 3], [5000, 77, 3]),                                            # rows of 231
+                         ([9, 1, 1, 3], [9, 4, 11, 3]),                                              # rows of 132
+                         ([1, 3], [1000003, 3]),                                                   # one row of 3 000 009
+                         ([77, 1, 2], [1, 34, 2]),                                                   # rows of 68, period 2
+                         ([33, 1, 3], [33, 4, 3]),                                                   # rows of 12: one thread per row
+                         ([1, 1, 3], [70001, 4, 3])):                                                # one row of 840 012
         so = [q if p == 1 else p for p, q in zip(s1, s2)]
         a = rng.uniform(-1, 1, s1).astype(T); b = rng.uniform(-1, 1, s2).astype(T)
         ta, tb = on(device, a), on(device, b)
-        for op, f in (("add", np.add), ("multiply", np.multiply), ("divide", np.divide)):
+        for op, f in (("add", np.add), ("multiply", np.multiply), ("divide", np.divide), ("subtract", np.subtract)):
             say("short rows", s1, s2, op)
             out = Tensor._on_device(device, T, so)
             device.launch_broadcast(op, -1, out, ta, tb)
