@@ -192,15 +192,19 @@ def percentiles(xs):
 
 
 def wall_ms(dev, call, reps, warm=10):
-    """Host wall clock per call in steady state: `reps` calls queued back to back, one synchronisation at the end."""
+    """Host wall clock per call in steady state: `reps` calls queued back to back, one synchronisation at the end; the
+    median of three such batches."""
     for _ in range(warm):
         call()
     dev.sync()
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        call()
-    dev.sync()
-    return (time.perf_counter() - t0) * 1e3 / reps
+    batches = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            call()
+        dev.sync()
+        batches.append((time.perf_counter() - t0) * 1e3 / reps)
+    return sorted(batches)[1]
 
 
 def memory_figures(dev, C, _lib):

@@ -270,13 +270,14 @@ class NDConvolution(Algorithm):
         return GOOD
 
     def prepare(self, call):             # linear/Convolution.java:91-103, ConvUtil.shapeOfCon (ConvUtil.java:61-66)
-        if call.arity <= 2:
-            call = call.withAddedInputAt(0, None)
-        if call.input(0) is None:
-            s1, s2 = call.input(1).shape, call.input(2).shape
-            shp = tuple(abs(s1[i] - s2[i]) + 1 for i in range(min(len(s1), len(s2))))
-            call = call.withInputAt(0, _new_output(call.device, call.input(1).dtype, shp, overwritten=True))
-        return call
+        inputs = call.inputs if len(call.inputs) > 2 else [None] + list(call.inputs)
+        if inputs[0] is None:
+            s1, s2 = inputs[1].shape, inputs[2].shape
+            shp = tuple([abs(p - q) + 1 for p, q in zip(s1, s2)])
+            inputs = [_new_output(call.device, inputs[1].dtype, shp, overwritten=True)] + list(inputs[1:])
+        if inputs is call.inputs:
+            return call
+        return ExecutionCall(call.device, call.operation, inputs, call.derivIdx, call.algorithm)
 
 
 class MatMulAlgorithm(Algorithm):

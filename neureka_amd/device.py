@@ -20,6 +20,7 @@ from .ndim import IllegalArgumentException, IllegalStateException, NDConfigurati
 _INT_CODES = {np.dtype(np.int32): 2, np.dtype(np.int64): 3, np.dtype(np.int16): 4, np.dtype(np.int8): 5}
 
 
+_ITEM_SIZES = {np.float32: 4, np.float64: 8, np.int32: 4, np.int64: 8, np.int16: 2, np.int8: 1, np.uint8: 1}
 _FLOAT_CODES = {np.float32: _lib.F32, np.float64: _lib.F64, np.dtype(np.float32): _lib.F32, np.dtype(np.float64): _lib.F64}
 
 
@@ -249,8 +250,11 @@ class HipDevice:
     def allocate(self, dtype, size: int) -> HipData:
         """Device.allocate (OpenCLDevice.java:520-530)."""
         self._check_open()
+        itemsize = _ITEM_SIZES.get(dtype)
+        if itemsize is None:
+            itemsize = np.dtype(dtype).itemsize
         ptr = C.c_uint64(0)
-        _lib.check(self._lib.nk_alloc(self.handle, int(size) * np.dtype(dtype).itemsize, C.byref(ptr)))
+        _lib.check(self._lib.nk_alloc(self.handle, int(size) * itemsize, C.byref(ptr)))
         return HipData(self, ptr.value, dtype, int(size))
 
     def allocateFromOne(self, dtype, size: int, value) -> HipData:

@@ -41,7 +41,7 @@ def execute(op_id: str, inputs: Sequence[Tensor], d: int = -1, record: bool = Tr
             raise IllegalArgumentException("Assignment does not support autograd!")
         record = False
     parents = list(inputs)                   # the tensors the caller holds: gradients attach to these
-    if len(inputs) > 1 and len({t.rank for t in inputs}) > 1 and op_id != "dot":
+    if len(inputs) > 1 and op_id != "dot" and any(len(t.ndc.shape) != len(inputs[0].ndc.shape) for t in inputs):
         inputs = make_fit(list(inputs))      # FunctionNode.execute pads ranks first (FunctionNode.java:92-93)
     call = ExecutionCall(device, operation, list(inputs), d)
     call.algorithm = operation.getAlgorithmFor(call)
