@@ -135,7 +135,7 @@ __device__ __forceinline__ double pow_ref(double a, double b) { return pow_doubl
 // the odd series up to s^13, relative error 2^-34), the product with the exponent in double, and 2^p as the hardware's
 // float exp2 of the fractional part scaled by ldexp.  The error of the product enters the result as p 2^-34 ln 2 <
 // 1e-8 and the float conversion of the fraction as 2e-8, so the result is within 3 ulp of (float) Math.pow.
-__device__ __forceinline__ float pow_positive(float a, float b) {
+__device__ __forceinline__ double log2_of_positive(float a) {       // 0 < a < infinity
     int e;
     double m = __builtin_frexp((double)a, &e);                   // [0.5, 1)
     const bool low = m < 0.70710678118654752;
@@ -149,13 +149,27 @@ __device__ __forceinline__ float pow_positive(float a, float b) {
     q = fma_const(q, s2, 0.2);
     q = fma_const(q, s2, 0.33333333333333331);
     const double ln_m_half = __builtin_fma(s * s2, q, s);        // atanh(s)
-    const double l2 = __builtin_fma(ln_m_half, 2.8853900817779268, (double)e);     // e + 2 atanh(s) log2(e)
-    double p = (double)b * l2;
+    return __builtin_fma(ln_m_half, 2.8853900817779268, (double)e);             // e + 2 atanh(s) log2(e)
+}
+__device__ __forceinline__ float pow_positive(float a, float b) {
+    double p = (double)b * log2_of_positive(a);
     p = p < -320.0 ? -320.0 : p;                                 // 2^-320 and 2^320 are 0 and infinity in float
     p = p > 320.0 ? 320.0 : p;
     const double n = __builtin_rint(p);
     const float r = __builtin_amdgcn_exp2f((float)(p - n));
     return __builtin_ldexpf(r, (int)n);
+}
+// a^b with the range of a double and the precision of a float (3 ulp of a float): what the float derivatives of the
+// power and of the cube root need -- the reference forms them in double (b * Math.pow(a, b - 1), Math.pow(a, b) *
+// Math.log(a), 1 / (3 * Math.pow(x, 2/3))) and rounds the product to float, so the power may leave the float range
+// where the product does not.  l2 = log2_of_positive(a).
+__device__ __forceinline__ double pow_from_log2(double l2, double b) {
+    double p = b * l2;
+    p = p < -1100.0 ? -1100.0 : p;                               // 2^-1100 and 2^1100 are 0 and infinity in double
+    p = p > 1100.0 ? 1100.0 : p;
+    const double n = __builtin_rint(p);
+    const float r = __builtin_amdgcn_exp2f((float)(p - n));
+    return __builtin_ldexp((double)r, (int)n);
 }
 __device__ __forceinline__ float pow_ref(float a, float b) {
     if (b == 2.0f) return a * a;
@@ -166,12 +180,38 @@ __device__ __forceinline__ float pow_ref(float a, float b) {
     return ::powf(a, b);
 }
 __device__ __forceinline__ double dpow_da_ref(double a, double b) { return b * pow_double(a, b - 1); }
-__device__ __forceinline__ float dpow_da_ref(float a, float b) { return (float)((double)b * pow_double((double)a, (double)(b - 1.0f))); }
+// (exponents 0, 1 and 2 have exact answers in pow_double; everything that is not a positive finite base with a finite
+// exponent -- signs, zeros, infinities, NaN -- keeps the library routine behind Math.pow's special cases)
+__device__ __forceinline__ bool pow_is_plain(float a, float e) {
+    return a > 0.0f && a < __builtin_inff() && ::fabsf(e) < __builtin_inff() && e != 0.0f && e != 1.0f && e != 2.0f;
+}
+__device__ __forceinline__ float dpow_da_ref(float a, float b) {
+    const float e = b - 1.0f;
+    if (pow_is_plain(a, e)) return (float)((double)b * pow_from_log2(log2_of_positive(a), (double)e));
+    return (float)((double)b * pow_double((double)a, (double)e));
+}
 // the broadcast twin multiplies by a, not by b (implementations/broadcast/CPUBroadcastPower.java:20-21)
 __device__ __forceinline__ double bcast_dpow_da_ref(double a, double b) { return a * pow_double(a, b - 1); }
-__device__ __forceinline__ float bcast_dpow_da_ref(float a, float b) { return (float)((double)a * pow_double((double)a, (double)(b - 1.0f))); }
+__device__ __forceinline__ float bcast_dpow_da_ref(float a, float b) {
+    const float e = b - 1.0f;
+    if (pow_is_plain(a, e)) return (float)((double)a * pow_from_log2(log2_of_positive(a), (double)e));
+    return (float)((double)a * pow_double((double)a, (double)e));
+}
 __device__ __forceinline__ double dpow_db_ref(double a, double b) { return pow_double(a, b) * ::log(a); }
-__device__ __forceinline__ float dpow_db_ref(float a, float b) { return (float)(pow_double((double)a, (double)b) * ::log((double)a)); }
+__device__ __forceinline__ float dpow_db_ref(float a, float b) {
+    if (pow_is_plain(a, b)) {                                    // one logarithm serves the power and the factor ln a
+        const double l2 = log2_of_positive(a);
+        return (float)(pow_from_log2(l2, (double)b) * (l2 * 0.69314718055994531));
+    }
+    return (float)(pow_double((double)a, (double)b) * ::log((double)a));
+}
+// x^(2/3) as the derivative of the cube root takes it: (T) Math.pow(x, (T) (2/3)) (fun/ScalarCbrt.java:31-32)
+__device__ __forceinline__ double cbrt_squared_ref(double x) { return ::pow(x, 2.0 / 3.0); }
+__device__ __forceinline__ float cbrt_squared_ref(float x) {
+    const double e = (double)(2.0f / 3.0f);
+    if (x > 0.0f && x < __builtin_inff()) return (float)pow_from_log2(log2_of_positive(x), e);
+    return (float)::pow((double)x, e);
+}
 __device__ __forceinline__ double ddiv_db_ref(double a, double b) { return -(a / (b * b)); }
 __device__ __forceinline__ float ddiv_db_ref(float a, float b) { return (float)-((double)a / ((double)b * (double)b)); }   // b*b is exact in double
 
@@ -430,7 +470,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
     constexpr bool NK_ONE_BY_ONE = ONE_BY_ONE;
     switch (id) {
         case NK_FUN_ABS: NK_EACH(x < T(0) ? T(-1) : T(1));
-        case NK_FUN_COS: NK_EACH(T(-::sin((double)x)));
+        case NK_FUN_COS: NK_EACH(sizeof(T) == 8 ? T(-::sin((double)x)) : T(-N::sin(x)));      // (nothing cancels: the float routine, 2 ulp, serves f32)
         case NK_FUN_GASU: NK_EACH(dgasu_ref(x));
         case NK_FUN_GATU: NK_EACH(dgatu_ref(x));
         case NK_FUN_GAUS: NK_EACH(T(-2.0 * (double)x * exp_fast(-((double)x * (double)x))));
@@ -443,7 +483,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
         case NK_FUN_SELU: NK_EACH(dselu_ref(x));
         case NK_FUN_SIG: NK_EACH(dsig_ref(x));
         case NK_FUN_SILU: NK_EACH(dsilu_ref(x));
-        case NK_FUN_SIN: NK_EACH(T(::cos((double)x)));
+        case NK_FUN_SIN: NK_EACH(sizeof(T) == 8 ? T(::cos((double)x)) : T(N::cos(x)));
         case NK_FUN_SOFTPLUS: NK_EACH(sig_as_ref(x));                   // the logistic function itself
         case NK_FUN_SOFTSIGN: NK_EACH(T(1) / (T(2) * N::abs(x) + x * x + T(1)));
         case NK_FUN_TANH: NK_EACH(dtanh_as_ref(x));
@@ -451,7 +491,7 @@ __device__ __forceinline__ void apply_dfun(int id, T (&a)[V]) {
         case NK_FUN_EXP: NK_EACH(T(exp_fast((double)x)));
         case NK_FUN_LOG10: NK_EACH(T(1) / (x * T(2.302585092994046)));   // x * ln(10)
         case NK_FUN_SQRT: NK_EACH(T(0.5) * inv_sqrt_ref(x));
-        case NK_FUN_CBRT: NK_EACH(T(1) / (T(3) * T(::pow((double)x, (double)(T(2.0) / T(3.0))))));
+        case NK_FUN_CBRT: NK_EACH(T(1) / (T(3) * cbrt_squared_ref(x)));
         default: NK_EACH(T(NAN) + x);
     }
 }

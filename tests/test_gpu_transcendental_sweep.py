@@ -45,8 +45,10 @@ def test_f32_exp_based_activations_dense_sweep(device, orc):
     tx = Tensor.of(np.float32, (n,), x).to(device)
     out = Tensor._on_device(device, np.float32, (n,))
     report = []
-    for name in SWEPT:
-        for d in (-1, 0):
+    # ... and the derivatives whose f32 kernels leave the reference's double routine for a float one (sin', cos') or for
+    # the logarithm-and-exp2 power (cbrt')
+    for name, d in [(name, d) for name in SWEPT for d in (-1, 0)] + [("sin", 0), ("cos", 0), ("cbrt", 0)]:
+        if True:
             print(f"[case] sweep {name} d={d} over {n} points", flush=True)
             device.launch_activation(name, d, out, tx)
             assert _lib.last_path() == "rows_vec_single", _lib.last_path()
@@ -100,25 +102,29 @@ def test_f32_power_dense_sweep(device, orc):
     cfg = orc.dense_cfg([n])
     ta, tb = Tensor.of(np.float32, (n,), a).to(device), Tensor.of(np.float32, (n,), b).to(device)
     out = Tensor._on_device(device, np.float32, (n,))
-    device.launch_elementwise("power", -1, out, ta, tb)
-    assert _lib.last_path() == "rows_vec_pair", _lib.last_path()        # one heavy operator: compiled in, not interpreted
-    got = out.getData().astype(np.float64)
-    with np.errstate(all="ignore"):
-        want = orc.elementwise("power", -1, np.zeros(n, dtype=np.float32), cfg, a, cfg, b, cfg, workers=16).astype(np.float64)
-    assert (np.isnan(got) == np.isnan(want)).all(), "NaNs differ"
-    inf = np.isinf(want)
-    assert (got[inf] == want[inf]).all(), "infinities differ"
-    finite = np.isfinite(want)
-    err = np.abs(got[finite] - want[finite])
-    # results below the smallest normal float are rounded to a multiple of 2^-149 by both sides: one such step apart at most
-    bound = RTOL * np.abs(want[finite]) + 1.5e-45
-    bad = err > bound
-    with np.errstate(all="ignore"):
-        rel = np.where(np.abs(want[finite]) > 1.2e-38, err / np.abs(want[finite]), 0.0)
-    w = int(np.argmax(rel))
-    print(f"[sweep] power worst relative error {rel[w]:.3e} at a = {a[finite][w]!r}, b = {b[finite][w]!r}", flush=True)
-    assert not bad.any(), (f"{int(bad.sum())} of {n} outside rtol {RTOL}; first at a = {a[finite][np.flatnonzero(bad)[0]]!r}, "
-                           f"b = {b[finite][np.flatnonzero(bad)[0]]!r}: got {got[finite][np.flatnonzero(bad)[0]]!r}, want {want[finite][np.flatnonzero(bad)[0]]!r}")
+    # the operator, then its derivatives by the base (b * a ** (b - 1)) and by the exponent (a ** b * ln a), which the
+    # reference forms in double and rounds once (CPUBiElementWisePower.java:13-31)
+    for d in (-1, 0, 1):
+        print(f"[case] sweep power d={d}", flush=True)
+        device.launch_elementwise("power", d, out, ta, tb)
+        assert _lib.last_path() == "rows_vec_pair", _lib.last_path()        # one heavy operator: compiled in, not interpreted
+        got = out.getData().astype(np.float64)
+        with np.errstate(all="ignore"):
+            want = orc.elementwise("power", d, np.zeros(n, dtype=np.float32), cfg, a, cfg, b, cfg, workers=16).astype(np.float64)
+        assert (np.isnan(got) == np.isnan(want)).all(), f"d={d}: NaNs differ"
+        inf = np.isinf(want)
+        assert (got[inf] == want[inf]).all(), f"d={d}: infinities differ"
+        finite = np.isfinite(want)
+        err = np.abs(got[finite] - want[finite])
+        # results below the smallest normal float are rounded to a multiple of 2^-149 by both sides: one such step apart at most
+        bound = RTOL * np.abs(want[finite]) + 1.5e-45
+        bad = err > bound
+        with np.errstate(all="ignore"):
+            rel = np.where(np.abs(want[finite]) > 1.2e-38, err / np.abs(want[finite]), 0.0)
+        w = int(np.argmax(rel))
+        print(f"[sweep] power d={d} worst relative error {rel[w]:.3e} at a = {a[finite][w]!r}, b = {b[finite][w]!r}", flush=True)
+        assert not bad.any(), (f"d={d}: {int(bad.sum())} of {n} outside rtol {RTOL}; first at a = {a[finite][np.flatnonzero(bad)[0]]!r}, "
+                               f"b = {b[finite][np.flatnonzero(bad)[0]]!r}: got {got[finite][np.flatnonzero(bad)[0]]!r}, want {want[finite][np.flatnonzero(bad)[0]]!r}")
     for t in (ta, tb, out):
         device.free(t)
 
