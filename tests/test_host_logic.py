@@ -312,3 +312,38 @@ def test_the_counted_traffic_record_belongs_to_the_sources_in_the_tree():
     traffic, note = bench.counted_traffic(HEADLINE_PATH)
     assert traffic == rec["traffic_bytes"] and "FETCH_SIZE" in note
     assert bench.counted_traffic("some_other_plan")[0] is None
+
+
+def test_java_binding_is_consistent_with_the_header_as_far_as_text_can_tell():
+    """No JDK exists here, so the Java files cannot be compiled; what text allows is checked: every `Nk.` member the other
+    classes use is declared in Nk.java, every MethodHandle there has the argument count and kinds (int / long / double /
+    address) of the ctypes binding of the same symbol, and brackets balance in every file outside strings and comments."""
+    import ctypes as C
+    import os
+    import re
+    from neureka_amd import _lib
+    root = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "java")
+    files = {}
+    for folder, _, names in os.walk(root):
+        for name in names:
+            if name.endswith(".java"):
+                with open(os.path.join(folder, name)) as f:
+                    files[name] = f.read()
+    assert {"Nk.java", "HipDevice.java", "HipBackend.java", "Hip.java", "HipFunctionCompiler.java"} <= set(files)
+    nk = files["Nk.java"]
+    handles = dict(re.findall(r'MethodHandle\s+(nk_\w+)\s*=\s*h\("nk_\w+",\s*([^;]*?)\);', nk))
+    assert set(handles) == set(_lib.SYMBOLS), sorted(set(handles) ^ set(_lib.SYMBOLS))
+    kind = {C.c_int: "I", C.c_uint64: "J", C.c_int64: "J", C.c_size_t: "J", C.c_double: "D", C.c_float: "F"}
+    for name, layouts in handles.items():
+        res, *args = [a.strip() for a in layouts.split(",")]
+        restype, argtypes = _lib.SYMBOLS[name]
+        want = [kind.get(t, "P") for t in argtypes]              # every pointer type (void*, T*, char*) is an address
+        assert args == want, (name, args, want)
+        assert res == ("P" if restype is C.c_char_p else "I"), (name, res)
+    members = set(handles) | set(re.findall(r"static\s+[\w<>\[\]?]+\s+(\w+)\s*\(", nk))
+    for name, text in files.items():
+        for used in re.findall(r"\bNk\.(\w+)", text):
+            assert used in members, f"{name} uses Nk.{used}, which Nk.java does not declare"
+        stripped = re.sub(r'"(?:\\.|[^"\\])*"|\'(?:\\.|[^\'\\])\'|//[^\n]*|/\*.*?\*/', "", text, flags=re.S)
+        for open_, close in ("{}", "()", "[]"):
+            assert stripped.count(open_) == stripped.count(close), f"{name}: unbalanced {open_}{close}"
