@@ -556,6 +556,7 @@ def main():
         hbm("elementwise_mul", 12 * n, dev.prepared_launch("elementwise", "multiply", -1, o, srcs[0], srcs[1]))
         # what the backward pass launches for an activation and for a division, and a heavy forward function
         hbm("activation_tanh_derivative", 8 * n, dev.prepared_launch("activation", "tanh", 0, o, srcs[0]))
+        hbm("activation_sig_derivative", 8 * n, dev.prepared_launch("activation", "sig", 0, o, srcs[0]))
         hbm("activation_relu_derivative", 8 * n, dev.prepared_launch("activation", "relu", 0, o, srcs[0]))
         hbm("divide_derivative", 12 * n, dev.prepared_launch("elementwise", "divide", 1, o, srcs[0], srcs[1]))
         hbm("activation_softplus", 8 * n, dev.prepared_launch("activation", "softplus", -1, o, srcs[0]))
@@ -566,6 +567,8 @@ def main():
         hbm("chain_derivative_by_input0", 16 * n, dev.prepared_launch("fused", dprog, dconsts, o, srcs))
         pos = Tensor.of(f32, (n,), rng.uniform(0.1, 2.0, n).astype(f32)).to(dev)
         hbm("power_tensor_exponent", 12 * n, dev.prepared_launch("elementwise", "power", -1, o, pos, srcs[1]))
+        # its derivative by the exponent, a ** b * ln a, which the reference forms in double and rounds once
+        hbm("power_derivative_by_exponent", 12 * n, dev.prepared_launch("elementwise", "power", 1, o, pos, srcs[1]))
         dev.free(pos)
         wide = Tensor(f32, NDConfiguration.ofShape((4096, 16384)), None); wide._set_data(srcs[0]._data, dev)
         strided = wide[::2, ::16]
