@@ -171,12 +171,31 @@ __device__ __forceinline__ double pow_from_log2(double l2, double b) {
     const float r = __builtin_amdgcn_exp2f((float)(p - n));
     return __builtin_ldexp((double)r, (int)n);
 }
+// A finite base below zero: Math.pow answers with the power of |a|, negated for an odd whole exponent, and with NaN for an
+// exponent that is no whole number.  The factor that carries this (floats from 2^24 on are even numbers): tensors of
+// mixed sign stay on the short path instead of sending every wavefront through the library routine as well.
+__device__ __forceinline__ float pow_sign_of(float a, float e) {
+    const bool whole = e == __builtin_rintf(e);
+    const bool odd = ::fabsf(e) < 16777216.0f && ((int)e & 1);
+    const float s = whole ? (odd ? -1.0f : 1.0f) : __builtin_nanf("");
+    return a < 0.0f ? s : 1.0f;
+}
+// ... looked at only by wavefronts that hold a negative base at all (a branch on the scalar unit): tensors of positive
+// bases pay one comparison for it
+__device__ __forceinline__ float pow_signed(float a, float e, float power_of_magnitude) {
+    if (__builtin_amdgcn_ballot_w64(a < 0.0f) != 0) return pow_sign_of(a, e) * power_of_magnitude;
+    return power_of_magnitude;
+}
+__device__ __forceinline__ double pow_signed(float a, float e, double power_of_magnitude) {
+    if (__builtin_amdgcn_ballot_w64(a < 0.0f) != 0) return (double)pow_sign_of(a, e) * power_of_magnitude;
+    return power_of_magnitude;
+}
 __device__ __forceinline__ float pow_ref(float a, float b) {
     if (b == 2.0f) return a * a;
     if (b == 1.0f) return a;
     if (b == 0.0f) return 1.0f;
     if (b != b || (::fabsf(a) == 1.0f && ::isinf(b))) return __builtin_nanf("");
-    if (a > 0.0f && a < __builtin_inff() && ::fabsf(b) < __builtin_inff()) return pow_positive(a, b);
+    if (a != 0.0f && ::fabsf(a) < __builtin_inff() && ::fabsf(b) < __builtin_inff()) return pow_signed(a, b, pow_positive(::fabsf(a), b));
     return ::powf(a, b);
 }
 __device__ __forceinline__ double dpow_da_ref(double a, double b) { return b * pow_double(a, b - 1); }
@@ -187,30 +206,47 @@ __device__ __forceinline__ bool pow_is_plain(float a, float e) {
 }
 __device__ __forceinline__ float dpow_da_ref(float a, float b) {
     const float e = b - 1.0f;
-    if (pow_is_plain(a, e)) return (float)((double)b * pow_from_log2(log2_of_positive(a), (double)e));
+    if (pow_is_plain(::fabsf(a), e)) return (float)((double)b * pow_signed(a, e, pow_from_log2(log2_of_positive(::fabsf(a)), (double)e)));
     return (float)((double)b * pow_double((double)a, (double)e));
 }
 // the broadcast twin multiplies by a, not by b (implementations/broadcast/CPUBroadcastPower.java:20-21)
 __device__ __forceinline__ double bcast_dpow_da_ref(double a, double b) { return a * pow_double(a, b - 1); }
 __device__ __forceinline__ float bcast_dpow_da_ref(float a, float b) {
     const float e = b - 1.0f;
-    if (pow_is_plain(a, e)) return (float)((double)a * pow_from_log2(log2_of_positive(a), (double)e));
+    if (pow_is_plain(::fabsf(a), e)) return (float)((double)a * pow_signed(a, e, pow_from_log2(log2_of_positive(::fabsf(a)), (double)e)));
     return (float)((double)a * pow_double((double)a, (double)e));
 }
 __device__ __forceinline__ double dpow_db_ref(double a, double b) { return pow_double(a, b) * ::log(a); }
 __device__ __forceinline__ float dpow_db_ref(float a, float b) {
-    if (pow_is_plain(a, b)) {                                    // one logarithm serves the power and the factor ln a
+    if (a < 0.0f) return __builtin_nanf("");                     // the logarithm of a negative base is NaN, and so is the product
+    if (a > 0.0f && a < __builtin_inff() && ::fabsf(b) < __builtin_inff()) {      // one logarithm serves the power and the factor ln a
         const double l2 = log2_of_positive(a);
-        return (float)(pow_from_log2(l2, (double)b) * (l2 * 0.69314718055994531));
+        double p = pow_from_log2(l2, (double)b);
+        p = b == 2.0f ? (double)a * (double)a : p;               // the exponents Math.pow answers exactly (pow_double)
+        p = b == 1.0f ? (double)a : p;
+        p = b == 0.0f ? 1.0 : p;
+        return (float)(p * (l2 * 0.69314718055994531));
     }
     return (float)(pow_double((double)a, (double)b) * ::log((double)a));
 }
 // x^(2/3) as the derivative of the cube root takes it: (T) Math.pow(x, (T) (2/3)) (fun/ScalarCbrt.java:31-32)
-__device__ __forceinline__ double cbrt_squared_ref(double x) { return ::pow(x, 2.0 / 3.0); }
+// Math.pow's answers off the positive finite numbers, for an exponent that is positive and no whole number: NaN below
+// zero, +0 for both zeros, +infinity for both infinities, NaN for NaN -- spelled out, so that a tensor of mixed sign
+// does not take every wavefront through the general routine.
+// f64: the square of the cube root; the exponent 2.0 / 3.0 lies 3.7e-17 below 2/3, so the two differ by that times
+// |ln x| < 745, relatively: 3e-14 at the ends of the range, against the 1e-12 the JDK's unspecified pow leaves room for.
+__device__ __forceinline__ double cbrt_squared_ref(double x) {
+    if (x > 0.0 && x < (double)__builtin_inff()) { const double c = ::cbrt(x); return c * c; }
+    if (x < 0.0 && x > -(double)__builtin_inff()) return __builtin_nan("");
+    return x == 0.0 ? 0.0 : ::fabs(x);
+}
 __device__ __forceinline__ float cbrt_squared_ref(float x) {
+    // (as branches: the same with selects over an unconditional power of |x| measured slower, 71 against 60 us for 2^25
+    // elements of mixed sign)
     const double e = (double)(2.0f / 3.0f);
     if (x > 0.0f && x < __builtin_inff()) return (float)pow_from_log2(log2_of_positive(x), e);
-    return (float)::pow((double)x, e);
+    if (x < 0.0f && x > -__builtin_inff()) return __builtin_nanf("");
+    return x == 0.0f ? 0.0f : ::fabsf(x);
 }
 __device__ __forceinline__ double ddiv_db_ref(double a, double b) { return -(a / (b * b)); }
 __device__ __forceinline__ float ddiv_db_ref(float a, float b) { return (float)-((double)a / ((double)b * (double)b)); }   // b*b is exact in double
