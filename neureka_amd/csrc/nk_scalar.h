@@ -31,12 +31,14 @@ template <> struct Num<float> {
     static __device__ __forceinline__ float tanh(float x) { return ::tanhf(x); }
     static __device__ __forceinline__ float fma(float a, float b, float c) { return ::fmaf(a, b, c); }
 };
+__device__ __forceinline__ double log_double(double x);        // below: the natural and the decimal logarithm of a double
+__device__ __forceinline__ double log10_double(double x);
 template <> struct Num<double> {
     static __device__ __forceinline__ double exp(double x) { return ::exp(x); }
     static __device__ __forceinline__ double expm1(double x) { return ::expm1(x); }
-    static __device__ __forceinline__ double log(double x) { return ::log(x); }
+    static __device__ __forceinline__ double log(double x) { return log_double(x); }
     static __device__ __forceinline__ double log1p(double x) { return ::log1p(x); }
-    static __device__ __forceinline__ double log10(double x) { return ::log10(x); }
+    static __device__ __forceinline__ double log10(double x) { return log10_double(x); }
     static __device__ __forceinline__ double sin(double x) { return ::sin(x); }
     static __device__ __forceinline__ double cos(double x) { return ::cos(x); }
     static __device__ __forceinline__ double sqrt(double x) { return ::sqrt(x); }
@@ -96,6 +98,58 @@ __device__ __forceinline__ double rcp_fast(double d) {
     r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
     r = __builtin_fma(__builtin_fma(-d, r, 1.0), r, r);
     return r;
+}
+// ln x in double for the f64 kernels (ln, softplus): x = m 2^e with m in [sqrt(1/2), sqrt 2), ln m = 2 atanh((m - 1)/(m + 1))
+// -- m - 1 is exact, so the result keeps its relative accuracy where x is close to 1 -- as the odd series up to s^19 (the
+// next term is below 3e-17 of the sum), e ln 2 with ln 2 in two parts (e ln2_hi is exact): about 3 units in the last
+// place (7e-16), some thirty full-rate instructions and one reciprocal, no table.  Math.log is specified to 1 ulp and
+// not bit for bit; the device library's log costs three times as much (2^25 doubles: 116 us, bound by it, against
+// 80 for a function that only moves the data).  Zero, negative numbers, infinity and NaN get Math.log's answers.
+// (the reduction: x = m 2^n, returns atanh((m - 1)/(m + 1)) = ln(m) / 2 for 0 < x < infinity)
+__device__ __forceinline__ double half_log_of_mantissa(double x, double& n) {
+    int e;
+    double m = __builtin_frexp(x, &e);                           // [0.5, 1), subnormal arguments included
+    const bool low = m < 0.70710678118654752;
+    m = low ? m + m : m;
+    e = low ? e - 1 : e;
+    n = (double)e;
+    const double s = (m - 1.0) * rcp_fast(m + 1.0);
+    const double s2 = s * s;
+    double q = fma_const(s2, 0.052631578947368418, 0.058823529411764705);      // 1/19, 1/17, ... 1/3
+    q = fma_const(q, s2, 0.066666666666666666);
+    q = fma_const(q, s2, 0.076923076923076927);
+    q = fma_const(q, s2, 0.090909090909090912);
+    q = fma_const(q, s2, 0.1111111111111111);
+    q = fma_const(q, s2, 0.14285714285714285);
+    q = fma_const(q, s2, 0.2);
+    q = fma_const(q, s2, 0.33333333333333331);
+    return __builtin_fma(s * s2, q, s);
+}
+__device__ __forceinline__ double log_double(double x) {
+    if (x > 0.0 && x < (double)__builtin_inff()) {
+        double n;
+        const double h = half_log_of_mantissa(x, n);
+        return __builtin_fma(n, 6.93147180369123816490e-01, __builtin_fma(n, 1.90821492927058770002e-10, h + h));
+    }
+    return x == 0.0 ? -(double)__builtin_inff() : (x < 0.0 ? __builtin_nan("") : x);
+}
+// log10 on the same reduction: n log10(2) in two parts plus ln(m) / ln 10.  Math.log10 promises the whole number n for an
+// argument that equals 10^n; the doubles that do are 10^0 ... 10^22, and a result that lands within 1e-13 of such an n is
+// compared with that power (a product of exact factors) and replaced by n when the argument is the power.
+__device__ __forceinline__ double log10_double(double x) {
+    if (x > 0.0 && x < (double)__builtin_inff()) {
+        double n;
+        const double h = half_log_of_mantissa(x, n);
+        double r = __builtin_fma(n, 3.01029995663611771306e-01, __builtin_fma(n, 3.69423907715893078616e-13, (h + h) * 4.34294481903251816668e-01));
+        const double k = __builtin_rint(r);
+        if (k >= 0.0 && k <= 22.0 && __builtin_fabs(r - k) < 1e-13) {
+            double power = 1.0;
+            for (int i = 0; i < (int)k; i++) power *= 10.0;      // exact up to 10^22
+            r = x == power ? k : r;
+        }
+        return r;
+    }
+    return x == 0.0 ? -(double)__builtin_inff() : (x < 0.0 ? __builtin_nan("") : x);
 }
 // 1 / (1 + e^(k x)) for a float x, |k| <= 2.  The argument stays within +-700, so that 1 + e^z stays finite for the
 // Newton steps (the answers there, 1 and 1e-304, are the saturated ones), by one float instruction on x instead of two
@@ -416,7 +470,7 @@ __device__ __forceinline__ float softplus_f32(float x) {
 }
 template <typename T> __device__ __forceinline__ T softplus_ref(T x) {
     using N = Num<T>;
-    if constexpr (sizeof(T) == 8) return N::log(T(1) + N::exp(x));
+    if constexpr (sizeof(T) == 8) return log_double(1.0 + exp_fast(x));
     else {
         if (x < T(-13)) return T(::log(1.0 + ::exp((double)x)));
         return softplus_f32(x);

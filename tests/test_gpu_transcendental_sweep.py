@@ -129,6 +129,55 @@ def test_f32_power_dense_sweep(device, orc):
         device.free(t)
 
 
+def test_f64_logarithm_softplus_and_cube_root_derivative_dense_sweep(device, orc):
+    """The f64 functions that do not go through the device library's routine -- ln, log10 and softplus on a table-free
+    double logarithm, the derivative of cbrt on the squared cube root -- against the oracle's libm evaluation of the reference's
+    formulas (ScalarLogarithm.java, ScalarLog10.java, ScalarSoftplus.java, ScalarCbrt.java:28-33), every element within 1e-12 relative (what
+    Math.log / Math.pow, specified to 1 ulp and not bit for bit, leave room for): every binade of the doubles, subnormals
+    included, the neighbourhood of 1 (where ln passes through zero and only a relatively accurate logarithm survives),
+    the seam of the range reduction at sqrt(1/2) and sqrt 2, both signs, zeros, infinities, NaN."""
+    rng = np.random.default_rng(2028)
+    parts = [np.ldexp(1 + rng.random(1500), e) for e in range(-1074, 1024)]              # 3.1 M points over every binade
+    parts += [1 + rng.uniform(-1e-3, 1e-3, 1 << 19), 1 + rng.uniform(-1e-9, 1e-9, 1 << 17), np.nextafter(1.0, 2.0) + np.zeros(1),
+              np.sqrt(0.5) * (1 + rng.uniform(-1e-6, 1e-6, 1 << 17)), np.sqrt(2.0) * (1 + rng.uniform(-1e-6, 1e-6, 1 << 17)),
+              rng.uniform(0.25, 4.0, 1 << 20)]
+    pos = np.concatenate(parts)
+    sp = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 5e-324, 2.2250738585072014e-308, 1.7976931348623157e308, 1.0, -1.0])
+    x_ln = np.concatenate([pos, -pos[::64], sp])
+    x_soft = np.concatenate([rng.uniform(-750, 750, 1 << 21), rng.uniform(-40, 40, 1 << 21), rng.standard_normal(1 << 20), sp])
+    tens = np.array([float(10 ** k) for k in range(23)])                                  # the doubles that are powers of ten
+    x_log10 = np.concatenate([x_ln, tens, np.nextafter(tens, np.inf), np.nextafter(tens, 0.0)])
+    for name, d, x in (("ln", -1, x_ln), ("log10", -1, x_log10), ("softplus", -1, x_soft), ("cbrt", 0, x_ln)):
+        n = x.size
+        print(f"[case] f64 sweep {name} d={d} over {n} points", flush=True)
+        cfg = orc.dense_cfg([n])
+        tx = Tensor.of(np.float64, (n,), x).to(device)
+        out = Tensor._on_device(device, np.float64, (n,))
+        device.launch_activation(name, d, out, tx)
+        assert _lib.last_path() == "rows_vec_single", _lib.last_path()
+        got = out.getData()
+        with np.errstate(all="ignore"):
+            want = orc.activation(name, d, np.zeros(n, dtype=np.float64), cfg, x, cfg, workers=16)
+        assert (np.isnan(got) == np.isnan(want)).all(), f"{name} d={d}: NaNs differ"
+        inf = np.isinf(want)
+        assert (got[inf] == want[inf]).all(), f"{name} d={d}: infinities differ"
+        finite = np.isfinite(want)
+        err = np.abs(got[finite] - want[finite])
+        # softplus: the reference's log(1 + e^x) rounds 1 + e^x to a multiple of 2.2e-16 before the logarithm, so a last-place
+        # difference between two exponentials can move the result by that quantum whatever its size
+        bad = err > 1e-12 * np.abs(want[finite]) + (2.3e-16 if name == "softplus" else 0.0)
+        with np.errstate(all="ignore"):
+            rel = np.where(want[finite] != 0, err / np.abs(want[finite]), 0.0)
+        w = int(np.argmax(rel))
+        print(f"[sweep] f64 {name} d={d} worst relative error {rel[w]:.3e} at x = {x[finite][w]!r}", flush=True)
+        assert not bad.any(), (f"{name} d={d}: {int(bad.sum())} of {n} outside rtol 1e-12; first at x = {x[finite][np.flatnonzero(bad)[0]]!r}: "
+                               f"got {got[finite][np.flatnonzero(bad)[0]]!r}, want {want[finite][np.flatnonzero(bad)[0]]!r}")
+        if name == "log10":                                      # Math.log10: the whole number n for an argument equal to 10^n
+            at = x_ln.size
+            assert (got[at:at + 23] == np.arange(23.0)).all(), got[at:at + 23]
+        device.free(tx); device.free(out)
+
+
 def test_config3_single_kernels_full_size(device, orc):
     """The four kernels the reference runs for tanh(sig(a)*b+c), each alone on 2^26 elements: sig and tanh within 1e-5
     of the oracle element by element, multiply and add bit for bit."""
