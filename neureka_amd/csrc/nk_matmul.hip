@@ -436,6 +436,113 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     }
 }
 
+// The same tiles with the k range split inside the block: KG groups of four wavefronts, each group the kernel above on
+// its own part of the k range with its own three stages of LDS, so that every SIMD holds KG wavefronts.  The groups meet
+// once, at the end, in LDS, where the first adds the others' accumulators in order and stores the tile.  K % (32 KG) == 0;
+// KG x 52.5 KiB of LDS, asked for at the launch.  1024^3: 26.5 -> 24.2 us, 1024 x 2048 x 1024: 49.4 -> 43.7 (the matrix
+// instructions alone, with no loads at all, take 19.1 and 33.4 in this kernel).
+template <bool OVERWRITE, int KG>
+__global__ __launch_bounds__(256 * KG) void matmul_mfma64_split_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C) {
+    using namespace t64;
+    extern __shared__ __attribute__((aligned(16))) float split_lds[];
+    int tm, tn;
+    tile_of_block(g, (int)blockIdx.x, tm, tn);
+    const int grp = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
+    const int tid = threadIdx.x & 255;
+    float* const lds = split_lds + grp * t64::LDS_FLOATS;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    const int l32 = lane & 31, h = lane >> 5;
+    const float* Ag = A + (int64_t)tm * TM * g.K;
+    const float* Bg = B + (int64_t)tn * TN;
+    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 * i
+    const int b_row = tid >> 4, b_col = (tid & 15) * 4;     // rows b_row + 16 * i
+    f32x4 ra[2], rb[2];
+    auto load_global = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
+            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 16 * i) * g.N + b_col);
+        }
+    };
+    auto store_lds = [&](int stage) {
+        float* as = lds + stage * STAGE;
+        float* bs = as + TM * A_P;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            *(f32x4*)(&as[(a_row + 32 * i) * A_P + a_col]) = ra[i];
+            *(f32x4*)(&bs[(b_row + 16 * i) * B_P + b_col]) = rb[i];
+        }
+    };
+    struct Chunk { f32x4 a; float b[4]; };
+    auto read_chunk = [&](Chunk& f, int stage, int c) {
+        const float* as = lds + stage * STAGE;
+        const float* bs = as + TM * A_P;
+        f.a = *(const f32x4*)(&as[(wm + l32) * A_P + 8 * c + 4 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; t++) f.b[t] = bs[(8 * c + 4 * h + t) * B_P + wn + l32];
+    };
+    f32x16 acc0, acc1;
+#pragma unroll
+    for (int v = 0; v < 16; v++) { acc0[v] = 0.0f; acc1[v] = 0.0f; }
+    auto mma = [&](const Chunk& even, const Chunk& odd) {
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(even.a[t], even.b[t], acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(odd.a[t], odd.b[t], acc1, 0, 0, 0);
+        }
+    };
+    const int nk = g.K / BK / KG;                             // slices of a group: the same for every group, so every wavefront
+    const int kbase = grp * nk * BK;                          // of the block reaches every barrier
+    auto clamped = [&](int slice) { return kbase + (slice < nk ? slice : nk - 1) * BK; };
+    load_global(clamped(0));
+    store_lds(0);
+    load_global(clamped(1));
+    store_lds(1);
+    load_global(clamped(2));
+    __syncthreads();
+    Chunk f0, f1, f2, f3;
+    read_chunk(f0, 0, 0);
+    read_chunk(f1, 0, 1);
+    int cur = 0;
+    for (int kt = 0; kt < nk; kt++) {
+        const int next = cur == 2 ? 0 : cur + 1, write = next == 2 ? 0 : next + 1;
+        read_chunk(f2, cur, 2);
+        read_chunk(f3, cur, 3);
+        mma(f0, f1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_lds(write);
+        load_global(clamped(kt + 3));
+        read_chunk(f0, next, 0);
+        read_chunk(f1, next, 1);
+        mma(f2, f3);
+        __syncthreads();
+        cur = next;
+    }
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = acc0[v] + acc1[v];
+    // the meeting: nobody reads a stage any more (every read was waited for before the loop's last barrier); element v of
+    // thread tid of group grp > 0 sits at (v (KG - 1) + grp - 1) 256 + tid
+    if (grp > 0) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) split_lds[(v * (KG - 1) + grp - 1) * 256 + tid] = acc[v];
+    }
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+        for (int v = 0; v < 16; v++)
+#pragma unroll
+            for (int o = 0; o < KG - 1; o++) acc[v] += split_lds[(v * (KG - 1) + o) * 256 + tid];
+        float* Cg = C + (int64_t)(tm * TM + wm) * g.N + tn * TN + wn + l32;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            float* p = Cg + (int64_t)(8 * (v >> 2) + 4 * h + (v & 3)) * g.N;
+            *p = OVERWRITE ? acc[v] : *p + acc[v];
+        }
+    }
+}
+
 // Whole tiles, no split, more tiles than resident blocks: blocks that stay.  A block walks the tiles blockIdx.x,
 // + gridDim.x, ... and the software pipeline over the k-slices runs on across them: the first slice of the next
 // tile is fetched and written to the free LDS buffer during the last slice of the current one, so only the
@@ -1411,6 +1518,28 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
 
 // `force_parts`, `bands`: how matmul_rm calls itself for the two row bands described below (callers leave them alone: `bands`
 // is true for a caller's product, which may be planned as bands or take one of the streaming kernels, and false for a band)
+// Kernels that need more LDS than a launch gets by default (the 256 x 256 tiles: 137 KiB; the 64 x 64 tiles with the k
+// range split inside the block: 105 KiB): asked for once per device; a device that does not grant it (or has less) keeps to
+// the other plans.  Device::big_tiles: 0 not asked yet, 1 granted, -1 not available.
+constexpr int T64_SPLIT = 2;
+constexpr int T64_SPLIT_LDS_BYTES = T64_SPLIT * t64::LDS_FLOATS * (int)sizeof(float);
+static bool large_lds(Device* dev) {
+    if (dev->big_tiles == 0) {
+        dev->big_tiles = -1;
+        constexpr int big_bytes = big::LDS_FLOATS * (int)sizeof(float);
+        if ((int64_t)dev->props.sharedMemPerBlockOptin >= big_bytes) {
+            const void* kernels[6] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
+                                      (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>,
+                                      (const void*)matmul_mfma64_split_kernel<true, T64_SPLIT>, (const void*)matmul_mfma64_split_kernel<false, T64_SPLIT>};
+            hipError_t attr = hipSuccess;
+            for (int k = 0; k < 6; k++)
+                if (attr == hipSuccess) attr = hipFuncSetAttribute(kernels[k], hipFuncAttributeMaxDynamicSharedMemorySize, k < 4 ? big_bytes : T64_SPLIT_LDS_BYTES);
+            if (attr == hipSuccess) dev->big_tiles = 1; else (void)hipGetLastError();
+        }
+    }
+    return dev->big_tiles > 0;
+}
+
 static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t K, int64_t N, nk_buf A, nk_buf B, nk_buf C,
                      int force_parts = 0, bool bands = true) {
     constexpr int64_t mfma_from = (int64_t)1 << 24;
@@ -1645,19 +1774,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 gb.tiles_m = (int)((M + big::TM - 1) / big::TM); gb.tiles_n = (int)((N + big::TN - 1) / big::TN);
                 gb.group_rows = gb.tiles_m < 4 ? gb.tiles_m : 4;
                 constexpr int lds_bytes = big::LDS_FLOATS * (int)sizeof(float);
-                // the kernel needs more LDS than a launch gets by default: asked for once per device; a device that does not
-                // grant it (or has less) keeps to the plans below
-                if (dev->big_tiles == 0) {
-                    dev->big_tiles = -1;
-                    if ((int64_t)dev->props.sharedMemPerBlockOptin >= lds_bytes) {
-                        const void* kernels[4] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
-                                                  (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>};
-                        hipError_t attr = hipSuccess;
-                        for (const void* k : kernels)
-                            if (attr == hipSuccess) attr = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-                        if (attr == hipSuccess) dev->big_tiles = 1; else (void)hipGetLastError();
-                    }
-                }
+                large_lds(dev);
                 if (dev->big_tiles > 0) {
                     const dim3 grid((unsigned)tiles);
                     if (whole_big) {
@@ -1683,10 +1800,17 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 MfmaArgs gs = g;
                 gs.tiles_m = (int)(M / t64::TM); gs.tiles_n = (int)(N / t64::TN);
                 gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
-                if (overwrite) hipLaunchKernelGGL(matmul_mfma64_kernel<true>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                else           hipLaunchKernelGGL(matmul_mfma64_kernel<false>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                // two wavefronts per SIMD, each group of four on its half of the k range (at least four slices each)
+                const bool split = K % (T64_SPLIT * BK) == 0 && K >= T64_SPLIT * 4 * BK && large_lds(dev);
+                if (split) {
+                    if (overwrite) hipLaunchKernelGGL((matmul_mfma64_split_kernel<true, T64_SPLIT>), dim3((unsigned)small), dim3(256 * T64_SPLIT), T64_SPLIT_LDS_BYTES, dev->stream, gs, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL((matmul_mfma64_split_kernel<false, T64_SPLIT>), dim3((unsigned)small), dim3(256 * T64_SPLIT), T64_SPLIT_LDS_BYTES, dev->stream, gs, Ap, Bp, Cp);
+                } else {
+                    if (overwrite) hipLaunchKernelGGL(matmul_mfma64_kernel<true>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL(matmul_mfma64_kernel<false>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                }
                 NK_HIP(hipGetLastError());
-                set_path("mfma_tiles_of_64");
+                set_path(split ? "mfma_tiles_of_64_split" : "mfma_tiles_of_64");
                 return NK_OK;
             }
         }

@@ -1796,7 +1796,8 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
     ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64"),
     ("f32", (4100, 9, 4096), "short_inner"), ("f64", (4096, 16, 2050), "short_inner_f64"),
-    ("f32", (32, 2048, 2048), "few_rows"), ("f64", (20, 4096, 512), "few_rows_f64")])
+    ("f32", (32, 2048, 2048), "few_rows"), ("f64", (20, 4096, 512), "few_rows_f64"),
+    ("f32", (1024, 1024, 1024), "mfma_tiles_of_64_split"), ("f32", (1024, 288, 1024), "mfma_tiles_of_64")])
 def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mkn, path):
     """nk_matmul_set (C = A @ B, the OpenCL device's `C[n + m*N] = acc`, CLMatMul.java:50) on every kernel plan, both
     layouts: the drain starts as NaN everywhere, so a single old value read would show; the result must equal, bit for
@@ -1817,6 +1818,53 @@ def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mk
         a, g = acc.getData(), got.getData()
         assert not np.isnan(g).any()
         assert (a.view(np.uint32 if dt == "f32" else np.uint64) == g.view(np.uint32 if dt == "f32" else np.uint64)).all()
+
+
+@pytest.mark.parametrize("mkn,path", [((1024, 1024, 1024), "mfma_tiles_of_64_split"), ((1024, 320, 1024), "mfma_tiles_of_64_split"),
+                                      ((512, 2048, 2048), "mfma_tiles_of_64_split"), ((1024, 256, 1024), "mfma_tiles_of_64_split"),
+                                      ((1024, 288, 1024), "mfma_tiles_of_64"), ((2048, 160, 512), "mfma_tiles_of_64")])
+def test_matmul_64_tiles_in_one_launch(device, mkn, path):
+    """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit: one launch of
+    the small-tile kernel -- with the k range split between two groups of wavefronts inside the block where it divides
+    into two runs of at least four slices, whole otherwise.  Integer data are exact against numpy in both layouts and
+    through both entry points; uniform data stay within the norm-wise bound; operands inside larger buffers full of NaN
+    show that nothing outside them is read."""
+    M, K, N = mkn
+    rng = np.random.default_rng(67)
+    say("matmul 64 tiles integer", mkn)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float32); B = rng.integers(-5, 6, (K, N)).astype(np.float32)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    tc = on(device, np.full((M, N), np.nan, dtype=np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want).all()
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)                  # C += A @ B
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == 2 * want).all()
+    say("matmul 64 tiles column major", mkn)
+    tc = on(device, np.zeros((N, M), dtype=np.float32))
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+    assert (tc.getData().reshape(N, M).T == want).all()
+    say("matmul 64 tiles uniform", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    tc = on(device, np.zeros((M, N), dtype=np.float32))
+    device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
+    assert _lib.last_path() == path, _lib.last_path()
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
+    say("matmul 64 tiles, operands inside larger buffers full of NaN", mkn)
+    pad = 64                                                                             # elements: keeps the 16-byte alignment
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(np.zeros((M, N), dtype=np.float32))
+    _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
 @pytest.mark.parametrize("mkn", [(4096, 1024, 4096), (2048, 2048, 8192), (4096, 1056, 4096), (8192, 1024, 8192), (4096, 512, 4096)])
