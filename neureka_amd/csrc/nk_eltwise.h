@@ -454,7 +454,7 @@ __global__ __launch_bounds__(256) void rows_kernel(RowsArgs A, Prog P, LightProg
 // path is rows_kernel's (plain vector loads, two units per block); the function is inlined instead of interpreted, so a
 // thread spends its instructions on the function alone.  That matters where the function, not memory, bounds the kernel:
 // the f32 derivatives that repeat the reference's double-precision formula (tanh', 2^26 elements: 56 vector instructions
-// per element and 0.49 of the HBM rate through the interpreter, 0.66 here) -- and the light functions lose nothing.
+// per element and 0.49 of the HBM rate through the interpreter, 0.61-0.63 here) -- and the light functions lose nothing.
 constexpr int SINGLE_PASSES = 2;
 template <typename T, int V, bool NT, bool DERIV, int FID>
 __global__ __launch_bounds__(256) void rows_single_kernel(RowsArgs A, T* __restrict__ drn, const T* __restrict__ src) {

@@ -38,7 +38,7 @@ struct Device {
     // grow-only scratch for two-pass kernels (partial sums); owned by the device, freed on close
     void* workspace = nullptr;
     uint64_t workspace_bytes = 0;
-    int big_tiles = 0;                   // matmul's 256 x 256 tiles need 137 KiB of LDS: 0 not asked yet, 1 granted, -1 not available
+    int big_tiles = 0;                   // matmul's kernels that need more LDS than a launch gets by default: 0 not asked yet, 1 granted, -1 not available
     // this device's copy of the file-scope array nk_sum_static keeps its partial results in
     void* sum_static_scratch = nullptr;
 };
