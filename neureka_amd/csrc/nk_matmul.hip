@@ -55,6 +55,7 @@ struct MfmaArgs {
     int splits;          // SPLIT kernels: parts the k range is cut into (grid = tiles * splits) ...
     int split_slices;    // ... and k-slices per part
     int overwrite;       // C = A @ B instead of C += A @ B: the old values of C are not read
+    int rows_a;          // MIXED kernels: tile rows whose tiles take the whole k range (the rest: parts, as in SPLIT)
 };
 
 __device__ __forceinline__ void tile_of_block(const MfmaArgs& g, int bid, int& tm, int& tn) {
@@ -173,17 +174,42 @@ constexpr int LDS_FLOATS = LDS_FLOATS_AB > LDS_FLOATS_C ? LDS_FLOATS_AB : LDS_FL
 // in both operands so that it adds exactly nothing; the epilogue stores element-wise along the edges.
 // SPLIT: few tiles (small or thin products): the k range is cut into g.splits parts, block (tile, part) stores its
 // partial tile to P[part] instead of adding it to C, and matmul_add_parts_kernel adds the parts in order.
-template <bool EDGE, bool SPLIT = false>
+// MIXED: one launch for a product with more tiles than compute units but fewer than the blocks that fit the machine (two
+// per unit): the blocks of the first g.rows_a tile rows come first and take a whole tile each, about one per unit; the
+// tiles of the remaining rows follow as parts of their k range, as in SPLIT, written to P (a matrix of those rows
+// only) and added by matmul_add_parts.  The short blocks fill the second place on every unit as they come and go, so
+// the units finish together instead of some with one tile and some with two.
+template <bool EDGE, bool SPLIT = false, bool MIXED = false>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const float* __restrict__ A,
                                                           const float* __restrict__ B, float* __restrict__ C, float* __restrict__ P = nullptr) {
+    static_assert(!MIXED || (!EDGE && !SPLIT), "the mixed launch is for whole tiles of an unsplit product");
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     float* const As0 = lds;                                   // [2][BM * A_PITCH]
     float* const Bs0 = lds + 2 * BM * A_PITCH;                // [2][BK * B_PITCH]
 
     int tm, tn;
     const int n_tiles = g.tiles_m * g.tiles_n;
-    const int part = SPLIT ? (int)blockIdx.x / n_tiles : 0;
-    tile_of_block(g, SPLIT ? (int)blockIdx.x - part * n_tiles : (int)blockIdx.x, tm, tn);
+    int part = SPLIT ? (int)blockIdx.x / n_tiles : 0;
+    bool parted = SPLIT;                                      // this block computes a part of its tile's k range, into P
+    if constexpr (MIXED) {
+        const int tiles_a = g.rows_a * g.tiles_n;
+        MfmaArgs band = g;
+        if ((int)blockIdx.x < tiles_a) {
+            band.tiles_m = g.rows_a;
+            band.group_rows = g.group_rows < band.tiles_m ? g.group_rows : band.tiles_m;
+            tile_of_block(band, (int)blockIdx.x, tm, tn);
+        } else {
+            band.tiles_m = g.tiles_m - g.rows_a;
+            band.group_rows = g.group_rows < band.tiles_m ? g.group_rows : band.tiles_m;
+            const int tiles_b = band.tiles_m * g.tiles_n, b = (int)blockIdx.x - tiles_a;
+            part = b / tiles_b;
+            tile_of_block(band, b - part * tiles_b, tm, tn);
+            tm += g.rows_a;
+            parted = true;
+        }
+    } else {
+        tile_of_block(g, SPLIT ? (int)blockIdx.x - part * n_tiles : (int)blockIdx.x, tm, tn);
+    }
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;     // wave's sub-tile origin inside the block tile
@@ -215,9 +241,9 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
     // buffer complete.
     static_assert(BK == 32, "the pipeline below is written for four depth-8 chunks per slice");
     const int all_slices = (g.K + BK - 1) / BK;
-    const int slice0 = SPLIT ? part * g.split_slices : 0;                           // first k-slice of this block
+    const int slice0 = parted ? part * g.split_slices : 0;                          // first k-slice of this block
     int nk = all_slices;                                                             // ... and how many it takes
-    if (SPLIT) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
+    if (parted) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
     const int kbase = slice0 * BK;
     Frag f0, f1;
     load_global(kbase);
@@ -294,7 +320,8 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
                 cs[row * C_PITCH + wn + 32 * j + l32] = acc[i][j][v];
             }
     __syncthreads();
-    float* Cg = (SPLIT ? P + (int64_t)part * g.M * g.N : C) + (int64_t)tm * BM * g.N + tn * BN;
+    float* Cg = C + (int64_t)tm * BM * g.N + tn * BN;
+    if (parted) Cg = P + ((int64_t)part * (g.M - (MIXED ? g.rows_a * BM : 0)) + (int64_t)(tm - (MIXED ? g.rows_a : 0)) * BM) * g.N + tn * BN;
     const int c_col = (tid & 31) * 4, c_row = tid >> 5;
     if (EDGE) {
         const int rows = g.M - tm * BM, cols = g.N - tn * BN;          // what is left of C from this tile's origin
@@ -310,7 +337,7 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
         }
         return;
     }
-    if (SPLIT || g.overwrite) {                            // the same for every block of a launch
+    if (parted || g.overwrite) {                           // the same for every thread of a block
 #pragma unroll
         for (int i = 0; i < 16; i++)
             *(f32x4*)(Cg + (int64_t)(c_row + 8 * i) * g.N + c_col) = *(const f32x4*)(&cs[(c_row + 8 * i) * C_PITCH + c_col]);
@@ -1844,6 +1871,36 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 NK_HIP(hipGetLastError());
                 set_path(split ? "mfma_tiles_of_64_split" : "mfma_tiles_of_64");
                 return NK_OK;
+            }
+        }
+        // A few more tiles than compute units: as one launch of whole tiles some units would work through two tiles side by
+        // side while the others finish with one.  Instead the upper tile rows, about one tile per unit, take the whole k
+        // range, and the tiles of the lower rows come as parts of their k range that fill the second places
+        // (matmul_mfma_kernel<false, false, true>); their sum follows as for every split product.  2304^3 (324 tiles): 278 ->
+        // 203 us; 2176 x 2048 x 2176: 247 -> 164; 2048 x 1024 x 2560: 126 -> 103.  With more than half a round of tiles in the
+        // lower rows it no longer pays (2560^3, 160 of 400 tiles: 310 -> 302; 4096 x 512 x 1536, 132 of 384: 68 -> 75).
+        if (bands && force_parts < 2 && whole_tiles) {
+            const int64_t cus = dev->props.multiProcessorCount, tiles = (int64_t)g.tiles_m * g.tiles_n, slices = K / BK;
+            const int64_t rows_a = cus / g.tiles_n;
+            const int64_t tiles_b = tiles - rows_a * g.tiles_n;
+            if (tiles > cus && 2 * tiles_b <= cus && rows_a >= 1 && rows_a < g.tiles_m && slices >= 16) {
+                const int64_t m_a = rows_a * BM, m_b = M - m_a;
+                int64_t parts = (2 * cus + tiles_b - 1) / tiles_b;                        // about two short blocks per unit at a time
+                if (parts > slices / 8) parts = slices / 8;
+                if (parts >= 2 && (uint64_t)parts * m_b * N * sizeof(float) <= ((uint64_t)1 << 30)) {
+                    MfmaArgs gm = g;
+                    gm.rows_a = (int)rows_a;
+                    gm.split_slices = (int)((slices + parts - 1) / parts);
+                    gm.splits = (int)((slices + gm.split_slices - 1) / gm.split_slices);
+                    void* ws = nullptr;
+                    if (int e = workspace(dev, (uint64_t)gm.splits * m_b * N * sizeof(float), &ws)) return e;
+                    const unsigned grid = (unsigned)(rows_a * g.tiles_n + tiles_b * gm.splits);
+                    hipLaunchKernelGGL((matmul_mfma_kernel<false, false, true>), dim3(grid), dim3(256), 0, dev->stream, gm, Ap, Bp, Cp, (float*)ws);
+                    launch_add_parts<float>(dev, m_b * N, gm.splits, g.overwrite, (const float*)ws, Cp + m_a * N);
+                    NK_HIP(hipGetLastError());
+                    set_path("mfma_mixed");
+                    return NK_OK;
+                }
             }
         }
         if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;

@@ -1820,6 +1820,48 @@ def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mk
         assert (a.view(np.uint32 if dt == "f32" else np.uint64) == g.view(np.uint32 if dt == "f32" else np.uint64)).all()
 
 
+@pytest.mark.parametrize("mkn,path", [((2304, 608, 2304), "mfma_mixed"), ((2176, 512, 2176), "mfma_mixed"), ((33024, 512, 128), "mfma_mixed"),
+                                      ((2048, 1056, 2560), "mfma_mixed"), ((2560, 512, 2560), "mfma"), ((4096, 512, 1536), "mfma")])
+def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
+    """Products with a few more 128 x 128 tiles than compute units run as one launch in which the upper tile rows take the
+    whole k range and the lower rows come as parts of it (their sum follows); with more than half a round of tiles in the
+    lower rows the plain launch stays.  Integer data are exact against numpy in both layouts and through both entry
+    points (the parts' run lengths do not divide the k range in every case); uniform data stay within the norm-wise
+    bound; NaN around the operands and in the drain of an overwriting call shows that nothing else is read."""
+    M, K, N = mkn
+    rng = np.random.default_rng(71)
+    say("matmul mixed integer", mkn)
+    A = rng.integers(-5, 6, (M, K)).astype(np.float32); B = rng.integers(-5, 6, (K, N)).astype(np.float32)
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    ta, tb = on(device, A), on(device, B)
+    tc = on(device, np.full((M, N), np.nan, dtype=np.float32))
+    device.launch_matmul(True, M, K, N, ta, tb, tc, accumulate=False)
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == want).all()
+    device.launch_matmul(True, M, K, N, ta, tb, tc)                                        # C += A @ B
+    assert _lib.last_path() == path, _lib.last_path()
+    assert (tc.getData().reshape(M, N) == 2 * want).all()
+    say("matmul mixed column major", mkn)
+    tc = on(device, np.zeros((N, M), dtype=np.float32))
+    device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
+    assert (tc.getData().reshape(N, M).T == want).all()
+    say("matmul mixed uniform, operands inside larger buffers full of NaN", mkn)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    ref = A.astype(np.float64) @ B.astype(np.float64)
+    bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
+    pad = 64
+    def parked(x):
+        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
+        host[pad:pad + x.size] = x.reshape(-1)
+        return on(device, host)
+    pa, pb, pc = parked(A), parked(B), parked(np.zeros((M, N), dtype=np.float32))
+    _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+    assert _lib.last_path() == path, _lib.last_path()
+    got = pc.getData()
+    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+    assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
+
+
 @pytest.mark.parametrize("mkn,path", [((1024, 1024, 1024), "mfma_tiles_of_64_split"), ((1024, 320, 1024), "mfma_tiles_of_64_split"),
                                       ((512, 2048, 2048), "mfma_tiles_of_64_split"), ((1024, 256, 1024), "mfma_tiles_of_64_split"),
                                       ((1024, 288, 1024), "mfma_tiles_of_64"), ((2048, 160, 512), "mfma_tiles_of_64")])
