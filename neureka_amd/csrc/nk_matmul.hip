@@ -98,26 +98,51 @@ struct TileF32 {
     };
     int a_row, a_col, b_row, b_col;      // a thread's pieces: rows a_row + 32 i of A, rows b_row + B_STEP i of B
     __device__ __forceinline__ explicit TileF32(int tid) : a_row(tid >> 3), a_col((tid & 7) * 4), b_row(tid / (TN / 4)), b_col((tid % (TN / 4)) * 4) {}
-    // whole tiles: Ag = the tile's first row of A, Bg = its first column of B
-    __device__ __forceinline__ void request(Staged& s, const float* Ag, const float* Bg, int K, int N, int k0) const {
+    // Whole tiles: Ag = the tile's first row of A, Bg = its first column of B.  A lane's byte offsets inside a slice are
+    // the same for the whole k loop (offsets(), kept in registers); the slice moves the base of two buffer descriptors,
+    // which is scalar arithmetic -- with a 64-bit address per load the vector unit spent two additions on each of them
+    // between the multiply-adds (4096^3: 941 -> 914 us).  (TM x K and 32 x N floats stay below the 2 GiB the descriptors span.)
+    struct Offsets { unsigned a[N_STAGED], b[N_STAGED]; };
+    __device__ __forceinline__ Offsets offsets(int K, int N) const {
+        Offsets o;
 #pragma unroll
         for (int i = 0; i < N_STAGED; i++) {
-            s.a[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * K + k0 + a_col);
-            s.b[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + B_STEP * i) * N + b_col);
+            o.a[i] = (unsigned)(((a_row + 32 * i) * K + a_col) * 4);
+            o.b[i] = (unsigned)(((b_row + B_STEP * i) * N + b_col) * 4);
+        }
+        return o;
+    }
+    __device__ __forceinline__ void request(Staged& s, const Offsets& o, const float* Ag, const float* Bg, int N, int k0) const {
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)(Ag + k0), 0, 0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)(Bg + (int64_t)k0 * N), 0, 0x80000000u, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < N_STAGED; i++) {
+            s.a[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, o.a[i], 0, 0)));
+            s.b[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rb, o.b[i], 0, 0)));
         }
     }
-    // any shape: through buffer descriptors over the whole matrices (nothing past their end is touched, the range check
-    // returns 0 there); rows past the edge and k rows past the end are clamped, columns past the edge left as they come:
-    // all of these only feed results that are not stored, once zero_tail has cleared the k tail
-    __device__ __forceinline__ void request_edge(Staged& s, __amdgpu_buffer_rsrc_t Abuf, __amdgpu_buffer_rsrc_t Bbuf, int M, int K, int N,
-                                                 int row0, int col0, int k0) const {
+    // any shape: through buffer descriptors that end where the matrices end (nothing past their end is touched, the range
+    // check returns 0 there); rows past the edge are clamped, columns past the edge left as they come: all of these only
+    // feed results that are not stored, once zero_tail has cleared the k tail
+    // (offsets of a lane's pieces from the first element of the matrices, rows past the edge clamped: fixed for the k loop)
+    __device__ __forceinline__ Offsets edge_offsets(int M, int K, int N, int row0, int col0) const {
+        Offsets o;
 #pragma unroll
         for (int i = 0; i < N_STAGED; i++) {
             int row = row0 + a_row + 32 * i; if (row > M - 1) row = M - 1;
-            s.a[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * K + k0 + a_col) * 4u, 0, 0)));
-            const int kb = k0 + b_row + B_STEP * i;
-            const int krow = kb < K ? kb : K - 1;
-            s.b[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * N + col0 + b_col) * 4u, 0, 0)));
+            o.a[i] = (unsigned)(row * K + a_col) * 4u;
+            o.b[i] = (unsigned)((b_row + B_STEP * i) * N + col0 + b_col) * 4u;
+        }
+        return o;
+    }
+    // the slice in the base of the descriptors, which end where the matrices end: k rows of B past the end read as 0
+    __device__ __forceinline__ void request_edge(Staged& s, const Offsets& o, const float* A, const float* B, int M, int K, int N, int k0) const {
+        const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)(A + k0), 0, (unsigned)(((int64_t)M * K - k0) * 4), 0x00020000);
+        const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc((void*)(B + (int64_t)k0 * N), 0, (unsigned)((int64_t)(K - k0) * N * 4), 0x00020000);
+#pragma unroll
+        for (int i = 0; i < N_STAGED; i++) {
+            s.a[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, o.a[i], 0, 0)));
+            s.b[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rb, o.b[i], 0, 0)));
         }
     }
     __device__ __forceinline__ void zero_tail(Staged& s, int K, int k0) const {
@@ -220,11 +245,10 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
 
     const Tile128 tile(tid);
     Tile128::Staged staged;
-    const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 4), 0x00020000);
-    const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 4), 0x00020000);
+    const Tile128::Offsets offs = EDGE ? tile.edge_offsets(g.M, g.K, g.N, tm * BM, tn * BN) : tile.offsets(g.K, g.N);
     auto load_global = [&](int k0) {
-        if (!EDGE) tile.request(staged, Ag, Bg, g.K, g.N, k0);
-        else tile.request_edge(staged, Abuf, Bbuf, g.M, g.K, g.N, tm * BM, tn * BN, k0);
+        if (!EDGE) tile.request(staged, offs, Ag, Bg, g.N, k0);
+        else tile.request_edge(staged, offs, A, B, g.M, g.K, g.N, k0);
     };
     // k0: the slice the staging registers hold.  The k tail is zeroed here, a slice after the request, and only in the one
     // slice that has a tail (a block-uniform branch): zeroed at the request, every slice would wait for its loads there
@@ -387,11 +411,20 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 * i
     const int b_row = tid >> 4, b_col = (tid & 15) * 4;     // rows b_row + 16 * i
     f32x4 ra[2], rb[2];
+    // (fixed byte offsets per lane, the slice in the base of the descriptors: see TileF32::request)
+    unsigned off_a[2], off_b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        off_a[i] = (unsigned)(((a_row + 32 * i) * g.K + a_col) * 4);
+        off_b[i] = (unsigned)(((b_row + 16 * i) * g.N + b_col) * 4);
+    }
     auto load_global = [&](int k0) {
+        const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc((void*)(Ag + k0), 0, 0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc((void*)(Bg + (int64_t)k0 * g.N), 0, 0x80000000u, 0x00020000);
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 16 * i) * g.N + b_col);
+            ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(da, off_a[i], 0, 0)));
+            rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(db, off_b[i], 0, 0)));
         }
     };
     auto store_lds = [&](int stage) {
@@ -491,11 +524,20 @@ __global__ __launch_bounds__(256 * KG) void matmul_mfma64_split_kernel(MfmaArgs 
     const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 * i
     const int b_row = tid >> 4, b_col = (tid & 15) * 4;     // rows b_row + 16 * i
     f32x4 ra[2], rb[2];
+    // (fixed byte offsets per lane, the slice in the base of the descriptors: see TileF32::request)
+    unsigned off_a[2], off_b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        off_a[i] = (unsigned)(((a_row + 32 * i) * g.K + a_col) * 4);
+        off_b[i] = (unsigned)(((b_row + 16 * i) * g.N + b_col) * 4);
+    }
     auto load_global = [&](int k0) {
+        const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc((void*)(Ag + k0), 0, 0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc((void*)(Bg + (int64_t)k0 * g.N), 0, 0x80000000u, 0x00020000);
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            ra[i] = *(const f32x4*)(Ag + (int64_t)(a_row + 32 * i) * g.K + k0 + a_col);
-            rb[i] = *(const f32x4*)(Bg + (int64_t)(k0 + b_row + 16 * i) * g.N + b_col);
+            ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(da, off_a[i], 0, 0)));
+            rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(db, off_b[i], 0, 0)));
         }
     };
     auto store_lds = [&](int stage) {
@@ -594,7 +636,8 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_stream_kernel(MfmaArgs g, 
     const int l32 = lane & 31, h = lane >> 5;
     const Tile128 stage(tid);
     Tile128::Staged staged;
-    auto load_global = [&](int tm, int tn, int k0) { stage.request(staged, A + (int64_t)tm * BM * g.K, B + (int64_t)tn * BN, g.K, g.N, k0); };
+    const Tile128::Offsets offs = stage.offsets(g.K, g.N);
+    auto load_global = [&](int tm, int tn, int k0) { stage.request(staged, offs, A + (int64_t)tm * BM * g.K, B + (int64_t)tn * BN, g.N, k0); };
     auto store_lds = [&](int buf) { stage.store(staged, As0 + buf * Tile128::A_FLOATS, Bs0 + buf * Tile128::B_FLOATS); };
     using Frag = Tile128::Frag;
     auto read_frag = [&](Frag& f, int buf, int c) { Tile128::read(f, As0 + buf * Tile128::A_FLOATS, Bs0 + buf * Tile128::B_FLOATS, wm, wn, l32, h, c); };
@@ -713,11 +756,10 @@ __global__ __launch_bounds__(256, 1) void matmul_mfma_big_kernel(MfmaArgs g, con
     const float* Bg = B + (int64_t)tn * TN;
     const Tile tile(tid);
     Tile::Staged staged;
-    const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 4), 0x00020000);
-    const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 4), 0x00020000);
+    const typename Tile::Offsets offs = EDGE ? tile.edge_offsets(g.M, g.K, g.N, tm * TM, tn * TN) : tile.offsets(g.K, g.N);
     auto load_global = [&](int k0) {
-        if (!EDGE) tile.request(staged, Ag, Bg, g.K, g.N, k0);
-        else tile.request_edge(staged, Abuf, Bbuf, g.M, g.K, g.N, tm * TM, tn * TN, k0);
+        if (!EDGE) tile.request(staged, offs, Ag, Bg, g.N, k0);
+        else tile.request_edge(staged, offs, A, B, g.M, g.K, g.N, k0);
     };
     // k0: the slice the staging registers hold.  The k tail is zeroed here, a slice after the request, and only in the
     // one slice that has a tail (a block-uniform branch): zeroing at the request would make every slice wait for its loads.
@@ -1437,22 +1479,25 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
     const int b_row = tid >> 6, b_col = (tid & 63) * 2;      // rows b_row + 4*i
     f64x2 ra[4], rb[4];
     typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-    const __amdgpu_buffer_rsrc_t Abuf = __builtin_amdgcn_make_buffer_rsrc((void*)A, 0, (unsigned)((int64_t)g.M * g.K * 8), 0x00020000);
-    const __amdgpu_buffer_rsrc_t Bbuf = __builtin_amdgcn_make_buffer_rsrc((void*)B, 0, (unsigned)((int64_t)g.K * g.N * 8), 0x00020000);
+    // A lane's byte offsets inside a slice are fixed for the k loop; the slice moves the base of two buffer descriptors
+    // (scalar arithmetic instead of a 64-bit vector addition per load).  EDGE: offsets from the first element of the
+    // matrices with the rows past the edge clamped, descriptors that end where the matrices end (k rows of B past the
+    // end read as 0); whole tiles: offsets from the tile's first row and column.
+    unsigned off_a[4], off_b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int row = tm * BM + a_row + 32 * i;
+        if (EDGE && row > g.M - 1) row = g.M - 1;
+        off_a[i] = (unsigned)(row * g.K + a_col) * 8u;
+        off_b[i] = (unsigned)((b_row + 4 * i) * g.N + tn * BN + b_col) * 8u;
+    }
     auto load_global = [&](int k0) {
+        const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc((void*)(A + k0), 0, EDGE ? (unsigned)(((int64_t)g.M * g.K - k0) * 8) : 0xffffffffu, 0x00020000);
+        const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc((void*)(B + (int64_t)k0 * g.N), 0, EDGE ? (unsigned)((int64_t)(g.K - k0) * g.N * 8) : 0xffffffffu, 0x00020000);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            if (!EDGE) {
-                ra[i] = *(const f64x2*)(A + ((int64_t)tm * BM + a_row + 32 * i) * g.K + k0 + a_col);
-                rb[i] = *(const f64x2*)(B + (int64_t)(k0 + b_row + 4 * i) * g.N + tn * BN + b_col);
-            } else {
-                int row = tm * BM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
-                const int ka = k0 + a_col;
-                ra[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Abuf, (unsigned)(row * g.K + ka) * 8u, 0, 0)));
-                const int kb = k0 + b_row + 4 * i;
-                const int krow = kb < g.K ? kb : g.K - 1;
-                rb[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(Bbuf, (unsigned)(krow * g.N + tn * BN + b_col) * 8u, 0, 0)));
-            }
+            ra[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(da, off_a[i], 0, 0)));
+            rb[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(db, off_b[i], 0, 0)));
         }
     };
     // k0: the slice the staging registers hold; its k tail is zeroed here, a slice after the request, and only in the one
@@ -1825,7 +1870,8 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         return launch_simple<double>(dev, M, K, N, overwrite, (const double*)A, (const double*)B, (double*)C);
     }
     const bool aligned = (A % 16 == 0) && (B % 16 == 0) && (C % 16 == 0);
-    const bool whole_tiles = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0;
+    // (the whole-tile kernels address a slice with 32-bit byte offsets from its first element: 256 rows of A, 32 rows of B)
+    const bool whole_tiles = aligned && M % BM == 0 && N % BN == 0 && K % BK == 0 && K < ((int64_t)1 << 20) && N < ((int64_t)1 << 23);
     // Small products stay on the simple kernel, which keeps the reference's summation order bit for bit; from
     // 2^24 multiply-adds on, shapes that are not whole tiles take the matrix cores through the edge variant.
     const bool edge = !whole_tiles && M * K * N >= mfma_from && M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);
