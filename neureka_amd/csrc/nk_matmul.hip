@@ -1532,32 +1532,60 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
     int nk = all_slices;
     if (SPLIT) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
     const int kbase = slice0 * DK;
+    // Software pipeline over the k-slices, as in the f32 kernels: while the matrix cores work on chunk c (depth 4, sixteen
+    // multiply-adds) the operands of chunk c + 1 are read from LDS -- behind the first multiply-adds of the chunk, pinned
+    // with scheduling groups, or the compiler sinks the reads behind all sixteen; the next slice, requested at the top of
+    // the slice, is written to the other LDS buffer before the last chunk's multiply-adds, and the barrier sits there
+    // too, so that the first chunk of the next slice is read under them and no slice begins by waiting for LDS.
+    static_assert(DK == 16, "the pipeline below is written for four depth-4 chunks per slice");
+    struct Frag64 { double a[4], b[4]; };
+    auto read_frag = [&](Frag64& f, int buf, int c) {
+        const double* as = As0 + buf * (BM * DA_PITCH);
+        const double* bs = Bs0 + buf * (DK * DB_PITCH);
+#pragma unroll
+        for (int i = 0; i < 4; i++) f.a[i] = as[(wm + 16 * i + l16) * DA_PITCH + 4 * c + q];
+#pragma unroll
+        for (int j = 0; j < 4; j++) f.b[j] = bs[(4 * c + q) * DB_PITCH + wn + 16 * j + l16];
+    };
+    auto mma = [&](const Frag64& f) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+    };
+#define NK_D_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
+#define NK_D_READ(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
+#define NK_D_CHUNK NK_D_MFMA(1); NK_D_READ(2); NK_D_MFMA(1); NK_D_READ(2); NK_D_MFMA(1); NK_D_READ(2); NK_D_MFMA(1); NK_D_READ(2); NK_D_MFMA(12); __builtin_amdgcn_sched_barrier(0)
+    Frag64 f0, f1;
     load_global(kbase);
     store_lds(0, kbase);
     __syncthreads();
+    read_frag(f0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
     for (int kt = 0; kt < nk; kt++) {
         const int cur = kt & 1;
         const bool more = kt + 1 < nk;
         if (more) load_global(kbase + (kt + 1) * DK);
-        const double* as = As0 + cur * (BM * DA_PITCH);
-        const double* bs = Bs0 + cur * (DK * DB_PITCH);
-#pragma unroll
-        for (int c = 0; c < DK / 4; c++) {
-            double a[4], b[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) a[i] = as[(wm + 16 * i + l16) * DA_PITCH + 4 * c + q];
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[j] = bs[(4 * c + q) * DB_PITCH + wn + 16 * j + l16];
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
+        read_frag(f1, cur, 1);
+        mma(f0);
+        NK_D_CHUNK;
+        read_frag(f0, cur, 2);
+        mma(f1);
+        NK_D_CHUNK;
+        read_frag(f1, cur, 3);
+        mma(f0);
+        NK_D_CHUNK;
         if (more) {
             store_lds(cur ^ 1, kbase + (kt + 1) * DK);
             __syncthreads();
+            read_frag(f0, cur ^ 1, 0);
         }
+        mma(f1);
+        __builtin_amdgcn_sched_barrier(0);
     }
+#undef NK_D_CHUNK
+#undef NK_D_READ
+#undef NK_D_MFMA
 
     // epilogue: C is accumulated into; a quarter-wavefront covers 16 consecutive doubles of a row
     const int rows = g.M - tm * BM, cols = g.N - tn * BN;
