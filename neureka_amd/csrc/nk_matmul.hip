@@ -481,12 +481,18 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
         read_chunk(f2, cur, 2);
         read_chunk(f3, cur, 3);
         mma(f0, f1);
-        __builtin_amdgcn_sched_barrier(0);
+        // The order of issue is pinned (left to the compiler, the reads of chunks 2 and 3 sat right before their first use
+        // and the reads of the next slice right before the barrier: 0.71 of the matrix rate in the k loop, 0.84 pinned).
+        // The six LDS reads of chunks 2 and 3 behind the first three multiply-adds of chunks 0 and 1 ...
+        NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(5); NK_FENCE;
         store_lds(write);
         load_global(clamped(kt + 3));
         read_chunk(f0, next, 0);
         read_chunk(f1, next, 1);
         mma(f2, f3);
+        // ... one LDS write and one request behind each of the next four, the reads of the next slice behind three more
+        NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1);
+        NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_FENCE;
         __syncthreads();
         cur = next;
     }
@@ -499,122 +505,6 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     for (int v = 0; v < 16; v++) {
         float* p = Cg + (int64_t)(8 * (v >> 2) + 4 * h + (v & 3)) * g.N;
         *p = OVERWRITE ? acc[v] : *p + acc[v];
-    }
-}
-
-// The same tiles with the k range split inside the block: KG groups of four wavefronts, each group the kernel above on
-// its own part of the k range with its own three stages of LDS, so that every SIMD holds KG wavefronts.  The groups meet
-// once, at the end, in LDS, where the first adds the others' accumulators in order and stores the tile.  K % (32 KG) == 0;
-// KG x 52.5 KiB of LDS, asked for at the launch.  1024^3: 26.5 -> 24.2 us, 1024 x 2048 x 1024: 49.4 -> 43.7 (the matrix
-// instructions alone, with no loads at all, take 19.1 and 33.4 in this kernel).
-template <bool OVERWRITE, int KG>
-__global__ __launch_bounds__(256 * KG) void matmul_mfma64_split_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C) {
-    using namespace t64;
-    extern __shared__ __attribute__((aligned(16))) float split_lds[];
-    int tm, tn;
-    tile_of_block(g, (int)blockIdx.x, tm, tn);
-    const int grp = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8);
-    const int tid = threadIdx.x & 255;
-    float* const lds = split_lds + grp * t64::LDS_FLOATS;
-    const int wave = tid >> 6, lane = tid & 63;
-    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
-    const int l32 = lane & 31, h = lane >> 5;
-    const float* Ag = A + (int64_t)tm * TM * g.K;
-    const float* Bg = B + (int64_t)tn * TN;
-    const int a_row = tid >> 3, a_col = (tid & 7) * 4;      // rows a_row + 32 * i
-    const int b_row = tid >> 4, b_col = (tid & 15) * 4;     // rows b_row + 16 * i
-    f32x4 ra[2], rb[2];
-    // (fixed byte offsets per lane, the slice in the base of the descriptors: see TileF32::request)
-    unsigned off_a[2], off_b[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        off_a[i] = (unsigned)(((a_row + 32 * i) * g.K + a_col) * 4);
-        off_b[i] = (unsigned)(((b_row + 16 * i) * g.N + b_col) * 4);
-    }
-    auto load_global = [&](int k0) {
-        const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc((void*)(Ag + k0), 0, 0x80000000u, 0x00020000);
-        const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc((void*)(Bg + (int64_t)k0 * g.N), 0, 0x80000000u, 0x00020000);
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(da, off_a[i], 0, 0)));
-            rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(db, off_b[i], 0, 0)));
-        }
-    };
-    auto store_lds = [&](int stage) {
-        float* as = lds + stage * STAGE;
-        float* bs = as + TM * A_P;
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            *(f32x4*)(&as[(a_row + 32 * i) * A_P + a_col]) = ra[i];
-            *(f32x4*)(&bs[(b_row + 16 * i) * B_P + b_col]) = rb[i];
-        }
-    };
-    struct Chunk { f32x4 a; float b[4]; };
-    auto read_chunk = [&](Chunk& f, int stage, int c) {
-        const float* as = lds + stage * STAGE;
-        const float* bs = as + TM * A_P;
-        f.a = *(const f32x4*)(&as[(wm + l32) * A_P + 8 * c + 4 * h]);
-#pragma unroll
-        for (int t = 0; t < 4; t++) f.b[t] = bs[(8 * c + 4 * h + t) * B_P + wn + l32];
-    };
-    f32x16 acc0, acc1;
-#pragma unroll
-    for (int v = 0; v < 16; v++) { acc0[v] = 0.0f; acc1[v] = 0.0f; }
-    auto mma = [&](const Chunk& even, const Chunk& odd) {
-#pragma unroll
-        for (int t = 0; t < 4; t++) {
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(even.a[t], even.b[t], acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(odd.a[t], odd.b[t], acc1, 0, 0, 0);
-        }
-    };
-    const int nk = g.K / BK / KG;                             // slices of a group: the same for every group, so every wavefront
-    const int kbase = grp * nk * BK;                          // of the block reaches every barrier
-    auto clamped = [&](int slice) { return kbase + (slice < nk ? slice : nk - 1) * BK; };
-    load_global(clamped(0));
-    store_lds(0);
-    load_global(clamped(1));
-    store_lds(1);
-    load_global(clamped(2));
-    __syncthreads();
-    Chunk f0, f1, f2, f3;
-    read_chunk(f0, 0, 0);
-    read_chunk(f1, 0, 1);
-    int cur = 0;
-    for (int kt = 0; kt < nk; kt++) {
-        const int next = cur == 2 ? 0 : cur + 1, write = next == 2 ? 0 : next + 1;
-        read_chunk(f2, cur, 2);
-        read_chunk(f3, cur, 3);
-        mma(f0, f1);
-        __builtin_amdgcn_sched_barrier(0);
-        store_lds(write);
-        load_global(clamped(kt + 3));
-        read_chunk(f0, next, 0);
-        read_chunk(f1, next, 1);
-        mma(f2, f3);
-        __syncthreads();
-        cur = next;
-    }
-    f32x16 acc;
-#pragma unroll
-    for (int v = 0; v < 16; v++) acc[v] = acc0[v] + acc1[v];
-    // the meeting: nobody reads a stage any more (every read was waited for before the loop's last barrier); element v of
-    // thread tid of group grp > 0 sits at (v (KG - 1) + grp - 1) 256 + tid
-    if (grp > 0) {
-#pragma unroll
-        for (int v = 0; v < 16; v++) split_lds[(v * (KG - 1) + grp - 1) * 256 + tid] = acc[v];
-    }
-    __syncthreads();
-    if (grp == 0) {
-#pragma unroll
-        for (int v = 0; v < 16; v++)
-#pragma unroll
-            for (int o = 0; o < KG - 1; o++) acc[v] += split_lds[(v * (KG - 1) + o) * 256 + tid];
-        float* Cg = C + (int64_t)(tm * TM + wm) * g.N + tn * TN + wn + l32;
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            float* p = Cg + (int64_t)(8 * (v >> 2) + 4 * h + (v & 3)) * g.N;
-            *p = OVERWRITE ? acc[v] : *p + acc[v];
-        }
     }
 }
 
@@ -1663,22 +1553,18 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
 
 // `force_parts`, `bands`: how matmul_rm calls itself for the two row bands described below (callers leave them alone: `bands`
 // is true for a caller's product, which may be planned as bands or take one of the streaming kernels, and false for a band)
-// Kernels that need more LDS than a launch gets by default (the 256 x 256 tiles: 137 KiB; the 64 x 64 tiles with the k
-// range split inside the block: 105 KiB): asked for once per device; a device that does not grant it (or has less) keeps to
-// the other plans.  Device::big_tiles: 0 not asked yet, 1 granted, -1 not available.
-constexpr int T64_SPLIT = 2;
-constexpr int T64_SPLIT_LDS_BYTES = T64_SPLIT * t64::LDS_FLOATS * (int)sizeof(float);
+// The 256 x 256 tiles need more LDS (137 KiB) than a launch gets by default: asked for once per device; a device that does
+// not grant it (or has less) keeps to the other plans.  Device::big_tiles: 0 not asked yet, 1 granted, -1 not available.
 static bool large_lds(Device* dev) {
     if (dev->big_tiles == 0) {
         dev->big_tiles = -1;
         constexpr int big_bytes = big::LDS_FLOATS * (int)sizeof(float);
         if ((int64_t)dev->props.sharedMemPerBlockOptin >= big_bytes) {
-            const void* kernels[6] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
-                                      (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>,
-                                      (const void*)matmul_mfma64_split_kernel<true, T64_SPLIT>, (const void*)matmul_mfma64_split_kernel<false, T64_SPLIT>};
+            const void* kernels[4] = {(const void*)matmul_mfma_big_kernel<true, false>, (const void*)matmul_mfma_big_kernel<false, false>,
+                                      (const void*)matmul_mfma_big_kernel<true, true>, (const void*)matmul_mfma_big_kernel<false, true>};
             hipError_t attr = hipSuccess;
-            for (int k = 0; k < 6; k++)
-                if (attr == hipSuccess) attr = hipFuncSetAttribute(kernels[k], hipFuncAttributeMaxDynamicSharedMemorySize, k < 4 ? big_bytes : T64_SPLIT_LDS_BYTES);
+            for (const void* k : kernels)
+                if (attr == hipSuccess) attr = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, big_bytes);
             if (attr == hipSuccess) dev->big_tiles = 1; else (void)hipGetLastError();
         }
     }
@@ -1940,23 +1826,16 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         if (bands && force_parts < 2 && aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0 && K >= 4 * BK) {
             const int64_t cus = dev->props.multiProcessorCount;
             const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = (M / t64::TM) * (N / t64::TN);
-            // (against the k range of the large tiles cut into parts: 1024^3 78 against 69 TFLOP/s; with more large tiles or a
-            // long k range the parts win: 1536^3 83 against 89, 1024 x 4096 x 1024 89 against 104)
-            if (large <= cus / 4 && small >= cus && K <= 2048) {
+            // (against the k range of the large tiles cut into parts: 1024^3 102 against 69 TFLOP/s, 1024 x 4096 x 1024 120
+            // against 115; with more large tiles the parts win: 1536^3 83 against 96)
+            if (large <= cus / 4 && small >= cus) {
                 MfmaArgs gs = g;
                 gs.tiles_m = (int)(M / t64::TM); gs.tiles_n = (int)(N / t64::TN);
                 gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
-                // two wavefronts per SIMD, each group of four on its half of the k range (at least four slices each)
-                const bool split = K % (T64_SPLIT * BK) == 0 && K >= T64_SPLIT * 4 * BK && large_lds(dev);
-                if (split) {
-                    if (overwrite) hipLaunchKernelGGL((matmul_mfma64_split_kernel<true, T64_SPLIT>), dim3((unsigned)small), dim3(256 * T64_SPLIT), T64_SPLIT_LDS_BYTES, dev->stream, gs, Ap, Bp, Cp);
-                    else           hipLaunchKernelGGL((matmul_mfma64_split_kernel<false, T64_SPLIT>), dim3((unsigned)small), dim3(256 * T64_SPLIT), T64_SPLIT_LDS_BYTES, dev->stream, gs, Ap, Bp, Cp);
-                } else {
-                    if (overwrite) hipLaunchKernelGGL(matmul_mfma64_kernel<true>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                    else           hipLaunchKernelGGL(matmul_mfma64_kernel<false>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                }
+                if (overwrite) hipLaunchKernelGGL(matmul_mfma64_kernel<true>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                else           hipLaunchKernelGGL(matmul_mfma64_kernel<false>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
                 NK_HIP(hipGetLastError());
-                set_path(split ? "mfma_tiles_of_64_split" : "mfma_tiles_of_64");
+                set_path("mfma_tiles_of_64");
                 return NK_OK;
             }
         }

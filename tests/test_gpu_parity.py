@@ -1797,7 +1797,7 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
     ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64"),
     ("f32", (4100, 9, 4096), "short_inner"), ("f64", (4096, 16, 2050), "short_inner_f64"),
     ("f32", (32, 2048, 2048), "few_rows"), ("f64", (20, 4096, 512), "few_rows_f64"),
-    ("f32", (1024, 1024, 1024), "mfma_tiles_of_64_split"), ("f32", (1024, 288, 1024), "mfma_tiles_of_64")])
+    ("f32", (1024, 1024, 1024), "mfma_tiles_of_64"), ("f32", (1024, 288, 1024), "mfma_tiles_of_64")])
 def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mkn, path):
     """nk_matmul_set (C = A @ B, the OpenCL device's `C[n + m*N] = acc`, CLMatMul.java:50) on every kernel plan, both
     layouts: the drain starts as NaN everywhere, so a single old value read would show; the result must equal, bit for
@@ -1862,13 +1862,12 @@ def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
     assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
-@pytest.mark.parametrize("mkn,path", [((1024, 1024, 1024), "mfma_tiles_of_64_split"), ((1024, 320, 1024), "mfma_tiles_of_64_split"),
-                                      ((512, 2048, 2048), "mfma_tiles_of_64_split"), ((1024, 256, 1024), "mfma_tiles_of_64_split"),
+@pytest.mark.parametrize("mkn,path", [((1024, 1024, 1024), "mfma_tiles_of_64"), ((1024, 320, 1024), "mfma_tiles_of_64"),
+                                      ((512, 4096, 2048), "mfma_tiles_of_64"), ((1024, 128, 1024), "mfma_tiles_of_64"),
                                       ((1024, 288, 1024), "mfma_tiles_of_64"), ((2048, 160, 512), "mfma_tiles_of_64")])
 def test_matmul_64_tiles_in_one_launch(device, mkn, path):
     """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit: one launch of
-    the small-tile kernel -- with the k range split between two groups of wavefronts inside the block where it divides
-    into two runs of at least four slices, whole otherwise.  Integer data are exact against numpy in both layouts and
+    the small-tile kernel, from four k-slices up to long k ranges.  Integer data are exact against numpy in both layouts and
     through both entry points; uniform data stay within the norm-wise bound; operands inside larger buffers full of NaN
     show that nothing outside them is read."""
     M, K, N = mkn
