@@ -1826,9 +1826,22 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         if (bands && force_parts < 2 && aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0 && K >= 4 * BK) {
             const int64_t cus = dev->props.multiProcessorCount;
             const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = (M / t64::TM) * (N / t64::TN);
-            // (against the k range of the large tiles cut into parts: 1024^3 102 against 69 TFLOP/s, 1024 x 4096 x 1024 120
-            // against 115; with more large tiles the parts win: 1536^3 83 against 96)
-            if (large <= cus / 4 && small >= cus) {
+            // Against the k range of the large tiles cut into parts, by two estimates fitted to measurements (microseconds):
+            // the small tiles run in rounds of one per unit at 0.48 per k-slice plus 5; the parts cost 1.93 per unit of
+            // split_plan's estimate plus 8 for the second launch and the shorter blocks.  1024^3 21 against 29 (measured: 21,
+            // 31), 1536 x 256 x 1536 17 against 26 (17, 31), 1024 x 1024 x 3072 51 against 60 (53, 64); the parts win
+            // 1152^3 36 against 40 (35, 39), 1792^3 108 against 113 (108, 111), 1280 x 4096 x 1280 116 against 128 (107, 127).
+            bool small_tiles = large < cus;
+            if (small_tiles) {
+                const int64_t slices = K / BK;
+                const double t_small = 0.48 * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
+                MfmaArgs trial = g;
+                const double t_parts = split_plan(dev, trial, BK, sizeof(float), 0) > 1
+                    ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
+                    : 1.93 * (double)slices + 7.0;
+                small_tiles = t_small < t_parts;
+            }
+            if (small_tiles) {
                 MfmaArgs gs = g;
                 gs.tiles_m = (int)(M / t64::TM); gs.tiles_n = (int)(N / t64::TN);
                 gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
