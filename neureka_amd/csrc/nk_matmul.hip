@@ -396,7 +396,10 @@ constexpr int A_P = BK + 4, B_P = TN + 4;                    // floats; rows sta
 constexpr int STAGE = TM * A_P + BK * B_P;                   // one k-slice of A and of B
 constexpr int LDS_FLOATS = 3 * STAGE;
 }
-template <bool OVERWRITE>
+// EDGE: any M, N, K and any (element-aligned) operands, as in the larger kernels: offsets from the first element of the
+// matrices with the rows past the edge clamped, descriptors that end where the matrices end (k rows of B past the end
+// read as 0), the k tail of A zeroed at the LDS write of the one slice that has it, stores guarded element by element.
+template <bool OVERWRITE, bool EDGE = false>
 __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C) {
     using namespace t64;
     __shared__ __attribute__((aligned(16))) float lds[t64::LDS_FLOATS];
@@ -415,19 +418,36 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     unsigned off_a[2], off_b[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        off_a[i] = (unsigned)(((a_row + 32 * i) * g.K + a_col) * 4);
-        off_b[i] = (unsigned)(((b_row + 16 * i) * g.N + b_col) * 4);
+        if (EDGE) {
+            int row = tm * TM + a_row + 32 * i; if (row > g.M - 1) row = g.M - 1;
+            off_a[i] = (unsigned)(row * g.K + a_col) * 4u;
+            off_b[i] = (unsigned)((b_row + 16 * i) * g.N + tn * TN + b_col) * 4u;
+        } else {
+            off_a[i] = (unsigned)(((a_row + 32 * i) * g.K + a_col) * 4);
+            off_b[i] = (unsigned)(((b_row + 16 * i) * g.N + b_col) * 4);
+        }
     }
     auto load_global = [&](int k0) {
-        const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc((void*)(Ag + k0), 0, 0x80000000u, 0x00020000);
-        const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc((void*)(Bg + (int64_t)k0 * g.N), 0, 0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t da = EDGE ? __builtin_amdgcn_make_buffer_rsrc((void*)(A + k0), 0, (unsigned)(((int64_t)g.M * g.K - k0) * 4), 0x00020000)
+                                               : __builtin_amdgcn_make_buffer_rsrc((void*)(Ag + k0), 0, 0x80000000u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t db = EDGE ? __builtin_amdgcn_make_buffer_rsrc((void*)(B + (int64_t)k0 * g.N), 0, (unsigned)((int64_t)(g.K - k0) * g.N * 4), 0x00020000)
+                                               : __builtin_amdgcn_make_buffer_rsrc((void*)(Bg + (int64_t)k0 * g.N), 0, 0x80000000u, 0x00020000);
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             ra[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(da, off_a[i], 0, 0)));
             rb[i] = __builtin_bit_cast(f32x4, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(db, off_b[i], 0, 0)));
         }
     };
-    auto store_lds = [&](int stage) {
+    // k0: the slice the staging registers hold (EDGE: its k tail is zeroed here, in the one slice that has it)
+    auto store_lds = [&](int stage, int k0) {
+        if (EDGE && k0 + BK > g.K) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (k0 + a_col + e >= g.K) ra[i][e] = 0.0f;
+                if (k0 + b_row + 16 * i >= g.K) rb[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
         float* as = lds + stage * STAGE;
         float* bs = as + TM * A_P;
 #pragma unroll
@@ -460,12 +480,12 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     // slice publishes the writes one slice before anybody reads them, so the first chunks of slice kt + 1 are read before
     // that barrier, behind the last multiply-adds of slice kt: no wavefront starts a slice by waiting for LDS, which the
     // single wavefront of a SIMD could hide behind nothing.
-    const int nk = g.K / BK;
+    const int nk = (g.K + BK - 1) / BK;
     auto clamped = [&](int slice) { return (slice < nk ? slice : nk - 1) * BK; };     // past the end: the last slice again, read by nobody
     load_global(0);
-    store_lds(0);
+    store_lds(0, 0);
     load_global(clamped(1));
-    store_lds(1);
+    store_lds(1, clamped(1));
     load_global(clamped(2));                                  // slice 2 waits in the staging registers
     __syncthreads();
     Chunk f0, f1, f2, f3;
@@ -485,7 +505,7 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
         // and the reads of the next slice right before the barrier: 0.71 of the matrix rate in the k loop, 0.84 pinned).
         // The six LDS reads of chunks 2 and 3 behind the first three multiply-adds of chunks 0 and 1 ...
         NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(5); NK_FENCE;
-        store_lds(write);
+        store_lds(write, clamped(kt + 2));
         load_global(clamped(kt + 3));
         read_chunk(f0, next, 0);
         read_chunk(f1, next, 1);
@@ -501,10 +521,14 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     for (int v = 0; v < 16; v++) acc[v] = acc0[v] + acc1[v];
     // accumulator v sits at row 8 * (v / 4) + 4 * h + v % 4, column l32 of the wavefront's 32 x 32 tile
     float* Cg = C + (int64_t)(tm * TM + wm) * g.N + tn * TN + wn + l32;
+    const int rows = g.M - (tm * TM + wm), cols = g.N - (tn * TN + wn + l32);      // EDGE: what is left of C from the lane's first element
 #pragma unroll
     for (int v = 0; v < 16; v++) {
-        float* p = Cg + (int64_t)(8 * (v >> 2) + 4 * h + (v & 3)) * g.N;
-        *p = OVERWRITE ? acc[v] : *p + acc[v];
+        const int r = 8 * (v >> 2) + 4 * h + (v & 3);
+        if (!EDGE || (r < rows && cols > 0)) {
+            float* p = Cg + (int64_t)r * g.N;
+            *p = OVERWRITE ? acc[v] : *p + acc[v];
+        }
     }
 }
 
@@ -1823,9 +1847,11 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             }
         }
         // fewer large tiles than compute units, but whole 64 x 64 tiles, at least one per unit: the small-tile kernel in one launch
-        if (bands && force_parts < 2 && aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0 && K >= 4 * BK) {
+        const bool whole_small = aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0;
+        const bool fits_32_bits = M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);       // (the edge kernels' offsets)
+        if (bands && force_parts < 2 && (whole_small || fits_32_bits) && K >= 4 * BK) {
             const int64_t cus = dev->props.multiProcessorCount;
-            const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = (M / t64::TM) * (N / t64::TN);
+            const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
             // Against the k range of the large tiles cut into parts, by two estimates fitted to measurements (microseconds):
             // the small tiles run in rounds of one per unit at 0.48 per k-slice plus 5; the parts cost 1.93 per unit of
             // split_plan's estimate plus 8 for the second launch and the shorter blocks.  1024^3 21 against 29 (measured: 21,
@@ -1833,22 +1859,28 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             // 1152^3 36 against 40 (35, 39), 1792^3 108 against 113 (108, 111), 1280 x 4096 x 1280 116 against 128 (107, 127).
             bool small_tiles = large < cus;
             if (small_tiles) {
-                const int64_t slices = K / BK;
+                const int64_t slices = (K + BK - 1) / BK;
                 const double t_small = 0.48 * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
                 MfmaArgs trial = g;
                 const double t_parts = split_plan(dev, trial, BK, sizeof(float), 0) > 1
                     ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
                     : 1.93 * (double)slices + 7.0;
-                small_tiles = t_small < t_parts;
+                // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
+                small_tiles = t_small < (whole_tiles ? 1.0 : 1.15) * t_parts;
             }
             if (small_tiles) {
                 MfmaArgs gs = g;
-                gs.tiles_m = (int)(M / t64::TM); gs.tiles_n = (int)(N / t64::TN);
+                gs.tiles_m = (int)((M + t64::TM - 1) / t64::TM); gs.tiles_n = (int)((N + t64::TN - 1) / t64::TN);
                 gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
-                if (overwrite) hipLaunchKernelGGL(matmul_mfma64_kernel<true>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                else           hipLaunchKernelGGL(matmul_mfma64_kernel<false>, dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                if (whole_small) {
+                    if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, false>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, false>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                } else {
+                    if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, true>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                    else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, true>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
+                }
                 NK_HIP(hipGetLastError());
-                set_path("mfma_tiles_of_64");
+                set_path(whole_small ? "mfma_tiles_of_64" : "mfma_tiles_of_64_edge");
                 return NK_OK;
             }
         }

@@ -1625,12 +1625,12 @@ def test_matmul_mfma_edge_path(device, orc, mkn):
     C0 = rng.integers(-9, 10, (M, N)).astype(np.float32)
     tc = on(device, C0)
     device.launch_matmul(True, M, K, N, on(device, A), on(device, B), tc)
-    assert _lib.last_path().replace("_split", "") == "mfma_edge"
+    assert _lib.last_path().replace("_split", "") in ("mfma_edge", "mfma_tiles_of_64_edge")     # (64 x 64 tiles where the estimate prefers them)
     assert (tc.getData().reshape(M, N) == (A.astype(np.float64) @ B.astype(np.float64) + C0)).all()
     say("matmul mfma edge column major", mkn)
     tc = on(device, np.zeros((M, N), dtype=np.float32))
     device.launch_matmul(False, M, K, N, on(device, A.T.copy()), on(device, B.T.copy()), tc)
-    assert _lib.last_path().replace("_split", "") == "mfma_edge"
+    assert _lib.last_path().replace("_split", "") in ("mfma_edge", "mfma_tiles_of_64_edge")
     assert (tc.getData().reshape(N, M).T == A.astype(np.float64) @ B.astype(np.float64)).all()
     say("matmul mfma edge uniform", mkn)
     A = rng.uniform(-1, 1, (M, K)).astype(np.float32); B = rng.uniform(-1, 1, (K, N)).astype(np.float32)
@@ -1790,7 +1790,7 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
 
 @pytest.mark.parametrize("dt,mkn,path", [
     ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_split"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 256, 2048), "mfma"),
-    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (1000, 300, 520), "mfma_edge_split"), ("f32", (2100, 130, 2100), "mfma_edge"),
+    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 130, 2100), "mfma_edge"),
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
     ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
@@ -1864,10 +1864,13 @@ def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
 
 @pytest.mark.parametrize("mkn,path", [((1024, 1024, 1024), "mfma_tiles_of_64"), ((1024, 320, 1024), "mfma_tiles_of_64"),
                                       ((512, 4096, 2048), "mfma_tiles_of_64"), ((1024, 128, 1024), "mfma_tiles_of_64"),
-                                      ((1024, 288, 1024), "mfma_tiles_of_64"), ((2048, 160, 512), "mfma_tiles_of_64")])
+                                      ((1024, 288, 1024), "mfma_tiles_of_64"), ((2048, 160, 512), "mfma_tiles_of_64"),
+                                      ((1000, 1000, 1000), "mfma_tiles_of_64_edge"), ((777, 333, 1025), "mfma_tiles_of_64_edge"),
+                                      ((65, 1001, 4097), "mfma_tiles_of_64_edge"), ((1023, 129, 1025), "mfma_tiles_of_64_edge")])
 def test_matmul_64_tiles_in_one_launch(device, mkn, path):
     """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit: one launch of
-    the small-tile kernel, from four k-slices up to long k ranges.  Integer data are exact against numpy in both layouts and
+    the small-tile kernel, from four k-slices up to long k ranges, and its edge variant for shapes that are no whole
+    number of tiles or slices (odd row lengths: operands' rows are then not 16-byte aligned).  Integer data are exact against numpy in both layouts and
     through both entry points; uniform data stay within the norm-wise bound; operands inside larger buffers full of NaN
     show that nothing outside them is read."""
     M, K, N = mkn
@@ -1895,17 +1898,17 @@ def test_matmul_64_tiles_in_one_launch(device, mkn, path):
     bound = 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64))
     assert (np.abs(tc.getData().reshape(M, N).astype(np.float64) - ref) <= bound).all()
     say("matmul 64 tiles, operands inside larger buffers full of NaN", mkn)
-    pad = 64                                                                             # elements: keeps the 16-byte alignment
-    def parked(x):
-        host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
-        host[pad:pad + x.size] = x.reshape(-1)
-        return on(device, host)
-    pa, pb, pc = parked(A), parked(B), parked(np.zeros((M, N), dtype=np.float32))
-    _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
-    assert _lib.last_path() == path, _lib.last_path()
-    got = pc.getData()
-    assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
-    assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
+    for pad in (64,) + ((61,) if path.endswith("_edge") else ()):                     # elements: 64 keeps the 16-byte alignment, 61 breaks it
+        def parked(x):
+            host = np.full(x.size + 2 * pad, np.nan, dtype=np.float32)
+            host[pad:pad + x.size] = x.reshape(-1)
+            return on(device, host)
+        pa, pb, pc = parked(A), parked(B), parked(np.zeros((M, N), dtype=np.float32))
+        _lib.check(device._lib.nk_matmul(device.handle, 0, _lib.ROW_MAJOR, M, K, N, pa._data.ptr + 4 * pad, pb._data.ptr + 4 * pad, pc._data.ptr + 4 * pad))
+        assert _lib.last_path() == path, _lib.last_path()
+        got = pc.getData()
+        assert np.isnan(got[:pad]).all() and np.isnan(got[pad + M * N:]).all()            # nothing written outside C
+        assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
 @pytest.mark.parametrize("mkn", [(4096, 1024, 4096), (2048, 2048, 8192), (4096, 1056, 4096), (8192, 1024, 8192), (4096, 512, 4096)])
