@@ -207,7 +207,7 @@ constexpr int LDS_FLOATS = LDS_FLOATS_AB > LDS_FLOATS_C ? LDS_FLOATS_AB : LDS_FL
 template <bool EDGE, bool SPLIT = false, bool MIXED = false>
 __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const float* __restrict__ A,
                                                           const float* __restrict__ B, float* __restrict__ C, float* __restrict__ P = nullptr) {
-    static_assert(!MIXED || (!EDGE && !SPLIT), "the mixed launch is for whole tiles of an unsplit product");
+    static_assert(!MIXED || !SPLIT, "the mixed launch splits part of an unsplit product itself");
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     float* const As0 = lds;                                   // [2][BM * A_PITCH]
     float* const Bs0 = lds + 2 * BM * A_PITCH;                // [2][BK * B_PITCH]
@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256) void matmul_mfma_kernel(MfmaArgs g, const floa
                 const float* add = &cs[r * C_PITCH + c_col];
                 float* dst = Cg + (int64_t)r * g.N + c_col;
 #pragma unroll
-                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = (SPLIT || g.overwrite) ? add[e] : dst[e] + add[e];
+                for (int e = 0; e < 4; e++) if (c_col + e < cols) dst[e] = (parted || g.overwrite) ? add[e] : dst[e] + add[e];
             }
         }
         return;
@@ -1884,17 +1884,20 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 return NK_OK;
             }
         }
-        // A few more tiles than compute units: as one launch of whole tiles some units would work through two tiles side by
-        // side while the others finish with one.  Instead the upper tile rows, about one tile per unit, take the whole k
-        // range, and the tiles of the lower rows come as parts of their k range that fill the second places
-        // (matmul_mfma_kernel<false, false, true>); their sum follows as for every split product.  2304^3 (324 tiles): 278 ->
-        // 203 us; 2176 x 2048 x 2176: 247 -> 164; 2048 x 1024 x 2560: 126 -> 103.  With more than half a round of tiles in the
-        // lower rows it no longer pays (2560^3, 160 of 400 tiles: 310 -> 302; 4096 x 512 x 1536, 132 of 384: 68 -> 75).
-        if (bands && force_parts < 2 && whole_tiles) {
-            const int64_t cus = dev->props.multiProcessorCount, tiles = (int64_t)g.tiles_m * g.tiles_n, slices = K / BK;
-            const int64_t rows_a = cus / g.tiles_n;
+        if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;
+        // A few more tiles than a whole number of rounds of one tile per compute unit: as one launch of whole tiles some units
+        // would work through one tile more than the others (side by side with another).  Instead the upper tile rows, whole
+        // rounds, take the whole k range, and the tiles of the lower rows come as parts of their k range that fill the
+        // gaps (matmul_mfma_kernel<false, false, true>); their sum follows as for every split product.  2304^3 (324 tiles):
+        // 278 -> 203 us; 2176 x 2048 x 2176: 247 -> 164; 3584^3 (784): 805 -> 648; 4608^3 (1296): 1549 -> 1353.  With more
+        // than half a round of tiles in the lower rows it no longer pays (2560^3, 160 of 400 tiles: 310 -> 302; 4096 x 512 x
+        // 1536, 132 of 384: 68 -> 75); where two row bands apply (above) they are level or ahead (3072^3: 414 against 426).
+        if (bands && force_parts < 2) {
+            const int64_t cus = dev->props.multiProcessorCount, tiles = (int64_t)g.tiles_m * g.tiles_n, slices = (K + BK - 1) / BK;
+            const int64_t rounds = tiles / cus;
+            const int64_t rows_a = rounds * cus / g.tiles_n;
             const int64_t tiles_b = tiles - rows_a * g.tiles_n;
-            if (tiles > cus && 2 * tiles_b <= cus && rows_a >= 1 && rows_a < g.tiles_m && slices >= 16) {
+            if (tiles > cus && rounds >= 1 && rounds <= 6 && tiles_b >= 1 && 2 * tiles_b <= cus && rows_a >= 1 && rows_a < g.tiles_m && slices >= 16) {
                 const int64_t m_a = rows_a * BM, m_b = M - m_a;
                 int64_t parts = (2 * cus + tiles_b - 1) / tiles_b;                        // about two short blocks per unit at a time
                 if (parts > slices / 8) parts = slices / 8;
@@ -1906,15 +1909,15 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                     void* ws = nullptr;
                     if (int e = workspace(dev, (uint64_t)gm.splits * m_b * N * sizeof(float), &ws)) return e;
                     const unsigned grid = (unsigned)(rows_a * g.tiles_n + tiles_b * gm.splits);
-                    hipLaunchKernelGGL((matmul_mfma_kernel<false, false, true>), dim3(grid), dim3(256), 0, dev->stream, gm, Ap, Bp, Cp, (float*)ws);
+                    if (whole_tiles) hipLaunchKernelGGL((matmul_mfma_kernel<false, false, true>), dim3(grid), dim3(256), 0, dev->stream, gm, Ap, Bp, Cp, (float*)ws);
+                    else             hipLaunchKernelGGL((matmul_mfma_kernel<true, false, true>), dim3(grid), dim3(256), 0, dev->stream, gm, Ap, Bp, Cp, (float*)ws);
                     launch_add_parts<float>(dev, m_b * N, gm.splits, g.overwrite, (const float*)ws, Cp + m_a * N);
                     NK_HIP(hipGetLastError());
-                    set_path("mfma_mixed");
+                    set_path(whole_tiles ? "mfma_mixed" : "mfma_edge_mixed");
                     return NK_OK;
                 }
             }
         }
-        if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;
         bool streamed = false;
         const int rc = launch_mfma<float>(dev, g, BK, Cp, [&](bool split, dim3 grid, float* P) {
             if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);

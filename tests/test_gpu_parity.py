@@ -1821,11 +1821,12 @@ def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mk
 
 
 @pytest.mark.parametrize("mkn,path", [((2304, 608, 2304), "mfma_mixed"), ((2176, 512, 2176), "mfma_mixed"), ((33024, 512, 128), "mfma_mixed"),
-                                      ((2048, 1056, 2560), "mfma_mixed"), ((2560, 512, 2560), "mfma"), ((4096, 512, 1536), "mfma")])
+                                      ((2048, 1056, 2560), "mfma_mixed"), ((2560, 512, 2560), "mfma"), ((4096, 512, 1536), "mfma"),
+                                      ((3584, 512, 3584), "mfma_mixed"), ((2300, 520, 2300), "mfma_edge_mixed"), ((2090, 515, 2091), "mfma_edge_mixed")])
 def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
-    """Products with a few more 128 x 128 tiles than compute units run as one launch in which the upper tile rows take the
-    whole k range and the lower rows come as parts of it (their sum follows); with more than half a round of tiles in the
-    lower rows the plain launch stays.  Integer data are exact against numpy in both layouts and through both entry
+    """Products with a few more 128 x 128 tiles than whole rounds of one per compute unit run as one launch in which the
+    upper tile rows take the whole k range and the lower rows come as parts of it (their sum follows), shapes that are no
+    whole tiles included; with more than half a round of tiles in the lower rows the plain launch stays.  Integer data are exact against numpy in both layouts and through both entry
     points (the parts' run lengths do not divide the k range in every case); uniform data stay within the norm-wise
     bound; NaN around the operands and in the drain of an overwriting call shows that nothing else is read."""
     M, K, N = mkn
