@@ -399,12 +399,35 @@ constexpr int LDS_FLOATS = 3 * STAGE;
 // EDGE: any M, N, K and any (element-aligned) operands, as in the larger kernels: offsets from the first element of the
 // matrices with the rows past the edge clamped, descriptors that end where the matrices end (k rows of B past the end
 // read as 0), the k tail of A zeroed at the LDS write of the one slice that has it, stores guarded element by element.
-template <bool OVERWRITE, bool EDGE = false>
-__global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C) {
+// MIXED (as in matmul_mfma_kernel): the blocks of the first g.rows_a tile rows come first and take a whole tile each; the
+// tiles of the remaining rows follow as g.splits parts of their k range, written to P (a matrix of those rows only), which
+// matmul_add_parts adds into C.
+template <bool OVERWRITE, bool EDGE = false, bool MIXED = false>
+__global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                                            float* __restrict__ P = nullptr) {
     using namespace t64;
     __shared__ __attribute__((aligned(16))) float lds[t64::LDS_FLOATS];
-    int tm, tn;
-    tile_of_block(g, (int)blockIdx.x, tm, tn);
+    int tm, tn, part = 0;
+    bool parted = false;                                      // this block computes a part of its tile's k range, into P
+    if constexpr (MIXED) {
+        const int tiles_a = g.rows_a * g.tiles_n;
+        MfmaArgs band = g;
+        if ((int)blockIdx.x < tiles_a) {
+            band.tiles_m = g.rows_a;
+            band.group_rows = g.group_rows < band.tiles_m ? g.group_rows : band.tiles_m;
+            tile_of_block(band, (int)blockIdx.x, tm, tn);
+        } else {
+            band.tiles_m = g.tiles_m - g.rows_a;
+            band.group_rows = g.group_rows < band.tiles_m ? g.group_rows : band.tiles_m;
+            const int tiles_b = band.tiles_m * g.tiles_n, b = (int)blockIdx.x - tiles_a;
+            part = b / tiles_b;
+            tile_of_block(band, b - part * tiles_b, tm, tn);
+            tm += g.rows_a;
+            parted = true;
+        }
+    } else {
+        tile_of_block(g, (int)blockIdx.x, tm, tn);
+    }
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
@@ -480,10 +503,13 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     // slice publishes the writes one slice before anybody reads them, so the first chunks of slice kt + 1 are read before
     // that barrier, behind the last multiply-adds of slice kt: no wavefront starts a slice by waiting for LDS, which the
     // single wavefront of a SIMD could hide behind nothing.
-    const int nk = (g.K + BK - 1) / BK;
-    auto clamped = [&](int slice) { return (slice < nk ? slice : nk - 1) * BK; };     // past the end: the last slice again, read by nobody
-    load_global(0);
-    store_lds(0, 0);
+    const int all_slices = (g.K + BK - 1) / BK;
+    const int slice0 = parted ? part * g.split_slices : 0;                           // first k-slice of this block ...
+    int nk = all_slices;                                                             // ... and how many it takes
+    if (parted) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
+    auto clamped = [&](int slice) { return (slice0 + (slice < nk ? slice : nk - 1)) * BK; };     // past the end: the last slice again, read by nobody
+    load_global(clamped(0));
+    store_lds(0, clamped(0));
     load_global(clamped(1));
     store_lds(1, clamped(1));
     load_global(clamped(2));                                  // slice 2 waits in the staging registers
@@ -521,13 +547,14 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     for (int v = 0; v < 16; v++) acc[v] = acc0[v] + acc1[v];
     // accumulator v sits at row 8 * (v / 4) + 4 * h + v % 4, column l32 of the wavefront's 32 x 32 tile
     float* Cg = C + (int64_t)(tm * TM + wm) * g.N + tn * TN + wn + l32;
+    if (parted) Cg = P + ((int64_t)part * (g.M - g.rows_a * TM) + (int64_t)((tm - g.rows_a) * TM + wm)) * g.N + tn * TN + wn + l32;
     const int rows = g.M - (tm * TM + wm), cols = g.N - (tn * TN + wn + l32);      // EDGE: what is left of C from the lane's first element
 #pragma unroll
     for (int v = 0; v < 16; v++) {
         const int r = 8 * (v >> 2) + 4 * h + (v & 3);
         if (!EDGE || (r < rows && cols > 0)) {
             float* p = Cg + (int64_t)r * g.N;
-            *p = OVERWRITE ? acc[v] : *p + acc[v];
+            *p = (OVERWRITE || parted) ? acc[v] : *p + acc[v];
         }
     }
 }
@@ -1858,9 +1885,25 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             // 31), 1536 x 256 x 1536 17 against 26 (17, 31), 1024 x 1024 x 3072 51 against 60 (53, 64); the parts win
             // 1152^3 36 against 40 (35, 39), 1792^3 108 against 113 (108, 111), 1280 x 4096 x 1280 116 against 128 (107, 127).
             bool small_tiles = large < cus;
+            const int64_t slices = (K + BK - 1) / BK;
+            const int small_n = (int)((N + t64::TN - 1) / t64::TN), small_m = (int)((M + t64::TM - 1) / t64::TM);
+            // ... or whole rounds of small tiles for the upper tile rows and the rest in parts of the k range, in one launch
+            // (MIXED, as for the large tiles): 1536^3, 576 small tiles: 2 rounds + 64 tiles in parts instead of 3 rounds, 76 -> 69 us;
+            // 1792^3 109 -> 95; 1500^3 78 -> 70 (estimate: the rounds, the parts' rounds of shorter blocks, + 6 for the second launch)
+            int64_t mixed_rows = 0, mixed_parts = 0;
             if (small_tiles) {
-                const int64_t slices = (K + BK - 1) / BK;
-                const double t_small = 0.48 * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
+                double t_small = 0.48 * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
+                const int64_t rounds = small / cus, rows_a = rounds * cus / small_n, tiles_b = small - rows_a * small_n;
+                if (rounds >= 1 && tiles_b >= 1 && rows_a < small_m && slices >= 16) {
+                    int64_t parts = (cus + tiles_b - 1) / tiles_b;
+                    if (parts > slices / 4) parts = slices / 4;
+                    if (parts < 2) parts = 2;
+                    const int64_t part_slices = (slices + parts - 1) / parts;
+                    const double t_mixed = 0.48 * ((double)rounds * (double)slices + (double)((tiles_b * parts + cus - 1) / cus) * (double)part_slices) + 5.0 + 6.0;
+                    if (t_mixed < t_small && (uint64_t)parts * (uint64_t)(M - rows_a * t64::TM) * N * sizeof(float) <= ((uint64_t)1 << 30)) {
+                        t_small = t_mixed; mixed_rows = rows_a; mixed_parts = parts;
+                    }
+                }
                 MfmaArgs trial = g;
                 const double t_parts = split_plan(dev, trial, BK, sizeof(float), 0) > 1
                     ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
@@ -1870,8 +1913,28 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             }
             if (small_tiles) {
                 MfmaArgs gs = g;
-                gs.tiles_m = (int)((M + t64::TM - 1) / t64::TM); gs.tiles_n = (int)((N + t64::TN - 1) / t64::TN);
+                gs.tiles_m = small_m; gs.tiles_n = small_n;
                 gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
+                if (mixed_rows > 0) {
+                    gs.rows_a = (int)mixed_rows;
+                    gs.split_slices = (int)((slices + mixed_parts - 1) / mixed_parts);
+                    gs.splits = (int)((slices + gs.split_slices - 1) / gs.split_slices);
+                    const int64_t m_a = mixed_rows * t64::TM, m_b = M - m_a;
+                    void* ws = nullptr;
+                    if (int e = workspace(dev, (uint64_t)gs.splits * m_b * N * sizeof(float), &ws)) return e;
+                    const unsigned grid = (unsigned)(mixed_rows * small_n + (small - mixed_rows * small_n) * gs.splits);
+                    if (whole_small) {
+                        if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, false, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
+                        else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, false, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
+                    } else {
+                        if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, true, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
+                        else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, true, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
+                    }
+                    launch_add_parts<float>(dev, m_b * N, gs.splits, g.overwrite, (const float*)ws, Cp + m_a * N);
+                    NK_HIP(hipGetLastError());
+                    set_path(whole_small ? "mfma_tiles_of_64_mixed" : "mfma_tiles_of_64_edge_mixed");
+                    return NK_OK;
+                }
                 if (whole_small) {
                     if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, false>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
                     else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, false>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);

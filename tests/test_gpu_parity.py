@@ -1867,11 +1867,14 @@ def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
                                       ((512, 4096, 2048), "mfma_tiles_of_64"), ((1024, 128, 1024), "mfma_tiles_of_64"),
                                       ((1024, 288, 1024), "mfma_tiles_of_64"), ((2048, 160, 512), "mfma_tiles_of_64"),
                                       ((1000, 1000, 1000), "mfma_tiles_of_64_edge"), ((777, 333, 1025), "mfma_tiles_of_64_edge"),
-                                      ((65, 1001, 4097), "mfma_tiles_of_64_edge"), ((1023, 129, 1025), "mfma_tiles_of_64_edge")])
+                                      ((65, 1001, 4097), "mfma_tiles_of_64_edge"), ((1023, 129, 1025), "mfma_tiles_of_64_edge"),
+                                      ((1536, 1024, 1536), "mfma_tiles_of_64_mixed"), ((1792, 1056, 1792), "mfma_tiles_of_64_mixed"),
+                                      ((1500, 1050, 1500), "mfma_tiles_of_64_edge_mixed"), ((1111, 1111, 1111), "mfma_tiles_of_64_edge_mixed")])
 def test_matmul_64_tiles_in_one_launch(device, mkn, path):
     """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit: one launch of
     the small-tile kernel, from four k-slices up to long k ranges, and its edge variant for shapes that are no whole
-    number of tiles or slices (odd row lengths: operands' rows are then not 16-byte aligned).  Integer data are exact against numpy in both layouts and
+    number of tiles or slices (odd row lengths: operands' rows are then not 16-byte aligned); with a few tiles more than
+    whole rounds, the upper tile rows whole and the rest as parts of the k range in the same launch.  Integer data are exact against numpy in both layouts and
     through both entry points; uniform data stay within the norm-wise bound; operands inside larger buffers full of NaN
     show that nothing outside them is read."""
     M, K, N = mkn
