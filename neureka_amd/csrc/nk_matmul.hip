@@ -1876,15 +1876,21 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         // fewer large tiles than compute units, but whole 64 x 64 tiles, at least one per unit: the small-tile kernel in one launch
         const bool whole_small = aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0;
         const bool fits_32_bits = M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);       // (the edge kernels' offsets)
-        if (bands && force_parts < 2 && (whole_small || fits_32_bits) && K >= 4 * BK) {
+        // (`many`: the product has at least a round of large tiles; the small tiles are then held against the plain launch of the
+        // large ones, ceil(tiles / units) x 1.85 us per k-slice + 7: 2560^3, 400 large tiles = 2 rounds for the work of 1.56)
+        auto small_tile_plan = [&](bool many) -> int {
+            if (!(bands && force_parts < 2 && (whole_small || fits_32_bits) && K >= 4 * BK)) return -1;
             const int64_t cus = dev->props.multiProcessorCount;
             const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
+            if (many != (large >= cus)) return -1;
+            // (very short k ranges over many whole tiles are the walking blocks' case, measured 10-14 % ahead of the small tiles there)
+            if (many && whole_tiles && K / BK <= 8 && large >= 4 * cus && large % 8 == 0) return -1;
             // Against the k range of the large tiles cut into parts, by two estimates fitted to measurements (microseconds):
             // the small tiles run in rounds of one per unit at 0.48 per k-slice plus 5; the parts cost 1.93 per unit of
             // split_plan's estimate plus 8 for the second launch and the shorter blocks.  1024^3 21 against 29 (measured: 21,
             // 31), 1536 x 256 x 1536 17 against 26 (17, 31), 1024 x 1024 x 3072 51 against 60 (53, 64); the parts win
             // 1152^3 36 against 40 (35, 39), 1792^3 108 against 113 (108, 111), 1280 x 4096 x 1280 116 against 128 (107, 127).
-            bool small_tiles = large < cus;
+            bool small_tiles = true;
             const int64_t slices = (K + BK - 1) / BK;
             const int small_n = (int)((N + t64::TN - 1) / t64::TN), small_m = (int)((M + t64::TM - 1) / t64::TM);
             // ... or whole rounds of small tiles for the upper tile rows and the rest in parts of the k range, in one launch
@@ -1905,7 +1911,8 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                     }
                 }
                 MfmaArgs trial = g;
-                const double t_parts = split_plan(dev, trial, BK, sizeof(float), 0) > 1
+                const double t_parts = many ? 1.85 * (double)((large + cus - 1) / cus) * (double)slices + 7.0
+                    : split_plan(dev, trial, BK, sizeof(float), 0) > 1
                     ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
                     : 1.93 * (double)slices + 7.0;
                 // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
@@ -1946,7 +1953,9 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 set_path(whole_small ? "mfma_tiles_of_64" : "mfma_tiles_of_64_edge");
                 return NK_OK;
             }
-        }
+            return -1;
+        };
+        if (const int rc = small_tile_plan(false); rc >= 0) return rc;
         if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;
         // A few more tiles than a whole number of rounds of one tile per compute unit: as one launch of whole tiles some units
         // would work through one tile more than the others (side by side with another).  Instead the upper tile rows, whole
@@ -1981,6 +1990,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 }
             }
         }
+        if (const int rc = small_tile_plan(true); rc >= 0) return rc;
         bool streamed = false;
         const int rc = launch_mfma<float>(dev, g, BK, Cp, [&](bool split, dim3 grid, float* P) {
             if (whole_tiles && split) hipLaunchKernelGGL((matmul_mfma_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);

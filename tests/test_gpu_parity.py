@@ -1789,8 +1789,8 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
 
 
 @pytest.mark.parametrize("dt,mkn,path", [
-    ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_split"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 256, 2048), "mfma"),
-    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 130, 2100), "mfma_edge"),
+    ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_split"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
+    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 100, 2100), "mfma_edge"),
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
     ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
@@ -1821,12 +1821,12 @@ def test_matmul_set_overwrites_and_equals_accumulation_into_zeros(device, dt, mk
 
 
 @pytest.mark.parametrize("mkn,path", [((2304, 608, 2304), "mfma_mixed"), ((2176, 512, 2176), "mfma_mixed"), ((33024, 512, 128), "mfma_mixed"),
-                                      ((2048, 1056, 2560), "mfma_mixed"), ((2560, 512, 2560), "mfma"), ((4096, 512, 1536), "mfma"),
+                                      ((2048, 1056, 2560), "mfma_mixed"), ((2560, 512, 2560), "mfma_tiles_of_64"), ((4096, 512, 1536), "mfma_tiles_of_64"),
                                       ((3584, 512, 3584), "mfma_mixed"), ((2300, 520, 2300), "mfma_edge_mixed"), ((2090, 515, 2091), "mfma_edge_mixed")])
 def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
     """Products with a few more 128 x 128 tiles than whole rounds of one per compute unit run as one launch in which the
     upper tile rows take the whole k range and the lower rows come as parts of it (their sum follows), shapes that are no
-    whole tiles included; with more than half a round of tiles in the lower rows the plain launch stays.  Integer data are exact against numpy in both layouts and through both entry
+    whole tiles included; with more than half a round of tiles in the lower rows this launch is not taken (64 x 64 tiles serve those here).  Integer data are exact against numpy in both layouts and through both entry
     points (the parts' run lengths do not divide the k range in every case); uniform data stay within the norm-wise
     bound; NaN around the operands and in the drain of an overwriting call shows that nothing else is read."""
     M, K, N = mkn
@@ -1869,9 +1869,12 @@ def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
                                       ((1000, 1000, 1000), "mfma_tiles_of_64_edge"), ((777, 333, 1025), "mfma_tiles_of_64_edge"),
                                       ((65, 1001, 4097), "mfma_tiles_of_64_edge"), ((1023, 129, 1025), "mfma_tiles_of_64_edge"),
                                       ((1536, 1024, 1536), "mfma_tiles_of_64_mixed"), ((1792, 1056, 1792), "mfma_tiles_of_64_mixed"),
-                                      ((1500, 1050, 1500), "mfma_tiles_of_64_edge_mixed"), ((1111, 1111, 1111), "mfma_tiles_of_64_edge_mixed")])
+                                      ((1500, 1050, 1500), "mfma_tiles_of_64_edge_mixed"), ((1111, 1111, 1111), "mfma_tiles_of_64_edge_mixed"),
+                                      ((2560, 512, 2560), "mfma_tiles_of_64"), ((2560, 1024, 2560), "mfma_tiles_of_64_mixed"),
+                                      ((2500, 520, 2500), "mfma_tiles_of_64_edge"), ((2500, 1030, 2500), "mfma_tiles_of_64_edge_mixed")])
 def test_matmul_64_tiles_in_one_launch(device, mkn, path):
-    """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit: one launch of
+    """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit, or with a last
+    round of 128 x 128 tiles that would leave most of the machine idle (2560 and 2500 square: 400 tiles on 256 units): one launch of
     the small-tile kernel, from four k-slices up to long k ranges, and its edge variant for shapes that are no whole
     number of tiles or slices (odd row lengths: operands' rows are then not 16-byte aligned); with a few tiles more than
     whole rounds, the upper tile rows whole and the rest as parts of the k range in the same launch.  Integer data are exact against numpy in both layouts and
