@@ -1910,6 +1910,19 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                         t_small = t_mixed; mixed_rows = rows_a; mixed_parts = parts;
                     }
                 }
+                // ... or, with less than a round of small tiles, every tile in parts (no upper rows): more blocks per unit at a time
+                // for long k ranges over few tiles, and no columns of padding where the large tiles would be half empty
+                if (rounds == 0 && slices >= 16) {
+                    int64_t best = 0; double t_best = t_small;
+                    for (int64_t parts = 2; parts <= slices / 4 && parts <= 64; parts++) {
+                        const int64_t part_slices = (slices + parts - 1) / parts;
+                        if ((parts - 1) * part_slices >= slices) continue;                  // the last part would be empty
+                        const double t = 0.48 * (double)((small * parts + cus - 1) / cus) * (double)part_slices + 5.0 + 6.0
+                                       + (double)parts * (double)M * (double)N * 8.0 / 4.0e6;
+                        if (t < t_best) { t_best = t; best = parts; }
+                    }
+                    if (best > 0 && (uint64_t)best * (uint64_t)M * N * sizeof(float) <= ((uint64_t)1 << 30)) { t_small = t_best; mixed_rows = 0; mixed_parts = best; }
+                }
                 MfmaArgs trial = g;
                 const double t_parts = many ? 1.85 * (double)((large + cus - 1) / cus) * (double)slices + 7.0
                     : split_plan(dev, trial, BK, sizeof(float), 0) > 1
@@ -1922,7 +1935,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                 MfmaArgs gs = g;
                 gs.tiles_m = small_m; gs.tiles_n = small_n;
                 gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
-                if (mixed_rows > 0) {
+                if (mixed_parts > 0) {
                     gs.rows_a = (int)mixed_rows;
                     gs.split_slices = (int)((slices + mixed_parts - 1) / mixed_parts);
                     gs.splits = (int)((slices + gs.split_slices - 1) / gs.split_slices);
@@ -1939,7 +1952,8 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                     }
                     launch_add_parts<float>(dev, m_b * N, gs.splits, g.overwrite, (const float*)ws, Cp + m_a * N);
                     NK_HIP(hipGetLastError());
-                    set_path(whole_small ? "mfma_tiles_of_64_mixed" : "mfma_tiles_of_64_edge_mixed");
+                    set_path(mixed_rows == 0 ? (whole_small ? "mfma_tiles_of_64_split" : "mfma_tiles_of_64_edge_split")
+                                             : (whole_small ? "mfma_tiles_of_64_mixed" : "mfma_tiles_of_64_edge_mixed"));
                     return NK_OK;
                 }
                 if (whole_small) {
