@@ -1879,7 +1879,10 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         // (`many`: the product has at least a round of large tiles; the small tiles are then held against the plain launch of the
         // large ones, ceil(tiles / units) x 1.85 us per k-slice + 7: 2560^3, 400 large tiles = 2 rounds for the work of 1.56)
         auto small_tile_plan = [&](bool many) -> int {
-            if (!(bands && force_parts < 2 && (whole_small || fits_32_bits) && K >= 4 * BK)) return -1;
+            // (from the shortest k ranges on, above the ones of the short-inner kernel: the kernel reads its slices clamped to
+            // the last one, and with one or two slices a small tile's fetch and write-back overlap better with the other blocks
+            // of its unit -- 3000 x 64 x 3000 31 -> 19 us, 100000 x 64 x 64 31 -> 16, 1000 x 100 x 1000 15 -> 6)
+            if (!(bands && force_parts < 2 && (whole_small || fits_32_bits) && K > 16)) return -1;
             const int64_t cus = dev->props.multiProcessorCount;
             const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
             if (many != (large >= cus)) return -1;

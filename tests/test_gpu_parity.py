@@ -1790,7 +1790,7 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
 
 @pytest.mark.parametrize("dt,mkn,path", [
     ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_tiles_of_64_split"), ("f32", (1152, 2048, 1152), "mfma_split"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
-    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_tiles_of_64_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 100, 2100), "mfma_edge"),
+    ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_tiles_of_64_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 100, 2100), "mfma_tiles_of_64_edge"),
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
     ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
@@ -1873,11 +1873,13 @@ def test_matmul_a_few_more_tiles_than_compute_units(device, mkn, path):
                                       ((2560, 512, 2560), "mfma_tiles_of_64"), ((2560, 1024, 2560), "mfma_tiles_of_64_mixed"),
                                       ((2500, 520, 2500), "mfma_tiles_of_64_edge"), ((2500, 1030, 2500), "mfma_tiles_of_64_edge_mixed"),
                                       ((384, 2048, 384), "mfma_tiles_of_64_split"), ((4096, 1024, 64), "mfma_tiles_of_64_split"), ((64, 4096, 1024), "mfma_tiles_of_64_split"),
-                                      ((300, 4000, 300), "mfma_tiles_of_64_edge_split"), ((1000, 3001, 100), "mfma_tiles_of_64_edge_split"), ((65, 8190, 129), "mfma_tiles_of_64_edge_split")])
+                                      ((300, 4000, 300), "mfma_tiles_of_64_edge_split"), ((1000, 3001, 100), "mfma_tiles_of_64_edge_split"), ((65, 8190, 129), "mfma_tiles_of_64_edge_split"),
+                                      ((1024, 64, 1024), "mfma_tiles_of_64"), ((1024, 32, 1024), "mfma_tiles_of_64"), ((512, 96, 512), "mfma_tiles_of_64"),
+                                      ((3000, 40, 3000), "mfma_tiles_of_64_edge"), ((1000, 100, 1000), "mfma_tiles_of_64_edge"), ((1500, 17, 1500), "mfma_tiles_of_64_edge")])
 def test_matmul_64_tiles_in_one_launch(device, mkn, path):
     """Products with too few 128 x 128 tiles for the machine but a 64 x 64 tile for every compute unit, or with a last
     round of 128 x 128 tiles that would leave most of the machine idle (2560 and 2500 square: 400 tiles on 256 units): one launch of
-    the small-tile kernel, from four k-slices up to long k ranges, and its edge variant for shapes that are no whole
+    the small-tile kernel, from a single k-slice (a partial one: k = 17) up to long k ranges, and its edge variant for shapes that are no whole
     number of tiles or slices (odd row lengths: operands' rows are then not 16-byte aligned); with less than a round of small tiles and a long k range every tile as parts of the k range; with a few tiles more than
     whole rounds, the upper tile rows whole and the rest as parts of the k range in the same launch.  Integer data are exact against numpy in both layouts and
     through both entry points; uniform data stay within the norm-wise bound; operands inside larger buffers full of NaN
