@@ -402,13 +402,8 @@ constexpr int LDS_FLOATS = 3 * STAGE;
 // MIXED (as in matmul_mfma_kernel): the blocks of the first g.rows_a tile rows come first and take a whole tile each; the
 // tiles of the remaining rows follow as g.splits parts of their k range, written to P (a matrix of those rows only), which
 // matmul_add_parts adds into C.
-template <bool OVERWRITE, bool EDGE = false, bool MIXED = false>
-__global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
-                                                            float* __restrict__ P = nullptr) {
-    using namespace t64;
-    __shared__ __attribute__((aligned(16))) float lds[t64::LDS_FLOATS];
-    int tm, tn, part = 0;
-    bool parted = false;                                      // this block computes a part of its tile's k range, into P
+template <bool MIXED>
+__device__ __forceinline__ void small_tile_of_block(const MfmaArgs& g, int& tm, int& tn, int& part, bool& parted) {
     if constexpr (MIXED) {
         const int tiles_a = g.rows_a * g.tiles_n;
         MfmaArgs band = g;
@@ -428,6 +423,15 @@ __global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const fl
     } else {
         tile_of_block(g, (int)blockIdx.x, tm, tn);
     }
+}
+template <bool OVERWRITE, bool EDGE = false, bool MIXED = false>
+__global__ __launch_bounds__(256) void matmul_mfma64_kernel(MfmaArgs g, const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+                                                            float* __restrict__ P = nullptr) {
+    using namespace t64;
+    __shared__ __attribute__((aligned(16))) float lds[t64::LDS_FLOATS];
+    int tm, tn, part = 0;
+    bool parted = false;                                      // this block computes a part of its tile's k range, into P
+    small_tile_of_block<MIXED>(g, tm, tn, part, parted);
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
@@ -1388,12 +1392,14 @@ __global__ __launch_bounds__(256) void matmul_short_inner_kernel(int M, int K, i
 // ---- f64 on the matrix cores ----------------------------------------------------------------------------------
 // 128x128 block tile, four wavefronts in a 2x2 arrangement, each owning 64x64 as 4x4 accumulators of
 // v_mfma_f64_16x16x4_f64 (register v of lane l holds row 4*v + l/16 of column l%16 of a 16x16 tile; it feeds A[row l%16]
-// [k l/16] and B[k l/16][column l%16]).  k-slices of 16 in double-buffered LDS: A rows have a pitch of 17
-// doubles, which spreads the 16 rows a quarter-wavefront reads over all banks.
+// [k l/16] and B[k l/16][column l%16]).  k-slices of 16 in double-buffered LDS.
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef double f64x2 __attribute__((ext_vector_type(2)));
 namespace d64 {
 constexpr int DK = 16;
+// (pitches: the LDS serves a 64-bit read of 32 lanes per cycle from 64 banks of four bytes, and with these pitches half of
+// the passes take a second cycle.  Pitches without any conflict, 18 and BN + 16 (counted: none), measured slower in this
+// kernel, 3072^3 892 against 845 us: the LDS is not what bounds it, and two blocks then hold 144 of the unit's 160 KiB.)
 constexpr int DA_PITCH = DK + 1;
 constexpr int DB_PITCH = BN + 2;
 constexpr int LDS_DOUBLES = 2 * BM * DA_PITCH + 2 * DK * DB_PITCH;
@@ -1545,6 +1551,155 @@ __global__ __launch_bounds__(256, 2) void matmul_mfma_f64_kernel(MfmaArgs g, con
             }
 }
 
+// 64 x 64 block tiles in f64, for the products the f32 kernel of that tile size serves (few large tiles, a last round of large
+// tiles that would idle most units, narrow results, long k ranges over few tiles): four wavefronts in a 2 x 2 arrangement,
+// each owning 32 x 32 as 2 x 2 accumulators of v_mfma_f64_16x16x4_f64; k-slices of 16 in three LDS stages with the pitches
+// of the large kernel.  A multiply-add keeps the matrix core busy for 64 cycles, so the four LDS reads of a depth-4 chunk hide
+// behind the multiply-adds of the chunk before it with a single wavefront per SIMD.  EDGE and MIXED as in matmul_mfma64_kernel.
+namespace t64d {
+constexpr int DK = d64::DK;
+// (pitches without bank conflicts: the LDS serves a 64-bit read of 32 lanes per cycle from 64 banks of four bytes.  The 32 lanes
+// of a pass read A[row l % 16][k q, q + 1]: with a pitch of 18 doubles the rows fall on the even pairs of banks and the second k
+// beside them; B's two k rows of 16 consecutive doubles must lie 32 banks apart: a pitch of 16 modulo 32)
+constexpr int A_P = DK + 2, B_P = t64::TN + 16;
+constexpr int STAGE = t64::TM * A_P + DK * B_P;
+constexpr int LDS_DOUBLES = 3 * STAGE;
+}
+// (launch bounds of two blocks per unit: with a budget of at most 256 registers the compiler keeps the accumulators in
+// ordinary registers; with 512 it moved three of the four between the two register files in every slice, behind a wait for
+// the last multiply-add: 0.71 us per slice instead of 0.43 of multiply-adds)
+template <bool OVERWRITE, bool EDGE = false, bool MIXED = false>
+__global__ __launch_bounds__(256, 2) void matmul_mfma64_f64_kernel(MfmaArgs g, const double* __restrict__ A, const double* __restrict__ B,
+                                                                double* __restrict__ C, double* __restrict__ P = nullptr) {
+    using namespace t64d;
+    constexpr int TM = t64::TM, TN = t64::TN;
+    __shared__ __attribute__((aligned(16))) double lds[LDS_DOUBLES];
+    int tm, tn, part = 0;
+    bool parted = false;
+    small_tile_of_block<MIXED>(g, tm, tn, part, parted);
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
+    const int l16 = lane & 15, q = lane >> 4;
+    // global -> registers: A slice 64 x 16 and B slice 16 x 64, two 16-byte pieces each per thread; byte offsets from the
+    // first element of the matrices, fixed for the k loop (the slice moves the base of the descriptors)
+    const int a_row = tid >> 3, a_col = (tid & 7) * 2;       // rows a_row + 32 * i
+    const int b_row = tid >> 5, b_col = (tid & 31) * 2;      // rows b_row + 8 * i
+    f64x2 ra[2], rb[2];
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    unsigned off_a[2], off_b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        int row = tm * TM + a_row + 32 * i;
+        if (EDGE && row > g.M - 1) row = g.M - 1;
+        off_a[i] = (unsigned)(row * g.K + a_col) * 8u;
+        off_b[i] = (unsigned)((b_row + 8 * i) * g.N + tn * TN + b_col) * 8u;
+    }
+    auto load_global = [&](int k0) {
+        const __amdgpu_buffer_rsrc_t da = __builtin_amdgcn_make_buffer_rsrc((void*)(A + k0), 0, EDGE ? (unsigned)(((int64_t)g.M * g.K - k0) * 8) : 0xffffffffu, 0x00020000);
+        const __amdgpu_buffer_rsrc_t db = __builtin_amdgcn_make_buffer_rsrc((void*)(B + (int64_t)k0 * g.N), 0, EDGE ? (unsigned)((int64_t)(g.K - k0) * g.N * 8) : 0xffffffffu, 0x00020000);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            ra[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(da, off_a[i], 0, 0)));
+            rb[i] = __builtin_bit_cast(f64x2, (u32x4)__builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(db, off_b[i], 0, 0)));
+        }
+    };
+    // k0: the slice the staging registers hold (EDGE: its k tail is zeroed here, in the one slice that has it)
+    auto store_lds = [&](int stage, int k0) {
+        if (EDGE && k0 + DK > g.K) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+#pragma unroll
+                for (int e = 0; e < 2; e++) if (k0 + a_col + e >= g.K) ra[i][e] = 0.0;
+                if (k0 + b_row + 8 * i >= g.K) rb[i] = f64x2{0.0, 0.0};
+            }
+        }
+        double* as = lds + stage * STAGE;
+        double* bs = as + TM * A_P;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            *(f64x2*)(&as[(a_row + 32 * i) * A_P + a_col]) = ra[i];
+            *(f64x2*)(&bs[(b_row + 8 * i) * B_P + b_col]) = rb[i];
+        }
+    };
+    // operands of one depth-4 chunk: lane quarter q owns k = 4c + q
+    struct Chunk { double a[2], b[2]; };
+    auto read_chunk = [&](Chunk& f, int stage, int c) {
+        const double* as = lds + stage * STAGE;
+        const double* bs = as + TM * A_P;
+#pragma unroll
+        for (int i = 0; i < 2; i++) f.a[i] = as[(wm + 16 * i + l16) * A_P + 4 * c + q];
+#pragma unroll
+        for (int j = 0; j < 2; j++) f.b[j] = bs[(4 * c + q) * B_P + wn + 16 * j + l16];
+    };
+    f64x4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = f64x4{0.0, 0.0, 0.0, 0.0};
+    auto mma = [&](const Chunk& f) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+    };
+    static_assert(DK == 16, "the pipeline below is written for four depth-4 chunks per slice");
+    // Three stages of LDS as in matmul_mfma64_kernel: during slice kt the block writes slice kt + 2 and reads slice kt, and
+    // the first chunks of slice kt + 1 are read before the barrier, behind the last multiply-adds of slice kt.
+    const int all_slices = (g.K + DK - 1) / DK;
+    const int slice0 = parted ? part * g.split_slices : 0;
+    int nk = all_slices;
+    if (parted) { nk = all_slices - slice0; if (nk > g.split_slices) nk = g.split_slices; }
+    auto clamped = [&](int slice) { return (slice0 + (slice < nk ? slice : nk - 1)) * DK; };     // past the end: the last slice again, read by nobody
+    load_global(clamped(0));
+    store_lds(0, clamped(0));
+    load_global(clamped(1));
+    store_lds(1, clamped(1));
+    load_global(clamped(2));                                  // slice 2 waits in the staging registers
+    __syncthreads();
+    Chunk f0, f1, f2, f3;
+    read_chunk(f0, 0, 0);
+    read_chunk(f1, 0, 1);
+    int cur = 0;
+    for (int kt = 0; kt < nk; kt++) {
+        const int next = cur == 2 ? 0 : cur + 1, write = next == 2 ? 0 : next + 1;      // stages of slices kt + 1, kt + 2
+        read_chunk(f2, cur, 2);
+        read_chunk(f3, cur, 3);
+        mma(f0);
+        mma(f1);
+        // the eight LDS reads of chunks 2 and 3 behind the first four multiply-adds of chunks 0 and 1 ...
+        NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(4); NK_FENCE;
+        store_lds(write, clamped(kt + 2));
+        load_global(clamped(kt + 3));
+        read_chunk(f0, next, 0);
+        read_chunk(f1, next, 1);
+        mma(f2);
+        mma(f3);
+        // ... one LDS write and one request behind each of the next four, the reads of the next slice behind the last four
+        NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1); NK_MFMA(1); NK_DS_WRITE(1); NK_VMEM_READ(1);
+        NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_MFMA(1); NK_DS_READ(2); NK_FENCE;
+        __syncthreads();
+        cur = next;
+    }
+    // register v of accumulator (i, j) sits at row 16 * i + 4 * v + q, column 16 * j + l16 of the wavefront's 32 x 32 tile;
+    // a quarter-wavefront covers 16 consecutive doubles of a row
+    double* Cg = C + (int64_t)(tm * TM + wm) * g.N + tn * TN + wn;
+    if (parted) Cg = P + ((int64_t)part * (g.M - g.rows_a * TM) + (int64_t)((tm - g.rows_a) * TM + wm)) * g.N + tn * TN + wn;
+    const int rows = g.M - (tm * TM + wm), cols = g.N - (tn * TN + wn);        // EDGE: what is left of C from the wavefront's first element
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int row = 16 * i + 4 * v + q, col = 16 * j + l16;
+                if (!EDGE || (row < rows && col < cols)) {
+                    double* p = Cg + (int64_t)row * g.N + col;
+                    *p = (OVERWRITE || parted) ? acc[i][j][v] : *p + acc[i][j][v];
+                }
+            }
+}
+
 template <typename T>
 static int launch_simple(Device* dev, int64_t M, int64_t K, int64_t N, bool overwrite, const T* A, const T* B, T* C) {
     dim3 grid((unsigned)((N + 63) / 64), (unsigned)((M + 3) / 4));
@@ -1599,6 +1754,91 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
         launch(false, dim3((unsigned)tiles), (T*)nullptr);
     }
     NK_HIP(hipGetLastError());
+    return NK_OK;
+}
+
+// The plans on 64 x 64 tiles, for both element types (`slice`: the depth of a k-slice, 32 floats or 16 doubles -- a slice of a
+// small tile then costs the same in both, as a slice of a large tile does).  `launch(mixed, edge, grid, args, P)` starts the
+// kernel.  Returns -1 when another plan should take the product.
+// `many`: the product has at least a round of large tiles; the small tiles are then held against the plain launch of the large
+// ones, ceil(tiles / units) x 1.85 us per k-slice + 7 (2560^3 f32, 400 large tiles = 2 rounds for the work of 1.56); otherwise
+// against the k range of the large tiles cut into parts.  `walking`: f32 whole tiles with at most eight k-slices.
+struct SmallTileNames { const char *whole, *edge, *whole_split, *edge_split, *whole_mixed, *edge_mixed; };
+template <typename T, typename Launch>
+static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many, bool whole_small, bool whole_tiles, bool walking,
+                           T* Cp, const SmallTileNames& names, Launch launch) {
+    // a k-slice of a small tile on a unit of its own, microseconds (f32: 0.89 of the rate of its multiply-adds; the f64 kernel
+    // measures 0.54, but its plans on large tiles fall short of their estimates by as much, and 0.48 chooses better there too:
+    // 1536^3 f64 127 us mixed against 140 in parts, 1111^3 62 against 73, 2048 x 256 x 2048 40 against 45 on large tiles)
+    constexpr double c_small = 0.48;
+    const int64_t M = g.M, K = g.K, N = g.N;
+    const int64_t cus = dev->props.multiProcessorCount;
+    const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
+    if (many != (large >= cus)) return -1;
+    // (very short k ranges over many whole tiles are the walking blocks' case, measured 10-14 % ahead of the small tiles there)
+    if (many && walking && large >= 4 * cus && large % 8 == 0) return -1;
+    // By estimates fitted to measurements (microseconds, f32): the small tiles run in rounds of one per unit at 0.48 per
+    // k-slice plus 5; the parts cost 1.93 per unit of split_plan's estimate plus 8 for the second launch and the shorter blocks.
+    // 1024^3 21 against 29 (measured: 21, 31), 1536 x 256 x 1536 17 against 26 (17, 31), 1024 x 1024 x 3072 51 against 60 (53, 64);
+    // the parts win 1152^3 36 against 40 (35, 39), 1792^3 108 against 113 (108, 111), 1280 x 4096 x 1280 116 against 128 (107, 127).
+    const int64_t slices = (K + slice - 1) / slice;
+    const int small_n = (int)((N + t64::TN - 1) / t64::TN), small_m = (int)((M + t64::TM - 1) / t64::TM);
+    // ... or whole rounds of small tiles for the upper tile rows and the rest in parts of the k range, in one launch
+    // (MIXED, as for the large tiles): 1536^3, 576 small tiles: 2 rounds + 64 tiles in parts instead of 3 rounds, 76 -> 69 us;
+    // 1792^3 109 -> 95; 1500^3 78 -> 70 (estimate: the rounds, the parts' rounds of shorter blocks, + 6 for the second launch)
+    int64_t mixed_rows = 0, mixed_parts = 0;
+    double t_small = c_small * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
+    const int64_t rounds = small / cus, rows_a = rounds * cus / small_n, tiles_b = small - rows_a * small_n;
+    if (rounds >= 1 && tiles_b >= 1 && rows_a < small_m && slices >= 16) {
+        int64_t parts = (cus + tiles_b - 1) / tiles_b;
+        if (parts > slices / 4) parts = slices / 4;
+        if (parts < 2) parts = 2;
+        const int64_t part_slices = (slices + parts - 1) / parts;
+        const double t_mixed = c_small * ((double)rounds * (double)slices + (double)((tiles_b * parts + cus - 1) / cus) * (double)part_slices) + 5.0 + 6.0;
+        if (t_mixed < t_small && (uint64_t)parts * (uint64_t)(M - rows_a * t64::TM) * N * sizeof(T) <= ((uint64_t)1 << 30)) {
+            t_small = t_mixed; mixed_rows = rows_a; mixed_parts = parts;
+        }
+    }
+    // ... or, with less than a round of small tiles, every tile in parts (no upper rows): more blocks per unit at a time
+    // for long k ranges over few tiles, and no columns of padding where the large tiles would be half empty
+    if (rounds == 0 && slices >= 16) {
+        int64_t best = 0; double t_best = t_small;
+        for (int64_t parts = 2; parts <= slices / 4 && parts <= 64; parts++) {
+            const int64_t part_slices = (slices + parts - 1) / parts;
+            if ((parts - 1) * part_slices >= slices) continue;                  // the last part would be empty
+            const double t = c_small * (double)((small * parts + cus - 1) / cus) * (double)part_slices + 5.0 + 6.0
+                           + (double)parts * (double)M * (double)N * 2.0 * sizeof(T) / 4.0e6;
+            if (t < t_best) { t_best = t; best = parts; }
+        }
+        if (best > 0 && (uint64_t)best * (uint64_t)M * N * sizeof(T) <= ((uint64_t)1 << 30)) { t_small = t_best; mixed_rows = 0; mixed_parts = best; }
+    }
+    MfmaArgs trial = g;
+    const double t_parts = many ? 1.85 * (double)((large + cus - 1) / cus) * (double)slices + 7.0
+        : split_plan(dev, trial, slice, sizeof(T), 0) > 1
+        ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
+        : 1.93 * (double)slices + 7.0;
+    // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
+    if (!(t_small < (whole_tiles ? 1.0 : 1.15) * t_parts)) return -1;
+    MfmaArgs gs = g;
+    gs.tiles_m = small_m; gs.tiles_n = small_n;
+    gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
+    if (mixed_parts > 0) {
+        gs.rows_a = (int)mixed_rows;
+        gs.split_slices = (int)((slices + mixed_parts - 1) / mixed_parts);
+        gs.splits = (int)((slices + gs.split_slices - 1) / gs.split_slices);
+        const int64_t m_a = mixed_rows * t64::TM, m_b = M - m_a;
+        void* ws = nullptr;
+        if (int e = workspace(dev, (uint64_t)gs.splits * m_b * N * sizeof(T), &ws)) return e;
+        const unsigned grid = (unsigned)(mixed_rows * small_n + (small - mixed_rows * small_n) * gs.splits);
+        launch(true, !whole_small, grid, gs, (T*)ws);
+        launch_add_parts<T>(dev, m_b * N, gs.splits, g.overwrite, (const T*)ws, Cp + m_a * N);
+        NK_HIP(hipGetLastError());
+        set_path(mixed_rows == 0 ? (whole_small ? names.whole_split : names.edge_split) : (whole_small ? names.whole_mixed : names.edge_mixed));
+        return NK_OK;
+    }
+    launch(false, !whole_small, (unsigned)small, gs, (T*)nullptr);
+    NK_HIP(hipGetLastError());
+    set_path(whole_small ? names.whole : names.edge);
     return NK_OK;
 }
 
@@ -1821,8 +2061,29 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         const bool fits = M * K * 8 < ((int64_t)1 << 32) && K * N * 8 < ((int64_t)1 << 32);
         if (M * K * N >= mfma_from && fits) {
             const bool whole = (A % 16 == 0) && (B % 16 == 0) && M % BM == 0 && N % BN == 0 && K % d64::DK == 0;
-            if (const int rc = run_bands(8, (K + d64::DK - 1) / d64::DK, whole ? "mfma_f64_bands" : "mfma_f64_edge_bands"); rc >= 0) return rc;
             const double* Ap = (const double*)A; const double* Bp = (const double*)B; double* Cp = (double*)C;
+            // the plans on 64 x 64 tiles, as for f32 below: before the bands for products with less than a round of large tiles,
+            // after them for larger ones
+            const bool whole_small = (A % 16 == 0) && (B % 16 == 0) && M % t64::TM == 0 && N % t64::TN == 0 && K % d64::DK == 0;
+            auto small_tile_plan = [&](bool many) -> int {
+                if (!(bands && force_parts < 2 && K > 16)) return -1;
+                static const SmallTileNames names = {"mfma_f64_tiles_of_64", "mfma_f64_tiles_of_64_edge", "mfma_f64_tiles_of_64_split", "mfma_f64_tiles_of_64_edge_split",
+                                                     "mfma_f64_tiles_of_64_mixed", "mfma_f64_tiles_of_64_edge_mixed"};
+                return nk::small_tile_plan<double>(dev, g, d64::DK, many, whole_small, whole, false, Cp, names,
+                    [&](bool mixed, bool edge_kernel, unsigned grid, const MfmaArgs& gs, double* P) {
+                        auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, P); };
+                        if (mixed) {
+                            if (edge_kernel) { if (overwrite) go(matmul_mfma64_f64_kernel<true, true, true>); else go(matmul_mfma64_f64_kernel<false, true, true>); }
+                            else             { if (overwrite) go(matmul_mfma64_f64_kernel<true, false, true>); else go(matmul_mfma64_f64_kernel<false, false, true>); }
+                        } else {
+                            if (edge_kernel) { if (overwrite) go(matmul_mfma64_f64_kernel<true, true, false>); else go(matmul_mfma64_f64_kernel<false, true, false>); }
+                            else             { if (overwrite) go(matmul_mfma64_f64_kernel<true, false, false>); else go(matmul_mfma64_f64_kernel<false, false, false>); }
+                        }
+                    });
+            };
+            if (const int rc = small_tile_plan(false); rc >= 0) return rc;
+            if (const int rc = run_bands(8, (K + d64::DK - 1) / d64::DK, whole ? "mfma_f64_bands" : "mfma_f64_edge_bands"); rc >= 0) return rc;
+            if (const int rc = small_tile_plan(true); rc >= 0) return rc;
             const int rc = launch_mfma<double>(dev, g, d64::DK, Cp, [&](bool split, dim3 grid, double* P) {
                 if (whole && split)       hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
                 else if (whole)           hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, false>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
@@ -1876,102 +2137,26 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         // fewer large tiles than compute units, but whole 64 x 64 tiles, at least one per unit: the small-tile kernel in one launch
         const bool whole_small = aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0;
         const bool fits_32_bits = M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);       // (the edge kernels' offsets)
-        // (`many`: the product has at least a round of large tiles; the small tiles are then held against the plain launch of the
-        // large ones, ceil(tiles / units) x 1.85 us per k-slice + 7: 2560^3, 400 large tiles = 2 rounds for the work of 1.56)
         auto small_tile_plan = [&](bool many) -> int {
             // (from the shortest k ranges on, above the ones of the short-inner kernel: the kernel reads its slices clamped to
             // the last one, and with one or two slices a small tile's fetch and write-back overlap better with the other blocks
             // of its unit -- 3000 x 64 x 3000 31 -> 19 us, 100000 x 64 x 64 31 -> 16, 1000 x 100 x 1000 15 -> 6)
             if (!(bands && force_parts < 2 && (whole_small || fits_32_bits) && K > 16)) return -1;
-            const int64_t cus = dev->props.multiProcessorCount;
-            const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
-            if (many != (large >= cus)) return -1;
-            // (very short k ranges over many whole tiles are the walking blocks' case, measured 10-14 % ahead of the small tiles there)
-            if (many && whole_tiles && K / BK <= 8 && large >= 4 * cus && large % 8 == 0) return -1;
-            // Against the k range of the large tiles cut into parts, by two estimates fitted to measurements (microseconds):
-            // the small tiles run in rounds of one per unit at 0.48 per k-slice plus 5; the parts cost 1.93 per unit of
-            // split_plan's estimate plus 8 for the second launch and the shorter blocks.  1024^3 21 against 29 (measured: 21,
-            // 31), 1536 x 256 x 1536 17 against 26 (17, 31), 1024 x 1024 x 3072 51 against 60 (53, 64); the parts win
-            // 1152^3 36 against 40 (35, 39), 1792^3 108 against 113 (108, 111), 1280 x 4096 x 1280 116 against 128 (107, 127).
-            bool small_tiles = true;
-            const int64_t slices = (K + BK - 1) / BK;
-            const int small_n = (int)((N + t64::TN - 1) / t64::TN), small_m = (int)((M + t64::TM - 1) / t64::TM);
-            // ... or whole rounds of small tiles for the upper tile rows and the rest in parts of the k range, in one launch
-            // (MIXED, as for the large tiles): 1536^3, 576 small tiles: 2 rounds + 64 tiles in parts instead of 3 rounds, 76 -> 69 us;
-            // 1792^3 109 -> 95; 1500^3 78 -> 70 (estimate: the rounds, the parts' rounds of shorter blocks, + 6 for the second launch)
-            int64_t mixed_rows = 0, mixed_parts = 0;
-            if (small_tiles) {
-                double t_small = 0.48 * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
-                const int64_t rounds = small / cus, rows_a = rounds * cus / small_n, tiles_b = small - rows_a * small_n;
-                if (rounds >= 1 && tiles_b >= 1 && rows_a < small_m && slices >= 16) {
-                    int64_t parts = (cus + tiles_b - 1) / tiles_b;
-                    if (parts > slices / 4) parts = slices / 4;
-                    if (parts < 2) parts = 2;
-                    const int64_t part_slices = (slices + parts - 1) / parts;
-                    const double t_mixed = 0.48 * ((double)rounds * (double)slices + (double)((tiles_b * parts + cus - 1) / cus) * (double)part_slices) + 5.0 + 6.0;
-                    if (t_mixed < t_small && (uint64_t)parts * (uint64_t)(M - rows_a * t64::TM) * N * sizeof(float) <= ((uint64_t)1 << 30)) {
-                        t_small = t_mixed; mixed_rows = rows_a; mixed_parts = parts;
-                    }
-                }
-                // ... or, with less than a round of small tiles, every tile in parts (no upper rows): more blocks per unit at a time
-                // for long k ranges over few tiles, and no columns of padding where the large tiles would be half empty
-                if (rounds == 0 && slices >= 16) {
-                    int64_t best = 0; double t_best = t_small;
-                    for (int64_t parts = 2; parts <= slices / 4 && parts <= 64; parts++) {
-                        const int64_t part_slices = (slices + parts - 1) / parts;
-                        if ((parts - 1) * part_slices >= slices) continue;                  // the last part would be empty
-                        const double t = 0.48 * (double)((small * parts + cus - 1) / cus) * (double)part_slices + 5.0 + 6.0
-                                       + (double)parts * (double)M * (double)N * 8.0 / 4.0e6;
-                        if (t < t_best) { t_best = t; best = parts; }
-                    }
-                    if (best > 0 && (uint64_t)best * (uint64_t)M * N * sizeof(float) <= ((uint64_t)1 << 30)) { t_small = t_best; mixed_rows = 0; mixed_parts = best; }
-                }
-                MfmaArgs trial = g;
-                const double t_parts = many ? 1.85 * (double)((large + cus - 1) / cus) * (double)slices + 7.0
-                    : split_plan(dev, trial, BK, sizeof(float), 0) > 1
-                    ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
-                    : 1.93 * (double)slices + 7.0;
-                // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
-                small_tiles = t_small < (whole_tiles ? 1.0 : 1.15) * t_parts;
-            }
-            if (small_tiles) {
-                MfmaArgs gs = g;
-                gs.tiles_m = small_m; gs.tiles_n = small_n;
-                gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;
-                if (mixed_parts > 0) {
-                    gs.rows_a = (int)mixed_rows;
-                    gs.split_slices = (int)((slices + mixed_parts - 1) / mixed_parts);
-                    gs.splits = (int)((slices + gs.split_slices - 1) / gs.split_slices);
-                    const int64_t m_a = mixed_rows * t64::TM, m_b = M - m_a;
-                    void* ws = nullptr;
-                    if (int e = workspace(dev, (uint64_t)gs.splits * m_b * N * sizeof(float), &ws)) return e;
-                    const unsigned grid = (unsigned)(mixed_rows * small_n + (small - mixed_rows * small_n) * gs.splits);
-                    if (whole_small) {
-                        if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, false, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
-                        else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, false, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
+            static const SmallTileNames names = {"mfma_tiles_of_64", "mfma_tiles_of_64_edge", "mfma_tiles_of_64_split", "mfma_tiles_of_64_edge_split",
+                                                 "mfma_tiles_of_64_mixed", "mfma_tiles_of_64_edge_mixed"};
+            return nk::small_tile_plan<float>(dev, g, BK, many, whole_small, whole_tiles, whole_tiles && K / BK <= 8, Cp, names,
+                [&](bool mixed, bool edge_kernel, unsigned grid, const MfmaArgs& gs, float* P) {
+                    auto go = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, P); };
+                    if (mixed) {
+                        if (edge_kernel) { if (overwrite) go(matmul_mfma64_kernel<true, true, true>); else go(matmul_mfma64_kernel<false, true, true>); }
+                        else             { if (overwrite) go(matmul_mfma64_kernel<true, false, true>); else go(matmul_mfma64_kernel<false, false, true>); }
                     } else {
-                        if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, true, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
-                        else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, true, true>), dim3(grid), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp, (float*)ws);
+                        if (edge_kernel) { if (overwrite) go(matmul_mfma64_kernel<true, true, false>); else go(matmul_mfma64_kernel<false, true, false>); }
+                        else             { if (overwrite) go(matmul_mfma64_kernel<true, false, false>); else go(matmul_mfma64_kernel<false, false, false>); }
                     }
-                    launch_add_parts<float>(dev, m_b * N, gs.splits, g.overwrite, (const float*)ws, Cp + m_a * N);
-                    NK_HIP(hipGetLastError());
-                    set_path(mixed_rows == 0 ? (whole_small ? "mfma_tiles_of_64_split" : "mfma_tiles_of_64_edge_split")
-                                             : (whole_small ? "mfma_tiles_of_64_mixed" : "mfma_tiles_of_64_edge_mixed"));
-                    return NK_OK;
-                }
-                if (whole_small) {
-                    if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, false>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                    else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, false>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                } else {
-                    if (overwrite) hipLaunchKernelGGL((matmul_mfma64_kernel<true, true>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                    else           hipLaunchKernelGGL((matmul_mfma64_kernel<false, true>), dim3((unsigned)small), dim3(256), 0, dev->stream, gs, Ap, Bp, Cp);
-                }
-                NK_HIP(hipGetLastError());
-                set_path(whole_small ? "mfma_tiles_of_64" : "mfma_tiles_of_64_edge");
-                return NK_OK;
-            }
-            return -1;
+                });
         };
+
         if (const int rc = small_tile_plan(false); rc >= 0) return rc;
         if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;
         // A few more tiles than a whole number of rounds of one tile per compute unit: as one launch of whole tiles some units

@@ -1653,12 +1653,18 @@ def test_matmul_mfma_edge_path(device, orc, mkn):
     assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
-@pytest.mark.parametrize("mkn,path", [((256, 256, 256), "mfma_f64"), ((384, 112, 512), "mfma_f64"), ((128, 1024, 128), "mfma_f64"),
-                                      ((300, 257, 270), "mfma_f64_edge"), ((129, 1001, 131), "mfma_f64_edge"),
-                                      ((1000, 33, 1000), "mfma_f64_edge"), ((127, 4097, 40), "mfma_f64_edge"),
+@pytest.mark.parametrize("mkn,path", [((256, 256, 256), "mfma_f64_tiles_of_64"), ((384, 112, 512), "mfma_f64_tiles_of_64"), ((128, 1024, 128), "mfma_f64_tiles_of_64"),
+                                      ((300, 257, 270), "mfma_f64_tiles_of_64_edge"), ((129, 1001, 131), "mfma_f64_tiles_of_64_edge"),
+                                      ((1000, 33, 1000), "mfma_f64_tiles_of_64_edge"), ((127, 4097, 40), "mfma_f64_tiles_of_64_edge"),
+                                      ((1024, 1024, 1024), "mfma_f64_tiles_of_64"), ((1500, 17, 1500), "mfma_f64_tiles_of_64_edge"),
+                                      ((1536, 1024, 1536), "mfma_f64_tiles_of_64_mixed"), ((1111, 1111, 1111), "mfma_f64_tiles_of_64_edge_mixed"),
+                                      ((2560, 512, 2560), "mfma_f64_tiles_of_64_mixed"), ((2500, 1030, 2500), "mfma_f64_tiles_of_64_edge_mixed"),
+                                      ((2048, 512, 2048), "mfma_f64"), ((1152, 2048, 1152), "mfma_f64"),
                                       ((255, 255, 250), "simple")])
 def test_matmul_f64_matrix_core_path(device, orc, mkn, path):
-    """f64 products from 2^24 multiply-adds on run on the f64 matrix cores: exact on integer-valued data, within
+    """f64 products from 2^24 multiply-adds on run on the f64 matrix cores -- on 64 x 64 tiles (whole, as parts of the k
+    range, whole rounds plus parts; shapes that are no whole tiles; a single partial k-slice) where that fills the machine
+    better, else on 128 x 128 tiles: exact on integer-valued data, within
     1e-12 norm-wise of the reference's order on uniform data, accumulation into C, both layouts, nothing written
     or read outside the operands; below the threshold the reference's order is kept bit for bit."""
     M, K, N = mkn
@@ -1791,8 +1797,10 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
 @pytest.mark.parametrize("dt,mkn,path", [
     ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_tiles_of_64_split"), ("f32", (1152, 2048, 1152), "mfma_split"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
     ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_tiles_of_64_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 100, 2100), "mfma_tiles_of_64_edge"),
-    ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_split"), ("f64", (2048, 64, 2048), "mfma_f64"),
-    ("f64", (1000, 300, 520), "mfma_f64_edge_split"), ("f64", (2100, 130, 2100), "mfma_f64_edge"),
+    ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_tiles_of_64_split"), ("f64", (2048, 64, 2048), "mfma_f64_tiles_of_64"),
+    ("f64", (1000, 300, 520), "mfma_f64_tiles_of_64_edge"), ("f64", (2100, 130, 2100), "mfma_f64_tiles_of_64_edge"),
+    ("f64", (2048, 512, 2048), "mfma_f64"), ("f64", (1152, 2048, 1152), "mfma_f64_split"), ("f64", (1536, 1024, 1536), "mfma_f64_tiles_of_64_mixed"),
+    ("f64", (130, 4100, 70), "mfma_f64_tiles_of_64_edge_split"), ("f64", (1500, 1050, 1500), "mfma_f64_tiles_of_64_edge_mixed"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
     ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64"),
     ("f32", (4100, 9, 4096), "short_inner"), ("f64", (4096, 16, 2050), "short_inner_f64"),
