@@ -130,7 +130,7 @@ def test_broadcast_forward_and_backward_into_8_gib(device, orc):
 
 def test_matmul_into_8_gib(device):
     rng = np.random.default_rng(34)
-    for M, K, N, path in ((65408, 64, 32768, "mfma_stream"), (65535, 64, 32768, "mfma_edge")):
+    for M, K, N, path in ((65408, 64, 32768, "mfma_stream"), (65535, 64, 32768, "mfma_tiles_of_64_edge")):
         say("max size matmul", (M, K, N))
         A = rng.integers(-3, 4, (M, K)).astype(f32); B = rng.integers(-3, 4, (K, N)).astype(f32)
         want = A @ B
