@@ -1761,19 +1761,20 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
 // small tile then costs the same in both, as a slice of a large tile does).  `launch(mixed, edge, grid, args, P)` starts the
 // kernel.  Returns -1 when another plan should take the product.
 // `many`: the product has at least a round of large tiles; the small tiles are then held against the plain launch of the large
-// ones, ceil(tiles / units) x 1.85 us per k-slice + 7 (2560^3 f32, 400 large tiles = 2 rounds for the work of 1.56); otherwise
+// ones in rounds of one tile per unit (2560^3 f32, 400 large tiles = 2 rounds for the work of 1.56); otherwise
 // against the k range of the large tiles cut into parts.  `walking`: f32 whole tiles with at most eight k-slices.
 struct SmallTileNames { const char *whole, *edge, *whole_split, *edge_split, *whole_mixed, *edge_mixed; };
 template <typename T, typename Launch>
 static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many, bool whole_small, bool whole_tiles, bool walking,
                            T* Cp, const SmallTileNames& names, Launch launch) {
-    // a k-slice of a small tile on a unit of its own, microseconds (f32: 0.89 of the rate of its multiply-adds; the f64 kernel
-    // measures 0.54, but its plans on large tiles fall short of their estimates by as much, and 0.48 chooses better there too:
-    // 1536^3 f64 127 us mixed against 140 in parts, 1111^3 62 against 73, 2048 x 256 x 2048 40 against 45 on large tiles)
-    constexpr double c_small = 0.48;
     const int64_t M = g.M, K = g.K, N = g.N;
     const int64_t cus = dev->props.multiProcessorCount;
     const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
+    // A k-slice of a small tile on a unit, microseconds, measured with uniform random operands (small integers run 5 % faster
+    // on the small tiles and so flatter them): f32 0.48 with a tile per unit, 0.51 over many rounds (3328^3: 589 us); f64
+    // 0.54 with a tile per unit and 0.50 with two blocks on a unit (3328^3: 1136 us).
+    constexpr bool F64 = sizeof(T) == 8;
+    const double c_small = F64 ? (small <= cus ? 0.54 : 0.50) : (many ? 0.51 : 0.48);
     if (many != (large >= cus)) return -1;
     // (very short k ranges over many whole tiles are the walking blocks' case, measured 10-14 % ahead of the small tiles there)
     if (many && walking && large >= 4 * cus && large % 8 == 0) return -1;
@@ -1787,16 +1788,28 @@ static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many,
     // (MIXED, as for the large tiles): 1536^3, 576 small tiles: 2 rounds + 64 tiles in parts instead of 3 rounds, 76 -> 69 us;
     // 1792^3 109 -> 95; 1500^3 78 -> 70 (estimate: the rounds, the parts' rounds of shorter blocks, + 6 for the second launch)
     int64_t mixed_rows = 0, mixed_parts = 0;
-    double t_small = c_small * (double)((small + cus - 1) / cus) * (double)slices + 5.0;
+    // (per round of tiles, first fetch and write-back: 0.65 for a small f32 tile, 0.95 for f64, against 3.5 and 4.2 for the large
+    // ones -- what decides k ranges of a few slices: 3000 x 64 x 3000 f32 19.6 us in 9 rounds of small tiles, 31 in 3 of large ones)
+    const double e_small = F64 ? 0.95 : 0.65, e_large = F64 ? 4.2 : 3.5;
+    double t_small = (double)((small + cus - 1) / cus) * (c_small * (double)slices + (many ? e_small : 0.0)) + 5.0;
     const int64_t rounds = small / cus, rows_a = rounds * cus / small_n, tiles_b = small - rows_a * small_n;
     if (rounds >= 1 && tiles_b >= 1 && rows_a < small_m && slices >= 16) {
-        int64_t parts = (cus + tiles_b - 1) / tiles_b;
-        if (parts > slices / 4) parts = slices / 4;
-        if (parts < 2) parts = 2;
-        const int64_t part_slices = (slices + parts - 1) / parts;
-        const double t_mixed = c_small * ((double)rounds * (double)slices + (double)((tiles_b * parts + cus - 1) / cus) * (double)part_slices) + 5.0 + 6.0;
-        if (t_mixed < t_small && (uint64_t)parts * (uint64_t)(M - rows_a * t64::TM) * N * sizeof(T) <= ((uint64_t)1 << 30)) {
-            t_small = t_mixed; mixed_rows = rows_a; mixed_parts = parts;
+        // the number of parts that finishes first: the units the whole rounds leave idle take parts from the start (as many
+        // in a row as fit into a whole tile's time), the rest of the parts runs in rounds of its own; each part is written
+        // and read again (1111^3, 252 whole tiles + 72 in parts: 3 parts = 216 blocks fit into one more round, 4 do not)
+        const int64_t idle = rounds * cus - rows_a * small_n, m_b = M - rows_a * t64::TM;
+        for (int64_t parts = 2; parts <= slices / 4 && parts <= 64; parts++) {
+            const int64_t part_slices = (slices + parts - 1) / parts;
+            if ((parts - 1) * part_slices >= slices) continue;                      // the last part would be empty
+            int64_t left = tiles_b * parts - idle * parts;                          // (idle: in the last of the whole rounds)
+            if (left < 0) left = 0;
+            const int64_t part_rounds = (left + cus - 1) / cus;
+            const double t_mixed = c_small * ((double)rounds * (double)slices + (double)part_rounds * (double)part_slices)
+                                 + (many ? e_small * (double)(rounds + part_rounds) : 0.0) + 5.0 + 6.0
+                                 + (double)parts * (double)m_b * (double)N * 2.0 * sizeof(T) / 4.0e6;
+            if (t_mixed < t_small && (uint64_t)parts * (uint64_t)m_b * N * sizeof(T) <= ((uint64_t)1 << 30)) {
+                t_small = t_mixed; mixed_rows = rows_a; mixed_parts = parts;
+            }
         }
     }
     // ... or, with less than a round of small tiles, every tile in parts (no upper rows): more blocks per unit at a time
@@ -1813,12 +1826,25 @@ static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many,
         if (best > 0 && (uint64_t)best * (uint64_t)M * N * sizeof(T) <= ((uint64_t)1 << 30)) { t_small = t_best; mixed_rows = 0; mixed_parts = best; }
     }
     MfmaArgs trial = g;
-    const double t_parts = many ? 1.85 * (double)((large + cus - 1) / cus) * (double)slices + 7.0
-        : split_plan(dev, trial, slice, sizeof(T), 0) > 1
-        ? 1.93 * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
-        : 1.93 * (double)slices + 7.0;
-    // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
-    if (!(t_small < (whole_tiles ? 1.0 : 1.15) * t_parts)) return -1;
+    // The large tiles.  f32: 1.80 per k-slice and round of one tile per unit (3840^3: 871 us), in parts 1.93 per unit of
+    // split_plan's estimate.  The f64 kernel needs its two blocks per unit: 1.84 per slice for each of a pair, 2.17 for a
+    // block alone on its unit (2048^3: 278 us; 3328^3, 676 tiles = 512 + 164: 1207 us), in parts 2.2 (1920^3: 300 us).
+    double t_large;
+    if (many && F64) {
+        const int64_t pairs = large / (2 * cus), rest = large - pairs * 2 * cus;
+        t_large = (double)slices * ((double)pairs * 2.0 * 1.84 + (rest == 0 ? 0.0 : rest <= cus ? 2.17 : 2.0 * 1.84))
+                + e_large * (double)(2 * pairs + (rest == 0 ? 0 : rest <= cus ? 1 : 2)) + 7.0;
+    } else if (many) {
+        t_large = (double)((large + cus - 1) / cus) * (1.80 * (double)slices + e_large) + 7.0;
+    } else {
+        const double rate = F64 ? 2.2 : 1.93;
+        t_large = split_plan(dev, trial, slice, sizeof(T), 0) > 1
+            ? rate * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
+            : rate * (double)slices + 7.0;
+        // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
+        if (!whole_tiles) t_large *= 1.15;
+    }
+    if (!(t_small < t_large)) return -1;
     MfmaArgs gs = g;
     gs.tiles_m = small_m; gs.tiles_n = small_n;
     gs.group_rows = gs.tiles_m < 8 ? gs.tiles_m : 8;

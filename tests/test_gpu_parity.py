@@ -1659,7 +1659,8 @@ def test_matmul_mfma_edge_path(device, orc, mkn):
                                       ((1024, 1024, 1024), "mfma_f64_tiles_of_64"), ((1500, 17, 1500), "mfma_f64_tiles_of_64_edge"),
                                       ((1536, 1024, 1536), "mfma_f64_tiles_of_64_mixed"), ((1111, 1111, 1111), "mfma_f64_tiles_of_64_edge_mixed"),
                                       ((2560, 512, 2560), "mfma_f64_tiles_of_64_mixed"), ((2500, 1030, 2500), "mfma_f64_tiles_of_64_edge_mixed"),
-                                      ((2048, 512, 2048), "mfma_f64"), ((1152, 2048, 1152), "mfma_f64"),
+                                      ((2048, 512, 2048), "mfma_f64_tiles_of_64"), ((1152, 2048, 1152), "mfma_f64_tiles_of_64_mixed"),
+                                      ((4096, 256, 4096), "mfma_f64"), ((1280, 1280, 1280), "mfma_f64_tiles_of_64"),
                                       ((255, 255, 250), "simple")])
 def test_matmul_f64_matrix_core_path(device, orc, mkn, path):
     """f64 products from 2^24 multiply-adds on run on the f64 matrix cores -- on 64 x 64 tiles (whole, as parts of the k
@@ -1795,11 +1796,11 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
 
 
 @pytest.mark.parametrize("dt,mkn,path", [
-    ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_tiles_of_64_split"), ("f32", (1152, 2048, 1152), "mfma_split"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
+    ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_tiles_of_64_split"), ("f32", (1280, 2048, 1280), "mfma_split"), ("f32", (1152, 2048, 1152), "mfma_tiles_of_64_mixed"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
     ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_tiles_of_64_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 100, 2100), "mfma_tiles_of_64_edge"),
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_tiles_of_64_split"), ("f64", (2048, 64, 2048), "mfma_f64_tiles_of_64"),
     ("f64", (1000, 300, 520), "mfma_f64_tiles_of_64_edge"), ("f64", (2100, 130, 2100), "mfma_f64_tiles_of_64_edge"),
-    ("f64", (2048, 512, 2048), "mfma_f64"), ("f64", (1152, 2048, 1152), "mfma_f64_split"), ("f64", (1536, 1024, 1536), "mfma_f64_tiles_of_64_mixed"),
+    ("f64", (4096, 256, 4096), "mfma_f64"), ("f64", (1152, 2048, 1152), "mfma_f64_tiles_of_64_mixed"), ("f64", (1536, 1024, 1536), "mfma_f64_tiles_of_64_mixed"),
     ("f64", (130, 4100, 70), "mfma_f64_tiles_of_64_edge_split"), ("f64", (1500, 1050, 1500), "mfma_f64_tiles_of_64_edge_mixed"),
     ("f32", (3072, 1024, 3072), "mfma_bands"), ("f32", (3000, 800, 3100), "mfma_edge_bands"), ("f64", (3072, 512, 3072), "mfma_f64_bands"),
     ("f32", (5, 4096, 4096), "few_rows"), ("f64", (16, 4096, 1024), "few_rows_f64"), ("f32", (8192, 2048, 1), "few_cols"), ("f64", (4099, 2048, 4), "few_cols_f64"),
