@@ -156,6 +156,11 @@ def torch_yardstick():
     del x, y, z, out
     for name, (M, K, N), dt in (("matmul_4096_us", (4096, 4096, 4096), torch.float32), ("matmul_4000_us", (4000, 4000, 4000), torch.float32),
                                 ("matmul_3072_us", (3072, 3072, 3072), torch.float32), ("matmul_3072_f64_us", (3072, 3072, 3072), torch.float64),
+                                ("matmul_2560_us", (2560, 2560, 2560), torch.float32), ("matmul_2048_us", (2048, 2048, 2048), torch.float32),
+                                ("matmul_1536_us", (1536, 1536, 1536), torch.float32), ("matmul_1024_us", (1024, 1024, 1024), torch.float32),
+                                ("matmul_narrow_result_us", (4096, 4096, 64), torch.float32), ("matmul_short_k_us", (3000, 64, 3000), torch.float32),
+                                ("matmul_2048_f64_us", (2048, 2048, 2048), torch.float64), ("matmul_1024_f64_us", (1024, 1024, 1024), torch.float64),
+                                ("matmul_narrow_result_f64_us", (4096, 4096, 64), torch.float64),
                                 ("matmul_tall_skinny_us", (65536, 256, 256), torch.float32), ("matmul_4096_f64_us", (4096, 4096, 4096), torch.float64),
                                 ("matmul_matrix_vector_us", (4096, 4096, 1), torch.float32), ("matmul_batch_of_16_rows_us", (16, 4096, 4096), torch.float32),
                                 ("matmul_16_outer_products_us", (4096, 16, 4096), torch.float32), ("matmul_batch_of_16_columns_us", (4096, 4096, 16), torch.float32)):
@@ -608,8 +613,11 @@ def main():
         # (4000^3: a large shape that is no whole number of tiles)
         for name, (M, K, N) in (("matmul_4096", (4096, 4096, 4096)), ("matmul_tall_skinny", (65536, 256, 256)), ("matmul_4000", (4000, 4000, 4000)),
                                 ("matmul_3072", (3072, 3072, 3072)),           # 576 tiles of 128 x 128: a round of the machine and an eighth
+                                ("matmul_2560", (2560, 2560, 2560)),           # 400 tiles: the last round of large tiles would idle most units
                                 ("matmul_2048", (2048, 2048, 2048)), ("matmul_1536", (1536, 1536, 1536)),   # a round of tiles, and less
-                                ("matmul_1024", (1024, 1024, 1024))):
+                                ("matmul_1024", (1024, 1024, 1024)),
+                                ("matmul_narrow_result", (4096, 4096, 64)),    # few tiles, a long k range
+                                ("matmul_short_k", (3000, 64, 3000))):          # two k-slices, no whole tiles
             A = Tensor.of(f32, (M, K), rng.uniform(-1, 1, M * K).astype(f32)).to(dev)
             B = Tensor.of(f32, (K, N), rng.uniform(-1, 1, K * N).astype(f32)).to(dev)
             Cm = Tensor._on_device(dev, f32, (M, N))
@@ -633,12 +641,13 @@ def main():
             Cm = Tensor._on_device(dev, f32, (M, N))
             hbm(name, 4 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm))
             for t in (A, B, Cm): dev.free(t)
-        M = K = N = 3072
-        A = Tensor.of(np.float64, (M, K), rng.uniform(-1, 1, M * K)).to(dev)
-        B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)
-        Cm = Tensor._on_device(dev, np.float64, (M, N))
-        flops("matmul_3072_f64", 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm), f64=True)
-        for t in (A, B, Cm): dev.free(t)
+        for name, (M, K, N) in (("matmul_3072_f64", (3072, 3072, 3072)), ("matmul_2048_f64", (2048, 2048, 2048)), ("matmul_1024_f64", (1024, 1024, 1024)),
+                                ("matmul_narrow_result_f64", (4096, 4096, 64))):
+            A = Tensor.of(np.float64, (M, K), rng.uniform(-1, 1, M * K)).to(dev)
+            B = Tensor.of(np.float64, (K, N), rng.uniform(-1, 1, K * N)).to(dev)
+            Cm = Tensor._on_device(dev, np.float64, (M, N))
+            flops(name, 2.0 * M * K * N, 8 * (M * K + K * N + M * N), dev.prepared_launch("matmul_set", True, M, K, N, A, B, Cm), f64=True)
+            for t in (A, B, Cm): dev.free(t)
 
         # C1 and C5 convolutions
         x1 = Tensor.of(f32, (64, 64), rng.uniform(-1, 1, 4096).astype(f32)).to(dev)
