@@ -14,6 +14,15 @@
 //   mfma_f64 / mfma_f64_edge  f64 from 2^24 multiply-adds on: v_mfma_f64_16x16x4_f64, same tiling.
 //   ..._split  the same kernels for products with fewer tiles than compute units: the k range cut into parts,
 //            partial tiles in the device workspace, added in order by a second launch.
+//   ..._bands  a few more tiles than whole rounds of the machine: two row bands, the lower one in parts of its k range.
+//   mfma_mixed / mfma_edge_mixed  f32, a few more tiles than whole rounds of one per compute unit: one launch whose
+//            upper tile rows take the whole k range and whose lower rows come as parts of it.
+//   mfma_stream  f32 whole tiles with at most eight k-slices and many tiles: blocks that stay and walk the tiles.
+//   mfma_tiles_of_64, mfma_f64_tiles_of_64 (…_edge, …_split, …_mixed)  64x64 block tiles, chosen by an estimate of the
+//            time: products with few large tiles, with a last round of large tiles that would idle most units, narrow
+//            results over long k ranges (every tile in parts), k ranges of a few slices.
+//   few_rows / few_cols / some_cols / short_inner  products that stream one large operand once (a batch of up to 32
+//            rows or 16 columns, K <= 16): no matrix-core tiles, the large operand read once at the memory rate.
 //   simple   everything else (small products): one thread per element of C, the k loop in the
 //            reference's order with the product rounded before the add, which makes it bit-identical
 //            to GEMM.partial_F32_MxN_RM + AXPY (J/backend/main/operations/linear/internal/blas/GEMM.java:282-304,
