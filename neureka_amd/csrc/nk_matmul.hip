@@ -1775,7 +1775,7 @@ static int launch_mfma(Device* dev, MfmaArgs& g, int slice, T* Cp, Launch launch
 struct SmallTileNames { const char *whole, *edge, *whole_split, *edge_split, *whole_mixed, *edge_mixed; };
 template <typename T, typename Launch>
 static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many, bool whole_small, bool whole_tiles, bool walking,
-                           T* Cp, const SmallTileNames& names, Launch launch) {
+                           T* Cp, const SmallTileNames& names, Launch launch, double t_beat = 0.0) {
     const int64_t M = g.M, K = g.K, N = g.N;
     const int64_t cus = dev->props.multiProcessorCount;
     const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
@@ -1853,6 +1853,7 @@ static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many,
         // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
         if (!whole_tiles) t_large *= 1.15;
     }
+    if (t_beat > 0.0 && t_beat < t_large) t_large = t_beat;          // (the estimate of another plan that applies: the row bands)
     if (!(t_small < t_large)) return -1;
     MfmaArgs gs = g;
     gs.tiles_m = small_m; gs.tiles_n = small_n;
@@ -1912,7 +1913,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
     // whole rounds of tiles, the lower band's few tiles cut their k range into parts so that they fill one more, short,
     // round (partial results through the workspace, added in order as for every split product).  Times are in units
     // of one tile's time on a compute unit of its own.  Returns -1 when the product is better off in one piece.
-    auto run_bands = [&](int elem_bytes, int64_t slices, const char* path) -> int {
+    auto run_bands = [&](int elem_bytes, int64_t slices, const char* path, double* estimate = nullptr) -> int {
         if (!bands) return -1;
         const int64_t cus = dev->props.multiProcessorCount, resident = 2 * cus;
         const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
@@ -1930,6 +1931,9 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         const double part_len = (double)((slices + parts - 1) / parts) / (double)slices;
         const double then = (double)((tiles_a + cus - 1) / cus) + 2.0 * part_len + 0.15;     // + two more launches
         if (then >= 0.95 * now) return -1;
+        // (`estimate`: only say what the bands would take, in microseconds: a tile's time on a unit is 1.80 per k-slice + 3.5
+        // in f32, 1.84 + 4.2 in f64 with its two blocks per unit, and the two further launches cost 8)
+        if (estimate) { *estimate = then * ((elem_bytes == 8 ? 1.84 : 1.80) * (double)slices + (elem_bytes == 8 ? 4.2 : 3.5)) + 15.0; return NK_OK; }
         if (int e = matmul_rm(dev, dtype, overwrite, m_a, K, N, A, B, C, 0, false)) return e;
         if (int e = matmul_rm(dev, dtype, overwrite, m_b, K, N, A + (uint64_t)(m_a * K) * elem_bytes, B, C + (uint64_t)(m_a * N) * elem_bytes, (int)parts, false)) return e;
         set_path(path);
@@ -2100,7 +2104,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
             // the plans on 64 x 64 tiles, as for f32 below: before the bands for products with less than a round of large tiles,
             // after them for larger ones
             const bool whole_small = (A % 16 == 0) && (B % 16 == 0) && M % t64::TM == 0 && N % t64::TN == 0 && K % d64::DK == 0;
-            auto small_tile_plan = [&](bool many) -> int {
+            auto small_tile_plan = [&](bool many, double t_beat = 0.0) -> int {
                 if (!(bands && force_parts < 2 && K > 16)) return -1;
                 static const SmallTileNames names = {"mfma_f64_tiles_of_64", "mfma_f64_tiles_of_64_edge", "mfma_f64_tiles_of_64_split", "mfma_f64_tiles_of_64_edge_split",
                                                      "mfma_f64_tiles_of_64_mixed", "mfma_f64_tiles_of_64_edge_mixed"};
@@ -2114,10 +2118,16 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                             if (edge_kernel) { if (overwrite) go(matmul_mfma64_f64_kernel<true, true, false>); else go(matmul_mfma64_f64_kernel<false, true, false>); }
                             else             { if (overwrite) go(matmul_mfma64_f64_kernel<true, false, false>); else go(matmul_mfma64_f64_kernel<false, false, false>); }
                         }
-                    });
+                    }, t_beat);
             };
             if (const int rc = small_tile_plan(false); rc >= 0) return rc;
-            if (const int rc = run_bands(8, (K + d64::DK - 1) / d64::DK, whole ? "mfma_f64_bands" : "mfma_f64_edge_bands"); rc >= 0) return rc;
+            // where the row bands apply, the small tiles must beat them clearly (short k ranges: 3072 x 320 x 3072)
+            double t_bands = 0.0;
+            const char* bands_name = whole ? "mfma_f64_bands" : "mfma_f64_edge_bands";
+            if (run_bands(8, (K + d64::DK - 1) / d64::DK, bands_name, &t_bands) >= 0) {
+                if (const int rc = small_tile_plan(true, 0.93 * t_bands); rc >= 0) return rc;
+                if (const int rc = run_bands(8, (K + d64::DK - 1) / d64::DK, bands_name); rc >= 0) return rc;
+            }
             if (const int rc = small_tile_plan(true); rc >= 0) return rc;
             const int rc = launch_mfma<double>(dev, g, d64::DK, Cp, [&](bool split, dim3 grid, double* P) {
                 if (whole && split)       hipLaunchKernelGGL((matmul_mfma_f64_kernel<false, true>), grid, dim3(256), 0, dev->stream, g, Ap, Bp, Cp, P);
@@ -2172,7 +2182,7 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
         // fewer large tiles than compute units, but whole 64 x 64 tiles, at least one per unit: the small-tile kernel in one launch
         const bool whole_small = aligned && M % t64::TM == 0 && N % t64::TN == 0 && K % BK == 0;
         const bool fits_32_bits = M * K * 4 < ((int64_t)1 << 32) && K * N * 4 < ((int64_t)1 << 32);       // (the edge kernels' offsets)
-        auto small_tile_plan = [&](bool many) -> int {
+        auto small_tile_plan = [&](bool many, double t_beat = 0.0) -> int {
             // (from the shortest k ranges on, above the ones of the short-inner kernel: the kernel reads its slices clamped to
             // the last one, and with one or two slices a small tile's fetch and write-back overlap better with the other blocks
             // of its unit -- 3000 x 64 x 3000 31 -> 19 us, 100000 x 64 x 64 31 -> 16, 1000 x 100 x 1000 15 -> 6)
@@ -2189,11 +2199,18 @@ static int matmul_rm(Device* dev, int dtype, bool overwrite, int64_t M, int64_t 
                         if (edge_kernel) { if (overwrite) go(matmul_mfma64_kernel<true, true, false>); else go(matmul_mfma64_kernel<false, true, false>); }
                         else             { if (overwrite) go(matmul_mfma64_kernel<true, false, false>); else go(matmul_mfma64_kernel<false, false, false>); }
                     }
-                });
+                }, t_beat);
         };
 
         if (const int rc = small_tile_plan(false); rc >= 0) return rc;
-        if (const int rc = run_bands(4, (K + BK - 1) / BK, whole_tiles ? "mfma_bands" : "mfma_edge_bands"); rc >= 0) return rc;
+        {
+            double t_bands = 0.0;
+            const char* bands_name = whole_tiles ? "mfma_bands" : "mfma_edge_bands";
+            if (run_bands(4, (K + BK - 1) / BK, bands_name, &t_bands) >= 0) {
+                if (const int rc = small_tile_plan(true, 0.93 * t_bands); rc >= 0) return rc;
+                if (const int rc = run_bands(4, (K + BK - 1) / BK, bands_name); rc >= 0) return rc;
+            }
+        }
         // A few more tiles than a whole number of rounds of one tile per compute unit: as one launch of whole tiles some units
         // would work through one tile more than the others (side by side with another).  Instead the upper tile rows, whole
         // rounds, take the whole k range, and the tiles of the lower rows come as parts of their k range that fill the
