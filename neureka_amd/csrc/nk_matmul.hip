@@ -1739,6 +1739,11 @@ static int split_plan(Device* dev, MfmaArgs& g, int slice, size_t elem_bytes, in
             const double cost = (double)(((int64_t)tiles * p + cus - 1) / cus) * ((slices + p - 1) / p) + 0.75 * p;
             if (parts < 2 || cost < best) { parts = p; best = cost; }
         }
+        // ... or no parts at all: with nearly a tile per unit (f32 1920^3, 225 tiles: 115 us whole, 124 in two parts) one round
+        // of whole tiles (1.80 us per k-slice + 3.5, f64 2.17 + 4.2, and 7 for the launch) beats the parts (1.93, f64 2.2, per
+        // unit of the cost above, and 8 for the second launch)
+        const bool f64 = elem_bytes == 8;
+        if (parts >= 2 && (f64 ? 2.17 : 1.80) * slices + (f64 ? 4.2 : 3.5) + 7.0 <= (f64 ? 2.2 : 1.93) * best + 8.0) return 1;
     }
     if (parts > slices / 4) parts = slices / 4;
     if (parts > 64) parts = 64;
@@ -1780,10 +1785,10 @@ static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many,
     const int64_t cus = dev->props.multiProcessorCount;
     const int64_t large = (int64_t)g.tiles_m * g.tiles_n, small = ((M + t64::TM - 1) / t64::TM) * ((N + t64::TN - 1) / t64::TN);
     // A k-slice of a small tile on a unit, microseconds, measured with uniform random operands (small integers run 5 % faster
-    // on the small tiles and so flatter them): f32 0.48 with a tile per unit, 0.51 over many rounds (3328^3: 589 us); f64
-    // 0.54 with a tile per unit and 0.50 with two blocks on a unit (3328^3: 1136 us).
+    // on the small tiles and so flatter them): f32 0.48-0.54 from box to box with a tile per unit, 0.51 over many rounds
+    // (3328^3: 589 us); f64 0.54 with a tile per unit and 0.50 with two blocks on a unit (3328^3: 1136 us).
     constexpr bool F64 = sizeof(T) == 8;
-    const double c_small = F64 ? (small <= cus ? 0.54 : 0.50) : (many ? 0.51 : 0.48);
+    const double c_small = F64 ? (small <= cus ? 0.54 : 0.50) : (many ? 0.51 : 0.50);
     if (many != (large >= cus)) return -1;
     // (very short k ranges over many whole tiles are the walking blocks' case, measured 10-14 % ahead of the small tiles there)
     if (many && walking && large >= 4 * cus && large % 8 == 0) return -1;
@@ -1847,11 +1852,10 @@ static int small_tile_plan(Device* dev, const MfmaArgs& g, int slice, bool many,
         t_large = (double)((large + cus - 1) / cus) * (1.80 * (double)slices + e_large) + 7.0;
     } else {
         const double rate = F64 ? 2.2 : 1.93;
-        t_large = split_plan(dev, trial, slice, sizeof(T), 0) > 1
-            ? rate * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0
-            : rate * (double)slices + 7.0;
         // (the 128 x 128 edge kernel stores element by element and pads more: 1500^3 measured 86 in parts for an estimate of 72)
-        if (!whole_tiles) t_large *= 1.15;
+        t_large = split_plan(dev, trial, slice, sizeof(T), 0) > 1
+            ? (rate * ((double)(((int64_t)large * trial.splits + cus - 1) / cus) * trial.split_slices + 0.75 * trial.splits) + 8.0) * (whole_tiles ? 1.0 : 1.15)
+            : ((F64 ? 2.17 : 1.80) * (double)slices + e_large + 7.0) * (whole_tiles ? 1.0 : 1.05);
     }
     if (t_beat > 0.0 && t_beat < t_large) t_large = t_beat;          // (the estimate of another plan that applies: the row bands)
     if (!(t_small < t_large)) return -1;

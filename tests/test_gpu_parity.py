@@ -1796,7 +1796,7 @@ def test_matmul_blocks_that_walk_the_tiles(device, orc, mkn):
 
 
 @pytest.mark.parametrize("dt,mkn,path", [
-    ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_tiles_of_64_split"), ("f32", (1280, 2048, 1280), "mfma_split"), ("f32", (1152, 2048, 1152), "mfma_tiles_of_64_mixed"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
+    ("f32", (64, 48, 80), "simple"), ("f32", (384, 2048, 384), "mfma_tiles_of_64_split"), ("f32", (1280, 2048, 1280), "mfma_split"), ("f32", (1536, 1024, 1536), "mfma_tiles_of_64_mixed"), ("f32", (512, 512, 512), "mfma_tiles_of_64"), ("f32", (2048, 1024, 2048), "mfma"),
     ("f32", (12288, 256, 1536), "mfma_stream"), ("f32", (130, 4100, 70), "mfma_tiles_of_64_edge_split"), ("f32", (1000, 300, 520), "mfma_tiles_of_64_edge"), ("f32", (2100, 100, 2100), "mfma_tiles_of_64_edge"),
     ("f64", (64, 48, 80), "simple"), ("f64", (512, 512, 512), "mfma_f64_tiles_of_64_split"), ("f64", (2048, 64, 2048), "mfma_f64_tiles_of_64"),
     ("f64", (1000, 300, 520), "mfma_f64_tiles_of_64_edge"), ("f64", (2100, 130, 2100), "mfma_f64_tiles_of_64_edge"),
