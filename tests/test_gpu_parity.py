@@ -1931,6 +1931,38 @@ def test_matmul_64_tiles_in_one_launch(device, mkn, path):
         assert (np.abs(got[pad:pad + M * N].reshape(M, N).astype(np.float64) - ref) <= bound).all()
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_matmul_random_shapes_are_exact_in_whatever_plan_they_take(device, seed):
+    """Shapes drawn at random from six families (any shape, whole small tiles, long k over few tiles, short k over many,
+    whole large tiles, mid-size) in both element types: whatever plan the estimates choose, small-integer operands give
+    the exact product, for C = A B into NaNs and for C += A B into a non-zero C."""
+    rng = np.random.default_rng(seed)
+    def draw():
+        kind = rng.integers(0, 6)
+        if kind == 0: return int(rng.integers(33, 3000)), int(rng.integers(17, 3000)), int(rng.integers(17, 3000))
+        if kind == 1: return 64 * int(rng.integers(1, 48)), 32 * int(rng.integers(1, 64)), 64 * int(rng.integers(1, 48))
+        if kind == 2: return int(rng.integers(33, 400)), int(rng.integers(1000, 12000)), int(rng.integers(17, 400))
+        if kind == 3: return int(rng.integers(1000, 6000)), int(rng.integers(17, 200)), int(rng.integers(1000, 6000))
+        if kind == 4: return 128 * int(rng.integers(8, 30)), 32 * int(rng.integers(4, 40)), 128 * int(rng.integers(8, 30))
+        return int(rng.integers(1500, 4200)), int(rng.integers(200, 1500)), int(rng.integers(1500, 4200))
+    plans = set()
+    for _ in range(12):
+        M, K, N = draw()
+        for dt in (np.float32, np.float64):
+            say("matmul random shape", (M, K, N), dt.__name__)
+            A = rng.integers(-3, 4, (M, K)).astype(dt); B = rng.integers(-3, 4, (K, N)).astype(dt); C0 = rng.integers(-9, 10, (M, N)).astype(dt)
+            want = A.astype(np.float64) @ B.astype(np.float64)
+            ta, tb = on(device, A), on(device, B)
+            tc = on(device, np.full((M, N), np.nan, dtype=dt))
+            device.launch_matmul(True, M, K, N, ta, tb, tc, accumulate=False)
+            plans.add(_lib.last_path())
+            assert (tc.getData().reshape(M, N) == want).all(), ((M, K, N), dt.__name__, _lib.last_path())
+            tc = on(device, C0)
+            device.launch_matmul(True, M, K, N, ta, tb, tc)
+            assert (tc.getData().reshape(M, N) == want + C0).all(), ((M, K, N), dt.__name__, _lib.last_path())
+    say("plans seen", sorted(plans))
+
+
 @pytest.mark.parametrize("mkn", [(4096, 1024, 4096), (2048, 2048, 8192), (4096, 1056, 4096), (8192, 1024, 8192), (4096, 512, 4096)])
 def test_matmul_256_tiles_one_wavefront_per_simd(device, mkn):
     """Large f32 products whose 256 x 256 tiles fill the machine take the kernel with one wavefront per SIMD.  It sums
